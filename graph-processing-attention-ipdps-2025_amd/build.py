@@ -1,0 +1,124 @@
+"""Build libspfa_hip.so (HIP kernels + C ABI, gfx950) and the six torch host wrappers in-tree.
+
+    python build.py            # everything
+    python build.py --lib      # only libspfa_hip.so
+    python build.py --ext      # only the spfa_* Python modules
+
+The wrappers are host-only C++ (g++): they check tensors the way the reference bindings do and
+call the C ABI.  All device code is in libspfa_hip.so, compiled by hipcc for gfx950 only.
+"""
+from __future__ import annotations
+
+import argparse
+import concurrent.futures as cf
+import os
+import subprocess
+import sys
+import sysconfig
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(HERE)
+CSRC = os.path.join(HERE, "csrc")
+EXT = os.path.join(HERE, "ext")
+OBJ = os.path.join(HERE, "build")
+INCLUDE = os.path.join(ROOT, "include")
+
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+HIP_FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
+    # keep the compiler from forming packed-fp32 VALU ops out of scalar float code
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wno-unused-command-line-argument",
+    "-I", INCLUDE, "-I", CSRC,
+]
+
+ELEM_TYPES = {"f32": "float", "f16": "spfa::f16", "bf16": "spfa::bf16"}
+MASK_KINDS = {"csr": 0, "stride": 1, "global": 2}
+
+MODULES = ["spfa_csr", "spfa_coo", "spfa_local", "spfa_local_1d_dilated", "spfa_local_2d_dilated",
+           "spfa_global_no_local"]
+
+
+def _run(cmd):
+    p = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if p.returncode != 0:
+        sys.stderr.write(" ".join(cmd) + "\n" + p.stdout + "\n")
+        raise RuntimeError("build step failed: " + os.path.basename(cmd[-1]))
+    return p.stdout
+
+
+def lib_jobs():
+    jobs = []
+    for mname, mid in MASK_KINDS.items():
+        for tname, tcpp in ELEM_TYPES.items():
+            obj = os.path.join(OBJ, "inst_%s_%s.o" % (mname, tname))
+            jobs.append((obj, [HIPCC, *HIP_FLAGS, "-DSPFA_INST_MASK=%d" % mid,
+                               "-DSPFA_INST_T=%s" % tcpp, "-c",
+                               os.path.join(CSRC, "spfa_inst.hip"), "-o", obj]))
+    for src in sorted(os.listdir(CSRC)):
+        if src.endswith(".hip") and src != "spfa_inst.hip":
+            obj = os.path.join(OBJ, src[:-4] + ".o")
+            jobs.append((obj, [HIPCC, *HIP_FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]))
+    return jobs
+
+
+def build_lib(workers: int) -> str:
+    os.makedirs(OBJ, exist_ok=True)
+    jobs = lib_jobs()
+    with cf.ThreadPoolExecutor(max_workers=workers) as ex:
+        list(ex.map(lambda j: _run(j[1]), jobs))
+    out = os.path.join(HERE, "libspfa_hip.so")
+    _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", out, *[j[0] for j in jobs]])
+    return out
+
+
+def build_ext(workers: int):
+    import torch
+    from torch.utils import cpp_extension as ce
+
+    os.makedirs(OBJ, exist_ok=True)
+    inc = []
+    for p in ce.include_paths("cuda"):  # on torch-ROCm this adds the HIP headers
+        inc += ["-I", p]
+    inc += ["-I", os.path.join(os.environ.get("ROCM_PATH", "/opt/rocm"), "include")]
+    inc += ["-I", sysconfig.get_paths()["include"], "-I", INCLUDE, "-I", EXT]
+    torch_lib = os.path.join(os.path.dirname(torch.__file__), "lib")
+    cxx = os.environ.get("CXX", "g++")
+    abi = int(torch._C._GLIBCXX_USE_CXX11_ABI)
+    outs = []
+    jobs = []
+    for mod in MODULES:
+        out = os.path.join(HERE, mod + ".so")
+        outs.append(out)
+        jobs.append([cxx, "-O2", "-std=c++17", "-fPIC", "-shared", "-fvisibility=hidden",
+                     "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1", "-DTORCH_EXTENSION_NAME=" + mod,
+                     "-DTORCH_API_INCLUDE_EXTENSION_H", "-D_GLIBCXX_USE_CXX11_ABI=%d" % abi,
+                     "-Wno-deprecated-declarations", *inc,
+                     os.path.join(EXT, mod + ".cpp"), "-o", out,
+                     "-L", HERE, "-lspfa_hip", "-L", torch_lib, "-ltorch_python", "-ltorch",
+                     "-ltorch_cpu", "-ltorch_hip", "-lc10", "-lc10_hip",
+                     "-Wl,-rpath,$ORIGIN", "-Wl,-rpath," + torch_lib])
+    with cf.ThreadPoolExecutor(max_workers=workers) as ex:
+        list(ex.map(_run, jobs))
+    return outs
+
+
+def build_all(workers: int | None = None):
+    workers = workers or min(8, os.cpu_count() or 4)
+    lib = build_lib(workers)
+    exts = build_ext(min(workers, 6))
+    return [lib, *exts]
+
+
+if __name__ == "__main__":
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--lib", action="store_true")
+    ap.add_argument("--ext", action="store_true")
+    ap.add_argument("-j", type=int, default=None)
+    a = ap.parse_args()
+    w = a.j or min(8, os.cpu_count() or 4)
+    if a.lib or not a.ext:
+        print(build_lib(w))
+    if a.ext or not a.lib:
+        for o in build_ext(min(w, 6)):
+            print(o)

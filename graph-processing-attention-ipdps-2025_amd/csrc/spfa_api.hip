@@ -1,0 +1,335 @@
+// extern "C" surface of libspfa_hip.so: argument checks, work sizing, workspace carving and the
+// dispatch on element type.  Declarations and the contract live in include/spfa_hip.h.
+#include "spfa_hip.h"
+
+#include <limits>
+
+#include "spfa_kernels.hpp"
+
+using namespace spfa;
+
+namespace {
+
+constexpr int64_t kInlineAll = std::numeric_limits<int64_t>::max();
+
+inline int64_t clamp64(int64_t x, int64_t lo, int64_t hi) { return x < lo ? lo : (x > hi ? hi : x); }
+
+inline size_t dtype_size(int dtype) { return dtype == SPFA_DTYPE_F32 ? 4 : 2; }
+
+inline bool dtype_ok(int dtype) {
+  return dtype == SPFA_DTYPE_F32 || dtype == SPFA_DTYPE_F16 || dtype == SPFA_DTYPE_BF16;
+}
+
+// segment length: enough segments to keep every wavefront slot busy several times over, long
+// enough that the per-segment overhead (q load, group merge, partial write) stays small
+inline int64_t pick_segment(int64_t nnz_long) {
+  return clamp64(pow2_ceil(nnz_long / 65536 + 1), 256, 8192);
+}
+
+EngineSizing size_csr(int64_t n_q, int64_t nnz) {
+  EngineSizing s{};
+  s.nnz_bound = nnz;
+  s.max_deg = nnz;
+  s.short_max = 32;
+  s.seg = pick_segment(nnz);
+  s.n_long_bound = n_q;
+  return s;
+}
+
+// Band / block masks are uniform: every row has about the same number of candidates, so rows
+// are finished in place unless there are too few rows to fill the device and they are long.
+EngineSizing size_stride(int64_t n, int64_t max_deg) {
+  EngineSizing s{};
+  s.max_deg = max_deg;
+  s.nnz_bound = n * max_deg;
+  s.n_long_bound = n;
+  if (n < 16384 && max_deg > 1024) {
+    s.short_max = 256;
+    s.seg = 256;
+  } else {
+    s.short_max = kInlineAll;
+    s.seg = 256;
+  }
+  return s;
+}
+
+EngineSizing size_global(int64_t n, int64_t n_globs) {
+  EngineSizing s{};
+  const int64_t g = n_globs < n ? n_globs : n;
+  s.max_deg = n;
+  if (n_globs <= 4096) {
+    // ordinary rows (n_globs candidates each) are finished in place, global rows are split
+    s.short_max = n_globs < 32 ? 32 : n_globs;
+    s.n_long_bound = g;
+    s.nnz_bound = g * n;
+  } else {
+    s.short_max = 256;
+    s.n_long_bound = n;
+    s.nnz_bound = g * n + n * n_globs;
+  }
+  s.seg = pick_segment(s.nnz_bound);
+  return s;
+}
+
+int check_problem(const spfa_problem_t* p) {
+  if (p == nullptr) return SPFA_ERR_BAD_ARG;
+  if (p->n_q < 0 || p->n_k < 0) return SPFA_ERR_BAD_ARG;
+  if (p->n_q >= (int64_t)1 << 31 || p->n_k >= (int64_t)1 << 31) return SPFA_ERR_BAD_ARG;
+  if (p->d < 1 || p->d > 1024) return SPFA_ERR_EMB_TOO_LARGE;
+  return SPFA_OK;
+}
+
+int check_pointers(const spfa_problem_t* p) {
+  if (!dtype_ok(p->dtype)) return SPFA_ERR_UNSUPPORTED;
+  if (p->state_dtype != p->dtype && p->state_dtype != SPFA_DTYPE_F32) return SPFA_ERR_UNSUPPORTED;
+  if (p->n_q == 0) return SPFA_OK;
+  if (!p->q || !p->k || !p->v || !p->m || !p->l || !p->out) return SPFA_ERR_BAD_ARG;
+  return SPFA_OK;
+}
+
+int check_workspace(const void* ws, size_t have, size_t need) {
+  if (need == 0) return SPFA_OK;
+  if (ws == nullptr || ((uintptr_t)ws & 255u) != 0 || have < need) return SPFA_ERR_WORKSPACE;
+  return SPFA_OK;
+}
+
+Tensors make_tensors(const spfa_problem_t* p) {
+  Tensors t{};
+  t.q = p->q;
+  t.k = p->k;
+  t.v = p->v;
+  t.m = p->m;
+  t.l = p->l;
+  t.out = p->out;
+  t.n_q = p->n_q;
+  t.d = (int32_t)p->d;
+  t.state_f32 = (p->state_dtype == SPFA_DTYPE_F32) ? 1 : 0;
+  return t;
+}
+
+int dispatch_csr(const spfa_problem_t* p, const CsrMask& mask, const EngineSizing& s, int use_nan,
+                 void* ws, hipStream_t stream) {
+  Tensors t = make_tensors(p);
+  switch (p->dtype) {
+    case SPFA_DTYPE_F32: return run_csr<float>(t, mask, s, use_nan, ws, stream);
+    case SPFA_DTYPE_F16: return run_csr<f16>(t, mask, s, use_nan, ws, stream);
+    case SPFA_DTYPE_BF16: return run_csr<bf16>(t, mask, s, use_nan, ws, stream);
+  }
+  return SPFA_ERR_UNSUPPORTED;
+}
+
+int dispatch_stride(const spfa_problem_t* p, const StrideMask& mask, const EngineSizing& s,
+                    int use_nan, void* ws, hipStream_t stream) {
+  Tensors t = make_tensors(p);
+  switch (p->dtype) {
+    case SPFA_DTYPE_F32: return run_stride<float>(t, mask, s, use_nan, ws, stream);
+    case SPFA_DTYPE_F16: return run_stride<f16>(t, mask, s, use_nan, ws, stream);
+    case SPFA_DTYPE_BF16: return run_stride<bf16>(t, mask, s, use_nan, ws, stream);
+  }
+  return SPFA_ERR_UNSUPPORTED;
+}
+
+int dispatch_global(const spfa_problem_t* p, const GlobalMask& mask, const EngineSizing& s,
+                    void* ws, hipStream_t stream) {
+  Tensors t = make_tensors(p);
+  switch (p->dtype) {
+    case SPFA_DTYPE_F32: return run_global<float>(t, mask, s, 0, ws, stream);
+    case SPFA_DTYPE_F16: return run_global<f16>(t, mask, s, 0, ws, stream);
+    case SPFA_DTYPE_BF16: return run_global<bf16>(t, mask, s, 0, ws, stream);
+  }
+  return SPFA_ERR_UNSUPPORTED;
+}
+
+int64_t band_max_deg(int64_t n, int64_t w) {
+  int64_t deg = 2 * w + 1;
+  return deg < n ? deg : n;
+}
+
+int64_t block_live_count(int64_t block, int64_t s) {
+  int64_t cnt = (block - 1) / s + 1;
+  return cnt < block ? cnt : block;
+}
+
+size_t global_flag_bytes(int64_t n) { return align_up((size_t)((n + 3) / 4 * 4), 256); }
+
+}  // namespace
+
+extern "C" {
+
+int spfa_version(void) { return 1; }
+
+const char* spfa_status_string(int status) {
+  switch (status) {
+    case SPFA_OK: return "ok";
+    case SPFA_ERR_BAD_ARG: return "spfa: bad argument (null pointer, negative size or index width not 4/8)";
+    case SPFA_ERR_UNSUPPORTED: return "spfa: unsupported element type";
+    case SPFA_ERR_WORKSPACE: return "spfa: workspace missing, misaligned or too small";
+    case SPFA_ERR_LAUNCH: return "spfa: kernel launch failed";
+    case SPFA_ERR_EMB_TOO_LARGE:
+      return "The embedded dimension is too large for the amount of shared memory on your GPU.";
+    case SPFA_ERR_LOCAL_SIZE:
+      return "The local size specified is either negative or greater than/equal to (1 - Sequence Length).";
+    case SPFA_ERR_DILATION_NEG: return "The dilation factor must be atleast 0.";
+    case SPFA_ERR_BLOCK_DIVISOR:
+      return "The block/window size must be a divisor of the whole tensor's size.";
+    case SPFA_ERR_BLOCK_DILATION: return "The dilation factor must be less than the block/window size.";
+    case SPFA_ERR_GLOBAL_COUNT:
+      return "There are either no global tokens provided or there are more than the sequence length given.";
+  }
+  return "spfa: unknown status";
+}
+
+/* ------------------------------------------------------------------------------ CSR */
+size_t spfa_csr_workspace_bytes(int64_t n_q, int64_t nnz, int64_t d, int dtype) {
+  (void)dtype;
+  if (n_q < 0 || nnz < 0 || d < 1) return 0;
+  return engine_workspace(size_csr(n_q, nnz), n_q, d).total;
+}
+
+int spfa_csr_forward(const spfa_problem_t* p, const void* row_off, int row_off_bytes,
+                     const void* col_ind, int64_t nnz, int use_nan, void* workspace,
+                     size_t workspace_bytes, void* stream) {
+  int rc = check_problem(p);
+  if (rc) return rc;
+  if (nnz < 0 || (row_off_bytes != 4 && row_off_bytes != 8)) return SPFA_ERR_BAD_ARG;
+  rc = check_pointers(p);
+  if (rc) return rc;
+  if (p->n_q == 0) return SPFA_OK;
+  if (!row_off || (nnz > 0 && !col_ind)) return SPFA_ERR_BAD_ARG;
+  EngineSizing s = size_csr(p->n_q, nnz);
+  rc = check_workspace(workspace, workspace_bytes, engine_workspace(s, p->n_q, p->d).total);
+  if (rc) return rc;
+  CsrMask mask{row_off, (const uint32_t*)col_ind, row_off_bytes == 8 ? 1 : 0};
+  return dispatch_csr(p, mask, s, use_nan ? 1 : 0, workspace, (hipStream_t)stream);
+}
+
+/* ------------------------------------------------------------------------------ COO */
+size_t spfa_coo_workspace_bytes(int64_t n_q, int64_t nnz, int64_t d, int dtype) {
+  (void)dtype;
+  if (n_q < 0 || nnz < 0 || d < 1) return 0;
+  return coo_workspace(n_q, nnz).total + engine_workspace(size_csr(n_q, nnz), n_q, d).total;
+}
+
+int spfa_coo_forward(const spfa_problem_t* p, const void* row_ind, int row_ind_bytes,
+                     const void* col_ind, int64_t nnz, int use_nan, void* workspace,
+                     size_t workspace_bytes, void* stream) {
+  int rc = check_problem(p);
+  if (rc) return rc;
+  if (nnz < 0 || nnz >= (int64_t)1 << 31 || (row_ind_bytes != 4 && row_ind_bytes != 8))
+    return SPFA_ERR_BAD_ARG;
+  rc = check_pointers(p);
+  if (rc) return rc;
+  if (p->n_q == 0) return SPFA_OK;
+  if (nnz > 0 && (!row_ind || !col_ind)) return SPFA_ERR_BAD_ARG;
+  EngineSizing s = size_csr(p->n_q, nnz);
+  const size_t coo_bytes = coo_workspace(p->n_q, nnz).total;
+  rc = check_workspace(workspace, workspace_bytes,
+                       coo_bytes + engine_workspace(s, p->n_q, p->d).total);
+  if (rc) return rc;
+  const uint32_t* row_off = nullptr;
+  const uint32_t* cols = nullptr;
+  rc = coo_bucket_by_row(row_ind, row_ind_bytes == 8 ? 1 : 0, (const uint32_t*)col_ind, nnz, p->n_q,
+                         workspace, (hipStream_t)stream, &row_off, &cols);
+  if (rc) return rc;
+  CsrMask mask{row_off, cols, 0};
+  return dispatch_csr(p, mask, s, use_nan ? 1 : 0, (char*)workspace + coo_bytes,
+                      (hipStream_t)stream);
+}
+
+/* ------------------------------------------------------------------------------ Local */
+size_t spfa_local_workspace_bytes(int64_t n, int64_t d, int dtype, int64_t local_size) {
+  (void)dtype;
+  if (n < 1 || d < 1 || local_size < 0) return 0;
+  return engine_workspace(size_stride(n, band_max_deg(n, local_size)), n, d).total;
+}
+
+int spfa_local_forward(const spfa_problem_t* p, int64_t local_size, void* workspace,
+                       size_t workspace_bytes, void* stream) {
+  return spfa_local_1d_dilated_forward(p, local_size, 0, workspace, workspace_bytes, stream);
+}
+
+/* ------------------------------------------------------------------------------ Local 1D dilated */
+size_t spfa_local_1d_dilated_workspace_bytes(int64_t n, int64_t d, int dtype, int64_t local_size,
+                                             int64_t dil_factor) {
+  (void)dil_factor;
+  return spfa_local_workspace_bytes(n, d, dtype, local_size);
+}
+
+int spfa_local_1d_dilated_forward(const spfa_problem_t* p, int64_t local_size, int64_t dil_factor,
+                                  void* workspace, size_t workspace_bytes, void* stream) {
+  int rc = check_problem(p);
+  if (rc) return rc;
+  if (local_size < 0 || local_size > p->n_q - 1) return SPFA_ERR_LOCAL_SIZE;
+  if (dil_factor < 0) return SPFA_ERR_DILATION_NEG;
+  if (dil_factor >= (int64_t)1 << 31) return SPFA_ERR_BAD_ARG;
+  rc = check_pointers(p);
+  if (rc) return rc;
+  const int64_t n = p->n_q;
+  EngineSizing s = size_stride(n, band_max_deg(n, local_size));
+  rc = check_workspace(workspace, workspace_bytes, engine_workspace(s, n, p->d).total);
+  if (rc) return rc;
+  StrideMask mask{n, local_size, dil_factor + 1, 0, 0};
+  return dispatch_stride(p, mask, s, 0, workspace, (hipStream_t)stream);
+}
+
+/* ------------------------------------------------------------------------------ Local 2D dilated */
+size_t spfa_local_2d_dilated_workspace_bytes(int64_t n, int64_t d, int dtype, int64_t block_size,
+                                             int64_t dil_factor) {
+  (void)dtype;
+  if (n < 1 || d < 1 || block_size < 1 || dil_factor < 0) return 0;
+  return engine_workspace(size_stride(n, block_live_count(block_size, dil_factor + 1)), n, d).total;
+}
+
+int spfa_local_2d_dilated_forward(const spfa_problem_t* p, int64_t block_size, int64_t dil_factor,
+                                  int use_nan, void* workspace, size_t workspace_bytes,
+                                  void* stream) {
+  int rc = check_problem(p);
+  if (rc) return rc;
+  if (block_size <= 0 || p->n_q % block_size != 0) return SPFA_ERR_BLOCK_DIVISOR;
+  if (dil_factor < 0) return SPFA_ERR_DILATION_NEG;
+  if (block_size / (dil_factor + 1) < 1) return SPFA_ERR_BLOCK_DILATION;
+  rc = check_pointers(p);
+  if (rc) return rc;
+  const int64_t n = p->n_q;
+  if (n == 0) return SPFA_OK;
+  const int64_t cnt = block_live_count(block_size, dil_factor + 1);
+  EngineSizing s = size_stride(n, cnt);
+  rc = check_workspace(workspace, workspace_bytes, engine_workspace(s, n, p->d).total);
+  if (rc) return rc;
+  StrideMask mask{n, 0, dil_factor + 1, block_size, cnt};
+  return dispatch_stride(p, mask, s, use_nan ? 1 : 0, workspace, (hipStream_t)stream);
+}
+
+/* ------------------------------------------------------------------------------ Global minus local */
+size_t spfa_global_no_local_workspace_bytes(int64_t n, int64_t d, int dtype, int64_t n_globals,
+                                            int64_t local_size) {
+  (void)dtype;
+  (void)local_size;
+  if (n < 1 || d < 1 || n_globals < 1) return 0;
+  return global_flag_bytes(n) + engine_workspace(size_global(n, n_globals), n, d).total;
+}
+
+int spfa_global_no_local_forward(const spfa_problem_t* p, const int32_t* global_inds,
+                                 int64_t n_globals, int64_t local_size, void* workspace,
+                                 size_t workspace_bytes, void* stream) {
+  int rc = check_problem(p);
+  if (rc) return rc;
+  if (n_globals <= 0 || n_globals > p->n_q) return SPFA_ERR_GLOBAL_COUNT;
+  if (local_size < 0 || local_size > p->n_q - 1) return SPFA_ERR_LOCAL_SIZE;
+  rc = check_pointers(p);
+  if (rc) return rc;
+  if (!global_inds) return SPFA_ERR_BAD_ARG;
+  const int64_t n = p->n_q;
+  EngineSizing s = size_global(n, n_globals);
+  const size_t flag_bytes = global_flag_bytes(n);
+  rc = check_workspace(workspace, workspace_bytes,
+                       flag_bytes + engine_workspace(s, n, p->d).total);
+  if (rc) return rc;
+  uint8_t* flags = (uint8_t*)workspace;
+  rc = mark_global_rows(global_inds, n_globals, n, flags, (hipStream_t)stream);
+  if (rc) return rc;
+  GlobalMask mask{n, local_size, global_inds, n_globals, flags};
+  return dispatch_global(p, mask, s, (char*)workspace + flag_bytes, (hipStream_t)stream);
+}
+
+}  // extern "C"

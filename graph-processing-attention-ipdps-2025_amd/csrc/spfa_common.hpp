@@ -1,0 +1,205 @@
+// Shared device helpers for the gfx950 sparse-attention kernels: element conversions,
+// wave64 lane layouts and cross-lane reductions.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace spfa {
+
+constexpr int kWave = 64;
+constexpr float kNegInf = -__builtin_inff();
+
+using f16 = _Float16;
+using bf16 = __bf16;
+
+typedef float float4v __attribute__((ext_vector_type(4)));
+typedef _Float16 half8v __attribute__((ext_vector_type(8)));
+typedef __bf16 bhalf8v __attribute__((ext_vector_type(8)));
+typedef uint32_t uint4v __attribute__((ext_vector_type(4)));
+
+template <typename T>
+__device__ __forceinline__ float to_f32(T x) { return (float)x; }
+template <typename T>
+__device__ __forceinline__ T from_f32(float x) { return (T)x; }
+
+// m and l may be stored in the element type (reference behaviour) or in fp32.
+template <typename T>
+__device__ __forceinline__ float load_state(const void* p, int64_t i, bool state_f32) {
+  return state_f32 ? ((const float*)p)[i] : to_f32(((const T*)p)[i]);
+}
+template <typename T>
+__device__ __forceinline__ void store_state(void* p, int64_t i, float x, bool state_f32) {
+  if (state_f32) ((float*)p)[i] = x;
+  else ((T*)p)[i] = from_f32<T>(x);
+}
+
+// ---------------------------------------------------------------------------------------
+// cross-lane moves
+// ---------------------------------------------------------------------------------------
+template <int CTRL>
+__device__ __forceinline__ float dpp_f32(float x) {
+  return __builtin_bit_cast(
+      float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, 0xf, 0xf, false));
+}
+
+__device__ __forceinline__ float shfl_xor_f32(float x, int mask) {
+  int lane = (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+  return __builtin_bit_cast(
+      float, __builtin_amdgcn_ds_bpermute((lane ^ mask) << 2, __builtin_bit_cast(int, x)));
+}
+__device__ __forceinline__ int shfl_i32(int x, int src_lane) {
+  return __builtin_amdgcn_ds_bpermute(src_lane << 2, x);
+}
+__device__ __forceinline__ float shfl_f32(float x, int src_lane) {
+  return __builtin_bit_cast(float,
+                            __builtin_amdgcn_ds_bpermute(src_lane << 2, __builtin_bit_cast(int, x)));
+}
+
+// Sum over aligned groups of LPR consecutive lanes; every lane of the group gets the total.
+// 4 lanes: two quad permutes; 8: half-row mirror; 16: row mirror (all DPP, no LDS traffic);
+// 32: ds_swizzle xor 16; 64: bpermute xor 32.
+template <int LPR>
+__device__ __forceinline__ float group_sum(float x) {
+  static_assert(LPR == 1 || LPR == 2 || LPR == 4 || LPR == 8 || LPR == 16 || LPR == 32 || LPR == 64,
+                "lanes per row must be a power of two");
+  if constexpr (LPR >= 2) x += dpp_f32<0xB1>(x);   // quad_perm [1,0,3,2]
+  if constexpr (LPR >= 4) x += dpp_f32<0x4E>(x);   // quad_perm [2,3,0,1]
+  if constexpr (LPR >= 8) x += dpp_f32<0x141>(x);  // row_half_mirror
+  if constexpr (LPR >= 16) x += dpp_f32<0x140>(x); // row_mirror
+  if constexpr (LPR >= 32)
+    x += __builtin_bit_cast(float,
+                            __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, x), 0x401F));
+  if constexpr (LPR >= 64) x += shfl_xor_f32(x, 32);
+  return x;
+}
+
+// ---------------------------------------------------------------------------------------
+// lane layouts: how the d elements of one K/V/Q/O row are spread over lanes
+// ---------------------------------------------------------------------------------------
+// VecLay: d * sizeof(T) == LPR * 16 bytes.  Lane c of a group owns 16 contiguous bytes of the
+// row, so one wave-wide load instruction fetches 64/LPR whole rows with full 16-byte lanes.
+template <typename T, int LPR_>
+struct VecLay {
+  using elem = T;
+  static constexpr int LPR = LPR_;
+  static constexpr int GROUPS = kWave / LPR;
+  static constexpr int NE = 16 / (int)sizeof(T);  // floats held per lane
+  static constexpr int D = LPR * NE;
+  static constexpr int U = 8;        // neighbours in flight per group in the segment kernel
+  static constexpr int U_SHORT = 4;  // ... in the row kernel
+  static constexpr bool kFixedD = true;
+  using raw = uint4v;
+
+  __device__ static __forceinline__ raw load(const T* row_ptr, int c, int) {
+    return *reinterpret_cast<const raw*>(reinterpret_cast<const char*>(row_ptr) + c * 16);
+  }
+  __device__ static __forceinline__ void unpack(const raw& r, float (&f)[NE]) {
+    if constexpr (sizeof(T) == 4) {
+      float4v x = __builtin_bit_cast(float4v, r);
+#pragma unroll
+      for (int e = 0; e < 4; e++) f[e] = x[e];
+    } else if constexpr (__is_same(T, f16)) {
+      half8v x = __builtin_bit_cast(half8v, r);
+#pragma unroll
+      for (int e = 0; e < 8; e++) f[e] = (float)x[e];
+    } else {
+      // bf16 -> f32 is a 16-bit left shift
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        f[2 * e] = __builtin_bit_cast(float, r[e] << 16);
+        f[2 * e + 1] = __builtin_bit_cast(float, r[e] & 0xffff0000u);
+      }
+    }
+  }
+  __device__ static __forceinline__ void store(T* row_ptr, int c, int, const float (&f)[NE]) {
+    raw r;
+    if constexpr (sizeof(T) == 4) {
+      float4v x;
+#pragma unroll
+      for (int e = 0; e < 4; e++) x[e] = f[e];
+      r = __builtin_bit_cast(raw, x);
+    } else if constexpr (__is_same(T, f16)) {
+      half8v x;
+#pragma unroll
+      for (int e = 0; e < 8; e++) x[e] = (f16)f[e];
+      r = __builtin_bit_cast(raw, x);
+    } else {
+      bhalf8v x;
+#pragma unroll
+      for (int e = 0; e < 8; e++) x[e] = (bf16)f[e];
+      r = __builtin_bit_cast(raw, x);
+    }
+    *reinterpret_cast<raw*>(reinterpret_cast<char*>(row_ptr) + c * 16) = r;
+  }
+  // fp32 partial rows in the workspace: element e of lane c is at c*NE + e
+  __device__ static __forceinline__ void load_f32(const float* row_ptr, int c, int, float (&f)[NE]) {
+#pragma unroll
+    for (int e = 0; e < NE; e += 4) {
+      float4v x = *reinterpret_cast<const float4v*>(row_ptr + c * NE + e);
+      f[e] = x[0]; f[e + 1] = x[1]; f[e + 2] = x[2]; f[e + 3] = x[3];
+    }
+  }
+  __device__ static __forceinline__ void store_f32(float* row_ptr, int c, int, const float (&f)[NE]) {
+#pragma unroll
+    for (int e = 0; e < NE; e += 4) {
+      float4v x = {f[e], f[e + 1], f[e + 2], f[e + 3]};
+      *reinterpret_cast<float4v*>(row_ptr + c * NE + e) = x;
+    }
+  }
+};
+
+// GenLay: any d <= 64*EPL.  One row per wave-wide load; lane c owns elements c, c+64, ...
+// Slower (scalar loads) but complete: the fallback for sizes VecLay does not cover.
+template <typename T, int EPL>
+struct GenLay {
+  using elem = T;
+  static constexpr int LPR = kWave;
+  static constexpr int GROUPS = 1;
+  static constexpr int NE = EPL;
+  static constexpr int U = (EPL <= 2) ? 8 : 2;
+  static constexpr int U_SHORT = U;
+  static constexpr bool kFixedD = false;
+  struct raw { T x[EPL]; };
+
+  __device__ static __forceinline__ raw load(const T* row_ptr, int c, int d) {
+    raw r;
+#pragma unroll
+    for (int e = 0; e < EPL; e++) {
+      int idx = c + e * kWave;
+      r.x[e] = idx < d ? row_ptr[idx] : from_f32<T>(0.f);
+    }
+    return r;
+  }
+  __device__ static __forceinline__ void unpack(const raw& r, float (&f)[NE]) {
+#pragma unroll
+    for (int e = 0; e < EPL; e++) f[e] = to_f32(r.x[e]);
+  }
+  __device__ static __forceinline__ void store(T* row_ptr, int c, int d, const float (&f)[NE]) {
+#pragma unroll
+    for (int e = 0; e < EPL; e++) {
+      int idx = c + e * kWave;
+      if (idx < d) row_ptr[idx] = from_f32<T>(f[e]);
+    }
+  }
+  __device__ static __forceinline__ void load_f32(const float* row_ptr, int c, int d, float (&f)[NE]) {
+#pragma unroll
+    for (int e = 0; e < EPL; e++) {
+      int idx = c + e * kWave;
+      f[e] = idx < d ? row_ptr[idx] : 0.f;
+    }
+  }
+  __device__ static __forceinline__ void store_f32(float* row_ptr, int c, int d, const float (&f)[NE]) {
+#pragma unroll
+    for (int e = 0; e < EPL; e++) {
+      int idx = c + e * kWave;
+      if (idx < d) row_ptr[idx] = f[e];
+    }
+  }
+};
+
+__device__ __forceinline__ int lane_id() {
+  return (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+}
+
+}  // namespace spfa

@@ -1,0 +1,488 @@
+// Row-gather attention engine for gfx950 (wave64).
+//
+// A mask is a functor that answers two questions for a query row: how many candidate columns
+// it has (deg) and which column the t-th candidate is.  The engine walks those candidates with
+// an online softmax.  Work decomposition:
+//
+//   rows_kernel      one group of LPR lanes per query row (64/LPR rows per wavefront).  Rows
+//                    with deg <= short_max are finished on the spot; longer rows are cut into
+//                    segments of `seg` candidates that are appended to a work list.
+//   segments_kernel  persistent grid; each wavefront pulls segments off the work list, its
+//                    64/LPR groups take interleaved candidates, the groups are merged with
+//                    cross-lane moves, and the result is either final (single-segment row) or a
+//                    partial (m, l, acc[d]) in the workspace.
+//   merge_kernel     one group per multi-segment row folds that row's partials together.
+//
+// All three finish a row the same way: fold the incoming (m, l, out) state in, write back.
+#pragma once
+
+#include "spfa_common.hpp"
+#include "spfa_prep.hpp"
+
+namespace spfa {
+
+struct Tensors {
+  const void* q;
+  const void* k;
+  const void* v;
+  void* m;
+  void* l;
+  void* out;
+  int64_t n_q;
+  int32_t d;
+  int32_t state_f32;
+};
+
+struct Counters {
+  uint32_t n_items;
+  uint32_t n_partials;
+  uint32_t n_multi;
+  uint32_t next_item;
+  uint32_t overflow;
+  uint32_t pad[3];
+};
+
+struct Item {
+  int32_t row;
+  int32_t seg;
+  int32_t slot;  // partial slot, or -1 when the row has a single segment
+  int32_t pad;
+};
+
+struct MultiRow {
+  int32_t row;
+  int32_t slot0;
+  int32_t nseg;
+  int32_t pad;
+};
+
+struct Plan {
+  Counters* cnt;
+  Item* items;
+  MultiRow* multi;
+  float* pm;
+  float* pl;
+  float* pacc;
+  uint32_t cap_items;
+  uint32_t cap_partials;
+  uint32_t cap_multi;
+  int32_t use_nan;
+  int64_t short_max;
+  int64_t seg;
+};
+
+static __global__ void reset_counters_kernel(Counters* cnt) {
+  if (threadIdx.x == 0) {
+    cnt->n_items = 0;
+    cnt->n_partials = 0;
+    cnt->n_multi = 0;
+    cnt->next_item = 0;
+    cnt->overflow = 0;
+  }
+}
+
+// Fold partial B into partial A (both un-normalised, relative to their own running max).
+template <int NE>
+__device__ __forceinline__ void merge_partial(float& m, float& l, float (&acc)[NE], float m2,
+                                              float l2, const float (&acc2)[NE]) {
+  float m_new = fmaxf(m, m2);
+  if (m_new == kNegInf) return;
+  float a = __expf(m - m_new);
+  float b = __expf(m2 - m_new);
+  l = l * a + l2 * b;
+#pragma unroll
+  for (int e = 0; e < NE; e++) acc[e] = acc[e] * a + acc2[e] * b;
+  m = m_new;
+}
+
+// Candidates t_begin, t_begin + t_stride, ... < t_end of one row, U at a time.  All K and V
+// rows of a batch are requested before any of them is consumed.
+template <class Lay, class Mask, int U>
+__device__ __forceinline__ void attend(const Mask& mask, const typename Mask::Row& rc,
+                                       const typename Lay::elem* __restrict__ K,
+                                       const typename Lay::elem* __restrict__ V, int d, float scale,
+                                       const float (&q)[Lay::NE], int64_t t_begin, int64_t t_end,
+                                       int64_t t_stride, int c, float& m, float& l,
+                                       float (&acc)[Lay::NE]) {
+  constexpr int NE = Lay::NE;
+  for (int64_t t0 = t_begin; t0 < t_end; t0 += (int64_t)U * t_stride) {
+    typename Lay::raw kr[U], vr[U];
+    bool ok[U];
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+      int64_t t = t0 + u * t_stride;
+      ok[u] = t < t_end;
+      if (ok[u]) {
+        bool valid = true;
+        int64_t col = mask.col(rc, t, valid);
+        ok[u] = valid;
+        if (valid) {
+          kr[u] = Lay::load(K + col * d, c, d);
+          vr[u] = Lay::load(V + col * d, c, d);
+        }
+      }
+    }
+    float s[U];
+    float mb = kNegInf;
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+      float part = 0.f;
+      if (ok[u]) {
+        float kf[NE];
+        Lay::unpack(kr[u], kf);
+#pragma unroll
+        for (int e = 0; e < NE; e++) part += q[e] * kf[e];
+      }
+      float tot = group_sum<Lay::LPR>(part) * scale;
+      s[u] = ok[u] ? tot : kNegInf;
+      mb = fmaxf(mb, s[u]);
+    }
+    if (mb > kNegInf) {
+      float m_new = fmaxf(m, mb);
+      float corr = __expf(m - m_new);
+      l *= corr;
+#pragma unroll
+      for (int e = 0; e < NE; e++) acc[e] *= corr;
+#pragma unroll
+      for (int u = 0; u < U; u++) {
+        if (ok[u]) {
+          float p = __expf(s[u] - m_new);
+          l += p;
+          float vf[NE];
+          Lay::unpack(vr[u], vf);
+#pragma unroll
+          for (int e = 0; e < NE; e++) acc[e] += p * vf[e];
+        }
+      }
+      m = m_new;
+    }
+  }
+}
+
+// Fold the state already in memory into (m, l, acc) and write the row back.  A row that saw
+// no live column (l == 0) is left untouched.
+template <class Lay>
+__device__ __forceinline__ void finish_row(const Tensors& t, int64_t row, int c, float m, float l,
+                                           float (&acc)[Lay::NE]) {
+  using T = typename Lay::elem;
+  constexpr int NE = Lay::NE;
+  if (!(l > 0.f)) return;
+  const bool sf = t.state_f32 != 0;
+  float m_in = load_state<T>(t.m, row, sf);
+  float l_in = load_state<T>(t.l, row, sf);
+  T* orow = (T*)t.out + row * t.d;
+  float m_new = m, l_new = l;
+  if (l_in != 0.f) {
+    float o_in[NE];
+    typename Lay::raw r = Lay::load(orow, c, t.d);
+    Lay::unpack(r, o_in);
+    m_new = fmaxf(m, m_in);
+    float wa = l_in * __expf(m_in - m_new);
+    float wb = __expf(m - m_new);
+    l_new = wa + l * wb;
+    float inv = 1.f / l_new;
+#pragma unroll
+    for (int e = 0; e < NE; e++) acc[e] = (wa * o_in[e] + wb * acc[e]) * inv;
+  } else {
+    float inv = 1.f / l;
+#pragma unroll
+    for (int e = 0; e < NE; e++) acc[e] *= inv;
+  }
+  Lay::store(orow, c, t.d, acc);
+  if (c == 0) {
+    store_state<T>(t.m, row, m_new, sf);
+    store_state<T>(t.l, row, l_new, sf);
+  }
+}
+
+template <class Lay>
+__device__ __forceinline__ void load_q(const Tensors& t, int64_t row, int c, float (&q)[Lay::NE]) {
+  using T = typename Lay::elem;
+  typename Lay::raw r = Lay::load((const T*)t.q + row * t.d, c, t.d);
+  Lay::unpack(r, q);
+}
+
+template <class Lay, class Mask>
+__global__ __launch_bounds__(256) void rows_kernel(Tensors t, Mask mask, Plan plan) {
+  using T = typename Lay::elem;
+  constexpr int NE = Lay::NE;
+  constexpr int LPR = Lay::LPR;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x >> 6;
+  const int g = lane / LPR;
+  const int c = lane % LPR;
+  const int64_t row = ((int64_t)blockIdx.x * 4 + wave) * Lay::GROUPS + g;
+  if (row >= t.n_q) return;
+
+  const typename Mask::Row rc = mask.row(row);
+  const int64_t deg = rc.deg;
+  if (deg <= 0) {
+    if (plan.use_nan) {
+      float nanv[NE];
+#pragma unroll
+      for (int e = 0; e < NE; e++) nanv[e] = __builtin_nanf("");
+      Lay::store((T*)t.out + row * t.d, c, t.d, nanv);
+    }
+    return;
+  }
+
+  if (deg <= plan.short_max) {
+    float q[NE];
+    load_q<Lay>(t, row, c, q);
+    float m = kNegInf, l = 0.f, acc[NE];
+#pragma unroll
+    for (int e = 0; e < NE; e++) acc[e] = 0.f;
+    const float scale = 1.0f / sqrtf((float)t.d);
+    attend<Lay, Mask, Lay::U_SHORT>(mask, rc, (const T*)t.k, (const T*)t.v, t.d, scale, q, 0, deg, 1,
+                                    c, m, l, acc);
+    finish_row<Lay>(t, row, c, m, l, acc);
+    return;
+  }
+
+  // long row: hand its segments to the work list
+  const uint32_t nseg = (uint32_t)((deg + plan.seg - 1) / plan.seg);
+  uint32_t base = 0, slot0 = 0;
+  int okw = 1;
+  if (c == 0) {
+    base = atomicAdd(&plan.cnt->n_items, nseg);
+    if (base + nseg > plan.cap_items) okw = 0;
+    if (nseg > 1) {
+      slot0 = atomicAdd(&plan.cnt->n_partials, nseg);
+      uint32_t mp = atomicAdd(&plan.cnt->n_multi, 1u);
+      if (slot0 + nseg > plan.cap_partials || mp >= plan.cap_multi) okw = 0;
+      if (okw) {
+        MultiRow mr;
+        mr.row = (int32_t)row;
+        mr.slot0 = (int32_t)slot0;
+        mr.nseg = (int32_t)nseg;
+        mr.pad = 0;
+        plan.multi[mp] = mr;
+      }
+    }
+    if (!okw) atomicOr(&plan.cnt->overflow, 1u);
+  }
+  const int leader = g * LPR;
+  base = (uint32_t)shfl_i32((int)base, leader);
+  slot0 = (uint32_t)shfl_i32((int)slot0, leader);
+  okw = shfl_i32(okw, leader);
+  if (!okw) return;
+  for (uint32_t j = c; j < nseg; j += LPR) {
+    Item it;
+    it.row = (int32_t)row;
+    it.seg = (int32_t)j;
+    it.slot = nseg > 1 ? (int32_t)(slot0 + j) : -1;
+    it.pad = 0;
+    plan.items[base + j] = it;
+  }
+}
+
+template <class Lay, class Mask>
+__global__ __launch_bounds__(256) void segments_kernel(Tensors t, Mask mask, Plan plan) {
+  using T = typename Lay::elem;
+  constexpr int NE = Lay::NE;
+  constexpr int LPR = Lay::LPR;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int g = lane / LPR;
+  const int c = lane % LPR;
+  if (plan.cnt->overflow) return;
+  uint32_t n_items = plan.cnt->n_items;
+  if (n_items > plan.cap_items) n_items = plan.cap_items;
+  const float scale = 1.0f / sqrtf((float)t.d);
+
+  while (true) {
+    uint32_t idx = 0;
+    if (lane == 0) idx = atomicAdd(&plan.cnt->next_item, 1u);
+    idx = (uint32_t)__builtin_amdgcn_readfirstlane((int)idx);
+    if (idx >= n_items) break;
+    const Item it = plan.items[idx];
+    const int64_t row = it.row;
+    const typename Mask::Row rc = mask.row(row);
+    const int64_t t0 = (int64_t)it.seg * plan.seg;
+    int64_t t1 = t0 + plan.seg;
+    if (t1 > rc.deg) t1 = rc.deg;
+
+    float q[NE];
+    load_q<Lay>(t, row, c, q);
+    float m = kNegInf, l = 0.f, acc[NE];
+#pragma unroll
+    for (int e = 0; e < NE; e++) acc[e] = 0.f;
+    attend<Lay, Mask, Lay::U>(mask, rc, (const T*)t.k, (const T*)t.v, t.d, scale, q, t0 + g, t1,
+                              Lay::GROUPS, c, m, l, acc);
+
+    // butterfly over the groups of the wavefront
+#pragma unroll
+    for (int off = LPR; off < kWave; off <<= 1) {
+      float m2 = shfl_xor_f32(m, off);
+      float l2 = shfl_xor_f32(l, off);
+      float acc2[NE];
+#pragma unroll
+      for (int e = 0; e < NE; e++) acc2[e] = shfl_xor_f32(acc[e], off);
+      merge_partial<NE>(m, l, acc, m2, l2, acc2);
+    }
+
+    if (g == 0) {
+      if (it.slot < 0) {
+        finish_row<Lay>(t, row, c, m, l, acc);
+      } else {
+        Lay::store_f32(plan.pacc + (int64_t)it.slot * t.d, c, t.d, acc);
+        if (c == 0) {
+          plan.pm[it.slot] = m;
+          plan.pl[it.slot] = l;
+        }
+      }
+    }
+    // Every lane of the wavefront must take the next trip together: the work index is read
+    // across lanes at the top of the loop.  A convergent operation in the only latch keeps the
+    // optimiser from giving the lanes that wrote the statistics a back edge of their own.
+    __builtin_amdgcn_wave_barrier();
+  }
+}
+
+template <class Lay>
+__global__ __launch_bounds__(256) void merge_kernel(Tensors t, Plan plan) {
+  constexpr int NE = Lay::NE;
+  constexpr int LPR = Lay::LPR;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x >> 6;
+  const int g = lane / LPR;
+  const int c = lane % LPR;
+  if (plan.cnt->overflow) return;
+  uint32_t n_multi = plan.cnt->n_multi;
+  if (n_multi > plan.cap_multi) n_multi = plan.cap_multi;
+  const int64_t idx = ((int64_t)blockIdx.x * 4 + wave) * Lay::GROUPS + g;
+  if (idx >= (int64_t)n_multi) return;
+  const MultiRow mr = plan.multi[idx];
+  float m = kNegInf, l = 0.f, acc[NE];
+#pragma unroll
+  for (int e = 0; e < NE; e++) acc[e] = 0.f;
+  for (int j = 0; j < mr.nseg; j++) {
+    const int64_t slot = (int64_t)mr.slot0 + j;
+    float acc2[NE];
+    Lay::load_f32(plan.pacc + slot * t.d, c, t.d, acc2);
+    merge_partial<NE>(m, l, acc, plan.pm[slot], plan.pl[slot], acc2);
+  }
+  finish_row<Lay>(t, mr.row, c, m, l, acc);
+}
+
+// ---------------------------------------------------------------------------------------
+// host side
+// ---------------------------------------------------------------------------------------
+struct EngineSizing {
+  int64_t nnz_bound;     // upper bound on the sum of deg over all rows
+  int64_t max_deg;       // upper bound on deg of one row
+  int64_t short_max;     // rows up to this many candidates are finished by rows_kernel
+  int64_t seg;           // segment length for longer rows
+  int64_t n_long_bound;  // upper bound on the number of rows with deg > short_max
+};
+
+struct WorkspaceLayout {
+  size_t off_cnt, off_items, off_multi, off_pm, off_pl, off_pacc, total;
+  uint32_t cap_items, cap_partials, cap_multi;
+};
+
+
+inline int64_t pow2_ceil(int64_t x) {
+  int64_t p = 1;
+  while (p < x) p <<= 1;
+  return p;
+}
+
+inline WorkspaceLayout engine_workspace(const EngineSizing& s, int64_t n_q, int64_t d) {
+  WorkspaceLayout w{};
+  int64_t cap_items = 0, cap_partials = 0, cap_multi = 0;
+  if (s.max_deg > s.short_max) {
+    int64_t n_long = s.nnz_bound / (s.short_max + 1);
+    if (n_long > n_q) n_long = n_q;
+    if (n_long > s.n_long_bound) n_long = s.n_long_bound;
+    cap_items = s.nnz_bound / s.seg + n_long + 1;
+    int64_t n_multi = s.nnz_bound / (s.seg + 1);
+    if (n_multi > n_long) n_multi = n_long;
+    cap_multi = n_multi + 1;
+    cap_partials = s.nnz_bound / s.seg + n_multi + 1;
+  }
+  w.cap_items = (uint32_t)cap_items;
+  w.cap_partials = (uint32_t)cap_partials;
+  w.cap_multi = (uint32_t)cap_multi;
+  size_t off = 0;
+  w.off_cnt = off;      off = align_up(off + sizeof(Counters), 256);
+  w.off_items = off;    off = align_up(off + (size_t)cap_items * sizeof(Item), 256);
+  w.off_multi = off;    off = align_up(off + (size_t)cap_multi * sizeof(MultiRow), 256);
+  w.off_pm = off;       off = align_up(off + (size_t)cap_partials * sizeof(float), 256);
+  w.off_pl = off;       off = align_up(off + (size_t)cap_partials * sizeof(float), 256);
+  w.off_pacc = off;     off = align_up(off + (size_t)cap_partials * (size_t)d * sizeof(float), 256);
+  w.total = off;
+  return w;
+}
+
+inline int device_cu_count() {
+  static int cus = 0;
+  if (cus == 0) {
+    int dev = 0;
+    hipDeviceProp_t prop;
+    if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
+      cus = prop.multiProcessorCount;
+    if (cus <= 0) cus = 256;
+  }
+  return cus;
+}
+
+template <class Lay, class Mask>
+int launch_engine(const Tensors& t, const Mask& mask, const EngineSizing& s, int use_nan, void* ws,
+                  hipStream_t stream) {
+  WorkspaceLayout w = engine_workspace(s, t.n_q, t.d);
+  char* base = (char*)ws;
+  Plan plan{};
+  plan.cnt = (Counters*)(base + w.off_cnt);
+  plan.items = (Item*)(base + w.off_items);
+  plan.multi = (MultiRow*)(base + w.off_multi);
+  plan.pm = (float*)(base + w.off_pm);
+  plan.pl = (float*)(base + w.off_pl);
+  plan.pacc = (float*)(base + w.off_pacc);
+  plan.cap_items = w.cap_items;
+  plan.cap_partials = w.cap_partials;
+  plan.cap_multi = w.cap_multi;
+  plan.use_nan = use_nan;
+  plan.short_max = s.short_max;
+  plan.seg = s.seg;
+  if (t.n_q == 0) return 0;
+
+  const bool has_long = s.max_deg > s.short_max;
+  if (has_long) hipLaunchKernelGGL(reset_counters_kernel, dim3(1), dim3(64), 0, stream, plan.cnt);
+
+  const int64_t rows_per_wg = 4 * Lay::GROUPS;
+  const int64_t grid1 = (t.n_q + rows_per_wg - 1) / rows_per_wg;
+  hipLaunchKernelGGL((rows_kernel<Lay, Mask>), dim3((unsigned)grid1), dim3(256), 0, stream, t, mask,
+                     plan);
+  if (has_long) {
+    int64_t grid2 = (int64_t)device_cu_count() * 8;
+    int64_t need = ((int64_t)w.cap_items + 3) / 4;
+    if (grid2 > need) grid2 = need;
+    if (grid2 < 1) grid2 = 1;
+    hipLaunchKernelGGL((segments_kernel<Lay, Mask>), dim3((unsigned)grid2), dim3(256), 0, stream, t,
+                       mask, plan);
+    const int64_t grid3 = ((int64_t)w.cap_multi + rows_per_wg - 1) / rows_per_wg;
+    hipLaunchKernelGGL((merge_kernel<Lay>), dim3((unsigned)grid3), dim3(256), 0, stream, t, plan);
+  }
+  return hipGetLastError() == hipSuccess ? 0 : 4;
+}
+
+inline bool aligned16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
+
+// Pick the lane layout for (T, d).
+template <typename T, class Mask>
+int run_engine(const Tensors& t, const Mask& mask, const EngineSizing& s, int use_nan, void* ws,
+               hipStream_t stream) {
+  const int64_t row_bytes = (int64_t)t.d * (int64_t)sizeof(T);
+  const bool vec_ok = aligned16(t.q) && aligned16(t.k) && aligned16(t.v) && aligned16(t.out);
+  if (vec_ok) {
+    if (row_bytes == 64) return launch_engine<VecLay<T, 4>, Mask>(t, mask, s, use_nan, ws, stream);
+    if (row_bytes == 128) return launch_engine<VecLay<T, 8>, Mask>(t, mask, s, use_nan, ws, stream);
+    if (row_bytes == 256) return launch_engine<VecLay<T, 16>, Mask>(t, mask, s, use_nan, ws, stream);
+    if (row_bytes == 512) return launch_engine<VecLay<T, 32>, Mask>(t, mask, s, use_nan, ws, stream);
+  }
+  if (t.d <= 128) return launch_engine<GenLay<T, 2>, Mask>(t, mask, s, use_nan, ws, stream);
+  if (t.d <= 1024) return launch_engine<GenLay<T, 16>, Mask>(t, mask, s, use_nan, ws, stream);
+  return 5;
+}
+
+}  // namespace spfa

@@ -1,0 +1,19 @@
+// Entry points of the per-(mask, element type) translation units.
+#pragma once
+
+#include "spfa_engine.hpp"
+#include "spfa_masks.hpp"
+
+namespace spfa {
+
+template <typename T>
+int run_csr(const Tensors& t, const CsrMask& mask, const EngineSizing& s, int use_nan, void* ws,
+            hipStream_t stream);
+template <typename T>
+int run_stride(const Tensors& t, const StrideMask& mask, const EngineSizing& s, int use_nan,
+               void* ws, hipStream_t stream);
+template <typename T>
+int run_global(const Tensors& t, const GlobalMask& mask, const EngineSizing& s, int use_nan,
+               void* ws, hipStream_t stream);
+
+}  // namespace spfa

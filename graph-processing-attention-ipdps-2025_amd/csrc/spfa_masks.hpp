@@ -1,0 +1,105 @@
+// Mask functors for the row-gather engine.  Each answers, for query row i,
+//   row(i)        -> the row's candidate count (deg) plus whatever col() needs, and
+//   col(rc, t, v) -> the column of candidate t (v := false if that candidate is masked).
+#pragma once
+
+#include "spfa_common.hpp"
+
+namespace spfa {
+
+// Explicit CSR adjacency: row i owns col_ind[row_off[i] .. row_off[i+1])
+// (reference: Sparse_FlashAttention_CSR/sp_flatt_csr_kernel.cu:29-33,117).
+struct CsrMask {
+  const void* row_off;
+  const uint32_t* cols;
+  int32_t off64;  // row_off entries are 8 bytes wide (else 4)
+  struct Row {
+    int64_t start;
+    int64_t deg;
+  };
+  __device__ __forceinline__ Row row(int64_t i) const {
+    int64_t a, b;
+    if (off64) {
+      const uint64_t* p = (const uint64_t*)row_off;
+      a = (int64_t)p[i];
+      b = (int64_t)p[i + 1];
+    } else {
+      const uint32_t* p = (const uint32_t*)row_off;
+      a = (int64_t)p[i];
+      b = (int64_t)p[i + 1];
+    }
+    return Row{a, b - a};
+  }
+  __device__ __forceinline__ int64_t col(const Row& r, int64_t t, bool&) const {
+    return (int64_t)cols[r.start + t];
+  }
+};
+
+// Strided runs: candidate t of row i is low(i) + t*s.
+//   block == 0: band.  low = max(i - w*s, i mod s), up = min(i + w*s, n-1), deg = (up-low)/s + 1
+//               (Sparse_FlashAttention_Local_1D_Dilated/sp_flatt_local_1d_dilated_kernel.cu:25-29,102;
+//               with s == 1 this is Sparse_FlashAttention_Local/sp_flatt_local_kernel.cu:24-28,101).
+//   block  > 0: block-diagonal with 2-D dilation.  low = (i / block) * block; the row is live
+//               only when (i - low) mod s == 0, then deg = cnt = min(block, (block-1)/s + 1)
+//               (Sparse_FlashAttention_Local_2D_Dilated/sp_flatt_local_2d_dilated_kernel.cu:26-39,123).
+struct StrideMask {
+  int64_t n;
+  int64_t w;
+  int64_t s;
+  int64_t block;
+  int64_t cnt;
+  struct Row {
+    int64_t low;
+    int64_t deg;
+  };
+  __device__ __forceinline__ Row row(int64_t i) const {
+    if (block > 0) {
+      int64_t low = (i / block) * block;
+      return Row{low, ((i - low) % s == 0) ? cnt : 0};
+    }
+    int64_t low = i - w * s;
+    int64_t r = i % s;
+    if (low < r) low = r;
+    int64_t up = i + w * s;
+    if (up > n - 1) up = n - 1;
+    return Row{low, (up - low) / s + 1};
+  }
+  __device__ __forceinline__ int64_t col(const Row& r, int64_t t, bool&) const {
+    return r.low + t * s;
+  }
+};
+
+// Global minus local window [low, up) = [max(0, i-w), min(n, i+w+1)):
+//   global row: candidates are all n - (up-low) columns outside the window;
+//   other rows: candidates are the n_globs listed indices, those inside the window are masked
+//   (Sparse_FlashAttention_Global_No_Local/sp_flatt_global_no_local_kernel.cu:38-64,134-162).
+// is_global[i] != 0 marks the listed rows.
+struct GlobalMask {
+  int64_t n;
+  int64_t w;
+  const int32_t* globs;
+  int64_t n_globs;
+  const uint8_t* is_global;
+  struct Row {
+    int64_t low;
+    int64_t up;
+    int64_t deg;
+    bool glob;
+  };
+  __device__ __forceinline__ Row row(int64_t i) const {
+    int64_t low = i - w;
+    if (low < 0) low = 0;
+    int64_t up = i + w + 1;
+    if (up > n) up = n;
+    bool glob = is_global[i] != 0;
+    return Row{low, up, glob ? n - (up - low) : n_globs, glob};
+  }
+  __device__ __forceinline__ int64_t col(const Row& r, int64_t t, bool& valid) const {
+    if (r.glob) return t < r.low ? t : t + (r.up - r.low);
+    int64_t c = (int64_t)globs[t];
+    valid = (c < r.low) || (c >= r.up);
+    return c;
+  }
+};
+
+}  // namespace spfa

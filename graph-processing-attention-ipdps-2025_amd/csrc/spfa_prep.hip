@@ -1,0 +1,210 @@
+// Mask pre-passes that run on the device before the attention kernels:
+//   - COO entries -> row buckets (histogram, exclusive scan, scatter), any entry order;
+//   - global-token list -> per-row flag bytes.
+#include "spfa_prep.hpp"
+
+#include "spfa_common.hpp"
+
+namespace spfa {
+
+namespace {
+
+constexpr int kScanThreads = 256;
+constexpr int kScanPerThread = 8;
+constexpr int kScanTile = kScanThreads * kScanPerThread;
+
+__global__ void fill_u32_kernel(uint32_t* p, int64_t n, uint32_t value) {
+  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (; i < n; i += stride) p[i] = value;
+}
+
+__device__ __forceinline__ int64_t load_index(const void* p, int64_t i, int wide) {
+  return wide ? (int64_t)((const uint64_t*)p)[i] : (int64_t)((const uint32_t*)p)[i];
+}
+
+__global__ void coo_histogram_kernel(const void* row_ind, int wide, int64_t nnz, int64_t n_rows,
+                                     uint32_t* counts) {
+  int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (; e < nnz; e += stride) {
+    int64_t r = load_index(row_ind, e, wide);
+    if (r >= 0 && r < n_rows) atomicAdd(&counts[r], 1u);
+  }
+}
+
+__global__ void coo_scatter_kernel(const void* row_ind, int wide, const uint32_t* col_ind,
+                                   int64_t nnz, int64_t n_rows, uint32_t* cursor,
+                                   uint32_t* cols_out) {
+  int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (; e < nnz; e += stride) {
+    int64_t r = load_index(row_ind, e, wide);
+    if (r >= 0 && r < n_rows) {
+      uint32_t pos = atomicAdd(&cursor[r], 1u);
+      cols_out[pos] = col_ind[e];
+    }
+  }
+}
+
+// inclusive scan over the wavefront
+__device__ __forceinline__ uint32_t wave_inclusive_scan(uint32_t x, int lane) {
+#pragma unroll
+  for (int off = 1; off < kWave; off <<= 1) {
+    uint32_t y = (uint32_t)__builtin_amdgcn_ds_bpermute(((lane - off) & 63) << 2, (int)x);
+    if (lane >= off) x += y;
+  }
+  return x;
+}
+
+// exclusive scan of one value per thread over a 256-thread block; returns the thread's prefix
+// and the block total
+__device__ __forceinline__ uint32_t block_exclusive_scan(uint32_t x, uint32_t& total,
+                                                         uint32_t* lds /*[4]*/) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  uint32_t inc = wave_inclusive_scan(x, lane);
+  if (lane == 63) lds[wave] = inc;
+  __syncthreads();
+  uint32_t wave_prefix = 0, tot = 0;
+#pragma unroll
+  for (int w = 0; w < kScanThreads / kWave; w++) {
+    uint32_t s = lds[w];
+    if (w < wave) wave_prefix += s;
+    tot += s;
+  }
+  __syncthreads();
+  total = tot;
+  return wave_prefix + inc - x;
+}
+
+__global__ __launch_bounds__(kScanThreads) void scan_tile_sums_kernel(const uint32_t* in, int64_t n,
+                                                                      uint32_t* tile_sums) {
+  __shared__ uint32_t lds[4];
+  const int64_t base = (int64_t)blockIdx.x * kScanTile + (int64_t)threadIdx.x * kScanPerThread;
+  uint32_t s = 0;
+#pragma unroll
+  for (int j = 0; j < kScanPerThread; j++)
+    if (base + j < n) s += in[base + j];
+  uint32_t total;
+  block_exclusive_scan(s, total, lds);
+  if (threadIdx.x == 0) tile_sums[blockIdx.x] = total;
+}
+
+// single block: exclusive scan of the tile sums in place
+__global__ __launch_bounds__(kScanThreads) void scan_sums_kernel(uint32_t* tile_sums, int64_t n_tiles) {
+  __shared__ uint32_t lds[4];
+  uint32_t carry = 0;
+  for (int64_t base = 0; base < n_tiles; base += kScanThreads) {
+    int64_t i = base + threadIdx.x;
+    uint32_t x = i < n_tiles ? tile_sums[i] : 0u;
+    uint32_t total;
+    uint32_t ex = block_exclusive_scan(x, total, lds);
+    if (i < n_tiles) tile_sums[i] = carry + ex;
+    carry += total;
+  }
+}
+
+// exclusive scan of in[0..n) into out[0..n) and out2[0..n); out[n] = out2[n] = grand total is
+// written by the block that owns element n-1
+__global__ __launch_bounds__(kScanThreads) void scan_apply_kernel(const uint32_t* in, int64_t n,
+                                                                  const uint32_t* tile_sums,
+                                                                  uint32_t* out, uint32_t* out2) {
+  __shared__ uint32_t lds[4];
+  const int64_t base = (int64_t)blockIdx.x * kScanTile + (int64_t)threadIdx.x * kScanPerThread;
+  uint32_t v[kScanPerThread];
+  uint32_t s = 0;
+#pragma unroll
+  for (int j = 0; j < kScanPerThread; j++) {
+    v[j] = (base + j < n) ? in[base + j] : 0u;
+    s += v[j];
+  }
+  uint32_t total;
+  uint32_t run = block_exclusive_scan(s, total, lds) + tile_sums[blockIdx.x];
+#pragma unroll
+  for (int j = 0; j < kScanPerThread; j++) {
+    if (base + j < n) {
+      out[base + j] = run;
+      out2[base + j] = run;
+    }
+    run += v[j];
+    if (base + j == n - 1) {
+      out[n] = run;
+      out2[n] = run;
+    }
+  }
+}
+
+__global__ void mark_globals_kernel(const int32_t* globs, int64_t n_globs, int64_t n,
+                                    uint8_t* flags) {
+  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n_globs) {
+    int64_t g = globs[i];
+    if (g >= 0 && g < n) flags[g] = 1;
+  }
+}
+
+inline unsigned grid_for(int64_t n, int threads, int64_t cap) {
+  int64_t g = (n + threads - 1) / threads;
+  if (g > cap) g = cap;
+  if (g < 1) g = 1;
+  return (unsigned)g;
+}
+
+}  // namespace
+
+CooWorkspace coo_workspace(int64_t n_rows, int64_t nnz) {
+  CooWorkspace w{};
+  const int64_t n_tiles = (n_rows + kScanTile - 1) / kScanTile + 1;
+  size_t off = 0;
+  w.off_counts = off;  off = align_up(off + (size_t)(n_rows + 1) * 4, 256);
+  w.off_row_off = off; off = align_up(off + (size_t)(n_rows + 1) * 4, 256);
+  w.off_cursor = off;  off = align_up(off + (size_t)(n_rows + 1) * 4, 256);
+  w.off_tiles = off;   off = align_up(off + (size_t)n_tiles * 4, 256);
+  w.off_cols = off;    off = align_up(off + (size_t)(nnz > 0 ? nnz : 1) * 4, 256);
+  w.total = off;
+  return w;
+}
+
+int coo_bucket_by_row(const void* row_ind, int row_wide, const uint32_t* col_ind, int64_t nnz,
+                      int64_t n_rows, void* ws, hipStream_t stream, const uint32_t** row_off_out,
+                      const uint32_t** cols_out) {
+  CooWorkspace w = coo_workspace(n_rows, nnz);
+  char* base = (char*)ws;
+  uint32_t* counts = (uint32_t*)(base + w.off_counts);
+  uint32_t* row_off = (uint32_t*)(base + w.off_row_off);
+  uint32_t* cursor = (uint32_t*)(base + w.off_cursor);
+  uint32_t* tiles = (uint32_t*)(base + w.off_tiles);
+  uint32_t* cols = (uint32_t*)(base + w.off_cols);
+  const int64_t n_tiles = (n_rows + kScanTile - 1) / kScanTile;
+
+  hipLaunchKernelGGL(fill_u32_kernel, dim3(grid_for(n_rows + 1, 256, 4096)), dim3(256), 0, stream,
+                     counts, n_rows + 1, 0u);
+  if (nnz > 0)
+    hipLaunchKernelGGL(coo_histogram_kernel, dim3(grid_for(nnz, 256, 16384)), dim3(256), 0, stream,
+                       row_ind, row_wide, nnz, n_rows, counts);
+  if (n_rows > 0) {
+    hipLaunchKernelGGL(scan_tile_sums_kernel, dim3((unsigned)n_tiles), dim3(kScanThreads), 0, stream,
+                       counts, n_rows, tiles);
+    hipLaunchKernelGGL(scan_sums_kernel, dim3(1), dim3(kScanThreads), 0, stream, tiles, n_tiles);
+    hipLaunchKernelGGL(scan_apply_kernel, dim3((unsigned)n_tiles), dim3(kScanThreads), 0, stream,
+                       counts, n_rows, tiles, row_off, cursor);
+  }
+  if (nnz > 0)
+    hipLaunchKernelGGL(coo_scatter_kernel, dim3(grid_for(nnz, 256, 16384)), dim3(256), 0, stream,
+                       row_ind, row_wide, col_ind, nnz, n_rows, cursor, cols);
+  *row_off_out = row_off;
+  *cols_out = cols;
+  return hipGetLastError() == hipSuccess ? 0 : 4;
+}
+
+int mark_global_rows(const int32_t* globs, int64_t n_globs, int64_t n, uint8_t* flags,
+                     hipStream_t stream) {
+  const int64_t words = (n + 3) / 4;
+  hipLaunchKernelGGL(fill_u32_kernel, dim3(grid_for(words, 256, 4096)), dim3(256), 0, stream,
+                     (uint32_t*)flags, words, 0u);
+  hipLaunchKernelGGL(mark_globals_kernel, dim3(grid_for(n_globs, 256, 1 << 30)), dim3(256), 0,
+                     stream, globs, n_globs, n, flags);
+  return hipGetLastError() == hipSuccess ? 0 : 4;
+}
+
+}  // namespace spfa

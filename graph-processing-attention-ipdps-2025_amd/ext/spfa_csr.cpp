@@ -1,0 +1,42 @@
+// Python module spfa_csr: forward(q, k, v, w_row_off, w_col_ind, w_val, m, l, out, use_nan).
+// Host wrapper with the reference binding's signature and checks
+// (Sparse_FlashAttention_CSR/sp_flatt_csr.cpp:28-59); the work is done by spfa_csr_forward in
+// libspfa_hip.so.
+#include "spfa_ext_common.h"
+
+torch::Tensor spfa_csr_forward_py(torch::Tensor Q, torch::Tensor K, torch::Tensor V,
+                                  torch::Tensor W_row_off, torch::Tensor W_col_ind,
+                                  torch::Tensor W_val, torch::Tensor m, torch::Tensor l,
+                                  torch::Tensor O, bool use_nan) {
+  CHECK_INPUT(Q);
+  CHECK_INPUT(K);
+  CHECK_INPUT(V);
+  CHECK_INPUT(W_row_off);
+  CHECK_INPUT(W_col_ind);
+  CHECK_INPUT(W_val);
+  CHECK_INPUT(m);
+  CHECK_INPUT(l);
+  CHECK_INPUT(O);
+
+  c10::DeviceGuard guard(Q.device());
+  spfa_problem_t p = spfa_ext::make_problem(Q, K, V, m, l, O);
+  TORCH_CHECK(W_row_off.dim() == 1 && W_row_off.size(0) == Q.size(0) + 1,
+              "W_row_off must hold rows+1 offsets");
+  TORCH_CHECK(W_col_ind.dim() == 1, "W_col_ind must be 1-D");
+  // the value vector is type-checked and otherwise unused, as in the reference kernel
+  TORCH_CHECK(W_val.scalar_type() == Q.scalar_type(), "W_val must have the dtype of Q");
+  const int off_bytes = spfa_ext::index_bytes(W_row_off, "W_row_off", true);
+  spfa_ext::index_bytes(W_col_ind, "W_col_ind", false);
+  const int64_t nnz = W_col_ind.size(0);
+
+  const size_t ws_bytes = spfa_csr_workspace_bytes(p.n_q, nnz, p.d, p.dtype);
+  torch::Tensor ws = spfa_ext::make_workspace(ws_bytes, Q);
+  spfa_ext::raise_on_error(spfa_csr_forward(&p, W_row_off.data_ptr(), off_bytes, W_col_ind.data_ptr(),
+                                            nnz, use_nan ? 1 : 0, ws.data_ptr(), (size_t)ws.numel(),
+                                            spfa_ext::current_stream(Q)));
+  return O;
+}
+
+PYBIND11_MODULE(TORCH_EXTENSION_NAME, mod) {
+  mod.def("forward", &spfa_csr_forward_py, "Sparse-FlashAttention forward, CSR mask (HIP, gfx950)");
+}

@@ -1,0 +1,99 @@
+// Shared host-side glue of the six spfa_* Python modules: the reference bindings' tensor checks,
+// the translation torch tensor -> C-ABI problem description, workspace allocation through torch's
+// allocator, the current HIP stream, and status -> exception mapping.  No device code here.
+#pragma once
+
+#include <c10/core/DeviceGuard.h>
+#include <c10/hip/HIPStream.h>
+#include <torch/extension.h>
+
+#include <stdexcept>
+
+#include "spfa_hip.h"
+
+// Same checks and texts as the reference bindings (sp_flatt_csr.cpp:7-9).
+#define CHECK_CUDA(x) TORCH_CHECK(x.device().is_cuda(), #x " must be a CUDA tensor")
+#define CHECK_CONTIGUOUS(x) TORCH_CHECK(x.is_contiguous(), #x " must be contiguous")
+#define CHECK_INPUT(x) \
+  CHECK_CUDA(x);       \
+  CHECK_CONTIGUOUS(x)
+
+namespace spfa_ext {
+
+inline int elem_dtype(const torch::Tensor& t) {
+  switch (t.scalar_type()) {
+    case torch::kFloat32: return SPFA_DTYPE_F32;
+    case torch::kFloat16: return SPFA_DTYPE_F16;
+    case torch::kBFloat16: return SPFA_DTYPE_BF16;
+    default: return -1;  // reported by the library after the parameter checks
+  }
+}
+
+// Width in bytes of an integer index tensor; signed and unsigned are bit-identical in range.
+inline int index_bytes(const torch::Tensor& t, const char* name, bool allow_wide) {
+  switch (t.scalar_type()) {
+    case torch::kInt32:
+    case torch::kUInt32: return 4;
+    case torch::kInt64:
+    case torch::kUInt64:
+      TORCH_CHECK(allow_wide, name, " must be a 32-bit integer tensor");
+      return 8;
+    default: TORCH_CHECK(false, name, " must be an integer index tensor (got ", t.scalar_type(), ")");
+  }
+  return 0;
+}
+
+inline spfa_problem_t make_problem(const torch::Tensor& Q, const torch::Tensor& K,
+                                   const torch::Tensor& V, const torch::Tensor& m,
+                                   const torch::Tensor& l, const torch::Tensor& O) {
+  TORCH_CHECK(Q.dim() == 2 && K.dim() == 2 && V.dim() == 2 && O.dim() == 2,
+              "Q, K, V and O must be 2-D [tokens, embedding]");
+  TORCH_CHECK(m.dim() == 1 && l.dim() == 1, "m and l must be 1-D [tokens]");
+  TORCH_CHECK(K.size(1) == Q.size(1) && V.size(1) == Q.size(1) && O.size(1) == Q.size(1),
+              "Q, K, V and O must share the embedding dimension");
+  TORCH_CHECK(K.size(0) == V.size(0), "K and V must have the same number of rows");
+  TORCH_CHECK(O.size(0) == Q.size(0) && m.size(0) == Q.size(0) && l.size(0) == Q.size(0),
+              "O, m and l must have one row per row of Q");
+  TORCH_CHECK(K.scalar_type() == Q.scalar_type() && V.scalar_type() == Q.scalar_type() &&
+                  O.scalar_type() == Q.scalar_type(),
+              "Q, K, V and O must have the same dtype");
+  TORCH_CHECK(m.scalar_type() == l.scalar_type() &&
+                  (m.scalar_type() == Q.scalar_type() || m.scalar_type() == torch::kFloat32),
+              "m and l must have the dtype of Q (or float32)");
+  TORCH_CHECK(K.device() == Q.device() && V.device() == Q.device() && O.device() == Q.device() &&
+                  m.device() == Q.device() && l.device() == Q.device(),
+              "all tensors must be on the same device");
+  spfa_problem_t p;
+  p.q = Q.data_ptr();
+  p.k = K.data_ptr();
+  p.v = V.data_ptr();
+  p.m = m.data_ptr();
+  p.l = l.data_ptr();
+  p.out = O.data_ptr();
+  p.n_q = Q.size(0);
+  p.n_k = K.size(0);
+  p.d = Q.size(1);
+  p.dtype = elem_dtype(Q);
+  p.state_dtype = (m.scalar_type() == Q.scalar_type()) ? p.dtype : SPFA_DTYPE_F32;
+  return p;
+}
+
+inline torch::Tensor make_workspace(size_t bytes, const torch::Tensor& like) {
+  if (bytes < 256) bytes = 256;
+  return torch::empty({(int64_t)bytes}, torch::TensorOptions().dtype(torch::kUInt8).device(like.device()));
+}
+
+inline void* current_stream(const torch::Tensor& like) {
+  return (void*)c10::hip::getCurrentHIPStream(like.device().index()).stream();
+}
+
+// Parameter errors keep the reference's exception type (std::invalid_argument -> ValueError) and
+// text; everything else is a RuntimeError.
+inline void raise_on_error(int status) {
+  if (status == SPFA_OK) return;
+  if (status >= SPFA_ERR_EMB_TOO_LARGE && status <= SPFA_ERR_GLOBAL_COUNT)
+    throw std::invalid_argument(spfa_status_string(status));
+  TORCH_CHECK(false, spfa_status_string(status), " (status ", status, ")");
+}
+
+}  // namespace spfa_ext

@@ -1,0 +1,32 @@
+// Python module spfa_local_1d_dilated: forward(q, k, v, m, l, out, LOCAL_SIZE, DILATE_FACTOR).
+// Host wrapper with the reference binding's signature and checks
+// (Sparse_FlashAttention_Local_1D_Dilated/sp_flatt_local_1d_dilated.cpp:26-52); the work is done
+// by spfa_local_1d_dilated_forward in libspfa_hip.so.
+#include "spfa_ext_common.h"
+
+torch::Tensor spfa_local_1d_dilated_forward_py(torch::Tensor Q, torch::Tensor K, torch::Tensor V,
+                                               torch::Tensor m, torch::Tensor l, torch::Tensor O,
+                                               int local_size_each_dir, int dil_factor) {
+  CHECK_INPUT(Q);
+  CHECK_INPUT(K);
+  CHECK_INPUT(V);
+  CHECK_INPUT(m);
+  CHECK_INPUT(l);
+  CHECK_INPUT(O);
+
+  c10::DeviceGuard guard(Q.device());
+  spfa_problem_t p = spfa_ext::make_problem(Q, K, V, m, l, O);
+  TORCH_CHECK(K.size(0) == Q.size(0), "Q, K and V must have the same number of rows");
+  const size_t ws_bytes =
+      spfa_local_1d_dilated_workspace_bytes(p.n_q, p.d, p.dtype, local_size_each_dir, dil_factor);
+  torch::Tensor ws = spfa_ext::make_workspace(ws_bytes, Q);
+  spfa_ext::raise_on_error(spfa_local_1d_dilated_forward(&p, local_size_each_dir, dil_factor,
+                                                         ws.data_ptr(), (size_t)ws.numel(),
+                                                         spfa_ext::current_stream(Q)));
+  return O;
+}
+
+PYBIND11_MODULE(TORCH_EXTENSION_NAME, mod) {
+  mod.def("forward", &spfa_local_1d_dilated_forward_py,
+          "Sparse-FlashAttention forward, 1D-dilated local mask (HIP, gfx950)");
+}

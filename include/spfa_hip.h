@@ -1,0 +1,131 @@
+/*
+ * spfa_hip.h - C ABI of libspfa_hip.so: masked single-head attention on gfx950 (MI355X)
+ * that does work only on un-masked positions.
+ *
+ * One entry point per mask kind.  Each replaces the host dispatcher + device kernel pair of
+ * one reference extension (paths relative to the reference tree):
+ *
+ *   spfa_csr_forward               Sparse_FlashAttention_CSR/sp_flatt_csr_kernel.cu:14-288
+ *   spfa_coo_forward               Sparse_FlashAttention_COO/sp_flatt_coo_kernel.cu:14-327
+ *   spfa_local_forward             Sparse_FlashAttention_Local/sp_flatt_local_kernel.cu:12-272
+ *   spfa_local_1d_dilated_forward  Sparse_FlashAttention_Local_1D_Dilated/sp_flatt_local_1d_dilated_kernel.cu:12-280
+ *   spfa_local_2d_dilated_forward  Sparse_FlashAttention_Local_2D_Dilated/sp_flatt_local_2d_dilated_kernel.cu:12-306
+ *   spfa_global_no_local_forward   Sparse_FlashAttention_Global_No_Local/sp_flatt_global_no_local_kernel.cu:12-353
+ *
+ * Contract shared by all entry points
+ *   - Every pointer is a device pointer on the current device; q, k, v, out are row-major
+ *     contiguous [n, d]; m and l are [n].  Nothing is allocated, retained or synchronised by
+ *     the library: work is enqueued on `stream` (a hipStream_t passed as void*, NULL = the
+ *     default stream) and the call returns.
+ *   - (m, l, out) is in/out state exactly as in the reference (sp_flatt_csr_kernel.cu:79-92,
+ *     162-201, 208-218): out is kept normalised, m is the running maximum score, l the running
+ *     sum of exp(score - m).  A fresh state is m = -inf, l = 0, out = anything (an incoming
+ *     row with l == 0 carries no weight and its out row is not read).  Masks handed to
+ *     successive calls on one state must be disjoint.
+ *   - A row without any live column: out row := NaN when use_nan != 0 (CSR, COO, 2D-dilated),
+ *     otherwise untouched; m and l of such a row are never touched
+ *     (sp_flatt_csr_kernel.cu:45-54).
+ *   - Scores are q.k / sqrt(d) (sp_flatt_csr_kernel.cu:137).  Accumulation is fp32 for every
+ *     element type.
+ *   - `workspace` is scratch device memory of at least *_workspace_bytes(...) bytes, 256-byte
+ *     aligned, owned by the caller, and may be reused by the next call on the same stream.
+ *   - Return value: SPFA_OK or one of the codes below; spfa_status_string() gives the text
+ *     (for the parameter checks it is the text of the reference's std::invalid_argument).
+ *     Parameter checks run in the reference's order before anything is enqueued.
+ */
+#ifndef SPFA_HIP_H
+#define SPFA_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* element type of q, k, v, out */
+enum { SPFA_DTYPE_F32 = 0, SPFA_DTYPE_F16 = 1, SPFA_DTYPE_BF16 = 2 };
+
+enum {
+  SPFA_OK = 0,
+  SPFA_ERR_BAD_ARG = 1,       /* null pointer, negative size, bad enum, index width not 4/8 */
+  SPFA_ERR_UNSUPPORTED = 2,   /* element type / size combination not built */
+  SPFA_ERR_WORKSPACE = 3,     /* workspace missing, misaligned or too small */
+  SPFA_ERR_LAUNCH = 4,        /* the HIP runtime refused a launch (hipGetLastError) */
+  SPFA_ERR_EMB_TOO_LARGE = 5, /* sp_flatt_csr_kernel.cu:264-266; here: d > 1024 or d < 1 */
+  SPFA_ERR_LOCAL_SIZE = 6,    /* sp_flatt_local_kernel.cu:252-254 */
+  SPFA_ERR_DILATION_NEG = 7,  /* sp_flatt_local_1d_dilated_kernel.cu:259-261 */
+  SPFA_ERR_BLOCK_DIVISOR = 8, /* sp_flatt_local_2d_dilated_kernel.cu:274-276 */
+  SPFA_ERR_BLOCK_DILATION = 9,/* sp_flatt_local_2d_dilated_kernel.cu:284-286 */
+  SPFA_ERR_GLOBAL_COUNT = 10  /* sp_flatt_global_no_local_kernel.cu:325-327 */
+};
+
+typedef struct spfa_problem {
+  const void* q;       /* [n_q, d] */
+  const void* k;       /* [n_k, d] */
+  const void* v;       /* [n_k, d] */
+  void* m;             /* [n_q] running max, in/out */
+  void* l;             /* [n_q] running sum, in/out */
+  void* out;           /* [n_q, d] normalised output, in/out */
+  int64_t n_q;
+  int64_t n_k;         /* implicit masks use n_q for both, as the reference does */
+  int64_t d;           /* 1 <= d <= 1024 */
+  int32_t dtype;       /* SPFA_DTYPE_* of q, k, v, out */
+  int32_t state_dtype; /* SPFA_DTYPE_* of m, l: the same as dtype (reference), or F32 */
+} spfa_problem_t;
+
+int spfa_version(void);
+const char* spfa_status_string(int status);
+
+/* CSR: row i attends col_ind[row_off[i] .. row_off[i+1]).  row_off has n_q+1 entries of
+ * row_off_bytes (4 or 8) bytes each, col_ind has nnz 4-byte entries; signed and unsigned
+ * index tensors are bit-identical in range.  The reference's value vector is never read
+ * (sp_flatt_csr_kernel.cu:21) and is not part of this interface. */
+size_t spfa_csr_workspace_bytes(int64_t n_q, int64_t nnz, int64_t d, int dtype);
+int spfa_csr_forward(const spfa_problem_t* p, const void* row_off, int row_off_bytes,
+                     const void* col_ind, int64_t nnz, int use_nan, void* workspace,
+                     size_t workspace_bytes, void* stream);
+
+/* COO: row i attends {col_ind[e] : row_ind[e] == i}.  Entries may come in any order (the
+ * reference needs them sorted by row, sp_flatt_coo_kernel.cu:47-79); they are bucketed by
+ * row on the device first.  row_ind entries are row_ind_bytes (4 or 8) bytes wide. */
+size_t spfa_coo_workspace_bytes(int64_t n_q, int64_t nnz, int64_t d, int dtype);
+int spfa_coo_forward(const spfa_problem_t* p, const void* row_ind, int row_ind_bytes,
+                     const void* col_ind, int64_t nnz, int use_nan, void* workspace,
+                     size_t workspace_bytes, void* stream);
+
+/* Local: row i attends columns max(0, i-w) .. min(n-1, i+w)  (sp_flatt_local_kernel.cu:24-28). */
+size_t spfa_local_workspace_bytes(int64_t n, int64_t d, int dtype, int64_t local_size);
+int spfa_local_forward(const spfa_problem_t* p, int64_t local_size, void* workspace,
+                       size_t workspace_bytes, void* stream);
+
+/* Local 1D dilated, s = dil_factor+1: columns low, low+s, ... <= up with
+ * low = max(i - w*s, i mod s), up = min(i + w*s, n-1)
+ * (sp_flatt_local_1d_dilated_kernel.cu:25-29,102). */
+size_t spfa_local_1d_dilated_workspace_bytes(int64_t n, int64_t d, int dtype, int64_t local_size,
+                                             int64_t dil_factor);
+int spfa_local_1d_dilated_forward(const spfa_problem_t* p, int64_t local_size, int64_t dil_factor,
+                                  void* workspace, size_t workspace_bytes, void* stream);
+
+/* Local 2D dilated: inside each block of block_size rows only rows and columns at multiples
+ * of s = dil_factor+1 from the block start are live; other rows are empty
+ * (sp_flatt_local_2d_dilated_kernel.cu:26-39,123). */
+size_t spfa_local_2d_dilated_workspace_bytes(int64_t n, int64_t d, int dtype, int64_t block_size,
+                                             int64_t dil_factor);
+int spfa_local_2d_dilated_forward(const spfa_problem_t* p, int64_t block_size, int64_t dil_factor,
+                                  int use_nan, void* workspace, size_t workspace_bytes,
+                                  void* stream);
+
+/* Global minus local: with window [max(0,i-w), min(n-1,i+w)], a row listed in global_inds
+ * attends every column outside its window, any other row attends the global_inds outside its
+ * window (sp_flatt_global_no_local_kernel.cu:38-64,134-162).  global_inds: n_globals int32. */
+size_t spfa_global_no_local_workspace_bytes(int64_t n, int64_t d, int dtype, int64_t n_globals,
+                                            int64_t local_size);
+int spfa_global_no_local_forward(const spfa_problem_t* p, const int32_t* global_inds,
+                                 int64_t n_globals, int64_t local_size, void* workspace,
+                                 size_t workspace_bytes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SPFA_HIP_H */

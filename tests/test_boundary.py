@@ -1,0 +1,133 @@
+"""CPU-side checks of the drop-in boundary: the C-ABI library loads and exports every symbol the
+header declares, parameter checks return the documented codes before anything touches a device,
+and the six Python modules import and reject host tensors the way the reference bindings do."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+PKG = os.path.join(ROOT, "graph-processing-attention-ipdps-2025_amd")
+LIB = os.path.join(PKG, "libspfa_hip.so")
+HEADER = os.path.join(ROOT, "include", "spfa_hip.h")
+
+
+class Problem(ctypes.Structure):
+    _fields_ = [("q", ctypes.c_void_p), ("k", ctypes.c_void_p), ("v", ctypes.c_void_p),
+                ("m", ctypes.c_void_p), ("l", ctypes.c_void_p), ("out", ctypes.c_void_p),
+                ("n_q", ctypes.c_int64), ("n_k", ctypes.c_int64), ("d", ctypes.c_int64),
+                ("dtype", ctypes.c_int32), ("state_dtype", ctypes.c_int32)]
+
+
+@pytest.fixture(scope="module")
+def lib():
+    assert os.path.exists(LIB), "libspfa_hip.so is not built (python __graft_entry__.py build)"
+    L = ctypes.CDLL(LIB)
+    L.spfa_status_string.restype = ctypes.c_char_p
+    for name in ("spfa_csr_workspace_bytes", "spfa_coo_workspace_bytes", "spfa_local_workspace_bytes",
+                 "spfa_local_1d_dilated_workspace_bytes", "spfa_local_2d_dilated_workspace_bytes",
+                 "spfa_global_no_local_workspace_bytes"):
+        getattr(L, name).restype = ctypes.c_size_t
+    return L
+
+
+def declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(spfa_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_every_declared_symbol_is_exported(lib):
+    names = declared_functions()
+    assert len(names) >= 14
+    for n in names:
+        assert hasattr(lib, n), n
+
+
+def test_status_strings_carry_reference_texts(lib):
+    assert lib.spfa_version() >= 1
+    s = lambda c: lib.spfa_status_string(c).decode()
+    assert s(0) == "ok"
+    assert s(5) == "The embedded dimension is too large for the amount of shared memory on your GPU."
+    assert s(6) == "The local size specified is either negative or greater than/equal to (1 - Sequence Length)."
+    assert s(7) == "The dilation factor must be atleast 0."
+    assert s(8) == "The block/window size must be a divisor of the whole tensor's size."
+    assert s(9) == "The dilation factor must be less than the block/window size."
+    assert s(10) == "There are either no global tokens provided or there are more than the sequence length given."
+
+
+def _problem(n=16, d=8, dtype=0):
+    return Problem(None, None, None, None, None, None, n, n, d, dtype, dtype)
+
+
+def test_parameter_checks_run_before_any_device_work(lib):
+    """All of these return from the host-side checks: pointers are null and no device exists."""
+    i64 = ctypes.c_int64
+    p = _problem()
+    r = ctypes.byref(p)
+    assert lib.spfa_local_forward(r, i64(16), None, 0, None) == 6
+    assert lib.spfa_local_forward(r, i64(-1), None, 0, None) == 6
+    assert lib.spfa_local_1d_dilated_forward(r, i64(3), i64(-1), None, 0, None) == 7
+    assert lib.spfa_local_1d_dilated_forward(r, i64(16), i64(-1), None, 0, None) == 6
+    assert lib.spfa_local_2d_dilated_forward(r, i64(3), i64(0), 0, None, 0, None) == 8
+    assert lib.spfa_local_2d_dilated_forward(r, i64(0), i64(0), 0, None, 0, None) == 8
+    assert lib.spfa_local_2d_dilated_forward(r, i64(4), i64(-1), 0, None, 0, None) == 7
+    assert lib.spfa_local_2d_dilated_forward(r, i64(4), i64(4), 0, None, 0, None) == 9
+    assert lib.spfa_global_no_local_forward(r, None, i64(0), i64(1), None, 0, None) == 10
+    assert lib.spfa_global_no_local_forward(r, None, i64(17), i64(1), None, 0, None) == 10
+    assert lib.spfa_global_no_local_forward(r, None, i64(2), i64(16), None, 0, None) == 6
+    big = _problem(d=2048)
+    assert lib.spfa_csr_forward(ctypes.byref(big), None, 8, None, i64(0), 0, None, 0, None) == 5
+    assert lib.spfa_local_forward(ctypes.byref(big), i64(99), None, 0, None) == 5  # d first
+    # valid parameters, null tensors -> bad argument, still no device work
+    assert lib.spfa_local_forward(r, i64(3), None, 0, None) == 1
+    assert lib.spfa_csr_forward(r, None, 5, None, i64(0), 0, None, 0, None) == 1  # index width
+    bad_dtype = _problem(dtype=7)
+    assert lib.spfa_local_forward(ctypes.byref(bad_dtype), i64(3), None, 0, None) == 2
+    assert lib.spfa_local_forward(None, i64(3), None, 0, None) == 1
+
+
+def test_workspace_sizes_are_sane(lib):
+    i64 = ctypes.c_int64
+    small = lib.spfa_csr_workspace_bytes(i64(1024), i64(10), i64(64), 0)
+    large = lib.spfa_csr_workspace_bytes(i64(131072), i64(13_000_000), i64(64), 0)
+    assert 256 <= small < (1 << 20)
+    assert small < large < (256 << 20)
+    assert lib.spfa_coo_workspace_bytes(i64(131072), i64(13_000_000), i64(64), 0) > large
+    assert lib.spfa_local_workspace_bytes(i64(65536), i64(64), 0, i64(128)) >= 256
+    assert lib.spfa_global_no_local_workspace_bytes(i64(1 << 20), i64(64), 0, i64(64), i64(64)) > (1 << 20)
+
+
+def test_modules_import_and_expose_forward(mods):
+    for name, mod in mods.items():
+        assert callable(mod.forward), name
+
+
+def test_host_tensors_are_rejected_like_the_reference(mods):
+    n, d = 8, 4
+    q = torch.zeros(n, d)
+    m = torch.full((n,), -float("inf"))
+    l = torch.zeros(n)
+    ro = torch.zeros(n + 1, dtype=torch.int64)
+    ci = torch.zeros(0, dtype=torch.int32)
+    val = torch.zeros(0)
+    g = torch.zeros(1, dtype=torch.int32)
+    calls = [
+        lambda: mods["spfa_csr"].forward(q, q, q, ro, ci, val, m, l, q, True),
+        lambda: mods["spfa_coo"].forward(q, q, q, ro, ci, val, m, l, q, True),
+        lambda: mods["spfa_local"].forward(q, q, q, m, l, q, 1),
+        lambda: mods["spfa_local_1d_dilated"].forward(q, q, q, m, l, q, 1, 1),
+        lambda: mods["spfa_local_2d_dilated"].forward(q, q, q, m, l, q, 4, 0, True),
+        lambda: mods["spfa_global_no_local"].forward(q, q, q, m, l, q, g, 1),
+    ]
+    for c in calls:
+        with pytest.raises(RuntimeError, match="Q must be a CUDA tensor"):
+            c()
+
+
+def test_wrong_argument_count_is_a_type_error(mods):
+    q = torch.zeros(2, 2)
+    with pytest.raises(TypeError):
+        mods["spfa_local"].forward(q, q, q)

@@ -1,0 +1,475 @@
+"""GPU parity tests: the six spfa_* modules (host wrapper -> C ABI -> HIP kernels) against the CPU
+oracle on the same seeded inputs.  Bars: max-abs 1e-4 (fp32), 2e-2 (fp16 / bf16) on the output,
+identical sets of computed rows, and m + log(l) equal to the oracle's log-sum-exp."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import spfa_synth as syn
+from helpers import OUT_TOL, check, csr_rows_subset, np64, oracle_rows
+from oracle import c_oracle
+from oracle import spfa_oracle as so
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+DTYPES = [torch.float32, torch.float16, torch.bfloat16]
+
+
+def sync():
+    torch.cuda.synchronize()
+
+
+def dev_qkv(n, d, dtype, seed, scale=1.0, n_k=None):
+    q, k, v = syn.qkv(n, d, dtype=dtype, device="cpu", seed=seed, scale=scale, n_k=n_k)
+    return q.to(DEV), k.to(DEV), v.to(DEV)
+
+
+def state(n, d, dtype, state_dtype=None):
+    return syn.fresh_state(n, d, dtype=dtype, device=DEV, state_dtype=state_dtype)
+
+
+def csr_tensors(ro, ci, off_dtype=torch.uint64, col_dtype=torch.uint32):
+    ro_t = torch.as_tensor(np.asarray(ro, dtype=np.int64)).to(off_dtype).to(DEV)
+    ci_t = torch.as_tensor(np.asarray(ci, dtype=np.int64)).to(col_dtype).to(DEV)
+    return ro_t, ci_t
+
+
+def run_csr(mods, q, k, v, ro, ci, use_nan, st=None, off_dtype=torch.uint64, col_dtype=torch.uint32,
+            state_dtype=None):
+    n, d = q.shape
+    m, l, o = st if st is not None else state(n, d, q.dtype, state_dtype)
+    ro_t, ci_t = csr_tensors(ro, ci, off_dtype, col_dtype)
+    val = torch.ones(ci_t.numel(), device=DEV, dtype=q.dtype)
+    ret = mods["spfa_csr"].forward(q, k, v, ro_t, ci_t, val, m, l, o, use_nan)
+    sync()
+    assert ret.data_ptr() == o.data_ptr()
+    return o, m, l
+
+
+# ------------------------------------------------------------------ the reference's own checks
+class TestVerifyScript:
+    """Seeded re-statements of the eleven comparisons of verification/verify.py (N=256, d=32,
+    fp32, uniform [0,1) inputs)."""
+    N, D = 256, 32
+
+    def setup_method(self, _):
+        g = torch.Generator().manual_seed(1234)
+        self.q, self.k, self.v = [torch.rand(self.N, self.D, generator=g).to(DEV) for _ in range(3)]
+        self.qn, self.kn, self.vn = np64(self.q), np64(self.k), np64(self.v)
+
+    def dense(self, mask):
+        return so.dense_masked_attention(self.qn, self.kn, self.vn, mask)
+
+    def test_csr_coo_local_full_agree_with_dense(self, mods):  # verify.py:42-152
+        n, d = self.N, self.D
+        mask = np.ones((n, n), dtype=bool)
+        ref = self.dense(mask)
+        ro, ci = so.csr_from_dense(mask)
+        o1, m1, l1 = run_csr(mods, self.q, self.k, self.v, ro, ci, True)
+        check(o1, m1, l1, *ref, torch.float32)
+        r, c = so.coo_from_dense(mask)
+        m, l, o2 = state(n, d, torch.float32)
+        mods["spfa_coo"].forward(self.q, self.k, self.v, torch.as_tensor(r).to(torch.uint64).to(DEV),
+                                 torch.as_tensor(c).to(torch.uint32).to(DEV),
+                                 torch.ones(len(c), device=DEV), m, l, o2, True)
+        sync()
+        check(o2, m, l, *ref, torch.float32)
+        m, l, o3 = state(n, d, torch.float32)
+        mods["spfa_local"].forward(self.q, self.k, self.v, m, l, o3, n - 1)
+        sync()
+        check(o3, m, l, *ref, torch.float32)
+        assert torch.allclose(o1, o2, atol=1e-5) and torch.allclose(o1, o3, atol=1e-5)
+
+    def test_local_window_zero_returns_v(self, mods):  # verify.py:158-177
+        m, l, o = state(self.N, self.D, torch.float32)
+        mods["spfa_local"].forward(self.q, self.k, self.v, m, l, o, 0)
+        sync()
+        assert torch.equal(o, self.v)
+        assert torch.all(l == 1.0)
+
+    def test_global_no_local(self, mods):  # verify.py:183-229
+        globs, w = [0, 1, 10, 40], 10
+        ref = self.dense(so.mask_global_no_local_dense(self.N, globs, w))
+        m, l, o = state(self.N, self.D, torch.float32)
+        g = torch.tensor(globs, dtype=torch.int32, device=DEV)
+        mods["spfa_global_no_local"].forward(self.q, self.k, self.v, m, l, o, g, w)
+        sync()
+        check(o, m, l, *ref, torch.float32)
+
+    def _bigbird(self, seed):
+        n = self.N
+        rng = np.random.default_rng(seed)
+        globs = np.sort(rng.choice(n, 5, replace=False))
+        w = 10
+        rnd = rng.random((n, n)) < 0.1
+        fixed = so.mask_local_dense(n, w) | so.mask_global_no_local_dense(n, globs, w)
+        return globs, w, rnd, fixed
+
+    def test_bigbird_as_one_csr(self, mods):  # verify.py:235-290
+        globs, w, rnd, fixed = self._bigbird(7)
+        mask = fixed | rnd
+        ro, ci = so.csr_from_dense(mask)
+        o, m, l = run_csr(mods, self.q, self.k, self.v, ro, ci, False)
+        check(o, m, l, *self.dense(mask), torch.float32)
+
+    def test_bigbird_chained_three_kernels(self, mods):  # verify.py:296-362
+        globs, w, rnd, fixed = self._bigbird(8)
+        m, l, o = state(self.N, self.D, torch.float32)
+        mods["spfa_local"].forward(self.q, self.k, self.v, m, l, o, w)
+        mods["spfa_global_no_local"].forward(self.q, self.k, self.v, m, l, o,
+                                             torch.tensor(globs, dtype=torch.int32, device=DEV), w)
+        ro, ci = so.csr_from_dense(rnd & ~fixed)
+        o, m, l = run_csr(mods, self.q, self.k, self.v, ro, ci, False, st=(m, l, o))
+        check(o, m, l, *self.dense(fixed | rnd), torch.float32)
+
+    def test_local_1d_dilated(self, mods):  # verify.py:368-409
+        w, dil = 10, 2
+        m, l, o = state(self.N, self.D, torch.float32)
+        mods["spfa_local_1d_dilated"].forward(self.q, self.k, self.v, m, l, o, w, dil)
+        sync()
+        check(o, m, l, *self.dense(so.mask_local_1d_dilated_dense(self.N, w, dil)), torch.float32)
+
+    @pytest.mark.parametrize("dil", [0, 1])
+    def test_local_2d_dilated(self, mods, dil):  # verify.py:415-505
+        m, l, o = state(self.N, self.D, torch.float32)
+        mods["spfa_local_2d_dilated"].forward(self.q, self.k, self.v, m, l, o, 16, dil, True)
+        sync()
+        check(o, m, l, *self.dense(so.mask_local_2d_dilated_dense(self.N, 16, dil)), torch.float32,
+              dead_expect="nan")
+
+
+# ------------------------------------------------------------------ golden vectors, every dtype
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("kind", ["csr", "coo", "local", "d1", "d2", "glob", "union"])
+def test_golden_vectors(mods, golden, kind, dtype):
+    q, k, v = [torch.tensor(golden[x], dtype=dtype, device=DEV) for x in ("q", "k", "v")]
+    n, d = q.shape
+    m, l, o = state(n, d, dtype, torch.float32)
+    dead_expect = None
+    key = kind
+    if kind in ("csr", "coo"):
+        key = "csr"
+        ro, ci = so.csr_from_dense(golden["csr_mask"])
+        val = torch.ones(len(ci), device=DEV, dtype=dtype)
+        if kind == "csr":
+            ro_t, ci_t = csr_tensors(ro, ci)
+            mods["spfa_csr"].forward(q, k, v, ro_t, ci_t, val, m, l, o, True)
+        else:
+            r, c = so.coo_from_dense(golden["csr_mask"])
+            perm = np.random.default_rng(5).permutation(len(r))
+            mods["spfa_coo"].forward(q, k, v, torch.as_tensor(r[perm]).to(torch.uint64).to(DEV),
+                                     torch.as_tensor(c[perm]).to(torch.uint32).to(DEV), val, m, l, o, True)
+        dead_expect = "nan"
+    elif kind == "local":
+        mods["spfa_local"].forward(q, k, v, m, l, o, int(golden["local_w"]))
+    elif kind == "d1":
+        mods["spfa_local_1d_dilated"].forward(q, k, v, m, l, o, int(golden["d1_w"]), int(golden["d1_dil"]))
+    elif kind == "d2":
+        mods["spfa_local_2d_dilated"].forward(q, k, v, m, l, o, int(golden["d2_block"]),
+                                              int(golden["d2_dil"]), True)
+        dead_expect = "nan"
+    else:
+        g = torch.tensor(golden["glob_inds"], dtype=torch.int32, device=DEV)
+        w = int(golden["glob_w"])
+        if kind == "union":
+            mods["spfa_local"].forward(q, k, v, m, l, o, w)
+        mods["spfa_global_no_local"].forward(q, k, v, m, l, o, g, w)
+        if kind == "union":
+            ro, ci = so.csr_from_dense(golden["union_rest_mask"])
+            ro_t, ci_t = csr_tensors(ro, ci)
+            mods["spfa_csr"].forward(q, k, v, ro_t, ci_t, torch.ones(len(ci), device=DEV, dtype=dtype),
+                                     m, l, o, False)
+    sync()
+    exp_out, exp_lse = golden[key + "_out"], golden[key + "_lse"]
+    live = np.isfinite(exp_lse)
+    ref_l = np.where(live, 1.0, 0.0)
+    ref_m = np.where(live, exp_lse, -np.inf)  # lse == m + log(1)
+    check(o, m, l, np.nan_to_num(exp_out), ref_m, ref_l, dtype, state_dtype=torch.float32,
+          dead_expect=dead_expect, check_m=False)
+    if not live.all():
+        assert torch.all(torch.isneginf(m[torch.tensor(~live, device=DEV)]))
+        assert torch.all(l[torch.tensor(~live, device=DEV)] == 0)
+
+
+# ------------------------------------------------------------------ CSR
+def test_csr_bernoulli_n4096_d64_fp32(mods):
+    """The CPU-runnable configuration: N=4096, d=64, fp32, 2% random mask plus diagonal, against the
+    dense float64 formulation."""
+    n, d = 4096, 64
+    q, k, v = dev_qkv(n, d, torch.float32, 0)
+    ro, ci = syn.bernoulli_csr(n, 0.02, seed=0)
+    o, m, l = run_csr(mods, q, k, v, ro, ci, True)
+    mask = so.dense_from_csr(ro.numpy(), ci.numpy(), n, n)
+    check(o, m, l, *so.dense_masked_attention(np64(q), np64(k), np64(v), mask), torch.float32)
+
+
+def _special_rows_csr(n, rng, lengths):
+    """Mask whose first rows have the given lengths (the rest random short rows)."""
+    cols, off = [], [0]
+    for i in range(n):
+        ln = lengths[i] if i < len(lengths) else int(rng.integers(0, 6))
+        c = np.sort(rng.choice(n, ln, replace=False)) if ln else np.zeros(0, np.int64)
+        cols.append(c)
+        off.append(off[-1] + ln)
+    return np.array(off, np.int64), np.concatenate(cols).astype(np.int64)
+
+
+@pytest.mark.parametrize("dtype,d", [(torch.float32, 64), (torch.float32, 32), (torch.float32, 128),
+                                     (torch.bfloat16, 64), (torch.float16, 128), (torch.float32, 256)])
+def test_csr_row_lengths_around_every_threshold(mods, dtype, d):
+    """Rows of length 0, 1, the in-place limit and one more, one segment and one more, several
+    segments exactly, and the longest possible row."""
+    n = 2048
+    rng = np.random.default_rng(3)
+    lengths = [0, 1, 2, 31, 32, 33, 63, 64, 65, 255, 256, 257, 511, 512, 513, 768, 1024, 2048, 0, 7]
+    ro, ci = _special_rows_csr(n, rng, lengths)
+    q, k, v = dev_qkv(n, d, dtype, 21)
+    o, m, l = run_csr(mods, q, k, v, ro, ci, True, state_dtype=torch.float32)
+    ref = c_oracle.csr(np64(q), np64(k), np64(v), ro, ci, use_nan=True)
+    check(o, m, l, *ref, dtype, state_dtype=torch.float32, dead_expect="nan")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_csr_power_law_rows(mods, dtype):
+    """Zipf(1.5) degrees clipped to [1, 4096] at N=16384: short rows, single-segment rows and
+    rows split over several segments in one call."""
+    n, d = 16384, 64
+    q, k, v = dev_qkv(n, d, dtype, 5)
+    ro, ci = syn.zipf_csr(n, 1.5, 1, 4096, seed=5)
+    o, m, l = run_csr(mods, q, k, v, ro, ci, False, state_dtype=torch.float32)
+    ref = c_oracle.csr(np64(q), np64(k), np64(v), ro.numpy(), ci.numpy())
+    check(o, m, l, *ref, dtype, state_dtype=torch.float32)
+
+
+@pytest.mark.parametrize("d", [1, 3, 40, 100, 200, 520])
+def test_csr_any_embedding_size(mods, d):
+    n = 300
+    q, k, v = dev_qkv(n, d, torch.float32, 9)
+    ro, ci = syn.zipf_csr(n, 1.3, 0, 300, seed=9)
+    o, m, l = run_csr(mods, q, k, v, ro, ci, True)
+    ref = c_oracle.csr(np64(q), np64(k), np64(v), ro.numpy(), ci.numpy(), use_nan=True)
+    check(o, m, l, *ref, torch.float32, dead_expect="nan")
+
+
+@pytest.mark.parametrize("off_dtype,col_dtype", [(torch.uint64, torch.uint32), (torch.int64, torch.int32),
+                                                 (torch.int32, torch.int32), (torch.uint32, torch.uint32)])
+def test_csr_index_dtypes(mods, off_dtype, col_dtype):
+    n, d = 512, 64
+    q, k, v = dev_qkv(n, d, torch.float32, 10)
+    ro, ci = syn.zipf_csr(n, 1.5, 0, 512, seed=10)
+    o, m, l = run_csr(mods, q, k, v, ro, ci, True, off_dtype=off_dtype, col_dtype=col_dtype)
+    ref = c_oracle.csr(np64(q), np64(k), np64(v), ro.numpy(), ci.numpy(), use_nan=True)
+    check(o, m, l, *ref, torch.float32, dead_expect="nan")
+
+
+def test_csr_rectangular_k(mods):
+    """K/V may have a different row count than Q: columns index K/V rows."""
+    n, n_k, d = 256, 1000, 64
+    q, k, v = dev_qkv(n, d, torch.float32, 12, n_k=n_k)
+    g = torch.Generator().manual_seed(12)
+    deg = torch.randint(0, 40, (n,), generator=g)
+    ro, ci = syn.csr_from_degrees(deg, n_k, g, "cpu", force_diagonal=False)
+    o, m, l = run_csr(mods, q, k, v, ro, ci, True)
+    ref = c_oracle.csr(np64(q), np64(k), np64(v), ro.numpy(), ci.numpy(), use_nan=True)
+    check(o, m, l, *ref, torch.float32, dead_expect="nan")
+
+
+@pytest.mark.parametrize("use_nan", [False, True])
+def test_csr_empty_rows_and_state_untouched(mods, use_nan):
+    n, d = 128, 64
+    q, k, v = dev_qkv(n, d, torch.float32, 13)
+    mask = np.zeros((n, n), dtype=bool)
+    mask[::2, 5] = True
+    ro, ci = so.csr_from_dense(mask)
+    m = torch.full((n,), -1.5, device=DEV)
+    l = torch.full((n,), 2.5, device=DEV)
+    o = torch.full((n, d), 7.0, device=DEV)
+    m0, l0, o0 = m.clone(), l.clone(), o.clone()
+    run_csr(mods, q, k, v, ro, ci, use_nan, st=(m, l, o))
+    ref = c_oracle.csr(np64(q), np64(k), np64(v), ro, ci, m=np64(m0), l=np64(l0), out=np64(o0), use_nan=use_nan)
+    dead = torch.arange(n, device=DEV) % 2 == 1
+    assert torch.equal(m[dead], m0[dead]) and torch.equal(l[dead], l0[dead])
+    if use_nan:
+        assert torch.isnan(o[dead]).all()
+    else:
+        assert torch.equal(o[dead], o0[dead])
+    live = ~dead
+    assert np.abs(np64(o[live]) - ref[0][np64(live) > 0]).max() <= 1e-4
+    assert np.abs(np64(m[live]) - ref[1][np64(live) > 0]).max() <= 1e-4
+    assert np.abs(np64(l[live]) / ref[2][np64(live) > 0] - 1).max() <= 1e-4
+
+
+def test_csr_split_and_chain_equals_single_call(mods):
+    n, d = 1024, 64
+    q, k, v = dev_qkv(n, d, torch.float32, 14)
+    rng = np.random.default_rng(14)
+    mask = rng.random((n, n)) < 0.08
+    part = rng.integers(0, 3, size=(n, n))
+    st = state(n, d, torch.float32)
+    for p in range(3):
+        ro, ci = so.csr_from_dense(mask & (part == p))
+        o, m, l = run_csr(mods, q, k, v, ro, ci, False, st=st)
+    check(o, m, l, *so.dense_masked_attention(np64(q), np64(k), np64(v), mask), torch.float32)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_csr_state_in_element_dtype(mods, dtype):
+    """m and l in the element type, as the reference allocates them."""
+    n, d = 512, 64
+    q, k, v = dev_qkv(n, d, dtype, 15)
+    ro, ci = syn.zipf_csr(n, 1.5, 1, 512, seed=15)
+    o, m, l = run_csr(mods, q, k, v, ro, ci, False)
+    assert m.dtype == dtype and l.dtype == dtype
+    ref = c_oracle.csr(np64(q), np64(k), np64(v), ro.numpy(), ci.numpy())
+    check(o, m, l, *ref, dtype)
+
+
+# ------------------------------------------------------------------ COO
+@pytest.mark.parametrize("row_dtype", [torch.uint64, torch.int64, torch.int32])
+def test_coo_unsorted_equals_csr(mods, row_dtype):
+    n, d = 4096, 64
+    q, k, v = dev_qkv(n, d, torch.float32, 16)
+    ro, ci = syn.zipf_csr(n, 1.4, 0, 2048, seed=16)
+    r, c = syn.coo_from_csr(ro, ci, shuffle_seed=16)
+    m, l, o = state(n, d, torch.float32)
+    mods["spfa_coo"].forward(q, k, v, r.to(row_dtype).to(DEV), c.to(torch.uint32).to(DEV),
+                             torch.ones(c.numel(), device=DEV), m, l, o, True)
+    sync()
+    ref = c_oracle.csr(np64(q), np64(k), np64(v), ro.numpy(), ci.numpy(), use_nan=True)
+    check(o, m, l, *ref, torch.float32, dead_expect="nan")
+    o2, m2, l2 = run_csr(mods, q, k, v, ro, ci, True)
+    assert torch.allclose(torch.nan_to_num(o), torch.nan_to_num(o2), atol=2e-5)
+
+
+def test_coo_power_law_with_many_empty_rows(mods):
+    n, d = 65536, 64
+    q, k, v = dev_qkv(n, d, torch.float32, 17)
+    r, c = syn.zipf_coo(n, 600_000, 1.3, seed=17)
+    m, l, o = state(n, d, torch.float32)
+    mods["spfa_coo"].forward(q, k, v, r.to(torch.uint64).to(DEV), c.to(torch.uint32).to(DEV),
+                             torch.ones(c.numel(), device=DEV), m, l, o, False)
+    sync()
+    ref = c_oracle.coo(np64(q), np64(k), np64(v), r.numpy(), c.numpy())
+    check(o, m, l, *ref, torch.float32)
+
+
+def test_coo_empty_mask(mods):
+    n, d = 64, 64
+    q, k, v = dev_qkv(n, d, torch.float32, 18)
+    m, l, o = state(n, d, torch.float32)
+    e64 = torch.zeros(0, dtype=torch.uint64, device=DEV)
+    e32 = torch.zeros(0, dtype=torch.uint32, device=DEV)
+    mods["spfa_coo"].forward(q, k, v, e64, e32, torch.zeros(0, device=DEV), m, l, o, True)
+    sync()
+    assert torch.isnan(o).all() and torch.all(l == 0) and torch.all(torch.isneginf(m))
+
+
+# ------------------------------------------------------------------ implicit masks
+@pytest.mark.parametrize("dtype,d", [(torch.float32, 64), (torch.bfloat16, 64), (torch.float16, 32),
+                                     (torch.bfloat16, 128), (torch.float32, 48)])
+@pytest.mark.parametrize("n,w", [(1000, 0), (1000, 1), (1000, 128), (777, 776), (4096, 300)])
+def test_local(mods, dtype, d, n, w):
+    q, k, v = dev_qkv(n, d, dtype, 30)
+    m, l, o = state(n, d, dtype, torch.float32)
+    mods["spfa_local"].forward(q, k, v, m, l, o, w)
+    sync()
+    ref = c_oracle.local(np64(q), np64(k), np64(v), w)
+    check(o, m, l, *ref, dtype, state_dtype=torch.float32)
+
+
+@pytest.mark.parametrize("dtype,d", [(torch.float32, 64), (torch.bfloat16, 128), (torch.float16, 64)])
+@pytest.mark.parametrize("n,w,dil", [(1000, 10, 2), (1000, 0, 3), (1000, 999, 0), (1001, 100, 1),
+                                     (2048, 256, 2), (300, 299, 6)])
+def test_local_1d_dilated(mods, dtype, d, n, w, dil):
+    q, k, v = dev_qkv(n, d, dtype, 31, scale=0.5)
+    m, l, o = state(n, d, dtype, torch.float32)
+    mods["spfa_local_1d_dilated"].forward(q, k, v, m, l, o, w, dil)
+    sync()
+    ref = c_oracle.local_1d_dilated(np64(q), np64(k), np64(v), w, dil)
+    check(o, m, l, *ref, dtype, state_dtype=torch.float32)
+
+
+@pytest.mark.parametrize("dtype,d", [(torch.float32, 64), (torch.bfloat16, 128), (torch.float16, 64)])
+@pytest.mark.parametrize("n,block,dil", [(1024, 16, 0), (1024, 16, 1), (1024, 256, 2), (1000, 1000, 3),
+                                         (1024, 1, 0), (960, 32, 31), (2048, 2048, 0)])
+@pytest.mark.parametrize("use_nan", [True, False])
+def test_local_2d_dilated(mods, dtype, d, n, block, dil, use_nan):
+    q, k, v = dev_qkv(n, d, dtype, 32, scale=0.5)
+    m, l, o = state(n, d, dtype, torch.float32)
+    mods["spfa_local_2d_dilated"].forward(q, k, v, m, l, o, block, dil, use_nan)
+    sync()
+    ref = c_oracle.local_2d_dilated(np64(q), np64(k), np64(v), block, dil, use_nan=use_nan)
+    check(o, m, l, *ref, dtype, state_dtype=torch.float32, dead_expect="nan" if use_nan else None)
+
+
+@pytest.mark.parametrize("dtype,d", [(torch.float32, 64), (torch.bfloat16, 64), (torch.float16, 128)])
+@pytest.mark.parametrize("n,n_globs,w", [(1024, 4, 10), (1024, 1, 0), (1024, 64, 64), (1500, 100, 1499),
+                                         (1024, 1024, 3), (8192, 16, 100)])
+def test_global_no_local(mods, dtype, d, n, n_globs, w):
+    q, k, v = dev_qkv(n, d, dtype, 33)
+    g = syn.global_indices(n, n_globs, seed=33)
+    m, l, o = state(n, d, dtype, torch.float32)
+    mods["spfa_global_no_local"].forward(q, k, v, m, l, o, g.to(DEV), w)
+    sync()
+    ref = c_oracle.global_no_local(np64(q), np64(k), np64(v), g.numpy(), w)
+    check(o, m, l, *ref, dtype, state_dtype=torch.float32)
+
+
+def test_global_indices_need_not_be_sorted(mods):
+    n, d, w = 512, 64, 7
+    q, k, v = dev_qkv(n, d, torch.float32, 34)
+    g = torch.tensor([400, 3, 77, 2, 300, 4], dtype=torch.int32)
+    m, l, o = state(n, d, torch.float32)
+    mods["spfa_global_no_local"].forward(q, k, v, m, l, o, g.to(DEV), w)
+    sync()
+    check(o, m, l, *so.dense_masked_attention(np64(q), np64(k), np64(v),
+                                              so.mask_global_no_local_dense(n, g.numpy(), w)), torch.float32)
+
+
+# ------------------------------------------------------------------ errors
+def test_errors_keep_reference_types_and_texts(mods):
+    n, d = 64, 64
+    q, k, v = dev_qkv(n, d, torch.float32, 40)
+    m, l, o = state(n, d, torch.float32)
+    g = torch.tensor([1, 2], dtype=torch.int32, device=DEV)
+    with pytest.raises(ValueError, match="local size specified"):
+        mods["spfa_local"].forward(q, k, v, m, l, o, n)
+    with pytest.raises(ValueError, match="local size specified"):
+        mods["spfa_local_1d_dilated"].forward(q, k, v, m, l, o, -1, 0)
+    with pytest.raises(ValueError, match="atleast 0"):
+        mods["spfa_local_1d_dilated"].forward(q, k, v, m, l, o, 3, -1)
+    with pytest.raises(ValueError, match="divisor"):
+        mods["spfa_local_2d_dilated"].forward(q, k, v, m, l, o, 5, 0, True)
+    with pytest.raises(ValueError, match="atleast 0"):
+        mods["spfa_local_2d_dilated"].forward(q, k, v, m, l, o, 8, -1, True)
+    with pytest.raises(ValueError, match="less than the block"):
+        mods["spfa_local_2d_dilated"].forward(q, k, v, m, l, o, 8, 8, True)
+    with pytest.raises(ValueError, match="no global tokens"):
+        mods["spfa_global_no_local"].forward(q, k, v, m, l, o, g[:0], 1)
+    with pytest.raises(ValueError, match="local size specified"):
+        mods["spfa_global_no_local"].forward(q, k, v, m, l, o, g, n)
+    with pytest.raises(RuntimeError, match="K must be contiguous"):
+        mods["spfa_local"].forward(q, k.t().contiguous().t(), v, m, l, o, 1)
+    with pytest.raises(RuntimeError, match="m must be a CUDA tensor"):
+        mods["spfa_local"].forward(q, k, v, m.cpu(), l, o, 1)
+    with pytest.raises(RuntimeError, match="unsupported element type"):
+        mods["spfa_local"].forward(q.double(), k.double(), v.double(), m.double(), l.double(), o.double(), 1)
+    with pytest.raises(RuntimeError, match="int32"):
+        mods["spfa_global_no_local"].forward(q, k, v, m, l, o, g.long(), 1)
+    # nothing above may have modified the state
+    sync()
+    assert torch.all(o == 0) and torch.all(l == 0)
+
+
+def test_runs_on_a_side_stream(mods):
+    n, d = 2048, 64
+    q, k, v = dev_qkv(n, d, torch.float32, 41)
+    ro, ci = syn.zipf_csr(n, 1.5, 1, 2048, seed=41)
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):
+        o, m, l = run_csr(mods, q, k, v, ro, ci, False)
+    ref = c_oracle.csr(np64(q), np64(k), np64(v), ro.numpy(), ci.numpy())
+    check(o, m, l, *ref, torch.float32)
