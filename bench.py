@@ -1,0 +1,394 @@
+#!/usr/bin/env python3
+"""Throughput of the sparse-attention hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--dtype f32|f16|bf16]
+
+Default workload: explicit CSR mask, N=131072, d=64, fp32, Zipf(1.5) row degrees clipped to
+[1, 4096], uniform distinct sorted columns, diagonal included (seeded, generated on the device).
+One step = one spfa_csr.forward call on a fresh (m, l, out) state with all inputs resident in HBM.
+
+Prints ONE JSON line: nnz-counted GFLOP/s (4*d*nnz flops per step) as `value`, the HBM roofline of
+the dominant kernel (algorithmic bytes / its launch time measured with HIP events on the launch
+stream), and a CPU baseline timed on a bounded sample of the same workload.
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+PKG = os.path.join(ROOT, "graph-processing-attention-ipdps-2025_amd")
+for p in (ROOT, PKG):
+    if p not in sys.path:
+        sys.path.insert(0, p)
+
+HBM_PEAK_GBS = 8000.0      # MI355X HBM3E
+FP32_PEAK_TFLOPS = 157.3   # MI355X dense fp32 matrix
+HALF_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 / fp16 matrix
+
+WORKLOADS = {
+    "csr_zipf": "CSR N=131072 d=64 Zipf(1.5) degrees clipped [1,4096], uniform sorted columns + diagonal",
+    "csr_bernoulli": "CSR N=4096 d=64 Bernoulli(2%) + diagonal",
+    "coo_zipf": "COO N=1048576 d=64 ~50M unsorted entries, row weights Zipf(1.3), uniform columns",
+    "local": "Local N=65536 d=64 LOCAL_SIZE=128 (|i-j|<=128)",
+    "local_1d": "Local-1D-dilated N=262144 d=128 LOCAL_SIZE=256 DILATE_FACTOR=2 (stride 3)",
+    "local_2d": "Local-2D-dilated N=262144 d=128 BLOCK_SIZE=256 DILATE_FACTOR=2 (stride 3)",
+    "global": "Global-no-local N=1048576 d=64 64 global tokens LOCAL_SIZE=64",
+}
+
+
+class HipEvents:
+    """hipEvent pair created straight from the HIP runtime (torch.cuda.Event only sees torch's
+    own record calls; these are recorded inside the library around one kernel)."""
+
+    def __init__(self):
+        self.hip = ctypes.CDLL("libamdhip64.so")
+        self.start = ctypes.c_void_p()
+        self.stop = ctypes.c_void_p()
+        assert self.hip.hipEventCreate(ctypes.byref(self.start)) == 0
+        assert self.hip.hipEventCreate(ctypes.byref(self.stop)) == 0
+
+    def elapsed_ms(self):
+        ms = ctypes.c_float()
+        assert self.hip.hipEventSynchronize(self.stop) == 0
+        rc = self.hip.hipEventElapsedTime(ctypes.byref(ms), self.start, self.stop)
+        assert rc == 0, "hipEventElapsedTime rc=%d" % rc
+        return float(ms.value)
+
+
+def load_library():
+    lib_path = os.path.join(PKG, "libspfa_hip.so")
+    if not os.path.exists(lib_path):
+        raise RuntimeError("libspfa_hip.so is not built: run `python -c 'import __graft_entry__ as g; g.build()'`")
+    lib = ctypes.CDLL(lib_path)
+    lib.spfa_set_kernel_events.argtypes = [ctypes.c_void_p, ctypes.c_void_p]
+    lib.spfa_set_kernel_events.restype = None
+    lib.spfa_explicit_inline_row_limit.restype = ctypes.c_int64
+    return lib
+
+
+def make_workload(name, dtype, torch, syn, inline_limit=32):
+    """Returns dict(call=fn(state) -> None, n, d, nnz, bytes_total, bytes_gathered, sample=fn())."""
+    dev = "cuda"
+    es = torch.tensor([], dtype=dtype).element_size()
+    w = {"name": name, "desc": WORKLOADS[name]}
+    if name in ("csr_zipf", "csr_bernoulli", "coo_zipf"):
+        if name == "csr_zipf":
+            n, d = 131072, 64
+            ro, ci = syn.zipf_csr(n, 1.5, 1, 4096, device=dev, seed=0)
+        elif name == "csr_bernoulli":
+            n, d = 4096, 64
+            ro, ci = syn.bernoulli_csr(n, 0.02, device=dev, seed=0)
+        else:
+            n, d = 1 << 20, 64
+            r, c = syn.zipf_coo(n, 50_000_000, 1.3, device=dev, seed=0)
+        q, k, v = syn.qkv(n, d, dtype=dtype, device=dev, seed=0)
+        if name == "coo_zipf":
+            import spfa_coo
+            nnz = int(c.numel())
+            r_t, c_t = r.to(torch.uint64), c.to(torch.uint32)
+            val = torch.empty(nnz, device=dev, dtype=dtype)
+            w["call"] = lambda st: spfa_coo.forward(q, k, v, r_t, c_t, val, st[0], st[1], st[2], False)
+            w["csr"] = None
+            w["coo"] = (r, c)
+            off_b = 8
+        else:
+            import spfa_csr
+            nnz = int(ci.numel())
+            ro_t, ci_t = ro.to(torch.uint64), ci.to(torch.uint32)
+            val = torch.empty(nnz, device=dev, dtype=dtype)
+            w["call"] = lambda st: spfa_csr.forward(q, k, v, ro_t, ci_t, val, st[0], st[1], st[2], False)
+            w["csr"] = (ro, ci)
+            off_b = 8
+        gathered, total = syn.explicit_mask_bytes(nnz, n, d, es, off_bytes=off_b)
+        if name == "coo_zipf":
+            total += nnz * 8  # row index of every entry
+            deg = torch.bincount(r, minlength=n)
+        else:
+            deg = ro[1:] - ro[:-1]
+        # the dominant (segment) kernel owns the rows longer than the library's in-place limit
+        long_rows = deg > inline_limit
+        nnz_long, rows_long = int(deg[long_rows].sum()), int(long_rows.sum())
+        _, kernel_bytes = syn.explicit_mask_bytes(nnz_long, rows_long, d, es, off_bytes=off_b)
+        w.update(n=n, d=d, nnz=nnz, bytes_total=total, bytes_gathered=gathered, bound="hbm",
+                 kernel_bytes=kernel_bytes, kernel_nnz=nnz_long, kernel_rows=rows_long)
+    else:
+        if name == "local":
+            import spfa_local
+            n, d, wsz = 65536, 64, 128
+            q, k, v = syn.qkv(n, d, dtype=dtype, device=dev, seed=0)
+            nnz = syn.local_nnz(n, wsz)
+            w["call"] = lambda st: spfa_local.forward(q, k, v, st[0], st[1], st[2], wsz)
+            w["params"] = {"LOCAL_SIZE": wsz}
+            live = n
+        elif name == "local_1d":
+            import spfa_local_1d_dilated
+            n, d, wsz, dil = 262144, 128, 256, 2
+            q, k, v = syn.qkv(n, d, dtype=dtype, device=dev, seed=0, scale=0.5)
+            nnz = syn.local_1d_dilated_nnz(n, wsz, dil)
+            w["call"] = lambda st: spfa_local_1d_dilated.forward(q, k, v, st[0], st[1], st[2], wsz, dil)
+            w["params"] = {"LOCAL_SIZE": wsz, "DILATE_FACTOR": dil}
+            live = n
+        elif name == "local_2d":
+            import spfa_local_2d_dilated
+            n, d, blk, dil = 262144, 128, 256, 2
+            q, k, v = syn.qkv(n, d, dtype=dtype, device=dev, seed=0, scale=0.5)
+            nnz = syn.local_2d_dilated_nnz(n, blk, dil)
+            w["call"] = lambda st: spfa_local_2d_dilated.forward(q, k, v, st[0], st[1], st[2], blk, dil, False)
+            w["params"] = {"BLOCK_SIZE": blk, "DILATE_FACTOR": dil}
+            live = (n // blk) * min(blk, (blk - 1) // (dil + 1) + 1)
+        else:
+            import spfa_global_no_local
+            n, d, g, wsz = 1 << 20, 64, 64, 64
+            q, k, v = syn.qkv(n, d, dtype=dtype, device=dev, seed=0)
+            globs = syn.global_indices(n, g, device=dev, seed=0)
+            nnz = syn.global_no_local_nnz(n, globs, wsz)
+            w["call"] = lambda st: spfa_global_no_local.forward(q, k, v, st[0], st[1], st[2], globs, wsz)
+            w["params"] = {"n_globals": g, "LOCAL_SIZE": wsz}
+            w["globs"] = globs
+            live = n
+        total = syn.implicit_mask_bytes(n, d, es, live_rows=live)
+        w.update(n=n, d=d, nnz=nnz, bytes_total=total, bytes_gathered=nnz * 2 * d * es, bound="hbm",
+                 kernel_bytes=total, kernel_nnz=nnz, kernel_rows=live)
+    w.update(q=q, k=k, v=v)
+    return w
+
+
+def verify_sample(w, state, torch, rows=192):
+    """Max-abs error of `rows` sampled output rows against the float64 CPU oracle."""
+    import numpy as np
+    from oracle import c_oracle
+    from oracle import spfa_oracle as so
+    n = w["n"]
+    g = torch.Generator().manual_seed(123)
+    idx = torch.sort(torch.randperm(n, generator=g)[:rows])[0]
+    qs = w["q"][idx.to("cuda")].float().cpu().numpy().astype(np.float64)
+    kk = w["k"].float().cpu().numpy().astype(np.float64)
+    vv = w["v"].float().cpu().numpy().astype(np.float64)
+    name = w["name"]
+    idx_np = idx.numpy()
+    if name.startswith("csr"):
+        ro, ci = w["csr"]
+        ro_c = ro.cpu().numpy()
+        lists = [ci[ro_c[i]:ro_c[i + 1]].cpu().numpy() for i in idx_np]
+    elif name == "coo_zipf":
+        r, c = w["coo"]
+        lists = [c[r == int(i)].cpu().numpy() for i in idx_np[:32]]
+        idx_np, qs = idx_np[:32], qs[:32]
+    elif name == "local":
+        lists = [so.live_local(n, w["params"]["LOCAL_SIZE"], int(i)) for i in idx_np]
+    elif name == "local_1d":
+        p = w["params"]
+        lists = [so.live_local_1d_dilated(n, p["LOCAL_SIZE"], p["DILATE_FACTOR"], int(i)) for i in idx_np]
+    elif name == "local_2d":
+        p = w["params"]
+        lists = [so.live_local_2d_dilated(n, p["BLOCK_SIZE"], p["DILATE_FACTOR"], int(i)) for i in idx_np]
+    else:
+        gl = w["globs"].cpu().numpy()
+        # one global row is enough (each is a 1M-column row for the CPU)
+        idx_np = np.concatenate([idx_np[:63], gl[:1].astype(np.int64)])
+        qs = w["q"][torch.as_tensor(idx_np).to("cuda")].float().cpu().numpy().astype(np.float64)
+        gset = set(int(x) for x in gl)
+        wsz = w["params"]["LOCAL_SIZE"]
+
+        def live(i):
+            low, up = max(0, i - wsz), min(n, i + wsz + 1)
+            if i in gset:
+                return np.concatenate([np.arange(0, low), np.arange(up, n)])
+            return np.array([x for x in gl if x < low or x >= up], dtype=np.int64)
+        lists = [live(int(i)) for i in idx_np]
+    off = np.zeros(len(lists) + 1, dtype=np.int64)
+    np.cumsum([len(x) for x in lists], out=off[1:])
+    cols = np.concatenate(lists).astype(np.int64) if len(lists) else np.zeros(0, np.int64)
+    ref_out, ref_m, ref_l = c_oracle.csr(qs, kk, vv, off, cols)
+    sel = torch.as_tensor(idx_np).to("cuda")
+    got = state[2][sel].float().cpu().numpy().astype(np.float64)
+    live_rows = ref_l > 0
+    err = float(np.abs(got[live_rows] - ref_out[live_rows]).max()) if live_rows.any() else 0.0
+    return err, int(live_rows.sum())
+
+
+def cpu_baseline(w, torch, target_s=12.0):
+    """The reference's verification formulation on host cores: dense masked
+    scaled_dot_product_attention in fp32 over a block of query rows against all keys."""
+    import numpy as np
+    name = w["name"]
+    if not name.startswith("csr"):
+        return None
+    n, d = w["n"], w["d"]
+    ro, ci = w["csr"]
+    ro_c, ci_c = ro.cpu(), ci.cpu()
+    k = w["k"].float().cpu()
+    v = w["v"].float().cpu()
+    q = w["q"].float().cpu()
+    block = min(1024, n)
+    g = torch.Generator().manual_seed(7)
+
+    def one_block():
+        rows = torch.sort(torch.randperm(n, generator=g)[:block])[0]
+        mask = torch.zeros(block, n, dtype=torch.bool)
+        nnz = 0
+        for j, i in enumerate(rows.tolist()):
+            cols = ci_c[ro_c[i]:ro_c[i + 1]]
+            mask[j, cols] = True
+            nnz += cols.numel()
+        qb = q[rows]
+        t0 = time.perf_counter()
+        torch.nn.functional.scaled_dot_product_attention(qb, k, v, attn_mask=mask)
+        return time.perf_counter() - t0, nnz
+
+    one_block()  # warm-up
+    t_tot, nnz_tot, blocks = 0.0, 0, 0
+    t_begin = time.perf_counter()
+    while (time.perf_counter() - t_begin) < target_s and blocks < 64:
+        t, z = one_block()
+        t_tot += t
+        nnz_tot += z
+        blocks += 1
+    gflops = 4.0 * d * nnz_tot / t_tot / 1e9
+    dense_gflops = 4.0 * d * block * blocks * n / t_tot / 1e9
+    return {
+        "value": gflops, "unit": "GFLOP/s (nnz-counted)", "cores": torch.get_num_threads(),
+        "kind": "port",
+        "sample": "%d blocks of %d random query rows x all %d keys, torch CPU dense masked "
+                  "scaled_dot_product_attention fp32 (the reference's verification formulation); "
+                  "%.2f s of SDPA time, %d live positions" % (blocks, block, n, t_tot, nnz_tot),
+        "dense_gflops": dense_gflops, "host_cpus": os.cpu_count(),
+    }
+
+
+def cpu_sparse_port(w, torch, rows=8192):
+    """The row-wise C restatement (float64, OpenMP) on a sample of rows - the same sparse algorithm
+    as the GPU path, for scale."""
+    import numpy as np
+    from oracle import c_oracle
+    if not w["name"].startswith("csr"):
+        return None
+    n, d = w["n"], w["d"]
+    ro, ci = w["csr"]
+    ro_c, ci_c = ro.cpu().numpy(), ci.cpu().numpy()
+    g = torch.Generator().manual_seed(11)
+    idx = torch.sort(torch.randperm(n, generator=g)[:min(rows, n)])[0].numpy()
+    lens = ro_c[idx + 1] - ro_c[idx]
+    off = np.zeros(len(idx) + 1, dtype=np.int64)
+    np.cumsum(lens, out=off[1:])
+    cols = np.concatenate([ci_c[ro_c[i]:ro_c[i + 1]] for i in idx]).astype(np.int64)
+    qs = w["q"].float().cpu().numpy().astype(np.float64)[idx]
+    kk = w["k"].float().cpu().numpy().astype(np.float64)
+    vv = w["v"].float().cpu().numpy().astype(np.float64)
+    c_oracle.csr(qs[:64], kk, vv, off[:65], cols[:off[64]])
+    t0 = time.perf_counter()
+    c_oracle.csr(qs, kk, vv, off, cols)
+    t = time.perf_counter() - t0
+    return {"value": 4.0 * d * int(lens.sum()) / t / 1e9, "unit": "GFLOP/s (nnz-counted)",
+            "cores": os.cpu_count(), "kind": "port",
+            "sample": "%d random rows, row-wise sparse float64 C restatement with OpenMP, %.2f s" % (len(idx), t)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="csr_zipf", choices=sorted(WORKLOADS))
+    ap.add_argument("--dtype", default="f32", choices=["f32", "f16", "bf16"])
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    a = ap.parse_args()
+    if a.gpus != 1:
+        sys.exit("bench.py measures one GPU: this path is a single-GPU kernel and every box here has "
+                 "one GPU; run with --gpus 1")
+
+    import torch
+    import spfa_synth as syn
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU")
+    torch.cuda.set_device(0)
+    dtype = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}[a.dtype]
+    lib = load_library()
+    w = make_workload(a.workload, dtype, torch, syn, int(lib.spfa_explicit_inline_row_limit()))
+    n, d, nnz = w["n"], w["d"], w["nnz"]
+
+    n_states = a.steps + a.warmup
+    state_bytes = n * d * torch.tensor([], dtype=dtype).element_size()
+    n_alloc = max(1, min(n_states, int(4e9 // max(1, state_bytes))))
+    states = [syn.fresh_state(n, d, dtype=dtype, device="cuda", state_dtype=torch.float32)
+              for _ in range(n_alloc)]
+
+    def fresh(i):
+        st = states[i % n_alloc]
+        if i >= n_alloc:  # recycled: reset outside the timed region is not possible, so do it here
+            st[0].fill_(-float("inf"))
+            st[1].zero_()
+        return st
+
+    ev = HipEvents()
+    for i in range(a.warmup):
+        w["call"](fresh(i))
+    torch.cuda.synchronize()
+
+    # timed region: exactly K steps
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(a.steps):
+        w["call"](fresh(a.warmup + i))
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    ms_per_step = dt / a.steps * 1e3
+
+    # dominant-kernel time: HIP events recorded inside the library around that kernel only
+    kernel_ms = []
+    lib.spfa_set_kernel_events(ev.start, ev.stop)
+    for i in range(min(a.steps, 10)):
+        st = states[i % n_alloc]
+        st[0].fill_(-float("inf"))
+        st[1].zero_()
+        torch.cuda.synchronize()
+        w["call"](st)
+        kernel_ms.append(ev.elapsed_ms())
+    lib.spfa_set_kernel_events(None, None)
+    torch.cuda.synchronize()
+    k_avg = sum(kernel_ms) / len(kernel_ms)
+
+    err, checked = verify_sample(w, states[0], torch)
+    tol = 1e-4 if dtype == torch.float32 else 2e-2
+
+    flops = syn.attention_flops(nnz, d)
+    achieved_gbs = w["kernel_bytes"] / (k_avg * 1e-3) / 1e9
+    out = {
+        "metric": "masked-attn GFLOP/s (nnz-counted) + effective HBM GB/s, CSR N=128K d=64 fp32",
+        "value": flops / (ms_per_step * 1e-3) / 1e9,
+        "unit": "GFLOP/s",
+        "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": ms_per_step,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": a.dtype, "data": "synthetic",
+        "config": {"workload": w["desc"], "n": n, "d": d, "nnz": nnz, "seed": 0,
+                   "index_dtypes": "uint64 offsets / uint32 columns", "state": "fresh m=-inf l=0 each step"},
+        "effective_gathered_GBs": w["bytes_gathered"] / (ms_per_step * 1e-3) / 1e9,
+        "algorithmic_GBs": w["bytes_total"] / (ms_per_step * 1e-3) / 1e9,
+        "roofline": {"bound": "hbm", "achieved": achieved_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": achieved_gbs / HBM_PEAK_GBS, "traffic": None,
+                     "kernel": "segments_kernel" if a.workload in ("csr_zipf", "csr_bernoulli", "coo_zipf", "global") else "rows_kernel",
+                     "kernel_ms_avg": k_avg, "kernel_ms_min": min(kernel_ms),
+                     "algorithmic_bytes": w["kernel_bytes"], "kernel_nnz": w["kernel_nnz"],
+                     "kernel_rows": w["kernel_rows"], "call_algorithmic_bytes": w["bytes_total"],
+                     "call_gathered_bytes": w["bytes_gathered"]},
+        "parity": {"max_abs_err": err, "rows_checked": checked, "tolerance": tol, "ok": bool(err <= tol)},
+    }
+    if not a.no_cpu:
+        cb = cpu_baseline(w, torch)
+        if cb is not None:
+            out["cpu_baseline"] = cb
+            sp = cpu_sparse_port(w, torch)
+            if sp is not None:
+                out["cpu_sparse_port"] = sp
+    print(json.dumps(out))
+    if err > tol:
+        sys.exit("parity check failed: max abs error %.3e > %.1e" % (err, tol))
+
+
+if __name__ == "__main__":
+    main()

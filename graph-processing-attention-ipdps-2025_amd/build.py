@@ -103,6 +103,48 @@ def build_ext(workers: int):
     return outs
 
 
+def check_loop_nests(workers: int | None = None) -> None:
+    """Compile the engine to assembly and check the loop nests the compiler formed.
+
+    segments_kernel fetches its work index with a cross-lane read at the top of its work loop, so
+    every lane of a wavefront must take every trip of that loop together.  The optimiser has been
+    seen to split the loop into an outer and an inner loop (one back edge for the lanes that write
+    the row statistics, one for the rest), after which the inner loop spins on work index 0.  The
+    source keeps a convergent operation in the loop's single latch; this check fails the build if a
+    segments_kernel ever shows more than the two source-level loops (work loop + candidate loop),
+    or a rows/merge kernel more than one.
+    """
+    import re
+    workers = workers or min(8, os.cpu_count() or 4)
+    os.makedirs(OBJ, exist_ok=True)
+    jobs = []
+    for mname, mid in MASK_KINDS.items():
+        for tname, tcpp in ELEM_TYPES.items():
+            asm = os.path.join(OBJ, "inst_%s_%s.s" % (mname, tname))
+            jobs.append((asm, [HIPCC, *HIP_FLAGS, "-DSPFA_INST_MASK=%d" % mid,
+                               "-DSPFA_INST_T=%s" % tcpp, "-S", "--cuda-device-only",
+                               os.path.join(CSRC, "spfa_inst.hip"), "-o", asm]))
+    with cf.ThreadPoolExecutor(max_workers=workers) as ex:
+        list(ex.map(lambda j: _run(j[1]), jobs))
+    for asm, _ in jobs:
+        depth, name = {}, None
+        for line in open(asm):
+            m = re.match(r"^(_ZN4spfa\w+):", line)
+            if m:
+                name = m.group(1)
+                depth[name] = 0
+            m = re.search(r"Loop Header: Depth=(\d+)", line)
+            if m and name:
+                depth[name] = max(depth[name], int(m.group(1)))
+        for kname, dep in depth.items():
+            limit = 2 if "segments_kernel" in kname else 1
+            if dep > limit:
+                raise RuntimeError("%s: %s has loop depth %d (limit %d): the work loop was split"
+                                   % (os.path.basename(asm), kname, dep, limit))
+        if not any("segments_kernel" in k for k in depth):
+            raise RuntimeError("no segments_kernel found in " + asm)
+
+
 def build_all(workers: int | None = None):
     workers = workers or min(8, os.cpu_count() or 4)
     lib = build_lib(workers)
@@ -114,9 +156,14 @@ if __name__ == "__main__":
     ap = argparse.ArgumentParser()
     ap.add_argument("--lib", action="store_true")
     ap.add_argument("--ext", action="store_true")
+    ap.add_argument("--check", action="store_true", help="only check the compiled loop nests")
     ap.add_argument("-j", type=int, default=None)
     a = ap.parse_args()
     w = a.j or min(8, os.cpu_count() or 4)
+    if a.check:
+        check_loop_nests(w)
+        print("loop nests ok")
+        sys.exit(0)
     if a.lib or not a.ext:
         print(build_lib(w))
     if a.ext or not a.lib:

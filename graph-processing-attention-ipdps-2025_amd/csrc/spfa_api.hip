@@ -26,11 +26,13 @@ inline int64_t pick_segment(int64_t nnz_long) {
   return clamp64(pow2_ceil(nnz_long / 65536 + 1), 256, 8192);
 }
 
+constexpr int64_t kExplicitInlineRowLimit = 32;
+
 EngineSizing size_csr(int64_t n_q, int64_t nnz) {
   EngineSizing s{};
   s.nnz_bound = nnz;
   s.max_deg = nnz;
-  s.short_max = 32;
+  s.short_max = kExplicitInlineRowLimit;
   s.seg = pick_segment(nnz);
   s.n_long_bound = n_q;
   return s;
@@ -154,9 +156,23 @@ size_t global_flag_bytes(int64_t n) { return align_up((size_t)((n + 3) / 4 * 4),
 
 }  // namespace
 
+namespace spfa {
+KernelEvents& kernel_events() {
+  static KernelEvents ev;
+  return ev;
+}
+}  // namespace spfa
+
 extern "C" {
 
 int spfa_version(void) { return 1; }
+
+int64_t spfa_explicit_inline_row_limit(void) { return kExplicitInlineRowLimit; }
+
+void spfa_set_kernel_events(void* start, void* stop) {
+  kernel_events().start = (hipEvent_t)start;
+  kernel_events().stop = (hipEvent_t)stop;
+}
 
 const char* spfa_status_string(int status) {
   switch (status) {

@@ -414,6 +414,13 @@ inline WorkspaceLayout engine_workspace(const EngineSizing& s, int64_t n_q, int6
   return w;
 }
 
+// optional event pair recorded around the dominant kernel (see spfa_set_kernel_events)
+struct KernelEvents {
+  hipEvent_t start = nullptr;
+  hipEvent_t stop = nullptr;
+};
+KernelEvents& kernel_events();
+
 inline int device_cu_count() {
   static int cus = 0;
   if (cus == 0) {
@@ -449,17 +456,23 @@ int launch_engine(const Tensors& t, const Mask& mask, const EngineSizing& s, int
   const bool has_long = s.max_deg > s.short_max;
   if (has_long) hipLaunchKernelGGL(reset_counters_kernel, dim3(1), dim3(64), 0, stream, plan.cnt);
 
+  const KernelEvents ev = kernel_events();
+  const bool timed = ev.start != nullptr && ev.stop != nullptr;
   const int64_t rows_per_wg = 4 * Lay::GROUPS;
   const int64_t grid1 = (t.n_q + rows_per_wg - 1) / rows_per_wg;
+  if (timed && !has_long) (void)hipEventRecord(ev.start, stream);
   hipLaunchKernelGGL((rows_kernel<Lay, Mask>), dim3((unsigned)grid1), dim3(256), 0, stream, t, mask,
                      plan);
+  if (timed && !has_long) (void)hipEventRecord(ev.stop, stream);
   if (has_long) {
     int64_t grid2 = (int64_t)device_cu_count() * 8;
     int64_t need = ((int64_t)w.cap_items + 3) / 4;
     if (grid2 > need) grid2 = need;
     if (grid2 < 1) grid2 = 1;
+    if (timed) (void)hipEventRecord(ev.start, stream);
     hipLaunchKernelGGL((segments_kernel<Lay, Mask>), dim3((unsigned)grid2), dim3(256), 0, stream, t,
                        mask, plan);
+    if (timed) (void)hipEventRecord(ev.stop, stream);
     const int64_t grid3 = ((int64_t)w.cap_multi + rows_per_wg - 1) / rows_per_wg;
     hipLaunchKernelGGL((merge_kernel<Lay>), dim3((unsigned)grid3), dim3(256), 0, stream, t, plan);
   }

@@ -77,6 +77,18 @@ typedef struct spfa_problem {
 int spfa_version(void);
 const char* spfa_status_string(int status);
 
+/* Measurement aid; no counterpart in the reference.  While both handles are non-NULL
+ * (hipEvent_t passed as void*), every forward call records `start` on its stream immediately
+ * before, and `stop` immediately after, the launch of the kernel that does the bulk of the
+ * call's attention work (the segment kernel when a mask has long rows, else the row kernel), so a
+ * benchmark can time that one kernel with hipEventElapsedTime.  Process-wide and not
+ * thread-safe: set it, run, read the events, reset it with NULLs. */
+void spfa_set_kernel_events(void* start, void* stop);
+
+/* Rows of an explicit mask with at most this many entries are finished by the row kernel; longer
+ * rows go through the segment kernel.  Exposed so a benchmark can attribute bytes to kernels. */
+int64_t spfa_explicit_inline_row_limit(void);
+
 /* CSR: row i attends col_ind[row_off[i] .. row_off[i+1]).  row_off has n_q+1 entries of
  * row_off_bytes (4 or 8) bytes each, col_ind has nnz 4-byte entries; signed and unsigned
  * index tensors are bit-identical in range.  The reference's value vector is never read
