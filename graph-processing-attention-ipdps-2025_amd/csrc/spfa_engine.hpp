@@ -4,9 +4,10 @@
 // it has (deg) and which column the t-th candidate is.  The engine walks those candidates with
 // an online softmax.  Work decomposition:
 //
-//   rows_kernel      one group of LPR lanes per query row (64/LPR rows per wavefront).  Rows
-//                    with deg <= short_max are finished on the spot; longer rows are cut into
-//                    segments of `seg` candidates that are appended to a work list.
+//   plan_kernel      one thread per query row; rows with more than short_max candidates are cut
+//                    into segments of `seg` candidates that are appended to a work list.
+//   rows_kernel      one group of LPR lanes per query row (64/LPR rows per wavefront) finishes
+//                    the rows with deg <= short_max on the spot.
 //   segments_kernel  persistent grid; each wavefront pulls segments off the work list, its
 //                    64/LPR groups take interleaved candidates, the groups are merged with
 //                    cross-lane moves, and the result is either final (single-segment row) or a
@@ -202,6 +203,69 @@ __device__ __forceinline__ void load_q(const Tensors& t, int64_t row, int c, flo
   Lay::unpack(r, q);
 }
 
+// inclusive prefix sum over the wavefront
+__device__ __forceinline__ uint32_t wave_inclusive_sum(uint32_t x, int lane) {
+#pragma unroll
+  for (int off = 1; off < kWave; off <<= 1) {
+    uint32_t y = (uint32_t)__builtin_amdgcn_ds_bpermute(((lane - off) & (kWave - 1)) << 2, (int)x);
+    if (lane >= off) x += y;
+  }
+  return x;
+}
+
+// One thread per query row: rows longer than short_max are cut into segments of plan.seg
+// candidates.  Each wavefront reserves room for all its rows with one atomic per counter (the
+// counters are shared by the whole grid, so per-row atomics would serialise on them).
+template <class Mask>
+__global__ __launch_bounds__(256) void plan_kernel(int64_t n_q, Mask mask, Plan plan) {
+  const int lane = lane_id();
+  const int64_t row = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  int64_t deg = 0;
+  if (row < n_q) deg = mask.row(row).deg;
+  const bool is_long = deg > plan.short_max;
+  if (__builtin_amdgcn_ballot_w64(is_long) == 0) return;  // same answer in every lane
+  const uint32_t nseg = is_long ? (uint32_t)((deg + plan.seg - 1) / plan.seg) : 0u;
+  const uint32_t multi = nseg > 1 ? 1u : 0u;
+  const uint32_t npart = multi ? nseg : 0u;
+  const uint32_t inc_items = wave_inclusive_sum(nseg, lane);
+  const uint32_t inc_part = wave_inclusive_sum(npart, lane);
+  const uint32_t inc_multi = wave_inclusive_sum(multi, lane);
+  uint32_t base_items = 0, base_part = 0, base_multi = 0, ok = 1;
+  if (lane == kWave - 1) {
+    base_items = atomicAdd(&plan.cnt->n_items, inc_items);
+    if (inc_part) base_part = atomicAdd(&plan.cnt->n_partials, inc_part);
+    if (inc_multi) base_multi = atomicAdd(&plan.cnt->n_multi, inc_multi);
+    if (base_items + inc_items > plan.cap_items || base_part + inc_part > plan.cap_partials ||
+        base_multi + inc_multi > plan.cap_multi) {
+      ok = 0;
+      atomicOr(&plan.cnt->overflow, 1u);
+    }
+  }
+  base_items = (uint32_t)__builtin_amdgcn_readlane((int)base_items, kWave - 1);
+  base_part = (uint32_t)__builtin_amdgcn_readlane((int)base_part, kWave - 1);
+  base_multi = (uint32_t)__builtin_amdgcn_readlane((int)base_multi, kWave - 1);
+  ok = (uint32_t)__builtin_amdgcn_readlane((int)ok, kWave - 1);
+  if (!ok || !is_long) return;
+  const uint32_t my_item = base_items + inc_items - nseg;
+  const uint32_t my_slot = base_part + inc_part - npart;
+  if (multi) {
+    MultiRow mr;
+    mr.row = (int32_t)row;
+    mr.slot0 = (int32_t)my_slot;
+    mr.nseg = (int32_t)nseg;
+    mr.pad = 0;
+    plan.multi[base_multi + inc_multi - 1] = mr;
+  }
+  for (uint32_t j = 0; j < nseg; j++) {
+    Item it;
+    it.row = (int32_t)row;
+    it.seg = (int32_t)j;
+    it.slot = multi ? (int32_t)(my_slot + j) : -1;
+    it.pad = 0;
+    plan.items[my_item + j] = it;
+  }
+}
+
 template <class Lay, class Mask>
 __global__ __launch_bounds__(256) void rows_kernel(Tensors t, Mask mask, Plan plan) {
   using T = typename Lay::elem;
@@ -236,44 +300,8 @@ __global__ __launch_bounds__(256) void rows_kernel(Tensors t, Mask mask, Plan pl
     attend<Lay, Mask, Lay::U_SHORT>(mask, rc, (const T*)t.k, (const T*)t.v, t.d, scale, q, 0, deg, 1,
                                     c, m, l, acc);
     finish_row<Lay>(t, row, c, m, l, acc);
-    return;
   }
-
-  // long row: hand its segments to the work list
-  const uint32_t nseg = (uint32_t)((deg + plan.seg - 1) / plan.seg);
-  uint32_t base = 0, slot0 = 0;
-  int okw = 1;
-  if (c == 0) {
-    base = atomicAdd(&plan.cnt->n_items, nseg);
-    if (base + nseg > plan.cap_items) okw = 0;
-    if (nseg > 1) {
-      slot0 = atomicAdd(&plan.cnt->n_partials, nseg);
-      uint32_t mp = atomicAdd(&plan.cnt->n_multi, 1u);
-      if (slot0 + nseg > plan.cap_partials || mp >= plan.cap_multi) okw = 0;
-      if (okw) {
-        MultiRow mr;
-        mr.row = (int32_t)row;
-        mr.slot0 = (int32_t)slot0;
-        mr.nseg = (int32_t)nseg;
-        mr.pad = 0;
-        plan.multi[mp] = mr;
-      }
-    }
-    if (!okw) atomicOr(&plan.cnt->overflow, 1u);
-  }
-  const int leader = g * LPR;
-  base = (uint32_t)shfl_i32((int)base, leader);
-  slot0 = (uint32_t)shfl_i32((int)slot0, leader);
-  okw = shfl_i32(okw, leader);
-  if (!okw) return;
-  for (uint32_t j = c; j < nseg; j += LPR) {
-    Item it;
-    it.row = (int32_t)row;
-    it.seg = (int32_t)j;
-    it.slot = nseg > 1 ? (int32_t)(slot0 + j) : -1;
-    it.pad = 0;
-    plan.items[base + j] = it;
-  }
+  // longer rows were cut into segments by plan_kernel and belong to segments_kernel
 }
 
 template <class Lay, class Mask>
@@ -454,7 +482,11 @@ int launch_engine(const Tensors& t, const Mask& mask, const EngineSizing& s, int
   if (t.n_q == 0) return 0;
 
   const bool has_long = s.max_deg > s.short_max;
-  if (has_long) hipLaunchKernelGGL(reset_counters_kernel, dim3(1), dim3(64), 0, stream, plan.cnt);
+  if (has_long) {
+    hipLaunchKernelGGL(reset_counters_kernel, dim3(1), dim3(64), 0, stream, plan.cnt);
+    hipLaunchKernelGGL((plan_kernel<Mask>), dim3((unsigned)((t.n_q + 255) / 256)), dim3(256), 0,
+                       stream, t.n_q, mask, plan);
+  }
 
   const KernelEvents ev = kernel_events();
   const bool timed = ev.start != nullptr && ev.stop != nullptr;
