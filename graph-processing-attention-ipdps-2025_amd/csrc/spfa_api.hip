@@ -131,6 +131,39 @@ int dispatch_stride(const spfa_problem_t* p, const StrideMask& mask, const Engin
   return SPFA_ERR_UNSUPPORTED;
 }
 
+// Band / block masks whose rows are long enough go to the dense-tile kernel.
+int dispatch_band(const spfa_problem_t* p, int64_t w, int64_t stride, int64_t block, int64_t cnt,
+                  int use_nan, hipStream_t stream) {
+  BandArgs a{};
+  a.t = make_tensors(p);
+  a.n = p->n_q;
+  a.s = stride;
+  a.block = block;
+  a.cnt = cnt;
+  int64_t n_sub, len_max;
+  if (block > 0) {
+    n_sub = p->n_q / block;
+    len_max = cnt;
+    a.w = cnt;
+  } else {
+    n_sub = stride < p->n_q ? stride : p->n_q;
+    len_max = (p->n_q + stride - 1) / stride;
+    a.w = w < len_max ? w : len_max;
+  }
+  a.tiles_per_sub = (len_max + 127) / 128;
+  a.n_tiles = n_sub * a.tiles_per_sub;
+  if (a.n_tiles + 8 >= ((int64_t)1 << 31)) return -1;
+  switch (p->dtype) {
+    case SPFA_DTYPE_F32: return run_band<float>(a, use_nan, stream);
+    case SPFA_DTYPE_F16: return run_band<f16>(a, use_nan, stream);
+    case SPFA_DTYPE_BF16: return run_band<bf16>(a, use_nan, stream);
+  }
+  return -1;
+}
+
+// rows shorter than this are cheaper on the row-gather engine than on 32x32 tiles
+constexpr int64_t kBandTileMinRow = 32;
+
 int dispatch_global(const spfa_problem_t* p, const GlobalMask& mask, const EngineSizing& s,
                     void* ws, hipStream_t stream) {
   Tensors t = make_tensors(p);
@@ -284,6 +317,14 @@ int spfa_local_1d_dilated_forward(const spfa_problem_t* p, int64_t local_size, i
   EngineSizing s = size_stride(n, band_max_deg(n, local_size));
   rc = check_workspace(workspace, workspace_bytes, engine_workspace(s, n, p->d).total);
   if (rc) return rc;
+  {
+    const int64_t len_max = (n + dil_factor) / (dil_factor + 1);
+    const int64_t span = 2 * local_size + 1 < len_max ? 2 * local_size + 1 : len_max;
+    if (span >= kBandTileMinRow && dtype_ok(p->dtype)) {
+      rc = dispatch_band(p, local_size, dil_factor + 1, 0, 0, 0, (hipStream_t)stream);
+      if (rc >= 0) return rc;
+    }
+  }
   StrideMask mask{n, local_size, dil_factor + 1, 0, 0};
   return dispatch_stride(p, mask, s, 0, workspace, (hipStream_t)stream);
 }
@@ -312,6 +353,10 @@ int spfa_local_2d_dilated_forward(const spfa_problem_t* p, int64_t block_size, i
   EngineSizing s = size_stride(n, cnt);
   rc = check_workspace(workspace, workspace_bytes, engine_workspace(s, n, p->d).total);
   if (rc) return rc;
+  if (cnt >= kBandTileMinRow && dtype_ok(p->dtype)) {
+    rc = dispatch_band(p, 0, dil_factor + 1, block_size, cnt, use_nan ? 1 : 0, (hipStream_t)stream);
+    if (rc >= 0) return rc;
+  }
   StrideMask mask{n, 0, dil_factor + 1, block_size, cnt};
   return dispatch_stride(p, mask, s, use_nan ? 1 : 0, workspace, (hipStream_t)stream);
 }

@@ -1,0 +1,396 @@
+// Dense-tile attention for band and block masks on the gfx950 matrix cores.
+//
+// A band / block mask is a set of independent *subsequences*: position t of a subsequence is
+// token base + t*s, and query t attends keys u with |t - u| <= w inside the subsequence.
+//   Local                 one subsequence (base 0, s = 1)
+//   Local 1D dilated      s subsequences, one per residue class mod s
+//   Local 2D dilated      one subsequence per block (base b*B, cnt live tokens, w = everything)
+// so all three are the same tile problem.  One workgroup (4 wavefronts) owns 128 consecutive
+// query positions, one wavefront 32 of them; keys are streamed in tiles of 64 through LDS and
+// shared by the four wavefronts.
+//
+// Everything is computed transposed, S^T = K Q^T and O^T = V^T P^T, with 32x32 MFMA tiles.  In
+// the 32x32 result layout lane (r, h) = (lane % 32, lane / 32) holds column r, rows
+// 8*(v/4) + 4*h + v%4 for register v.  With queries on the columns
+//   - a query's running max / sum live in one lane pair (r,0),(r,1): the row reductions of the
+//     softmax are in-register plus one exchange across the two halves of the wavefront;
+//   - the P^T registers are already the B operand of the second product (the summation index of
+//     that product is the key, and any key order works as long as V^T uses the same one).
+// Half types use v_mfma_f32_32x32x16 (8 consecutive k per lane), fp32 uses v_mfma_f32_32x32x2
+// (no down-cast of fp32 inputs).
+#pragma once
+
+#include "spfa_engine.hpp"
+
+namespace spfa {
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+
+struct BandArgs {
+  Tensors t;
+  int64_t n;              // tokens
+  int64_t w;              // window half-width in subsequence positions
+  int64_t s;              // token stride of a subsequence
+  int64_t block;          // 0: band mode, else block size
+  int64_t cnt;            // block mode: live positions per block
+  int64_t tiles_per_sub;  // query tiles per subsequence (of the longest subsequence)
+  int64_t n_tiles;
+};
+
+template <typename T, int D>
+struct BandCfg {
+  static constexpr bool kF32 = sizeof(T) == 4;
+  static constexpr int BM = 128;  // queries per workgroup
+  static constexpr int BN = 64;   // keys per LDS tile
+  // K tile: [key][k] rows padded so that the 32 keys read by one operand fetch spread over the
+  // banks.  V tile: half types are stored transposed [e][key'] (16-byte operand reads), fp32
+  // row-major [key][e].
+  static constexpr int K_STRIDE = kF32 ? D + 2 : D + 8;
+  static constexpr int V_STRIDE = kF32 ? D + 8 : BN + 8;
+  static constexpr int K_ELEMS = BN * K_STRIDE;
+  static constexpr int V_ELEMS = kF32 ? BN * V_STRIDE : D * V_STRIDE;
+  static constexpr int LDS_BYTES = (K_ELEMS + V_ELEMS) * (int)sizeof(T);
+  static constexpr int EB = D / 32;                 // 32-row blocks of O^T
+  static constexpr int QREGS = kF32 ? D / 2 : D / 16;
+};
+
+// key order inside a 64-key tile for the transposed V tile of the half types: swap bits 2 and 3
+__device__ __forceinline__ int key_slot(int j) {
+  return (j & ~12) | ((j & 4) << 1) | ((j & 8) >> 1);
+}
+
+template <typename T>
+__device__ __forceinline__ f32x16 mfma16(const uint4v& a, const uint4v& b, f32x16 c) {
+  if constexpr (__is_same(T, bf16)) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a),
+                                                   __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+  } else {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a),
+                                                  __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+  }
+}
+
+template <typename T>
+__device__ __forceinline__ uint32_t pack2(float lo, float hi) {
+  typedef T t2 __attribute__((ext_vector_type(2)));
+  t2 x = {(T)lo, (T)hi};
+  return __builtin_bit_cast(uint32_t, x);
+}
+
+template <typename T, int D>
+__global__ __launch_bounds__(256, 2) void band_kernel(BandArgs a) {
+  using C = BandCfg<T, D>;
+  constexpr bool kF32 = C::kF32;
+  constexpr int BM = C::BM, BN = C::BN, EB = C::EB;
+  __shared__ __attribute__((aligned(16))) T lds[C::K_ELEMS + C::V_ELEMS];
+  T* Ks = lds;
+  T* Vs = lds + C::K_ELEMS;
+
+  // workgroups are dealt round-robin to the 8 XCDs: give each XCD a contiguous run of tiles so
+  // that neighbouring query tiles (which share most of their keys) meet in one L2
+  const int64_t per_xcd = (a.n_tiles + 7) / 8;
+  const int64_t lt = (int64_t)(blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+  if (lt >= a.n_tiles) return;
+  const int64_t sub = lt / a.tiles_per_sub;
+  const int64_t tile = lt - sub * a.tiles_per_sub;
+  int64_t base, len;
+  if (a.block > 0) {
+    base = sub * a.block;
+    len = a.cnt;
+  } else {
+    base = sub;
+    len = (a.n - sub + a.s - 1) / a.s;
+  }
+  const int64_t t0 = tile * BM;
+  if (t0 >= len) return;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int r = lane & 31, h = lane >> 5;
+  const int64_t tw0 = t0 + 32 * wave;  // first query of this wavefront
+  const int64_t tq = tw0 + r;          // this lane's query
+  const bool q_ok = tq < len;
+  const T* Qp = (const T*)a.t.q;
+  const T* Kp = (const T*)a.t.k;
+  const T* Vp = (const T*)a.t.v;
+
+  // ---- Q^T operand, kept in registers
+  uint4v qh[kF32 ? 1 : C::QREGS];
+  float qf[kF32 ? C::QREGS : 1];
+  {
+    const T* qrow = Qp + (base + (q_ok ? tq : len - 1) * a.s) * D;
+    if constexpr (kF32) {
+#pragma unroll
+      for (int c4 = 0; c4 < D / 4; c4++) {
+        float4v x = *reinterpret_cast<const float4v*>(qrow + 4 * c4);
+        qf[2 * c4] = h ? x[1] : x[0];
+        qf[2 * c4 + 1] = h ? x[3] : x[2];
+      }
+    } else {
+#pragma unroll
+      for (int ks = 0; ks < C::QREGS; ks++)
+        qh[ks] = *reinterpret_cast<const uint4v*>(qrow + 16 * ks + 8 * h);
+    }
+  }
+
+  f32x16 o[EB];
+#pragma unroll
+  for (int eb = 0; eb < EB; eb++)
+#pragma unroll
+    for (int v = 0; v < 16; v++) o[eb][v] = 0.f;
+  float m = kNegInf;  // running max in log2 units
+  float l = 0.f;      // running sum over this lane's half of the keys
+  const float sc = 1.4426950408889634f / sqrtf((float)D);
+
+  int64_t u_lo = t0 - a.w;
+  if (u_lo < 0) u_lo = 0;
+  int64_t u_hi = t0 + BM + a.w;
+  if (u_hi > len || u_hi < 0) u_hi = len;
+
+  for (int64_t ut = u_lo; ut < u_hi; ut += BN) {
+    __syncthreads();  // the previous tile has been consumed
+    // ---- stage K and V rows ut .. ut+63 (zeros past the end of the subsequence)
+    if constexpr (kF32) {
+      constexpr int CH = D / 4;  // 16-byte chunks per row
+#pragma unroll
+      for (int it = 0; it < BN * CH / 256; it++) {
+        const int idx = it * 256 + tid;
+        const int j = idx / CH, c = idx % CH;
+        const int64_t u = ut + j;
+        float4v kx = {0.f, 0.f, 0.f, 0.f}, vx = {0.f, 0.f, 0.f, 0.f};
+        if (u < len) {
+          const int64_t off = (base + u * a.s) * D + 4 * c;
+          kx = *reinterpret_cast<const float4v*>(Kp + off);
+          vx = *reinterpret_cast<const float4v*>(Vp + off);
+        }
+        float* kd = (float*)Ks + j * C::K_STRIDE + 4 * c;  // 8-byte aligned rows
+        kd[0] = kx[0]; kd[1] = kx[1]; kd[2] = kx[2]; kd[3] = kx[3];
+        *reinterpret_cast<float4v*>((float*)Vs + j * C::V_STRIDE + 4 * c) = vx;
+      }
+    } else {
+      constexpr int CH = D / 8;
+#pragma unroll
+      for (int it = 0; it < BN * CH / 256; it++) {
+        const int idx = it * 256 + tid;
+        const int j = idx / CH, c = idx % CH;
+        const int64_t u = ut + j;
+        uint4v kx = {0u, 0u, 0u, 0u};
+        if (u < len) kx = *reinterpret_cast<const uint4v*>(Kp + (base + u * a.s) * D + 8 * c);
+        *reinterpret_cast<uint4v*>(Ks + j * C::K_STRIDE + 8 * c) = kx;
+      }
+      // V: a lane takes the key pair (2*jp, 2*jp+1) and 8 columns e, and writes the 8 packed
+      // pairs down a column of the transposed tile
+#pragma unroll
+      for (int it = 0; it < (BN / 2) * CH / 256; it++) {
+        const int jp = lane & 31;
+        const int c = (lane >> 5) + 2 * (wave + 4 * it);
+        const int64_t u = ut + 2 * jp;
+        uint4v v0 = {0u, 0u, 0u, 0u}, v1 = {0u, 0u, 0u, 0u};
+        if (u < len) v0 = *reinterpret_cast<const uint4v*>(Vp + (base + u * a.s) * D + 8 * c);
+        if (u + 1 < len) v1 = *reinterpret_cast<const uint4v*>(Vp + (base + (u + 1) * a.s) * D + 8 * c);
+        const int slot = key_slot(2 * jp);
+        uint32_t* col = reinterpret_cast<uint32_t*>(Vs + (8 * c) * C::V_STRIDE + slot);
+#pragma unroll
+        for (int x = 0; x < 4; x++) {
+          // dword x of v0/v1 holds columns 2x, 2x+1
+          col[(2 * x) * (C::V_STRIDE / 2)] = (v0[x] & 0xffffu) | (v1[x] << 16);
+          col[(2 * x + 1) * (C::V_STRIDE / 2)] = (v0[x] >> 16) | (v1[x] & 0xffff0000u);
+        }
+      }
+    }
+    __syncthreads();
+
+    // ---- this wavefront's share of the tile: up to two 32-key blocks
+    // block jb holds keys ut + 32*jb .. +31; it matters iff it overlaps the wavefront's band
+    bool need[2];
+#pragma unroll
+    for (int jb = 0; jb < 2; jb++) {
+      const int64_t ub = ut + 32 * jb;
+      need[jb] = (tw0 < len) && (ub < len) && (ub <= tw0 + 31 + a.w) && (ub + 31 + a.w >= tw0);
+    }
+    if (!need[0] && !need[1]) continue;
+
+    f32x16 sreg[2];
+#pragma unroll
+    for (int jb = 0; jb < 2; jb++) {
+#pragma unroll
+      for (int v = 0; v < 16; v++) sreg[jb][v] = 0.f;
+      if (!need[jb]) continue;
+      if constexpr (kF32) {
+        const float* krow = (const float*)Ks + (32 * jb + r) * C::K_STRIDE + h;
+#pragma unroll
+        for (int ks = 0; ks < D / 2; ks++)
+          sreg[jb] = __builtin_amdgcn_mfma_f32_32x32x2f32(krow[2 * ks], qf[ks], sreg[jb], 0, 0, 0);
+      } else {
+        const T* krow = Ks + (32 * jb + r) * C::K_STRIDE + 8 * h;
+#pragma unroll
+        for (int ks = 0; ks < D / 16; ks++) {
+          uint4v kx = *reinterpret_cast<const uint4v*>(krow + 16 * ks);
+          sreg[jb] = mfma16<T>(kx, qh[ks], sreg[jb]);
+        }
+      }
+    }
+
+    // ---- scale, mask, running max
+    float mx = kNegInf;
+#pragma unroll
+    for (int jb = 0; jb < 2; jb++) {
+#pragma unroll
+      for (int v = 0; v < 16; v++) {
+        const int64_t u = ut + 32 * jb + 8 * (v / 4) + 4 * h + (v % 4);
+        const bool ok = need[jb] && q_ok && (u < len) && (u + a.w >= tq) && (u <= tq + a.w);
+        const float x = ok ? sreg[jb][v] * sc : kNegInf;
+        sreg[jb][v] = x;
+        mx = fmaxf(mx, x);
+      }
+    }
+    mx = fmaxf(mx, shfl_xor_f32(mx, 32));
+    const float m_new = fmaxf(m, mx);
+    const bool live = m_new > kNegInf;
+    const float alpha = live ? exp2f(m - m_new) : 1.f;
+    const float m_use = live ? m_new : 0.f;
+    float lsum = 0.f;
+#pragma unroll
+    for (int jb = 0; jb < 2; jb++)
+#pragma unroll
+      for (int v = 0; v < 16; v++) {
+        const float p = exp2f(sreg[jb][v] - m_use);  // exp2(-inf) = 0 for masked entries
+        sreg[jb][v] = p;
+        lsum += p;
+      }
+    l = l * alpha + lsum;
+    m = m_new;
+    if (__builtin_amdgcn_ballot_w64(alpha != 1.f) != 0) {
+#pragma unroll
+      for (int eb = 0; eb < EB; eb++)
+#pragma unroll
+        for (int v = 0; v < 16; v++) o[eb][v] *= alpha;
+    }
+
+    // ---- O^T += V^T P^T
+#pragma unroll
+    for (int jb = 0; jb < 2; jb++) {
+      if (!need[jb]) continue;
+      if constexpr (kF32) {
+#pragma unroll
+        for (int v = 0; v < 16; v++) {
+          const float* vrow = (const float*)Vs + (32 * jb + 8 * (v / 4) + 4 * h + (v % 4)) * C::V_STRIDE + r;
+#pragma unroll
+          for (int eb = 0; eb < EB; eb++)
+            o[eb] = __builtin_amdgcn_mfma_f32_32x32x2f32(vrow[32 * eb], sreg[jb][v], o[eb], 0, 0, 0);
+        }
+      } else {
+#pragma unroll
+        for (int sl = 0; sl < 2; sl++) {
+          uint4v pb;
+#pragma unroll
+          for (int x = 0; x < 4; x++)
+            pb[x] = pack2<T>(sreg[jb][8 * sl + 2 * x], sreg[jb][8 * sl + 2 * x + 1]);
+          const T* vcol = Vs + r * C::V_STRIDE + 32 * jb + 16 * sl + 8 * h;
+#pragma unroll
+          for (int eb = 0; eb < EB; eb++) {
+            uint4v va = *reinterpret_cast<const uint4v*>(vcol + 32 * eb * C::V_STRIDE);
+            o[eb] = mfma16<T>(va, pb, o[eb]);
+          }
+        }
+      }
+    }
+  }
+
+  // ---- finish: combine the two key halves, fold the incoming state in, write back
+  l += shfl_xor_f32(l, 32);
+  if (!q_ok || !(l > 0.f)) return;
+  const int64_t row = base + tq * a.s;
+  const bool sf = a.t.state_f32 != 0;
+  const float m_nat = m * 0.6931471805599453f;
+  float m_out = m_nat, l_out = l;
+  float wa = 0.f, wb = 1.f;
+  const float l_in = load_state<T>(a.t.l, row, sf);
+  if (l_in != 0.f) {
+    const float m_in = load_state<T>(a.t.m, row, sf);
+    m_out = fmaxf(m_nat, m_in);
+    wa = l_in * __expf(m_in - m_out);
+    wb = __expf(m_nat - m_out);
+    l_out = wa + l * wb;
+  }
+  const float inv = 1.f / l_out;
+  wb *= inv;
+  wa *= inv;
+  T* orow = (T*)a.t.out + row * D;
+#pragma unroll
+  for (int eb = 0; eb < EB; eb++) {
+#pragma unroll
+    for (int g4 = 0; g4 < 4; g4++) {
+      const int e = 32 * eb + 8 * g4 + 4 * h;
+      float x[4];
+#pragma unroll
+      for (int i = 0; i < 4; i++) x[i] = o[eb][4 * g4 + i] * wb;
+      if constexpr (kF32) {
+        if (wa != 0.f) {
+          float4v oi = *reinterpret_cast<const float4v*>(orow + e);
+#pragma unroll
+          for (int i = 0; i < 4; i++) x[i] += wa * oi[i];
+        }
+        float4v y = {x[0], x[1], x[2], x[3]};
+        *reinterpret_cast<float4v*>(orow + e) = y;
+      } else {
+        typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+        if (wa != 0.f) {
+          typedef T t4 __attribute__((ext_vector_type(4)));
+          t4 oi = *reinterpret_cast<const t4*>(orow + e);
+#pragma unroll
+          for (int i = 0; i < 4; i++) x[i] += wa * (float)oi[i];
+        }
+        u32x2 y = {pack2<T>(x[0], x[1]), pack2<T>(x[2], x[3])};
+        *reinterpret_cast<u32x2*>(orow + e) = y;
+      }
+    }
+  }
+  if (h == 0) {
+    store_state<T>(a.t.m, row, m_out, sf);
+    store_state<T>(a.t.l, row, l_out, sf);
+  }
+}
+
+// rows of a block mask that have no live column: out := NaN (m, l untouched)
+template <typename T>
+__global__ void band_dead_rows_kernel(T* out, int64_t n, int d, int64_t block, int64_t s) {
+  const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t row = idx / d;
+  if (row >= n) return;
+  if (((row % block) % s) != 0) out[idx] = from_f32<T>(__builtin_nanf(""));
+}
+
+template <typename T, int D>
+int launch_band(const BandArgs& a, int use_nan, hipStream_t stream) {
+  const KernelEvents ev = kernel_events();
+  const bool timed = ev.start != nullptr && ev.stop != nullptr;
+  if (a.n_tiles > 0) {
+    const int64_t grid = (a.n_tiles + 7) / 8 * 8;
+    if (timed) (void)hipEventRecord(ev.start, stream);
+    hipLaunchKernelGGL((band_kernel<T, D>), dim3((unsigned)grid), dim3(256), 0, stream, a);
+    if (timed) (void)hipEventRecord(ev.stop, stream);
+  }
+  if (a.block > 0 && use_nan && a.s > 1) {
+    const int64_t total = a.n * D;
+    hipLaunchKernelGGL((band_dead_rows_kernel<T>), dim3((unsigned)((total + 255) / 256)), dim3(256),
+                       0, stream, (T*)a.t.out, a.n, D, a.block, a.s);
+  }
+  return hipGetLastError() == hipSuccess ? 0 : 4;
+}
+
+// Returns -1 when the shape is not covered (caller falls back to the row-gather engine).
+template <typename T>
+int run_band_tiles(const BandArgs& a, int use_nan, hipStream_t stream) {
+  if (!aligned16(a.t.q) || !aligned16(a.t.k) || !aligned16(a.t.v) || !aligned16(a.t.out)) return -1;
+  if (a.t.d == 64) return launch_band<T, 64>(a, use_nan, stream);
+  if constexpr (sizeof(T) == 2) {
+    // (the fp32 tiles for d = 128 would need more than 64 KB of LDS)
+    if (a.t.d == 128) return launch_band<T, 128>(a, use_nan, stream);
+  }
+  return -1;
+}
+
+}  // namespace spfa

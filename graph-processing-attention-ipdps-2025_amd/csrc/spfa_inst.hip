@@ -16,6 +16,10 @@ int run_stride<SPFA_INST_T>(const Tensors& t, const StrideMask& mask, const Engi
                             int use_nan, void* ws, hipStream_t stream) {
   return run_engine<SPFA_INST_T, StrideMask>(t, mask, s, use_nan, ws, stream);
 }
+template <>
+int run_band<SPFA_INST_T>(const BandArgs& a, int use_nan, hipStream_t stream) {
+  return run_band_tiles<SPFA_INST_T>(a, use_nan, stream);
+}
 #elif SPFA_INST_MASK == 2
 template <>
 int run_global<SPFA_INST_T>(const Tensors& t, const GlobalMask& mask, const EngineSizing& s,
