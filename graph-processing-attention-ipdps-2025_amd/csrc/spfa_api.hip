@@ -185,7 +185,34 @@ int64_t block_live_count(int64_t block, int64_t s) {
   return cnt < block ? cnt : block;
 }
 
-size_t global_flag_bytes(int64_t n) { return align_up((size_t)((n + 3) / 4 * 4), 256); }
+// workspace of the global-minus-local path: [bitmap + counter][distinct rows][engine][partials]
+struct GlobalLayout {
+  size_t off_bits, off_uq, off_engine, off_pm, off_pl, off_pacc, total;
+  int64_t key_run, n_split;
+};
+
+GlobalLayout global_layout(int64_t n, int64_t n_globs, int64_t d) {
+  GlobalLayout g{};
+  const int64_t q_tiles = (n_globs + 127) / 128;
+  // enough key splits for ~2048 workgroups, none shorter than 512 keys
+  int64_t want = 2048 / q_tiles;
+  if (want < 1) want = 1;
+  int64_t run = (n + want - 1) / want;
+  if (run < 512) run = 512;
+  run = (run + 63) / 64 * 64;
+  g.key_run = run;
+  g.n_split = (n + run - 1) / run;
+  const size_t slots = (size_t)n_globs * (size_t)g.n_split;
+  size_t off = 0;
+  g.off_bits = off;   off = align_up(off + global_bits_words(n) * 4, 256);
+  g.off_uq = off;     off = align_up(off + (size_t)n_globs * 4, 256);
+  g.off_engine = off; off = align_up(off + engine_workspace(size_global(n, n_globs), n, d).total, 256);
+  g.off_pm = off;     off = align_up(off + slots * 4, 256);
+  g.off_pl = off;     off = align_up(off + slots * 4, 256);
+  g.off_pacc = off;   off = align_up(off + slots * (size_t)d * 4, 256);
+  g.total = off;
+  return g;
+}
 
 }  // namespace
 
@@ -367,7 +394,7 @@ size_t spfa_global_no_local_workspace_bytes(int64_t n, int64_t d, int dtype, int
   (void)dtype;
   (void)local_size;
   if (n < 1 || d < 1 || n_globals < 1) return 0;
-  return global_flag_bytes(n) + engine_workspace(size_global(n, n_globals), n, d).total;
+  return global_layout(n, n_globals, d).total;
 }
 
 int spfa_global_no_local_forward(const spfa_problem_t* p, const int32_t* global_inds,
@@ -381,16 +408,45 @@ int spfa_global_no_local_forward(const spfa_problem_t* p, const int32_t* global_
   if (rc) return rc;
   if (!global_inds) return SPFA_ERR_BAD_ARG;
   const int64_t n = p->n_q;
+  const GlobalLayout lay = global_layout(n, n_globals, p->d);
+  rc = check_workspace(workspace, workspace_bytes, lay.total);
+  if (rc) return rc;
+  char* base = (char*)workspace;
+  uint32_t* bits = (uint32_t*)(base + lay.off_bits);
+  int32_t* uq = (int32_t*)(base + lay.off_uq);
+  rc = prepare_global_rows(global_inds, n_globals, n, bits, uq, (hipStream_t)stream);
+  if (rc) return rc;
+
+  // dense tiles when the shape allows it
+  BandArgs a{};
+  a.t = make_tensors(p);
+  a.n = n;
+  a.w = local_size;
+  a.s = 1;
+  a.globs = global_inds;
+  a.n_globs = n_globals;
+  a.gbits = bits;
+  a.uq = uq;
+  a.n_uq = bits + (global_bits_words(n) - 1);
+  a.key_run = lay.key_run;
+  a.n_split = lay.n_split;
+  a.pm = (float*)(base + lay.off_pm);
+  a.pl = (float*)(base + lay.off_pl);
+  a.pacc = (float*)(base + lay.off_pacc);
+  const int64_t q_tiles = (n_globals + 127) / 128;
+  if (q_tiles * lay.n_split < ((int64_t)1 << 31) && n_globals < ((int64_t)1 << 31)) {
+    rc = -1;
+    switch (p->dtype) {
+      case SPFA_DTYPE_F32: rc = run_global_dense<float>(a, (hipStream_t)stream); break;
+      case SPFA_DTYPE_F16: rc = run_global_dense<f16>(a, (hipStream_t)stream); break;
+      case SPFA_DTYPE_BF16: rc = run_global_dense<bf16>(a, (hipStream_t)stream); break;
+    }
+    if (rc >= 0) return rc;
+  }
+
   EngineSizing s = size_global(n, n_globals);
-  const size_t flag_bytes = global_flag_bytes(n);
-  rc = check_workspace(workspace, workspace_bytes,
-                       flag_bytes + engine_workspace(s, n, p->d).total);
-  if (rc) return rc;
-  uint8_t* flags = (uint8_t*)workspace;
-  rc = mark_global_rows(global_inds, n_globals, n, flags, (hipStream_t)stream);
-  if (rc) return rc;
-  GlobalMask mask{n, local_size, global_inds, n_globals, flags};
-  return dispatch_global(p, mask, s, (char*)workspace + flag_bytes, (hipStream_t)stream);
+  GlobalMask mask{n, local_size, global_inds, n_globals, bits};
+  return dispatch_global(p, mask, s, base + lay.off_engine, (hipStream_t)stream);
 }
 
 }  // extern "C"

@@ -28,15 +28,33 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 
+// What a tile problem looks like.  Band: queries and keys are the positions of one subsequence.
+// GlobalRows: queries are the (distinct) global rows, keys are all tokens outside the query's
+// window; the key range is split over workgroups and each writes a partial (m, l, acc).
+// GlobalCols: queries are all non-global tokens, keys are the listed global tokens outside the
+// query's window (Sparse_FlashAttention_Global_No_Local/sp_flatt_global_no_local_kernel.cu:38-64).
+enum { kTileBand = 0, kTileGlobalRows = 1, kTileGlobalCols = 2 };
+
 struct BandArgs {
   Tensors t;
   int64_t n;              // tokens
-  int64_t w;              // window half-width in subsequence positions
+  int64_t w;              // window half-width (band: subsequence positions; global: tokens)
   int64_t s;              // token stride of a subsequence
   int64_t block;          // 0: band mode, else block size
   int64_t cnt;            // block mode: live positions per block
   int64_t tiles_per_sub;  // query tiles per subsequence (of the longest subsequence)
   int64_t n_tiles;
+  // global modes
+  const int32_t* globs;   // listed global tokens (keys of GlobalCols)
+  int64_t n_globs;
+  const uint32_t* gbits;  // bit i set <=> token i is a global row
+  const int32_t* uq;      // distinct global rows (queries of GlobalRows)
+  const uint32_t* n_uq;   // how many
+  int64_t key_run;        // GlobalRows: keys per split (multiple of 64)
+  int64_t n_split;
+  float* pm;              // GlobalRows partials, slot = query * n_split + split
+  float* pl;
+  float* pacc;
 };
 
 template <typename T, int D>
@@ -79,39 +97,75 @@ __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
   return __builtin_bit_cast(uint32_t, x);
 }
 
-template <typename T, int D>
+template <typename T, int D, int MODE>
 __global__ __launch_bounds__(256, 2) void band_kernel(BandArgs a) {
   using C = BandCfg<T, D>;
   constexpr bool kF32 = C::kF32;
   constexpr int BM = C::BM, BN = C::BN, EB = C::EB;
   __shared__ __attribute__((aligned(16))) T lds[C::K_ELEMS + C::V_ELEMS];
+  __shared__ int ktok_s[BN];  // GlobalCols: token of every key of the tile
   T* Ks = lds;
   T* Vs = lds + C::K_ELEMS;
 
-  // workgroups are dealt round-robin to the 8 XCDs: give each XCD a contiguous run of tiles so
-  // that neighbouring query tiles (which share most of their keys) meet in one L2
-  const int64_t per_xcd = (a.n_tiles + 7) / 8;
-  const int64_t lt = (int64_t)(blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
-  if (lt >= a.n_tiles) return;
-  const int64_t sub = lt / a.tiles_per_sub;
-  const int64_t tile = lt - sub * a.tiles_per_sub;
-  int64_t base, len;
-  if (a.block > 0) {
-    base = sub * a.block;
-    len = a.cnt;
+  // base/len: token of position 0 and number of positions (band); qlen/klen: query and key
+  // position counts; [u_lo, u_hi): key positions this workgroup walks
+  int64_t base = 0, qlen, klen, t0, u_lo, u_hi, split = 0;
+  if constexpr (MODE == kTileBand) {
+    // workgroups are dealt round-robin to the 8 XCDs: give each XCD a contiguous run of tiles
+    // so that neighbouring query tiles (which share most of their keys) meet in one L2
+    const int64_t per_xcd = (a.n_tiles + 7) / 8;
+    const int64_t lt = (int64_t)(blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+    if (lt >= a.n_tiles) return;
+    const int64_t sub = lt / a.tiles_per_sub;
+    const int64_t tile = lt - sub * a.tiles_per_sub;
+    if (a.block > 0) {
+      base = sub * a.block;
+      qlen = a.cnt;
+    } else {
+      base = sub;
+      qlen = (a.n - sub + a.s - 1) / a.s;
+    }
+    klen = qlen;
+    t0 = tile * BM;
+    if (t0 >= qlen) return;
+    u_lo = t0 - a.w;
+    if (u_lo < 0) u_lo = 0;
+    u_hi = t0 + BM + a.w;
+    if (u_hi > klen || u_hi < 0) u_hi = klen;
+  } else if constexpr (MODE == kTileGlobalRows) {
+    const int64_t qt = blockIdx.x / a.n_split;
+    split = blockIdx.x - qt * a.n_split;
+    qlen = (int64_t)*a.n_uq;
+    klen = a.n;
+    t0 = qt * BM;
+    if (t0 >= qlen) return;
+    u_lo = split * a.key_run;
+    u_hi = u_lo + a.key_run;
+    if (u_hi > klen) u_hi = klen;
   } else {
-    base = sub;
-    len = (a.n - sub + a.s - 1) / a.s;
+    qlen = a.n;
+    klen = a.n_globs;
+    t0 = (int64_t)blockIdx.x * BM;
+    if (t0 >= qlen) return;
+    u_lo = 0;
+    u_hi = klen;
   }
-  const int64_t t0 = tile * BM;
-  if (t0 >= len) return;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
   const int r = lane & 31, h = lane >> 5;
   const int64_t tw0 = t0 + 32 * wave;  // first query of this wavefront
-  const int64_t tq = tw0 + r;          // this lane's query
-  const bool q_ok = tq < len;
+  const int64_t tq = tw0 + r;          // this lane's query position
+  bool q_ok = tq < qlen;
+  int64_t q_tok;                       // its token (row of Q / out)
+  if constexpr (MODE == kTileBand) {
+    q_tok = base + (q_ok ? tq : qlen - 1) * a.s;
+  } else if constexpr (MODE == kTileGlobalRows) {
+    q_tok = a.uq[q_ok ? tq : qlen - 1];
+  } else {
+    q_tok = q_ok ? tq : qlen - 1;
+    if (q_ok && bit_is_set(a.gbits, q_tok)) q_ok = false;  // global rows belong to GlobalRows
+  }
   const T* Qp = (const T*)a.t.q;
   const T* Kp = (const T*)a.t.k;
   const T* Vp = (const T*)a.t.v;
@@ -120,7 +174,7 @@ __global__ __launch_bounds__(256, 2) void band_kernel(BandArgs a) {
   uint4v qh[kF32 ? 1 : C::QREGS];
   float qf[kF32 ? C::QREGS : 1];
   {
-    const T* qrow = Qp + (base + (q_ok ? tq : len - 1) * a.s) * D;
+    const T* qrow = Qp + q_tok * D;
     if constexpr (kF32) {
 #pragma unroll
       for (int c4 = 0; c4 < D / 4; c4++) {
@@ -144,14 +198,18 @@ __global__ __launch_bounds__(256, 2) void band_kernel(BandArgs a) {
   float l = 0.f;      // running sum over this lane's half of the keys
   const float sc = 1.4426950408889634f / sqrtf((float)D);
 
-  int64_t u_lo = t0 - a.w;
-  if (u_lo < 0) u_lo = 0;
-  int64_t u_hi = t0 + BM + a.w;
-  if (u_hi > len || u_hi < 0) u_hi = len;
 
   for (int64_t ut = u_lo; ut < u_hi; ut += BN) {
     __syncthreads();  // the previous tile has been consumed
-    // ---- stage K and V rows ut .. ut+63 (zeros past the end of the subsequence)
+    // ---- stage K and V rows of key positions ut .. ut+63 (zeros from u_hi on)
+    auto key_tok = [&](int64_t u) -> int64_t {
+      if constexpr (MODE == kTileBand) return base + u * a.s;
+      else if constexpr (MODE == kTileGlobalRows) return u;
+      else return (int64_t)a.globs[u];
+    };
+    if constexpr (MODE == kTileGlobalCols) {
+      if (tid < BN) ktok_s[tid] = (ut + tid < u_hi) ? a.globs[ut + tid] : 0;
+    }
     if constexpr (kF32) {
       constexpr int CH = D / 4;  // 16-byte chunks per row
 #pragma unroll
@@ -160,8 +218,8 @@ __global__ __launch_bounds__(256, 2) void band_kernel(BandArgs a) {
         const int j = idx / CH, c = idx % CH;
         const int64_t u = ut + j;
         float4v kx = {0.f, 0.f, 0.f, 0.f}, vx = {0.f, 0.f, 0.f, 0.f};
-        if (u < len) {
-          const int64_t off = (base + u * a.s) * D + 4 * c;
+        if (u < u_hi) {
+          const int64_t off = key_tok(u) * D + 4 * c;
           kx = *reinterpret_cast<const float4v*>(Kp + off);
           vx = *reinterpret_cast<const float4v*>(Vp + off);
         }
@@ -177,7 +235,7 @@ __global__ __launch_bounds__(256, 2) void band_kernel(BandArgs a) {
         const int j = idx / CH, c = idx % CH;
         const int64_t u = ut + j;
         uint4v kx = {0u, 0u, 0u, 0u};
-        if (u < len) kx = *reinterpret_cast<const uint4v*>(Kp + (base + u * a.s) * D + 8 * c);
+        if (u < u_hi) kx = *reinterpret_cast<const uint4v*>(Kp + key_tok(u) * D + 8 * c);
         *reinterpret_cast<uint4v*>(Ks + j * C::K_STRIDE + 8 * c) = kx;
       }
       // V: a lane takes the key pair (2*jp, 2*jp+1) and 8 columns e, and writes the 8 packed
@@ -188,8 +246,8 @@ __global__ __launch_bounds__(256, 2) void band_kernel(BandArgs a) {
         const int c = (lane >> 5) + 2 * (wave + 4 * it);
         const int64_t u = ut + 2 * jp;
         uint4v v0 = {0u, 0u, 0u, 0u}, v1 = {0u, 0u, 0u, 0u};
-        if (u < len) v0 = *reinterpret_cast<const uint4v*>(Vp + (base + u * a.s) * D + 8 * c);
-        if (u + 1 < len) v1 = *reinterpret_cast<const uint4v*>(Vp + (base + (u + 1) * a.s) * D + 8 * c);
+        if (u < u_hi) v0 = *reinterpret_cast<const uint4v*>(Vp + key_tok(u) * D + 8 * c);
+        if (u + 1 < u_hi) v1 = *reinterpret_cast<const uint4v*>(Vp + key_tok(u + 1) * D + 8 * c);
         const int slot = key_slot(2 * jp);
         uint32_t* col = reinterpret_cast<uint32_t*>(Vs + (8 * c) * C::V_STRIDE + slot);
 #pragma unroll
@@ -208,7 +266,10 @@ __global__ __launch_bounds__(256, 2) void band_kernel(BandArgs a) {
 #pragma unroll
     for (int jb = 0; jb < 2; jb++) {
       const int64_t ub = ut + 32 * jb;
-      need[jb] = (tw0 < len) && (ub < len) && (ub <= tw0 + 31 + a.w) && (ub + 31 + a.w >= tw0);
+      if constexpr (MODE == kTileBand)
+        need[jb] = (tw0 < qlen) && (ub < u_hi) && (ub <= tw0 + 31 + a.w) && (ub + 31 + a.w >= tw0);
+      else
+        need[jb] = (tw0 < qlen) && (ub < u_hi);
     }
     if (!need[0] && !need[1]) continue;
 
@@ -240,7 +301,15 @@ __global__ __launch_bounds__(256, 2) void band_kernel(BandArgs a) {
 #pragma unroll
       for (int v = 0; v < 16; v++) {
         const int64_t u = ut + 32 * jb + 8 * (v / 4) + 4 * h + (v % 4);
-        const bool ok = need[jb] && q_ok && (u < len) && (u + a.w >= tq) && (u <= tq + a.w);
+        bool ok = need[jb] && q_ok && (u < u_hi);
+        if constexpr (MODE == kTileBand) {
+          ok = ok && (u + a.w >= tq) && (u <= tq + a.w);
+        } else {
+          int64_t kt;
+          if constexpr (MODE == kTileGlobalRows) kt = u;
+          else kt = ktok_s[32 * jb + 8 * (v / 4) + 4 * h + (v % 4)];
+          ok = ok && ((kt + a.w < q_tok) || (kt > q_tok + a.w));
+        }
         const float x = ok ? sreg[jb][v] * sc : kNegInf;
         sreg[jb][v] = x;
         mx = fmaxf(mx, x);
@@ -301,8 +370,30 @@ __global__ __launch_bounds__(256, 2) void band_kernel(BandArgs a) {
 
   // ---- finish: combine the two key halves, fold the incoming state in, write back
   l += shfl_xor_f32(l, 32);
+  if constexpr (MODE == kTileGlobalRows) {
+    // partial result of this key split; an empty one is (m, l, acc) = (-inf, 0, 0)
+    if (!q_ok) return;
+    const int64_t slot = tq * a.n_split + split;
+    const bool any = l > 0.f;
+    float* prow = a.pacc + slot * D;
+#pragma unroll
+    for (int eb = 0; eb < EB; eb++)
+#pragma unroll
+      for (int g4 = 0; g4 < 4; g4++) {
+        float4v y = {0.f, 0.f, 0.f, 0.f};
+        if (any) {
+          y[0] = o[eb][4 * g4]; y[1] = o[eb][4 * g4 + 1]; y[2] = o[eb][4 * g4 + 2]; y[3] = o[eb][4 * g4 + 3];
+        }
+        *reinterpret_cast<float4v*>(prow + 32 * eb + 8 * g4 + 4 * h) = y;
+      }
+    if (h == 0) {
+      a.pm[slot] = any ? m * 0.6931471805599453f : kNegInf;
+      a.pl[slot] = any ? l : 0.f;
+    }
+    return;
+  }
   if (!q_ok || !(l > 0.f)) return;
-  const int64_t row = base + tq * a.s;
+  const int64_t row = q_tok;
   const bool sf = a.t.state_f32 != 0;
   const float m_nat = m * 0.6931471805599453f;
   float m_out = m_nat, l_out = l;
@@ -363,6 +454,57 @@ __global__ void band_dead_rows_kernel(T* out, int64_t n, int d, int64_t block, i
   if (((row % block) % s) != 0) out[idx] = from_f32<T>(__builtin_nanf(""));
 }
 
+// One wavefront per distinct global row: fold the key-split partials (two passes: overall max,
+// then weighted sums), fold the incoming state in, write the row.
+template <typename T, int D>
+__global__ __launch_bounds__(64) void global_rows_merge_kernel(BandArgs a) {
+  const int64_t g = blockIdx.x;
+  if (g >= (int64_t)*a.n_uq) return;
+  const int lane = threadIdx.x;
+  const int64_t s0 = g * a.n_split;
+  float mx = kNegInf;
+  for (int64_t k = lane; k < a.n_split; k += kWave) mx = fmaxf(mx, a.pm[s0 + k]);
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) mx = fmaxf(mx, shfl_xor_f32(mx, off));
+  if (mx == kNegInf) return;  // no live column at all: row untouched
+  float lsum = 0.f;
+  for (int64_t k = lane; k < a.n_split; k += kWave) lsum += a.pl[s0 + k] * __expf(a.pm[s0 + k] - mx);
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) lsum += shfl_xor_f32(lsum, off);
+  constexpr int EPL = D / kWave;
+  float acc[EPL];
+#pragma unroll
+  for (int e = 0; e < EPL; e++) acc[e] = 0.f;
+  for (int64_t k = 0; k < a.n_split; k++) {
+    const float wk = __expf(a.pm[s0 + k] - mx);
+#pragma unroll
+    for (int e = 0; e < EPL; e++) acc[e] += wk * a.pacc[(s0 + k) * D + lane + kWave * e];
+  }
+  const int64_t row = a.uq[g];
+  const bool sf = a.t.state_f32 != 0;
+  float m_out = mx, l_out = lsum, wa = 0.f, wb = 1.f;
+  const float l_in = load_state<T>(a.t.l, row, sf);
+  if (l_in != 0.f) {
+    const float m_in = load_state<T>(a.t.m, row, sf);
+    m_out = fmaxf(mx, m_in);
+    wa = l_in * __expf(m_in - m_out);
+    wb = __expf(mx - m_out);
+    l_out = wa + lsum * wb;
+  }
+  const float inv = 1.f / l_out;
+  T* orow = (T*)a.t.out + row * D;
+#pragma unroll
+  for (int e = 0; e < EPL; e++) {
+    float x = acc[e] * wb;
+    if (wa != 0.f) x += wa * to_f32(orow[lane + kWave * e]);
+    orow[lane + kWave * e] = from_f32<T>(x * inv);
+  }
+  if (lane == 0) {
+    store_state<T>(a.t.m, row, m_out, sf);
+    store_state<T>(a.t.l, row, l_out, sf);
+  }
+}
+
 template <typename T, int D>
 int launch_band(const BandArgs& a, int use_nan, hipStream_t stream) {
   const KernelEvents ev = kernel_events();
@@ -370,7 +512,7 @@ int launch_band(const BandArgs& a, int use_nan, hipStream_t stream) {
   if (a.n_tiles > 0) {
     const int64_t grid = (a.n_tiles + 7) / 8 * 8;
     if (timed) (void)hipEventRecord(ev.start, stream);
-    hipLaunchKernelGGL((band_kernel<T, D>), dim3((unsigned)grid), dim3(256), 0, stream, a);
+    hipLaunchKernelGGL((band_kernel<T, D, kTileBand>), dim3((unsigned)grid), dim3(256), 0, stream, a);
     if (timed) (void)hipEventRecord(ev.stop, stream);
   }
   if (a.block > 0 && use_nan && a.s > 1) {
@@ -381,14 +523,48 @@ int launch_band(const BandArgs& a, int use_nan, hipStream_t stream) {
   return hipGetLastError() == hipSuccess ? 0 : 4;
 }
 
+// Global minus local: non-global rows against the listed globals, then the global rows against
+// everything (key range split over workgroups), then the fold of the splits.
+template <typename T, int D>
+int launch_global_tiles(const BandArgs& a, hipStream_t stream) {
+  const KernelEvents ev = kernel_events();
+  const bool timed = ev.start != nullptr && ev.stop != nullptr;
+  const int64_t grid_cols = (a.n + 127) / 128;
+  hipLaunchKernelGGL((band_kernel<T, D, kTileGlobalCols>), dim3((unsigned)grid_cols), dim3(256), 0,
+                     stream, a);
+  const int64_t q_tiles = (a.n_globs + 127) / 128;
+  if (timed) (void)hipEventRecord(ev.start, stream);
+  hipLaunchKernelGGL((band_kernel<T, D, kTileGlobalRows>), dim3((unsigned)(q_tiles * a.n_split)),
+                     dim3(256), 0, stream, a);
+  if (timed) (void)hipEventRecord(ev.stop, stream);
+  hipLaunchKernelGGL((global_rows_merge_kernel<T, D>), dim3((unsigned)a.n_globs), dim3(64), 0, stream,
+                     a);
+  return hipGetLastError() == hipSuccess ? 0 : 4;
+}
+
+inline bool tile_shape_ok(const Tensors& t, size_t elem_bytes) {
+  if (!aligned16(t.q) || !aligned16(t.k) || !aligned16(t.v) || !aligned16(t.out)) return false;
+  // (the fp32 tiles for d = 128 would need more than 64 KB of LDS)
+  return t.d == 64 || (t.d == 128 && elem_bytes == 2);
+}
+
 // Returns -1 when the shape is not covered (caller falls back to the row-gather engine).
 template <typename T>
 int run_band_tiles(const BandArgs& a, int use_nan, hipStream_t stream) {
-  if (!aligned16(a.t.q) || !aligned16(a.t.k) || !aligned16(a.t.v) || !aligned16(a.t.out)) return -1;
+  if (!tile_shape_ok(a.t, sizeof(T))) return -1;
   if (a.t.d == 64) return launch_band<T, 64>(a, use_nan, stream);
   if constexpr (sizeof(T) == 2) {
-    // (the fp32 tiles for d = 128 would need more than 64 KB of LDS)
     if (a.t.d == 128) return launch_band<T, 128>(a, use_nan, stream);
+  }
+  return -1;
+}
+
+template <typename T>
+int run_global_tiles(const BandArgs& a, hipStream_t stream) {
+  if (!tile_shape_ok(a.t, sizeof(T))) return -1;
+  if (a.t.d == 64) return launch_global_tiles<T, 64>(a, stream);
+  if constexpr (sizeof(T) == 2) {
+    if (a.t.d == 128) return launch_global_tiles<T, 128>(a, stream);
   }
   return -1;
 }

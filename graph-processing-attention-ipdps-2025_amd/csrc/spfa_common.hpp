@@ -198,6 +198,10 @@ struct GenLay {
   }
 };
 
+__device__ __forceinline__ bool bit_is_set(const uint32_t* bits, int64_t i) {
+  return (bits[i >> 5] >> (i & 31)) & 1u;
+}
+
 __device__ __forceinline__ int lane_id() {
   return (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
 }

@@ -16,6 +16,9 @@ int run_stride(const Tensors& t, const StrideMask& mask, const EngineSizing& s, 
 // Dense-tile (MFMA) path for band / block masks; -1 when the shape is not covered.
 template <typename T>
 int run_band(const BandArgs& a, int use_nan, hipStream_t stream);
+// Dense-tile path for the global-minus-local mask; -1 when the shape is not covered.
+template <typename T>
+int run_global_dense(const BandArgs& a, hipStream_t stream);
 template <typename T>
 int run_global(const Tensors& t, const GlobalMask& mask, const EngineSizing& s, int use_nan,
                void* ws, hipStream_t stream);

@@ -73,13 +73,13 @@ struct StrideMask {
 //   global row: candidates are all n - (up-low) columns outside the window;
 //   other rows: candidates are the n_globs listed indices, those inside the window are masked
 //   (Sparse_FlashAttention_Global_No_Local/sp_flatt_global_no_local_kernel.cu:38-64,134-162).
-// is_global[i] != 0 marks the listed rows.
+// Bit i of gbits marks the listed rows.
 struct GlobalMask {
   int64_t n;
   int64_t w;
   const int32_t* globs;
   int64_t n_globs;
-  const uint8_t* is_global;
+  const uint32_t* gbits;
   struct Row {
     int64_t low;
     int64_t up;
@@ -91,7 +91,7 @@ struct GlobalMask {
     if (low < 0) low = 0;
     int64_t up = i + w + 1;
     if (up > n) up = n;
-    bool glob = is_global[i] != 0;
+    bool glob = bit_is_set(gbits, i);
     return Row{low, up, glob ? n - (up - low) : n_globs, glob};
   }
   __device__ __forceinline__ int64_t col(const Row& r, int64_t t, bool& valid) const {

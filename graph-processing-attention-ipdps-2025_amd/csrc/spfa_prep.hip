@@ -134,12 +134,16 @@ __global__ __launch_bounds__(kScanThreads) void scan_apply_kernel(const uint32_t
   }
 }
 
-__global__ void mark_globals_kernel(const int32_t* globs, int64_t n_globs, int64_t n,
-                                    uint8_t* flags) {
+__global__ void mark_globals_kernel(const int32_t* globs, int64_t n_globs, int64_t n, uint32_t* bits,
+                                    uint32_t* count, int32_t* uq) {
   int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i < n_globs) {
     int64_t g = globs[i];
-    if (g >= 0 && g < n) flags[g] = 1;
+    if (g >= 0 && g < n) {
+      const uint32_t bit = 1u << (g & 31);
+      const uint32_t old = atomicOr(&bits[g >> 5], bit);
+      if (!(old & bit)) uq[atomicAdd(count, 1u)] = (int32_t)g;  // first time this row is listed
+    }
   }
 }
 
@@ -197,13 +201,13 @@ int coo_bucket_by_row(const void* row_ind, int row_wide, const uint32_t* col_ind
   return hipGetLastError() == hipSuccess ? 0 : 4;
 }
 
-int mark_global_rows(const int32_t* globs, int64_t n_globs, int64_t n, uint8_t* flags,
-                     hipStream_t stream) {
-  const int64_t words = (n + 3) / 4;
-  hipLaunchKernelGGL(fill_u32_kernel, dim3(grid_for(words, 256, 4096)), dim3(256), 0, stream,
-                     (uint32_t*)flags, words, 0u);
+int prepare_global_rows(const int32_t* globs, int64_t n_globs, int64_t n, uint32_t* bits,
+                        int32_t* uq, hipStream_t stream) {
+  const int64_t words = (int64_t)global_bits_words(n);
+  hipLaunchKernelGGL(fill_u32_kernel, dim3(grid_for(words, 256, 4096)), dim3(256), 0, stream, bits,
+                     words, 0u);
   hipLaunchKernelGGL(mark_globals_kernel, dim3(grid_for(n_globs, 256, 1 << 30)), dim3(256), 0,
-                     stream, globs, n_globs, n, flags);
+                     stream, globs, n_globs, n, bits, bits + (words - 1), uq);
   return hipGetLastError() == hipSuccess ? 0 : 4;
 }
 

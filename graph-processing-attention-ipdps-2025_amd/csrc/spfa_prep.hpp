@@ -22,8 +22,11 @@ int coo_bucket_by_row(const void* row_ind, int row_wide, const uint32_t* col_ind
                       int64_t n_rows, void* ws, hipStream_t stream, const uint32_t** row_off_out,
                       const uint32_t** cols_out);
 
-// flags[i] = 1 for every listed i in [0, n), 0 elsewhere.  flags holds (n+3)/4*4 bytes.
-int mark_global_rows(const int32_t* globs, int64_t n_globs, int64_t n, uint8_t* flags,
-                     hipStream_t stream);
+// Global-row bookkeeping for the global-minus-local mask.  `bits` holds (n+31)/32 bitmap words
+// followed by one counter word; afterwards bit i is set for every listed i in [0, n), `uq` holds
+// the distinct listed rows (any order) and the counter word their number.
+inline size_t global_bits_words(int64_t n) { return (size_t)((n + 31) / 32) + 1; }
+int prepare_global_rows(const int32_t* globs, int64_t n_globs, int64_t n, uint32_t* bits,
+                        int32_t* uq, hipStream_t stream);
 
 }  // namespace spfa
