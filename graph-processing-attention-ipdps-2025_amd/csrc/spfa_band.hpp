@@ -199,55 +199,74 @@ __global__ __launch_bounds__(256, 2) void band_kernel(BandArgs a) {
   const float sc = 1.4426950408889634f / sqrtf((float)D);
 
 
-  for (int64_t ut = u_lo; ut < u_hi; ut += BN) {
-    __syncthreads();  // the previous tile has been consumed
-    // ---- stage K and V rows of key positions ut .. ut+63 (zeros from u_hi on)
-    auto key_tok = [&](int64_t u) -> int64_t {
-      if constexpr (MODE == kTileBand) return base + u * a.s;
-      else if constexpr (MODE == kTileGlobalRows) return u;
-      else return (int64_t)a.globs[u];
-    };
-    if constexpr (MODE == kTileGlobalCols) {
-      if (tid < BN) ktok_s[tid] = (ut + tid < u_hi) ? a.globs[ut + tid] : 0;
+  // Tiles are fetched one ahead: the global loads of tile n+1 are issued before tile n is
+  // consumed and land in registers; they are written to LDS once tile n has been consumed.
+  auto key_tok = [&](int64_t u) -> int64_t {
+    if constexpr (MODE == kTileBand) return base + u * a.s;
+    else if constexpr (MODE == kTileGlobalRows) return u;
+    else return (int64_t)a.globs[u];
+  };
+  constexpr int CH = kF32 ? D / 4 : D / 8;       // 16-byte chunks per row
+  constexpr int KIT = BN * CH / 256;             // chunks of K per thread and tile
+  constexpr int VIT = kF32 ? KIT : (BN / 2) * CH / 256;
+  uint4v kreg[KIT], vreg[kF32 ? KIT : 2 * VIT];
+  int ktok_reg = 0;
+
+  auto fetch = [&](int64_t ut) {
+#pragma unroll
+    for (int it = 0; it < KIT; it++) {
+      const int idx = it * 256 + tid;
+      const int j = idx / CH, c = idx % CH;
+      const int64_t u = ut + j;
+      uint4v kx = {0u, 0u, 0u, 0u}, vx = {0u, 0u, 0u, 0u};
+      if (u < u_hi) {
+        const int64_t off = key_tok(u) * D + (16 / (int)sizeof(T)) * c;
+        kx = *reinterpret_cast<const uint4v*>(Kp + off);
+        if constexpr (kF32) vx = *reinterpret_cast<const uint4v*>(Vp + off);
+      }
+      kreg[it] = kx;
+      if constexpr (kF32) vreg[it] = vx;
     }
-    if constexpr (kF32) {
-      constexpr int CH = D / 4;  // 16-byte chunks per row
+    if constexpr (!kF32) {
+      // V: a lane takes the key pair (2*jp, 2*jp+1) and 8 columns e
 #pragma unroll
-      for (int it = 0; it < BN * CH / 256; it++) {
-        const int idx = it * 256 + tid;
-        const int j = idx / CH, c = idx % CH;
-        const int64_t u = ut + j;
-        float4v kx = {0.f, 0.f, 0.f, 0.f}, vx = {0.f, 0.f, 0.f, 0.f};
-        if (u < u_hi) {
-          const int64_t off = key_tok(u) * D + 4 * c;
-          kx = *reinterpret_cast<const float4v*>(Kp + off);
-          vx = *reinterpret_cast<const float4v*>(Vp + off);
-        }
-        float* kd = (float*)Ks + j * C::K_STRIDE + 4 * c;  // 8-byte aligned rows
-        kd[0] = kx[0]; kd[1] = kx[1]; kd[2] = kx[2]; kd[3] = kx[3];
-        *reinterpret_cast<float4v*>((float*)Vs + j * C::V_STRIDE + 4 * c) = vx;
-      }
-    } else {
-      constexpr int CH = D / 8;
-#pragma unroll
-      for (int it = 0; it < BN * CH / 256; it++) {
-        const int idx = it * 256 + tid;
-        const int j = idx / CH, c = idx % CH;
-        const int64_t u = ut + j;
-        uint4v kx = {0u, 0u, 0u, 0u};
-        if (u < u_hi) kx = *reinterpret_cast<const uint4v*>(Kp + key_tok(u) * D + 8 * c);
-        *reinterpret_cast<uint4v*>(Ks + j * C::K_STRIDE + 8 * c) = kx;
-      }
-      // V: a lane takes the key pair (2*jp, 2*jp+1) and 8 columns e, and writes the 8 packed
-      // pairs down a column of the transposed tile
-#pragma unroll
-      for (int it = 0; it < (BN / 2) * CH / 256; it++) {
+      for (int it = 0; it < VIT; it++) {
         const int jp = lane & 31;
         const int c = (lane >> 5) + 2 * (wave + 4 * it);
         const int64_t u = ut + 2 * jp;
         uint4v v0 = {0u, 0u, 0u, 0u}, v1 = {0u, 0u, 0u, 0u};
         if (u < u_hi) v0 = *reinterpret_cast<const uint4v*>(Vp + key_tok(u) * D + 8 * c);
         if (u + 1 < u_hi) v1 = *reinterpret_cast<const uint4v*>(Vp + key_tok(u + 1) * D + 8 * c);
+        vreg[2 * it] = v0;
+        vreg[2 * it + 1] = v1;
+      }
+    }
+    if constexpr (MODE == kTileGlobalCols) {
+      if (tid < BN) ktok_reg = (ut + tid < u_hi) ? a.globs[ut + tid] : 0;
+    }
+  };
+
+  auto stash = [&]() {
+#pragma unroll
+    for (int it = 0; it < KIT; it++) {
+      const int idx = it * 256 + tid;
+      const int j = idx / CH, c = idx % CH;
+      if constexpr (kF32) {
+        float4v kx = __builtin_bit_cast(float4v, kreg[it]);
+        float* kd = (float*)Ks + j * C::K_STRIDE + 4 * c;  // rows are only 8-byte aligned
+        kd[0] = kx[0]; kd[1] = kx[1]; kd[2] = kx[2]; kd[3] = kx[3];
+        *reinterpret_cast<uint4v*>((float*)Vs + j * C::V_STRIDE + 4 * c) = vreg[it];
+      } else {
+        *reinterpret_cast<uint4v*>(Ks + j * C::K_STRIDE + 8 * c) = kreg[it];
+      }
+    }
+    if constexpr (!kF32) {
+      // the 8 packed key pairs go down a column of the transposed tile
+#pragma unroll
+      for (int it = 0; it < VIT; it++) {
+        const int jp = lane & 31;
+        const int c = (lane >> 5) + 2 * (wave + 4 * it);
+        const uint4v v0 = vreg[2 * it], v1 = vreg[2 * it + 1];
         const int slot = key_slot(2 * jp);
         uint32_t* col = reinterpret_cast<uint32_t*>(Vs + (8 * c) * C::V_STRIDE + slot);
 #pragma unroll
@@ -258,7 +277,17 @@ __global__ __launch_bounds__(256, 2) void band_kernel(BandArgs a) {
         }
       }
     }
+    if constexpr (MODE == kTileGlobalCols) {
+      if (tid < BN) ktok_s[tid] = ktok_reg;
+    }
+  };
+
+  if (u_lo < u_hi) fetch(u_lo);
+  for (int64_t ut = u_lo; ut < u_hi; ut += BN) {
+    __syncthreads();  // the previous tile has been consumed
+    stash();
     __syncthreads();
+    if (ut + BN < u_hi) fetch(ut + BN);
 
     // ---- this wavefront's share of the tile: up to two 32-key blocks
     // block jb holds keys ut + 32*jb .. +31; it matters iff it overlaps the wavefront's band
@@ -454,32 +483,57 @@ __global__ void band_dead_rows_kernel(T* out, int64_t n, int d, int64_t block, i
   if (((row % block) % s) != 0) out[idx] = from_f32<T>(__builtin_nanf(""));
 }
 
-// One wavefront per distinct global row: fold the key-split partials (two passes: overall max,
-// then weighted sums), fold the incoming state in, write the row.
+// One workgroup per distinct global row: fold the key-split partials (two passes: overall max,
+// then weighted sums with the splits spread over the threads), fold the incoming state in,
+// write the row.
 template <typename T, int D>
-__global__ __launch_bounds__(64) void global_rows_merge_kernel(BandArgs a) {
+__global__ __launch_bounds__(256) void global_rows_merge_kernel(BandArgs a) {
+  constexpr int NSUB = 256 / D;  // threads per output element
+  __shared__ float red[4];
+  __shared__ float part[256];
   const int64_t g = blockIdx.x;
   if (g >= (int64_t)*a.n_uq) return;
-  const int lane = threadIdx.x;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int64_t s0 = g * a.n_split;
+
   float mx = kNegInf;
-  for (int64_t k = lane; k < a.n_split; k += kWave) mx = fmaxf(mx, a.pm[s0 + k]);
+  for (int64_t k = tid; k < a.n_split; k += 256) mx = fmaxf(mx, a.pm[s0 + k]);
 #pragma unroll
   for (int off = 32; off >= 1; off >>= 1) mx = fmaxf(mx, shfl_xor_f32(mx, off));
-  if (mx == kNegInf) return;  // no live column at all: row untouched
+  if (lane == 0) red[wave] = mx;
+  __syncthreads();
+  mx = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+  __syncthreads();
+  if (mx == kNegInf) return;  // no live column at all: row untouched (same answer in every thread)
+
   float lsum = 0.f;
-  for (int64_t k = lane; k < a.n_split; k += kWave) lsum += a.pl[s0 + k] * __expf(a.pm[s0 + k] - mx);
+  for (int64_t k = tid; k < a.n_split; k += 256) lsum += a.pl[s0 + k] * __expf(a.pm[s0 + k] - mx);
 #pragma unroll
   for (int off = 32; off >= 1; off >>= 1) lsum += shfl_xor_f32(lsum, off);
-  constexpr int EPL = D / kWave;
-  float acc[EPL];
+  if (lane == 0) red[wave] = lsum;
+  __syncthreads();
+  lsum = (red[0] + red[1]) + (red[2] + red[3]);
+
+  const int e = tid % D, sub = tid / D;
+  float acc = 0.f;
+  int64_t k = sub;
+  for (; k + 3 * NSUB < a.n_split; k += 4 * NSUB) {
+    float x[4], wgt[4];
 #pragma unroll
-  for (int e = 0; e < EPL; e++) acc[e] = 0.f;
-  for (int64_t k = 0; k < a.n_split; k++) {
-    const float wk = __expf(a.pm[s0 + k] - mx);
+    for (int u = 0; u < 4; u++) {
+      x[u] = a.pacc[(s0 + k + u * NSUB) * D + e];
+      wgt[u] = a.pm[s0 + k + u * NSUB];
+    }
 #pragma unroll
-    for (int e = 0; e < EPL; e++) acc[e] += wk * a.pacc[(s0 + k) * D + lane + kWave * e];
+    for (int u = 0; u < 4; u++) acc += __expf(wgt[u] - mx) * x[u];
   }
+  for (; k < a.n_split; k += NSUB) acc += __expf(a.pm[s0 + k] - mx) * a.pacc[(s0 + k) * D + e];
+  part[tid] = acc;
+  __syncthreads();
+  if (sub != 0) return;
+#pragma unroll
+  for (int u = 1; u < NSUB; u++) acc += part[u * D + e];
+
   const int64_t row = a.uq[g];
   const bool sf = a.t.state_f32 != 0;
   float m_out = mx, l_out = lsum, wa = 0.f, wb = 1.f;
@@ -493,13 +547,10 @@ __global__ __launch_bounds__(64) void global_rows_merge_kernel(BandArgs a) {
   }
   const float inv = 1.f / l_out;
   T* orow = (T*)a.t.out + row * D;
-#pragma unroll
-  for (int e = 0; e < EPL; e++) {
-    float x = acc[e] * wb;
-    if (wa != 0.f) x += wa * to_f32(orow[lane + kWave * e]);
-    orow[lane + kWave * e] = from_f32<T>(x * inv);
-  }
-  if (lane == 0) {
+  float x = acc * wb;
+  if (wa != 0.f) x += wa * to_f32(orow[e]);
+  orow[e] = from_f32<T>(x * inv);
+  if (e == 0) {
     store_state<T>(a.t.m, row, m_out, sf);
     store_state<T>(a.t.l, row, l_out, sf);
   }
@@ -537,7 +588,7 @@ int launch_global_tiles(const BandArgs& a, hipStream_t stream) {
   hipLaunchKernelGGL((band_kernel<T, D, kTileGlobalRows>), dim3((unsigned)(q_tiles * a.n_split)),
                      dim3(256), 0, stream, a);
   if (timed) (void)hipEventRecord(ev.stop, stream);
-  hipLaunchKernelGGL((global_rows_merge_kernel<T, D>), dim3((unsigned)a.n_globs), dim3(64), 0, stream,
+  hipLaunchKernelGGL((global_rows_merge_kernel<T, D>), dim3((unsigned)a.n_globs), dim3(256), 0, stream,
                      a);
   return hipGetLastError() == hipSuccess ? 0 : 4;
 }
