@@ -297,6 +297,9 @@ def main():
     ap.add_argument("--workload", default="csr_zipf", choices=sorted(WORKLOADS))
     ap.add_argument("--dtype", default="f32", choices=["f32", "f16", "bf16"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="after the timed region, run one plain 256 MiB device copy (a kernel of known "
+                         "traffic that counter runs use to scale FETCH_SIZE / WRITE_SIZE)")
     a = ap.parse_args()
     if a.gpus != 1:
         sys.exit("bench.py measures one GPU: this path is a single-GPU kernel and every box here has "
@@ -352,6 +355,14 @@ def main():
     lib.spfa_set_kernel_events(None, None)
     torch.cuda.synchronize()
     k_avg = sum(kernel_ms) / len(kernel_ms)
+
+    if a.copy_calibration:
+        src = torch.empty(64 * 1024 * 1024, dtype=torch.float32, device="cuda").normal_()
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        dst.copy_(src)  # reads 256 MiB, writes 256 MiB
+        torch.cuda.synchronize()
+        del src, dst
 
     err, checked = verify_sample(w, states[0], torch)
     tol = 1e-4 if dtype == torch.float32 else 2e-2

@@ -163,6 +163,8 @@ int dispatch_band(const spfa_problem_t* p, int64_t w, int64_t stride, int64_t bl
 
 // rows shorter than this are cheaper on the row-gather engine than on 32x32 tiles
 constexpr int64_t kBandTileMinRow = 32;
+// the tile kernels test windows in 32-bit arithmetic: (unsigned)(delta + w) <= 2w
+constexpr int64_t kTileMaxWindow = (int64_t)1 << 30;
 
 int dispatch_global(const spfa_problem_t* p, const GlobalMask& mask, const EngineSizing& s,
                     void* ws, hipStream_t stream) {
@@ -347,7 +349,7 @@ int spfa_local_1d_dilated_forward(const spfa_problem_t* p, int64_t local_size, i
   {
     const int64_t len_max = (n + dil_factor) / (dil_factor + 1);
     const int64_t span = 2 * local_size + 1 < len_max ? 2 * local_size + 1 : len_max;
-    if (span >= kBandTileMinRow && dtype_ok(p->dtype)) {
+    if (span >= kBandTileMinRow && dtype_ok(p->dtype) && local_size <= kTileMaxWindow) {
       rc = dispatch_band(p, local_size, dil_factor + 1, 0, 0, 0, (hipStream_t)stream);
       if (rc >= 0) return rc;
     }
@@ -434,7 +436,8 @@ int spfa_global_no_local_forward(const spfa_problem_t* p, const int32_t* global_
   a.pl = (float*)(base + lay.off_pl);
   a.pacc = (float*)(base + lay.off_pacc);
   const int64_t q_tiles = (n_globals + 127) / 128;
-  if (q_tiles * lay.n_split < ((int64_t)1 << 31) && n_globals < ((int64_t)1 << 31)) {
+  if (q_tiles * lay.n_split < ((int64_t)1 << 31) && n_globals < ((int64_t)1 << 31) &&
+      local_size <= kTileMaxWindow) {
     rc = -1;
     switch (p->dtype) {
       case SPFA_DTYPE_F32: rc = run_global_dense<float>(a, (hipStream_t)stream); break;

@@ -272,8 +272,8 @@ __global__ __launch_bounds__(256, 2) void band_kernel(BandArgs a) {
 #pragma unroll
         for (int x = 0; x < 4; x++) {
           // dword x of v0/v1 holds columns 2x, 2x+1
-          col[(2 * x) * (C::V_STRIDE / 2)] = (v0[x] & 0xffffu) | (v1[x] << 16);
-          col[(2 * x + 1) * (C::V_STRIDE / 2)] = (v0[x] >> 16) | (v1[x] & 0xffff0000u);
+          col[(2 * x) * (C::V_STRIDE / 2)] = __builtin_amdgcn_perm(v1[x], v0[x], 0x05040100u);
+          col[(2 * x + 1) * (C::V_STRIDE / 2)] = __builtin_amdgcn_perm(v1[x], v0[x], 0x07060302u);
         }
       }
     }
@@ -323,38 +323,55 @@ __global__ __launch_bounds__(256, 2) void band_kernel(BandArgs a) {
       }
     }
 
-    // ---- scale, mask, running max
+    // ---- mask, running max, exponentials.  Scores stay un-scaled in the registers; the
+    // 1/sqrt(d) * log2(e) factor is folded into the exponent's fma (it is positive, so the max
+    // can be taken first).  Masks are 32-bit: a key is live iff (unsigned)(delta + w) <= 2w
+    // (band; delta = key position - query position) or > 2w (global; delta in tokens).
+    const uint32_t w32 = (uint32_t)a.w, w2 = 2u * (uint32_t)a.w;
+    const int rem = (int)((u_hi - ut) < BN ? (u_hi - ut) : BN);  // live key slots of this tile
+    uint32_t d0;
+    if constexpr (MODE == kTileBand) d0 = (uint32_t)(int32_t)(ut - tq) + w32;
+    else if constexpr (MODE == kTileGlobalRows) d0 = (uint32_t)(int32_t)(ut - q_tok) + w32;
+    else d0 = w32 - (uint32_t)(int32_t)q_tok;
     float mx = kNegInf;
 #pragma unroll
     for (int jb = 0; jb < 2; jb++) {
+      if (!need[jb]) {
 #pragma unroll
-      for (int v = 0; v < 16; v++) {
-        const int64_t u = ut + 32 * jb + 8 * (v / 4) + 4 * h + (v % 4);
-        bool ok = need[jb] && q_ok && (u < u_hi);
-        if constexpr (MODE == kTileBand) {
-          ok = ok && (u + a.w >= tq) && (u <= tq + a.w);
-        } else {
-          int64_t kt;
-          if constexpr (MODE == kTileGlobalRows) kt = u;
-          else kt = ktok_s[32 * jb + 8 * (v / 4) + 4 * h + (v % 4)];
-          ok = ok && ((kt + a.w < q_tok) || (kt > q_tok + a.w));
-        }
-        const float x = ok ? sreg[jb][v] * sc : kNegInf;
-        sreg[jb][v] = x;
-        mx = fmaxf(mx, x);
+        for (int v = 0; v < 16; v++) sreg[jb][v] = kNegInf;
+        continue;
       }
+      bool full = false;  // every (query, key) pair of the block is live: no per-element test
+      if constexpr (MODE == kTileBand) {
+        const int64_t ub = ut + 32 * jb;
+        full = (ub + 31 < u_hi) && (ub + a.w >= tw0 + 31) && (ub + 31 <= tw0 + a.w);
+      }
+      if (!full) {
+#pragma unroll
+        for (int v = 0; v < 16; v++) {
+          const int j = 32 * jb + 8 * (v / 4) + 4 * h + (v % 4);
+          bool ok;
+          if constexpr (MODE == kTileBand) ok = (d0 + (uint32_t)j <= w2);
+          else if constexpr (MODE == kTileGlobalRows) ok = (d0 + (uint32_t)j > w2);
+          else ok = (d0 + (uint32_t)ktok_s[j] > w2);
+          if (!(ok && j < rem)) sreg[jb][v] = kNegInf;
+        }
+      }
+#pragma unroll
+      for (int v = 0; v < 16; v++) mx = fmaxf(mx, sreg[jb][v]);
     }
-    mx = fmaxf(mx, shfl_xor_f32(mx, 32));
+    mx = fmaxf(mx, shfl_xor_f32(mx, 32)) * sc;
     const float m_new = fmaxf(m, mx);
     const bool live = m_new > kNegInf;
-    const float alpha = live ? exp2f(m - m_new) : 1.f;
-    const float m_use = live ? m_new : 0.f;
+    const float alpha = live ? __builtin_amdgcn_exp2f(m - m_new) : 1.f;
+    const float neg_m = live ? -m_new : 0.f;
     float lsum = 0.f;
 #pragma unroll
     for (int jb = 0; jb < 2; jb++)
 #pragma unroll
       for (int v = 0; v < 16; v++) {
-        const float p = exp2f(sreg[jb][v] - m_use);  // exp2(-inf) = 0 for masked entries
+        // exp2(-inf) = 0 for masked entries
+        const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(sreg[jb][v], sc, neg_m));
         sreg[jb][v] = p;
         lsum += p;
       }
