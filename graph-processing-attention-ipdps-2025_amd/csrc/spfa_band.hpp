@@ -6,7 +6,7 @@
 //   Local 1D dilated      s subsequences, one per residue class mod s
 //   Local 2D dilated      one subsequence per block (base b*B, cnt live tokens, w = everything)
 // so all three are the same tile problem.  One workgroup (4 wavefronts) owns 128 consecutive
-// query positions, one wavefront 32 of them; keys are streamed in tiles of 64 through LDS and
+// query positions, one wavefront 32 of them; keys are streamed in tiles of 64 (32 for fp32 at d = 128) through LDS and
 // shared by the four wavefronts.
 //
 // Everything is computed transposed, S^T = K Q^T and O^T = V^T P^T, with 32x32 MFMA tiles.  In
@@ -61,7 +61,9 @@ template <typename T, int D>
 struct BandCfg {
   static constexpr bool kF32 = sizeof(T) == 4;
   static constexpr int BM = 128;  // queries per workgroup
-  static constexpr int BN = 64;   // keys per LDS tile
+  // keys per LDS tile (fp32 at d = 128 takes half tiles to stay inside 64 KB of LDS)
+  static constexpr int BN = (kF32 && D > 64) ? 32 : 64;
+  static constexpr int NB = BN / 32;  // 32-key blocks per tile
   // K tile: [key][k] rows padded so that the 32 keys read by one operand fetch spread over the
   // banks.  V tile: half types are stored transposed [e][key'] (16-byte operand reads), fp32
   // row-major [key][e].
@@ -101,7 +103,7 @@ template <typename T, int D, int MODE>
 __global__ __launch_bounds__(256, 2) void band_kernel(BandArgs a) {
   using C = BandCfg<T, D>;
   constexpr bool kF32 = C::kF32;
-  constexpr int BM = C::BM, BN = C::BN, EB = C::EB;
+  constexpr int BM = C::BM, BN = C::BN, EB = C::EB, NB = C::NB;
   __shared__ __attribute__((aligned(16))) T lds[C::K_ELEMS + C::V_ELEMS];
   __shared__ int ktok_s[BN];  // GlobalCols: token of every key of the tile
   T* Ks = lds;
@@ -291,20 +293,22 @@ __global__ __launch_bounds__(256, 2) void band_kernel(BandArgs a) {
 
     // ---- this wavefront's share of the tile: up to two 32-key blocks
     // block jb holds keys ut + 32*jb .. +31; it matters iff it overlaps the wavefront's band
-    bool need[2];
+    bool need[NB];
+    bool any_need = false;
 #pragma unroll
-    for (int jb = 0; jb < 2; jb++) {
+    for (int jb = 0; jb < NB; jb++) {
       const int64_t ub = ut + 32 * jb;
       if constexpr (MODE == kTileBand)
         need[jb] = (tw0 < qlen) && (ub < u_hi) && (ub <= tw0 + 31 + a.w) && (ub + 31 + a.w >= tw0);
       else
         need[jb] = (tw0 < qlen) && (ub < u_hi);
+      any_need = any_need || need[jb];
     }
-    if (!need[0] && !need[1]) continue;
+    if (!any_need) continue;
 
-    f32x16 sreg[2];
+    f32x16 sreg[NB];
 #pragma unroll
-    for (int jb = 0; jb < 2; jb++) {
+    for (int jb = 0; jb < NB; jb++) {
 #pragma unroll
       for (int v = 0; v < 16; v++) sreg[jb][v] = 0.f;
       if (!need[jb]) continue;
@@ -335,7 +339,7 @@ __global__ __launch_bounds__(256, 2) void band_kernel(BandArgs a) {
     else d0 = w32 - (uint32_t)(int32_t)q_tok;
     float mx = kNegInf;
 #pragma unroll
-    for (int jb = 0; jb < 2; jb++) {
+    for (int jb = 0; jb < NB; jb++) {
       if (!need[jb]) {
 #pragma unroll
         for (int v = 0; v < 16; v++) sreg[jb][v] = kNegInf;
@@ -367,7 +371,7 @@ __global__ __launch_bounds__(256, 2) void band_kernel(BandArgs a) {
     const float neg_m = live ? -m_new : 0.f;
     float lsum = 0.f;
 #pragma unroll
-    for (int jb = 0; jb < 2; jb++)
+    for (int jb = 0; jb < NB; jb++)
 #pragma unroll
       for (int v = 0; v < 16; v++) {
         // exp2(-inf) = 0 for masked entries
@@ -386,7 +390,7 @@ __global__ __launch_bounds__(256, 2) void band_kernel(BandArgs a) {
 
     // ---- O^T += V^T P^T
 #pragma unroll
-    for (int jb = 0; jb < 2; jb++) {
+    for (int jb = 0; jb < NB; jb++) {
       if (!need[jb]) continue;
       if constexpr (kF32) {
 #pragma unroll
@@ -612,8 +616,8 @@ int launch_global_tiles(const BandArgs& a, hipStream_t stream) {
 
 inline bool tile_shape_ok(const Tensors& t, size_t elem_bytes) {
   if (!aligned16(t.q) || !aligned16(t.k) || !aligned16(t.v) || !aligned16(t.out)) return false;
-  // (the fp32 tiles for d = 128 would need more than 64 KB of LDS)
-  return t.d == 64 || (t.d == 128 && elem_bytes == 2);
+  (void)elem_bytes;
+  return t.d == 64 || t.d == 128;
 }
 
 // Returns -1 when the shape is not covered (caller falls back to the row-gather engine).
@@ -621,9 +625,7 @@ template <typename T>
 int run_band_tiles(const BandArgs& a, int use_nan, hipStream_t stream) {
   if (!tile_shape_ok(a.t, sizeof(T))) return -1;
   if (a.t.d == 64) return launch_band<T, 64>(a, use_nan, stream);
-  if constexpr (sizeof(T) == 2) {
-    if (a.t.d == 128) return launch_band<T, 128>(a, use_nan, stream);
-  }
+  if (a.t.d == 128) return launch_band<T, 128>(a, use_nan, stream);
   return -1;
 }
 
@@ -631,9 +633,7 @@ template <typename T>
 int run_global_tiles(const BandArgs& a, hipStream_t stream) {
   if (!tile_shape_ok(a.t, sizeof(T))) return -1;
   if (a.t.d == 64) return launch_global_tiles<T, 64>(a, stream);
-  if constexpr (sizeof(T) == 2) {
-    if (a.t.d == 128) return launch_global_tiles<T, 128>(a, stream);
-  }
+  if (a.t.d == 128) return launch_global_tiles<T, 128>(a, stream);
   return -1;
 }
 

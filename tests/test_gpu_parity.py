@@ -368,8 +368,8 @@ def test_coo_empty_mask(mods):
 
 # ------------------------------------------------------------------ implicit masks
 @pytest.mark.parametrize("dtype,d", [(torch.float32, 64), (torch.bfloat16, 64), (torch.float16, 32),
-                                     (torch.bfloat16, 128), (torch.float32, 48)])
-@pytest.mark.parametrize("n,w", [(1000, 0), (1000, 1), (1000, 128), (777, 776), (4096, 300)])
+                                     (torch.bfloat16, 128), (torch.float32, 48), (torch.float32, 128)])
+@pytest.mark.parametrize("n,w", [(1000, 0), (1000, 1), (1000, 128), (777, 776), (4096, 300), (130, 20)])
 def test_local(mods, dtype, d, n, w):
     q, k, v = dev_qkv(n, d, dtype, 30)
     m, l, o = state(n, d, dtype, torch.float32)
@@ -379,9 +379,10 @@ def test_local(mods, dtype, d, n, w):
     check(o, m, l, *ref, dtype, state_dtype=torch.float32)
 
 
-@pytest.mark.parametrize("dtype,d", [(torch.float32, 64), (torch.bfloat16, 128), (torch.float16, 64)])
+@pytest.mark.parametrize("dtype,d", [(torch.float32, 64), (torch.bfloat16, 128), (torch.float16, 64),
+                                     (torch.float32, 128)])
 @pytest.mark.parametrize("n,w,dil", [(1000, 10, 2), (1000, 0, 3), (1000, 999, 0), (1001, 100, 1),
-                                     (2048, 256, 2), (300, 299, 6)])
+                                     (2048, 256, 2), (300, 299, 6), (5000, 40, 4)])
 def test_local_1d_dilated(mods, dtype, d, n, w, dil):
     q, k, v = dev_qkv(n, d, dtype, 31, scale=0.5)
     m, l, o = state(n, d, dtype, torch.float32)
@@ -391,9 +392,10 @@ def test_local_1d_dilated(mods, dtype, d, n, w, dil):
     check(o, m, l, *ref, dtype, state_dtype=torch.float32)
 
 
-@pytest.mark.parametrize("dtype,d", [(torch.float32, 64), (torch.bfloat16, 128), (torch.float16, 64)])
+@pytest.mark.parametrize("dtype,d", [(torch.float32, 64), (torch.bfloat16, 128), (torch.float16, 64),
+                                     (torch.float32, 128)])
 @pytest.mark.parametrize("n,block,dil", [(1024, 16, 0), (1024, 16, 1), (1024, 256, 2), (1000, 1000, 3),
-                                         (1024, 1, 0), (960, 32, 31), (2048, 2048, 0)])
+                                         (1024, 1, 0), (960, 32, 31), (2048, 2048, 0), (1200, 300, 1)])
 @pytest.mark.parametrize("use_nan", [True, False])
 def test_local_2d_dilated(mods, dtype, d, n, block, dil, use_nan):
     q, k, v = dev_qkv(n, d, dtype, 32, scale=0.5)
@@ -404,9 +406,10 @@ def test_local_2d_dilated(mods, dtype, d, n, block, dil, use_nan):
     check(o, m, l, *ref, dtype, state_dtype=torch.float32, dead_expect="nan" if use_nan else None)
 
 
-@pytest.mark.parametrize("dtype,d", [(torch.float32, 64), (torch.bfloat16, 64), (torch.float16, 128)])
+@pytest.mark.parametrize("dtype,d", [(torch.float32, 64), (torch.bfloat16, 64), (torch.float16, 128),
+                                     (torch.float32, 128), (torch.float32, 32)])
 @pytest.mark.parametrize("n,n_globs,w", [(1024, 4, 10), (1024, 1, 0), (1024, 64, 64), (1500, 100, 1499),
-                                         (1024, 1024, 3), (8192, 16, 100)])
+                                         (1024, 1024, 3), (8192, 16, 100), (3000, 200, 7)])
 def test_global_no_local(mods, dtype, d, n, n_globs, w):
     q, k, v = dev_qkv(n, d, dtype, 33)
     g = syn.global_indices(n, n_globs, seed=33)
