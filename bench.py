@@ -289,6 +289,22 @@ def cpu_sparse_port(w, torch, rows=8192):
             "sample": "%d random rows, row-wise sparse float64 C restatement with OpenMP, %.2f s" % (len(idx), t)}
 
 
+def measured_traffic(workload, dtype_name):
+    """HBM-side bytes per launch of the dominant kernel from the committed counter summary of this
+    workload (profiles/<workload>..._pmc.md, line `traffic_bytes_per_launch = N`), else None."""
+    import glob
+    import re
+    names = {"csr_zipf": "csr_zipf_n131072_d64"}
+    stem = names.get(workload)
+    if stem is None:
+        return None
+    for path in glob.glob(os.path.join(ROOT, "profiles", "%s_%s_pmc.md" % (stem, {"f32": "f32"}.get(dtype_name, dtype_name)))):
+        m = re.search(r"^traffic_bytes_per_launch\s*=\s*(\d+)", open(path).read(), re.M)
+        if m:
+            return int(m.group(1))
+    return None
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -381,7 +397,7 @@ def main():
         "effective_gathered_GBs": w["bytes_gathered"] / (ms_per_step * 1e-3) / 1e9,
         "algorithmic_GBs": w["bytes_total"] / (ms_per_step * 1e-3) / 1e9,
         "roofline": {"bound": "hbm", "achieved": achieved_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved_gbs / HBM_PEAK_GBS, "traffic": None,
+                     "frac": achieved_gbs / HBM_PEAK_GBS, "traffic": measured_traffic(a.workload, a.dtype),
                      "kernel": "segments_kernel" if a.workload in ("csr_zipf", "csr_bernoulli", "coo_zipf", "global") else "rows_kernel",
                      "kernel_ms_avg": k_avg, "kernel_ms_min": min(kernel_ms),
                      "algorithmic_bytes": w["kernel_bytes"], "kernel_nnz": w["kernel_nnz"],
