@@ -61,7 +61,7 @@ class HipEvents:
 
 
 def load_library():
-    lib_path = os.path.join(PKG, "libspfa_hip.so")
+    lib_path = os.path.join(os.environ.get("SPFA_LIB_DIR", PKG), "libspfa_hip.so")
     if not os.path.exists(lib_path):
         raise RuntimeError("libspfa_hip.so is not built: run `python -c 'import __graft_entry__ as g; g.build()'`")
     lib = ctypes.CDLL(lib_path)

@@ -86,13 +86,25 @@ struct VecLay {
   static constexpr int GROUPS = kWave / LPR;
   static constexpr int NE = 16 / (int)sizeof(T);  // floats held per lane
   static constexpr int D = LPR * NE;
-  static constexpr int U = 8;        // neighbours in flight per group in the segment kernel
+#ifndef SPFA_TUNE_U
+#define SPFA_TUNE_U 8
+#endif
+  static constexpr int U = SPFA_TUNE_U;  // neighbours in flight per group in the segment kernel
   static constexpr int U_SHORT = 4;  // ... in the row kernel
   static constexpr bool kFixedD = true;
   using raw = uint4v;
 
   __device__ static __forceinline__ raw load(const T* row_ptr, int c, int) {
     return *reinterpret_cast<const raw*>(reinterpret_cast<const char*>(row_ptr) + c * 16);
+  }
+  // gathered K / V rows
+  __device__ static __forceinline__ raw load_gather(const T* row_ptr, int c, int) {
+#if defined(SPFA_TUNE_NT)
+    return __builtin_nontemporal_load(
+        reinterpret_cast<const raw*>(reinterpret_cast<const char*>(row_ptr) + c * 16));
+#else
+    return *reinterpret_cast<const raw*>(reinterpret_cast<const char*>(row_ptr) + c * 16);
+#endif
   }
   __device__ static __forceinline__ void unpack(const raw& r, float (&f)[NE]) {
     if constexpr (sizeof(T) == 4) {
@@ -170,6 +182,9 @@ struct GenLay {
       r.x[e] = idx < d ? row_ptr[idx] : from_f32<T>(0.f);
     }
     return r;
+  }
+  __device__ static __forceinline__ raw load_gather(const T* row_ptr, int c, int d) {
+    return load(row_ptr, c, d);
   }
   __device__ static __forceinline__ void unpack(const raw& r, float (&f)[NE]) {
 #pragma unroll

@@ -96,66 +96,92 @@ __device__ __forceinline__ void merge_partial(float& m, float& l, float (&acc)[N
   m = m_new;
 }
 
-// Candidates t_begin, t_begin + t_stride, ... < t_end of one row, U at a time.  All K and V
-// rows of a batch are requested before any of them is consumed.
-template <class Lay, class Mask, int U>
+// Candidates t_begin .. t_end of one row, walked by SPAN consecutive lanes (the whole wavefront
+// in segments_kernel, one lane group in rows_kernel).
+//
+// Column indices are fetched SPAN at a time, one per lane (a coalesced load for CSR), one chunk
+// ahead of their use, and handed to the groups with cross-lane reads - a column index is never
+// waited for inside the gather sequence.  A batch is U candidates per group: all 2*U row loads
+// of a batch are issued back to back before any is consumed.
+template <class Lay, class Mask, int U_, int SPAN>
 __device__ __forceinline__ void attend(const Mask& mask, const typename Mask::Row& rc,
                                        const typename Lay::elem* __restrict__ K,
                                        const typename Lay::elem* __restrict__ V, int d, float scale,
                                        const float (&q)[Lay::NE], int64_t t_begin, int64_t t_end,
-                                       int64_t t_stride, int c, float& m, float& l,
-                                       float (&acc)[Lay::NE]) {
+                                       int lane, float& m, float& l, float (&acc)[Lay::NE]) {
   constexpr int NE = Lay::NE;
-  for (int64_t t0 = t_begin; t0 < t_end; t0 += (int64_t)U * t_stride) {
-    typename Lay::raw kr[U], vr[U];
-    bool ok[U];
+  constexpr int LPR = Lay::LPR;
+  constexpr int GS = SPAN / LPR;                  // groups sharing the row
+  constexpr int U = (U_ * GS > SPAN) ? SPAN / GS : U_;
+  constexpr int PER = U * GS;                     // candidates per batch
+  constexpr int PARTS = SPAN / PER;               // batches per index chunk
+  static_assert(SPAN % LPR == 0 && PARTS >= 1 && PARTS * PER == SPAN, "bad span / unroll");
+  const int ls = lane % SPAN;   // slot of this lane in an index chunk
+  const int lb = lane - ls;     // first lane of the span
+  const int gi = ls / LPR;      // group within the span
+  const int c = lane % LPR;
+
+  // column of candidate t + ls, or -1 (past the end / masked)
+  auto fetch = [&](int64_t t) -> int {
+    const int64_t tt = t + ls;
+    bool valid = tt < t_end;
+    int64_t col = 0;
+    if (valid) col = mask.col(rc, tt, valid);
+    return valid ? (int)col : -1;
+  };
+
+  int next = fetch(t_begin);
+  for (int64_t tb = t_begin; tb < t_end; tb += SPAN) {
+    const int cur = next;
+    if (tb + SPAN < t_end) next = fetch(tb + SPAN);
+#pragma unroll(PARTS <= 2 ? PARTS : 1)
+    for (int part = 0; part < PARTS; part++) {
+      if (tb + part * PER >= t_end) break;
+      int cols[U];
 #pragma unroll
-    for (int u = 0; u < U; u++) {
-      int64_t t = t0 + u * t_stride;
-      ok[u] = t < t_end;
-      if (ok[u]) {
-        bool valid = true;
-        int64_t col = mask.col(rc, t, valid);
-        ok[u] = valid;
-        if (valid) {
-          kr[u] = Lay::load(K + col * d, c, d);
-          vr[u] = Lay::load(V + col * d, c, d);
-        }
-      }
-    }
-    float s[U];
-    float mb = kNegInf;
-#pragma unroll
-    for (int u = 0; u < U; u++) {
-      float part = 0.f;
-      if (ok[u]) {
-        float kf[NE];
-        Lay::unpack(kr[u], kf);
-#pragma unroll
-        for (int e = 0; e < NE; e++) part += q[e] * kf[e];
-      }
-      float tot = group_sum<Lay::LPR>(part) * scale;
-      s[u] = ok[u] ? tot : kNegInf;
-      mb = fmaxf(mb, s[u]);
-    }
-    if (mb > kNegInf) {
-      float m_new = fmaxf(m, mb);
-      float corr = __expf(m - m_new);
-      l *= corr;
-#pragma unroll
-      for (int e = 0; e < NE; e++) acc[e] *= corr;
+      for (int u = 0; u < U; u++) cols[u] = shfl_i32(cur, lb + part * PER + u * GS + gi);
+      typename Lay::raw kr[U], vr[U];
 #pragma unroll
       for (int u = 0; u < U; u++) {
-        if (ok[u]) {
-          float p = __expf(s[u] - m_new);
-          l += p;
-          float vf[NE];
-          Lay::unpack(vr[u], vf);
-#pragma unroll
-          for (int e = 0; e < NE; e++) acc[e] += p * vf[e];
+        if (cols[u] >= 0) {
+          kr[u] = Lay::load_gather(K + (int64_t)cols[u] * d, c, d);
+          vr[u] = Lay::load_gather(V + (int64_t)cols[u] * d, c, d);
         }
       }
-      m = m_new;
+      float s[U];
+      float mb = kNegInf;
+#pragma unroll
+      for (int u = 0; u < U; u++) {
+        float part_dot = 0.f;
+        if (cols[u] >= 0) {
+          float kf[NE];
+          Lay::unpack(kr[u], kf);
+#pragma unroll
+          for (int e = 0; e < NE; e++) part_dot += q[e] * kf[e];
+        }
+        float tot = group_sum<LPR>(part_dot) * scale;
+        s[u] = cols[u] >= 0 ? tot : kNegInf;
+        mb = fmaxf(mb, s[u]);
+      }
+      if (mb > kNegInf) {
+        float m_new = fmaxf(m, mb);
+        float corr = __expf(m - m_new);
+        l *= corr;
+#pragma unroll
+        for (int e = 0; e < NE; e++) acc[e] *= corr;
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+          if (cols[u] >= 0) {
+            float p = __expf(s[u] - m_new);
+            l += p;
+            float vf[NE];
+            Lay::unpack(vr[u], vf);
+#pragma unroll
+            for (int e = 0; e < NE; e++) acc[e] += p * vf[e];
+          }
+        }
+        m = m_new;
+      }
     }
   }
 }
@@ -214,47 +240,67 @@ __device__ __forceinline__ uint32_t wave_inclusive_sum(uint32_t x, int lane) {
 }
 
 // One thread per query row: rows longer than short_max are cut into segments of plan.seg
-// candidates.  Each wavefront reserves room for all its rows with one atomic per counter (the
-// counters are shared by the whole grid, so per-row atomics would serialise on them).
+// candidates.  A workgroup of 1024 rows reserves room for all its rows with one atomic per
+// counter (the counters are shared by the whole grid: per-row, even per-wavefront, atomics
+// serialise on them and dominate the kernel).
+constexpr int kPlanThreads = 1024;
+
 template <class Mask>
-__global__ __launch_bounds__(256) void plan_kernel(int64_t n_q, Mask mask, Plan plan) {
+__global__ __launch_bounds__(kPlanThreads) void plan_kernel(int64_t n_q, Mask mask, Plan plan) {
+  constexpr int NW = kPlanThreads / kWave;
+  __shared__ uint32_t wave_tot[NW][3];
+  __shared__ uint32_t block_base[3];
+  __shared__ uint32_t block_ok;
   const int lane = lane_id();
-  const int64_t row = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int wave = threadIdx.x / kWave;
+  const int64_t row = (int64_t)blockIdx.x * kPlanThreads + threadIdx.x;
   int64_t deg = 0;
   if (row < n_q) deg = mask.row(row).deg;
   const bool is_long = deg > plan.short_max;
-  if (__builtin_amdgcn_ballot_w64(is_long) == 0) return;  // same answer in every lane
   const uint32_t nseg = is_long ? (uint32_t)((deg + plan.seg - 1) / plan.seg) : 0u;
   const uint32_t multi = nseg > 1 ? 1u : 0u;
   const uint32_t npart = multi ? nseg : 0u;
   const uint32_t inc_items = wave_inclusive_sum(nseg, lane);
   const uint32_t inc_part = wave_inclusive_sum(npart, lane);
   const uint32_t inc_multi = wave_inclusive_sum(multi, lane);
-  uint32_t base_items = 0, base_part = 0, base_multi = 0, ok = 1;
   if (lane == kWave - 1) {
-    base_items = atomicAdd(&plan.cnt->n_items, inc_items);
-    if (inc_part) base_part = atomicAdd(&plan.cnt->n_partials, inc_part);
-    if (inc_multi) base_multi = atomicAdd(&plan.cnt->n_multi, inc_multi);
-    if (base_items + inc_items > plan.cap_items || base_part + inc_part > plan.cap_partials ||
-        base_multi + inc_multi > plan.cap_multi) {
-      ok = 0;
-      atomicOr(&plan.cnt->overflow, 1u);
-    }
+    wave_tot[wave][0] = inc_items;
+    wave_tot[wave][1] = inc_part;
+    wave_tot[wave][2] = inc_multi;
   }
-  base_items = (uint32_t)__builtin_amdgcn_readlane((int)base_items, kWave - 1);
-  base_part = (uint32_t)__builtin_amdgcn_readlane((int)base_part, kWave - 1);
-  base_multi = (uint32_t)__builtin_amdgcn_readlane((int)base_multi, kWave - 1);
-  ok = (uint32_t)__builtin_amdgcn_readlane((int)ok, kWave - 1);
-  if (!ok || !is_long) return;
-  const uint32_t my_item = base_items + inc_items - nseg;
-  const uint32_t my_slot = base_part + inc_part - npart;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    uint32_t tot[3] = {0u, 0u, 0u};
+    for (int w = 0; w < NW; w++)
+      for (int k = 0; k < 3; k++) {
+        const uint32_t x = wave_tot[w][k];
+        wave_tot[w][k] = tot[k];  // exclusive prefix over the wavefronts
+        tot[k] += x;
+      }
+    uint32_t ok = 1;
+    if (tot[0]) {
+      block_base[0] = atomicAdd(&plan.cnt->n_items, tot[0]);
+      block_base[1] = tot[1] ? atomicAdd(&plan.cnt->n_partials, tot[1]) : 0u;
+      block_base[2] = tot[2] ? atomicAdd(&plan.cnt->n_multi, tot[2]) : 0u;
+      if (block_base[0] + tot[0] > plan.cap_items || block_base[1] + tot[1] > plan.cap_partials ||
+          block_base[2] + tot[2] > plan.cap_multi) {
+        ok = 0;
+        atomicOr(&plan.cnt->overflow, 1u);
+      }
+    }
+    block_ok = ok;
+  }
+  __syncthreads();
+  if (!block_ok || !is_long) return;
+  const uint32_t my_item = block_base[0] + wave_tot[wave][0] + inc_items - nseg;
+  const uint32_t my_slot = block_base[1] + wave_tot[wave][1] + inc_part - npart;
   if (multi) {
     MultiRow mr;
     mr.row = (int32_t)row;
     mr.slot0 = (int32_t)my_slot;
     mr.nseg = (int32_t)nseg;
     mr.pad = 0;
-    plan.multi[base_multi + inc_multi - 1] = mr;
+    plan.multi[block_base[2] + wave_tot[wave][2] + inc_multi - 1] = mr;
   }
   for (uint32_t j = 0; j < nseg; j++) {
     Item it;
@@ -297,8 +343,8 @@ __global__ __launch_bounds__(256) void rows_kernel(Tensors t, Mask mask, Plan pl
 #pragma unroll
     for (int e = 0; e < NE; e++) acc[e] = 0.f;
     const float scale = 1.0f / sqrtf((float)t.d);
-    attend<Lay, Mask, Lay::U_SHORT>(mask, rc, (const T*)t.k, (const T*)t.v, t.d, scale, q, 0, deg, 1,
-                                    c, m, l, acc);
+    attend<Lay, Mask, Lay::U_SHORT, LPR>(mask, rc, (const T*)t.k, (const T*)t.v, t.d, scale, q, 0, deg,
+                                         lane, m, l, acc);
     finish_row<Lay>(t, row, c, m, l, acc);
   }
   // longer rows were cut into segments by plan_kernel and belong to segments_kernel
@@ -334,8 +380,8 @@ __global__ __launch_bounds__(256) void segments_kernel(Tensors t, Mask mask, Pla
     float m = kNegInf, l = 0.f, acc[NE];
 #pragma unroll
     for (int e = 0; e < NE; e++) acc[e] = 0.f;
-    attend<Lay, Mask, Lay::U>(mask, rc, (const T*)t.k, (const T*)t.v, t.d, scale, q, t0 + g, t1,
-                              Lay::GROUPS, c, m, l, acc);
+    attend<Lay, Mask, Lay::U, kWave>(mask, rc, (const T*)t.k, (const T*)t.v, t.d, scale, q, t0, t1, lane,
+                                     m, l, acc);
 
     // butterfly over the groups of the wavefront
 #pragma unroll
@@ -484,8 +530,8 @@ int launch_engine(const Tensors& t, const Mask& mask, const EngineSizing& s, int
   const bool has_long = s.max_deg > s.short_max;
   if (has_long) {
     hipLaunchKernelGGL(reset_counters_kernel, dim3(1), dim3(64), 0, stream, plan.cnt);
-    hipLaunchKernelGGL((plan_kernel<Mask>), dim3((unsigned)((t.n_q + 255) / 256)), dim3(256), 0,
-                       stream, t.n_q, mask, plan);
+    hipLaunchKernelGGL((plan_kernel<Mask>), dim3((unsigned)((t.n_q + kPlanThreads - 1) / kPlanThreads)),
+                       dim3(kPlanThreads), 0, stream, t.n_q, mask, plan);
   }
 
   const KernelEvents ev = kernel_events();
