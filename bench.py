@@ -34,6 +34,7 @@ WORKLOADS = {
     "csr_zipf": "CSR N=131072 d=64 Zipf(1.5) degrees clipped [1,4096], uniform sorted columns + diagonal",
     "csr_bernoulli": "CSR N=4096 d=64 Bernoulli(2%) + diagonal",
     "coo_zipf": "COO N=1048576 d=64 ~50M unsorted entries, row weights Zipf(1.3), uniform columns",
+    "coo_zipf_sorted": "COO N=1048576 d=64 ~50M entries sorted by row, row weights Zipf(1.3), uniform columns",
     "local": "Local N=65536 d=64 LOCAL_SIZE=128 (|i-j|<=128)",
     "local_1d": "Local-1D-dilated N=262144 d=128 LOCAL_SIZE=256 DILATE_FACTOR=2 (stride 3)",
     "local_2d": "Local-2D-dilated N=262144 d=128 BLOCK_SIZE=256 DILATE_FACTOR=2 (stride 3)",
@@ -76,7 +77,7 @@ def make_workload(name, dtype, torch, syn, inline_limit=32):
     dev = "cuda"
     es = torch.tensor([], dtype=dtype).element_size()
     w = {"name": name, "desc": WORKLOADS[name]}
-    if name in ("csr_zipf", "csr_bernoulli", "coo_zipf"):
+    if name in ("csr_zipf", "csr_bernoulli", "coo_zipf", "coo_zipf_sorted"):
         if name == "csr_zipf":
             n, d = 131072, 64
             ro, ci = syn.zipf_csr(n, 1.5, 1, 4096, device=dev, seed=0)
@@ -86,8 +87,11 @@ def make_workload(name, dtype, torch, syn, inline_limit=32):
         else:
             n, d = 1 << 20, 64
             r, c = syn.zipf_coo(n, 50_000_000, 1.3, device=dev, seed=0)
+            if name == "coo_zipf_sorted":
+                order = torch.argsort(r, stable=True)
+                r, c = r[order].contiguous(), c[order].contiguous()
         q, k, v = syn.qkv(n, d, dtype=dtype, device=dev, seed=0)
-        if name == "coo_zipf":
+        if name.startswith("coo"):
             import spfa_coo
             nnz = int(c.numel())
             r_t, c_t = r.to(torch.uint64), c.to(torch.uint32)
@@ -105,7 +109,7 @@ def make_workload(name, dtype, torch, syn, inline_limit=32):
             w["csr"] = (ro, ci)
             off_b = 8
         gathered, total = syn.explicit_mask_bytes(nnz, n, d, es, off_bytes=off_b)
-        if name == "coo_zipf":
+        if name.startswith("coo"):
             total += nnz * 8  # row index of every entry
             deg = torch.bincount(r, minlength=n)
         else:
@@ -175,7 +179,7 @@ def verify_sample(w, state, torch, rows=192):
         ro, ci = w["csr"]
         ro_c = ro.cpu().numpy()
         lists = [ci[ro_c[i]:ro_c[i + 1]].cpu().numpy() for i in idx_np]
-    elif name == "coo_zipf":
+    elif name.startswith("coo"):
         r, c = w["coo"]
         lists = [c[r == int(i)].cpu().numpy() for i in idx_np[:32]]
         idx_np, qs = idx_np[:32], qs[:32]
@@ -398,7 +402,7 @@ def main():
         "algorithmic_GBs": w["bytes_total"] / (ms_per_step * 1e-3) / 1e9,
         "roofline": {"bound": "hbm", "achieved": achieved_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved_gbs / HBM_PEAK_GBS, "traffic": measured_traffic(a.workload, a.dtype),
-                     "kernel": "segments_kernel" if a.workload in ("csr_zipf", "csr_bernoulli", "coo_zipf", "global") else "rows_kernel",
+                     "kernel": "segments_kernel" if a.workload.startswith(("csr", "coo")) else "band_kernel",
                      "kernel_ms_avg": k_avg, "kernel_ms_min": min(kernel_ms),
                      "algorithmic_bytes": w["kernel_bytes"], "kernel_nnz": w["kernel_nnz"],
                      "kernel_rows": w["kernel_rows"], "call_algorithmic_bytes": w["bytes_total"],

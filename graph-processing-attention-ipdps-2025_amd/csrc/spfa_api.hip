@@ -277,7 +277,7 @@ int spfa_csr_forward(const spfa_problem_t* p, const void* row_off, int row_off_b
   EngineSizing s = size_csr(p->n_q, nnz);
   rc = check_workspace(workspace, workspace_bytes, engine_workspace(s, p->n_q, p->d).total);
   if (rc) return rc;
-  CsrMask mask{row_off, (const uint32_t*)col_ind, row_off_bytes == 8 ? 1 : 0};
+  CsrMask mask{row_off, (const uint32_t*)col_ind, row_off_bytes == 8 ? 1 : 0, nullptr, nullptr};
   return dispatch_csr(p, mask, s, use_nan ? 1 : 0, workspace, (hipStream_t)stream);
 }
 
@@ -304,12 +304,11 @@ int spfa_coo_forward(const spfa_problem_t* p, const void* row_ind, int row_ind_b
   rc = check_workspace(workspace, workspace_bytes,
                        coo_bytes + engine_workspace(s, p->n_q, p->d).total);
   if (rc) return rc;
-  const uint32_t* row_off = nullptr;
-  const uint32_t* cols = nullptr;
-  rc = coo_bucket_by_row(row_ind, row_ind_bytes == 8 ? 1 : 0, (const uint32_t*)col_ind, nnz, p->n_q,
-                         workspace, (hipStream_t)stream, &row_off, &cols);
+  CooCsr csr{};
+  rc = coo_to_csr(row_ind, row_ind_bytes == 8 ? 1 : 0, (const uint32_t*)col_ind, nnz, p->n_q,
+                  workspace, (hipStream_t)stream, &csr);
   if (rc) return rc;
-  CsrMask mask{row_off, cols, 0};
+  CsrMask mask{csr.row_off, (const uint32_t*)col_ind, 0, csr.cols, csr.unsorted};
   return dispatch_csr(p, mask, s, use_nan ? 1 : 0, (char*)workspace + coo_bytes,
                       (hipStream_t)stream);
 }

@@ -13,9 +13,13 @@ struct CsrMask {
   const void* row_off;
   const uint32_t* cols;
   int32_t off64;  // row_off entries are 8 bytes wide (else 4)
+  // COO only: when *use_alt != 0 the columns are read from alt_cols (the bucketed copy) instead
+  const uint32_t* alt_cols;
+  const uint32_t* use_alt;
   struct Row {
     int64_t start;
     int64_t deg;
+    const uint32_t* cols;
   };
   __device__ __forceinline__ Row row(int64_t i) const {
     int64_t a, b;
@@ -28,10 +32,12 @@ struct CsrMask {
       a = (int64_t)p[i];
       b = (int64_t)p[i + 1];
     }
-    return Row{a, b - a};
+    const uint32_t* cp = cols;
+    if (use_alt != nullptr && *use_alt != 0u) cp = alt_cols;
+    return Row{a, b - a, cp};
   }
   __device__ __forceinline__ int64_t col(const Row& r, int64_t t, bool&) const {
-    return (int64_t)cols[r.start + t];
+    return (int64_t)r.cols[r.start + t];
   }
 };
 

@@ -23,8 +23,36 @@ __device__ __forceinline__ int64_t load_index(const void* p, int64_t i, int wide
   return wide ? (int64_t)((const uint64_t*)p)[i] : (int64_t)((const uint32_t*)p)[i];
 }
 
+// 1 -> *flag when the entries are not sorted by row or hold a row outside [0, n_rows)
+__global__ void coo_check_sorted_kernel(const void* row_ind, int wide, int64_t nnz, int64_t n_rows,
+                                        uint32_t* flag) {
+  int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  bool bad = false;
+  for (; e < nnz; e += stride) {
+    const int64_t r = load_index(row_ind, e, wide);
+    if (r < 0 || r >= n_rows) bad = true;
+    if (e > 0 && load_index(row_ind, e - 1, wide) > r) bad = true;
+  }
+  if (bad) *flag = 1u;
+}
+
+// sorted entries: row_off[r] = first entry whose row is >= r
+__global__ void coo_sorted_offsets_kernel(const void* row_ind, int wide, int64_t nnz, int64_t n_rows,
+                                          const uint32_t* flag, uint32_t* row_off) {
+  if (*flag) return;
+  int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (; e <= nnz; e += stride) {
+    const int64_t prev = e > 0 ? load_index(row_ind, e - 1, wide) : -1;
+    const int64_t cur = e < nnz ? load_index(row_ind, e, wide) : n_rows;
+    for (int64_t r = prev + 1; r <= cur; r++) row_off[r] = (uint32_t)e;
+  }
+}
+
 __global__ void coo_histogram_kernel(const void* row_ind, int wide, int64_t nnz, int64_t n_rows,
-                                     uint32_t* counts) {
+                                     const uint32_t* flag, uint32_t* counts) {
+  if (!*flag) return;
   int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   const int64_t stride = (int64_t)gridDim.x * blockDim.x;
   for (; e < nnz; e += stride) {
@@ -34,8 +62,9 @@ __global__ void coo_histogram_kernel(const void* row_ind, int wide, int64_t nnz,
 }
 
 __global__ void coo_scatter_kernel(const void* row_ind, int wide, const uint32_t* col_ind,
-                                   int64_t nnz, int64_t n_rows, uint32_t* cursor,
-                                   uint32_t* cols_out) {
+                                   int64_t nnz, int64_t n_rows, const uint32_t* flag,
+                                   uint32_t* cursor, uint32_t* cols_out) {
+  if (!*flag) return;
   int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   const int64_t stride = (int64_t)gridDim.x * blockDim.x;
   for (; e < nnz; e += stride) {
@@ -77,9 +106,12 @@ __device__ __forceinline__ uint32_t block_exclusive_scan(uint32_t x, uint32_t& t
   return wave_prefix + inc - x;
 }
 
+// (the scan kernels take an optional gate: they return at once when *gate == 0)
 __global__ __launch_bounds__(kScanThreads) void scan_tile_sums_kernel(const uint32_t* in, int64_t n,
-                                                                      uint32_t* tile_sums) {
+                                                                      uint32_t* tile_sums,
+                                                                      const uint32_t* gate) {
   __shared__ uint32_t lds[4];
+  if (gate != nullptr && !*gate) return;
   const int64_t base = (int64_t)blockIdx.x * kScanTile + (int64_t)threadIdx.x * kScanPerThread;
   uint32_t s = 0;
 #pragma unroll
@@ -91,8 +123,10 @@ __global__ __launch_bounds__(kScanThreads) void scan_tile_sums_kernel(const uint
 }
 
 // single block: exclusive scan of the tile sums in place
-__global__ __launch_bounds__(kScanThreads) void scan_sums_kernel(uint32_t* tile_sums, int64_t n_tiles) {
+__global__ __launch_bounds__(kScanThreads) void scan_sums_kernel(uint32_t* tile_sums, int64_t n_tiles,
+                                                                 const uint32_t* gate) {
   __shared__ uint32_t lds[4];
+  if (gate != nullptr && !*gate) return;
   uint32_t carry = 0;
   for (int64_t base = 0; base < n_tiles; base += kScanThreads) {
     int64_t i = base + threadIdx.x;
@@ -108,8 +142,10 @@ __global__ __launch_bounds__(kScanThreads) void scan_sums_kernel(uint32_t* tile_
 // written by the block that owns element n-1
 __global__ __launch_bounds__(kScanThreads) void scan_apply_kernel(const uint32_t* in, int64_t n,
                                                                   const uint32_t* tile_sums,
-                                                                  uint32_t* out, uint32_t* out2) {
+                                                                  uint32_t* out, uint32_t* out2,
+                                                                  const uint32_t* gate) {
   __shared__ uint32_t lds[4];
+  if (gate != nullptr && !*gate) return;
   const int64_t base = (int64_t)blockIdx.x * kScanTile + (int64_t)threadIdx.x * kScanPerThread;
   uint32_t v[kScanPerThread];
   uint32_t s = 0;
@@ -165,13 +201,13 @@ CooWorkspace coo_workspace(int64_t n_rows, int64_t nnz) {
   w.off_cursor = off;  off = align_up(off + (size_t)(n_rows + 1) * 4, 256);
   w.off_tiles = off;   off = align_up(off + (size_t)n_tiles * 4, 256);
   w.off_cols = off;    off = align_up(off + (size_t)(nnz > 0 ? nnz : 1) * 4, 256);
+  w.off_flag = off;    off = align_up(off + 4, 256);
   w.total = off;
   return w;
 }
 
-int coo_bucket_by_row(const void* row_ind, int row_wide, const uint32_t* col_ind, int64_t nnz,
-                      int64_t n_rows, void* ws, hipStream_t stream, const uint32_t** row_off_out,
-                      const uint32_t** cols_out) {
+int coo_to_csr(const void* row_ind, int row_wide, const uint32_t* col_ind, int64_t nnz,
+               int64_t n_rows, void* ws, hipStream_t stream, CooCsr* out) {
   CooWorkspace w = coo_workspace(n_rows, nnz);
   char* base = (char*)ws;
   uint32_t* counts = (uint32_t*)(base + w.off_counts);
@@ -179,25 +215,33 @@ int coo_bucket_by_row(const void* row_ind, int row_wide, const uint32_t* col_ind
   uint32_t* cursor = (uint32_t*)(base + w.off_cursor);
   uint32_t* tiles = (uint32_t*)(base + w.off_tiles);
   uint32_t* cols = (uint32_t*)(base + w.off_cols);
+  uint32_t* flag = (uint32_t*)(base + w.off_flag);
   const int64_t n_tiles = (n_rows + kScanTile - 1) / kScanTile;
 
   hipLaunchKernelGGL(fill_u32_kernel, dim3(grid_for(n_rows + 1, 256, 4096)), dim3(256), 0, stream,
                      counts, n_rows + 1, 0u);
+  hipLaunchKernelGGL(fill_u32_kernel, dim3(1), dim3(64), 0, stream, flag, (int64_t)1, 0u);
   if (nnz > 0)
+    hipLaunchKernelGGL(coo_check_sorted_kernel, dim3(grid_for(nnz, 256, 8192)), dim3(256), 0, stream,
+                       row_ind, row_wide, nnz, n_rows, flag);
+  // sorted: offsets straight from the row array
+  hipLaunchKernelGGL(coo_sorted_offsets_kernel, dim3(grid_for(nnz + 1, 256, 16384)), dim3(256), 0,
+                     stream, row_ind, row_wide, nnz, n_rows, flag, row_off);
+  // unsorted: bucket by row
+  if (nnz > 0) {
     hipLaunchKernelGGL(coo_histogram_kernel, dim3(grid_for(nnz, 256, 16384)), dim3(256), 0, stream,
-                       row_ind, row_wide, nnz, n_rows, counts);
-  if (n_rows > 0) {
+                       row_ind, row_wide, nnz, n_rows, flag, counts);
     hipLaunchKernelGGL(scan_tile_sums_kernel, dim3((unsigned)n_tiles), dim3(kScanThreads), 0, stream,
-                       counts, n_rows, tiles);
-    hipLaunchKernelGGL(scan_sums_kernel, dim3(1), dim3(kScanThreads), 0, stream, tiles, n_tiles);
+                       counts, n_rows, tiles, flag);
+    hipLaunchKernelGGL(scan_sums_kernel, dim3(1), dim3(kScanThreads), 0, stream, tiles, n_tiles, flag);
     hipLaunchKernelGGL(scan_apply_kernel, dim3((unsigned)n_tiles), dim3(kScanThreads), 0, stream,
-                       counts, n_rows, tiles, row_off, cursor);
-  }
-  if (nnz > 0)
+                       counts, n_rows, tiles, row_off, cursor, flag);
     hipLaunchKernelGGL(coo_scatter_kernel, dim3(grid_for(nnz, 256, 16384)), dim3(256), 0, stream,
-                       row_ind, row_wide, col_ind, nnz, n_rows, cursor, cols);
-  *row_off_out = row_off;
-  *cols_out = cols;
+                       row_ind, row_wide, col_ind, nnz, n_rows, flag, cursor, cols);
+  }
+  out->row_off = row_off;
+  out->cols = cols;
+  out->unsorted = flag;
   return hipGetLastError() == hipSuccess ? 0 : 4;
 }
 

@@ -10,17 +10,26 @@ namespace spfa {
 inline size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 
 struct CooWorkspace {
-  size_t off_counts, off_row_off, off_cursor, off_tiles, off_cols, total;
+  size_t off_counts, off_row_off, off_cursor, off_tiles, off_cols, off_flag, total;
 };
 
 CooWorkspace coo_workspace(int64_t n_rows, int64_t nnz);
 
-// Buckets COO entries by row into 32-bit CSR arrays placed in `ws` (coo_workspace().total bytes).
-// Entries with a row outside [0, n_rows) are dropped.  Columns keep no particular order inside
-// a row.
-int coo_bucket_by_row(const void* row_ind, int row_wide, const uint32_t* col_ind, int64_t nnz,
-                      int64_t n_rows, void* ws, hipStream_t stream, const uint32_t** row_off_out,
-                      const uint32_t** cols_out);
+struct CooCsr {
+  const uint32_t* row_off;    // n_rows + 1 offsets (32-bit)
+  const uint32_t* cols;       // bucketed columns, valid when *unsorted != 0
+  const uint32_t* unsorted;   // device flag: 0 = the entries came sorted by row, use the
+                              // caller's column array as it is
+};
+
+// Turns COO entries into 32-bit CSR offsets placed in `ws` (coo_workspace().total bytes).
+// Entries that already come sorted by row (the reference's contract) only need the offsets;
+// otherwise they are bucketed by row (histogram, scan, scatter) and the columns copied, in no
+// particular order inside a row.  The choice is made on the device (no host synchronisation):
+// both sets of kernels are enqueued and the ones that are not needed return at once.
+// Entries with a row outside [0, n_rows) are dropped (and force the bucketing path).
+int coo_to_csr(const void* row_ind, int row_wide, const uint32_t* col_ind, int64_t nnz,
+               int64_t n_rows, void* ws, hipStream_t stream, CooCsr* out);
 
 // Global-row bookkeeping for the global-minus-local mask.  `bits` holds (n+31)/32 bitmap words
 // followed by one counter word; afterwards bit i is set for every listed i in [0, n), `uq` holds

@@ -343,6 +343,33 @@ def test_coo_unsorted_equals_csr(mods, row_dtype):
     assert torch.allclose(torch.nan_to_num(o), torch.nan_to_num(o2), atol=2e-5)
 
 
+@pytest.mark.parametrize("row_dtype", [torch.uint64, torch.int32])
+def test_coo_sorted_by_row_takes_the_callers_columns(mods, row_dtype):
+    """Row-sorted entries (the reference's contract), columns in any order inside a row, leading,
+    inner and trailing empty rows."""
+    n, d = 3000, 64
+    q, k, v = dev_qkv(n, d, torch.float32, 19)
+    g = torch.Generator().manual_seed(19)
+    deg = torch.randint(0, 50, (n,), generator=g)
+    deg[:7] = 0
+    deg[100:300] = 0
+    deg[-40:] = 0
+    deg[1234] = 1500
+    ro, ci = syn.csr_from_degrees(deg, n, g, "cpu", force_diagonal=False)
+    r, c = syn.coo_from_csr(ro, ci)
+    # shuffle the columns inside every row: still sorted by row
+    key = r.double() + torch.rand(c.numel(), generator=g).double() * 0.5
+    order = torch.argsort(key)
+    r, c = r[order].contiguous(), c[order].contiguous()
+    assert torch.all(r[1:] >= r[:-1])
+    m, l, o = state(n, d, torch.float32)
+    mods["spfa_coo"].forward(q, k, v, r.to(row_dtype).to(DEV), c.to(torch.uint32).to(DEV),
+                             torch.ones(c.numel(), device=DEV), m, l, o, True)
+    sync()
+    ref = c_oracle.csr(np64(q), np64(k), np64(v), ro.numpy(), ci.numpy(), use_nan=True)
+    check(o, m, l, *ref, torch.float32, dead_expect="nan")
+
+
 def test_coo_power_law_with_many_empty_rows(mods):
     n, d = 65536, 64
     q, k, v = dev_qkv(n, d, torch.float32, 17)
