@@ -402,7 +402,7 @@ def main():
         "algorithmic_GBs": w["bytes_total"] / (ms_per_step * 1e-3) / 1e9,
         "roofline": {"bound": "hbm", "achieved": achieved_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved_gbs / HBM_PEAK_GBS, "traffic": measured_traffic(a.workload, a.dtype),
-                     "kernel": "segments_kernel" if a.workload.startswith(("csr", "coo")) else "band_kernel",
+                     "kernel": "segments_kernel" if a.workload.startswith(("csr", "coo")) else "tile_kernel",
                      "kernel_ms_avg": k_avg, "kernel_ms_min": min(kernel_ms),
                      "algorithmic_bytes": w["kernel_bytes"], "kernel_nnz": w["kernel_nnz"],
                      "kernel_rows": w["kernel_rows"], "call_algorithmic_bytes": w["bytes_total"],

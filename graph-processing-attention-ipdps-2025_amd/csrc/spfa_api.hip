@@ -134,7 +134,7 @@ int dispatch_stride(const spfa_problem_t* p, const StrideMask& mask, const Engin
 // Band / block masks whose rows are long enough go to the dense-tile kernel.
 int dispatch_band(const spfa_problem_t* p, int64_t w, int64_t stride, int64_t block, int64_t cnt,
                   int use_nan, hipStream_t stream) {
-  BandArgs a{};
+  TileArgs a{};
   a.t = make_tensors(p);
   a.n = p->n_q;
   a.s = stride;
@@ -419,7 +419,7 @@ int spfa_global_no_local_forward(const spfa_problem_t* p, const int32_t* global_
   if (rc) return rc;
 
   // dense tiles when the shape allows it
-  BandArgs a{};
+  TileArgs a{};
   a.t = make_tensors(p);
   a.n = n;
   a.w = local_size;

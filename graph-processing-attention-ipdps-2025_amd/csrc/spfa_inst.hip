@@ -17,7 +17,7 @@ int run_stride<SPFA_INST_T>(const Tensors& t, const StrideMask& mask, const Engi
   return run_engine<SPFA_INST_T, StrideMask>(t, mask, s, use_nan, ws, stream);
 }
 template <>
-int run_band<SPFA_INST_T>(const BandArgs& a, int use_nan, hipStream_t stream) {
+int run_band<SPFA_INST_T>(const TileArgs& a, int use_nan, hipStream_t stream) {
   return run_band_tiles<SPFA_INST_T>(a, use_nan, stream);
 }
 #elif SPFA_INST_MASK == 2
@@ -27,7 +27,7 @@ int run_global<SPFA_INST_T>(const Tensors& t, const GlobalMask& mask, const Engi
   return run_engine<SPFA_INST_T, GlobalMask>(t, mask, s, use_nan, ws, stream);
 }
 template <>
-int run_global_dense<SPFA_INST_T>(const BandArgs& a, hipStream_t stream) {
+int run_global_dense<SPFA_INST_T>(const TileArgs& a, hipStream_t stream) {
   return run_global_tiles<SPFA_INST_T>(a, stream);
 }
 #else

@@ -1,7 +1,7 @@
 // Entry points of the per-(mask, element type) translation units.
 #pragma once
 
-#include "spfa_band.hpp"
+#include "spfa_tiles.hpp"
 #include "spfa_engine.hpp"
 #include "spfa_masks.hpp"
 
@@ -15,10 +15,10 @@ int run_stride(const Tensors& t, const StrideMask& mask, const EngineSizing& s, 
                void* ws, hipStream_t stream);
 // Dense-tile (MFMA) path for band / block masks; -1 when the shape is not covered.
 template <typename T>
-int run_band(const BandArgs& a, int use_nan, hipStream_t stream);
+int run_band(const TileArgs& a, int use_nan, hipStream_t stream);
 // Dense-tile path for the global-minus-local mask; -1 when the shape is not covered.
 template <typename T>
-int run_global_dense(const BandArgs& a, hipStream_t stream);
+int run_global_dense(const TileArgs& a, hipStream_t stream);
 template <typename T>
 int run_global(const Tensors& t, const GlobalMask& mask, const EngineSizing& s, int use_nan,
                void* ws, hipStream_t stream);

@@ -35,7 +35,7 @@ typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 // query's window (Sparse_FlashAttention_Global_No_Local/sp_flatt_global_no_local_kernel.cu:38-64).
 enum { kTileBand = 0, kTileGlobalRows = 1, kTileGlobalCols = 2 };
 
-struct BandArgs {
+struct TileArgs {
   Tensors t;
   int64_t n;              // tokens
   int64_t w;              // window half-width (band: subsequence positions; global: tokens)
@@ -58,7 +58,7 @@ struct BandArgs {
 };
 
 template <typename T, int D>
-struct BandCfg {
+struct TileCfg {
   static constexpr bool kF32 = sizeof(T) == 4;
   static constexpr int BM = 128;  // queries per workgroup
   // keys per LDS tile (fp32 at d = 128 takes half tiles to stay inside 64 KB of LDS)
@@ -100,8 +100,8 @@ __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
 }
 
 template <typename T, int D, int MODE>
-__global__ __launch_bounds__(256, 2) void band_kernel(BandArgs a) {
-  using C = BandCfg<T, D>;
+__global__ __launch_bounds__(256, 2) void tile_kernel(TileArgs a) {
+  using C = TileCfg<T, D>;
   constexpr bool kF32 = C::kF32;
   constexpr int BM = C::BM, BN = C::BN, EB = C::EB, NB = C::NB;
   __shared__ __attribute__((aligned(16))) T lds[C::K_ELEMS + C::V_ELEMS];
@@ -508,7 +508,7 @@ __global__ void band_dead_rows_kernel(T* out, int64_t n, int d, int64_t block, i
 // then weighted sums with the splits spread over the threads), fold the incoming state in,
 // write the row.
 template <typename T, int D>
-__global__ __launch_bounds__(256) void global_rows_merge_kernel(BandArgs a) {
+__global__ __launch_bounds__(256) void global_rows_merge_kernel(TileArgs a) {
   constexpr int NSUB = 256 / D;  // threads per output element
   __shared__ float red[4];
   __shared__ float part[256];
@@ -578,13 +578,13 @@ __global__ __launch_bounds__(256) void global_rows_merge_kernel(BandArgs a) {
 }
 
 template <typename T, int D>
-int launch_band(const BandArgs& a, int use_nan, hipStream_t stream) {
+int launch_band_tiles(const TileArgs& a, int use_nan, hipStream_t stream) {
   const KernelEvents ev = kernel_events();
   const bool timed = ev.start != nullptr && ev.stop != nullptr;
   if (a.n_tiles > 0) {
     const int64_t grid = (a.n_tiles + 7) / 8 * 8;
     if (timed) (void)hipEventRecord(ev.start, stream);
-    hipLaunchKernelGGL((band_kernel<T, D, kTileBand>), dim3((unsigned)grid), dim3(256), 0, stream, a);
+    hipLaunchKernelGGL((tile_kernel<T, D, kTileBand>), dim3((unsigned)grid), dim3(256), 0, stream, a);
     if (timed) (void)hipEventRecord(ev.stop, stream);
   }
   if (a.block > 0 && use_nan && a.s > 1) {
@@ -598,15 +598,15 @@ int launch_band(const BandArgs& a, int use_nan, hipStream_t stream) {
 // Global minus local: non-global rows against the listed globals, then the global rows against
 // everything (key range split over workgroups), then the fold of the splits.
 template <typename T, int D>
-int launch_global_tiles(const BandArgs& a, hipStream_t stream) {
+int launch_global_tiles(const TileArgs& a, hipStream_t stream) {
   const KernelEvents ev = kernel_events();
   const bool timed = ev.start != nullptr && ev.stop != nullptr;
   const int64_t grid_cols = (a.n + 127) / 128;
-  hipLaunchKernelGGL((band_kernel<T, D, kTileGlobalCols>), dim3((unsigned)grid_cols), dim3(256), 0,
+  hipLaunchKernelGGL((tile_kernel<T, D, kTileGlobalCols>), dim3((unsigned)grid_cols), dim3(256), 0,
                      stream, a);
   const int64_t q_tiles = (a.n_globs + 127) / 128;
   if (timed) (void)hipEventRecord(ev.start, stream);
-  hipLaunchKernelGGL((band_kernel<T, D, kTileGlobalRows>), dim3((unsigned)(q_tiles * a.n_split)),
+  hipLaunchKernelGGL((tile_kernel<T, D, kTileGlobalRows>), dim3((unsigned)(q_tiles * a.n_split)),
                      dim3(256), 0, stream, a);
   if (timed) (void)hipEventRecord(ev.stop, stream);
   hipLaunchKernelGGL((global_rows_merge_kernel<T, D>), dim3((unsigned)a.n_globs), dim3(256), 0, stream,
@@ -622,15 +622,15 @@ inline bool tile_shape_ok(const Tensors& t, size_t elem_bytes) {
 
 // Returns -1 when the shape is not covered (caller falls back to the row-gather engine).
 template <typename T>
-int run_band_tiles(const BandArgs& a, int use_nan, hipStream_t stream) {
+int run_band_tiles(const TileArgs& a, int use_nan, hipStream_t stream) {
   if (!tile_shape_ok(a.t, sizeof(T))) return -1;
-  if (a.t.d == 64) return launch_band<T, 64>(a, use_nan, stream);
-  if (a.t.d == 128) return launch_band<T, 128>(a, use_nan, stream);
+  if (a.t.d == 64) return launch_band_tiles<T, 64>(a, use_nan, stream);
+  if (a.t.d == 128) return launch_band_tiles<T, 128>(a, use_nan, stream);
   return -1;
 }
 
 template <typename T>
-int run_global_tiles(const BandArgs& a, hipStream_t stream) {
+int run_global_tiles(const TileArgs& a, hipStream_t stream) {
   if (!tile_shape_ok(a.t, sizeof(T))) return -1;
   if (a.t.d == 64) return launch_global_tiles<T, 64>(a, stream);
   if (a.t.d == 128) return launch_global_tiles<T, 128>(a, stream);

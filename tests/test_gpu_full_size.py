@@ -1,0 +1,189 @@
+"""The benchmark configurations at their full sizes, on the GPU, checked through properties that do
+not need a full-size CPU result: closed forms (window 0 => out == v, V == 1 => out == 1), the
+statistics of a constant-score problem, chained == single call, COO == CSR, and the float64 oracle
+on a random sample of rows."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import spfa_synth as syn
+from helpers import OUT_TOL, np64
+from oracle import c_oracle
+from oracle import spfa_oracle as so
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+def sample_check(q, k, v, out, m, l, rows, live_fn, dtype, expect_dead=None):
+    """Oracle on the sampled rows only (live_fn(i) -> column list of row i)."""
+    rows = np.asarray(rows, dtype=np.int64)
+    cols = [np.asarray(live_fn(int(i)), dtype=np.int64) for i in rows]
+    off = np.zeros(len(rows) + 1, dtype=np.int64)
+    np.cumsum([len(c) for c in cols], out=off[1:])
+    ci = np.concatenate(cols) if len(cols) else np.zeros(0, np.int64)
+    sel = torch.as_tensor(rows).to(DEV)
+    ref_o, ref_m, ref_l = c_oracle.csr(np64(q[sel]), np64(k), np64(v), off, ci)
+    got_o, got_m, got_l = np64(out[sel]), np64(m[sel]), np64(l[sel])
+    live = ref_l > 0
+    assert live.any()
+    err = np.abs(got_o[live] - ref_o[live]).max()
+    assert err <= OUT_TOL[dtype], "max-abs %.3e" % err
+    with np.errstate(divide="ignore", invalid="ignore"):
+        lse_err = np.abs((got_m + np.log(got_l))[live] - (ref_m + np.log(ref_l))[live]).max()
+    assert lse_err <= (1e-4 if dtype == torch.float32 else 2e-3)
+    if (~live).any():
+        if expect_dead == "nan":
+            assert np.isnan(got_o[~live]).all()
+        else:
+            assert np.all(got_o[~live] == 0) and np.all(got_l[~live] == 0)
+
+
+def rand_rows(n, count, seed):
+    g = torch.Generator().manual_seed(seed)
+    return torch.sort(torch.randperm(n, generator=g)[:count])[0].numpy()
+
+
+# ------------------------------------------------------------------ Local N=65536 d=64, fp32 / bf16
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_local_n65536(mods, dtype):
+    n, d, w = 65536, 64, 128
+    q, k, v = syn.qkv(n, d, dtype=dtype, device=DEV, seed=0)
+    m, l, o = syn.fresh_state(n, d, dtype=dtype, device=DEV, state_dtype=torch.float32)
+    mods["spfa_local"].forward(q, k, v, m, l, o, w)
+    rows = np.concatenate([[0, 1, 127, 128, 129, n - 130, n - 129, n - 128, n - 1], rand_rows(n, 150, 1)])
+    sample_check(q, k, v, o, m, l, rows, lambda i: so.live_local(n, w, i), dtype)
+    # closed forms at full size
+    m, l, o = syn.fresh_state(n, d, dtype=dtype, device=DEV, state_dtype=torch.float32)
+    mods["spfa_local"].forward(q, k, v, m, l, o, 0)
+    assert torch.equal(o, v) and torch.all(l == 1)
+    ones = torch.ones_like(v)
+    m, l, o = syn.fresh_state(n, d, dtype=dtype, device=DEV, state_dtype=torch.float32)
+    mods["spfa_local"].forward(q, k, ones, m, l, o, w)
+    assert torch.allclose(o.float(), torch.ones_like(o, dtype=torch.float32), atol=1e-2 if dtype != torch.float32 else 1e-5)
+    # q == 0: every score is 0 -> m == 0 and l == number of live columns (closed form)
+    m, l, o = syn.fresh_state(n, d, dtype=dtype, device=DEV, state_dtype=torch.float32)
+    mods["spfa_local"].forward(torch.zeros_like(q), k, v, m, l, o, w)
+    i = torch.arange(n, device=DEV)
+    cnt = (torch.clamp(i + w + 1, max=n) - torch.clamp(i - w, min=0)).float()
+    assert torch.all(m == 0) and torch.equal(l, cnt)
+    assert int(l.sum().item()) == so.nnz_local(n, w)
+
+
+# ------------------------------------------------------------------ CSR N=131072 d=64 fp32, Zipf(1.5)
+def test_csr_zipf_n131072(mods):
+    n, d = 131072, 64
+    q, k, v = syn.qkv(n, d, device=DEV, seed=0)
+    ro, ci = syn.zipf_csr(n, 1.5, 1, 4096, device=DEV, seed=0)
+    ro_t, ci_t = ro.to(torch.uint64), ci.to(torch.uint32)
+    val = torch.empty(ci.numel(), device=DEV)
+    m, l, o = syn.fresh_state(n, d, device=DEV)
+    mods["spfa_csr"].forward(q, k, v, ro_t, ci_t, val, m, l, o, False)
+    ro_c, ci_c = ro.cpu().numpy(), ci.cpu().numpy()
+    deg = ro_c[1:] - ro_c[:-1]
+    assert deg.min() >= 1 and deg.max() == 4096
+    # sample every length class: shortest, longest, around the in-place limit, random
+    rows = np.concatenate([np.nonzero(deg == 1)[0][:20], np.nonzero(deg == 4096)[0][:20],
+                           np.nonzero((deg >= 30) & (deg <= 36))[0][:20],
+                           np.nonzero((deg > 250) & (deg < 520))[0][:20], rand_rows(n, 100, 2)])
+    sample_check(q, k, v, o, m, l, rows, lambda i: ci_c[ro_c[i]:ro_c[i + 1]], torch.float32)
+    # q == 0 -> l == row length exactly, m == 0
+    m2, l2, o2 = syn.fresh_state(n, d, device=DEV)
+    mods["spfa_csr"].forward(torch.zeros_like(q), k, v, ro_t, ci_t, val, m2, l2, o2, False)
+    assert torch.all(m2 == 0) and torch.equal(l2, (ro[1:] - ro[:-1]).float())
+    # the same mask as shuffled COO gives the same result
+    r, c = syn.coo_from_csr(ro, ci, shuffle_seed=3)
+    m3, l3, o3 = syn.fresh_state(n, d, device=DEV)
+    mods["spfa_coo"].forward(q, k, v, r.to(torch.uint64), c.to(torch.uint32), val, m3, l3, o3, False)
+    assert torch.allclose(o3, o, atol=2e-5) and torch.allclose(m3, m, atol=1e-6)
+    assert torch.allclose(l3, l, rtol=1e-5)
+    # two disjoint halves chained == one call
+    keep = torch.rand(ci.numel(), device=DEV, generator=torch.Generator(device=DEV).manual_seed(4)) < 0.5
+    rows_of = torch.repeat_interleave(torch.arange(n, device=DEV), ro[1:] - ro[:-1])
+    m4, l4, o4 = syn.fresh_state(n, d, device=DEV)
+    for part in (keep, ~keep):
+        cnt = torch.bincount(rows_of[part], minlength=n)
+        off = torch.zeros(n + 1, dtype=torch.int64, device=DEV)
+        off[1:] = torch.cumsum(cnt, 0)
+        cp = ci[part].to(torch.uint32)
+        mods["spfa_csr"].forward(q, k, v, off.to(torch.uint64), cp, torch.empty(cp.numel(), device=DEV), m4, l4, o4, False)
+    assert torch.allclose(o4, o, atol=2e-5) and torch.allclose(m4, m, atol=1e-6)
+    assert torch.allclose(l4, l, rtol=1e-5)
+
+
+# ------------------------------------------------------------------ dilated masks N=262144 d=128 bf16
+def test_local_1d_dilated_n262144(mods):
+    n, d, w, dil = 262144, 128, 256, 2
+    dtype = torch.bfloat16
+    q, k, v = syn.qkv(n, d, dtype=dtype, device=DEV, seed=0, scale=0.5)
+    m, l, o = syn.fresh_state(n, d, dtype=dtype, device=DEV, state_dtype=torch.float32)
+    mods["spfa_local_1d_dilated"].forward(q, k, v, m, l, o, w, dil)
+    rows = np.concatenate([[0, 1, 2, 3, 767, 768, 769, n - 770, n - 3, n - 2, n - 1], rand_rows(n, 100, 5)])
+    sample_check(q, k, v, o, m, l, rows, lambda i: so.live_local_1d_dilated(n, w, dil, i), dtype)
+    m, l, o = syn.fresh_state(n, d, dtype=dtype, device=DEV, state_dtype=torch.float32)
+    mods["spfa_local_1d_dilated"].forward(torch.zeros_like(q), k, v, m, l, o, w, dil)
+    assert torch.all(m == 0)
+    assert int(l.double().sum().item()) == so.nnz_local_1d_dilated(n, w, dil)
+
+
+@pytest.mark.parametrize("use_nan", [True, False])
+def test_local_2d_dilated_n262144(mods, use_nan):
+    n, d, block, dil = 262144, 128, 256, 2
+    dtype = torch.bfloat16
+    q, k, v = syn.qkv(n, d, dtype=dtype, device=DEV, seed=0, scale=0.5)
+    m, l, o = syn.fresh_state(n, d, dtype=dtype, device=DEV, state_dtype=torch.float32)
+    mods["spfa_local_2d_dilated"].forward(q, k, v, m, l, o, block, dil, use_nan)
+    rows = np.concatenate([[0, 1, 3, 255, 256, n - 256, n - 1], rand_rows(n, 120, 6)])
+    sample_check(q, k, v, o, m, l, rows, lambda i: so.live_local_2d_dilated(n, block, dil, i), dtype,
+                 expect_dead="nan" if use_nan else None)
+    live = ((torch.arange(n, device=DEV) % block) % (dil + 1)) == 0
+    assert int(live.sum()) == 88064
+    assert torch.all(l[~live] == 0) and torch.all(torch.isneginf(m[~live]))
+    assert torch.isnan(o[~live]).all() if use_nan else torch.all(o[~live] == 0)
+    assert torch.isfinite(o[live].float()).all()
+
+
+# ------------------------------------------------------------------ N = 1,048,576 d=64 fp32
+def test_global_no_local_n1m(mods):
+    n, d, g, w = 1 << 20, 64, 64, 64
+    q, k, v = syn.qkv(n, d, device=DEV, seed=0)
+    globs = syn.global_indices(n, g, device=DEV, seed=0)
+    m, l, o = syn.fresh_state(n, d, device=DEV)
+    mods["spfa_global_no_local"].forward(q, k, v, m, l, o, globs, w)
+    gl = globs.cpu().numpy()
+    near = np.clip(np.concatenate([gl[:8] - 1, gl[:8] + 1, gl[:4] - w, gl[:4] + w + 1]), 0, n - 1)
+    rows = np.unique(np.concatenate([gl[:3], near, rand_rows(n, 60, 7)]))
+    sample_check(q, k, v, o, m, l, rows, lambda i: so.live_global_no_local(n, gl, w, i), torch.float32)
+    # q == 0: l counts the live columns; the total is the closed-form nnz
+    m, l, o = syn.fresh_state(n, d, device=DEV)
+    mods["spfa_global_no_local"].forward(torch.zeros_like(q), k, v, m, l, o, globs, w)
+    assert int(l.double().sum().item()) == so.nnz_global_no_local(n, gl, w)
+
+
+def test_coo_zipf_n1m_50m_entries(mods):
+    n, d = 1 << 20, 64
+    q, k, v = syn.qkv(n, d, device=DEV, seed=0)
+    r, c = syn.zipf_coo(n, 50_000_000, 1.3, device=DEV, seed=0)
+    nnz = c.numel()
+    assert nnz == 50_000_000
+    r_t, c_t = r.to(torch.uint64), c.to(torch.uint32)
+    val = torch.empty(nnz, device=DEV)
+    m, l, o = syn.fresh_state(n, d, device=DEV)
+    mods["spfa_coo"].forward(q, k, v, r_t, c_t, val, m, l, o, False)
+    deg = torch.bincount(r, minlength=n)
+    # q == 0 -> l == degree of the row (also checks that no entry was lost or duplicated)
+    m2, l2, o2 = syn.fresh_state(n, d, device=DEV)
+    mods["spfa_coo"].forward(torch.zeros_like(q), k, v, r_t, c_t, val, m2, l2, o2, False)
+    assert torch.equal(l2, deg.float())
+    # the row-sorted copy of the same entries gives the same result (other code path)
+    order = torch.argsort(r, stable=True)
+    m3, l3, o3 = syn.fresh_state(n, d, device=DEV)
+    mods["spfa_coo"].forward(q, k, v, r[order].to(torch.uint64), c[order].to(torch.uint32), val, m3, l3, o3, False)
+    assert torch.allclose(o3, o, atol=2e-5) and torch.allclose(l3, l, rtol=1e-5)
+    # oracle on sampled rows (heaviest rows, empty rows, random rows)
+    heavy = torch.topk(deg, 4)[1].cpu().numpy()
+    empty = torch.nonzero(deg == 0)[:4, 0].cpu().numpy()
+    rows = np.unique(np.concatenate([heavy, empty, rand_rows(n, 40, 8)]))
+    sample_check(q, k, v, o, m, l, rows, lambda i: c[r == i].cpu().numpy(), torch.float32)
