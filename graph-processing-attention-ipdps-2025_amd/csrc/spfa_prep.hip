@@ -183,6 +183,100 @@ __global__ void mark_globals_kernel(const int32_t* globs, int64_t n_globs, int64
   }
 }
 
+// ---- two-pass partition of unsorted COO entries by row -----------------------------------
+constexpr int kPartThreads = 256;
+constexpr int kPartTile = 8192;      // entries per workgroup in pass 1
+constexpr int kPartMaxBuckets = 2048;
+
+// pass 1a: per-tile histogram of the high digit, stored bucket-major: hist[b * n_tiles + tile]
+__global__ __launch_bounds__(kPartThreads) void coo_part_count_kernel(
+    const void* row_ind, int wide, int64_t nnz, int64_t n_rows, int lo_bits, int n_hi,
+    int64_t n_tiles, const uint32_t* flag, uint32_t* hist) {
+  __shared__ uint32_t cnt[kPartMaxBuckets];
+  if (!*flag) return;
+  for (int b = threadIdx.x; b < n_hi; b += kPartThreads) cnt[b] = 0;
+  __syncthreads();
+  const int64_t beg = (int64_t)blockIdx.x * kPartTile;
+  const int64_t end = beg + kPartTile < nnz ? beg + kPartTile : nnz;
+  for (int64_t e = beg + threadIdx.x; e < end; e += kPartThreads) {
+    const int64_t r = load_index(row_ind, e, wide);
+    if (r >= 0 && r < n_rows) atomicAdd(&cnt[r >> lo_bits], 1u);
+  }
+  __syncthreads();
+  for (int b = threadIdx.x; b < n_hi; b += kPartThreads) hist[(int64_t)b * n_tiles + blockIdx.x] = cnt[b];
+}
+
+// pass 1b: hist now holds exclusive prefixes; scatter (row, col) into high-digit order
+__global__ __launch_bounds__(kPartThreads) void coo_part_scatter_kernel(
+    const void* row_ind, int wide, const uint32_t* col_ind, int64_t nnz, int64_t n_rows, int lo_bits,
+    int n_hi, int64_t n_tiles, const uint32_t* flag, const uint32_t* hist, uint32_t* tmp_rows,
+    uint32_t* tmp_cols) {
+  __shared__ uint32_t cur[kPartMaxBuckets];
+  if (!*flag) return;
+  for (int b = threadIdx.x; b < n_hi; b += kPartThreads) cur[b] = hist[(int64_t)b * n_tiles + blockIdx.x];
+  __syncthreads();
+  const int64_t beg = (int64_t)blockIdx.x * kPartTile;
+  const int64_t end = beg + kPartTile < nnz ? beg + kPartTile : nnz;
+  for (int64_t e = beg + threadIdx.x; e < end; e += kPartThreads) {
+    const int64_t r = load_index(row_ind, e, wide);
+    if (r >= 0 && r < n_rows) {
+      const uint32_t pos = atomicAdd(&cur[r >> lo_bits], 1u);
+      tmp_rows[pos] = (uint32_t)r;
+      tmp_cols[pos] = col_ind[e];
+    }
+  }
+}
+
+// pass 2: one workgroup per high bucket; its entries are contiguous in tmp_*.  Count the low
+// digit in LDS, scan, emit the row offsets of the bucket's rows and place the columns.
+__global__ __launch_bounds__(kPartThreads) void coo_part_rows_kernel(
+    int64_t n_rows, int lo_bits, int n_hi, int64_t n_tiles, int64_t n_hist, const uint32_t* flag,
+    const uint32_t* hist, const uint32_t* tmp_rows, const uint32_t* tmp_cols, uint32_t* row_off,
+    uint32_t* cols_out) {
+  __shared__ uint32_t cnt[kPartMaxBuckets];
+  __shared__ uint32_t wave_sums[kPartThreads / kWave];
+  if (!*flag) return;
+  const int b = blockIdx.x;
+  const int n_lo = 1 << lo_bits;
+  const uint32_t beg = hist[(int64_t)b * n_tiles];
+  const uint32_t end = (b + 1 < n_hi) ? hist[(int64_t)(b + 1) * n_tiles] : hist[n_hist];
+  for (int i = threadIdx.x; i < n_lo; i += kPartThreads) cnt[i] = 0;
+  __syncthreads();
+  const uint32_t lo_mask = (uint32_t)n_lo - 1u;
+  for (uint32_t e = beg + threadIdx.x; e < end; e += kPartThreads) atomicAdd(&cnt[tmp_rows[e] & lo_mask], 1u);
+  __syncthreads();
+  // exclusive scan of cnt[0 .. n_lo) in place, kPartThreads values at a time
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  uint32_t carry = beg;
+  for (int base = 0; base < n_lo; base += kPartThreads) {
+    const int i = base + threadIdx.x;
+    const uint32_t x = i < n_lo ? cnt[i] : 0u;
+    const uint32_t inc = wave_inclusive_scan(x, lane);
+    if (lane == kWave - 1) wave_sums[wave] = inc;
+    __syncthreads();
+    uint32_t prefix = 0, total = 0;
+#pragma unroll
+    for (int w = 0; w < kPartThreads / kWave; w++) {
+      const uint32_t sw = wave_sums[w];
+      if (w < wave) prefix += sw;
+      total += sw;
+    }
+    const uint32_t ex = carry + prefix + inc - x;
+    if (i < n_lo) {
+      cnt[i] = ex;  // becomes the cursor of this row
+      const int64_t row = ((int64_t)b << lo_bits) + i;
+      if (row < n_rows) row_off[row] = ex;
+    }
+    carry += total;
+    __syncthreads();
+  }
+  if (b == n_hi - 1 && threadIdx.x == 0) row_off[n_rows] = end;
+  for (uint32_t e = beg + threadIdx.x; e < end; e += kPartThreads) {
+    const uint32_t pos = atomicAdd(&cnt[tmp_rows[e] & lo_mask], 1u);
+    cols_out[pos] = tmp_cols[e];
+  }
+}
+
 inline unsigned grid_for(int64_t n, int threads, int64_t cap) {
   int64_t g = (n + threads - 1) / threads;
   if (g > cap) g = cap;
@@ -194,7 +288,16 @@ inline unsigned grid_for(int64_t n, int threads, int64_t cap) {
 
 CooWorkspace coo_workspace(int64_t n_rows, int64_t nnz) {
   CooWorkspace w{};
-  const int64_t n_tiles = (n_rows + kScanTile - 1) / kScanTile + 1;
+  int bits = 1;
+  while (((int64_t)1 << bits) < n_rows) bits++;
+  w.partition = (bits <= 22 && nnz > 0) ? 1 : 0;
+  const int hi_bits = (bits + 1) / 2;
+  w.lo_bits = bits - hi_bits;
+  w.n_hi = ((n_rows > 0 ? n_rows : 1) + ((int64_t)1 << w.lo_bits) - 1) >> w.lo_bits;
+  w.n_tiles1 = (nnz + kPartTile - 1) / kPartTile;
+  const int64_t n_hist = w.partition ? w.n_hi * w.n_tiles1 : 0;
+  const int64_t scan_len = n_hist > n_rows ? n_hist : n_rows;
+  const int64_t n_tiles = (scan_len + kScanTile - 1) / kScanTile + 1;
   size_t off = 0;
   w.off_counts = off;  off = align_up(off + (size_t)(n_rows + 1) * 4, 256);
   w.off_row_off = off; off = align_up(off + (size_t)(n_rows + 1) * 4, 256);
@@ -202,6 +305,9 @@ CooWorkspace coo_workspace(int64_t n_rows, int64_t nnz) {
   w.off_tiles = off;   off = align_up(off + (size_t)n_tiles * 4, 256);
   w.off_cols = off;    off = align_up(off + (size_t)(nnz > 0 ? nnz : 1) * 4, 256);
   w.off_flag = off;    off = align_up(off + 4, 256);
+  w.off_hist = off;    off = align_up(off + (size_t)(n_hist + 1) * 4, 256);
+  w.off_tmp_rows = off; off = align_up(off + (size_t)(w.partition ? nnz : 0) * 4, 256);
+  w.off_tmp_cols = off; off = align_up(off + (size_t)(w.partition ? nnz : 0) * 4, 256);
   w.total = off;
   return w;
 }
@@ -228,7 +334,26 @@ int coo_to_csr(const void* row_ind, int row_wide, const uint32_t* col_ind, int64
   hipLaunchKernelGGL(coo_sorted_offsets_kernel, dim3(grid_for(nnz + 1, 256, 16384)), dim3(256), 0,
                      stream, row_ind, row_wide, nnz, n_rows, flag, row_off);
   // unsorted: bucket by row
-  if (nnz > 0) {
+  if (nnz > 0 && w.partition) {
+    uint32_t* hist = (uint32_t*)(base + w.off_hist);
+    uint32_t* tmp_rows = (uint32_t*)(base + w.off_tmp_rows);
+    uint32_t* tmp_cols = (uint32_t*)(base + w.off_tmp_cols);
+    const int64_t n_hist = w.n_hi * w.n_tiles1;
+    const int64_t hist_tiles = (n_hist + kScanTile - 1) / kScanTile;
+    hipLaunchKernelGGL(coo_part_count_kernel, dim3((unsigned)w.n_tiles1), dim3(kPartThreads), 0, stream,
+                       row_ind, row_wide, nnz, n_rows, w.lo_bits, (int)w.n_hi, w.n_tiles1, flag, hist);
+    hipLaunchKernelGGL(scan_tile_sums_kernel, dim3((unsigned)hist_tiles), dim3(kScanThreads), 0, stream,
+                       hist, n_hist, tiles, flag);
+    hipLaunchKernelGGL(scan_sums_kernel, dim3(1), dim3(kScanThreads), 0, stream, tiles, hist_tiles, flag);
+    hipLaunchKernelGGL(scan_apply_kernel, dim3((unsigned)hist_tiles), dim3(kScanThreads), 0, stream,
+                       hist, n_hist, tiles, hist, hist, flag);
+    hipLaunchKernelGGL(coo_part_scatter_kernel, dim3((unsigned)w.n_tiles1), dim3(kPartThreads), 0,
+                       stream, row_ind, row_wide, col_ind, nnz, n_rows, w.lo_bits, (int)w.n_hi,
+                       w.n_tiles1, flag, hist, tmp_rows, tmp_cols);
+    hipLaunchKernelGGL(coo_part_rows_kernel, dim3((unsigned)w.n_hi), dim3(kPartThreads), 0, stream,
+                       n_rows, w.lo_bits, (int)w.n_hi, w.n_tiles1, n_hist, flag, hist, tmp_rows, tmp_cols,
+                       row_off, cols);
+  } else if (nnz > 0) {
     hipLaunchKernelGGL(coo_histogram_kernel, dim3(grid_for(nnz, 256, 16384)), dim3(256), 0, stream,
                        row_ind, row_wide, nnz, n_rows, flag, counts);
     hipLaunchKernelGGL(scan_tile_sums_kernel, dim3((unsigned)n_tiles), dim3(kScanThreads), 0, stream,

@@ -10,7 +10,13 @@ namespace spfa {
 inline size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 
 struct CooWorkspace {
-  size_t off_counts, off_row_off, off_cursor, off_tiles, off_cols, off_flag, total;
+  size_t off_counts, off_row_off, off_cursor, off_tiles, off_cols, off_flag;
+  // two-pass partition (used when the row index fits 22 bits)
+  size_t off_hist, off_tmp_rows, off_tmp_cols, total;
+  int partition;       // 1: two-pass LDS partition, 0: per-entry global atomics
+  int lo_bits;         // low digit width; high digit = row >> lo_bits
+  int64_t n_hi;        // high-digit buckets
+  int64_t n_tiles1;    // entry tiles of pass 1
 };
 
 CooWorkspace coo_workspace(int64_t n_rows, int64_t nnz);
@@ -24,8 +30,9 @@ struct CooCsr {
 
 // Turns COO entries into 32-bit CSR offsets placed in `ws` (coo_workspace().total bytes).
 // Entries that already come sorted by row (the reference's contract) only need the offsets;
-// otherwise they are bucketed by row (histogram, scan, scatter) and the columns copied, in no
-// particular order inside a row.  The choice is made on the device (no host synchronisation):
+// otherwise they are bucketed by row and the columns copied, in no particular order inside a
+// row: a two-pass partition with LDS-private histograms (high digit of the row, then low digit
+// inside each high bucket) when the row index fits 22 bits, per-entry global atomics otherwise.  The choice is made on the device (no host synchronisation):
 // both sets of kernels are enqueued and the ones that are not needed return at once.
 // Entries with a row outside [0, n_rows) are dropped (and force the bucketing path).
 int coo_to_csr(const void* row_ind, int row_wide, const uint32_t* col_ind, int64_t nnz,
