@@ -154,7 +154,10 @@ __global__ __launch_bounds__(256, 2) void tile_kernel(TileArgs a) {
   }
 
   const int tid = threadIdx.x;
-  const int lane = tid & 63, wave = tid >> 6;
+  const int lane = tid & 63;
+  // the wavefront index as a scalar: everything derived from it (which key blocks this
+  // wavefront needs) then branches on scalars instead of lane masks
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r = lane & 31, h = lane >> 5;
   const int64_t tw0 = t0 + 32 * wave;  // first query of this wavefront
   const int64_t tq = tw0 + r;          // this lane's query position
@@ -307,20 +310,21 @@ __global__ __launch_bounds__(256, 2) void tile_kernel(TileArgs a) {
     if (!any_need) continue;
 
     f32x16 sreg[NB];
+    const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int jb = 0; jb < NB; jb++) {
-#pragma unroll
-      for (int v = 0; v < 16; v++) sreg[jb][v] = 0.f;
-      if (!need[jb]) continue;
+      if (!need[jb]) continue;  // (filled with -inf below)
       if constexpr (kF32) {
         const float* krow = (const float*)Ks + (32 * jb + r) * C::K_STRIDE + h;
+        sreg[jb] = __builtin_amdgcn_mfma_f32_32x32x2f32(krow[0], qf[0], zero16, 0, 0, 0);
 #pragma unroll
-        for (int ks = 0; ks < D / 2; ks++)
+        for (int ks = 1; ks < D / 2; ks++)
           sreg[jb] = __builtin_amdgcn_mfma_f32_32x32x2f32(krow[2 * ks], qf[ks], sreg[jb], 0, 0, 0);
       } else {
         const T* krow = Ks + (32 * jb + r) * C::K_STRIDE + 8 * h;
+        sreg[jb] = mfma16<T>(*reinterpret_cast<const uint4v*>(krow), qh[0], zero16);
 #pragma unroll
-        for (int ks = 0; ks < D / 16; ks++) {
+        for (int ks = 1; ks < D / 16; ks++) {
           uint4v kx = *reinterpret_cast<const uint4v*>(krow + 16 * ks);
           sreg[jb] = mfma16<T>(kx, qh[ks], sreg[jb]);
         }
