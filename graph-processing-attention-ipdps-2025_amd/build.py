@@ -108,6 +108,10 @@ def _source_loop_depth(kname: str) -> int:
     loop > batch loop; the batch loop is only a real loop when a chunk holds more than two
     batches (it is unrolled otherwise)."""
     import re
+    if "11tile_kernelI" in kname:
+        # key-tile loop; the global-columns mode (third template argument 2) also loops over
+        # query tiles
+        return 2 if re.search(r"Li2EEEv", kname) else 1
     if "15segments_kernelI" not in kname and "11rows_kernelI" not in kname:
         return 1
     seg = "15segments_kernelI" in kname

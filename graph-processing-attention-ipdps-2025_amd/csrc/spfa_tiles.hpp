@@ -50,6 +50,11 @@ struct TileArgs {
   const uint32_t* gbits;  // bit i set <=> token i is a global row
   const int32_t* uq;      // distinct global rows (queries of GlobalRows)
   const uint32_t* n_uq;   // how many
+  int32_t persist;        // GlobalCols: all keys fit one LDS tile; workgroups keep it and walk
+                          // over query tiles (grid-stride)
+  int32_t pair_split;     // GlobalRows with at most 64 global rows: wavefronts 0,1 take the first
+                          // 32 keys of every tile, wavefronts 2,3 the second 32, for the same two
+                          // query blocks; the pairs are folded through LDS at the end
   int64_t key_run;        // GlobalRows: keys per split (multiple of 64)
   int64_t n_split;
   float* pm;              // GlobalRows partials, slot = query * n_split + split
@@ -159,7 +164,20 @@ __global__ __launch_bounds__(256, 2) void tile_kernel(TileArgs a) {
   // wavefront needs) then branches on scalars instead of lane masks
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r = lane & 31, h = lane >> 5;
-  const int64_t tw0 = t0 + 32 * wave;  // first query of this wavefront
+  const T* Qp = (const T*)a.t.q;
+  const T* Kp = (const T*)a.t.k;
+  const T* Vp = (const T*)a.t.v;
+  const float sc = 1.4426950408889634f / sqrtf((float)D);
+  const bool persist = (MODE == kTileGlobalCols) && a.persist != 0;
+  bool staged = false;  // persist: the key tile is already in LDS
+
+  // One trip per query tile.  Only a persistent GlobalCols workgroup makes more than one.
+  for (;; t0 += (int64_t)gridDim.x * BM) {
+  if (t0 >= qlen) break;
+  const bool pair_split = (MODE == kTileGlobalRows) && NB == 2 && a.pair_split != 0;
+  const int wave_q = pair_split ? (wave & 1) : wave;  // query block of this wavefront
+  const int wave_k = pair_split ? (wave >> 1) : -1;   // key block it is restricted to (-1: all)
+  const int64_t tw0 = t0 + 32 * wave_q;  // first query of this wavefront
   const int64_t tq = tw0 + r;          // this lane's query position
   bool q_ok = tq < qlen;
   int64_t q_tok;                       // its token (row of Q / out)
@@ -171,9 +189,6 @@ __global__ __launch_bounds__(256, 2) void tile_kernel(TileArgs a) {
     q_tok = q_ok ? tq : qlen - 1;
     if (q_ok && bit_is_set(a.gbits, q_tok)) q_ok = false;  // global rows belong to GlobalRows
   }
-  const T* Qp = (const T*)a.t.q;
-  const T* Kp = (const T*)a.t.k;
-  const T* Vp = (const T*)a.t.v;
 
   // ---- Q^T operand, kept in registers
   uint4v qh[kF32 ? 1 : C::QREGS];
@@ -201,7 +216,6 @@ __global__ __launch_bounds__(256, 2) void tile_kernel(TileArgs a) {
     for (int v = 0; v < 16; v++) o[eb][v] = 0.f;
   float m = kNegInf;  // running max in log2 units
   float l = 0.f;      // running sum over this lane's half of the keys
-  const float sc = 1.4426950408889634f / sqrtf((float)D);
 
 
   // Tiles are fetched one ahead: the global loads of tile n+1 are issued before tile n is
@@ -287,12 +301,15 @@ __global__ __launch_bounds__(256, 2) void tile_kernel(TileArgs a) {
     }
   };
 
-  if (u_lo < u_hi) fetch(u_lo);
+  if (u_lo < u_hi && !staged) fetch(u_lo);
   for (int64_t ut = u_lo; ut < u_hi; ut += BN) {
-    __syncthreads();  // the previous tile has been consumed
-    stash();
-    __syncthreads();
-    if (ut + BN < u_hi) fetch(ut + BN);
+    if (!staged) {
+      __syncthreads();  // the previous tile has been consumed
+      stash();
+      __syncthreads();
+      if (ut + BN < u_hi) fetch(ut + BN);
+    }
+    if (persist) staged = true;
 
     // ---- this wavefront's share of the tile: up to two 32-key blocks
     // block jb holds keys ut + 32*jb .. +31; it matters iff it overlaps the wavefront's band
@@ -304,7 +321,7 @@ __global__ __launch_bounds__(256, 2) void tile_kernel(TileArgs a) {
       if constexpr (MODE == kTileBand)
         need[jb] = (tw0 < qlen) && (ub < u_hi) && (ub <= tw0 + 31 + a.w) && (ub + 31 + a.w >= tw0);
       else
-        need[jb] = (tw0 < qlen) && (ub < u_hi);
+        need[jb] = (tw0 < qlen) && (ub < u_hi) && (wave_k < 0 || wave_k == jb);
       any_need = any_need || need[jb];
     }
     if (!any_need) continue;
@@ -424,9 +441,39 @@ __global__ __launch_bounds__(256, 2) void tile_kernel(TileArgs a) {
 
   // ---- finish: combine the two key halves, fold the incoming state in, write back
   l += shfl_xor_f32(l, 32);
+  if constexpr (MODE == kTileGlobalRows && NB == 2) {
+    if (pair_split) {
+      // fold wavefront (q, 1) into wavefront (q, 0) through LDS (the tiles are no longer needed)
+      constexpr int XR = EB * 16 + 2;
+      static_assert(2 * XR * kWave * 4 <= C::LDS_BYTES, "exchange area does not fit the tile buffers");
+      float* xs = reinterpret_cast<float*>(lds) + (size_t)wave_q * XR * kWave + lane;
+      __syncthreads();
+      if (wave_k == 1) {
+#pragma unroll
+        for (int eb = 0; eb < EB; eb++)
+#pragma unroll
+          for (int v = 0; v < 16; v++) xs[(eb * 16 + v) * kWave] = o[eb][v];
+        xs[(EB * 16) * kWave] = m;
+        xs[(EB * 16 + 1) * kWave] = l;
+      }
+      __syncthreads();
+      if (wave_k == 1) return;
+      const float m2 = xs[(EB * 16) * kWave], l2 = xs[(EB * 16 + 1) * kWave];
+      const float m_new = fmaxf(m, m2);
+      if (m_new > kNegInf) {
+        const float fa = __builtin_amdgcn_exp2f(m - m_new), fb = __builtin_amdgcn_exp2f(m2 - m_new);
+        l = l * fa + l2 * fb;
+#pragma unroll
+        for (int eb = 0; eb < EB; eb++)
+#pragma unroll
+          for (int v = 0; v < 16; v++) o[eb][v] = o[eb][v] * fa + xs[(eb * 16 + v) * kWave] * fb;
+        m = m_new;
+      }
+    }
+  }
   if constexpr (MODE == kTileGlobalRows) {
     // partial result of this key split; an empty one is (m, l, acc) = (-inf, 0, 0)
-    if (!q_ok) return;
+    if (!q_ok) return;  // (this mode makes a single trip)
     const int64_t slot = tq * a.n_split + split;
     const bool any = l > 0.f;
     float* prow = a.pacc + slot * D;
@@ -446,7 +493,7 @@ __global__ __launch_bounds__(256, 2) void tile_kernel(TileArgs a) {
     }
     return;
   }
-  if (!q_ok || !(l > 0.f)) return;
+  if (q_ok && l > 0.f) {
   const int64_t row = q_tok;
   const bool sf = a.t.state_f32 != 0;
   const float m_nat = m * 0.6931471805599453f;
@@ -497,6 +544,9 @@ __global__ __launch_bounds__(256, 2) void tile_kernel(TileArgs a) {
     store_state<T>(a.t.m, row, m_out, sf);
     store_state<T>(a.t.l, row, l_out, sf);
   }
+  }  // row written
+  if (!persist) break;
+  }  // query tiles
 }
 
 // rows of a block mask that have no live column: out := NaN (m, l untouched)
@@ -605,13 +655,21 @@ template <typename T, int D>
 int launch_global_tiles(const TileArgs& a, hipStream_t stream) {
   const KernelEvents ev = kernel_events();
   const bool timed = ev.start != nullptr && ev.stop != nullptr;
-  const int64_t grid_cols = (a.n + 127) / 128;
+  int64_t grid_cols = (a.n + 127) / 128;
+  TileArgs ac = a;
+  ac.persist = (a.n_globs <= TileCfg<T, D>::BN) ? 1 : 0;
+  if (ac.persist) {
+    const int64_t resident = (int64_t)device_cu_count() * 2;  // two workgroups fit a CU
+    if (grid_cols > resident) grid_cols = resident;
+  }
   hipLaunchKernelGGL((tile_kernel<T, D, kTileGlobalCols>), dim3((unsigned)grid_cols), dim3(256), 0,
-                     stream, a);
+                     stream, ac);
   const int64_t q_tiles = (a.n_globs + 127) / 128;
+  TileArgs ar = a;
+  ar.pair_split = (a.n_globs <= 64 && TileCfg<T, D>::NB == 2) ? 1 : 0;
   if (timed) (void)hipEventRecord(ev.start, stream);
   hipLaunchKernelGGL((tile_kernel<T, D, kTileGlobalRows>), dim3((unsigned)(q_tiles * a.n_split)),
-                     dim3(256), 0, stream, a);
+                     dim3(256), 0, stream, ar);
   if (timed) (void)hipEventRecord(ev.stop, stream);
   hipLaunchKernelGGL((global_rows_merge_kernel<T, D>), dim3((unsigned)a.n_globs), dim3(256), 0, stream,
                      a);
