@@ -189,14 +189,12 @@ __device__ __forceinline__ void attend(const Mask& mask, const typename Mask::Ro
 // Fold the state already in memory into (m, l, acc) and write the row back.  A row that saw
 // no live column (l == 0) is left untouched.
 template <class Lay>
-__device__ __forceinline__ void finish_row(const Tensors& t, int64_t row, int c, float m, float l,
-                                           float (&acc)[Lay::NE]) {
+__device__ __forceinline__ void finish_row_with(const Tensors& t, int64_t row, int c, float m, float l,
+                                                float (&acc)[Lay::NE], float m_in, float l_in) {
   using T = typename Lay::elem;
   constexpr int NE = Lay::NE;
   if (!(l > 0.f)) return;
   const bool sf = t.state_f32 != 0;
-  float m_in = load_state<T>(t.m, row, sf);
-  float l_in = load_state<T>(t.l, row, sf);
   T* orow = (T*)t.out + row * t.d;
   float m_new = m, l_new = l;
   if (l_in != 0.f) {
@@ -220,6 +218,17 @@ __device__ __forceinline__ void finish_row(const Tensors& t, int64_t row, int c,
     store_state<T>(t.m, row, m_new, sf);
     store_state<T>(t.l, row, l_new, sf);
   }
+}
+
+template <class Lay>
+__device__ __forceinline__ void finish_row(const Tensors& t, int64_t row, int c, float m, float l,
+                                           float (&acc)[Lay::NE]) {
+  using T = typename Lay::elem;
+  if (!(l > 0.f)) return;
+  const bool sf = t.state_f32 != 0;
+  const float m_in = load_state<T>(t.m, row, sf);
+  const float l_in = load_state<T>(t.l, row, sf);
+  finish_row_with<Lay>(t, row, c, m, l, acc, m_in, l_in);
 }
 
 template <class Lay>

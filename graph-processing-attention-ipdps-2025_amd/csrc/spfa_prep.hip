@@ -206,49 +206,103 @@ __global__ __launch_bounds__(kPartThreads) void coo_part_count_kernel(
   for (int b = threadIdx.x; b < n_hi; b += kPartThreads) hist[(int64_t)b * n_tiles + blockIdx.x] = cnt[b];
 }
 
-// pass 1b: hist now holds exclusive prefixes; scatter (row, col) into high-digit order
+// pass 1b: hist now holds exclusive prefixes.  The tile is first sorted by high digit inside LDS,
+// then written out, so that the entries a tile sends to one bucket leave as one contiguous run
+// of (row, col) pairs instead of as isolated 4-byte stores.
+constexpr int kPartPerThread = kPartTile / kPartThreads;
+constexpr size_t kPartScatterLds = (size_t)kPartTile * 8 + 3 * (size_t)kPartMaxBuckets * 4;
+
 __global__ __launch_bounds__(kPartThreads) void coo_part_scatter_kernel(
     const void* row_ind, int wide, const uint32_t* col_ind, int64_t nnz, int64_t n_rows, int lo_bits,
-    int n_hi, int64_t n_tiles, const uint32_t* flag, const uint32_t* hist, uint32_t* tmp_rows,
-    uint32_t* tmp_cols) {
-  __shared__ uint32_t cur[kPartMaxBuckets];
+    int n_hi, int64_t n_tiles, const uint32_t* flag, const uint32_t* hist, uint64_t* tmp_pairs) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char part_lds[];
+  uint64_t* stage = reinterpret_cast<uint64_t*>(part_lds);
+  uint32_t* cnt = reinterpret_cast<uint32_t*>(part_lds + (size_t)kPartTile * 8);
+  uint32_t* lstart = cnt + kPartMaxBuckets;
+  uint32_t* gstart = lstart + kPartMaxBuckets;
+  __shared__ uint32_t wave_sums[kPartThreads / kWave];
   if (!*flag) return;
-  for (int b = threadIdx.x; b < n_hi; b += kPartThreads) cur[b] = hist[(int64_t)b * n_tiles + blockIdx.x];
+  const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+  for (int b = tid; b < n_hi; b += kPartThreads) {
+    cnt[b] = 0;
+    gstart[b] = hist[(int64_t)b * n_tiles + blockIdx.x];
+  }
   __syncthreads();
   const int64_t beg = (int64_t)blockIdx.x * kPartTile;
   const int64_t end = beg + kPartTile < nnz ? beg + kPartTile : nnz;
-  for (int64_t e = beg + threadIdx.x; e < end; e += kPartThreads) {
-    const int64_t r = load_index(row_ind, e, wide);
-    if (r >= 0 && r < n_rows) {
-      const uint32_t pos = atomicAdd(&cur[r >> lo_bits], 1u);
-      tmp_rows[pos] = (uint32_t)r;
-      tmp_cols[pos] = col_ind[e];
+  uint32_t rows[kPartPerThread], cols[kPartPerThread], rank[kPartPerThread];
+#pragma unroll
+  for (int i = 0; i < kPartPerThread; i++) {
+    const int64_t e = beg + (int64_t)i * kPartThreads + tid;
+    rows[i] = 0xffffffffu;  // dropped
+    if (e < end) {
+      const int64_t r = load_index(row_ind, e, wide);
+      if (r >= 0 && r < n_rows) {
+        rows[i] = (uint32_t)r;
+        cols[i] = col_ind[e];
+        rank[i] = atomicAdd(&cnt[r >> lo_bits], 1u);
+      }
     }
+  }
+  __syncthreads();
+  // exclusive scan of cnt -> lstart
+  uint32_t carry = 0;
+  for (int base = 0; base < n_hi; base += kPartThreads) {
+    const int i = base + tid;
+    const uint32_t x = i < n_hi ? cnt[i] : 0u;
+    const uint32_t inc = wave_inclusive_scan(x, lane);
+    if (lane == kWave - 1) wave_sums[wave] = inc;
+    __syncthreads();
+    uint32_t prefix = 0, total = 0;
+#pragma unroll
+    for (int w = 0; w < kPartThreads / kWave; w++) {
+      const uint32_t sw = wave_sums[w];
+      if (w < wave) prefix += sw;
+      total += sw;
+    }
+    if (i < n_hi) lstart[i] = carry + prefix + inc - x;
+    carry += total;
+    __syncthreads();
+  }
+  const uint32_t kept = carry;
+#pragma unroll
+  for (int i = 0; i < kPartPerThread; i++) {
+    if (rows[i] != 0xffffffffu)
+      stage[lstart[rows[i] >> lo_bits] + rank[i]] = ((uint64_t)rows[i] << 32) | cols[i];
+  }
+  __syncthreads();
+  for (uint32_t i = tid; i < kept; i += kPartThreads) {
+    const uint64_t x = stage[i];
+    const uint32_t b = (uint32_t)(x >> 32) >> lo_bits;
+    tmp_pairs[gstart[b] + (i - lstart[b])] = x;
   }
 }
 
-// pass 2: one workgroup per high bucket; its entries are contiguous in tmp_*.  Count the low
-// digit in LDS, scan, emit the row offsets of the bucket's rows and place the columns.
-__global__ __launch_bounds__(kPartThreads) void coo_part_rows_kernel(
+// pass 2: one workgroup per high bucket; its (row, col) pairs are contiguous in tmp_pairs.
+// Count the low digit in LDS, scan, emit the row offsets of the bucket's rows and place the
+// columns.
+constexpr int kPartRowsThreads = 1024;
+
+__global__ __launch_bounds__(kPartRowsThreads) void coo_part_rows_kernel(
     int64_t n_rows, int lo_bits, int n_hi, int64_t n_tiles, int64_t n_hist, const uint32_t* flag,
-    const uint32_t* hist, const uint32_t* tmp_rows, const uint32_t* tmp_cols, uint32_t* row_off,
-    uint32_t* cols_out) {
+    const uint32_t* hist, const uint64_t* tmp_pairs, uint32_t* row_off, uint32_t* cols_out) {
   __shared__ uint32_t cnt[kPartMaxBuckets];
-  __shared__ uint32_t wave_sums[kPartThreads / kWave];
+  __shared__ uint32_t wave_sums[kPartRowsThreads / kWave];
   if (!*flag) return;
   const int b = blockIdx.x;
   const int n_lo = 1 << lo_bits;
   const uint32_t beg = hist[(int64_t)b * n_tiles];
   const uint32_t end = (b + 1 < n_hi) ? hist[(int64_t)(b + 1) * n_tiles] : hist[n_hist];
-  for (int i = threadIdx.x; i < n_lo; i += kPartThreads) cnt[i] = 0;
+  for (int i = threadIdx.x; i < n_lo; i += kPartRowsThreads) cnt[i] = 0;
   __syncthreads();
   const uint32_t lo_mask = (uint32_t)n_lo - 1u;
-  for (uint32_t e = beg + threadIdx.x; e < end; e += kPartThreads) atomicAdd(&cnt[tmp_rows[e] & lo_mask], 1u);
+  for (uint32_t e = beg + threadIdx.x; e < end; e += kPartRowsThreads)
+    atomicAdd(&cnt[(uint32_t)(tmp_pairs[e] >> 32) & lo_mask], 1u);
   __syncthreads();
-  // exclusive scan of cnt[0 .. n_lo) in place, kPartThreads values at a time
+  // exclusive scan of cnt[0 .. n_lo) in place, kPartRowsThreads values at a time
   const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
   uint32_t carry = beg;
-  for (int base = 0; base < n_lo; base += kPartThreads) {
+  for (int base = 0; base < n_lo; base += kPartRowsThreads) {
     const int i = base + threadIdx.x;
     const uint32_t x = i < n_lo ? cnt[i] : 0u;
     const uint32_t inc = wave_inclusive_scan(x, lane);
@@ -256,7 +310,7 @@ __global__ __launch_bounds__(kPartThreads) void coo_part_rows_kernel(
     __syncthreads();
     uint32_t prefix = 0, total = 0;
 #pragma unroll
-    for (int w = 0; w < kPartThreads / kWave; w++) {
+    for (int w = 0; w < kPartRowsThreads / kWave; w++) {
       const uint32_t sw = wave_sums[w];
       if (w < wave) prefix += sw;
       total += sw;
@@ -271,9 +325,10 @@ __global__ __launch_bounds__(kPartThreads) void coo_part_rows_kernel(
     __syncthreads();
   }
   if (b == n_hi - 1 && threadIdx.x == 0) row_off[n_rows] = end;
-  for (uint32_t e = beg + threadIdx.x; e < end; e += kPartThreads) {
-    const uint32_t pos = atomicAdd(&cnt[tmp_rows[e] & lo_mask], 1u);
-    cols_out[pos] = tmp_cols[e];
+  for (uint32_t e = beg + threadIdx.x; e < end; e += kPartRowsThreads) {
+    const uint64_t x = tmp_pairs[e];
+    const uint32_t pos = atomicAdd(&cnt[(uint32_t)(x >> 32) & lo_mask], 1u);
+    cols_out[pos] = (uint32_t)x;
   }
 }
 
@@ -306,8 +361,7 @@ CooWorkspace coo_workspace(int64_t n_rows, int64_t nnz) {
   w.off_cols = off;    off = align_up(off + (size_t)(nnz > 0 ? nnz : 1) * 4, 256);
   w.off_flag = off;    off = align_up(off + 4, 256);
   w.off_hist = off;    off = align_up(off + (size_t)(n_hist + 1) * 4, 256);
-  w.off_tmp_rows = off; off = align_up(off + (size_t)(w.partition ? nnz : 0) * 4, 256);
-  w.off_tmp_cols = off; off = align_up(off + (size_t)(w.partition ? nnz : 0) * 4, 256);
+  w.off_tmp_pairs = off; off = align_up(off + (size_t)(w.partition ? nnz : 0) * 8, 256);
   w.total = off;
   return w;
 }
@@ -336,8 +390,16 @@ int coo_to_csr(const void* row_ind, int row_wide, const uint32_t* col_ind, int64
   // unsorted: bucket by row
   if (nnz > 0 && w.partition) {
     uint32_t* hist = (uint32_t*)(base + w.off_hist);
-    uint32_t* tmp_rows = (uint32_t*)(base + w.off_tmp_rows);
-    uint32_t* tmp_cols = (uint32_t*)(base + w.off_tmp_cols);
+    uint64_t* tmp_pairs = (uint64_t*)(base + w.off_tmp_pairs);
+    static bool lds_attr_set = false;
+    if (!lds_attr_set) {
+      // 88 KB of LDS per workgroup: above the 64 KB a kernel gets without asking
+      if (hipFuncSetAttribute(reinterpret_cast<const void*>(coo_part_scatter_kernel),
+                              hipFuncAttributeMaxDynamicSharedMemorySize,
+                              (int)kPartScatterLds) != hipSuccess)
+        return 4;
+      lds_attr_set = true;
+    }
     const int64_t n_hist = w.n_hi * w.n_tiles1;
     const int64_t hist_tiles = (n_hist + kScanTile - 1) / kScanTile;
     hipLaunchKernelGGL(coo_part_count_kernel, dim3((unsigned)w.n_tiles1), dim3(kPartThreads), 0, stream,
@@ -347,12 +409,12 @@ int coo_to_csr(const void* row_ind, int row_wide, const uint32_t* col_ind, int64
     hipLaunchKernelGGL(scan_sums_kernel, dim3(1), dim3(kScanThreads), 0, stream, tiles, hist_tiles, flag);
     hipLaunchKernelGGL(scan_apply_kernel, dim3((unsigned)hist_tiles), dim3(kScanThreads), 0, stream,
                        hist, n_hist, tiles, hist, hist, flag);
-    hipLaunchKernelGGL(coo_part_scatter_kernel, dim3((unsigned)w.n_tiles1), dim3(kPartThreads), 0,
-                       stream, row_ind, row_wide, col_ind, nnz, n_rows, w.lo_bits, (int)w.n_hi,
-                       w.n_tiles1, flag, hist, tmp_rows, tmp_cols);
-    hipLaunchKernelGGL(coo_part_rows_kernel, dim3((unsigned)w.n_hi), dim3(kPartThreads), 0, stream,
-                       n_rows, w.lo_bits, (int)w.n_hi, w.n_tiles1, n_hist, flag, hist, tmp_rows, tmp_cols,
-                       row_off, cols);
+    hipLaunchKernelGGL(coo_part_scatter_kernel, dim3((unsigned)w.n_tiles1), dim3(kPartThreads),
+                       kPartScatterLds, stream, row_ind, row_wide, col_ind, nnz, n_rows, w.lo_bits,
+                       (int)w.n_hi, w.n_tiles1, flag, hist, tmp_pairs);
+    hipLaunchKernelGGL(coo_part_rows_kernel, dim3((unsigned)w.n_hi), dim3(kPartRowsThreads), 0, stream,
+                       n_rows, w.lo_bits, (int)w.n_hi, w.n_tiles1, n_hist, flag, hist, tmp_pairs, row_off,
+                       cols);
   } else if (nnz > 0) {
     hipLaunchKernelGGL(coo_histogram_kernel, dim3(grid_for(nnz, 256, 16384)), dim3(256), 0, stream,
                        row_ind, row_wide, nnz, n_rows, flag, counts);

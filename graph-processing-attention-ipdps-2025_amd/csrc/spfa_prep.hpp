@@ -12,7 +12,7 @@ inline size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 struct CooWorkspace {
   size_t off_counts, off_row_off, off_cursor, off_tiles, off_cols, off_flag;
   // two-pass partition (used when the row index fits 22 bits)
-  size_t off_hist, off_tmp_rows, off_tmp_cols, total;
+  size_t off_hist, off_tmp_pairs, total;
   int partition;       // 1: two-pass LDS partition, 0: per-entry global atomics
   int lo_bits;         // low digit width; high digit = row >> lo_bits
   int64_t n_hi;        // high-digit buckets
