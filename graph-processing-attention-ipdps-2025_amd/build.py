@@ -117,7 +117,7 @@ def _source_loop_depth(kname: str) -> int:
     seg = "15segments_kernelI" in kname
     m = re.search(r"6VecLayI\w+?Li(\d+)E", kname)
     if m:
-        lpr, unroll = int(m.group(1)), (8 if seg else 4)
+        lpr, unroll = int(m.group(1)), (16 if seg else 4)
     else:
         m = re.search(r"6GenLayI\w+?Li(\d+)E", kname)
         lpr, unroll = 64, (8 if int(m.group(1)) <= 2 else 2)

@@ -12,7 +12,6 @@ namespace {
 
 constexpr int64_t kInlineAll = std::numeric_limits<int64_t>::max();
 
-inline int64_t clamp64(int64_t x, int64_t lo, int64_t hi) { return x < lo ? lo : (x > hi ? hi : x); }
 
 inline size_t dtype_size(int dtype) { return dtype == SPFA_DTYPE_F32 ? 4 : 2; }
 
@@ -22,8 +21,13 @@ inline bool dtype_ok(int dtype) {
 
 // segment length: enough segments to keep every wavefront slot busy several times over, long
 // enough that the per-segment overhead (q load, group merge, partial write) stays small
+// Segment length for long rows: long enough to amortise the pipeline fill and the partial
+// result of a segment (1024 candidates: 64 per lane group at d*s = 256 bytes), short enough
+// that the work list holds several items per persistent wavefront (about 1024 of them).
 inline int64_t pick_segment(int64_t nnz_long) {
-  return clamp64(pow2_ceil(nnz_long / 65536 + 1), 256, 8192);
+  int64_t seg = 128;
+  while (seg < 1024 && seg * 2 * 8192 <= nnz_long) seg *= 2;
+  return seg;
 }
 
 constexpr int64_t kExplicitInlineRowLimit = 32;

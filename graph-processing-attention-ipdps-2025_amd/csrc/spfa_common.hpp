@@ -86,10 +86,7 @@ struct VecLay {
   static constexpr int GROUPS = kWave / LPR;
   static constexpr int NE = 16 / (int)sizeof(T);  // floats held per lane
   static constexpr int D = LPR * NE;
-#ifndef SPFA_TUNE_U
-#define SPFA_TUNE_U 8
-#endif
-  static constexpr int U = SPFA_TUNE_U;  // neighbours in flight per group in the segment kernel
+  static constexpr int U = 16;       // neighbours in flight per group in the segment kernel
   static constexpr int U_SHORT = 4;  // ... in the row kernel
   static constexpr bool kFixedD = true;
   using raw = uint4v;
@@ -99,12 +96,7 @@ struct VecLay {
   }
   // gathered K / V rows
   __device__ static __forceinline__ raw load_gather(const T* row_ptr, int c, int) {
-#if defined(SPFA_TUNE_NT)
-    return __builtin_nontemporal_load(
-        reinterpret_cast<const raw*>(reinterpret_cast<const char*>(row_ptr) + c * 16));
-#else
     return *reinterpret_cast<const raw*>(reinterpret_cast<const char*>(row_ptr) + c * 16);
-#endif
   }
   __device__ static __forceinline__ void unpack(const raw& r, float (&f)[NE]) {
     if constexpr (sizeof(T) == 4) {
