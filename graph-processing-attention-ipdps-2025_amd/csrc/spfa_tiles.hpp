@@ -104,6 +104,70 @@ __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
   return __builtin_bit_cast(uint32_t, x);
 }
 
+template <bool B>
+struct BoolConst {
+  static constexpr bool value = B;
+};
+
+// Fold the incoming state of row `row` into a finished tile result and write the row back.
+// o holds O^T in the 32x32 result layout (element e = 32*eb + 8*(v/4) + 4*h + v%4 of the row in
+// o[eb][v]); m is the running max in log2 units, l the row sum (already summed over both halves
+// of the wavefront); o * o_scale is the accumulator that goes with (m, l).
+template <typename T, int D>
+__device__ __forceinline__ void tile_write_row(const Tensors& t, int64_t row, int h, float m, float l,
+                                               const f32x16 (&o)[D / 32], float o_scale = 1.f) {
+  constexpr bool kF32 = sizeof(T) == 4;
+  const bool sf = t.state_f32 != 0;
+  const float m_nat = m * 0.6931471805599453f;
+  float m_out = m_nat, l_out = l;
+  float wa = 0.f, wb = 1.f;
+  const float l_in = load_state<T>(t.l, row, sf);
+  if (l_in != 0.f) {
+    const float m_in = load_state<T>(t.m, row, sf);
+    m_out = fmaxf(m_nat, m_in);
+    wa = l_in * __expf(m_in - m_out);
+    wb = __expf(m_nat - m_out);
+    l_out = wa + l * wb;
+  }
+  const float inv = 1.f / l_out;
+  wb *= inv * o_scale;  // o_scale: o was accumulated against a reference below the maximum m
+  wa *= inv;
+  T* orow = (T*)t.out + row * D;
+#pragma unroll
+  for (int eb = 0; eb < D / 32; eb++) {
+#pragma unroll
+    for (int g4 = 0; g4 < 4; g4++) {
+      const int e = 32 * eb + 8 * g4 + 4 * h;
+      float x[4];
+#pragma unroll
+      for (int i = 0; i < 4; i++) x[i] = o[eb][4 * g4 + i] * wb;
+      if constexpr (kF32) {
+        if (wa != 0.f) {
+          float4v oi = *reinterpret_cast<const float4v*>(orow + e);
+#pragma unroll
+          for (int i = 0; i < 4; i++) x[i] += wa * oi[i];
+        }
+        float4v y = {x[0], x[1], x[2], x[3]};
+        *reinterpret_cast<float4v*>(orow + e) = y;
+      } else {
+        typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+        if (wa != 0.f) {
+          typedef T t4 __attribute__((ext_vector_type(4)));
+          t4 oi = *reinterpret_cast<const t4*>(orow + e);
+#pragma unroll
+          for (int i = 0; i < 4; i++) x[i] += wa * (float)oi[i];
+        }
+        u32x2 y = {pack2<T>(x[0], x[1]), pack2<T>(x[2], x[3])};
+        *reinterpret_cast<u32x2*>(orow + e) = y;
+      }
+    }
+  }
+  if (h == 0) {
+    store_state<T>(t.m, row, m_out, sf);
+    store_state<T>(t.l, row, l_out, sf);
+  }
+}
+
 template <typename T, int D, int MODE>
 __global__ __launch_bounds__(256, 2) void tile_kernel(TileArgs a) {
   using C = TileCfg<T, D>;
@@ -493,60 +557,283 @@ __global__ __launch_bounds__(256, 2) void tile_kernel(TileArgs a) {
     }
     return;
   }
-  if (q_ok && l > 0.f) {
-  const int64_t row = q_tok;
-  const bool sf = a.t.state_f32 != 0;
-  const float m_nat = m * 0.6931471805599453f;
-  float m_out = m_nat, l_out = l;
-  float wa = 0.f, wb = 1.f;
-  const float l_in = load_state<T>(a.t.l, row, sf);
-  if (l_in != 0.f) {
-    const float m_in = load_state<T>(a.t.m, row, sf);
-    m_out = fmaxf(m_nat, m_in);
-    wa = l_in * __expf(m_in - m_out);
-    wb = __expf(m_nat - m_out);
-    l_out = wa + l * wb;
-  }
-  const float inv = 1.f / l_out;
-  wb *= inv;
-  wa *= inv;
-  T* orow = (T*)a.t.out + row * D;
-#pragma unroll
-  for (int eb = 0; eb < EB; eb++) {
-#pragma unroll
-    for (int g4 = 0; g4 < 4; g4++) {
-      const int e = 32 * eb + 8 * g4 + 4 * h;
-      float x[4];
-#pragma unroll
-      for (int i = 0; i < 4; i++) x[i] = o[eb][4 * g4 + i] * wb;
-      if constexpr (kF32) {
-        if (wa != 0.f) {
-          float4v oi = *reinterpret_cast<const float4v*>(orow + e);
-#pragma unroll
-          for (int i = 0; i < 4; i++) x[i] += wa * oi[i];
-        }
-        float4v y = {x[0], x[1], x[2], x[3]};
-        *reinterpret_cast<float4v*>(orow + e) = y;
-      } else {
-        typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
-        if (wa != 0.f) {
-          typedef T t4 __attribute__((ext_vector_type(4)));
-          t4 oi = *reinterpret_cast<const t4*>(orow + e);
-#pragma unroll
-          for (int i = 0; i < 4; i++) x[i] += wa * (float)oi[i];
-        }
-        u32x2 y = {pack2<T>(x[0], x[1]), pack2<T>(x[2], x[3])};
-        *reinterpret_cast<u32x2*>(orow + e) = y;
-      }
-    }
-  }
-  if (h == 0) {
-    store_state<T>(a.t.m, row, m_out, sf);
-    store_state<T>(a.t.l, row, l_out, sf);
-  }
-  }  // row written
+  if (q_ok && l > 0.f) tile_write_row<T, D>(a.t, q_tok, h, m, l, o);
   if (!persist) break;
   }  // query tiles
+}
+
+// ---------------------------------------------------------------------------------------
+// Band masks, half types: tiles go from global memory straight into LDS
+// ---------------------------------------------------------------------------------------
+// Same tile problem and register layouts as tile_kernel<T, D, kTileBand>, different plumbing:
+//   - K and V tiles are written to LDS by the load instructions themselves (16 bytes per lane,
+//     64 lanes = 1 KB of consecutive LDS per instruction), row-major and unpadded; no staging
+//     registers, no LDS store instructions.  Two tile buffers, one barrier per tile: tile n+1 is
+//     requested right after the barrier that publishes tile n.
+//   - Rows are 128 or 256 bytes, a multiple of the bank cycle, so bank conflicts are avoided by
+//     permuting the 16-byte chunks inside a row instead of padding: chunk c of row j is stored at
+//     chunk position c ^ f(j).  K is read with 16-byte operand fetches by 8 consecutive rows at a
+//     time (f = j mod chunks per row).  V is read with the transposing 8-byte load: a group of
+//     16 lanes reads 4 keys x 16 columns (4 lanes per key, 4 columns per lane) and lane i
+//     receives column i of the 4 keys, which is the V^T operand; f = 2 * (bank-cycle index mod 4)
+//     keeps the 4 keys of a group apart.
+//   - The softmax runs per 32-key block; both S products of a tile are issued before the first
+//     softmax step, so the matrix pipe works on the second block while the vector ALU is busy
+//     with the first.
+template <typename T, int D>
+struct BandDmaCfg {
+  static constexpr int BM = 128, BN = 64;
+  static constexpr int ROWB = D * 2;            // bytes per K / V row
+  static constexpr int CH = D / 8;              // 16-byte chunks per row
+  static constexpr int RPC = 256 / ROWB;        // rows per 256-byte bank cycle
+  static constexpr int TILE_B = BN * ROWB;      // bytes of one K (or V) tile
+  static constexpr int BUF_B = 2 * TILE_B;      // K tile then V tile
+  static constexpr int NI = TILE_B / 4096;      // load instructions per wavefront, tile and matrix
+  static constexpr int EB = D / 32, QREGS = D / 16;
+};
+
+template <typename T, int D>
+__global__ __launch_bounds__(256, 2) void band_dma_kernel(TileArgs a) {
+  using C = BandDmaCfg<T, D>;
+  constexpr int BM = C::BM, BN = C::BN, EB = C::EB, ROWB = C::ROWB, CH = C::CH, RPC = C::RPC;
+  constexpr int TILE_B = C::TILE_B, BUF_B = C::BUF_B, NI = C::NI;
+  static_assert(sizeof(T) == 2 && (D == 64 || D == 128), "half types, d = 64 or 128");
+  // two tile buffers as two separate arrays: the compiler can then tell the loads that fill one
+  // buffer from the operand reads of the other and does not wait for the former before the latter
+  __shared__ __attribute__((aligned(1024))) char lds_even[BUF_B];
+  __shared__ __attribute__((aligned(1024))) char lds_odd[BUF_B];
+
+  // workgroups are dealt round-robin to the 8 XCDs: give each XCD a contiguous run of tiles.
+  // Positions inside a subsequence fit 32 bits (there are fewer than 2^31 tokens); everything
+  // that is the same for the whole workgroup is moved to scalar registers.
+  auto uni = [](int x) { return __builtin_amdgcn_readfirstlane(x); };
+  const int64_t per_xcd = (a.n_tiles + 7) / 8;
+  const int64_t lt = (int64_t)(blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+  if (lt >= a.n_tiles) return;
+  const int64_t sub = lt / a.tiles_per_sub;
+  const int tile = uni((int)(lt - sub * a.tiles_per_sub));
+  int64_t base;
+  int qlen;
+  if (a.block > 0) {
+    base = sub * a.block;
+    qlen = (int)a.cnt;
+  } else {
+    base = sub;
+    qlen = uni((int)((a.n - sub + a.s - 1) / a.s));
+  }
+  const int wlim = (int)(a.w < (int64_t)0x3fffffff ? a.w : (int64_t)0x3fffffff);  // window, clamped
+  const int t0 = tile * BM;
+  if (t0 >= qlen) return;
+  const int u_lo = t0 > wlim ? t0 - wlim : 0;
+  const int u_hi = (qlen - BM - wlim > t0) ? t0 + BM + wlim : qlen;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int r = lane & 31, h = lane >> 5;
+  const char* Kp = (const char*)a.t.k;
+  const char* Vp = (const char*)a.t.v;
+  const float sc = 1.4426950408889634f / sqrtf((float)D);
+
+  const int tw0 = t0 + 32 * wave;  // first query of this wavefront
+  const int tq = tw0 + r;          // this lane's query position
+  const bool q_ok = tq < qlen;
+  const int64_t q_tok = base + (int64_t)(q_ok ? tq : qlen - 1) * a.s;
+
+  // ---- Q^T operand, kept in registers
+  uint4v qh[C::QREGS];
+  {
+    const T* qrow = (const T*)a.t.q + q_tok * D;
+#pragma unroll
+    for (int ks = 0; ks < C::QREGS; ks++)
+      qh[ks] = *reinterpret_cast<const uint4v*>(qrow + 16 * ks + 8 * h);
+  }
+
+  // ---- tile loads: instruction `it` of this wavefront fills the 1-KB segment 4*it + wave of a
+  // tile; this lane's 16 bytes are row j, chunk position p of it
+  uint32_t koff[NI], voff[NI];  // byte offset of the lane's source chunk from the tile's first row
+  const uint32_t row_step = (uint32_t)a.s * (uint32_t)ROWB;  // bytes between consecutive keys
+#pragma unroll
+  for (int it = 0; it < NI; it++) {
+    const int at = (4 * it + wave) * 1024 + lane * 16;
+    const int j = at / ROWB, p = (at % ROWB) / 16;
+    koff[it] = (uint32_t)j * row_step + (uint32_t)((p ^ (j % CH)) * 16);
+    voff[it] = (uint32_t)j * row_step + (uint32_t)((p ^ (2 * ((j / RPC) % 4))) * 16);
+  }
+  auto request = [&](int ut, char* dst_buf) {
+    const int64_t tile_byte = (base + (int64_t)ut * a.s) * (int64_t)ROWB;  // scalar
+    const bool whole = ut + BN <= u_hi;
+#pragma unroll
+    for (int it = 0; it < NI; it++) {
+      uint32_t ko = koff[it], vo = voff[it];
+      if (!whole) {
+        // rows past the last key repeat the last key (finite values; they are masked out)
+        const int last = u_hi - 1 - ut;
+        const int j = ((4 * it + wave) * 1024 + lane * 16) / ROWB;
+        if (j > last) {
+          const uint32_t back = (uint32_t)(j - last) * row_step;
+          ko -= back;
+          vo -= back;
+        }
+      }
+      char* dst = dst_buf + (4 * it + wave) * 1024;
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(Kp + tile_byte + ko),
+                                       (__attribute__((address_space(3))) void*)dst, 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(Vp + tile_byte + vo),
+                                       (__attribute__((address_space(3))) void*)(dst + TILE_B), 16, 0, 0);
+    }
+  };
+
+  // ---- operand addresses inside a tile buffer (bytes)
+  // K block jb, step ks: row 32*jb + r, chunk 2*ks + h
+  int kadr[C::QREGS];
+#pragma unroll
+  for (int ks = 0; ks < C::QREGS; ks++) kadr[ks] = r * ROWB + (((2 * ks + h) ^ (r % CH)) * 16);
+  // V: group of 16 lanes = (column half r_hi, key half h); lane 4*x + y of the group points at
+  // key 4*h + x (+ 8 for the second half of an operand), columns 16*r_hi + 4*y .. +3
+  int vadr[2];
+  {
+    const int x = (lane & 15) >> 2, y = lane & 3, r_hi = (lane >> 4) & 1;
+    const int key = 4 * h + x;
+    const int g = 2 * ((key / RPC) % 4);                 // chunk permutation of that row
+    const int c_lo = (2 * r_hi + (y >> 1)) ^ (g & 3);     // chunk inside a group of 4 (one eb)
+    const int gb = (g >> 2) & 1;                         // eb pairs swap when bit 2 of g is set
+    const int common = TILE_B + key * ROWB + c_lo * 16 + (y & 1) * 8;
+    vadr[0] = common + 64 * (0 ^ gb);
+    vadr[1] = common + 64 * (1 ^ gb);
+  }
+
+  f32x16 o[EB];
+#pragma unroll
+  for (int eb = 0; eb < EB; eb++)
+#pragma unroll
+    for (int v = 0; v < 16; v++) o[eb][v] = 0.f;
+  constexpr float kSlack = 8.f;
+  float m = kNegInf;   // reference maximum of the exponentials, log2 units
+  float mt = kNegInf;  // true running maximum
+  float l = 0.f;       // running sum (relative to m) over this lane's half of the keys
+
+  // one tile: wait for it, publish it, request the next one into the other buffer, consume it
+  auto step = [&](int ut, const char* tb, char* other) __attribute__((always_inline)) {
+    __builtin_amdgcn_s_waitcnt(0);  // this wavefront's part of the tile has landed
+    __syncthreads();                // everyone's has, and everyone is done with the other buffer
+    if (ut + BN < u_hi) request(ut + BN, other);
+
+    // Both 32-key blocks of the tile are always computed (a block outside this wavefront's
+    // band is masked out completely; the band is much wider than a block), which keeps the
+    // tile body one straight line of code.  all_full: every (query, key) pair of the tile is
+    // live for this wavefront, no per-element test needed.
+    // (positions and the clamped window are below 2^30, so the sums stay inside 32 bits)
+    const bool all_full = (ut + BN <= u_hi) && (ut >= tw0 + 31 - wlim) && (ut + BN - 1 - wlim <= tw0);
+    const bool none = (tw0 >= qlen) || (ut - wlim > tw0 + 31) || (ut + BN - 1 < tw0 - wlim);
+    if (none) return;
+
+    auto qk = [&](int jb) -> f32x16 {
+      const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+      const char* kb = tb + 32 * jb * ROWB;
+      f32x16 acc = mfma16<T>(*reinterpret_cast<const uint4v*>(kb + kadr[0]), qh[0], zero16);
+#pragma unroll
+      for (int ks = 1; ks < C::QREGS; ks++)
+        acc = mfma16<T>(*reinterpret_cast<const uint4v*>(kb + kadr[ks]), qh[ks], acc);
+      return acc;
+    };
+
+    // key slot j of the tile is live for this lane's query iff jlo <= j <= jhi; the slots this
+    // lane holds are c + 4*h for compile-time c, so the bounds are shifted by 4*h once
+    const int live_slots = (u_hi - ut) < BN ? (u_hi - ut) : BN;
+    const int jlo = (tq - wlim - ut) - 4 * h;
+    const int jhi_band = tq + wlim - ut;
+    const int jhi = (jhi_band < live_slots - 1 ? jhi_band : live_slots - 1) - 4 * h;
+    const uint32_t span = (uint32_t)(jhi - jlo);  // jhi < jlo: wraps to a huge value, handled below
+    const bool any_live = jhi >= jlo;
+
+    // One online-softmax step over a 32-key block; leaves the exponentials in s.  The
+    // exponentials are taken against a reference maximum m that is only moved (and the
+    // accumulators rescaled) when a row's maximum has grown by more than kSlack (log2 units)
+    // since the reference was set: the weights then stay below 2^kSlack, the final division by
+    // l cancels the reference, and the rescale is rare instead of happening on every block
+    // while the maxima are still settling.  mt keeps the true maximum for the row statistics.
+    auto soft = [&](f32x16& s, int jb) {
+      if (!all_full) {
+#pragma unroll
+        for (int v = 0; v < 16; v++) {
+          const int c = 32 * jb + 8 * (v / 4) + (v % 4);
+          const bool ok = any_live && ((uint32_t)(c - jlo) <= span);
+          s[v] = ok ? s[v] : kNegInf;
+        }
+      }
+      float mx = s[0];
+#pragma unroll
+      for (int v = 1; v < 16; v++) mx = fmaxf(mx, s[v]);
+      mx = fmaxf(mx, shfl_xor_f32(mx, 32)) * sc;
+      mt = fmaxf(mt, mx);
+      if (__builtin_expect(__builtin_amdgcn_ballot_w64(mx > m + kSlack) != 0, 0)) {
+        // (m = -inf: first live block of a row, nothing accumulated yet)
+        const float m_new = (mx > m + kSlack) ? mx : m;
+        const float alpha = (m > kNegInf) ? __builtin_amdgcn_exp2f(m - m_new) : 0.f;
+        m = m_new;
+        l *= alpha;
+#pragma unroll
+        for (int eb = 0; eb < EB; eb++)
+#pragma unroll
+          for (int v = 0; v < 16; v++) o[eb][v] *= alpha;
+      }
+      const float neg_m = (m > kNegInf) ? -m : 0.f;
+      float lsum = 0.f;
+#pragma unroll
+      for (int v = 0; v < 16; v++) {
+        const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(s[v], sc, neg_m));  // exp2(-inf) = 0
+        s[v] = p;
+        lsum += p;
+      }
+      l += lsum;
+    };
+
+    // O^T += V_block^T P_block^T
+    auto pv = [&](const f32x16& s, int jb) {
+      typedef short s16x4 __attribute__((ext_vector_type(4)));
+      typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+#pragma unroll
+      for (int sl = 0; sl < 2; sl++) {
+        uint4v pb;
+#pragma unroll
+        for (int x = 0; x < 4; x++) pb[x] = pack2<T>(s[8 * sl + 2 * x], s[8 * sl + 2 * x + 1]);
+        const char* vb = tb + (32 * jb + 16 * sl) * ROWB;
+#pragma unroll
+        for (int eb = 0; eb < EB; eb++) {
+          const char* va_p = vb + vadr[eb & 1] + 128 * (eb >> 1);
+          const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)va_p);
+          const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(va_p + 8 * ROWB));
+          typedef short s16x8 __attribute__((ext_vector_type(8)));
+          const s16x8 both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+          o[eb] = mfma16<T>(__builtin_bit_cast(uint4v, both), pb, o[eb]);
+        }
+      }
+    };
+
+    // both products are issued before the first softmax step, so the second one runs on the
+    // matrix pipe while the vector ALU works on the first block
+    f32x16 s0 = qk(0);
+    f32x16 s1 = qk(1);
+    soft(s0, 0);
+    pv(s0, 0);
+    soft(s1, 1);
+    pv(s1, 1);
+  };
+
+  if (u_lo < u_hi) request(u_lo, lds_even);
+  for (int ut = u_lo; ut < u_hi; ut += 2 * BN) {
+    step(ut, lds_even, lds_odd);
+    if (ut + BN < u_hi) step(ut + BN, lds_odd, lds_even);
+  }
+
+  l += shfl_xor_f32(l, 32);
+  if (q_ok && l > 0.f) {
+    // hand the row over relative to its true maximum: (m, l, o) -> (mt, l * 2^(m - mt), o)
+    // (o is divided by l later, so only l changes)
+    const float shrink = __builtin_amdgcn_exp2f(m - mt);
+    tile_write_row<T, D>(a.t, q_tok, h, mt, l * shrink, o, shrink);
+  }
 }
 
 // rows of a block mask that have no live column: out := NaN (m, l untouched)
@@ -638,7 +925,18 @@ int launch_band_tiles(const TileArgs& a, int use_nan, hipStream_t stream) {
   if (a.n_tiles > 0) {
     const int64_t grid = (a.n_tiles + 7) / 8 * 8;
     if (timed) (void)hipEventRecord(ev.start, stream);
-    hipLaunchKernelGGL((tile_kernel<T, D, kTileBand>), dim3((unsigned)grid), dim3(256), 0, stream, a);
+    if constexpr (sizeof(T) == 2) {
+      // the direct-to-LDS kernel addresses a tile's rows with 32-bit offsets
+      // and windows / positions with 32-bit arithmetic
+      const int64_t max_len = a.block > 0 ? a.cnt : (a.n + a.s - 1) / a.s;
+      if (a.s * (int64_t)(2 * D) * 64 < ((int64_t)1 << 31) &&
+          (a.w <= (int64_t)0x3fffffff || max_len <= (int64_t)0x3fffffff))
+        hipLaunchKernelGGL((band_dma_kernel<T, D>), dim3((unsigned)grid), dim3(256), 0, stream, a);
+      else
+        hipLaunchKernelGGL((tile_kernel<T, D, kTileBand>), dim3((unsigned)grid), dim3(256), 0, stream, a);
+    } else {
+      hipLaunchKernelGGL((tile_kernel<T, D, kTileBand>), dim3((unsigned)grid), dim3(256), 0, stream, a);
+    }
     if (timed) (void)hipEventRecord(ev.stop, stream);
   }
   if (a.block > 0 && use_nan && a.s > 1) {
