@@ -575,8 +575,8 @@ __global__ __launch_bounds__(256, 2) void tile_kernel(TileArgs a) {
 //     chunk position c ^ f(j).  K is read with 16-byte operand fetches by 8 consecutive rows at a
 //     time (f = j mod chunks per row).  V is read with the transposing 8-byte load: a group of
 //     16 lanes reads 4 keys x 16 columns (4 lanes per key, 4 columns per lane) and lane i
-//     receives column i of the 4 keys, which is the V^T operand; f = 2 * (bank-cycle index mod 4)
-//     keeps the 4 keys of a group apart.
+//     receives column i of the 4 keys, which is the V^T operand; f = 4 * (bank-cycle index mod
+//     chunks/4) keeps the keys read by one instruction apart.
 //   - The softmax runs per 32-key block; both S products of a tile are issued before the first
 //     softmax step, so the matrix pipe works on the second block while the vector ALU is busy
 //     with the first.
@@ -658,7 +658,7 @@ __global__ __launch_bounds__(256, 2) void band_dma_kernel(TileArgs a) {
     const int at = (4 * it + wave) * 1024 + lane * 16;
     const int j = at / ROWB, p = (at % ROWB) / 16;
     koff[it] = (uint32_t)j * row_step + (uint32_t)((p ^ (j % CH)) * 16);
-    voff[it] = (uint32_t)j * row_step + (uint32_t)((p ^ (2 * ((j / RPC) % 4))) * 16);
+    voff[it] = (uint32_t)j * row_step + (uint32_t)((p ^ (4 * ((j / RPC) % (CH / 4)))) * 16);
   }
   auto request = [&](int ut, char* dst_buf) {
     const int64_t tile_byte = (base + (int64_t)ut * a.s) * (int64_t)ROWB;  // scalar
@@ -690,17 +690,17 @@ __global__ __launch_bounds__(256, 2) void band_dma_kernel(TileArgs a) {
 #pragma unroll
   for (int ks = 0; ks < C::QREGS; ks++) kadr[ks] = r * ROWB + (((2 * ks + h) ^ (r % CH)) * 16);
   // V: group of 16 lanes = (column half r_hi, key half h); lane 4*x + y of the group points at
-  // key 4*h + x (+ 8 for the second half of an operand), columns 16*r_hi + 4*y .. +3
-  int vadr[2];
+  // key 4*h + x (+ 8 for the second half of an operand), columns 32*eb + 16*r_hi + 4*y .. +3,
+  // i.e. chunk 4*eb + 2*r_hi + y/2, stored at that chunk ^ g with g = 4 * gx a whole number of
+  // eb steps: the row's eb order is permuted, the chunk inside an eb is not
+  int vadr[EB];
   {
     const int x = (lane & 15) >> 2, y = lane & 3, r_hi = (lane >> 4) & 1;
     const int key = 4 * h + x;
-    const int g = 2 * ((key / RPC) % 4);                 // chunk permutation of that row
-    const int c_lo = (2 * r_hi + (y >> 1)) ^ (g & 3);     // chunk inside a group of 4 (one eb)
-    const int gb = (g >> 2) & 1;                         // eb pairs swap when bit 2 of g is set
-    const int common = TILE_B + key * ROWB + c_lo * 16 + (y & 1) * 8;
-    vadr[0] = common + 64 * (0 ^ gb);
-    vadr[1] = common + 64 * (1 ^ gb);
+    const int gx = (key / RPC) % (CH / 4);
+    const int common = TILE_B + key * ROWB + (2 * r_hi + (y >> 1)) * 16 + (y & 1) * 8;
+#pragma unroll
+    for (int eb = 0; eb < EB; eb++) vadr[eb] = common + 64 * (eb ^ gx);
   }
 
   f32x16 o[EB];
@@ -717,7 +717,11 @@ __global__ __launch_bounds__(256, 2) void band_dma_kernel(TileArgs a) {
   auto step = [&](int ut, const char* tb, char* other) __attribute__((always_inline)) {
     __builtin_amdgcn_s_waitcnt(0);  // this wavefront's part of the tile has landed
     __syncthreads();                // everyone's has, and everyone is done with the other buffer
+#ifdef SPFA_EXP_SAMETILE
+    if (ut + BN < u_hi) request(u_lo, other);
+#else
     if (ut + BN < u_hi) request(ut + BN, other);
+#endif
 
     // Both 32-key blocks of the tile are always computed (a block outside this wavefront's
     // band is masked out completely; the band is much wider than a block), which keeps the
@@ -727,16 +731,6 @@ __global__ __launch_bounds__(256, 2) void band_dma_kernel(TileArgs a) {
     const bool all_full = (ut + BN <= u_hi) && (ut >= tw0 + 31 - wlim) && (ut + BN - 1 - wlim <= tw0);
     const bool none = (tw0 >= qlen) || (ut - wlim > tw0 + 31) || (ut + BN - 1 < tw0 - wlim);
     if (none) return;
-
-    auto qk = [&](int jb) -> f32x16 {
-      const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-      const char* kb = tb + 32 * jb * ROWB;
-      f32x16 acc = mfma16<T>(*reinterpret_cast<const uint4v*>(kb + kadr[0]), qh[0], zero16);
-#pragma unroll
-      for (int ks = 1; ks < C::QREGS; ks++)
-        acc = mfma16<T>(*reinterpret_cast<const uint4v*>(kb + kadr[ks]), qh[ks], acc);
-      return acc;
-    };
 
     // key slot j of the tile is live for this lane's query iff jlo <= j <= jhi; the slots this
     // lane holds are c + 4*h for compile-time c, so the bounds are shifted by 4*h once
@@ -789,36 +783,69 @@ __global__ __launch_bounds__(256, 2) void band_dma_kernel(TileArgs a) {
       l += lsum;
     };
 
+    // Operands are fetched from LDS well ahead of the products that use them, in an order
+    // the scheduler is told to keep: all K operands of block 0, then the K operands of block 1
+    // while the S product of block 0 runs, the V operands of a block before its softmax step.
+    typedef short s16x4 __attribute__((ext_vector_type(4)));
+    typedef short s16x8 __attribute__((ext_vector_type(8)));
+    typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+    constexpr int QR = C::QREGS;
+    const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    uint4v ka[QR], kb[QR];
+#pragma unroll
+    for (int ks = 0; ks < QR; ks++) ka[ks] = *reinterpret_cast<const uint4v*>(tb + kadr[ks]);
+    __builtin_amdgcn_sched_barrier(0);
+    f32x16 s0 = zero16, s1 = zero16;
+#pragma unroll
+    for (int ks = 0; ks < QR; ks++) {
+      kb[ks] = *reinterpret_cast<const uint4v*>(tb + 32 * ROWB + kadr[ks]);
+      s0 = mfma16<T>(ka[ks], qh[ks], s0);
+    }
+    // one LDS read behind every matrix instruction
+#pragma unroll
+    for (int ks = 0; ks < QR; ks++) {
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+
+    // V^T operands of block jb: [sl][eb], two transposing 8-byte reads each
+    auto v_fetch = [&](int jb, uint4v (&va)[2 * EB]) {
+#pragma unroll
+      for (int sl = 0; sl < 2; sl++)
+#pragma unroll
+        for (int eb = 0; eb < EB; eb++) {
+          const char* va_p = tb + (32 * jb + 16 * sl) * ROWB + vadr[eb];
+          const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)va_p);
+          const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(va_p + 8 * ROWB));
+          const s16x8 both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+          va[sl * EB + eb] = __builtin_bit_cast(uint4v, both);
+        }
+    };
     // O^T += V_block^T P_block^T
-    auto pv = [&](const f32x16& s, int jb) {
-      typedef short s16x4 __attribute__((ext_vector_type(4)));
-      typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+    auto pv = [&](const f32x16& s, const uint4v (&va)[2 * EB]) {
 #pragma unroll
       for (int sl = 0; sl < 2; sl++) {
         uint4v pb;
 #pragma unroll
         for (int x = 0; x < 4; x++) pb[x] = pack2<T>(s[8 * sl + 2 * x], s[8 * sl + 2 * x + 1]);
-        const char* vb = tb + (32 * jb + 16 * sl) * ROWB;
 #pragma unroll
-        for (int eb = 0; eb < EB; eb++) {
-          const char* va_p = vb + vadr[eb & 1] + 128 * (eb >> 1);
-          const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)va_p);
-          const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(va_p + 8 * ROWB));
-          typedef short s16x8 __attribute__((ext_vector_type(8)));
-          const s16x8 both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-          o[eb] = mfma16<T>(__builtin_bit_cast(uint4v, both), pb, o[eb]);
-        }
+        for (int eb = 0; eb < EB; eb++) o[eb] = mfma16<T>(va[sl * EB + eb], pb, o[eb]);
       }
     };
 
-    // both products are issued before the first softmax step, so the second one runs on the
-    // matrix pipe while the vector ALU works on the first block
-    f32x16 s0 = qk(0);
-    f32x16 s1 = qk(1);
+    uint4v va[2 * EB];
+#pragma unroll
+    for (int ks = 0; ks < QR; ks++) s1 = mfma16<T>(kb[ks], qh[ks], s1);
+    v_fetch(0, va);
+    __builtin_amdgcn_sched_barrier(0);
     soft(s0, 0);
-    pv(s0, 0);
+    pv(s0, va);
+    __builtin_amdgcn_sched_barrier(0);
+    v_fetch(1, va);
+    __builtin_amdgcn_sched_barrier(0);
     soft(s1, 1);
-    pv(s1, 1);
+    pv(s1, va);
   };
 
   if (u_lo < u_hi) request(u_lo, lds_even);
