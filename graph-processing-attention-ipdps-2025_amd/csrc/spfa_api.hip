@@ -200,8 +200,9 @@ struct GlobalLayout {
 GlobalLayout global_layout(int64_t n, int64_t n_globs, int64_t d) {
   GlobalLayout g{};
   const int64_t q_tiles = (n_globs + 127) / 128;
-  // enough key splits for ~2048 workgroups, none shorter than 512 keys
-  int64_t want = 2048 / q_tiles;
+  // one key split per workgroup slot of the device (two workgroups fit a CU): more splits only
+  // add partial results for the merge to read; none shorter than 512 keys
+  int64_t want = 2 * (int64_t)device_cu_count() / q_tiles;
   if (want < 1) want = 1;
   int64_t run = (n + want - 1) / want;
   if (run < 512) run = 512;

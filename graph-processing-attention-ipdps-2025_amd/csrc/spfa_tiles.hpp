@@ -434,6 +434,18 @@ __global__ __launch_bounds__(256, 2) void tile_kernel(TileArgs a) {
       if constexpr (MODE == kTileBand) {
         const int64_t ub = ut + 32 * jb;
         full = (ub + 31 < u_hi) && (ub + a.w >= tw0 + 31) && (ub + 31 <= tw0 + a.w);
+      } else if constexpr (MODE == kTileGlobalRows) {
+        // keys are the tokens ub .. ub+31: live for every query unless the block touches the
+        // window of one of this wavefront's query tokens
+        const int64_t ub = ut + 32 * jb;
+        const bool hit = (ub + 31 + a.w >= q_tok) && (ub <= q_tok + a.w);
+        full = (ub + 31 < u_hi) && (__builtin_amdgcn_ballot_w64(hit) == 0);
+      } else {
+        // keys are listed tokens, queries the tokens tw0 .. tw0+31: live unless one of the
+        // block's keys lies in the window of one of them
+        const int64_t kt = (int64_t)ktok_s[32 * jb + r];
+        const bool hit = (kt + a.w >= tw0) && (kt <= tw0 + 31 + a.w);
+        full = (32 * jb + 31 < rem) && (__builtin_amdgcn_ballot_w64(hit) == 0);
       }
       if (!full) {
 #pragma unroll
