@@ -133,15 +133,15 @@ __device__ __forceinline__ void tile_write_row(const Tensors& t, int64_t row, in
   wb *= inv * o_scale;  // o_scale: o was accumulated against a reference below the maximum m
   wa *= inv;
   T* orow = (T*)t.out + row * D;
+  if constexpr (kF32) {
 #pragma unroll
-  for (int eb = 0; eb < D / 32; eb++) {
+    for (int eb = 0; eb < D / 32; eb++) {
 #pragma unroll
-    for (int g4 = 0; g4 < 4; g4++) {
-      const int e = 32 * eb + 8 * g4 + 4 * h;
-      float x[4];
+      for (int g4 = 0; g4 < 4; g4++) {
+        const int e = 32 * eb + 8 * g4 + 4 * h;
+        float x[4];
 #pragma unroll
-      for (int i = 0; i < 4; i++) x[i] = o[eb][4 * g4 + i] * wb;
-      if constexpr (kF32) {
+        for (int i = 0; i < 4; i++) x[i] = o[eb][4 * g4 + i] * wb;
         if (wa != 0.f) {
           float4v oi = *reinterpret_cast<const float4v*>(orow + e);
 #pragma unroll
@@ -149,16 +149,43 @@ __device__ __forceinline__ void tile_write_row(const Tensors& t, int64_t row, in
         }
         float4v y = {x[0], x[1], x[2], x[3]};
         *reinterpret_cast<float4v*>(orow + e) = y;
-      } else {
-        typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+      }
+    }
+  } else {
+    // A lane holds 4 consecutive elements (8 bytes) of each group of 8; the other 4 are in the
+    // lane of the other half of the wavefront that works on the same row.  The two trade
+    // halves so that each writes whole 16-byte pieces (groups 0, 1 of every 32 elements stay
+    // with the lower lane, 2, 3 with the upper one).
+    typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+    const int partner = (int)((__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u)) ^ 32u) << 2);
+#pragma unroll
+    for (int eb = 0; eb < D / 32; eb++) {
+      u32x2 y[4];
+#pragma unroll
+      for (int g4 = 0; g4 < 4; g4++) {
+        const int e = 32 * eb + 8 * g4 + 4 * h;
+        float x[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) x[i] = o[eb][4 * g4 + i] * wb;
         if (wa != 0.f) {
           typedef T t4 __attribute__((ext_vector_type(4)));
           t4 oi = *reinterpret_cast<const t4*>(orow + e);
 #pragma unroll
           for (int i = 0; i < 4; i++) x[i] += wa * (float)oi[i];
         }
-        u32x2 y = {pack2<T>(x[0], x[1]), pack2<T>(x[2], x[3])};
-        *reinterpret_cast<u32x2*>(orow + e) = y;
+        y[g4][0] = pack2<T>(x[0], x[1]);
+        y[g4][1] = pack2<T>(x[2], x[3]);
+      }
+#pragma unroll
+      for (int k = 0; k < 2; k++) {
+        const u32x2 give = h ? y[k] : y[2 + k];
+        const u32x2 keep = h ? y[2 + k] : y[k];
+        u32x2 got;
+        got[0] = (uint32_t)__builtin_amdgcn_ds_bpermute(partner, (int)give[0]);
+        got[1] = (uint32_t)__builtin_amdgcn_ds_bpermute(partner, (int)give[1]);
+        const uint4v piece = h ? uint4v{got[0], got[1], keep[0], keep[1]}
+                               : uint4v{keep[0], keep[1], got[0], got[1]};
+        *reinterpret_cast<uint4v*>(orow + 32 * eb + 8 * (2 * h + k)) = piece;
       }
     }
   }
