@@ -114,14 +114,28 @@ Tensors make_tensors(const spfa_problem_t* p) {
 }
 
 int dispatch_csr(const spfa_problem_t* p, const CsrMask& mask, const EngineSizing& s, int use_nan,
-                 void* ws, hipStream_t stream) {
+                 void* ws, hipStream_t stream, int phase = kEngineAll, const void* plan_buf = nullptr) {
   Tensors t = make_tensors(p);
   switch (p->dtype) {
-    case SPFA_DTYPE_F32: return run_csr<float>(t, mask, s, use_nan, ws, stream);
-    case SPFA_DTYPE_F16: return run_csr<f16>(t, mask, s, use_nan, ws, stream);
-    case SPFA_DTYPE_BF16: return run_csr<bf16>(t, mask, s, use_nan, ws, stream);
+    case SPFA_DTYPE_F32: return run_csr<float>(t, mask, s, use_nan, ws, stream, phase, plan_buf);
+    case SPFA_DTYPE_F16: return run_csr<f16>(t, mask, s, use_nan, ws, stream, phase, plan_buf);
+    case SPFA_DTYPE_BF16: return run_csr<bf16>(t, mask, s, use_nan, ws, stream, phase, plan_buf);
   }
   return SPFA_ERR_UNSUPPORTED;
+}
+
+// The work list of an explicit mask does not depend on Q, K, V or their type: it is built with a
+// problem that only carries the row count.
+int build_work_list(int64_t n_q, const CsrMask& mask, const EngineSizing& s, void* plan_buf,
+                    hipStream_t stream) {
+  Tensors t{};
+  t.n_q = n_q;
+  t.d = 64;
+  return run_csr<float>(t, mask, s, 0, plan_buf, stream, kEnginePlanOnly, nullptr);
+}
+
+size_t work_list_bytes(int64_t n_q, int64_t nnz) {
+  return engine_workspace(size_csr(n_q, nnz), n_q, 64).off_pm;
 }
 
 int dispatch_stride(const spfa_problem_t* p, const StrideMask& mask, const EngineSizing& s,
@@ -286,6 +300,44 @@ int spfa_csr_forward(const spfa_problem_t* p, const void* row_off, int row_off_b
   return dispatch_csr(p, mask, s, use_nan ? 1 : 0, workspace, (hipStream_t)stream);
 }
 
+size_t spfa_csr_plan_bytes(int64_t n_q, int64_t nnz) {
+  if (n_q < 0 || nnz < 0) return 0;
+  return work_list_bytes(n_q, nnz);
+}
+
+int spfa_csr_plan(int64_t n_q, const void* row_off, int row_off_bytes, const void* col_ind,
+                  int64_t nnz, void* plan, size_t plan_bytes, void* stream) {
+  if (n_q < 0 || n_q >= (int64_t)1 << 31 || nnz < 0 || (row_off_bytes != 4 && row_off_bytes != 8))
+    return SPFA_ERR_BAD_ARG;
+  if (n_q == 0) return SPFA_OK;
+  if (!row_off || (nnz > 0 && !col_ind)) return SPFA_ERR_BAD_ARG;
+  int rc = check_workspace(plan, plan_bytes, work_list_bytes(n_q, nnz));
+  if (rc) return rc;
+  CsrMask mask{row_off, (const uint32_t*)col_ind, row_off_bytes == 8 ? 1 : 0, nullptr, nullptr};
+  return build_work_list(n_q, mask, size_csr(n_q, nnz), plan, (hipStream_t)stream);
+}
+
+int spfa_csr_forward_planned(const spfa_problem_t* p, const void* row_off, int row_off_bytes,
+                             const void* col_ind, int64_t nnz, int use_nan, const void* plan,
+                             size_t plan_bytes, void* workspace, size_t workspace_bytes,
+                             void* stream) {
+  int rc = check_problem(p);
+  if (rc) return rc;
+  if (nnz < 0 || (row_off_bytes != 4 && row_off_bytes != 8)) return SPFA_ERR_BAD_ARG;
+  rc = check_pointers(p);
+  if (rc) return rc;
+  if (p->n_q == 0) return SPFA_OK;
+  if (!row_off || (nnz > 0 && !col_ind)) return SPFA_ERR_BAD_ARG;
+  EngineSizing s = size_csr(p->n_q, nnz);
+  rc = check_workspace(plan, plan_bytes, work_list_bytes(p->n_q, nnz));
+  if (rc) return rc;
+  rc = check_workspace(workspace, workspace_bytes, engine_workspace(s, p->n_q, p->d).total);
+  if (rc) return rc;
+  CsrMask mask{row_off, (const uint32_t*)col_ind, row_off_bytes == 8 ? 1 : 0, nullptr, nullptr};
+  return dispatch_csr(p, mask, s, use_nan ? 1 : 0, workspace, (hipStream_t)stream, kEngineRunOnly,
+                      plan);
+}
+
 /* ------------------------------------------------------------------------------ COO */
 size_t spfa_coo_workspace_bytes(int64_t n_q, int64_t nnz, int64_t d, int dtype) {
   (void)dtype;
@@ -310,12 +362,69 @@ int spfa_coo_forward(const spfa_problem_t* p, const void* row_ind, int row_ind_b
                        coo_bytes + engine_workspace(s, p->n_q, p->d).total);
   if (rc) return rc;
   CooCsr csr{};
+  const CooWorkspace cw = coo_workspace(p->n_q, nnz);
   rc = coo_to_csr(row_ind, row_ind_bytes == 8 ? 1 : 0, (const uint32_t*)col_ind, nnz, p->n_q,
-                  workspace, (hipStream_t)stream, &csr);
+                  workspace, (char*)workspace + cw.keep_total, (hipStream_t)stream, &csr);
   if (rc) return rc;
   CsrMask mask{csr.row_off, (const uint32_t*)col_ind, 0, csr.cols, csr.unsorted};
   return dispatch_csr(p, mask, s, use_nan ? 1 : 0, (char*)workspace + coo_bytes,
                       (hipStream_t)stream);
+}
+
+size_t spfa_coo_plan_bytes(int64_t n_q, int64_t nnz) {
+  if (n_q < 0 || nnz < 0) return 0;
+  return coo_workspace(n_q, nnz).keep_total + work_list_bytes(n_q, nnz);
+}
+
+size_t spfa_coo_plan_workspace_bytes(int64_t n_q, int64_t nnz) {
+  if (n_q < 0 || nnz < 0) return 0;
+  const CooWorkspace w = coo_workspace(n_q, nnz);
+  return w.total - w.keep_total;
+}
+
+int spfa_coo_plan(int64_t n_q, const void* row_ind, int row_ind_bytes, const void* col_ind,
+                  int64_t nnz, void* plan, size_t plan_bytes, void* workspace,
+                  size_t workspace_bytes, void* stream) {
+  if (n_q < 0 || n_q >= (int64_t)1 << 31 || nnz < 0 || nnz >= (int64_t)1 << 31 ||
+      (row_ind_bytes != 4 && row_ind_bytes != 8))
+    return SPFA_ERR_BAD_ARG;
+  if (n_q == 0) return SPFA_OK;
+  if (nnz > 0 && (!row_ind || !col_ind)) return SPFA_ERR_BAD_ARG;
+  const CooWorkspace w = coo_workspace(n_q, nnz);
+  int rc = check_workspace(plan, plan_bytes, w.keep_total + work_list_bytes(n_q, nnz));
+  if (rc) return rc;
+  rc = check_workspace(workspace, workspace_bytes, w.total - w.keep_total);
+  if (rc) return rc;
+  CooCsr csr{};
+  rc = coo_to_csr(row_ind, row_ind_bytes == 8 ? 1 : 0, (const uint32_t*)col_ind, nnz, n_q, plan,
+                  workspace, (hipStream_t)stream, &csr);
+  if (rc) return rc;
+  CsrMask mask{csr.row_off, (const uint32_t*)col_ind, 0, csr.cols, csr.unsorted};
+  return build_work_list(n_q, mask, size_csr(n_q, nnz), (char*)plan + w.keep_total,
+                         (hipStream_t)stream);
+}
+
+int spfa_coo_forward_planned(const spfa_problem_t* p, const void* col_ind, int64_t nnz, int use_nan,
+                             const void* plan, size_t plan_bytes, void* workspace,
+                             size_t workspace_bytes, void* stream) {
+  int rc = check_problem(p);
+  if (rc) return rc;
+  if (nnz < 0 || nnz >= (int64_t)1 << 31) return SPFA_ERR_BAD_ARG;
+  rc = check_pointers(p);
+  if (rc) return rc;
+  if (p->n_q == 0) return SPFA_OK;
+  if (nnz > 0 && !col_ind) return SPFA_ERR_BAD_ARG;
+  EngineSizing s = size_csr(p->n_q, nnz);
+  const CooWorkspace w = coo_workspace(p->n_q, nnz);
+  rc = check_workspace(plan, plan_bytes, w.keep_total + work_list_bytes(p->n_q, nnz));
+  if (rc) return rc;
+  rc = check_workspace(workspace, workspace_bytes, engine_workspace(s, p->n_q, p->d).total);
+  if (rc) return rc;
+  const char* pb = (const char*)plan;
+  CsrMask mask{pb + w.off_row_off, (const uint32_t*)col_ind, 0, (const uint32_t*)(pb + w.off_cols),
+               (const uint32_t*)(pb + w.off_flag)};
+  return dispatch_csr(p, mask, s, use_nan ? 1 : 0, workspace, (hipStream_t)stream, kEngineRunOnly,
+                      pb + w.keep_total);
 }
 
 /* ------------------------------------------------------------------------------ Local */

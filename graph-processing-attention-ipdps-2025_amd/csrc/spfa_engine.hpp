@@ -59,6 +59,8 @@ struct MultiRow {
 
 struct Plan {
   Counters* cnt;
+  uint32_t* cursor;  // next work item of segments_kernel (separate from cnt so that a plan can
+                     // be shared by calls that each bring their own scratch)
   Item* items;
   MultiRow* multi;
   float* pm;
@@ -71,6 +73,10 @@ struct Plan {
   int64_t short_max;
   int64_t seg;
 };
+
+static __global__ void reset_cursor_kernel(uint32_t* cursor) {
+  if (threadIdx.x == 0) *cursor = 0;
+}
 
 static __global__ void reset_counters_kernel(Counters* cnt) {
   if (threadIdx.x == 0) {
@@ -374,7 +380,7 @@ __global__ __launch_bounds__(256) void segments_kernel(Tensors t, Mask mask, Pla
 
   while (true) {
     uint32_t idx = 0;
-    if (lane == 0) idx = atomicAdd(&plan.cnt->next_item, 1u);
+    if (lane == 0) idx = atomicAdd(plan.cursor, 1u);
     idx = (uint32_t)__builtin_amdgcn_readfirstlane((int)idx);
     if (idx >= n_items) break;
     const Item it = plan.items[idx];
@@ -518,15 +524,23 @@ inline int device_cu_count() {
   return cus;
 }
 
+// What a call does: the whole thing, only the work list of the mask (a "plan": counters, items,
+// multi-segment rows - the first off_pm bytes of the workspace layout, independent of Q, K, V), or
+// only the attention against a work list built earlier (`plan_buf`, read-only; `ws` then only
+// provides the work cursor and the partial results, in the same layout).
+enum { kEngineAll = 0, kEnginePlanOnly = 1, kEngineRunOnly = 2 };
+
 template <class Lay, class Mask>
 int launch_engine(const Tensors& t, const Mask& mask, const EngineSizing& s, int use_nan, void* ws,
-                  hipStream_t stream) {
+                  hipStream_t stream, int phase = kEngineAll, const void* plan_buf = nullptr) {
   WorkspaceLayout w = engine_workspace(s, t.n_q, t.d);
   char* base = (char*)ws;
+  char* pbase = (phase == kEngineRunOnly) ? (char*)const_cast<void*>(plan_buf) : base;
   Plan plan{};
-  plan.cnt = (Counters*)(base + w.off_cnt);
-  plan.items = (Item*)(base + w.off_items);
-  plan.multi = (MultiRow*)(base + w.off_multi);
+  plan.cnt = (Counters*)(pbase + w.off_cnt);
+  plan.items = (Item*)(pbase + w.off_items);
+  plan.multi = (MultiRow*)(pbase + w.off_multi);
+  plan.cursor = &((Counters*)(base + w.off_cnt))->next_item;
   plan.pm = (float*)(base + w.off_pm);
   plan.pl = (float*)(base + w.off_pl);
   plan.pacc = (float*)(base + w.off_pacc);
@@ -539,11 +553,14 @@ int launch_engine(const Tensors& t, const Mask& mask, const EngineSizing& s, int
   if (t.n_q == 0) return 0;
 
   const bool has_long = s.max_deg > s.short_max;
-  if (has_long) {
+  if (has_long && phase != kEngineRunOnly) {
     hipLaunchKernelGGL(reset_counters_kernel, dim3(1), dim3(64), 0, stream, plan.cnt);
     hipLaunchKernelGGL((plan_kernel<Mask>), dim3((unsigned)((t.n_q + kPlanThreads - 1) / kPlanThreads)),
                        dim3(kPlanThreads), 0, stream, t.n_q, mask, plan);
   }
+  if (phase == kEnginePlanOnly) return hipGetLastError() == hipSuccess ? 0 : 4;
+  if (has_long && phase == kEngineRunOnly)
+    hipLaunchKernelGGL(reset_cursor_kernel, dim3(1), dim3(64), 0, stream, plan.cursor);
 
   const KernelEvents ev = kernel_events();
   const bool timed = ev.start != nullptr && ev.stop != nullptr;
@@ -576,17 +593,17 @@ inline bool aligned16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
 // Pick the lane layout for (T, d).
 template <typename T, class Mask>
 int run_engine(const Tensors& t, const Mask& mask, const EngineSizing& s, int use_nan, void* ws,
-               hipStream_t stream) {
+               hipStream_t stream, int phase = kEngineAll, const void* plan_buf = nullptr) {
   const int64_t row_bytes = (int64_t)t.d * (int64_t)sizeof(T);
   const bool vec_ok = aligned16(t.q) && aligned16(t.k) && aligned16(t.v) && aligned16(t.out);
   if (vec_ok) {
-    if (row_bytes == 64) return launch_engine<VecLay<T, 4>, Mask>(t, mask, s, use_nan, ws, stream);
-    if (row_bytes == 128) return launch_engine<VecLay<T, 8>, Mask>(t, mask, s, use_nan, ws, stream);
-    if (row_bytes == 256) return launch_engine<VecLay<T, 16>, Mask>(t, mask, s, use_nan, ws, stream);
-    if (row_bytes == 512) return launch_engine<VecLay<T, 32>, Mask>(t, mask, s, use_nan, ws, stream);
+    if (row_bytes == 64) return launch_engine<VecLay<T, 4>, Mask>(t, mask, s, use_nan, ws, stream, phase, plan_buf);
+    if (row_bytes == 128) return launch_engine<VecLay<T, 8>, Mask>(t, mask, s, use_nan, ws, stream, phase, plan_buf);
+    if (row_bytes == 256) return launch_engine<VecLay<T, 16>, Mask>(t, mask, s, use_nan, ws, stream, phase, plan_buf);
+    if (row_bytes == 512) return launch_engine<VecLay<T, 32>, Mask>(t, mask, s, use_nan, ws, stream, phase, plan_buf);
   }
-  if (t.d <= 128) return launch_engine<GenLay<T, 2>, Mask>(t, mask, s, use_nan, ws, stream);
-  if (t.d <= 1024) return launch_engine<GenLay<T, 16>, Mask>(t, mask, s, use_nan, ws, stream);
+  if (t.d <= 128) return launch_engine<GenLay<T, 2>, Mask>(t, mask, s, use_nan, ws, stream, phase, plan_buf);
+  if (t.d <= 1024) return launch_engine<GenLay<T, 16>, Mask>(t, mask, s, use_nan, ws, stream, phase, plan_buf);
   return 5;
 }
 

@@ -7,8 +7,8 @@ namespace spfa {
 #if SPFA_INST_MASK == 0
 template <>
 int run_csr<SPFA_INST_T>(const Tensors& t, const CsrMask& mask, const EngineSizing& s, int use_nan,
-                         void* ws, hipStream_t stream) {
-  return run_engine<SPFA_INST_T, CsrMask>(t, mask, s, use_nan, ws, stream);
+                         void* ws, hipStream_t stream, int phase, const void* plan_buf) {
+  return run_engine<SPFA_INST_T, CsrMask>(t, mask, s, use_nan, ws, stream, phase, plan_buf);
 }
 #elif SPFA_INST_MASK == 1
 template <>

@@ -7,9 +7,11 @@
 
 namespace spfa {
 
+// phase / plan_buf: see launch_engine (whole call, work list only, or attention against a work
+// list built earlier)
 template <typename T>
 int run_csr(const Tensors& t, const CsrMask& mask, const EngineSizing& s, int use_nan, void* ws,
-            hipStream_t stream);
+            hipStream_t stream, int phase = kEngineAll, const void* plan_buf = nullptr);
 template <typename T>
 int run_stride(const Tensors& t, const StrideMask& mask, const EngineSizing& s, int use_nan,
                void* ws, hipStream_t stream);

@@ -354,12 +354,13 @@ CooWorkspace coo_workspace(int64_t n_rows, int64_t nnz) {
   const int64_t scan_len = n_hist > n_rows ? n_hist : n_rows;
   const int64_t n_tiles = (scan_len + kScanTile - 1) / kScanTile + 1;
   size_t off = 0;
-  w.off_counts = off;  off = align_up(off + (size_t)(n_rows + 1) * 4, 256);
   w.off_row_off = off; off = align_up(off + (size_t)(n_rows + 1) * 4, 256);
-  w.off_cursor = off;  off = align_up(off + (size_t)(n_rows + 1) * 4, 256);
-  w.off_tiles = off;   off = align_up(off + (size_t)n_tiles * 4, 256);
   w.off_cols = off;    off = align_up(off + (size_t)(nnz > 0 ? nnz : 1) * 4, 256);
   w.off_flag = off;    off = align_up(off + 4, 256);
+  w.keep_total = off;
+  w.off_counts = off;  off = align_up(off + (size_t)(n_rows + 1) * 4, 256);
+  w.off_cursor = off;  off = align_up(off + (size_t)(n_rows + 1) * 4, 256);
+  w.off_tiles = off;   off = align_up(off + (size_t)n_tiles * 4, 256);
   w.off_hist = off;    off = align_up(off + (size_t)(n_hist + 1) * 4, 256);
   w.off_tmp_pairs = off; off = align_up(off + (size_t)(w.partition ? nnz : 0) * 8, 256);
   w.total = off;
@@ -367,15 +368,16 @@ CooWorkspace coo_workspace(int64_t n_rows, int64_t nnz) {
 }
 
 int coo_to_csr(const void* row_ind, int row_wide, const uint32_t* col_ind, int64_t nnz,
-               int64_t n_rows, void* ws, hipStream_t stream, CooCsr* out) {
+               int64_t n_rows, void* keep, void* scratch, hipStream_t stream, CooCsr* out) {
   CooWorkspace w = coo_workspace(n_rows, nnz);
-  char* base = (char*)ws;
+  char* kbase = (char*)keep;
+  char* base = (char*)scratch - w.keep_total;  // scratch offsets are counted from the start of keep
   uint32_t* counts = (uint32_t*)(base + w.off_counts);
-  uint32_t* row_off = (uint32_t*)(base + w.off_row_off);
+  uint32_t* row_off = (uint32_t*)(kbase + w.off_row_off);
   uint32_t* cursor = (uint32_t*)(base + w.off_cursor);
   uint32_t* tiles = (uint32_t*)(base + w.off_tiles);
-  uint32_t* cols = (uint32_t*)(base + w.off_cols);
-  uint32_t* flag = (uint32_t*)(base + w.off_flag);
+  uint32_t* cols = (uint32_t*)(kbase + w.off_cols);
+  uint32_t* flag = (uint32_t*)(kbase + w.off_flag);
   const int64_t n_tiles = (n_rows + kScanTile - 1) / kScanTile;
 
   hipLaunchKernelGGL(fill_u32_kernel, dim3(grid_for(n_rows + 1, 256, 4096)), dim3(256), 0, stream,

@@ -10,7 +10,10 @@ namespace spfa {
 inline size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 
 struct CooWorkspace {
-  size_t off_counts, off_row_off, off_cursor, off_tiles, off_cols, off_flag;
+  // what the attention kernels read afterwards: offsets, bucketed columns, the "unsorted" flag
+  size_t off_row_off, off_cols, off_flag, keep_total;
+  // scratch of the conversion itself (follows the part above)
+  size_t off_counts, off_cursor, off_tiles;
   // two-pass partition (used when the row index fits 22 bits)
   size_t off_hist, off_tmp_pairs, total;
   int partition;       // 1: two-pass LDS partition, 0: per-entry global atomics
@@ -28,15 +31,16 @@ struct CooCsr {
                               // caller's column array as it is
 };
 
-// Turns COO entries into 32-bit CSR offsets placed in `ws` (coo_workspace().total bytes).
+// Turns COO entries into 32-bit CSR offsets (coo_workspace() sizes the two buffers).
 // Entries that already come sorted by row (the reference's contract) only need the offsets;
 // otherwise they are bucketed by row and the columns copied, in no particular order inside a
 // row: a two-pass partition with LDS-private histograms (high digit of the row, then low digit
 // inside each high bucket) when the row index fits 22 bits, per-entry global atomics otherwise.  The choice is made on the device (no host synchronisation):
 // both sets of kernels are enqueued and the ones that are not needed return at once.
 // Entries with a row outside [0, n_rows) are dropped (and force the bucketing path).
+// `keep` receives the result (keep_total bytes), `scratch` is total - keep_total bytes.
 int coo_to_csr(const void* row_ind, int row_wide, const uint32_t* col_ind, int64_t nnz,
-               int64_t n_rows, void* ws, hipStream_t stream, CooCsr* out);
+               int64_t n_rows, void* keep, void* scratch, hipStream_t stream, CooCsr* out);
 
 // Global-row bookkeeping for the global-minus-local mask.  `bits` holds (n+31)/32 bitmap words
 // followed by one counter word; afterwards bit i is set for every listed i in [0, n), `uq` holds

@@ -36,6 +36,66 @@ torch::Tensor spfa_coo_forward_py(torch::Tensor Q, torch::Tensor K, torch::Tenso
   return O;
 }
 
+// plan(w_row_ind, w_col_ind, n_rows) -> uint8 device tensor: row offsets, bucketed columns (when
+// the entries are not sorted by row) and the work list, reusable by forward_planned for any
+// number of calls with the same w_col_ind (masks are built once and reused by the reference's
+// callers, verification/verify.py:95-98).
+torch::Tensor spfa_coo_plan_py(torch::Tensor W_row_ind, torch::Tensor W_col_ind, int64_t n_rows) {
+  CHECK_INPUT(W_row_ind);
+  CHECK_INPUT(W_col_ind);
+  c10::DeviceGuard guard(W_row_ind.device());
+  TORCH_CHECK(W_row_ind.dim() == 1 && W_col_ind.dim() == 1 &&
+                  W_row_ind.size(0) == W_col_ind.size(0),
+              "W_row_ind and W_col_ind must be 1-D and of equal length");
+  TORCH_CHECK(n_rows >= 0, "n_rows must not be negative");
+  const int row_bytes = spfa_ext::index_bytes(W_row_ind, "W_row_ind", true);
+  spfa_ext::index_bytes(W_col_ind, "W_col_ind", false);
+  const int64_t nnz = W_col_ind.size(0);
+  torch::Tensor plan = spfa_ext::make_workspace(spfa_coo_plan_bytes(n_rows, nnz), W_row_ind);
+  torch::Tensor ws = spfa_ext::make_workspace(spfa_coo_plan_workspace_bytes(n_rows, nnz), W_row_ind);
+  spfa_ext::raise_on_error(spfa_coo_plan(n_rows, W_row_ind.data_ptr(), row_bytes, W_col_ind.data_ptr(),
+                                         nnz, plan.data_ptr(), (size_t)plan.numel(), ws.data_ptr(),
+                                         (size_t)ws.numel(), spfa_ext::current_stream(W_row_ind)));
+  return plan;
+}
+
+torch::Tensor spfa_coo_forward_planned_py(torch::Tensor Q, torch::Tensor K, torch::Tensor V,
+                                          torch::Tensor W_row_ind, torch::Tensor W_col_ind,
+                                          torch::Tensor W_val, torch::Tensor m, torch::Tensor l,
+                                          torch::Tensor O, bool use_nan, torch::Tensor plan) {
+  CHECK_INPUT(Q);
+  CHECK_INPUT(K);
+  CHECK_INPUT(V);
+  CHECK_INPUT(W_row_ind);
+  CHECK_INPUT(W_col_ind);
+  CHECK_INPUT(W_val);
+  CHECK_INPUT(m);
+  CHECK_INPUT(l);
+  CHECK_INPUT(O);
+  CHECK_INPUT(plan);
+
+  c10::DeviceGuard guard(Q.device());
+  spfa_problem_t p = spfa_ext::make_problem(Q, K, V, m, l, O);
+  TORCH_CHECK(W_row_ind.dim() == 1 && W_col_ind.dim() == 1 &&
+                  W_row_ind.size(0) == W_col_ind.size(0),
+              "W_row_ind and W_col_ind must be 1-D and of equal length");
+  TORCH_CHECK(W_val.scalar_type() == Q.scalar_type(), "W_val must have the dtype of Q");
+  TORCH_CHECK(plan.scalar_type() == torch::kUInt8 && plan.dim() == 1, "plan must come from plan()");
+  spfa_ext::index_bytes(W_col_ind, "W_col_ind", false);
+  const int64_t nnz = W_col_ind.size(0);
+
+  // (the attention part of the plain call's workspace would do; the plain size is simply enough)
+  const size_t ws_bytes = spfa_csr_workspace_bytes(p.n_q, nnz, p.d, p.dtype);
+  torch::Tensor ws = spfa_ext::make_workspace(ws_bytes, Q);
+  spfa_ext::raise_on_error(spfa_coo_forward_planned(
+      &p, W_col_ind.data_ptr(), nnz, use_nan ? 1 : 0, plan.data_ptr(), (size_t)plan.numel(),
+      ws.data_ptr(), (size_t)ws.numel(), spfa_ext::current_stream(Q)));
+  return O;
+}
+
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, mod) {
   mod.def("forward", &spfa_coo_forward_py, "Sparse-FlashAttention forward, COO mask (HIP, gfx950)");
+  mod.def("plan", &spfa_coo_plan_py, "Mask pre-pass of a COO mask, for forward_planned");
+  mod.def("forward_planned", &spfa_coo_forward_planned_py,
+          "forward(...) with the mask pre-pass taken from plan(...)");
 }

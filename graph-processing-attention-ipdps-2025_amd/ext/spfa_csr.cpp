@@ -37,6 +37,62 @@ torch::Tensor spfa_csr_forward_py(torch::Tensor Q, torch::Tensor K, torch::Tenso
   return O;
 }
 
+// plan(w_row_off, w_col_ind) -> uint8 device tensor: the mask pre-pass, reusable by
+// forward_planned for any number of calls with the same two mask tensors (masks are built once
+// and reused by the reference's callers, verification/verify.py:68-71).
+torch::Tensor spfa_csr_plan_py(torch::Tensor W_row_off, torch::Tensor W_col_ind) {
+  CHECK_INPUT(W_row_off);
+  CHECK_INPUT(W_col_ind);
+  c10::DeviceGuard guard(W_row_off.device());
+  TORCH_CHECK(W_row_off.dim() == 1 && W_row_off.size(0) >= 1, "W_row_off must hold rows+1 offsets");
+  TORCH_CHECK(W_col_ind.dim() == 1, "W_col_ind must be 1-D");
+  const int off_bytes = spfa_ext::index_bytes(W_row_off, "W_row_off", true);
+  spfa_ext::index_bytes(W_col_ind, "W_col_ind", false);
+  const int64_t n_q = W_row_off.size(0) - 1, nnz = W_col_ind.size(0);
+  torch::Tensor plan = spfa_ext::make_workspace(spfa_csr_plan_bytes(n_q, nnz), W_row_off);
+  spfa_ext::raise_on_error(spfa_csr_plan(n_q, W_row_off.data_ptr(), off_bytes, W_col_ind.data_ptr(), nnz,
+                                         plan.data_ptr(), (size_t)plan.numel(),
+                                         spfa_ext::current_stream(W_row_off)));
+  return plan;
+}
+
+torch::Tensor spfa_csr_forward_planned_py(torch::Tensor Q, torch::Tensor K, torch::Tensor V,
+                                          torch::Tensor W_row_off, torch::Tensor W_col_ind,
+                                          torch::Tensor W_val, torch::Tensor m, torch::Tensor l,
+                                          torch::Tensor O, bool use_nan, torch::Tensor plan) {
+  CHECK_INPUT(Q);
+  CHECK_INPUT(K);
+  CHECK_INPUT(V);
+  CHECK_INPUT(W_row_off);
+  CHECK_INPUT(W_col_ind);
+  CHECK_INPUT(W_val);
+  CHECK_INPUT(m);
+  CHECK_INPUT(l);
+  CHECK_INPUT(O);
+  CHECK_INPUT(plan);
+
+  c10::DeviceGuard guard(Q.device());
+  spfa_problem_t p = spfa_ext::make_problem(Q, K, V, m, l, O);
+  TORCH_CHECK(W_row_off.dim() == 1 && W_row_off.size(0) == Q.size(0) + 1,
+              "W_row_off must hold rows+1 offsets");
+  TORCH_CHECK(W_col_ind.dim() == 1, "W_col_ind must be 1-D");
+  TORCH_CHECK(W_val.scalar_type() == Q.scalar_type(), "W_val must have the dtype of Q");
+  TORCH_CHECK(plan.scalar_type() == torch::kUInt8 && plan.dim() == 1, "plan must come from plan()");
+  const int off_bytes = spfa_ext::index_bytes(W_row_off, "W_row_off", true);
+  spfa_ext::index_bytes(W_col_ind, "W_col_ind", false);
+  const int64_t nnz = W_col_ind.size(0);
+
+  const size_t ws_bytes = spfa_csr_workspace_bytes(p.n_q, nnz, p.d, p.dtype);
+  torch::Tensor ws = spfa_ext::make_workspace(ws_bytes, Q);
+  spfa_ext::raise_on_error(spfa_csr_forward_planned(
+      &p, W_row_off.data_ptr(), off_bytes, W_col_ind.data_ptr(), nnz, use_nan ? 1 : 0, plan.data_ptr(),
+      (size_t)plan.numel(), ws.data_ptr(), (size_t)ws.numel(), spfa_ext::current_stream(Q)));
+  return O;
+}
+
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, mod) {
   mod.def("forward", &spfa_csr_forward_py, "Sparse-FlashAttention forward, CSR mask (HIP, gfx950)");
+  mod.def("plan", &spfa_csr_plan_py, "Mask pre-pass of a CSR mask, for forward_planned");
+  mod.def("forward_planned", &spfa_csr_forward_planned_py,
+          "forward(...) with the mask pre-pass taken from plan(...)");
 }

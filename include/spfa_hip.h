@@ -106,6 +106,39 @@ int spfa_coo_forward(const spfa_problem_t* p, const void* row_ind, int row_ind_b
                      const void* col_ind, int64_t nnz, int use_nan, void* workspace,
                      size_t workspace_bytes, void* stream);
 
+/* Mask plans for the explicit masks.  The reference rebuilds nothing between calls because its
+ * kernel reads the mask directly; its callers build a mask once and reuse it for many calls
+ * (verification/verify.py:68-71,95-98 build the CSR / COO tensors once; 337-352 chain calls on
+ * them).  Here the mask pre-pass (the work list of long rows; for COO also the row offsets and, for
+ * unsorted entries, the bucketed columns) does not depend on Q, K, V or their type, so it can be
+ * built once into a caller-owned device buffer and reused:
+ *
+ *   plan = device buffer of spfa_*_plan_bytes(...) bytes, 256-byte aligned
+ *   spfa_*_plan(...)              fills it (asynchronous on `stream`)
+ *   spfa_*_forward_planned(...)   same result as spfa_*_forward with the same mask arrays, without
+ *                                 the pre-pass; reads the plan, writes only `workspace`
+ *                                 (spfa_*_workspace_bytes(...) bytes as for the plain call).
+ *
+ * The mask arrays passed to forward_planned must be the ones the plan was built from (CSR: both;
+ * COO: col_ind - it is read in place when the entries were sorted by row).  Calls that share a
+ * plan but use different workspaces are independent.  spfa_coo_plan also needs a scratch buffer
+ * of spfa_coo_plan_workspace_bytes(...) bytes that is free again when the call has run. */
+size_t spfa_csr_plan_bytes(int64_t n_q, int64_t nnz);
+int spfa_csr_plan(int64_t n_q, const void* row_off, int row_off_bytes, const void* col_ind,
+                  int64_t nnz, void* plan, size_t plan_bytes, void* stream);
+int spfa_csr_forward_planned(const spfa_problem_t* p, const void* row_off, int row_off_bytes,
+                             const void* col_ind, int64_t nnz, int use_nan, const void* plan,
+                             size_t plan_bytes, void* workspace, size_t workspace_bytes,
+                             void* stream);
+size_t spfa_coo_plan_bytes(int64_t n_q, int64_t nnz);
+size_t spfa_coo_plan_workspace_bytes(int64_t n_q, int64_t nnz);
+int spfa_coo_plan(int64_t n_q, const void* row_ind, int row_ind_bytes, const void* col_ind,
+                  int64_t nnz, void* plan, size_t plan_bytes, void* workspace,
+                  size_t workspace_bytes, void* stream);
+int spfa_coo_forward_planned(const spfa_problem_t* p, const void* col_ind, int64_t nnz, int use_nan,
+                             const void* plan, size_t plan_bytes, void* workspace,
+                             size_t workspace_bytes, void* stream);
+
 /* Local: row i attends columns max(0, i-w) .. min(n-1, i+w)  (sp_flatt_local_kernel.cu:24-28). */
 size_t spfa_local_workspace_bytes(int64_t n, int64_t d, int dtype, int64_t local_size);
 int spfa_local_forward(const spfa_problem_t* p, int64_t local_size, void* workspace,

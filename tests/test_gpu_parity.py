@@ -326,6 +326,92 @@ def test_csr_state_in_element_dtype(mods, dtype):
     check(o, m, l, *ref, dtype)
 
 
+# ------------------------------------------------------------------ mask plans
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_csr_plan_is_reused_across_calls_and_dtypes(mods, dtype):
+    """One plan, built once from the mask alone, serves calls with different Q, K, V (and element
+    types); each result matches the oracle and the plain call."""
+    n, d = 8192, 64
+    ro, ci = syn.zipf_csr(n, 1.4, 0, 3000, seed=41)
+    ro_t, ci_t = csr_tensors(ro, ci)
+    plan = mods["spfa_csr"].plan(ro_t, ci_t)
+    plan_before = plan.clone()
+    for seed in (41, 42):
+        q, k, v = dev_qkv(n, d, dtype, seed)
+        val = torch.ones(ci_t.numel(), device=DEV, dtype=dtype)
+        m, l, o = state(n, d, dtype, torch.float32)
+        ret = mods["spfa_csr"].forward_planned(q, k, v, ro_t, ci_t, val, m, l, o, True, plan)
+        sync()
+        assert ret.data_ptr() == o.data_ptr()
+        ref = c_oracle.csr(np64(q), np64(k), np64(v), ro.numpy(), ci.numpy(), use_nan=True)
+        check(o, m, l, *ref, dtype, state_dtype=torch.float32, dead_expect="nan")
+        o2, m2, l2 = run_csr(mods, q, k, v, ro, ci, True, state_dtype=torch.float32)
+        tol = 2e-5 if dtype == torch.float32 else 2e-2
+        assert torch.allclose(torch.nan_to_num(o).float(), torch.nan_to_num(o2).float(), atol=tol)
+    assert torch.equal(plan, plan_before), "a planned call must not write to the plan"
+
+
+def test_csr_plan_short_rows_only_and_chaining(mods):
+    """A mask without long rows has an empty work list; chained planned calls accumulate."""
+    n, d = 2048, 64
+    q, k, v = dev_qkv(n, d, torch.float32, 43)
+    ro, ci = syn.bernoulli_csr(n, 0.004, seed=43)
+    half = len(ci) // 2
+    # split every row's columns over two masks
+    rows = np.repeat(np.arange(n), np.diff(ro.numpy()))
+    first = np.arange(len(ci)) % 2 == 0
+    ro1 = np.concatenate([[0], np.cumsum(np.bincount(rows[first], minlength=n))])
+    ro2 = np.concatenate([[0], np.cumsum(np.bincount(rows[~first], minlength=n))])
+    ci1, ci2 = ci.numpy()[first], ci.numpy()[~first]
+    m, l, o = state(n, d, torch.float32)
+    for ro_x, ci_x in ((ro1, ci1), (ro2, ci2)):
+        ro_t, ci_t = csr_tensors(ro_x, ci_x)
+        plan = mods["spfa_csr"].plan(ro_t, ci_t)
+        mods["spfa_csr"].forward_planned(q, k, v, ro_t, ci_t, torch.ones(len(ci_x), device=DEV), m, l, o,
+                                         False, plan)
+    sync()
+    ref = c_oracle.csr(np64(q), np64(k), np64(v), ro.numpy(), ci.numpy())
+    check(o, m, l, *ref, torch.float32)
+    assert half > 0
+
+
+@pytest.mark.parametrize("shuffle", [True, False])
+def test_coo_plan_sorted_and_unsorted(mods, shuffle):
+    n, d = 4096, 64
+    ro, ci = syn.zipf_csr(n, 1.4, 0, 2048, seed=44)
+    r, c = syn.coo_from_csr(ro, ci, shuffle_seed=44 if shuffle else None)
+    r_t, c_t = r.to(torch.uint64).to(DEV), c.to(torch.uint32).to(DEV)
+    plan = mods["spfa_coo"].plan(r_t, c_t, n)
+    plan_before = plan.clone()
+    for seed, dtype in ((44, torch.float32), (45, torch.bfloat16)):
+        q, k, v = dev_qkv(n, d, dtype, seed)
+        m, l, o = state(n, d, dtype, torch.float32)
+        mods["spfa_coo"].forward_planned(q, k, v, r_t, c_t, torch.ones(c.numel(), device=DEV, dtype=dtype),
+                                         m, l, o, True, plan)
+        sync()
+        ref = c_oracle.csr(np64(q), np64(k), np64(v), ro.numpy(), ci.numpy(), use_nan=True)
+        check(o, m, l, *ref, dtype, state_dtype=torch.float32, dead_expect="nan")
+    assert torch.equal(plan, plan_before)
+
+
+def test_plans_of_empty_masks(mods):
+    n, d = 64, 64
+    q, k, v = dev_qkv(n, d, torch.float32, 46)
+    e64 = torch.zeros(0, dtype=torch.uint64, device=DEV)
+    e32 = torch.zeros(0, dtype=torch.uint32, device=DEV)
+    m, l, o = state(n, d, torch.float32)
+    plan = mods["spfa_coo"].plan(e64, e32, n)
+    mods["spfa_coo"].forward_planned(q, k, v, e64, e32, torch.zeros(0, device=DEV), m, l, o, True, plan)
+    sync()
+    assert torch.isnan(o).all() and torch.all(l == 0)
+    ro_t = torch.zeros(n + 1, dtype=torch.uint64, device=DEV)
+    m, l, o = state(n, d, torch.float32)
+    plan = mods["spfa_csr"].plan(ro_t, e32)
+    mods["spfa_csr"].forward_planned(q, k, v, ro_t, e32, torch.zeros(0, device=DEV), m, l, o, True, plan)
+    sync()
+    assert torch.isnan(o).all() and torch.all(l == 0)
+
+
 # ------------------------------------------------------------------ COO
 @pytest.mark.parametrize("row_dtype", [torch.uint64, torch.int64, torch.int32])
 def test_coo_unsorted_equals_csr(mods, row_dtype):
