@@ -131,3 +131,29 @@ def test_wrong_argument_count_is_a_type_error(mods):
     q = torch.zeros(2, 2)
     with pytest.raises(TypeError):
         mods["spfa_local"].forward(q, q, q)
+
+
+def test_mask_arrays_from_torch_sparse_tensors():
+    """csr_arrays / coo_arrays restate verification/verify.py:68-71,95-98; checked against the
+    oracle's own dense -> CSR / COO conversions."""
+    import numpy as np
+    import torch
+    import spfa_masks
+    from oracle import spfa_oracle as so
+
+    rng = np.random.default_rng(5)
+    dense = rng.random((37, 53)) < 0.2
+    dense[4] = False  # an empty row
+    mask = torch.as_tensor(dense).to(torch.float32)
+    ro, ci, val = spfa_masks.csr_arrays(mask.to_sparse_csr())
+    ro_ref, ci_ref = so.csr_from_dense(dense)
+    assert ro.dtype == torch.uint64 and ci.dtype == torch.uint32 and val.dtype == torch.float32
+    assert np.array_equal(ro.to(torch.int64).numpy(), ro_ref) and np.array_equal(ci.to(torch.int64).numpy(), ci_ref)
+    r, c, val = spfa_masks.coo_arrays(mask.to_sparse_coo(), value_dtype=torch.bfloat16)
+    r_ref, c_ref = so.coo_from_dense(dense)
+    assert r.dtype == torch.uint64 and c.dtype == torch.uint32 and val.dtype == torch.bfloat16
+    assert np.array_equal(r.to(torch.int64).numpy(), r_ref) and np.array_equal(c.to(torch.int64).numpy(), c_ref)
+    with pytest.raises(ValueError):
+        spfa_masks.csr_arrays(mask.to_sparse_coo())
+    with pytest.raises(ValueError):
+        spfa_masks.coo_arrays(mask)
