@@ -72,7 +72,7 @@ def load_library():
     return lib
 
 
-def make_workload(name, dtype, torch, syn, inline_limit=32, planned=False):
+def make_workload(name, dtype, torch, syn, inline_limit=32, planned=False, heads=1, loop_heads=False):
     """Returns dict(call=fn(state) -> None, n, d, nnz, bytes_total, bytes_gathered, sample=fn())."""
     dev = "cuda"
     es = torch.tensor([], dtype=dtype).element_size()
@@ -91,6 +91,9 @@ def make_workload(name, dtype, torch, syn, inline_limit=32, planned=False):
                 order = torch.argsort(r, stable=True)
                 r, c = r[order].contiguous(), c[order].contiguous()
         q, k, v = syn.qkv(n, d, dtype=dtype, device=dev, seed=0)
+        if heads > 1:  # independent problems sharing the mask: [heads, n, d]
+            q, k, v = [torch.stack([syn.qkv(n, d, dtype=dtype, device=dev, seed=h)[j] for h in range(heads)])
+                       for j in range(3)]
         if name.startswith("coo"):
             import spfa_coo
             nnz = int(c.numel())
@@ -116,6 +119,11 @@ def make_workload(name, dtype, torch, syn, inline_limit=32, planned=False):
                                                                 False, plan)
             else:
                 w["call"] = lambda st: spfa_csr.forward(q, k, v, ro_t, ci_t, val, st[0], st[1], st[2], False)
+            if heads > 1 and loop_heads:  # the reference's way: one call per head
+                def looped(st):
+                    for h in range(heads):
+                        spfa_csr.forward(q[h], k[h], v[h], ro_t, ci_t, val, st[0][h], st[1][h], st[2][h], False)
+                w["call"] = looped
             w["csr"] = (ro, ci)
             off_b = 8
         gathered, total = syn.explicit_mask_bytes(nnz, n, d, es, off_bytes=off_b)
@@ -128,8 +136,9 @@ def make_workload(name, dtype, torch, syn, inline_limit=32, planned=False):
         long_rows = deg > inline_limit
         nnz_long, rows_long = int(deg[long_rows].sum()), int(long_rows.sum())
         _, kernel_bytes = syn.explicit_mask_bytes(nnz_long, rows_long, d, es, off_bytes=off_b)
-        w.update(n=n, d=d, nnz=nnz, bytes_total=total, bytes_gathered=gathered, bound="hbm",
-                 kernel_bytes=kernel_bytes, kernel_nnz=nnz_long, kernel_rows=rows_long)
+        w.update(n=n, d=d, nnz=nnz * heads, bytes_total=total * heads, bytes_gathered=gathered * heads,
+                 bound="hbm", kernel_bytes=kernel_bytes * heads, kernel_nnz=nnz_long * heads,
+                 kernel_rows=rows_long * heads)
     else:
         if name == "local":
             import spfa_local
@@ -171,7 +180,7 @@ def make_workload(name, dtype, torch, syn, inline_limit=32, planned=False):
         total = syn.implicit_mask_bytes(n, d, es, live_rows=live)
         w.update(n=n, d=d, nnz=nnz, bytes_total=total, bytes_gathered=nnz * 2 * d * es, bound="hbm",
                  kernel_bytes=total, kernel_nnz=nnz, kernel_rows=live)
-    w.update(q=q, k=k, v=v)
+    w.update(q=q, k=k, v=v, heads=heads)
     return w
 
 
@@ -181,6 +190,9 @@ def verify_sample(w, state, torch, rows=192):
     from oracle import c_oracle
     from oracle import spfa_oracle as so
     n = w["n"]
+    if w.get("heads", 1) > 1:  # a batch of heads: the last one is checked
+        w = dict(w, q=w["q"][-1], k=w["k"][-1], v=w["v"][-1])
+        state = [x[-1] for x in state]
     g = torch.Generator().manual_seed(123)
     idx = torch.sort(torch.randperm(n, generator=g)[:rows])[0]
     qs = w["q"][idx.to("cuda")].float().cpu().numpy().astype(np.float64)
@@ -330,6 +342,10 @@ def main():
     ap.add_argument("--workload", default="csr_zipf", choices=sorted(WORKLOADS))
     ap.add_argument("--dtype", default="f32", choices=["f32", "f16", "bf16"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--heads", type=int, default=1,
+                    help="csr_* workloads: this many independent problems sharing the mask, stacked [heads, n, d]")
+    ap.add_argument("--loop-heads", action="store_true",
+                    help="with --heads: one call per head (the reference's only way) instead of one batched call")
     ap.add_argument("--planned", action="store_true",
                     help="explicit masks: build the mask plan once, outside the timed region, and time "
                          "forward_planned (a mask reused across calls)")
@@ -350,14 +366,22 @@ def main():
     lib = load_library()
     if a.planned and not (a.workload.startswith("csr") or a.workload.startswith("coo")):
         sys.exit("bench.py: --planned applies to the explicit-mask workloads (csr_*, coo_*)")
-    w = make_workload(a.workload, dtype, torch, syn, int(lib.spfa_explicit_inline_row_limit()), a.planned)
+    if a.heads > 1 and not a.workload.startswith("csr"):
+        sys.exit("bench.py: --heads applies to the csr_* workloads")
+    w = make_workload(a.workload, dtype, torch, syn, int(lib.spfa_explicit_inline_row_limit()), a.planned,
+                      max(1, a.heads), a.loop_heads)
     n, d, nnz = w["n"], w["d"], w["nnz"]
 
     n_states = a.steps + a.warmup
-    state_bytes = n * d * torch.tensor([], dtype=dtype).element_size()
+    state_bytes = max(1, a.heads) * n * d * torch.tensor([], dtype=dtype).element_size()
     n_alloc = max(1, min(n_states, int(4e9 // max(1, state_bytes))))
-    states = [syn.fresh_state(n, d, dtype=dtype, device="cuda", state_dtype=torch.float32)
-              for _ in range(n_alloc)]
+    def new_state():
+        if a.heads > 1:
+            per = [syn.fresh_state(n, d, dtype=dtype, device="cuda", state_dtype=torch.float32)
+                   for _ in range(a.heads)]
+            return tuple(torch.stack([p[j] for p in per]) for j in range(3))
+        return syn.fresh_state(n, d, dtype=dtype, device="cuda", state_dtype=torch.float32)
+    states = [new_state() for _ in range(n_alloc)]
 
     def fresh(i):
         st = states[i % n_alloc]
@@ -437,7 +461,9 @@ def main():
         "dtype": a.dtype, "data": "synthetic",
         "config": {"workload": w["desc"], "n": n, "d": d, "nnz": nnz, "seed": 0,
                    "index_dtypes": "uint64 offsets / uint32 columns", "state": "fresh m=-inf l=0 each step",
-                   "mask_plan": "reused (built outside the timed region)" if a.planned else "rebuilt every call"},
+                   "mask_plan": "reused (built outside the timed region)" if a.planned else "rebuilt every call",
+                   "heads": max(1, a.heads),
+                   "heads_call": ("one call per head" if a.loop_heads else "one batched call") if a.heads > 1 else "single"},
         "effective_gathered_GBs": w["bytes_gathered"] / (ms_per_step * 1e-3) / 1e9,
         "algorithmic_GBs": w["bytes_total"] / (ms_per_step * 1e-3) / 1e9,
         "roofline": roofline,

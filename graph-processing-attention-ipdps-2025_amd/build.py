@@ -112,16 +112,17 @@ def _source_loop_depth(kname: str) -> int:
         # key-tile loop; the global-columns mode (third template argument 2) also loops over
         # query tiles
         return 2 if re.search(r"Li2EEEv", kname) else 1
-    if "15segments_kernelI" not in kname and "11rows_kernelI" not in kname:
+    med = "18medium_rows_kernelI" in kname
+    if "15segments_kernelI" not in kname and "11rows_kernelI" not in kname and not med:
         return 1
     seg = "15segments_kernelI" in kname
     m = re.search(r"6VecLayI\w+?Li(\d+)E", kname)
     if m:
-        lpr, unroll = int(m.group(1)), (16 if seg else 4)
+        lpr, unroll = int(m.group(1)), (16 if seg else 8 if med else 4)
     else:
         m = re.search(r"6GenLayI\w+?Li(\d+)E", kname)
         lpr, unroll = 64, (8 if int(m.group(1)) <= 2 else 2)
-    span = 64 if seg else lpr
+    span = 64 if (seg or med) else lpr
     groups = span // lpr
     unroll = min(unroll, span // groups)
     parts = span // (unroll * groups)

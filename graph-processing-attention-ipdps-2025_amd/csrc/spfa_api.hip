@@ -30,13 +30,20 @@ inline int64_t pick_segment(int64_t nnz_long) {
   return seg;
 }
 
-constexpr int64_t kExplicitInlineRowLimit = 32;
+#ifndef SPFA_TUNE_SHORT_MAX
+#define SPFA_TUNE_SHORT_MAX 32
+#endif
+constexpr int64_t kExplicitInlineRowLimit = SPFA_TUNE_SHORT_MAX;
 
 EngineSizing size_csr(int64_t n_q, int64_t nnz) {
   EngineSizing s{};
   s.nnz_bound = nnz;
   s.max_deg = nnz;
   s.short_max = kExplicitInlineRowLimit;
+#ifndef SPFA_TUNE_MEDIUM_MAX
+#define SPFA_TUNE_MEDIUM_MAX 256
+#endif
+  s.medium_max = SPFA_TUNE_MEDIUM_MAX;
   s.seg = pick_segment(nnz);
   s.n_long_bound = n_q;
   return s;
@@ -79,7 +86,7 @@ EngineSizing size_global(int64_t n, int64_t n_globs) {
 
 int check_problem(const spfa_problem_t* p) {
   if (p == nullptr) return SPFA_ERR_BAD_ARG;
-  if (p->n_q < 0 || p->n_k < 0) return SPFA_ERR_BAD_ARG;
+  if (p->n_q < 0 || p->n_k < 0 || p->n_batch < 0) return SPFA_ERR_BAD_ARG;
   if (p->n_q >= (int64_t)1 << 31 || p->n_k >= (int64_t)1 << 31) return SPFA_ERR_BAD_ARG;
   if (p->d < 1 || p->d > 1024) return SPFA_ERR_EMB_TOO_LARGE;
   return SPFA_OK;
@@ -110,7 +117,28 @@ Tensors make_tensors(const spfa_problem_t* p) {
   t.n_q = p->n_q;
   t.d = (int32_t)p->d;
   t.state_f32 = (p->state_dtype == SPFA_DTYPE_F32) ? 1 : 0;
+  t.n_batch = p->n_batch > 1 ? p->n_batch : 1;
+  t.kv_stride = p->n_k * p->d;
   return t;
+}
+
+int64_t batch_of(const spfa_problem_t* p) { return p->n_batch > 1 ? p->n_batch : 1; }
+
+size_t elem_bytes(int dtype) { return dtype == SPFA_DTYPE_F32 ? 4 : 2; }
+
+// Problem b of a batch as a problem of its own (the paths without batched kernels walk the batch
+// on the host, one problem after the other on the same stream and workspace).
+spfa_problem_t batch_slice(const spfa_problem_t* p, int64_t b) {
+  spfa_problem_t s = *p;
+  const size_t es = elem_bytes(p->dtype), ss = elem_bytes(p->state_dtype);
+  s.q = (const char*)p->q + (size_t)b * p->n_q * p->d * es;
+  s.k = (const char*)p->k + (size_t)b * p->n_k * p->d * es;
+  s.v = (const char*)p->v + (size_t)b * p->n_k * p->d * es;
+  s.out = (char*)p->out + (size_t)b * p->n_q * p->d * es;
+  s.m = (char*)p->m + (size_t)b * p->n_q * ss;
+  s.l = (char*)p->l + (size_t)b * p->n_q * ss;
+  s.n_batch = 1;
+  return s;
 }
 
 int dispatch_csr(const spfa_problem_t* p, const CsrMask& mask, const EngineSizing& s, int use_nan,
@@ -131,7 +159,16 @@ int build_work_list(int64_t n_q, const CsrMask& mask, const EngineSizing& s, voi
   Tensors t{};
   t.n_q = n_q;
   t.d = 64;
+  t.n_batch = 1;
   return run_csr<float>(t, mask, s, 0, plan_buf, stream, kEnginePlanOnly, nullptr);
+}
+
+// The batched engine counts work items of all problems in one 32-bit cursor.
+bool batch_fits_engine(const EngineSizing& s, const spfa_problem_t* p) {
+  const int64_t b = batch_of(p);
+  if (b == 1) return true;
+  const WorkspaceLayout w = engine_workspace(s, p->n_q, p->d, 1);
+  return (int64_t)w.cap_items * b < ((int64_t)1 << 32) - 1 && p->n_q * b < ((int64_t)1 << 40);
 }
 
 size_t work_list_bytes(int64_t n_q, int64_t nnz) {
@@ -248,7 +285,7 @@ extern "C" {
 
 int spfa_version(void) { return 1; }
 
-int64_t spfa_explicit_inline_row_limit(void) { return kExplicitInlineRowLimit; }
+int64_t spfa_explicit_inline_row_limit(void) { return SPFA_TUNE_MEDIUM_MAX; }
 
 void spfa_set_kernel_events(void* start, void* stop) {
   kernel_events().start = (hipEvent_t)start;
@@ -294,7 +331,17 @@ int spfa_csr_forward(const spfa_problem_t* p, const void* row_off, int row_off_b
   if (p->n_q == 0) return SPFA_OK;
   if (!row_off || (nnz > 0 && !col_ind)) return SPFA_ERR_BAD_ARG;
   EngineSizing s = size_csr(p->n_q, nnz);
-  rc = check_workspace(workspace, workspace_bytes, engine_workspace(s, p->n_q, p->d).total);
+  if (!batch_fits_engine(s, p)) {
+    for (int64_t b = 0; b < batch_of(p); b++) {
+      const spfa_problem_t one = batch_slice(p, b);
+      rc = spfa_csr_forward(&one, row_off, row_off_bytes, col_ind, nnz, use_nan, workspace,
+                            workspace_bytes, stream);
+      if (rc) return rc;
+    }
+    return SPFA_OK;
+  }
+  rc = check_workspace(workspace, workspace_bytes,
+                       engine_workspace(s, p->n_q, p->d, batch_of(p)).total);
   if (rc) return rc;
   CsrMask mask{row_off, (const uint32_t*)col_ind, row_off_bytes == 8 ? 1 : 0, nullptr, nullptr};
   return dispatch_csr(p, mask, s, use_nan ? 1 : 0, workspace, (hipStream_t)stream);
@@ -331,7 +378,17 @@ int spfa_csr_forward_planned(const spfa_problem_t* p, const void* row_off, int r
   EngineSizing s = size_csr(p->n_q, nnz);
   rc = check_workspace(plan, plan_bytes, work_list_bytes(p->n_q, nnz));
   if (rc) return rc;
-  rc = check_workspace(workspace, workspace_bytes, engine_workspace(s, p->n_q, p->d).total);
+  if (!batch_fits_engine(s, p)) {
+    for (int64_t b = 0; b < batch_of(p); b++) {
+      const spfa_problem_t one = batch_slice(p, b);
+      rc = spfa_csr_forward_planned(&one, row_off, row_off_bytes, col_ind, nnz, use_nan, plan,
+                                    plan_bytes, workspace, workspace_bytes, stream);
+      if (rc) return rc;
+    }
+    return SPFA_OK;
+  }
+  rc = check_workspace(workspace, workspace_bytes,
+                       engine_workspace(s, p->n_q, p->d, batch_of(p)).total);
   if (rc) return rc;
   CsrMask mask{row_off, (const uint32_t*)col_ind, row_off_bytes == 8 ? 1 : 0, nullptr, nullptr};
   return dispatch_csr(p, mask, s, use_nan ? 1 : 0, workspace, (hipStream_t)stream, kEngineRunOnly,
@@ -358,8 +415,9 @@ int spfa_coo_forward(const spfa_problem_t* p, const void* row_ind, int row_ind_b
   if (nnz > 0 && (!row_ind || !col_ind)) return SPFA_ERR_BAD_ARG;
   EngineSizing s = size_csr(p->n_q, nnz);
   const size_t coo_bytes = coo_workspace(p->n_q, nnz).total;
+  const bool batched = batch_fits_engine(s, p);
   rc = check_workspace(workspace, workspace_bytes,
-                       coo_bytes + engine_workspace(s, p->n_q, p->d).total);
+                       coo_bytes + engine_workspace(s, p->n_q, p->d, batched ? batch_of(p) : 1).total);
   if (rc) return rc;
   CooCsr csr{};
   const CooWorkspace cw = coo_workspace(p->n_q, nnz);
@@ -367,6 +425,15 @@ int spfa_coo_forward(const spfa_problem_t* p, const void* row_ind, int row_ind_b
                   workspace, (char*)workspace + cw.keep_total, (hipStream_t)stream, &csr);
   if (rc) return rc;
   CsrMask mask{csr.row_off, (const uint32_t*)col_ind, 0, csr.cols, csr.unsorted};
+  if (!batched) {  // one conversion, then problem after problem
+    for (int64_t b = 0; b < batch_of(p); b++) {
+      const spfa_problem_t one = batch_slice(p, b);
+      rc = dispatch_csr(&one, mask, s, use_nan ? 1 : 0, (char*)workspace + coo_bytes,
+                        (hipStream_t)stream);
+      if (rc) return rc;
+    }
+    return SPFA_OK;
+  }
   return dispatch_csr(p, mask, s, use_nan ? 1 : 0, (char*)workspace + coo_bytes,
                       (hipStream_t)stream);
 }
@@ -418,7 +485,17 @@ int spfa_coo_forward_planned(const spfa_problem_t* p, const void* col_ind, int64
   const CooWorkspace w = coo_workspace(p->n_q, nnz);
   rc = check_workspace(plan, plan_bytes, w.keep_total + work_list_bytes(p->n_q, nnz));
   if (rc) return rc;
-  rc = check_workspace(workspace, workspace_bytes, engine_workspace(s, p->n_q, p->d).total);
+  if (!batch_fits_engine(s, p)) {
+    for (int64_t b = 0; b < batch_of(p); b++) {
+      const spfa_problem_t one = batch_slice(p, b);
+      rc = spfa_coo_forward_planned(&one, col_ind, nnz, use_nan, plan, plan_bytes, workspace,
+                                    workspace_bytes, stream);
+      if (rc) return rc;
+    }
+    return SPFA_OK;
+  }
+  rc = check_workspace(workspace, workspace_bytes,
+                       engine_workspace(s, p->n_q, p->d, batch_of(p)).total);
   if (rc) return rc;
   const char* pb = (const char*)plan;
   CsrMask mask{pb + w.off_row_off, (const uint32_t*)col_ind, 0, (const uint32_t*)(pb + w.off_cols),
@@ -450,6 +527,14 @@ int spfa_local_1d_dilated_forward(const spfa_problem_t* p, int64_t local_size, i
                                   void* workspace, size_t workspace_bytes, void* stream) {
   int rc = check_problem(p);
   if (rc) return rc;
+  if (batch_of(p) > 1) {  // no batched kernels on this path yet: one problem after the other
+    for (int64_t b = 0; b < batch_of(p); b++) {
+      const spfa_problem_t one = batch_slice(p, b);
+      rc = spfa_local_1d_dilated_forward(&one, local_size, dil_factor, workspace, workspace_bytes, stream);
+      if (rc) return rc;
+    }
+    return SPFA_OK;
+  }
   if (local_size < 0 || local_size > p->n_q - 1) return SPFA_ERR_LOCAL_SIZE;
   if (dil_factor < 0) return SPFA_ERR_DILATION_NEG;
   if (dil_factor >= (int64_t)1 << 31) return SPFA_ERR_BAD_ARG;
@@ -484,6 +569,15 @@ int spfa_local_2d_dilated_forward(const spfa_problem_t* p, int64_t block_size, i
                                   void* stream) {
   int rc = check_problem(p);
   if (rc) return rc;
+  if (batch_of(p) > 1) {  // no batched kernels on this path yet: one problem after the other
+    for (int64_t b = 0; b < batch_of(p); b++) {
+      const spfa_problem_t one = batch_slice(p, b);
+      rc = spfa_local_2d_dilated_forward(&one, block_size, dil_factor, use_nan, workspace,
+                                         workspace_bytes, stream);
+      if (rc) return rc;
+    }
+    return SPFA_OK;
+  }
   if (block_size <= 0 || p->n_q % block_size != 0) return SPFA_ERR_BLOCK_DIVISOR;
   if (dil_factor < 0) return SPFA_ERR_DILATION_NEG;
   if (block_size / (dil_factor + 1) < 1) return SPFA_ERR_BLOCK_DILATION;
@@ -517,6 +611,15 @@ int spfa_global_no_local_forward(const spfa_problem_t* p, const int32_t* global_
                                  size_t workspace_bytes, void* stream) {
   int rc = check_problem(p);
   if (rc) return rc;
+  if (batch_of(p) > 1) {  // no batched kernels on this path yet: one problem after the other
+    for (int64_t b = 0; b < batch_of(p); b++) {
+      const spfa_problem_t one = batch_slice(p, b);
+      rc = spfa_global_no_local_forward(&one, global_inds, n_globals, local_size, workspace,
+                                        workspace_bytes, stream);
+      if (rc) return rc;
+    }
+    return SPFA_OK;
+  }
   if (n_globals <= 0 || n_globals > p->n_q) return SPFA_ERR_GLOBAL_COUNT;
   if (local_size < 0 || local_size > p->n_q - 1) return SPFA_ERR_LOCAL_SIZE;
   rc = check_pointers(p);

@@ -29,10 +29,24 @@ struct Tensors {
   void* m;
   void* l;
   void* out;
-  int64_t n_q;
+  int64_t n_q;        // rows of one problem
   int32_t d;
   int32_t state_f32;
+  // batch of independent problems that share the mask: q, out are [n_batch, n_q, d], m, l
+  // [n_batch, n_q], k, v [n_batch, n_k, d]
+  int64_t n_batch;    // >= 1
+  int64_t kv_stride;  // n_k * d, elements between the K (V) tensors of two problems
 };
+
+// Row r of the stacked problems is row i of problem b.
+__device__ __forceinline__ void split_row(const Tensors& t, int64_t r, int64_t& b, int64_t& i) {
+  b = 0;
+  i = r;
+  if (t.n_batch > 1) {
+    b = r / t.n_q;
+    i = r - b * t.n_q;
+  }
+}
 
 struct Counters {
   uint32_t n_items;
@@ -40,7 +54,8 @@ struct Counters {
   uint32_t n_multi;
   uint32_t next_item;
   uint32_t overflow;
-  uint32_t pad[3];
+  uint32_t n_medium;
+  uint32_t pad[2];
 };
 
 struct Item {
@@ -63,14 +78,17 @@ struct Plan {
                      // be shared by calls that each bring their own scratch)
   Item* items;
   MultiRow* multi;
+  int32_t* medium;   // rows with short_max < deg <= medium_max: one wavefront each, no queue
   float* pm;
   float* pl;
   float* pacc;
   uint32_t cap_items;
   uint32_t cap_partials;
   uint32_t cap_multi;
+  uint32_t cap_medium;
   int32_t use_nan;
   int64_t short_max;
+  int64_t medium_max;  // == short_max: no medium rows
   int64_t seg;
 };
 
@@ -85,6 +103,7 @@ static __global__ void reset_counters_kernel(Counters* cnt) {
     cnt->n_multi = 0;
     cnt->next_item = 0;
     cnt->overflow = 0;
+    cnt->n_medium = 0;
   }
 }
 
@@ -263,31 +282,35 @@ constexpr int kPlanThreads = 1024;
 template <class Mask>
 __global__ __launch_bounds__(kPlanThreads) void plan_kernel(int64_t n_q, Mask mask, Plan plan) {
   constexpr int NW = kPlanThreads / kWave;
-  __shared__ uint32_t wave_tot[NW][3];
-  __shared__ uint32_t block_base[3];
+  __shared__ uint32_t wave_tot[NW][4];
+  __shared__ uint32_t block_base[4];
   __shared__ uint32_t block_ok;
   const int lane = lane_id();
   const int wave = threadIdx.x / kWave;
   const int64_t row = (int64_t)blockIdx.x * kPlanThreads + threadIdx.x;
   int64_t deg = 0;
   if (row < n_q) deg = mask.row(row).deg;
-  const bool is_long = deg > plan.short_max;
+  const bool is_medium = deg > plan.short_max && deg <= plan.medium_max;
+  const bool is_long = deg > plan.medium_max;
   const uint32_t nseg = is_long ? (uint32_t)((deg + plan.seg - 1) / plan.seg) : 0u;
   const uint32_t multi = nseg > 1 ? 1u : 0u;
   const uint32_t npart = multi ? nseg : 0u;
+  const uint32_t med = is_medium ? 1u : 0u;
   const uint32_t inc_items = wave_inclusive_sum(nseg, lane);
   const uint32_t inc_part = wave_inclusive_sum(npart, lane);
   const uint32_t inc_multi = wave_inclusive_sum(multi, lane);
+  const uint32_t inc_med = wave_inclusive_sum(med, lane);
   if (lane == kWave - 1) {
     wave_tot[wave][0] = inc_items;
     wave_tot[wave][1] = inc_part;
     wave_tot[wave][2] = inc_multi;
+    wave_tot[wave][3] = inc_med;
   }
   __syncthreads();
   if (threadIdx.x == 0) {
-    uint32_t tot[3] = {0u, 0u, 0u};
+    uint32_t tot[4] = {0u, 0u, 0u, 0u};
     for (int w = 0; w < NW; w++)
-      for (int k = 0; k < 3; k++) {
+      for (int k = 0; k < 4; k++) {
         const uint32_t x = wave_tot[w][k];
         wave_tot[w][k] = tot[k];  // exclusive prefix over the wavefronts
         tot[k] += x;
@@ -303,10 +326,19 @@ __global__ __launch_bounds__(kPlanThreads) void plan_kernel(int64_t n_q, Mask ma
         atomicOr(&plan.cnt->overflow, 1u);
       }
     }
+    if (tot[3]) {
+      block_base[3] = atomicAdd(&plan.cnt->n_medium, tot[3]);
+      if (block_base[3] + tot[3] > plan.cap_medium) {
+        ok = 0;
+        atomicOr(&plan.cnt->overflow, 1u);
+      }
+    }
     block_ok = ok;
   }
   __syncthreads();
-  if (!block_ok || !is_long) return;
+  if (!block_ok) return;
+  if (is_medium) plan.medium[block_base[3] + wave_tot[wave][3] + inc_med - 1] = (int32_t)row;
+  if (!is_long) return;
   const uint32_t my_item = block_base[0] + wave_tot[wave][0] + inc_items - nseg;
   const uint32_t my_slot = block_base[1] + wave_tot[wave][1] + inc_part - npart;
   if (multi) {
@@ -336,10 +368,12 @@ __global__ __launch_bounds__(256) void rows_kernel(Tensors t, Mask mask, Plan pl
   const int wave = threadIdx.x >> 6;
   const int g = lane / LPR;
   const int c = lane % LPR;
-  const int64_t row = ((int64_t)blockIdx.x * 4 + wave) * Lay::GROUPS + g;
-  if (row >= t.n_q) return;
+  const int64_t row = ((int64_t)blockIdx.x * 4 + wave) * Lay::GROUPS + g;  // among all problems
+  if (row >= t.n_q * t.n_batch) return;
+  int64_t b, ri;
+  split_row(t, row, b, ri);
 
-  const typename Mask::Row rc = mask.row(row);
+  const typename Mask::Row rc = mask.row(ri);
   const int64_t deg = rc.deg;
   if (deg <= 0) {
     if (plan.use_nan) {
@@ -358,8 +392,9 @@ __global__ __launch_bounds__(256) void rows_kernel(Tensors t, Mask mask, Plan pl
 #pragma unroll
     for (int e = 0; e < NE; e++) acc[e] = 0.f;
     const float scale = 1.0f / sqrtf((float)t.d);
-    attend<Lay, Mask, Lay::U_SHORT, LPR>(mask, rc, (const T*)t.k, (const T*)t.v, t.d, scale, q, 0, deg,
-                                         lane, m, l, acc);
+    attend<Lay, Mask, Lay::U_SHORT, LPR>(mask, rc, (const T*)t.k + b * t.kv_stride,
+                                         (const T*)t.v + b * t.kv_stride, t.d, scale, q, 0, deg, lane,
+                                         m, l, acc);
     finish_row<Lay>(t, row, c, m, l, acc);
   }
   // longer rows were cut into segments by plan_kernel and belong to segments_kernel
@@ -376,16 +411,24 @@ __global__ __launch_bounds__(256) void segments_kernel(Tensors t, Mask mask, Pla
   if (plan.cnt->overflow) return;
   uint32_t n_items = plan.cnt->n_items;
   if (n_items > plan.cap_items) n_items = plan.cap_items;
+  // every problem of the batch walks the same work list (the host keeps items * batch < 2^32)
+  const uint32_t n_work = n_items * (uint32_t)t.n_batch;
   const float scale = 1.0f / sqrtf((float)t.d);
 
   while (true) {
     uint32_t idx = 0;
     if (lane == 0) idx = atomicAdd(plan.cursor, 1u);
     idx = (uint32_t)__builtin_amdgcn_readfirstlane((int)idx);
-    if (idx >= n_items) break;
+    if (idx >= n_work) break;
+    uint32_t b = 0;
+    if (t.n_batch > 1) {
+      b = idx / n_items;
+      idx -= b * n_items;
+    }
     const Item it = plan.items[idx];
-    const int64_t row = it.row;
-    const typename Mask::Row rc = mask.row(row);
+    const int64_t row = (int64_t)b * t.n_q + it.row;
+    const int64_t slot = (int64_t)b * plan.cap_partials + it.slot;
+    const typename Mask::Row rc = mask.row(it.row);
     const int64_t t0 = (int64_t)it.seg * plan.seg;
     int64_t t1 = t0 + plan.seg;
     if (t1 > rc.deg) t1 = rc.deg;
@@ -395,8 +438,9 @@ __global__ __launch_bounds__(256) void segments_kernel(Tensors t, Mask mask, Pla
     float m = kNegInf, l = 0.f, acc[NE];
 #pragma unroll
     for (int e = 0; e < NE; e++) acc[e] = 0.f;
-    attend<Lay, Mask, Lay::U, kWave>(mask, rc, (const T*)t.k, (const T*)t.v, t.d, scale, q, t0, t1, lane,
-                                     m, l, acc);
+    attend<Lay, Mask, Lay::U, kWave>(mask, rc, (const T*)t.k + (int64_t)b * t.kv_stride,
+                                     (const T*)t.v + (int64_t)b * t.kv_stride, t.d, scale, q, t0, t1,
+                                     lane, m, l, acc);
 
     // butterfly over the groups of the wavefront
 #pragma unroll
@@ -413,10 +457,10 @@ __global__ __launch_bounds__(256) void segments_kernel(Tensors t, Mask mask, Pla
       if (it.slot < 0) {
         finish_row<Lay>(t, row, c, m, l, acc);
       } else {
-        Lay::store_f32(plan.pacc + (int64_t)it.slot * t.d, c, t.d, acc);
+        Lay::store_f32(plan.pacc + slot * t.d, c, t.d, acc);
         if (c == 0) {
-          plan.pm[it.slot] = m;
-          plan.pl[it.slot] = l;
+          plan.pm[slot] = m;
+          plan.pl[slot] = l;
         }
       }
     }
@@ -425,6 +469,56 @@ __global__ __launch_bounds__(256) void segments_kernel(Tensors t, Mask mask, Pla
     // optimiser from giving the lanes that wrote the statistics a back edge of their own.
     __builtin_amdgcn_wave_barrier();
   }
+}
+
+// Rows of medium length (short_max < deg <= medium_max): one wavefront per row and problem, the
+// lane groups share the row's candidates as in segments_kernel, but launched as an ordinary
+// grid.  A row of this size is a handful of dependent memory round trips and little else: in
+// the persistent kernel (one wavefront per SIMD) nothing hides them, here the other resident
+// wavefronts do.  (A device-sized grid with a stride loop instead of one wavefront per list
+// slot was measured slower: 1.02 against 0.66 ms on 64 x 4096 rows of ~83 entries.)
+template <class Lay, class Mask>
+__global__ __launch_bounds__(256) void medium_rows_kernel(Tensors t, Mask mask, Plan plan) {
+  using T = typename Lay::elem;
+  constexpr int NE = Lay::NE;
+  constexpr int LPR = Lay::LPR;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x >> 6;
+  const int g = lane / LPR;
+  const int c = lane % LPR;
+  if (plan.cnt->overflow) return;
+  uint32_t n_medium = plan.cnt->n_medium;
+  if (n_medium > plan.cap_medium) n_medium = plan.cap_medium;
+  int64_t idx = (int64_t)blockIdx.x * 4 + wave;
+  if (idx >= (int64_t)n_medium * t.n_batch) return;
+  int64_t b = 0;
+  if (t.n_batch > 1) {
+    b = idx / n_medium;
+    idx -= b * n_medium;
+  }
+  const int64_t ri = plan.medium[idx];
+  const int64_t row = b * t.n_q + ri;
+  const typename Mask::Row rc = mask.row(ri);
+  const float scale = 1.0f / sqrtf((float)t.d);
+
+  float q[NE];
+  load_q<Lay>(t, row, c, q);
+  float m = kNegInf, l = 0.f, acc[NE];
+#pragma unroll
+  for (int e = 0; e < NE; e++) acc[e] = 0.f;
+  attend<Lay, Mask, Lay::U_MEDIUM, kWave>(mask, rc, (const T*)t.k + b * t.kv_stride,
+                                          (const T*)t.v + b * t.kv_stride, t.d, scale, q, 0, rc.deg,
+                                          lane, m, l, acc);
+#pragma unroll
+  for (int off = LPR; off < kWave; off <<= 1) {
+    float m2 = shfl_xor_f32(m, off);
+    float l2 = shfl_xor_f32(l, off);
+    float acc2[NE];
+#pragma unroll
+    for (int e = 0; e < NE; e++) acc2[e] = shfl_xor_f32(acc[e], off);
+    merge_partial<NE>(m, l, acc, m2, l2, acc2);
+  }
+  if (g == 0) finish_row<Lay>(t, row, c, m, l, acc);
 }
 
 template <class Lay>
@@ -438,19 +532,24 @@ __global__ __launch_bounds__(256) void merge_kernel(Tensors t, Plan plan) {
   if (plan.cnt->overflow) return;
   uint32_t n_multi = plan.cnt->n_multi;
   if (n_multi > plan.cap_multi) n_multi = plan.cap_multi;
-  const int64_t idx = ((int64_t)blockIdx.x * 4 + wave) * Lay::GROUPS + g;
-  if (idx >= (int64_t)n_multi) return;
+  int64_t idx = ((int64_t)blockIdx.x * 4 + wave) * Lay::GROUPS + g;
+  if (idx >= (int64_t)n_multi * t.n_batch) return;
+  int64_t b = 0;
+  if (t.n_batch > 1) {
+    b = idx / n_multi;
+    idx -= b * n_multi;
+  }
   const MultiRow mr = plan.multi[idx];
   float m = kNegInf, l = 0.f, acc[NE];
 #pragma unroll
   for (int e = 0; e < NE; e++) acc[e] = 0.f;
   for (int j = 0; j < mr.nseg; j++) {
-    const int64_t slot = (int64_t)mr.slot0 + j;
+    const int64_t slot = b * plan.cap_partials + mr.slot0 + j;
     float acc2[NE];
     Lay::load_f32(plan.pacc + slot * t.d, c, t.d, acc2);
     merge_partial<NE>(m, l, acc, plan.pm[slot], plan.pl[slot], acc2);
   }
-  finish_row<Lay>(t, mr.row, c, m, l, acc);
+  finish_row<Lay>(t, b * t.n_q + mr.row, c, m, l, acc);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -460,13 +559,14 @@ struct EngineSizing {
   int64_t nnz_bound;     // upper bound on the sum of deg over all rows
   int64_t max_deg;       // upper bound on deg of one row
   int64_t short_max;     // rows up to this many candidates are finished by rows_kernel
+  int64_t medium_max;    // rows up to this many get a wavefront of their own (0: same as short_max)
   int64_t seg;           // segment length for longer rows
   int64_t n_long_bound;  // upper bound on the number of rows with deg > short_max
 };
 
 struct WorkspaceLayout {
-  size_t off_cnt, off_items, off_multi, off_pm, off_pl, off_pacc, total;
-  uint32_t cap_items, cap_partials, cap_multi;
+  size_t off_cnt, off_items, off_multi, off_medium, off_pm, off_pl, off_pacc, total;
+  uint32_t cap_items, cap_partials, cap_multi, cap_medium;
 };
 
 
@@ -476,13 +576,15 @@ inline int64_t pow2_ceil(int64_t x) {
   return p;
 }
 
-inline WorkspaceLayout engine_workspace(const EngineSizing& s, int64_t n_q, int64_t d) {
+inline WorkspaceLayout engine_workspace(const EngineSizing& s, int64_t n_q, int64_t d,
+                                        int64_t n_batch = 1) {
   WorkspaceLayout w{};
-  int64_t cap_items = 0, cap_partials = 0, cap_multi = 0;
+  int64_t cap_items = 0, cap_partials = 0, cap_multi = 0, cap_medium = 0;
   if (s.max_deg > s.short_max) {
     int64_t n_long = s.nnz_bound / (s.short_max + 1);
     if (n_long > n_q) n_long = n_q;
     if (n_long > s.n_long_bound) n_long = s.n_long_bound;
+    if (s.medium_max > s.short_max) cap_medium = n_long + 1;
     cap_items = s.nnz_bound / s.seg + n_long + 1;
     int64_t n_multi = s.nnz_bound / (s.seg + 1);
     if (n_multi > n_long) n_multi = n_long;
@@ -492,13 +594,17 @@ inline WorkspaceLayout engine_workspace(const EngineSizing& s, int64_t n_q, int6
   w.cap_items = (uint32_t)cap_items;
   w.cap_partials = (uint32_t)cap_partials;
   w.cap_multi = (uint32_t)cap_multi;
+  w.cap_medium = (uint32_t)cap_medium;
   size_t off = 0;
   w.off_cnt = off;      off = align_up(off + sizeof(Counters), 256);
   w.off_items = off;    off = align_up(off + (size_t)cap_items * sizeof(Item), 256);
   w.off_multi = off;    off = align_up(off + (size_t)cap_multi * sizeof(MultiRow), 256);
-  w.off_pm = off;       off = align_up(off + (size_t)cap_partials * sizeof(float), 256);
-  w.off_pl = off;       off = align_up(off + (size_t)cap_partials * sizeof(float), 256);
-  w.off_pacc = off;     off = align_up(off + (size_t)cap_partials * (size_t)d * sizeof(float), 256);
+  w.off_medium = off;   off = align_up(off + (size_t)cap_medium * sizeof(int32_t), 256);
+  // (the work list is shared by the problems of a batch, the partial results are not)
+  const size_t nb = (size_t)(n_batch > 1 ? n_batch : 1);
+  w.off_pm = off;       off = align_up(off + nb * (size_t)cap_partials * sizeof(float), 256);
+  w.off_pl = off;       off = align_up(off + nb * (size_t)cap_partials * sizeof(float), 256);
+  w.off_pacc = off;     off = align_up(off + nb * (size_t)cap_partials * (size_t)d * sizeof(float), 256);
   w.total = off;
   return w;
 }
@@ -533,13 +639,14 @@ enum { kEngineAll = 0, kEnginePlanOnly = 1, kEngineRunOnly = 2 };
 template <class Lay, class Mask>
 int launch_engine(const Tensors& t, const Mask& mask, const EngineSizing& s, int use_nan, void* ws,
                   hipStream_t stream, int phase = kEngineAll, const void* plan_buf = nullptr) {
-  WorkspaceLayout w = engine_workspace(s, t.n_q, t.d);
+  WorkspaceLayout w = engine_workspace(s, t.n_q, t.d, t.n_batch);
   char* base = (char*)ws;
   char* pbase = (phase == kEngineRunOnly) ? (char*)const_cast<void*>(plan_buf) : base;
   Plan plan{};
   plan.cnt = (Counters*)(pbase + w.off_cnt);
   plan.items = (Item*)(pbase + w.off_items);
   plan.multi = (MultiRow*)(pbase + w.off_multi);
+  plan.medium = (int32_t*)(pbase + w.off_medium);
   plan.cursor = &((Counters*)(base + w.off_cnt))->next_item;
   plan.pm = (float*)(base + w.off_pm);
   plan.pl = (float*)(base + w.off_pl);
@@ -547,8 +654,10 @@ int launch_engine(const Tensors& t, const Mask& mask, const EngineSizing& s, int
   plan.cap_items = w.cap_items;
   plan.cap_partials = w.cap_partials;
   plan.cap_multi = w.cap_multi;
+  plan.cap_medium = w.cap_medium;
   plan.use_nan = use_nan;
   plan.short_max = s.short_max;
+  plan.medium_max = s.medium_max > s.short_max ? s.medium_max : s.short_max;
   plan.seg = s.seg;
   if (t.n_q == 0) return 0;
 
@@ -565,24 +674,29 @@ int launch_engine(const Tensors& t, const Mask& mask, const EngineSizing& s, int
   const KernelEvents ev = kernel_events();
   const bool timed = ev.start != nullptr && ev.stop != nullptr;
   const int64_t rows_per_wg = 4 * Lay::GROUPS;
-  const int64_t grid1 = (t.n_q + rows_per_wg - 1) / rows_per_wg;
+  const int64_t grid1 = (t.n_q * t.n_batch + rows_per_wg - 1) / rows_per_wg;
   if (timed && !has_long) (void)hipEventRecord(ev.start, stream);
   hipLaunchKernelGGL((rows_kernel<Lay, Mask>), dim3((unsigned)grid1), dim3(256), 0, stream, t, mask,
                      plan);
   if (timed && !has_long) (void)hipEventRecord(ev.stop, stream);
+  if (has_long && w.cap_medium > 0) {
+    const int64_t gridm = ((int64_t)w.cap_medium * t.n_batch + 3) / 4;
+    hipLaunchKernelGGL((medium_rows_kernel<Lay, Mask>), dim3((unsigned)gridm), dim3(256), 0, stream, t,
+                       mask, plan);
+  }
   if (has_long) {
         // One workgroup (one wavefront per SIMD) per CU with 16 neighbours in flight per lane group
     // is the fastest shape measured: more resident wavefronts only add contention in the
     // vector L1 (8 workgroups per CU: 0.98 ms at the 12.8 M-position Zipf mask, 1: 0.79 ms).
     int64_t grid2 = (int64_t)device_cu_count() * kSegmentWorkgroupsPerCu;
-    int64_t need = ((int64_t)w.cap_items + 3) / 4;
+    int64_t need = ((int64_t)w.cap_items * t.n_batch + 3) / 4;
     if (grid2 > need) grid2 = need;
     if (grid2 < 1) grid2 = 1;
     if (timed) (void)hipEventRecord(ev.start, stream);
     hipLaunchKernelGGL((segments_kernel<Lay, Mask>), dim3((unsigned)grid2), dim3(256), 0, stream, t,
                        mask, plan);
     if (timed) (void)hipEventRecord(ev.stop, stream);
-    const int64_t grid3 = ((int64_t)w.cap_multi + rows_per_wg - 1) / rows_per_wg;
+    const int64_t grid3 = ((int64_t)w.cap_multi * t.n_batch + rows_per_wg - 1) / rows_per_wg;
     hipLaunchKernelGGL((merge_kernel<Lay>), dim3((unsigned)grid3), dim3(256), 0, stream, t, plan);
   }
   return hipGetLastError() == hipSuccess ? 0 : 4;

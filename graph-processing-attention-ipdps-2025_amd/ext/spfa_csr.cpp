@@ -20,7 +20,7 @@ torch::Tensor spfa_csr_forward_py(torch::Tensor Q, torch::Tensor K, torch::Tenso
 
   c10::DeviceGuard guard(Q.device());
   spfa_problem_t p = spfa_ext::make_problem(Q, K, V, m, l, O);
-  TORCH_CHECK(W_row_off.dim() == 1 && W_row_off.size(0) == Q.size(0) + 1,
+  TORCH_CHECK(W_row_off.dim() == 1 && W_row_off.size(0) == p.n_q + 1,
               "W_row_off must hold rows+1 offsets");
   TORCH_CHECK(W_col_ind.dim() == 1, "W_col_ind must be 1-D");
   // the value vector is type-checked and otherwise unused, as in the reference kernel
@@ -29,7 +29,7 @@ torch::Tensor spfa_csr_forward_py(torch::Tensor Q, torch::Tensor K, torch::Tenso
   spfa_ext::index_bytes(W_col_ind, "W_col_ind", false);
   const int64_t nnz = W_col_ind.size(0);
 
-  const size_t ws_bytes = spfa_csr_workspace_bytes(p.n_q, nnz, p.d, p.dtype);
+  const size_t ws_bytes = spfa_ext::batched(spfa_csr_workspace_bytes(p.n_q, nnz, p.d, p.dtype), p);
   torch::Tensor ws = spfa_ext::make_workspace(ws_bytes, Q);
   spfa_ext::raise_on_error(spfa_csr_forward(&p, W_row_off.data_ptr(), off_bytes, W_col_ind.data_ptr(),
                                             nnz, use_nan ? 1 : 0, ws.data_ptr(), (size_t)ws.numel(),
@@ -73,7 +73,7 @@ torch::Tensor spfa_csr_forward_planned_py(torch::Tensor Q, torch::Tensor K, torc
 
   c10::DeviceGuard guard(Q.device());
   spfa_problem_t p = spfa_ext::make_problem(Q, K, V, m, l, O);
-  TORCH_CHECK(W_row_off.dim() == 1 && W_row_off.size(0) == Q.size(0) + 1,
+  TORCH_CHECK(W_row_off.dim() == 1 && W_row_off.size(0) == p.n_q + 1,
               "W_row_off must hold rows+1 offsets");
   TORCH_CHECK(W_col_ind.dim() == 1, "W_col_ind must be 1-D");
   TORCH_CHECK(W_val.scalar_type() == Q.scalar_type(), "W_val must have the dtype of Q");
@@ -82,7 +82,7 @@ torch::Tensor spfa_csr_forward_planned_py(torch::Tensor Q, torch::Tensor K, torc
   spfa_ext::index_bytes(W_col_ind, "W_col_ind", false);
   const int64_t nnz = W_col_ind.size(0);
 
-  const size_t ws_bytes = spfa_csr_workspace_bytes(p.n_q, nnz, p.d, p.dtype);
+  const size_t ws_bytes = spfa_ext::batched(spfa_csr_workspace_bytes(p.n_q, nnz, p.d, p.dtype), p);
   torch::Tensor ws = spfa_ext::make_workspace(ws_bytes, Q);
   spfa_ext::raise_on_error(spfa_csr_forward_planned(
       &p, W_row_off.data_ptr(), off_bytes, W_col_ind.data_ptr(), nnz, use_nan ? 1 : 0, plan.data_ptr(),

@@ -43,16 +43,25 @@ inline int index_bytes(const torch::Tensor& t, const char* name, bool allow_wide
   return 0;
 }
 
+// Q, K, V, O are [tokens, embedding] as in the reference, or carry leading batch dimensions
+// ([batch, tokens, embedding], [batch, heads, tokens, embedding], ...) with m and l shaped like
+// Q without its last dimension: independent problems that share the mask.
 inline spfa_problem_t make_problem(const torch::Tensor& Q, const torch::Tensor& K,
                                    const torch::Tensor& V, const torch::Tensor& m,
                                    const torch::Tensor& l, const torch::Tensor& O) {
-  TORCH_CHECK(Q.dim() == 2 && K.dim() == 2 && V.dim() == 2 && O.dim() == 2,
-              "Q, K, V and O must be 2-D [tokens, embedding]");
-  TORCH_CHECK(m.dim() == 1 && l.dim() == 1, "m and l must be 1-D [tokens]");
-  TORCH_CHECK(K.size(1) == Q.size(1) && V.size(1) == Q.size(1) && O.size(1) == Q.size(1),
+  const int64_t nd = Q.dim();
+  TORCH_CHECK(nd >= 2 && K.dim() == nd && V.dim() == nd && O.dim() == nd,
+              "Q, K, V and O must be [tokens, embedding], optionally with the same leading batch dimensions");
+  TORCH_CHECK(m.dim() == nd - 1 && l.dim() == nd - 1, "m and l must be shaped like Q without its last dimension");
+  for (int64_t i = 0; i + 2 < nd; i++)
+    TORCH_CHECK(K.size(i) == Q.size(i) && V.size(i) == Q.size(i) && O.size(i) == Q.size(i) &&
+                    m.size(i) == Q.size(i) && l.size(i) == Q.size(i),
+                "all tensors must share the leading batch dimensions");
+  const int64_t rq = nd - 2, rd = nd - 1;
+  TORCH_CHECK(K.size(rd) == Q.size(rd) && V.size(rd) == Q.size(rd) && O.size(rd) == Q.size(rd),
               "Q, K, V and O must share the embedding dimension");
-  TORCH_CHECK(K.size(0) == V.size(0), "K and V must have the same number of rows");
-  TORCH_CHECK(O.size(0) == Q.size(0) && m.size(0) == Q.size(0) && l.size(0) == Q.size(0),
+  TORCH_CHECK(K.size(rq) == V.size(rq), "K and V must have the same number of rows");
+  TORCH_CHECK(O.size(rq) == Q.size(rq) && m.size(rq) == Q.size(rq) && l.size(rq) == Q.size(rq),
               "O, m and l must have one row per row of Q");
   TORCH_CHECK(K.scalar_type() == Q.scalar_type() && V.scalar_type() == Q.scalar_type() &&
                   O.scalar_type() == Q.scalar_type(),
@@ -63,6 +72,8 @@ inline spfa_problem_t make_problem(const torch::Tensor& Q, const torch::Tensor& 
   TORCH_CHECK(K.device() == Q.device() && V.device() == Q.device() && O.device() == Q.device() &&
                   m.device() == Q.device() && l.device() == Q.device(),
               "all tensors must be on the same device");
+  int64_t batch = 1;
+  for (int64_t i = 0; i + 2 < nd; i++) batch *= Q.size(i);
   spfa_problem_t p;
   p.q = Q.data_ptr();
   p.k = K.data_ptr();
@@ -70,12 +81,18 @@ inline spfa_problem_t make_problem(const torch::Tensor& Q, const torch::Tensor& 
   p.m = m.data_ptr();
   p.l = l.data_ptr();
   p.out = O.data_ptr();
-  p.n_q = Q.size(0);
-  p.n_k = K.size(0);
-  p.d = Q.size(1);
+  p.n_q = Q.size(rq);
+  p.n_k = K.size(rq);
+  p.d = Q.size(rd);
   p.dtype = elem_dtype(Q);
   p.state_dtype = (m.scalar_type() == Q.scalar_type()) ? p.dtype : SPFA_DTYPE_F32;
+  p.n_batch = batch;
   return p;
+}
+
+// workspace of a (possibly batched) call: the single-problem size times the batch count
+inline size_t batched(size_t bytes, const spfa_problem_t& p) {
+  return bytes * (size_t)(p.n_batch > 1 ? p.n_batch : 1);
 }
 
 inline torch::Tensor make_workspace(size_t bytes, const torch::Tensor& like) {

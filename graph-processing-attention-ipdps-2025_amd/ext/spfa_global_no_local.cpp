@@ -17,7 +17,7 @@ torch::Tensor spfa_global_no_local_forward_py(torch::Tensor Q, torch::Tensor K, 
 
   c10::DeviceGuard guard(Q.device());
   spfa_problem_t p = spfa_ext::make_problem(Q, K, V, m, l, O);
-  TORCH_CHECK(K.size(0) == Q.size(0), "Q, K and V must have the same number of rows");
+  TORCH_CHECK(p.n_k == p.n_q, "Q, K and V must have the same number of rows");
   TORCH_CHECK(global_inds.dim() == 1, "global_inds must be 1-D");
   // the reference reads the list through an int accessor (sp_flatt_global_no_local_kernel.cu:345)
   TORCH_CHECK(global_inds.scalar_type() == torch::kInt32, "global_inds must be an int32 tensor");

@@ -16,8 +16,8 @@ torch::Tensor spfa_local_forward_py(torch::Tensor Q, torch::Tensor K, torch::Ten
 
   c10::DeviceGuard guard(Q.device());
   spfa_problem_t p = spfa_ext::make_problem(Q, K, V, m, l, O);
-  TORCH_CHECK(K.size(0) == Q.size(0), "Q, K and V must have the same number of rows");
-  const size_t ws_bytes = spfa_local_workspace_bytes(p.n_q, p.d, p.dtype, local_size_each_dir);
+  TORCH_CHECK(p.n_k == p.n_q, "Q, K and V must have the same number of rows");
+  const size_t ws_bytes = spfa_ext::batched(spfa_local_workspace_bytes(p.n_q, p.d, p.dtype, local_size_each_dir), p);
   torch::Tensor ws = spfa_ext::make_workspace(ws_bytes, Q);
   spfa_ext::raise_on_error(spfa_local_forward(&p, local_size_each_dir, ws.data_ptr(),
                                               (size_t)ws.numel(), spfa_ext::current_stream(Q)));

@@ -16,7 +16,7 @@ torch::Tensor spfa_local_2d_dilated_forward_py(torch::Tensor Q, torch::Tensor K,
 
   c10::DeviceGuard guard(Q.device());
   spfa_problem_t p = spfa_ext::make_problem(Q, K, V, m, l, O);
-  TORCH_CHECK(K.size(0) == Q.size(0), "Q, K and V must have the same number of rows");
+  TORCH_CHECK(p.n_k == p.n_q, "Q, K and V must have the same number of rows");
   const size_t ws_bytes =
       spfa_local_2d_dilated_workspace_bytes(p.n_q, p.d, p.dtype, block_size, dil_factor);
   torch::Tensor ws = spfa_ext::make_workspace(ws_bytes, Q);

@@ -72,6 +72,11 @@ typedef struct spfa_problem {
   int64_t d;           /* 1 <= d <= 1024 */
   int32_t dtype;       /* SPFA_DTYPE_* of q, k, v, out */
   int32_t state_dtype; /* SPFA_DTYPE_* of m, l: the same as dtype (reference), or F32 */
+  /* Independent problems that share the mask (batch x heads; the reference is limited to one,
+   * README.md:10).  0 or 1: a single problem.  With n_batch > 1 the tensors are stacked:
+   * q, out [n_batch, n_q, d], k, v [n_batch, n_k, d], m, l [n_batch, n_q], all contiguous; the
+   * workspace must hold n_batch times the bytes *_workspace_bytes(...) reports. */
+  int64_t n_batch;
 } spfa_problem_t;
 
 int spfa_version(void);

@@ -18,7 +18,7 @@ class Problem(ctypes.Structure):
     _fields_ = [("q", ctypes.c_void_p), ("k", ctypes.c_void_p), ("v", ctypes.c_void_p),
                 ("m", ctypes.c_void_p), ("l", ctypes.c_void_p), ("out", ctypes.c_void_p),
                 ("n_q", ctypes.c_int64), ("n_k", ctypes.c_int64), ("d", ctypes.c_int64),
-                ("dtype", ctypes.c_int32), ("state_dtype", ctypes.c_int32)]
+                ("dtype", ctypes.c_int32), ("state_dtype", ctypes.c_int32), ("n_batch", ctypes.c_int64)]
 
 
 @pytest.fixture(scope="module")

@@ -326,6 +326,96 @@ def test_csr_state_in_element_dtype(mods, dtype):
     check(o, m, l, *ref, dtype)
 
 
+# ------------------------------------------------------------------ batch x heads
+def _stacked(n, d, dtype, shape, seed, n_k=None):
+    """q, k, v with leading batch dimensions `shape`, and a fresh state."""
+    b = int(np.prod(shape))
+    qs, ks, vs = [], [], []
+    for i in range(b):
+        q, k, v = syn.qkv(n, d, dtype=dtype, device="cpu", seed=seed + i, n_k=n_k)
+        qs.append(q), ks.append(k), vs.append(v)
+    n_k = n if n_k is None else n_k
+    q = torch.stack(qs).reshape(*shape, n, d).to(DEV)
+    k = torch.stack(ks).reshape(*shape, n_k, d).to(DEV)
+    v = torch.stack(vs).reshape(*shape, n_k, d).to(DEV)
+    m = torch.full((*shape, n), -float("inf"), device=DEV, dtype=torch.float32)
+    l = torch.zeros((*shape, n), device=DEV, dtype=torch.float32)
+    o = torch.zeros((*shape, n, d), device=DEV, dtype=dtype)
+    return q, k, v, m, l, o
+
+
+def _check_heads(q, k, v, o, m, l, ref_fn, dtype, **kw):
+    n, d = q.shape[-2:]
+    qf, kf, vf = q.reshape(-1, n, d), k.reshape(-1, k.shape[-2], d), v.reshape(-1, v.shape[-2], d)
+    of, mf, lf = o.reshape(-1, n, d), m.reshape(-1, n), l.reshape(-1, n)
+    for b in range(qf.shape[0]):
+        ref = ref_fn(np64(qf[b]), np64(kf[b]), np64(vf[b]))
+        check(of[b], mf[b], lf[b], *ref, dtype, state_dtype=torch.float32, **kw)
+
+
+@pytest.mark.parametrize("dtype,shape", [(torch.float32, (3,)), (torch.bfloat16, (2, 3)), (torch.float16, (5,))])
+def test_csr_batch_of_heads_shares_the_mask(mods, dtype, shape):
+    """[batch..., tokens, embedding] tensors: every problem of the batch against the oracle; long
+    rows (segments + merge) and short rows, empty rows NaN."""
+    n, d = 3000, 64
+    ro, ci = syn.zipf_csr(n, 1.3, 0, 2500, seed=51)
+    ro_t, ci_t = csr_tensors(ro, ci)
+    q, k, v, m, l, o = _stacked(n, d, dtype, shape, 51)
+    val = torch.ones(ci_t.numel(), device=DEV, dtype=dtype)
+    ret = mods["spfa_csr"].forward(q, k, v, ro_t, ci_t, val, m, l, o, True)
+    sync()
+    assert ret.data_ptr() == o.data_ptr()
+    _check_heads(q, k, v, o, m, l,
+                 lambda a, b, c: c_oracle.csr(a, b, c, ro.numpy(), ci.numpy(), use_nan=True), dtype,
+                 dead_expect="nan")
+    # the planned call takes the same plan for any batch
+    plan = mods["spfa_csr"].plan(ro_t, ci_t)
+    q, k, v, m2, l2, o2 = q, k, v, torch.full_like(m, -float("inf")), torch.zeros_like(l), torch.zeros_like(o)
+    mods["spfa_csr"].forward_planned(q, k, v, ro_t, ci_t, val, m2, l2, o2, True, plan)
+    sync()
+    tol = 2e-5 if dtype == torch.float32 else 2e-2
+    assert torch.allclose(torch.nan_to_num(o).float(), torch.nan_to_num(o2).float(), atol=tol)
+
+
+def test_coo_batch_rectangular_keys(mods):
+    n, n_k, d = 1500, 2200, 64
+    g = torch.Generator().manual_seed(52)
+    deg = torch.randint(0, 90, (n,), generator=g)
+    deg[17] = 1800
+    ro, ci = syn.csr_from_degrees(deg, n_k, g, "cpu", force_diagonal=False)
+    r, c = syn.coo_from_csr(ro, ci, shuffle_seed=52)
+    q, k, v, m, l, o = _stacked(n, d, torch.float32, (4,), 52, n_k=n_k)
+    mods["spfa_coo"].forward(q, k, v, r.to(torch.uint64).to(DEV), c.to(torch.uint32).to(DEV),
+                             torch.ones(c.numel(), device=DEV), m, l, o, False)
+    sync()
+    _check_heads(q, k, v, o, m, l, lambda a, b, cc: c_oracle.csr(a, b, cc, ro.numpy(), ci.numpy()),
+                 torch.float32)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_implicit_masks_batch_of_heads(mods, dtype):
+    n, d = 1024, 64
+    shape = (2, 2)
+    w, dil, blk = 40, 1, 64
+    globs = [3, 500, 501, 900]
+    cases = [
+        ("spfa_local", (w,), so.mask_local_dense(n, w), None),
+        ("spfa_local_1d_dilated", (w, dil), so.mask_local_1d_dilated_dense(n, w, dil), None),
+        ("spfa_local_2d_dilated", (blk, dil, True), so.mask_local_2d_dilated_dense(n, blk, dil), "nan"),
+    ]
+    for name, args, dense, dead in cases:
+        q, k, v, m, l, o = _stacked(n, d, dtype, shape, 53)
+        mods[name].forward(q, k, v, m, l, o, *args)
+        sync()
+        _check_heads(q, k, v, o, m, l, lambda a, b, c: so.dense_masked_attention(a, b, c, dense), dtype,
+                     dead_expect=dead)
+    q, k, v, m, l, o = _stacked(n, d, dtype, shape, 54)
+    mods["spfa_global_no_local"].forward(q, k, v, m, l, o, torch.tensor(globs, dtype=torch.int32, device=DEV), w)
+    sync()
+    dense = so.mask_global_no_local_dense(n, globs, w)
+    _check_heads(q, k, v, o, m, l, lambda a, b, c: so.dense_masked_attention(a, b, c, dense), dtype)
+
+
 # ------------------------------------------------------------------ mask plans
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_csr_plan_is_reused_across_calls_and_dtypes(mods, dtype):
