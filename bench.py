@@ -432,7 +432,17 @@ def main():
     flops = syn.attention_flops(nnz, d)
     achieved_gbs = w["kernel_bytes"] / (k_avg * 1e-3) / 1e9
     explicit = a.workload.startswith(("csr", "coo"))
-    if explicit:
+    if explicit and w["kernel_nnz"] == 0:
+        # no row is long enough for the segment kernel (all of them go to the row kernels): the
+        # whole call stands in, with the call's algorithmic bytes
+        k_avg = ms_per_step
+        kernel_ms = [ms_per_step]
+        achieved_gbs = w["bytes_total"] / (ms_per_step * 1e-3) / 1e9
+        roofline = {"bound": "hbm", "achieved": achieved_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                    "frac": achieved_gbs / HBM_PEAK_GBS, "traffic": None,
+                    "kernel": "whole call (rows_kernel + medium_rows_kernel; nothing for segments_kernel)"}
+        w = dict(w, kernel_bytes=w["bytes_total"], kernel_nnz=w["nnz"], kernel_rows=w["n"] * w.get("heads", 1))
+    elif explicit:
         # gather work: bound by memory, algorithmic bytes of the segment kernel over its time
         roofline = {"bound": "hbm", "achieved": achieved_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                     "frac": achieved_gbs / HBM_PEAK_GBS, "traffic": measured_traffic(a.workload, a.dtype),

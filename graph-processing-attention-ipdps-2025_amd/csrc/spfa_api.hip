@@ -30,20 +30,19 @@ inline int64_t pick_segment(int64_t nnz_long) {
   return seg;
 }
 
-#ifndef SPFA_TUNE_SHORT_MAX
-#define SPFA_TUNE_SHORT_MAX 32
-#endif
-constexpr int64_t kExplicitInlineRowLimit = SPFA_TUNE_SHORT_MAX;
+constexpr int64_t kExplicitInlineRowLimit = 32;
+// Rows between the two limits get a wavefront of their own (medium_rows_kernel).  Measured with
+// the limit at 64 / 128 / 256 / 512: the Zipf mask (12.8 M positions) does not care (0.867-0.873
+// ms); 64 heads of the 2 % Bernoulli mask (rows of ~83) need it above their row length (3.03 ms
+// without, 0.65 with).
+constexpr int64_t kExplicitMediumRowLimit = 256;
 
 EngineSizing size_csr(int64_t n_q, int64_t nnz) {
   EngineSizing s{};
   s.nnz_bound = nnz;
   s.max_deg = nnz;
   s.short_max = kExplicitInlineRowLimit;
-#ifndef SPFA_TUNE_MEDIUM_MAX
-#define SPFA_TUNE_MEDIUM_MAX 256
-#endif
-  s.medium_max = SPFA_TUNE_MEDIUM_MAX;
+  s.medium_max = kExplicitMediumRowLimit;
   s.seg = pick_segment(nnz);
   s.n_long_bound = n_q;
   return s;
@@ -285,7 +284,7 @@ extern "C" {
 
 int spfa_version(void) { return 1; }
 
-int64_t spfa_explicit_inline_row_limit(void) { return SPFA_TUNE_MEDIUM_MAX; }
+int64_t spfa_explicit_inline_row_limit(void) { return kExplicitMediumRowLimit; }
 
 void spfa_set_kernel_events(void* start, void* stop) {
   kernel_events().start = (hipEvent_t)start;

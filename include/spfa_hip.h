@@ -90,8 +90,9 @@ const char* spfa_status_string(int status);
  * thread-safe: set it, run, read the events, reset it with NULLs. */
 void spfa_set_kernel_events(void* start, void* stop);
 
-/* Rows of an explicit mask with at most this many entries are finished by the row kernel; longer
- * rows go through the segment kernel.  Exposed so a benchmark can attribute bytes to kernels. */
+/* Rows of an explicit mask with at most this many entries are finished by the row kernels (a
+ * lane group or a wavefront per row); longer rows go through the segment kernel.  Exposed so a
+ * benchmark can attribute bytes to kernels. */
 int64_t spfa_explicit_inline_row_limit(void);
 
 /* CSR: row i attends col_ind[row_off[i] .. row_off[i+1]).  row_off has n_q+1 entries of
