@@ -206,7 +206,8 @@ int dispatch_band(const spfa_problem_t* p, int64_t w, int64_t stride, int64_t bl
   }
   a.tiles_per_sub = (len_max + 127) / 128;
   a.n_tiles = n_sub * a.tiles_per_sub;
-  if (a.n_tiles + 8 >= ((int64_t)1 << 31)) return -1;
+  if (a.n_tiles * a.t.n_batch + 8 >= ((int64_t)1 << 31)) return -1;
+  if (p->n_q * a.t.n_batch * p->d >= ((int64_t)1 << 40)) return -1;
   switch (p->dtype) {
     case SPFA_DTYPE_F32: return run_band<float>(a, use_nan, stream);
     case SPFA_DTYPE_F16: return run_band<f16>(a, use_nan, stream);
@@ -526,14 +527,6 @@ int spfa_local_1d_dilated_forward(const spfa_problem_t* p, int64_t local_size, i
                                   void* workspace, size_t workspace_bytes, void* stream) {
   int rc = check_problem(p);
   if (rc) return rc;
-  if (batch_of(p) > 1) {  // no batched kernels on this path yet: one problem after the other
-    for (int64_t b = 0; b < batch_of(p); b++) {
-      const spfa_problem_t one = batch_slice(p, b);
-      rc = spfa_local_1d_dilated_forward(&one, local_size, dil_factor, workspace, workspace_bytes, stream);
-      if (rc) return rc;
-    }
-    return SPFA_OK;
-  }
   if (local_size < 0 || local_size > p->n_q - 1) return SPFA_ERR_LOCAL_SIZE;
   if (dil_factor < 0) return SPFA_ERR_DILATION_NEG;
   if (dil_factor >= (int64_t)1 << 31) return SPFA_ERR_BAD_ARG;
@@ -541,7 +534,7 @@ int spfa_local_1d_dilated_forward(const spfa_problem_t* p, int64_t local_size, i
   if (rc) return rc;
   const int64_t n = p->n_q;
   EngineSizing s = size_stride(n, band_max_deg(n, local_size));
-  rc = check_workspace(workspace, workspace_bytes, engine_workspace(s, n, p->d).total);
+  rc = check_workspace(workspace, workspace_bytes, engine_workspace(s, n, p->d, batch_of(p)).total);
   if (rc) return rc;
   {
     const int64_t len_max = (n + dil_factor) / (dil_factor + 1);
@@ -568,15 +561,6 @@ int spfa_local_2d_dilated_forward(const spfa_problem_t* p, int64_t block_size, i
                                   void* stream) {
   int rc = check_problem(p);
   if (rc) return rc;
-  if (batch_of(p) > 1) {  // no batched kernels on this path yet: one problem after the other
-    for (int64_t b = 0; b < batch_of(p); b++) {
-      const spfa_problem_t one = batch_slice(p, b);
-      rc = spfa_local_2d_dilated_forward(&one, block_size, dil_factor, use_nan, workspace,
-                                         workspace_bytes, stream);
-      if (rc) return rc;
-    }
-    return SPFA_OK;
-  }
   if (block_size <= 0 || p->n_q % block_size != 0) return SPFA_ERR_BLOCK_DIVISOR;
   if (dil_factor < 0) return SPFA_ERR_DILATION_NEG;
   if (block_size / (dil_factor + 1) < 1) return SPFA_ERR_BLOCK_DILATION;
@@ -586,7 +570,7 @@ int spfa_local_2d_dilated_forward(const spfa_problem_t* p, int64_t block_size, i
   if (n == 0) return SPFA_OK;
   const int64_t cnt = block_live_count(block_size, dil_factor + 1);
   EngineSizing s = size_stride(n, cnt);
-  rc = check_workspace(workspace, workspace_bytes, engine_workspace(s, n, p->d).total);
+  rc = check_workspace(workspace, workspace_bytes, engine_workspace(s, n, p->d, batch_of(p)).total);
   if (rc) return rc;
   if (cnt >= kBandTileMinRow && dtype_ok(p->dtype)) {
     rc = dispatch_band(p, 0, dil_factor + 1, block_size, cnt, use_nan ? 1 : 0, (hipStream_t)stream);

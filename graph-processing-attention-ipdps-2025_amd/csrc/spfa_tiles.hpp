@@ -211,16 +211,20 @@ __global__ __launch_bounds__(256, 2) void tile_kernel(TileArgs a) {
   if constexpr (MODE == kTileBand) {
     // workgroups are dealt round-robin to the 8 XCDs: give each XCD a contiguous run of tiles
     // so that neighbouring query tiles (which share most of their keys) meet in one L2
-    const int64_t per_xcd = (a.n_tiles + 7) / 8;
-    const int64_t lt = (int64_t)(blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
-    if (lt >= a.n_tiles) return;
+    // (the tiles of all problems of a batch form one list; problem bb starts at token bb * n)
+    const int64_t n_all = a.n_tiles * a.t.n_batch;
+    const int64_t per_xcd = (n_all + 7) / 8;
+    int64_t lt = (int64_t)(blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+    if (lt >= n_all) return;
+    const int64_t bb = lt / a.n_tiles;
+    lt -= bb * a.n_tiles;
     const int64_t sub = lt / a.tiles_per_sub;
     const int64_t tile = lt - sub * a.tiles_per_sub;
     if (a.block > 0) {
-      base = sub * a.block;
+      base = sub * a.block + bb * a.n;
       qlen = a.cnt;
     } else {
-      base = sub;
+      base = sub + bb * a.n;
       qlen = (a.n - sub + a.s - 1) / a.s;
     }
     klen = qlen;
@@ -646,18 +650,22 @@ __global__ __launch_bounds__(256, 2) void band_dma_kernel(TileArgs a) {
   // Positions inside a subsequence fit 32 bits (there are fewer than 2^31 tokens); everything
   // that is the same for the whole workgroup is moved to scalar registers.
   auto uni = [](int x) { return __builtin_amdgcn_readfirstlane(x); };
-  const int64_t per_xcd = (a.n_tiles + 7) / 8;
-  const int64_t lt = (int64_t)(blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
-  if (lt >= a.n_tiles) return;
+  // (the tiles of all problems of a batch form one list; problem bb starts at token bb * n)
+  const int64_t n_all = a.n_tiles * a.t.n_batch;
+  const int64_t per_xcd = (n_all + 7) / 8;
+  int64_t lt = (int64_t)(blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+  if (lt >= n_all) return;
+  const int64_t bb = lt / a.n_tiles;
+  lt -= bb * a.n_tiles;
   const int64_t sub = lt / a.tiles_per_sub;
   const int tile = uni((int)(lt - sub * a.tiles_per_sub));
   int64_t base;
   int qlen;
   if (a.block > 0) {
-    base = sub * a.block;
+    base = sub * a.block + bb * a.n;
     qlen = (int)a.cnt;
   } else {
-    base = sub;
+    base = sub + bb * a.n;
     qlen = uni((int)((a.n - sub + a.s - 1) / a.s));
   }
   const int wlim = (int)(a.w < (int64_t)0x3fffffff ? a.w : (int64_t)0x3fffffff);  // window, clamped
@@ -905,6 +913,7 @@ __global__ __launch_bounds__(256, 2) void band_dma_kernel(TileArgs a) {
 // rows of a block mask that have no live column: out := NaN (m, l untouched)
 template <typename T>
 __global__ void band_dead_rows_kernel(T* out, int64_t n, int d, int64_t block, int64_t s) {
+  // (n: rows of all problems of a batch; the block size divides the rows of one problem)
   const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   const int64_t row = idx / d;
   if (row >= n) return;
@@ -989,7 +998,7 @@ int launch_band_tiles(const TileArgs& a, int use_nan, hipStream_t stream) {
   const KernelEvents ev = kernel_events();
   const bool timed = ev.start != nullptr && ev.stop != nullptr;
   if (a.n_tiles > 0) {
-    const int64_t grid = (a.n_tiles + 7) / 8 * 8;
+    const int64_t grid = (a.n_tiles * a.t.n_batch + 7) / 8 * 8;
     if (timed) (void)hipEventRecord(ev.start, stream);
     if constexpr (sizeof(T) == 2) {
       // the direct-to-LDS kernel addresses a tile's rows with 32-bit offsets
@@ -1006,9 +1015,10 @@ int launch_band_tiles(const TileArgs& a, int use_nan, hipStream_t stream) {
     if (timed) (void)hipEventRecord(ev.stop, stream);
   }
   if (a.block > 0 && use_nan && a.s > 1) {
-    const int64_t total = a.n * D;
+    const int64_t rows = a.n * a.t.n_batch;
+    const int64_t total = rows * D;
     hipLaunchKernelGGL((band_dead_rows_kernel<T>), dim3((unsigned)((total + 255) / 256)), dim3(256),
-                       0, stream, (T*)a.t.out, a.n, D, a.block, a.s);
+                       0, stream, (T*)a.t.out, rows, D, a.block, a.s);
   }
   return hipGetLastError() == hipSuccess ? 0 : 4;
 }

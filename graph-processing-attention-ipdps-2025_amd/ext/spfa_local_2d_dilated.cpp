@@ -18,7 +18,7 @@ torch::Tensor spfa_local_2d_dilated_forward_py(torch::Tensor Q, torch::Tensor K,
   spfa_problem_t p = spfa_ext::make_problem(Q, K, V, m, l, O);
   TORCH_CHECK(p.n_k == p.n_q, "Q, K and V must have the same number of rows");
   const size_t ws_bytes =
-      spfa_local_2d_dilated_workspace_bytes(p.n_q, p.d, p.dtype, block_size, dil_factor);
+      spfa_ext::batched(spfa_local_2d_dilated_workspace_bytes(p.n_q, p.d, p.dtype, block_size, dil_factor), p);
   torch::Tensor ws = spfa_ext::make_workspace(ws_bytes, Q);
   spfa_ext::raise_on_error(spfa_local_2d_dilated_forward(&p, block_size, dil_factor, use_nan ? 1 : 0,
                                                          ws.data_ptr(), (size_t)ws.numel(),

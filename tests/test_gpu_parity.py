@@ -392,9 +392,10 @@ def test_coo_batch_rectangular_keys(mods):
                  torch.float32)
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_implicit_masks_batch_of_heads(mods, dtype):
-    n, d = 1024, 64
+@pytest.mark.parametrize("dtype,d", [(torch.float32, 64), (torch.bfloat16, 64), (torch.float32, 40)])
+def test_implicit_masks_batch_of_heads(mods, dtype, d):
+    """d = 64 runs the dense-tile kernels, d = 40 the row-gather engine."""
+    n = 1024
     shape = (2, 2)
     w, dil, blk = 40, 1, 64
     globs = [3, 500, 501, 900]
