@@ -143,9 +143,20 @@ def make_workload(name, dtype, torch, syn, inline_limit=32, planned=False, heads
         if name == "local":
             import spfa_local
             n, d, wsz = 65536, 64, 128
+            if heads > 1:  # many heads of a short sequence instead of one long one
+                n = 4096
+                w["desc"] = "Local N=4096 d=64 LOCAL_SIZE=128 (|i-j|<=128)"
             q, k, v = syn.qkv(n, d, dtype=dtype, device=dev, seed=0)
+            if heads > 1:
+                q, k, v = [torch.stack([syn.qkv(n, d, dtype=dtype, device=dev, seed=h)[j] for h in range(heads)])
+                           for j in range(3)]
             nnz = syn.local_nnz(n, wsz)
             w["call"] = lambda st: spfa_local.forward(q, k, v, st[0], st[1], st[2], wsz)
+            if heads > 1 and loop_heads:
+                def looped(st):
+                    for h in range(heads):
+                        spfa_local.forward(q[h], k[h], v[h], st[0][h], st[1][h], st[2][h], wsz)
+                w["call"] = looped
             w["params"] = {"LOCAL_SIZE": wsz}
             live = n
         elif name == "local_1d":
@@ -178,8 +189,8 @@ def make_workload(name, dtype, torch, syn, inline_limit=32, planned=False, heads
             w["n_global_rows_nnz"] = g * n - int(sum(min(n, int(x) + wsz + 1) - max(0, int(x) - wsz)
                                                       for x in globs.cpu().tolist()))
         total = syn.implicit_mask_bytes(n, d, es, live_rows=live)
-        w.update(n=n, d=d, nnz=nnz, bytes_total=total, bytes_gathered=nnz * 2 * d * es, bound="hbm",
-                 kernel_bytes=total, kernel_nnz=nnz, kernel_rows=live)
+        w.update(n=n, d=d, nnz=nnz * heads, bytes_total=total * heads, bytes_gathered=nnz * 2 * d * es * heads,
+                 bound="hbm", kernel_bytes=total * heads, kernel_nnz=nnz * heads, kernel_rows=live * heads)
     w.update(q=q, k=k, v=v, heads=heads)
     return w
 
@@ -343,7 +354,8 @@ def main():
     ap.add_argument("--dtype", default="f32", choices=["f32", "f16", "bf16"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--heads", type=int, default=1,
-                    help="csr_* workloads: this many independent problems sharing the mask, stacked [heads, n, d]")
+                    help="csr_* and local workloads: this many independent problems sharing the mask, stacked "
+                         "[heads, n, d] (local: of N=4096 tokens each)")
     ap.add_argument("--loop-heads", action="store_true",
                     help="with --heads: one call per head (the reference's only way) instead of one batched call")
     ap.add_argument("--planned", action="store_true",
@@ -366,8 +378,8 @@ def main():
     lib = load_library()
     if a.planned and not (a.workload.startswith("csr") or a.workload.startswith("coo")):
         sys.exit("bench.py: --planned applies to the explicit-mask workloads (csr_*, coo_*)")
-    if a.heads > 1 and not a.workload.startswith("csr"):
-        sys.exit("bench.py: --heads applies to the csr_* workloads")
+    if a.heads > 1 and not (a.workload.startswith("csr") or a.workload == "local"):
+        sys.exit("bench.py: --heads applies to the csr_* and local workloads")
     w = make_workload(a.workload, dtype, torch, syn, int(lib.spfa_explicit_inline_row_limit()), a.planned,
                       max(1, a.heads), a.loop_heads)
     n, d, nnz = w["n"], w["d"], w["nnz"]

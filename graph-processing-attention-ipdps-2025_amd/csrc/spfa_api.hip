@@ -248,7 +248,7 @@ struct GlobalLayout {
   int64_t key_run, n_split;
 };
 
-GlobalLayout global_layout(int64_t n, int64_t n_globs, int64_t d) {
+GlobalLayout global_layout(int64_t n, int64_t n_globs, int64_t d, int64_t n_batch = 1) {
   GlobalLayout g{};
   const int64_t q_tiles = (n_globs + 127) / 128;
   // one key split per workgroup slot of the device (two workgroups fit a CU): more splits only
@@ -260,11 +260,11 @@ GlobalLayout global_layout(int64_t n, int64_t n_globs, int64_t d) {
   run = (run + 63) / 64 * 64;
   g.key_run = run;
   g.n_split = (n + run - 1) / run;
-  const size_t slots = (size_t)n_globs * (size_t)g.n_split;
+  const size_t slots = (size_t)n_globs * (size_t)g.n_split * (size_t)(n_batch > 1 ? n_batch : 1);
   size_t off = 0;
   g.off_bits = off;   off = align_up(off + global_bits_words(n) * 4, 256);
   g.off_uq = off;     off = align_up(off + (size_t)n_globs * 4, 256);
-  g.off_engine = off; off = align_up(off + engine_workspace(size_global(n, n_globs), n, d).total, 256);
+  g.off_engine = off; off = align_up(off + engine_workspace(size_global(n, n_globs), n, d, n_batch).total, 256);
   g.off_pm = off;     off = align_up(off + slots * 4, 256);
   g.off_pl = off;     off = align_up(off + slots * 4, 256);
   g.off_pacc = off;   off = align_up(off + slots * (size_t)d * 4, 256);
@@ -594,22 +594,13 @@ int spfa_global_no_local_forward(const spfa_problem_t* p, const int32_t* global_
                                  size_t workspace_bytes, void* stream) {
   int rc = check_problem(p);
   if (rc) return rc;
-  if (batch_of(p) > 1) {  // no batched kernels on this path yet: one problem after the other
-    for (int64_t b = 0; b < batch_of(p); b++) {
-      const spfa_problem_t one = batch_slice(p, b);
-      rc = spfa_global_no_local_forward(&one, global_inds, n_globals, local_size, workspace,
-                                        workspace_bytes, stream);
-      if (rc) return rc;
-    }
-    return SPFA_OK;
-  }
   if (n_globals <= 0 || n_globals > p->n_q) return SPFA_ERR_GLOBAL_COUNT;
   if (local_size < 0 || local_size > p->n_q - 1) return SPFA_ERR_LOCAL_SIZE;
   rc = check_pointers(p);
   if (rc) return rc;
   if (!global_inds) return SPFA_ERR_BAD_ARG;
   const int64_t n = p->n_q;
-  const GlobalLayout lay = global_layout(n, n_globals, p->d);
+  const GlobalLayout lay = global_layout(n, n_globals, p->d, batch_of(p));
   rc = check_workspace(workspace, workspace_bytes, lay.total);
   if (rc) return rc;
   char* base = (char*)workspace;
@@ -635,7 +626,8 @@ int spfa_global_no_local_forward(const spfa_problem_t* p, const int32_t* global_
   a.pl = (float*)(base + lay.off_pl);
   a.pacc = (float*)(base + lay.off_pacc);
   const int64_t q_tiles = (n_globals + 127) / 128;
-  if (q_tiles * lay.n_split < ((int64_t)1 << 31) && n_globals < ((int64_t)1 << 31) &&
+  if (q_tiles * lay.n_split * batch_of(p) < ((int64_t)1 << 31) &&
+      n_globals * batch_of(p) < ((int64_t)1 << 31) && batch_of(p) < 65536 &&
       local_size <= kTileMaxWindow) {
     rc = -1;
     switch (p->dtype) {

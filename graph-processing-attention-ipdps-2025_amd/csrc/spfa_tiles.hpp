@@ -208,23 +208,24 @@ __global__ __launch_bounds__(256, 2) void tile_kernel(TileArgs a) {
   // base/len: token of position 0 and number of positions (band); qlen/klen: query and key
   // position counts; [u_lo, u_hi): key positions this workgroup walks
   int64_t base = 0, qlen, klen, t0, u_lo, u_hi, split = 0;
+  int64_t bb = 0;  // problem of the batch (global modes; band mode folds it into base)
   if constexpr (MODE == kTileBand) {
     // workgroups are dealt round-robin to the 8 XCDs: give each XCD a contiguous run of tiles
     // so that neighbouring query tiles (which share most of their keys) meet in one L2
-    // (the tiles of all problems of a batch form one list; problem bb starts at token bb * n)
+    // (the tiles of all problems of a batch form one list; problem pb starts at token pb * n)
     const int64_t n_all = a.n_tiles * a.t.n_batch;
     const int64_t per_xcd = (n_all + 7) / 8;
     int64_t lt = (int64_t)(blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
     if (lt >= n_all) return;
-    const int64_t bb = lt / a.n_tiles;
-    lt -= bb * a.n_tiles;
+    const int64_t pb = lt / a.n_tiles;
+    lt -= pb * a.n_tiles;
     const int64_t sub = lt / a.tiles_per_sub;
     const int64_t tile = lt - sub * a.tiles_per_sub;
     if (a.block > 0) {
-      base = sub * a.block + bb * a.n;
+      base = sub * a.block + pb * a.n;
       qlen = a.cnt;
     } else {
-      base = sub + bb * a.n;
+      base = sub + pb * a.n;
       qlen = (a.n - sub + a.s - 1) / a.s;
     }
     klen = qlen;
@@ -235,8 +236,12 @@ __global__ __launch_bounds__(256, 2) void tile_kernel(TileArgs a) {
     u_hi = t0 + BM + a.w;
     if (u_hi > klen || u_hi < 0) u_hi = klen;
   } else if constexpr (MODE == kTileGlobalRows) {
-    const int64_t qt = blockIdx.x / a.n_split;
-    split = blockIdx.x - qt * a.n_split;
+    // grid: [problem][query tile][key split]
+    const int64_t per_problem = (int64_t)gridDim.x / a.t.n_batch;
+    bb = blockIdx.x / per_problem;
+    const int64_t in_problem = blockIdx.x - bb * per_problem;
+    const int64_t qt = in_problem / a.n_split;
+    split = in_problem - qt * a.n_split;
     qlen = (int64_t)*a.n_uq;
     klen = a.n;
     t0 = qt * BM;
@@ -245,6 +250,7 @@ __global__ __launch_bounds__(256, 2) void tile_kernel(TileArgs a) {
     u_hi = u_lo + a.key_run;
     if (u_hi > klen) u_hi = klen;
   } else {
+    bb = blockIdx.y;  // one grid row per problem
     qlen = a.n;
     klen = a.n_globs;
     t0 = (int64_t)blockIdx.x * BM;
@@ -264,6 +270,9 @@ __global__ __launch_bounds__(256, 2) void tile_kernel(TileArgs a) {
   const T* Vp = (const T*)a.t.v;
   const float sc = 1.4426950408889634f / sqrtf((float)D);
   const bool persist = (MODE == kTileGlobalCols) && a.persist != 0;
+  // global modes: tokens of problem bb are rows bb * n + token of the stacked tensors (masks work
+  // on the tokens, only addresses take the offset)
+  const int64_t tok_off = (MODE == kTileBand) ? 0 : bb * a.n;
   bool staged = false;  // persist: the key tile is already in LDS
 
   // One trip per query tile.  Only a persistent GlobalCols workgroup makes more than one.
@@ -289,7 +298,7 @@ __global__ __launch_bounds__(256, 2) void tile_kernel(TileArgs a) {
   uint4v qh[kF32 ? 1 : C::QREGS];
   float qf[kF32 ? C::QREGS : 1];
   {
-    const T* qrow = Qp + q_tok * D;
+    const T* qrow = Qp + (q_tok + tok_off) * D;
     if constexpr (kF32) {
 #pragma unroll
       for (int c4 = 0; c4 < D / 4; c4++) {
@@ -317,8 +326,8 @@ __global__ __launch_bounds__(256, 2) void tile_kernel(TileArgs a) {
   // consumed and land in registers; they are written to LDS once tile n has been consumed.
   auto key_tok = [&](int64_t u) -> int64_t {
     if constexpr (MODE == kTileBand) return base + u * a.s;
-    else if constexpr (MODE == kTileGlobalRows) return u;
-    else return (int64_t)a.globs[u];
+    else if constexpr (MODE == kTileGlobalRows) return u + tok_off;
+    else return (int64_t)a.globs[u] + tok_off;
   };
   constexpr int CH = kF32 ? D / 4 : D / 8;       // 16-byte chunks per row
   constexpr int KIT = BN * CH / 256;             // chunks of K per thread and tile
@@ -581,7 +590,7 @@ __global__ __launch_bounds__(256, 2) void tile_kernel(TileArgs a) {
   if constexpr (MODE == kTileGlobalRows) {
     // partial result of this key split; an empty one is (m, l, acc) = (-inf, 0, 0)
     if (!q_ok) return;  // (this mode makes a single trip)
-    const int64_t slot = tq * a.n_split + split;
+    const int64_t slot = (bb * a.n_globs + tq) * a.n_split + split;
     const bool any = l > 0.f;
     float* prow = a.pacc + slot * D;
 #pragma unroll
@@ -600,7 +609,7 @@ __global__ __launch_bounds__(256, 2) void tile_kernel(TileArgs a) {
     }
     return;
   }
-  if (q_ok && l > 0.f) tile_write_row<T, D>(a.t, q_tok, h, m, l, o);
+  if (q_ok && l > 0.f) tile_write_row<T, D>(a.t, q_tok + tok_off, h, m, l, o);
   if (!persist) break;
   }  // query tiles
 }
@@ -928,10 +937,12 @@ __global__ __launch_bounds__(256) void global_rows_merge_kernel(TileArgs a) {
   constexpr int NSUB = 256 / D;  // threads per output element
   __shared__ float red[4];
   __shared__ float part[256];
-  const int64_t g = blockIdx.x;
+  // grid: [problem][listed global]; the first n_uq of a problem's slots are its distinct rows
+  const int64_t bb = blockIdx.x / a.n_globs;
+  const int64_t g = blockIdx.x - bb * a.n_globs;
   if (g >= (int64_t)*a.n_uq) return;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int64_t s0 = g * a.n_split;
+  const int64_t s0 = (bb * a.n_globs + g) * a.n_split;
 
   float mx = kNegInf;
   for (int64_t k = tid; k < a.n_split; k += 256) mx = fmaxf(mx, a.pm[s0 + k]);
@@ -971,7 +982,7 @@ __global__ __launch_bounds__(256) void global_rows_merge_kernel(TileArgs a) {
 #pragma unroll
   for (int u = 1; u < NSUB; u++) acc += part[u * D + e];
 
-  const int64_t row = a.uq[g];
+  const int64_t row = a.uq[g] + bb * a.n;
   const bool sf = a.t.state_f32 != 0;
   float m_out = mx, l_out = lsum, wa = 0.f, wb = 1.f;
   const float l_in = load_state<T>(a.t.l, row, sf);
@@ -1036,17 +1047,22 @@ int launch_global_tiles(const TileArgs& a, hipStream_t stream) {
     const int64_t resident = (int64_t)device_cu_count() * 2;  // two workgroups fit a CU
     if (grid_cols > resident) grid_cols = resident;
   }
-  hipLaunchKernelGGL((tile_kernel<T, D, kTileGlobalCols>), dim3((unsigned)grid_cols), dim3(256), 0,
+  const unsigned nb = (unsigned)a.t.n_batch;
+  if (ac.persist && nb > 1) {  // the resident workgroups are shared out over the problems
+    grid_cols = grid_cols / nb;
+    if (grid_cols < 1) grid_cols = 1;
+  }
+  hipLaunchKernelGGL((tile_kernel<T, D, kTileGlobalCols>), dim3((unsigned)grid_cols, nb), dim3(256), 0,
                      stream, ac);
   const int64_t q_tiles = (a.n_globs + 127) / 128;
   TileArgs ar = a;
   ar.pair_split = (a.n_globs <= 64 && TileCfg<T, D>::NB == 2) ? 1 : 0;
   if (timed) (void)hipEventRecord(ev.start, stream);
-  hipLaunchKernelGGL((tile_kernel<T, D, kTileGlobalRows>), dim3((unsigned)(q_tiles * a.n_split)),
+  hipLaunchKernelGGL((tile_kernel<T, D, kTileGlobalRows>), dim3((unsigned)(q_tiles * a.n_split * nb)),
                      dim3(256), 0, stream, ar);
   if (timed) (void)hipEventRecord(ev.stop, stream);
-  hipLaunchKernelGGL((global_rows_merge_kernel<T, D>), dim3((unsigned)a.n_globs), dim3(256), 0, stream,
-                     a);
+  hipLaunchKernelGGL((global_rows_merge_kernel<T, D>), dim3((unsigned)(a.n_globs * nb)), dim3(256), 0,
+                     stream, a);
   return hipGetLastError() == hipSuccess ? 0 : 4;
 }
 

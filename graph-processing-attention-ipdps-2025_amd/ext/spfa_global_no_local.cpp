@@ -23,7 +23,7 @@ torch::Tensor spfa_global_no_local_forward_py(torch::Tensor Q, torch::Tensor K, 
   TORCH_CHECK(global_inds.scalar_type() == torch::kInt32, "global_inds must be an int32 tensor");
   const int64_t n_globs = global_inds.size(0);
   const size_t ws_bytes =
-      spfa_global_no_local_workspace_bytes(p.n_q, p.d, p.dtype, n_globs, local_size_each_dir);
+      spfa_ext::batched(spfa_global_no_local_workspace_bytes(p.n_q, p.d, p.dtype, n_globs, local_size_each_dir), p);
   torch::Tensor ws = spfa_ext::make_workspace(ws_bytes, Q);
   spfa_ext::raise_on_error(spfa_global_no_local_forward(
       &p, (const int32_t*)global_inds.data_ptr(), n_globs, local_size_each_dir, ws.data_ptr(),
