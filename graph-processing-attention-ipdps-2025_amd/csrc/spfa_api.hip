@@ -13,7 +13,6 @@ namespace {
 constexpr int64_t kInlineAll = std::numeric_limits<int64_t>::max();
 
 
-inline size_t dtype_size(int dtype) { return dtype == SPFA_DTYPE_F32 ? 4 : 2; }
 
 inline bool dtype_ok(int dtype) {
   return dtype == SPFA_DTYPE_F32 || dtype == SPFA_DTYPE_F16 || dtype == SPFA_DTYPE_BF16;

@@ -89,7 +89,6 @@ struct VecLay {
   static constexpr int U = 16;       // neighbours in flight per group in the segment kernel
   static constexpr int U_SHORT = 4;  // ... in the row kernel
   static constexpr int U_MEDIUM = 8; // ... in the medium-row kernel
-  static constexpr bool kFixedD = true;
   using raw = uint4v;
 
   __device__ static __forceinline__ raw load(const T* row_ptr, int c, int) {
@@ -165,7 +164,6 @@ struct GenLay {
   static constexpr int U = (EPL <= 2) ? 8 : 2;
   static constexpr int U_SHORT = U;
   static constexpr int U_MEDIUM = U;
-  static constexpr bool kFixedD = false;
   struct raw { T x[EPL]; };
 
   __device__ static __forceinline__ raw load(const T* row_ptr, int c, int d) {

@@ -4,17 +4,21 @@
 // it has (deg) and which column the t-th candidate is.  The engine walks those candidates with
 // an online softmax.  Work decomposition:
 //
-//   plan_kernel      one thread per query row; rows with more than short_max candidates are cut
-//                    into segments of `seg` candidates that are appended to a work list.
-//   rows_kernel      one group of LPR lanes per query row (64/LPR rows per wavefront) finishes
-//                    the rows with deg <= short_max on the spot.
-//   segments_kernel  persistent grid; each wavefront pulls segments off the work list, its
-//                    64/LPR groups take interleaved candidates, the groups are merged with
-//                    cross-lane moves, and the result is either final (single-segment row) or a
-//                    partial (m, l, acc[d]) in the workspace.
-//   merge_kernel     one group per multi-segment row folds that row's partials together.
+//   plan_kernel        one thread per query row: rows with short_max < deg <= medium_max go on a
+//                      list of their own, longer rows are cut into segments of `seg` candidates
+//                      that are appended to a work list.
+//   rows_kernel        one group of LPR lanes per query row (64/LPR rows per wavefront) finishes
+//                      the rows with deg <= short_max on the spot.
+//   medium_rows_kernel one wavefront per listed medium row, its 64/LPR groups share the row.
+//   segments_kernel    persistent grid; each wavefront pulls segments off the work list, its
+//                      64/LPR groups take interleaved candidates, the groups are merged with
+//                      cross-lane moves, and the result is either final (single-segment row) or
+//                      a partial (m, l, acc[d]) in the workspace.
+//   merge_kernel       one group per multi-segment row folds that row's partials together.
 //
-// All three finish a row the same way: fold the incoming (m, l, out) state in, write back.
+// All of them finish a row the same way: fold the incoming (m, l, out) state in, write back.
+// A batch of problems that share the mask is walked by the same kernels: rows of all problems
+// form one grid, the work list is shared, partial results are per problem.
 #pragma once
 
 #include "spfa_common.hpp"

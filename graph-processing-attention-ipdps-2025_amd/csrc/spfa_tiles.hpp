@@ -6,8 +6,10 @@
 //   Local 1D dilated      s subsequences, one per residue class mod s
 //   Local 2D dilated      one subsequence per block (base b*B, cnt live tokens, w = everything)
 // so all three are the same tile problem.  One workgroup (4 wavefronts) owns 128 consecutive
-// query positions, one wavefront 32 of them; keys are streamed in tiles of 64 (32 for fp32 at d = 128) through LDS and
-// shared by the four wavefronts.
+// query positions, one wavefront 32 of them; keys are streamed in tiles of 64 (32 for fp32 at
+// d = 128) through LDS and shared by the four wavefronts.  tile_kernel stages the tiles through
+// registers (fp32 band masks, every type of the global mask); band_dma_kernel lets the loads
+// write LDS directly (bf16 / fp16 band masks).
 //
 // Everything is computed transposed, S^T = K Q^T and O^T = V^T P^T, with 32x32 MFMA tiles.  In
 // the 32x32 result layout lane (r, h) = (lane % 32, lane / 32) holds column r, rows
@@ -773,11 +775,7 @@ __global__ __launch_bounds__(256, 2) void band_dma_kernel(TileArgs a) {
   auto step = [&](int ut, const char* tb, char* other) __attribute__((always_inline)) {
     __builtin_amdgcn_s_waitcnt(0);  // this wavefront's part of the tile has landed
     __syncthreads();                // everyone's has, and everyone is done with the other buffer
-#ifdef SPFA_EXP_SAMETILE
-    if (ut + BN < u_hi) request(u_lo, other);
-#else
     if (ut + BN < u_hi) request(ut + BN, other);
-#endif
 
     // Both 32-key blocks of the tile are always computed (a block outside this wavefront's
     // band is masked out completely; the band is much wider than a block), which keeps the
