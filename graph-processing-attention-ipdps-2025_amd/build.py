@@ -36,7 +36,7 @@ ELEM_TYPES = {"f32": "float", "f16": "spfa::f16", "bf16": "spfa::bf16"}
 MASK_KINDS = {"csr": 0, "stride": 1, "global": 2}
 
 MODULES = ["spfa_csr", "spfa_coo", "spfa_local", "spfa_local_1d_dilated", "spfa_local_2d_dilated",
-           "spfa_global_no_local"]
+           "spfa_global_no_local", "spfa_bigbird"]
 
 
 def _run(cmd):

@@ -145,6 +145,21 @@ int spfa_coo_forward_planned(const spfa_problem_t* p, const void* col_ind, int64
                              const void* plan, size_t plan_bytes, void* workspace,
                              size_t workspace_bytes, void* stream);
 
+/* Window + global + CSR in one call (the "BigBird" / "Longformer" pattern).  The reference's
+ * callers get it by chaining three calls on one (m, l, out) state: Local, Global-no-local with the
+ * same window, CSR with the random part (verification/verify.py:337-352); this entry point is that
+ * chain: row i attends its window [i-w, i+w], the listed global tokens outside it (a listed row
+ * attends every token), and the columns of the CSR rows.  The three parts must not overlap (a
+ * column present twice counts twice, exactly as in the chain); n_globals == 0 or nnz == 0 leave
+ * that part out.  n_k must equal n_q.  No row is ever empty (the window holds the diagonal). */
+size_t spfa_window_global_csr_workspace_bytes(int64_t n, int64_t d, int dtype, int64_t local_size,
+                                              int64_t n_globals, int64_t nnz);
+int spfa_window_global_csr_forward(const spfa_problem_t* p, int64_t local_size,
+                                   const int32_t* global_inds, int64_t n_globals,
+                                   const void* row_off, int row_off_bytes, const void* col_ind,
+                                   int64_t nnz, void* workspace, size_t workspace_bytes,
+                                   void* stream);
+
 /* Local: row i attends columns max(0, i-w) .. min(n-1, i+w)  (sp_flatt_local_kernel.cu:24-28). */
 size_t spfa_local_workspace_bytes(int64_t n, int64_t d, int dtype, int64_t local_size);
 int spfa_local_forward(const spfa_problem_t* p, int64_t local_size, void* workspace,

@@ -37,9 +37,9 @@ def golden():
 
 @pytest.fixture(scope="session")
 def mods():
-    """The six Python modules of the product (must already be built in-tree)."""
+    """The Python modules of the product (must already be built in-tree)."""
     import importlib
     names = ["spfa_csr", "spfa_coo", "spfa_local", "spfa_local_1d_dilated", "spfa_local_2d_dilated",
-             "spfa_global_no_local"]
+             "spfa_global_no_local", "spfa_bigbird"]
     import torch  # noqa: F401  (the extensions link against libtorch)
     return {n: importlib.import_module(n) for n in names}

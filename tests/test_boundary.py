@@ -98,6 +98,11 @@ def test_workspace_sizes_are_sane(lib):
     assert lib.spfa_coo_workspace_bytes(i64(131072), i64(13_000_000), i64(64), 0) > large
     assert lib.spfa_local_workspace_bytes(i64(65536), i64(64), 0, i64(128)) >= 256
     assert lib.spfa_global_no_local_workspace_bytes(i64(1 << 20), i64(64), 0, i64(64), i64(64)) > (1 << 20)
+    # the one-call window + global + CSR entry needs the largest of its three parts
+    lib.spfa_window_global_csr_workspace_bytes.restype = ctypes.c_size_t
+    both = lib.spfa_window_global_csr_workspace_bytes(i64(1 << 20), i64(64), 0, i64(64), i64(64), i64(1000))
+    assert both >= lib.spfa_global_no_local_workspace_bytes(i64(1 << 20), i64(64), 0, i64(64), i64(64))
+    assert both >= lib.spfa_csr_workspace_bytes(i64(1 << 20), i64(1000), i64(64), 0)
 
 
 def test_modules_import_and_expose_forward(mods):

@@ -417,6 +417,51 @@ def test_implicit_masks_batch_of_heads(mods, dtype, d):
     _check_heads(q, k, v, o, m, l, lambda a, b, c: so.dense_masked_attention(a, b, c, dense), dtype)
 
 
+# ------------------------------------------------------------------ window + global + CSR in one call
+@pytest.mark.parametrize("dtype,d", [(torch.float32, 64), (torch.bfloat16, 64), (torch.float16, 128),
+                                      (torch.float32, 40)])
+@pytest.mark.parametrize("n,w,n_globs", [(1024, 10, 5), (2000, 64, 70), (1500, 0, 1)])
+def test_bigbird_one_call_equals_dense_union(mods, dtype, d, n, w, n_globs):
+    """spfa_bigbird.forward == dense attention over Local | Global-no-local | random (the chain of
+    verification/verify.py:337-352 in one call)."""
+    rng = np.random.default_rng(n + w)
+    globs = np.sort(rng.choice(n, n_globs, replace=False))
+    fixed = so.mask_local_dense(n, w) | so.mask_global_no_local_dense(n, globs, w)
+    rnd = (rng.random((n, n)) < 0.03) & ~fixed
+    ro, ci = so.csr_from_dense(rnd)
+    q, k, v = dev_qkv(n, d, dtype, 61)
+    m, l, o = state(n, d, dtype, torch.float32)
+    ro_t, ci_t = csr_tensors(ro, ci)
+    ret = mods["spfa_bigbird"].forward(q, k, v, m, l, o, w, torch.tensor(globs, dtype=torch.int32, device=DEV),
+                                       ro_t, ci_t, torch.ones(len(ci), device=DEV, dtype=dtype))
+    sync()
+    assert ret.data_ptr() == o.data_ptr()
+    ref = so.dense_masked_attention(np64(q), np64(k), np64(v), fixed | rnd)
+    check(o, m, l, *ref, dtype, state_dtype=torch.float32)
+
+
+def test_bigbird_parts_may_be_empty_and_batched(mods):
+    n, d, w = 1024, 64, 16
+    globs = [7, 300, 1000]
+    q, k, v, m, l, o = _stacked(n, d, torch.float32, (3,), 62)
+    e_i32 = torch.zeros(0, dtype=torch.int32, device=DEV)
+    e_u64 = torch.zeros(0, dtype=torch.uint64, device=DEV)
+    e_u32 = torch.zeros(0, dtype=torch.uint32, device=DEV)
+    e_val = torch.zeros(0, device=DEV)
+    # window + globals, no CSR part, three problems at once
+    mods["spfa_bigbird"].forward(q, k, v, m, l, o, w, torch.tensor(globs, dtype=torch.int32, device=DEV),
+                                 e_u64, e_u32, e_val)
+    sync()
+    dense = so.mask_local_dense(n, w) | so.mask_global_no_local_dense(n, globs, w)
+    _check_heads(q, k, v, o, m, l, lambda a, b, c: so.dense_masked_attention(a, b, c, dense), torch.float32)
+    # window only
+    q, k, v, m, l, o = _stacked(n, d, torch.float32, (1,), 63)
+    mods["spfa_bigbird"].forward(q, k, v, m, l, o, w, e_i32, e_u64, e_u32, e_val)
+    sync()
+    dense = so.mask_local_dense(n, w)
+    _check_heads(q, k, v, o, m, l, lambda a, b, c: so.dense_masked_attention(a, b, c, dense), torch.float32)
+
+
 # ------------------------------------------------------------------ mask plans
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_csr_plan_is_reused_across_calls_and_dtypes(mods, dtype):
