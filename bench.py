@@ -39,6 +39,8 @@ WORKLOADS = {
     "local_1d": "Local-1D-dilated N=262144 d=128 LOCAL_SIZE=256 DILATE_FACTOR=2 (stride 3)",
     "local_2d": "Local-2D-dilated N=262144 d=128 BLOCK_SIZE=256 DILATE_FACTOR=2 (stride 3)",
     "global": "Global-no-local N=1048576 d=64 64 global tokens LOCAL_SIZE=64",
+    "bigbird": "Window + global + random in one call: N=65536 d=64 LOCAL_SIZE=128, 64 global tokens, "
+               "192 random columns per row (CSR)",
 }
 
 
@@ -175,6 +177,46 @@ def make_workload(name, dtype, torch, syn, inline_limit=32, planned=False, heads
             w["call"] = lambda st: spfa_local_2d_dilated.forward(q, k, v, st[0], st[1], st[2], blk, dil, False)
             w["params"] = {"BLOCK_SIZE": blk, "DILATE_FACTOR": dil}
             live = (n // blk) * min(blk, (blk - 1) // (dil + 1) + 1)
+        elif name == "bigbird":
+            import spfa_bigbird
+            import spfa_csr
+            import spfa_global_no_local
+            import spfa_local
+            n, d, g, wsz, per_row = 65536, 64, 64, 128, 192
+            q, k, v = syn.qkv(n, d, dtype=dtype, device=dev, seed=0)
+            globs = syn.global_indices(n, g, device=dev, seed=0)
+            # random part: per_row columns per row, none inside the window or among the globals
+            gen = torch.Generator(device=dev).manual_seed(0)
+            cols = torch.randint(0, n, (n, per_row), generator=gen, device=dev)
+            rows = torch.arange(n, device=dev).unsqueeze(1)
+            is_glob = torch.zeros(n, dtype=torch.bool, device=dev)
+            is_glob[globs.long()] = True
+            keep = ((cols - rows).abs() > wsz) & ~is_glob[cols] & ~is_glob[rows.expand_as(cols)]
+            cols_sorted, _ = torch.sort(torch.where(keep, cols, torch.full_like(cols, n)), dim=1)
+            dup = torch.zeros_like(keep)
+            dup[:, 1:] = cols_sorted[:, 1:] == cols_sorted[:, :-1]
+            keep = (cols_sorted < n) & ~dup
+            ro = torch.zeros(n + 1, dtype=torch.int64, device=dev)
+            ro[1:] = torch.cumsum(keep.sum(dim=1), 0)
+            ci = cols_sorted[keep]
+            ro_t, ci_t = ro.to(torch.uint64), ci.to(torch.uint32)
+            val = torch.empty(ci.numel(), device=dev, dtype=dtype)
+            nnz_csr = int(ci.numel())
+            nnz = syn.local_nnz(n, wsz) + syn.global_no_local_nnz(n, globs, wsz) + nnz_csr
+            if loop_heads:  # (re-used flag) the reference's way: three chained calls
+                def chained(st):
+                    spfa_local.forward(q, k, v, st[0], st[1], st[2], wsz)
+                    spfa_global_no_local.forward(q, k, v, st[0], st[1], st[2], globs, wsz)
+                    spfa_csr.forward(q, k, v, ro_t, ci_t, val, st[0], st[1], st[2], False)
+                w["call"] = chained
+            else:
+                w["call"] = lambda st: spfa_bigbird.forward(q, k, v, st[0], st[1], st[2], wsz, globs, ro_t, ci_t, val)
+            w["params"] = {"n_globals": g, "LOCAL_SIZE": wsz, "csr_nnz": nnz_csr}
+            w["globs"] = globs
+            w["csr"] = (ro, ci)
+            w["whole_call"] = True
+            live = n
+            w["extra_bytes"] = syn.explicit_mask_bytes(nnz_csr, n, d, es, off_bytes=8)[1]
         else:
             import spfa_global_no_local
             n, d, g, wsz = 1 << 20, 64, 64, 64
@@ -188,7 +230,7 @@ def make_workload(name, dtype, torch, syn, inline_limit=32, planned=False, heads
             # live positions of the global rows alone (what the event-timed kernel covers)
             w["n_global_rows_nnz"] = g * n - int(sum(min(n, int(x) + wsz + 1) - max(0, int(x) - wsz)
                                                       for x in globs.cpu().tolist()))
-        total = syn.implicit_mask_bytes(n, d, es, live_rows=live)
+        total = syn.implicit_mask_bytes(n, d, es, live_rows=live) + w.get("extra_bytes", 0)
         w.update(n=n, d=d, nnz=nnz * heads, bytes_total=total * heads, bytes_gathered=nnz * 2 * d * es * heads,
                  bound="hbm", kernel_bytes=total * heads, kernel_nnz=nnz * heads, kernel_rows=live * heads)
     w.update(q=q, k=k, v=v, heads=heads)
@@ -227,6 +269,22 @@ def verify_sample(w, state, torch, rows=192):
     elif name == "local_2d":
         p = w["params"]
         lists = [so.live_local_2d_dilated(n, p["BLOCK_SIZE"], p["DILATE_FACTOR"], int(i)) for i in idx_np]
+    elif name == "bigbird":
+        gl = w["globs"].cpu().numpy()
+        gset = set(int(x) for x in gl)
+        wsz = w["params"]["LOCAL_SIZE"]
+        ro, ci = w["csr"]
+        ro_c = ro.cpu().numpy()
+        idx_np = np.concatenate([idx_np[:63], gl[:1].astype(np.int64)])
+        qs = w["q"][torch.as_tensor(idx_np).to("cuda")].float().cpu().numpy().astype(np.float64)
+
+        def live_bb(i):
+            low, up = max(0, i - wsz), min(n, i + wsz + 1)
+            if i in gset:
+                return np.arange(0, n)
+            outside = np.array([x for x in gl if x < low or x >= up], dtype=np.int64)
+            return np.concatenate([np.arange(low, up), outside, ci[ro_c[i]:ro_c[i + 1]].cpu().numpy()])
+        lists = [live_bb(int(i)) for i in idx_np]
     else:
         gl = w["globs"].cpu().numpy()
         # one global row is enough (each is a 1M-column row for the CPU)
@@ -357,7 +415,8 @@ def main():
                     help="csr_* and local workloads: this many independent problems sharing the mask, stacked "
                          "[heads, n, d] (local: of N=4096 tokens each)")
     ap.add_argument("--loop-heads", action="store_true",
-                    help="with --heads: one call per head (the reference's only way) instead of one batched call")
+                    help="with --heads: one call per head (the reference's only way) instead of one batched "
+                         "call; with --workload bigbird: the three chained calls instead of spfa_bigbird")
     ap.add_argument("--planned", action="store_true",
                     help="explicit masks: build the mask plan once, outside the timed region, and time "
                          "forward_planned (a mask reused across calls)")
@@ -444,7 +503,7 @@ def main():
     flops = syn.attention_flops(nnz, d)
     achieved_gbs = w["kernel_bytes"] / (k_avg * 1e-3) / 1e9
     explicit = a.workload.startswith(("csr", "coo"))
-    if explicit and w["kernel_nnz"] == 0:
+    if w.get("whole_call") or (explicit and w["kernel_nnz"] == 0):
         # no row is long enough for the segment kernel (all of them go to the row kernels): the
         # whole call stands in, with the call's algorithmic bytes
         k_avg = ms_per_step
@@ -452,7 +511,7 @@ def main():
         achieved_gbs = w["bytes_total"] / (ms_per_step * 1e-3) / 1e9
         roofline = {"bound": "hbm", "achieved": achieved_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                     "frac": achieved_gbs / HBM_PEAK_GBS, "traffic": None,
-                    "kernel": "whole call (rows_kernel + medium_rows_kernel; nothing for segments_kernel)"}
+                    "kernel": "whole call (several kernels, none dominant)"}
         w = dict(w, kernel_bytes=w["bytes_total"], kernel_nnz=w["nnz"], kernel_rows=w["n"] * w.get("heads", 1))
     elif explicit:
         # gather work: bound by memory, algorithmic bytes of the segment kernel over its time
@@ -485,7 +544,9 @@ def main():
                    "index_dtypes": "uint64 offsets / uint32 columns", "state": "fresh m=-inf l=0 each step",
                    "mask_plan": "reused (built outside the timed region)" if a.planned else "rebuilt every call",
                    "heads": max(1, a.heads),
-                   "heads_call": ("one call per head" if a.loop_heads else "one batched call") if a.heads > 1 else "single"},
+                   "heads_call": ("one call per head" if a.loop_heads else "one batched call") if a.heads > 1 else "single",
+                   "composite_call": (("three chained calls" if a.loop_heads else "one call (spfa_bigbird)")
+                                      if a.workload == "bigbird" else None)},
         "effective_gathered_GBs": w["bytes_gathered"] / (ms_per_step * 1e-3) / 1e9,
         "algorithmic_GBs": w["bytes_total"] / (ms_per_step * 1e-3) / 1e9,
         "roofline": roofline,
