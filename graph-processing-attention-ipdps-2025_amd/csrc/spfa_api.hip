@@ -4,6 +4,7 @@
 
 #include <limits>
 
+#include "spfa_f64.hpp"
 #include "spfa_kernels.hpp"
 
 using namespace spfa;
@@ -90,9 +91,15 @@ int check_problem(const spfa_problem_t* p) {
   return SPFA_OK;
 }
 
+bool is_f64(const spfa_problem_t* p) { return p->dtype == SPFA_DTYPE_F64; }
+
 int check_pointers(const spfa_problem_t* p) {
-  if (!dtype_ok(p->dtype)) return SPFA_ERR_UNSUPPORTED;
-  if (p->state_dtype != p->dtype && p->state_dtype != SPFA_DTYPE_F32) return SPFA_ERR_UNSUPPORTED;
+  if (is_f64(p)) {
+    if (p->state_dtype != SPFA_DTYPE_F64) return SPFA_ERR_UNSUPPORTED;
+  } else {
+    if (!dtype_ok(p->dtype)) return SPFA_ERR_UNSUPPORTED;
+    if (p->state_dtype != p->dtype && p->state_dtype != SPFA_DTYPE_F32) return SPFA_ERR_UNSUPPORTED;
+  }
   if (p->n_q == 0) return SPFA_OK;
   if (!p->q || !p->k || !p->v || !p->m || !p->l || !p->out) return SPFA_ERR_BAD_ARG;
   return SPFA_OK;
@@ -122,7 +129,9 @@ Tensors make_tensors(const spfa_problem_t* p) {
 
 int64_t batch_of(const spfa_problem_t* p) { return p->n_batch > 1 ? p->n_batch : 1; }
 
-size_t elem_bytes(int dtype) { return dtype == SPFA_DTYPE_F32 ? 4 : 2; }
+size_t elem_bytes(int dtype) {
+  return dtype == SPFA_DTYPE_F64 ? 8 : dtype == SPFA_DTYPE_F32 ? 4 : 2;
+}
 
 // Problem b of a batch as a problem of its own (the paths without batched kernels walk the batch
 // on the host, one problem after the other on the same stream and workspace).
@@ -329,6 +338,10 @@ int spfa_csr_forward(const spfa_problem_t* p, const void* row_off, int row_off_b
   if (rc) return rc;
   if (p->n_q == 0) return SPFA_OK;
   if (!row_off || (nnz > 0 && !col_ind)) return SPFA_ERR_BAD_ARG;
+  if (is_f64(p)) {
+    CsrMask mask{row_off, (const uint32_t*)col_ind, row_off_bytes == 8 ? 1 : 0, nullptr, nullptr};
+    return run_f64(make_tensors(p), mask, use_nan ? 1 : 0, (hipStream_t)stream);
+  }
   EngineSizing s = size_csr(p->n_q, nnz);
   if (!batch_fits_engine(s, p)) {
     for (int64_t b = 0; b < batch_of(p); b++) {
@@ -374,6 +387,10 @@ int spfa_csr_forward_planned(const spfa_problem_t* p, const void* row_off, int r
   if (rc) return rc;
   if (p->n_q == 0) return SPFA_OK;
   if (!row_off || (nnz > 0 && !col_ind)) return SPFA_ERR_BAD_ARG;
+  if (is_f64(p)) {  // (the fp64 kernel needs no work list)
+    CsrMask mask{row_off, (const uint32_t*)col_ind, row_off_bytes == 8 ? 1 : 0, nullptr, nullptr};
+    return run_f64(make_tensors(p), mask, use_nan ? 1 : 0, (hipStream_t)stream);
+  }
   EngineSizing s = size_csr(p->n_q, nnz);
   rc = check_workspace(plan, plan_bytes, work_list_bytes(p->n_q, nnz));
   if (rc) return rc;
@@ -424,6 +441,7 @@ int spfa_coo_forward(const spfa_problem_t* p, const void* row_ind, int row_ind_b
                   workspace, (char*)workspace + cw.keep_total, (hipStream_t)stream, &csr);
   if (rc) return rc;
   CsrMask mask{csr.row_off, (const uint32_t*)col_ind, 0, csr.cols, csr.unsorted};
+  if (is_f64(p)) return run_f64(make_tensors(p), mask, use_nan ? 1 : 0, (hipStream_t)stream);
   if (!batched) {  // one conversion, then problem after problem
     for (int64_t b = 0; b < batch_of(p); b++) {
       const spfa_problem_t one = batch_slice(p, b);
@@ -499,6 +517,7 @@ int spfa_coo_forward_planned(const spfa_problem_t* p, const void* col_ind, int64
   const char* pb = (const char*)plan;
   CsrMask mask{pb + w.off_row_off, (const uint32_t*)col_ind, 0, (const uint32_t*)(pb + w.off_cols),
                (const uint32_t*)(pb + w.off_flag)};
+  if (is_f64(p)) return run_f64(make_tensors(p), mask, use_nan ? 1 : 0, (hipStream_t)stream);
   return dispatch_csr(p, mask, s, use_nan ? 1 : 0, workspace, (hipStream_t)stream, kEngineRunOnly,
                       pb + w.keep_total);
 }
@@ -544,6 +563,7 @@ int spfa_local_1d_dilated_forward(const spfa_problem_t* p, int64_t local_size, i
     }
   }
   StrideMask mask{n, local_size, dil_factor + 1, 0, 0};
+  if (is_f64(p)) return run_f64(make_tensors(p), mask, 0, (hipStream_t)stream);
   return dispatch_stride(p, mask, s, 0, workspace, (hipStream_t)stream);
 }
 
@@ -576,6 +596,7 @@ int spfa_local_2d_dilated_forward(const spfa_problem_t* p, int64_t block_size, i
     if (rc >= 0) return rc;
   }
   StrideMask mask{n, 0, dil_factor + 1, block_size, cnt};
+  if (is_f64(p)) return run_f64(make_tensors(p), mask, use_nan ? 1 : 0, (hipStream_t)stream);
   return dispatch_stride(p, mask, s, use_nan ? 1 : 0, workspace, (hipStream_t)stream);
 }
 
@@ -607,6 +628,10 @@ int spfa_global_no_local_forward(const spfa_problem_t* p, const int32_t* global_
   int32_t* uq = (int32_t*)(base + lay.off_uq);
   rc = prepare_global_rows(global_inds, n_globals, n, bits, uq, (hipStream_t)stream);
   if (rc) return rc;
+  if (is_f64(p)) {
+    GlobalMask mask{n, local_size, global_inds, n_globals, bits};
+    return run_f64(make_tensors(p), mask, 0, (hipStream_t)stream);
+  }
 
   // dense tiles when the shape allows it
   TileArgs a{};

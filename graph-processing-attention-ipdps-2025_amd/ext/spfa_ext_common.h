@@ -25,6 +25,7 @@ inline int elem_dtype(const torch::Tensor& t) {
     case torch::kFloat32: return SPFA_DTYPE_F32;
     case torch::kFloat16: return SPFA_DTYPE_F16;
     case torch::kBFloat16: return SPFA_DTYPE_BF16;
+    case torch::kFloat64: return SPFA_DTYPE_F64;
     default: return -1;  // reported by the library after the parameter checks
   }
 }

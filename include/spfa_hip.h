@@ -44,7 +44,9 @@ extern "C" {
 #endif
 
 /* element type of q, k, v, out */
-enum { SPFA_DTYPE_F32 = 0, SPFA_DTYPE_F16 = 1, SPFA_DTYPE_BF16 = 2 };
+/* F64 (the reference dispatches double too, sp_flatt_csr_kernel.cu:270) runs a plain kernel
+ * with double arithmetic, for parity rather than speed; m and l must then be F64 as well. */
+enum { SPFA_DTYPE_F32 = 0, SPFA_DTYPE_F16 = 1, SPFA_DTYPE_BF16 = 2, SPFA_DTYPE_F64 = 3 };
 
 enum {
   SPFA_OK = 0,

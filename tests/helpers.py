@@ -6,14 +6,17 @@ from oracle import c_oracle
 from oracle import spfa_oracle as so
 
 # max-abs bars on the output: fp32 1e-4, half types 2e-2
-OUT_TOL = {torch.float32: 1e-4, torch.float16: 2e-2, torch.bfloat16: 2e-2}
+OUT_TOL = {torch.float32: 1e-4, torch.float16: 2e-2, torch.bfloat16: 2e-2, torch.float64: 1e-11}
 # bar on m + log(l): fp32 statistics 1e-4 / 2e-3 (half inputs, fp32 state); statistics stored in
 # a half type carry that type's rounding of m (|m| up to ~10): 1e-1
 LSE_TOL_F32_STATE = {torch.float32: 1e-4, torch.float16: 2e-3, torch.bfloat16: 2e-3}
+LSE_TOL_F64 = 1e-11
 LSE_TOL_HALF_STATE = 1e-1
 
 
 def np64(t):
+    if t.dtype == torch.float64:
+        return t.detach().cpu().numpy()
     return t.detach().to(torch.float32).cpu().numpy().astype(np.float64)
 
 
@@ -36,7 +39,10 @@ def check(out, m, l, ref_out, ref_m, ref_l, dtype, state_dtype=None, dead_expect
     assert np.isfinite(o[live]).all(), "non-finite values in live rows"
     err = np.abs(o[live] - ref_out[live]).max() if live.any() else 0.0
     assert err <= OUT_TOL[dtype], "out max-abs error %.3e > %.1e" % (err, OUT_TOL[dtype])
-    tol = LSE_TOL_F32_STATE[dtype] if state_dtype == torch.float32 else LSE_TOL_HALF_STATE
+    if dtype == torch.float64:
+        tol = LSE_TOL_F64
+    else:
+        tol = LSE_TOL_F32_STATE[dtype] if state_dtype == torch.float32 else LSE_TOL_HALF_STATE
     if live.any():
         lerr = np.abs(lse(mm, ll)[live] - lse(np.asarray(ref_m), np.asarray(ref_l))[live]).max()
         assert lerr <= tol, "m + log l error %.3e > %.1e" % (lerr, tol)

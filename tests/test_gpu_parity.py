@@ -417,6 +417,74 @@ def test_implicit_masks_batch_of_heads(mods, dtype, d):
     _check_heads(q, k, v, o, m, l, lambda a, b, c: so.dense_masked_attention(a, b, c, dense), dtype)
 
 
+# ------------------------------------------------------------------ fp64
+def _f64_problem(n, d, seed, n_k=None):
+    g = torch.Generator().manual_seed(seed)
+    n_k = n if n_k is None else n_k
+    q = torch.randn(n, d, generator=g, dtype=torch.float64).to(DEV)
+    k = torch.randn(n_k, d, generator=g, dtype=torch.float64).to(DEV)
+    v = torch.randn(n_k, d, generator=g, dtype=torch.float64).to(DEV)
+    m = torch.full((n,), -float("inf"), device=DEV, dtype=torch.float64)
+    l = torch.zeros(n, device=DEV, dtype=torch.float64)
+    o = torch.zeros(n, d, device=DEV, dtype=torch.float64)
+    return q, k, v, m, l, o
+
+
+@pytest.mark.parametrize("d", [64, 40, 200])
+def test_fp64_every_mask_matches_the_oracle_to_rounding(mods, d):
+    """double tensors (the reference dispatches double, sp_flatt_csr_kernel.cu:270): double
+    arithmetic on the device, compared with the float64 oracle at 1e-11."""
+    n = 700
+    f64 = torch.float64
+    # CSR with empty, short and long rows, rectangular K; then the same entries as shuffled COO
+    n_k = 900
+    g = torch.Generator().manual_seed(71)
+    deg = torch.randint(0, 40, (n,), generator=g)
+    deg[5] = 0
+    deg[123] = 850
+    ro, ci = syn.csr_from_degrees(deg, n_k, g, "cpu", force_diagonal=False)
+    ro_t, ci_t = csr_tensors(ro, ci)
+    q, k, v, m, l, o = _f64_problem(n, d, 71, n_k)
+    val = torch.ones(ci_t.numel(), device=DEV, dtype=f64)
+    mods["spfa_csr"].forward(q, k, v, ro_t, ci_t, val, m, l, o, True)
+    sync()
+    ref = c_oracle.csr(np64(q), np64(k), np64(v), ro.numpy(), ci.numpy(), use_nan=True)
+    check(o, m, l, *ref, f64, dead_expect="nan")
+    r, c = syn.coo_from_csr(ro, ci, shuffle_seed=71)
+    m2 = torch.full_like(m, -float("inf"))
+    l2, o2 = torch.zeros_like(l), torch.zeros_like(o)
+    mods["spfa_coo"].forward(q, k, v, r.to(torch.uint64).to(DEV), c.to(torch.uint32).to(DEV), val, m2, l2, o2, True)
+    sync()
+    check(o2, m2, l2, *ref, f64, dead_expect="nan")
+    # implicit masks
+    w, dil, blk = 30, 2, 70
+    globs = [0, 350, 699]
+    for name, args, dense, dead in [
+            ("spfa_local", (w,), so.mask_local_dense(n, w), None),
+            ("spfa_local_1d_dilated", (w, dil), so.mask_local_1d_dilated_dense(n, w, dil), None),
+            ("spfa_local_2d_dilated", (blk, dil, True), so.mask_local_2d_dilated_dense(n, blk, dil), "nan")]:
+        q, k, v, m, l, o = _f64_problem(n, d, 72)
+        mods[name].forward(q, k, v, m, l, o, *args)
+        sync()
+        check(o, m, l, *so.dense_masked_attention(np64(q), np64(k), np64(v), dense), f64, dead_expect=dead)
+    q, k, v, m, l, o = _f64_problem(n, d, 73)
+    mods["spfa_global_no_local"].forward(q, k, v, m, l, o, torch.tensor(globs, dtype=torch.int32, device=DEV), w)
+    sync()
+    dense = so.mask_global_no_local_dense(n, globs, w)
+    check(o, m, l, *so.dense_masked_attention(np64(q), np64(k), np64(v), dense), f64)
+
+
+def test_fp64_chained_calls_accumulate(mods):
+    n, d, w = 512, 32, 12
+    globs = [9, 200]
+    q, k, v, m, l, o = _f64_problem(n, d, 74)
+    mods["spfa_local"].forward(q, k, v, m, l, o, w)
+    mods["spfa_global_no_local"].forward(q, k, v, m, l, o, torch.tensor(globs, dtype=torch.int32, device=DEV), w)
+    sync()
+    dense = so.mask_local_dense(n, w) | so.mask_global_no_local_dense(n, globs, w)
+    check(o, m, l, *so.dense_masked_attention(np64(q), np64(k), np64(v), dense), torch.float64)
+
+
 # ------------------------------------------------------------------ window + global + CSR in one call
 @pytest.mark.parametrize("dtype,d", [(torch.float32, 64), (torch.bfloat16, 64), (torch.float16, 128),
                                       (torch.float32, 40)])
@@ -707,7 +775,7 @@ def test_errors_keep_reference_types_and_texts(mods):
     with pytest.raises(RuntimeError, match="m must be a CUDA tensor"):
         mods["spfa_local"].forward(q, k, v, m.cpu(), l, o, 1)
     with pytest.raises(RuntimeError, match="unsupported element type"):
-        mods["spfa_local"].forward(q.double(), k.double(), v.double(), m.double(), l.double(), o.double(), 1)
+        mods["spfa_local"].forward(q.int(), k.int(), v.int(), m.int(), l.int(), o.int(), 1)
     with pytest.raises(RuntimeError, match="int32"):
         mods["spfa_global_no_local"].forward(q, k, v, m, l, o, g.long(), 1)
     # nothing above may have modified the state
