@@ -4,6 +4,7 @@
 
 #include <limits>
 
+#include "spfa_backward.hpp"
 #include "spfa_f64.hpp"
 #include "spfa_kernels.hpp"
 
@@ -715,6 +716,114 @@ int spfa_window_global_csr_forward(const spfa_problem_t* p, int64_t local_size,
   if (nnz > 0)
     rc = spfa_csr_forward(p, row_off, row_off_bytes, col_ind, nnz, 0, workspace, workspace_bytes, stream);
   return rc;
+}
+
+/* ------------------------------------------------------------------------------ Gradients */
+namespace {
+
+// q, k, v, m, l, out of a finished forward state plus the four gradient tensors.
+int check_grads(const spfa_problem_t* p, const spfa_grads_t* g) {
+  if (g == nullptr) return SPFA_ERR_BAD_ARG;
+  int rc = check_pointers(p);
+  if (rc) return rc;
+  if (p->n_q == 0) return SPFA_OK;
+  if (!g->d_out || !g->d_q || !g->d_k || !g->d_v) return SPFA_ERR_BAD_ARG;
+  return SPFA_OK;
+}
+
+Grads make_grads(const spfa_grads_t* g) { return Grads{g->d_out, g->d_q, g->d_k, g->d_v}; }
+
+}  // namespace
+
+int spfa_csr_backward(const spfa_problem_t* p, const spfa_grads_t* g, const void* row_off,
+                      int row_off_bytes, const void* col_ind, int64_t nnz, void* stream) {
+  int rc = check_problem(p);
+  if (rc) return rc;
+  if (nnz < 0 || (row_off_bytes != 4 && row_off_bytes != 8)) return SPFA_ERR_BAD_ARG;
+  rc = check_grads(p, g);
+  if (rc) return rc;
+  if (p->n_q == 0) return SPFA_OK;
+  if (!row_off || (nnz > 0 && !col_ind)) return SPFA_ERR_BAD_ARG;
+  CsrMask mask{row_off, (const uint32_t*)col_ind, row_off_bytes == 8 ? 1 : 0, nullptr, nullptr};
+  return run_backward_csr(p->dtype, make_tensors(p), mask, make_grads(g), (hipStream_t)stream);
+}
+
+int spfa_coo_backward(const spfa_problem_t* p, const spfa_grads_t* g, const void* row_ind,
+                      int row_ind_bytes, const void* col_ind, int64_t nnz, void* workspace,
+                      size_t workspace_bytes, void* stream) {
+  int rc = check_problem(p);
+  if (rc) return rc;
+  if (nnz < 0 || nnz >= (int64_t)1 << 31 || (row_ind_bytes != 4 && row_ind_bytes != 8))
+    return SPFA_ERR_BAD_ARG;
+  rc = check_grads(p, g);
+  if (rc) return rc;
+  if (p->n_q == 0) return SPFA_OK;
+  if (nnz > 0 && (!row_ind || !col_ind)) return SPFA_ERR_BAD_ARG;
+  const CooWorkspace cw = coo_workspace(p->n_q, nnz);
+  rc = check_workspace(workspace, workspace_bytes, cw.total);
+  if (rc) return rc;
+  CooCsr csr{};
+  rc = coo_to_csr(row_ind, row_ind_bytes == 8 ? 1 : 0, (const uint32_t*)col_ind, nnz, p->n_q,
+                  workspace, (char*)workspace + cw.keep_total, (hipStream_t)stream, &csr);
+  if (rc) return rc;
+  CsrMask mask{csr.row_off, (const uint32_t*)col_ind, 0, csr.cols, csr.unsorted};
+  return run_backward_csr(p->dtype, make_tensors(p), mask, make_grads(g), (hipStream_t)stream);
+}
+
+int spfa_local_backward(const spfa_problem_t* p, const spfa_grads_t* g, int64_t local_size,
+                        void* stream) {
+  return spfa_local_1d_dilated_backward(p, g, local_size, 0, stream);
+}
+
+int spfa_local_1d_dilated_backward(const spfa_problem_t* p, const spfa_grads_t* g,
+                                   int64_t local_size, int64_t dil_factor, void* stream) {
+  int rc = check_problem(p);
+  if (rc) return rc;
+  if (local_size < 0 || local_size > p->n_q - 1) return SPFA_ERR_LOCAL_SIZE;
+  if (dil_factor < 0) return SPFA_ERR_DILATION_NEG;
+  if (dil_factor >= (int64_t)1 << 31) return SPFA_ERR_BAD_ARG;
+  rc = check_grads(p, g);
+  if (rc) return rc;
+  StrideMask mask{p->n_q, local_size, dil_factor + 1, 0, 0};
+  return run_backward_stride(p->dtype, make_tensors(p), mask, make_grads(g), (hipStream_t)stream);
+}
+
+int spfa_local_2d_dilated_backward(const spfa_problem_t* p, const spfa_grads_t* g,
+                                   int64_t block_size, int64_t dil_factor, void* stream) {
+  int rc = check_problem(p);
+  if (rc) return rc;
+  if (block_size <= 0 || p->n_q % block_size != 0) return SPFA_ERR_BLOCK_DIVISOR;
+  if (dil_factor < 0) return SPFA_ERR_DILATION_NEG;
+  if (block_size / (dil_factor + 1) < 1) return SPFA_ERR_BLOCK_DILATION;
+  rc = check_grads(p, g);
+  if (rc) return rc;
+  StrideMask mask{p->n_q, 0, dil_factor + 1, block_size,
+                  block_live_count(block_size, dil_factor + 1)};
+  return run_backward_stride(p->dtype, make_tensors(p), mask, make_grads(g), (hipStream_t)stream);
+}
+
+int spfa_global_no_local_backward(const spfa_problem_t* p, const spfa_grads_t* g,
+                                  const int32_t* global_inds, int64_t n_globals,
+                                  int64_t local_size, void* workspace, size_t workspace_bytes,
+                                  void* stream) {
+  int rc = check_problem(p);
+  if (rc) return rc;
+  if (n_globals <= 0 || n_globals > p->n_q) return SPFA_ERR_GLOBAL_COUNT;
+  if (local_size < 0 || local_size > p->n_q - 1) return SPFA_ERR_LOCAL_SIZE;
+  rc = check_grads(p, g);
+  if (rc) return rc;
+  if (!global_inds) return SPFA_ERR_BAD_ARG;
+  const int64_t n = p->n_q;
+  const GlobalLayout lay = global_layout(n, n_globals, p->d, 1);
+  rc = check_workspace(workspace, workspace_bytes, lay.off_engine);  // the bit map and the row list
+  if (rc) return rc;
+  char* base = (char*)workspace;
+  uint32_t* bits = (uint32_t*)(base + lay.off_bits);
+  rc = prepare_global_rows(global_inds, n_globals, n, bits, (int32_t*)(base + lay.off_uq),
+                           (hipStream_t)stream);
+  if (rc) return rc;
+  GlobalMask mask{n, local_size, global_inds, n_globals, bits};
+  return run_backward_global(p->dtype, make_tensors(p), mask, make_grads(g), (hipStream_t)stream);
 }
 
 }  // extern "C"

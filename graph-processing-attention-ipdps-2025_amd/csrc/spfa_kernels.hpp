@@ -25,4 +25,13 @@ template <typename T>
 int run_global(const Tensors& t, const GlobalMask& mask, const EngineSizing& s, int use_nan,
                void* ws, hipStream_t stream);
 
+// Gradients (spfa_backward.hpp); dtype is the C enum of the element type.
+struct Grads;
+int run_backward_csr(int dtype, const Tensors& t, const CsrMask& mask, const Grads& g,
+                     hipStream_t stream);
+int run_backward_stride(int dtype, const Tensors& t, const StrideMask& mask, const Grads& g,
+                        hipStream_t stream);
+int run_backward_global(int dtype, const Tensors& t, const GlobalMask& mask, const Grads& g,
+                        hipStream_t stream);
+
 }  // namespace spfa

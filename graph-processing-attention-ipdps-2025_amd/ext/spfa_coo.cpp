@@ -93,9 +93,43 @@ torch::Tensor spfa_coo_forward_planned_py(torch::Tensor Q, torch::Tensor K, torc
   return O;
 }
 
+// backward(<the arguments of forward, without use_nan>, dO, dQ, dK, dV) -> (dQ, dK, dV): adds the
+// gradients of the attention this module's forward computes to dQ, dK, dV (float32; float64 for
+// float64 inputs).  m, l, O are the finished forward state.  The reference binds no backward.
+std::tuple<torch::Tensor, torch::Tensor, torch::Tensor> spfa_coo_backward_py(torch::Tensor Q, torch::Tensor K, torch::Tensor V,
+                                                                   torch::Tensor W_row_ind, torch::Tensor W_col_ind,
+                                                                   torch::Tensor W_val, torch::Tensor m, torch::Tensor l,
+                                                                   torch::Tensor O, torch::Tensor dO, torch::Tensor dQ, torch::Tensor dK, torch::Tensor dV) {
+  CHECK_INPUT(Q);
+  CHECK_INPUT(K);
+  CHECK_INPUT(V);
+  CHECK_INPUT(m);
+  CHECK_INPUT(l);
+  CHECK_INPUT(O);
+  SPFA_CHECK_GRAD_INPUTS();
+  CHECK_INPUT(W_row_ind);
+  CHECK_INPUT(W_col_ind);
+  c10::DeviceGuard guard(Q.device());
+  spfa_problem_t p = spfa_ext::make_problem(Q, K, V, m, l, O);
+  spfa_grads_t g = spfa_ext::make_grads(Q, K, dO, dQ, dK, dV);
+  TORCH_CHECK(W_row_ind.dim() == 1 && W_col_ind.dim() == 1 &&
+                  W_row_ind.size(0) == W_col_ind.size(0),
+              "W_row_ind and W_col_ind must be 1-D and of equal length");
+  (void)W_val;
+  const int row_bytes = spfa_ext::index_bytes(W_row_ind, "W_row_ind", true);
+  spfa_ext::index_bytes(W_col_ind, "W_col_ind", false);
+  const int64_t nnz = W_col_ind.size(0);
+  torch::Tensor ws = spfa_ext::make_workspace(spfa_coo_workspace_bytes(p.n_q, nnz, p.d, p.dtype), Q);
+  spfa_ext::raise_on_error(spfa_coo_backward(&p, &g, W_row_ind.data_ptr(), row_bytes, W_col_ind.data_ptr(),
+                                             nnz, ws.data_ptr(), (size_t)ws.numel(),
+                                             spfa_ext::current_stream(Q)));
+  return std::make_tuple(dQ, dK, dV);
+}
+
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, mod) {
   mod.def("forward", &spfa_coo_forward_py, "Sparse-FlashAttention forward, COO mask (HIP, gfx950)");
   mod.def("plan", &spfa_coo_plan_py, "Mask pre-pass of a COO mask, for forward_planned");
   mod.def("forward_planned", &spfa_coo_forward_planned_py,
           "forward(...) with the mask pre-pass taken from plan(...)");
+  mod.def("backward", &spfa_coo_backward_py, "Gradients of forward(...), added to dQ, dK, dV");
 }

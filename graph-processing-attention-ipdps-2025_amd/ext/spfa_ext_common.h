@@ -91,6 +91,35 @@ inline spfa_problem_t make_problem(const torch::Tensor& Q, const torch::Tensor& 
   return p;
 }
 
+// The gradient tensors of a backward call: d_out shaped and typed like Q; d_q like Q, d_k and d_v
+// like K, all three float32 (float64 when Q is float64).  They are added to.
+inline spfa_grads_t make_grads(const torch::Tensor& Q, const torch::Tensor& K, const torch::Tensor& dO,
+                               const torch::Tensor& dQ, const torch::Tensor& dK,
+                               const torch::Tensor& dV) {
+  const auto acc = Q.scalar_type() == torch::kFloat64 ? torch::kFloat64 : torch::kFloat32;
+  TORCH_CHECK(dO.sizes() == Q.sizes() && dO.scalar_type() == Q.scalar_type(),
+              "dO must have the shape and dtype of Q");
+  TORCH_CHECK(dQ.sizes() == Q.sizes() && dK.sizes() == K.sizes() && dV.sizes() == K.sizes(),
+              "dQ must be shaped like Q, dK and dV like K");
+  TORCH_CHECK(dQ.scalar_type() == acc && dK.scalar_type() == acc && dV.scalar_type() == acc,
+              "dQ, dK and dV must be float32 (float64 for float64 inputs)");
+  TORCH_CHECK(dO.device() == Q.device() && dQ.device() == Q.device() && dK.device() == Q.device() &&
+                  dV.device() == Q.device(),
+              "all tensors must be on the same device");
+  spfa_grads_t g;
+  g.d_out = dO.data_ptr();
+  g.d_q = dQ.data_ptr();
+  g.d_k = dK.data_ptr();
+  g.d_v = dV.data_ptr();
+  return g;
+}
+
+#define SPFA_CHECK_GRAD_INPUTS() \
+  CHECK_INPUT(dO);               \
+  CHECK_INPUT(dQ);               \
+  CHECK_INPUT(dK);               \
+  CHECK_INPUT(dV)
+
 // workspace of a (possibly batched) call: the single-problem size times the batch count
 inline size_t batched(size_t bytes, const spfa_problem_t& p) {
   return bytes * (size_t)(p.n_batch > 1 ? p.n_batch : 1);

@@ -26,7 +26,30 @@ torch::Tensor spfa_local_1d_dilated_forward_py(torch::Tensor Q, torch::Tensor K,
   return O;
 }
 
+// backward(<the arguments of forward, without use_nan>, dO, dQ, dK, dV) -> (dQ, dK, dV): adds the
+// gradients of the attention this module's forward computes to dQ, dK, dV (float32; float64 for
+// float64 inputs).  m, l, O are the finished forward state.  The reference binds no backward.
+std::tuple<torch::Tensor, torch::Tensor, torch::Tensor> spfa_local_1d_dilated_backward_py(
+    torch::Tensor Q, torch::Tensor K, torch::Tensor V, torch::Tensor m, torch::Tensor l, torch::Tensor O,
+    int local_size_each_dir, int dil_factor, torch::Tensor dO, torch::Tensor dQ, torch::Tensor dK, torch::Tensor dV) {
+  CHECK_INPUT(Q);
+  CHECK_INPUT(K);
+  CHECK_INPUT(V);
+  CHECK_INPUT(m);
+  CHECK_INPUT(l);
+  CHECK_INPUT(O);
+  SPFA_CHECK_GRAD_INPUTS();
+  c10::DeviceGuard guard(Q.device());
+  spfa_problem_t p = spfa_ext::make_problem(Q, K, V, m, l, O);
+  spfa_grads_t g = spfa_ext::make_grads(Q, K, dO, dQ, dK, dV);
+  TORCH_CHECK(p.n_k == p.n_q, "Q, K and V must have the same number of rows");
+  spfa_ext::raise_on_error(spfa_local_1d_dilated_backward(&p, &g, local_size_each_dir, dil_factor,
+                                                          spfa_ext::current_stream(Q)));
+  return std::make_tuple(dQ, dK, dV);
+}
+
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, mod) {
   mod.def("forward", &spfa_local_1d_dilated_forward_py,
           "Sparse-FlashAttention forward, 1D-dilated local mask (HIP, gfx950)");
+  mod.def("backward", &spfa_local_1d_dilated_backward_py, "Gradients of forward(...), added to dQ, dK, dV");
 }

@@ -193,6 +193,47 @@ int spfa_global_no_local_forward(const spfa_problem_t* p, const int32_t* global_
                                  int64_t n_globals, int64_t local_size, void* workspace,
                                  size_t workspace_bytes, void* stream);
 
+/* ---------------------------------------------------------------------------------------------
+ * Gradients.  The reference has no backward pass (its extensions bind `forward` only,
+ * Sparse_FlashAttention_CSR/sp_flatt_csr.cpp:57-59); these entry points have no counterpart there.
+ * They differentiate the attention the matching *_forward computes: with (m, l, out) the FINISHED
+ * forward state of `p` and d_out the gradient of the loss with respect to out, they ADD
+ *     d_q[i] += sum_j dS_ij k_j / sqrt(d),  d_k[j] += sum_i dS_ij q_i / sqrt(d),
+ *     d_v[j] += sum_i P_ij d_out[i],
+ * where P_ij = exp(q_i.k_j / sqrt(d) - m_i - log l_i) on the live positions of the mask and
+ * dS_ij = P_ij (d_out[i].v_j - d_out[i].out[i]).  A state built by several chained forward calls is
+ * differentiated by one backward call per mask on the same gradient tensors.  Rows with l == 0
+ * (never any live column) carry no gradient.
+ *   d_out        [n_batch * n_q, d], element type of the problem
+ *   d_q          [n_batch * n_q, d]  fp32 (fp64 for F64 problems); the caller zeroes it
+ *   d_k, d_v     [n_batch * n_k, d]  likewise; added to with floating-point atomics, so two runs
+ *                                    may differ in the last bits
+ * Parameter checks and their codes are those of the matching forward call. */
+typedef struct spfa_grads {
+  const void* d_out;
+  void* d_q;
+  void* d_k;
+  void* d_v;
+} spfa_grads_t;
+
+int spfa_csr_backward(const spfa_problem_t* p, const spfa_grads_t* g, const void* row_off,
+                      int row_off_bytes, const void* col_ind, int64_t nnz, void* stream);
+/* workspace: at least spfa_coo_workspace_bytes(n_q, nnz, d, dtype) */
+int spfa_coo_backward(const spfa_problem_t* p, const spfa_grads_t* g, const void* row_ind,
+                      int row_ind_bytes, const void* col_ind, int64_t nnz, void* workspace,
+                      size_t workspace_bytes, void* stream);
+int spfa_local_backward(const spfa_problem_t* p, const spfa_grads_t* g, int64_t local_size,
+                        void* stream);
+int spfa_local_1d_dilated_backward(const spfa_problem_t* p, const spfa_grads_t* g,
+                                   int64_t local_size, int64_t dil_factor, void* stream);
+int spfa_local_2d_dilated_backward(const spfa_problem_t* p, const spfa_grads_t* g,
+                                   int64_t block_size, int64_t dil_factor, void* stream);
+/* workspace: at least spfa_global_no_local_workspace_bytes(n, d, dtype, n_globals, local_size) */
+int spfa_global_no_local_backward(const spfa_problem_t* p, const spfa_grads_t* g,
+                                  const int32_t* global_inds, int64_t n_globals,
+                                  int64_t local_size, void* workspace, size_t workspace_bytes,
+                                  void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -31,6 +31,12 @@ How each function is pinned (none of them is checked against itself):
                                forms are compared with counted nnz.
   * merge_state              - associativity/identity properties and the
                                split-and-chain test.
+  * dense_masked_attention_backward
+                             - torch CPU autograd through the library's
+                               scaled_dot_product_attention in float64, central
+                               finite differences of dense_masked_attention, and
+                               the closed forms "one live column => dq = dk = 0,
+                               dv = d_out" and "sum_j dS_ij == 0".
 """
 from __future__ import annotations
 
@@ -77,6 +83,37 @@ def dense_masked_attention(q, k, v, mask):
 # --------------------------------------------------------------------------
 # running-softmax state (sp_flatt_csr_kernel.cu:79-92, 162-201, 208-218)
 # --------------------------------------------------------------------------
+def dense_masked_attention_backward(q, k, v, mask, d_out):
+    """Gradients of ``dense_masked_attention`` with respect to q, k and v, float64.
+
+    The reference has no backward pass; this is the textbook differentiation of the formulation
+    its verification uses (verification/verify.py:61-63).  With P the masked softmax,
+    ``dV = P^T dO``, ``dP = dO V^T``, ``dS = P * (dP - rowsum(dO * O))``,
+    ``dQ = dS K / sqrt(d)``, ``dK = dS^T Q / sqrt(d)``.  Rows without a live column carry no
+    gradient.
+    """
+    q = np.asarray(q, dtype=np.float64)
+    k = np.asarray(k, dtype=np.float64)
+    v = np.asarray(v, dtype=np.float64)
+    d_out = np.asarray(d_out, dtype=np.float64)
+    mask = np.asarray(mask, dtype=bool)
+    scale = 1.0 / math.sqrt(float(q.shape[1]))
+    s = np.where(mask, (q @ k.T) * scale, NEG_INF)
+    mx = s.max(axis=1)
+    live = np.isfinite(mx)
+    p = np.where(mask, np.exp(s - np.where(live, mx, 0.0)[:, None]), 0.0)
+    den = p.sum(axis=1)
+    p = p / np.where(live, den, 1.0)[:, None]
+    d_out = np.where(live[:, None], d_out, 0.0)
+    out = p @ v
+    d_v = p.T @ d_out
+    d_p = d_out @ v.T
+    d_s = p * (d_p - (d_out * out).sum(axis=1)[:, None])
+    d_q = (d_s @ k) * scale
+    d_k = (d_s.T @ q) * scale
+    return d_q, d_k, d_v
+
+
 def merge_state(m_a, l_a, o_a, m_b, l_b, o_b):
     """Merge two normalised partial results of the same row.
 

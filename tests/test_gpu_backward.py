@@ -1,0 +1,165 @@
+"""GPU parity of the gradient entry points with the float64 oracle (dense masked attention
+differentiated by hand, itself pinned against library autograd and finite differences on the CPU).
+
+The reference has no backward pass, so there is no reference test to mirror; the bars are
+rounding-level for float64, 2e-4 of the gradient's scale for float32 and 3e-2 of it for the half
+types (their q, k, v, out and d_out are rounded to 8 / 11 bits)."""
+import numpy as np
+import pytest
+import torch
+
+import spfa_autograd
+import spfa_synth as syn
+from helpers import np64
+from oracle import spfa_oracle as so
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+GRAD_TOL = {torch.float64: 1e-10, torch.float32: 2e-4, torch.float16: 3e-2, torch.bfloat16: 3e-2}
+
+
+def _problem(n, d, dtype, seed, n_k=None, lead=()):
+    g = torch.Generator().manual_seed(seed)
+    n_k = n if n_k is None else n_k
+    mk = lambda rows: torch.randn(*lead, rows, d, generator=g, dtype=torch.float64).to(dtype).to(DEV)
+    return mk(n), mk(n_k), mk(n_k), mk(n)  # q, k, v, d_out
+
+
+def _check_grads(got, ref, dtype, what):
+    for name, a, b in zip(("dq", "dk", "dv"), got, ref):
+        a = np64(a)
+        scale = max(1.0, float(np.abs(b).max()))
+        err = float(np.abs(a - b).max())
+        assert np.isfinite(a).all(), "%s %s: non-finite gradient" % (what, name)
+        assert err <= GRAD_TOL[dtype] * scale, "%s %s: max-abs error %.3e > %.1e * %.2f" % (
+            what, name, err, GRAD_TOL[dtype], scale)
+
+
+def _grads_of(q, k, v, d_out, parts):
+    q, k, v = (x.clone().requires_grad_(True) for x in (q, k, v))
+    out = spfa_autograd.attention(q, k, v, parts)
+    out.backward(d_out)
+    torch.cuda.synchronize()
+    return out.detach(), (q.grad, k.grad, v.grad)
+
+
+def _csr_part(dense):
+    ro, ci = so.csr_from_dense(dense)
+    return ("csr", torch.as_tensor(ro).to(torch.uint64).to(DEV), torch.as_tensor(ci).to(torch.uint32).to(DEV))
+
+
+def _coo_part(dense, seed):
+    r, c = so.coo_from_dense(dense)
+    perm = np.random.default_rng(seed).permutation(len(r))
+    return ("coo", torch.as_tensor(r[perm]).to(torch.uint64).to(DEV),
+            torch.as_tensor(c[perm]).to(torch.uint32).to(DEV))
+
+
+def _random_mask(n, n_k, seed):
+    rng = np.random.default_rng(seed)
+    dense = rng.random((n, n_k)) < 0.08
+    dense[3] = False           # an empty row
+    dense[4] = False
+    dense[4, n_k // 2] = True  # one live column
+    dense[10] = True           # a full row (several chunks of 64 candidates)
+    return dense
+
+
+@pytest.mark.parametrize("dtype", [torch.float64, torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("d", [64, 40, 200])
+def test_explicit_masks_match_the_oracle(mods, dtype, d):
+    n, n_k = 300, 420
+    q, k, v, d_out = _problem(n, d, dtype, 5, n_k)
+    dense = _random_mask(n, n_k, 6)
+    ref = so.dense_masked_attention_backward(np64(q), np64(k), np64(v), dense, np64(d_out))
+    _, got = _grads_of(q, k, v, d_out, [_csr_part(dense)])
+    _check_grads(got, ref, dtype, "csr")
+    assert not np64(got[0])[3].any()  # the empty row carries nothing
+    _, got = _grads_of(q, k, v, d_out, [_coo_part(dense, 7)])
+    _check_grads(got, ref, dtype, "coo (shuffled)")
+
+
+@pytest.mark.parametrize("dtype", [torch.float64, torch.float32, torch.bfloat16])
+def test_implicit_masks_match_the_oracle(mods, dtype):
+    n, d = 480, 64
+    w, dil, blk = 70, 2, 96
+    globs = [0, 17, 200, 479]
+    gl = torch.tensor(globs, dtype=torch.int32, device=DEV)
+    cases = [
+        ([("local", w)], so.mask_local_dense(n, w)),
+        ([("local", 0)], so.mask_local_dense(n, 0)),
+        ([("local_1d_dilated", w, dil)], so.mask_local_1d_dilated_dense(n, w, dil)),
+        ([("local_2d_dilated", blk, dil)], so.mask_local_2d_dilated_dense(n, blk, dil)),
+        ([("global_no_local", gl, 9)], so.mask_global_no_local_dense(n, globs, 9)),
+    ]
+    for parts, dense in cases:
+        q, k, v, d_out = _problem(n, d, dtype, 11)
+        ref = so.dense_masked_attention_backward(np64(q), np64(k), np64(v), dense, np64(d_out))
+        _, got = _grads_of(q, k, v, d_out, parts)
+        _check_grads(got, ref, dtype, parts[0][0])
+
+
+@pytest.mark.parametrize("dtype", [torch.float64, torch.float32])
+def test_chained_parts_are_differentiated_as_their_union(mods, dtype):
+    """window + global + random, the chain of verification/verify.py:337-352: one backward call
+    per part against the finished state equals the gradient of attention over the union."""
+    n, d, w = 400, 32, 12
+    globs = [5, 250]
+    rng = np.random.default_rng(21)
+    rand = rng.random((n, n)) < 0.03
+    union = so.mask_local_dense(n, w) | so.mask_global_no_local_dense(n, globs, w)
+    rand &= ~union
+    gl = torch.tensor(globs, dtype=torch.int32, device=DEV)
+    q, k, v, d_out = _problem(n, d, dtype, 22)
+    ref = so.dense_masked_attention_backward(np64(q), np64(k), np64(v), union | rand, np64(d_out))
+    out, got = _grads_of(q, k, v, d_out, [("local", w), ("global_no_local", gl, w), _csr_part(rand)])
+    _check_grads(got, ref, dtype, "chain")
+    ref_out = so.dense_masked_attention(np64(q), np64(k), np64(v), union | rand)[0]
+    assert np.abs(np64(out) - ref_out).max() <= (1e-11 if dtype == torch.float64 else 1e-4)
+
+
+def test_batch_of_heads_shares_the_mask(mods):
+    n, d, lead = 200, 64, (2, 3)
+    q, k, v, d_out = _problem(n, d, torch.float32, 31, lead=lead)
+    dense = _random_mask(n, n, 32)
+    _, got = _grads_of(q, k, v, d_out, [_csr_part(dense), ])
+    for b in range(lead[0]):
+        for h in range(lead[1]):
+            ref = so.dense_masked_attention_backward(np64(q[b, h]), np64(k[b, h]), np64(v[b, h]), dense,
+                                                     np64(d_out[b, h]))
+            _check_grads([g[b, h] for g in got], ref, torch.float32, "head %d,%d" % (b, h))
+
+
+def test_gradcheck_float64(mods):
+    """torch's own numerical gradient check through the autograd function (float64; the atomics
+    make two runs differ in the last bits, hence nondet_tol)."""
+    n, d = 24, 8
+    q, k, v, _ = _problem(n, d, torch.float64, 41)
+    dense = np.random.default_rng(42).random((n, n)) < 0.3
+    dense[np.arange(n), np.arange(n)] = False
+    parts = [("local", 0), _csr_part(dense)]
+    q, k, v = (x.requires_grad_(True) for x in (q, k, v))
+    assert torch.autograd.gradcheck(lambda a, b, c: spfa_autograd.attention(a, b, c, parts), (q, k, v),
+                                    eps=1e-6, atol=1e-7, rtol=1e-6, nondet_tol=1e-9)
+
+
+def test_backward_adds_to_the_given_gradients_and_checks_parameters(mods):
+    n, d = 64, 16
+    q, k, v, d_out = _problem(n, d, torch.float32, 51)
+    m = torch.full((n,), -float("inf"), device=DEV)
+    l = torch.zeros(n, device=DEV)
+    o = torch.zeros_like(q)
+    mods["spfa_local"].forward(q, k, v, m, l, o, 3)
+    base = torch.full((n, d), 2.0, device=DEV)
+    dq, dk, dv = base.clone(), base.clone(), base.clone()
+    ret = mods["spfa_local"].backward(q, k, v, m, l, o, 3, d_out, dq, dk, dv)
+    torch.cuda.synchronize()
+    assert ret[0].data_ptr() == dq.data_ptr()
+    ref = so.dense_masked_attention_backward(np64(q), np64(k), np64(v), so.mask_local_dense(n, 3), np64(d_out))
+    _check_grads((dq - 2.0, dk - 2.0, dv - 2.0), ref, torch.float32, "accumulate")
+    with pytest.raises(ValueError, match="local size"):
+        mods["spfa_local"].backward(q, k, v, m, l, o, n, d_out, dq, dk, dv)
+    with pytest.raises(RuntimeError, match="float32"):
+        mods["spfa_local"].backward(q, k, v, m, l, o, 3, d_out, dq.half(), dk, dv)
+    with pytest.raises(RuntimeError, match="dO must have the shape"):
+        mods["spfa_local"].backward(q, k, v, m, l, o, 3, d_out[:-1].contiguous(), dq, dk, dv)

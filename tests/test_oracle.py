@@ -74,6 +74,71 @@ def test_dense_closed_forms():
     np.testing.assert_allclose(out, expect, atol=1e-13)
 
 
+# ---------------------------------------------------------------- gradients of the dense formulation
+@pytest.mark.parametrize("seed,density", [(0, 0.1), (1, 0.5), (2, 1.0)])
+def test_backward_matches_torch_autograd_fp64(seed, density):
+    """Library autograd through the library's SDPA, float64, rows without a live column left out
+    of the loss (torch gives NaN gradients there; the oracle gives them none)."""
+    n, n_k, d = 48, 40, 16
+    q, k, v = _rand(n, d, seed, n_k)
+    rng = np.random.default_rng(200 + seed)
+    mask = rng.random((n, n_k)) < density
+    mask[5, :] = False
+    mask[6, :] = False
+    mask[6, 3] = True  # a single live column
+    d_out = rng.standard_normal((n, d))
+    tq, tk, tv = (torch.tensor(x, requires_grad=True) for x in (q, k, v))
+    live = torch.tensor(mask.any(axis=1))
+    out = torch.nn.functional.scaled_dot_product_attention(tq[live], tk, tv,
+                                                           attn_mask=torch.tensor(mask)[live])
+    (out * torch.tensor(d_out)[live]).sum().backward()
+    d_q, d_k, d_v = so.dense_masked_attention_backward(q, k, v, mask, d_out)
+    np.testing.assert_allclose(d_q, tq.grad.numpy(), rtol=0, atol=1e-12)
+    np.testing.assert_allclose(d_k, tk.grad.numpy(), rtol=0, atol=1e-12)
+    np.testing.assert_allclose(d_v, tv.grad.numpy(), rtol=0, atol=1e-12)
+    assert not d_q[5].any()  # dead row
+    np.testing.assert_allclose(d_q[6], 0, atol=1e-13)  # one live column: the softmax is constant
+
+
+def test_backward_matches_finite_differences_of_the_forward_oracle():
+    n, d = 12, 4
+    q, k, v = _rand(n, d, 9)
+    rng = np.random.default_rng(10)
+    mask = rng.random((n, n)) < 0.4
+    mask[np.arange(n), np.arange(n)] = True
+    d_out = rng.standard_normal((n, d))
+    loss = lambda a, b, c: float((so.dense_masked_attention(a, b, c, mask)[0] * d_out).sum())
+    grads = so.dense_masked_attention_backward(q, k, v, mask, d_out)
+    eps = 1e-6
+    for which, g in enumerate(grads):
+        num = np.zeros_like(g)
+        for i in range(n):
+            for e in range(d):
+                args = [q.copy(), k.copy(), v.copy()]
+                args[which][i, e] += eps
+                up = loss(*args)
+                args[which][i, e] -= 2 * eps
+                num[i, e] = (up - loss(*args)) / (2 * eps)
+        np.testing.assert_allclose(g, num, rtol=0, atol=1e-7)
+
+
+def test_backward_closed_forms():
+    n, d = 30, 8
+    q, k, v = _rand(n, d, 11)
+    d_out = np.random.default_rng(12).standard_normal((n, d))
+    # window 0: out == v, so dv == d_out and nothing flows to q or k
+    d_q, d_k, d_v = so.dense_masked_attention_backward(q, k, v, np.eye(n, dtype=bool), d_out)
+    np.testing.assert_allclose(d_q, 0, atol=1e-13)
+    np.testing.assert_allclose(d_k, 0, atol=1e-13)
+    np.testing.assert_allclose(d_v, d_out, atol=1e-15)
+    # V == 1 on a full mask: out == 1 whatever q and k are, so dq == dk == 0 and dv sums d_out
+    full = np.ones((n, n), dtype=bool)
+    d_q, d_k, d_v = so.dense_masked_attention_backward(q, k, np.ones_like(v), full, d_out)
+    np.testing.assert_allclose(d_q, 0, atol=1e-13)
+    np.testing.assert_allclose(d_k, 0, atol=1e-13)
+    np.testing.assert_allclose(d_v.sum(axis=0), d_out.sum(axis=0), atol=1e-12)
+
+
 def test_scale_rule_is_one_over_sqrt_d():
     # one query, two keys with a known score gap: weights must be sigmoid(gap / sqrt(d))
     d = 16
