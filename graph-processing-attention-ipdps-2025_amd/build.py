@@ -55,8 +55,12 @@ def lib_jobs():
             jobs.append((obj, [HIPCC, *HIP_FLAGS, "-DSPFA_INST_MASK=%d" % mid,
                                "-DSPFA_INST_T=%s" % tcpp, "-c",
                                os.path.join(CSRC, "spfa_inst.hip"), "-o", obj]))
+            obj = os.path.join(OBJ, "grad_%s_%s.o" % (mname, tname))
+            jobs.append((obj, [HIPCC, *HIP_FLAGS, "-DSPFA_INST_MASK=%d" % mid,
+                               "-DSPFA_INST_T=%s" % tcpp, "-c",
+                               os.path.join(CSRC, "spfa_grad_inst.hip"), "-o", obj]))
     for src in sorted(os.listdir(CSRC)):
-        if src.endswith(".hip") and src != "spfa_inst.hip":
+        if src.endswith(".hip") and src not in ("spfa_inst.hip", "spfa_grad_inst.hip"):
             obj = os.path.join(OBJ, src[:-4] + ".o")
             jobs.append((obj, [HIPCC, *HIP_FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]))
     return jobs

@@ -5,6 +5,7 @@
 #include <limits>
 
 #include "spfa_backward.hpp"
+#include "spfa_grad.hpp"
 #include "spfa_f64.hpp"
 #include "spfa_kernels.hpp"
 
@@ -721,6 +722,8 @@ int spfa_window_global_csr_forward(const spfa_problem_t* p, int64_t local_size,
 /* ------------------------------------------------------------------------------ Gradients */
 namespace {
 
+constexpr int64_t kGradSegment = 1024;  // candidates one wavefront takes of an owner row
+
 // q, k, v, m, l, out of a finished forward state plus the four gradient tensors.
 int check_grads(const spfa_problem_t* p, const spfa_grads_t* g) {
   if (g == nullptr) return SPFA_ERR_BAD_ARG;
@@ -733,19 +736,159 @@ int check_grads(const spfa_problem_t* p, const spfa_grads_t* g) {
 
 Grads make_grads(const spfa_grads_t* g) { return Grads{g->d_out, g->d_q, g->d_k, g->d_v}; }
 
+// Workspace of a gradient call: lse and delta of every query row, the two lists of (owner,
+// segment) items of long rows, then whatever the mask needs (`mask_bytes`).
+struct GradLayout {
+  size_t off_lse, off_delta, off_cnt, off_items, off_mask, total;
+  uint32_t cap_items;
+  bool ok;
+};
+
+// items_bound: most (owner, segment) items one pass can leave behind, per problem
+GradLayout grad_layout(int64_t n_q, int64_t n_batch, int64_t items_bound, size_t mask_bytes) {
+  GradLayout g{};
+  const int64_t b = n_batch > 1 ? n_batch : 1;
+  const int64_t cap = items_bound * b + 1;
+  g.ok = cap < ((int64_t)1 << 31);
+  g.cap_items = (uint32_t)(g.ok ? cap : 1);
+  size_t off = 0;
+  g.off_lse = off;   off = align_up(off + (size_t)(n_q * b) * 4, 256);
+  g.off_delta = off; off = align_up(off + (size_t)(n_q * b) * 4, 256);
+  g.off_cnt = off;   off += 256;
+  g.off_items = off; off = align_up(off + (size_t)g.cap_items * 16, 256);  // two lists of pairs
+  g.off_mask = off;  off = align_up(off + mask_bytes, 256);
+  g.total = off;
+  return g;
+}
+
+int64_t explicit_items_bound(int64_t nnz) { return nnz / kGradSegment + 1; }
+int64_t uniform_items_bound(int64_t n_rows, int64_t max_deg) {
+  return max_deg > kGradSegment ? n_rows * ((max_deg - 1) / kGradSegment) : 0;
+}
+int64_t global_items_bound(int64_t n, int64_t n_globals) {
+  return n_globals * ((n - 1) / kGradSegment) + uniform_items_bound(n, n_globals);
+}
+
+// what the transposed explicit mask needs: the entry list (rows, columns) and the conversion
+struct TransposeLayout {
+  size_t off_rows, off_cols, off_coo, total;
+};
+TransposeLayout transpose_layout(int64_t n_k, int64_t nnz) {
+  TransposeLayout t{};
+  size_t off = 0;
+  t.off_rows = off; off = align_up(off + (size_t)nnz * 4, 256);
+  t.off_cols = off; off = align_up(off + (size_t)nnz * 4, 256);
+  t.off_coo = off;  off = align_up(off + coo_workspace(n_k, nnz).total, 256);
+  t.total = off;
+  return t;
+}
+
+GradArgs make_grad_args(const spfa_problem_t* p, const spfa_grads_t* g, const GradLayout& lay,
+                        void* workspace) {
+  char* base = (char*)workspace;
+  GradArgs a{};
+  a.q = p->q;
+  a.k = p->k;
+  a.v = p->v;
+  a.d_out = g->d_out;
+  a.lse = (float*)(base + lay.off_lse);
+  a.delta = (float*)(base + lay.off_delta);
+  a.d_q = (float*)g->d_q;
+  a.d_k = (float*)g->d_k;
+  a.d_v = (float*)g->d_v;
+  a.n_q = p->n_q;
+  a.n_k = p->n_k;
+  a.n_batch = batch_of(p);
+  a.d = (int32_t)p->d;
+  a.seg = (int32_t)kGradSegment;
+  a.n_items = (uint32_t*)(base + lay.off_cnt);
+  a.items = (uint32_t*)(base + lay.off_items);
+  a.cap_items = lay.cap_items;
+  return a;
+}
+
+// Gradients through an explicit mask given as a CsrMask over the query rows: transpose it (entry
+// list -> bucketed by column), then the two passes.
+int explicit_backward(const spfa_problem_t* p, const spfa_grads_t* g, const CsrMask& rows, int64_t nnz,
+                      const GradLayout& lay, void* workspace, hipStream_t stream) {
+  if (is_f64(p)) return run_backward_csr(p->dtype, make_tensors(p), rows, make_grads(g), stream);
+  char* mbase = (char*)workspace + lay.off_mask;
+  const TransposeLayout tl = transpose_layout(p->n_k, nnz);
+  uint32_t* e_rows = (uint32_t*)(mbase + tl.off_rows);
+  uint32_t* e_cols = (uint32_t*)(mbase + tl.off_cols);
+  int rc = csr_entry_list(rows.row_off, rows.off64, rows.cols, rows.alt_cols, rows.use_alt, p->n_q,
+                          e_rows, e_cols, stream);
+  if (rc) return rc;
+  const CooWorkspace cw = coo_workspace(p->n_k, nnz);
+  CooCsr tr{};
+  rc = coo_to_csr(e_cols, 0, e_rows, nnz, p->n_k, mbase + tl.off_coo, mbase + tl.off_coo + cw.keep_total,
+                  stream, &tr);
+  if (rc) return rc;
+  CsrMask cols{tr.row_off, e_rows, 0, tr.cols, tr.unsorted};
+  const GradArgs a = make_grad_args(p, g, lay, workspace);
+  const Tensors t = make_tensors(p);
+  switch (p->dtype) {
+    case SPFA_DTYPE_F32: return run_grad_csr<float>(t, a, rows, cols, stream);
+    case SPFA_DTYPE_F16: return run_grad_csr<f16>(t, a, rows, cols, stream);
+    case SPFA_DTYPE_BF16: return run_grad_csr<bf16>(t, a, rows, cols, stream);
+  }
+  return SPFA_ERR_UNSUPPORTED;
+}
+
+int stride_backward(const spfa_problem_t* p, const spfa_grads_t* g, const StrideMask& mask,
+                    const GradLayout& lay, void* workspace, hipStream_t stream) {
+  if (is_f64(p)) return run_backward_stride(p->dtype, make_tensors(p), mask, make_grads(g), stream);
+  const GradArgs a = make_grad_args(p, g, lay, workspace);
+  const Tensors t = make_tensors(p);
+  switch (p->dtype) {
+    case SPFA_DTYPE_F32: return run_grad_stride<float>(t, a, mask, stream);
+    case SPFA_DTYPE_F16: return run_grad_stride<f16>(t, a, mask, stream);
+    case SPFA_DTYPE_BF16: return run_grad_stride<bf16>(t, a, mask, stream);
+  }
+  return SPFA_ERR_UNSUPPORTED;
+}
+
+size_t global_mask_bytes(int64_t n, int64_t n_globals) {
+  return align_up(global_bits_words(n) * 4, 256) + align_up((size_t)n_globals * 4, 256);
+}
+
 }  // namespace
 
+size_t spfa_csr_backward_workspace_bytes(int64_t n_q, int64_t n_k, int64_t nnz, int64_t d, int dtype,
+                                         int64_t n_batch) {
+  (void)d;
+  (void)dtype;
+  if (n_q < 0 || n_k < 0 || nnz < 0) return 0;
+  return grad_layout(n_q, n_batch, explicit_items_bound(nnz), transpose_layout(n_k, nnz).total).total;
+}
+
 int spfa_csr_backward(const spfa_problem_t* p, const spfa_grads_t* g, const void* row_off,
-                      int row_off_bytes, const void* col_ind, int64_t nnz, void* stream) {
+                      int row_off_bytes, const void* col_ind, int64_t nnz, void* workspace,
+                      size_t workspace_bytes, void* stream) {
   int rc = check_problem(p);
   if (rc) return rc;
-  if (nnz < 0 || (row_off_bytes != 4 && row_off_bytes != 8)) return SPFA_ERR_BAD_ARG;
+  if (nnz < 0 || nnz >= (int64_t)1 << 31 || (row_off_bytes != 4 && row_off_bytes != 8))
+    return SPFA_ERR_BAD_ARG;
   rc = check_grads(p, g);
   if (rc) return rc;
-  if (p->n_q == 0) return SPFA_OK;
-  if (!row_off || (nnz > 0 && !col_ind)) return SPFA_ERR_BAD_ARG;
-  CsrMask mask{row_off, (const uint32_t*)col_ind, row_off_bytes == 8 ? 1 : 0, nullptr, nullptr};
-  return run_backward_csr(p->dtype, make_tensors(p), mask, make_grads(g), (hipStream_t)stream);
+  if (p->n_q == 0 || nnz == 0) return SPFA_OK;
+  if (!row_off || !col_ind) return SPFA_ERR_BAD_ARG;
+  const GradLayout lay =
+      grad_layout(p->n_q, batch_of(p), explicit_items_bound(nnz), transpose_layout(p->n_k, nnz).total);
+  if (!lay.ok) return SPFA_ERR_BAD_ARG;
+  rc = check_workspace(workspace, workspace_bytes, lay.total);
+  if (rc) return rc;
+  CsrMask rows{row_off, (const uint32_t*)col_ind, row_off_bytes == 8 ? 1 : 0, nullptr, nullptr};
+  return explicit_backward(p, g, rows, nnz, lay, workspace, (hipStream_t)stream);
+}
+
+size_t spfa_coo_backward_workspace_bytes(int64_t n_q, int64_t n_k, int64_t nnz, int64_t d, int dtype,
+                                         int64_t n_batch) {
+  (void)d;
+  (void)dtype;
+  if (n_q < 0 || n_k < 0 || nnz < 0) return 0;
+  const size_t mask_bytes = align_up(coo_workspace(n_q, nnz).total, 256) + transpose_layout(n_k, nnz).total;
+  return grad_layout(n_q, n_batch, explicit_items_bound(nnz), mask_bytes).total;
 }
 
 int spfa_coo_backward(const spfa_problem_t* p, const spfa_grads_t* g, const void* row_ind,
@@ -757,26 +900,49 @@ int spfa_coo_backward(const spfa_problem_t* p, const spfa_grads_t* g, const void
     return SPFA_ERR_BAD_ARG;
   rc = check_grads(p, g);
   if (rc) return rc;
-  if (p->n_q == 0) return SPFA_OK;
-  if (nnz > 0 && (!row_ind || !col_ind)) return SPFA_ERR_BAD_ARG;
+  if (p->n_q == 0 || nnz == 0) return SPFA_OK;
+  if (!row_ind || !col_ind) return SPFA_ERR_BAD_ARG;
   const CooWorkspace cw = coo_workspace(p->n_q, nnz);
-  rc = check_workspace(workspace, workspace_bytes, cw.total);
+  const size_t fwd_bytes = align_up(cw.total, 256);
+  GradLayout lay = grad_layout(p->n_q, batch_of(p), explicit_items_bound(nnz),
+                               fwd_bytes + transpose_layout(p->n_k, nnz).total);
+  if (!lay.ok) return SPFA_ERR_BAD_ARG;
+  rc = check_workspace(workspace, workspace_bytes, lay.total);
   if (rc) return rc;
+  // the mask by query row first (as the forward call does), then as an explicit CSR mask
+  char* fwd = (char*)workspace + lay.off_mask;
   CooCsr csr{};
-  rc = coo_to_csr(row_ind, row_ind_bytes == 8 ? 1 : 0, (const uint32_t*)col_ind, nnz, p->n_q,
-                  workspace, (char*)workspace + cw.keep_total, (hipStream_t)stream, &csr);
+  rc = coo_to_csr(row_ind, row_ind_bytes == 8 ? 1 : 0, (const uint32_t*)col_ind, nnz, p->n_q, fwd,
+                  fwd + cw.keep_total, (hipStream_t)stream, &csr);
   if (rc) return rc;
-  CsrMask mask{csr.row_off, (const uint32_t*)col_ind, 0, csr.cols, csr.unsorted};
-  return run_backward_csr(p->dtype, make_tensors(p), mask, make_grads(g), (hipStream_t)stream);
+  CsrMask rows{csr.row_off, (const uint32_t*)col_ind, 0, csr.cols, csr.unsorted};
+  lay.off_mask += fwd_bytes;
+  return explicit_backward(p, g, rows, nnz, lay, workspace, (hipStream_t)stream);
+}
+
+size_t spfa_local_backward_workspace_bytes(int64_t n, int64_t d, int dtype, int64_t local_size,
+                                           int64_t n_batch) {
+  (void)d;
+  (void)dtype;
+  if (n < 1 || local_size < 0) return 0;
+  return grad_layout(n, n_batch, uniform_items_bound(n, band_max_deg(n, local_size)), 0).total;
 }
 
 int spfa_local_backward(const spfa_problem_t* p, const spfa_grads_t* g, int64_t local_size,
-                        void* stream) {
-  return spfa_local_1d_dilated_backward(p, g, local_size, 0, stream);
+                        void* workspace, size_t workspace_bytes, void* stream) {
+  return spfa_local_1d_dilated_backward(p, g, local_size, 0, workspace, workspace_bytes, stream);
+}
+
+size_t spfa_local_1d_dilated_backward_workspace_bytes(int64_t n, int64_t d, int dtype,
+                                                      int64_t local_size, int64_t dil_factor,
+                                                      int64_t n_batch) {
+  (void)dil_factor;
+  return spfa_local_backward_workspace_bytes(n, d, dtype, local_size, n_batch);
 }
 
 int spfa_local_1d_dilated_backward(const spfa_problem_t* p, const spfa_grads_t* g,
-                                   int64_t local_size, int64_t dil_factor, void* stream) {
+                                   int64_t local_size, int64_t dil_factor, void* workspace,
+                                   size_t workspace_bytes, void* stream) {
   int rc = check_problem(p);
   if (rc) return rc;
   if (local_size < 0 || local_size > p->n_q - 1) return SPFA_ERR_LOCAL_SIZE;
@@ -784,12 +950,30 @@ int spfa_local_1d_dilated_backward(const spfa_problem_t* p, const spfa_grads_t* 
   if (dil_factor >= (int64_t)1 << 31) return SPFA_ERR_BAD_ARG;
   rc = check_grads(p, g);
   if (rc) return rc;
-  StrideMask mask{p->n_q, local_size, dil_factor + 1, 0, 0};
-  return run_backward_stride(p->dtype, make_tensors(p), mask, make_grads(g), (hipStream_t)stream);
+  if (p->n_k != p->n_q) return SPFA_ERR_BAD_ARG;
+  const int64_t n = p->n_q;
+  const GradLayout lay =
+      grad_layout(n, batch_of(p), uniform_items_bound(n, band_max_deg(n, local_size)), 0);
+  if (!lay.ok) return SPFA_ERR_BAD_ARG;
+  rc = check_workspace(workspace, workspace_bytes, lay.total);
+  if (rc) return rc;
+  StrideMask mask{n, local_size, dil_factor + 1, 0, 0};
+  return stride_backward(p, g, mask, lay, workspace, (hipStream_t)stream);
+}
+
+size_t spfa_local_2d_dilated_backward_workspace_bytes(int64_t n, int64_t d, int dtype,
+                                                      int64_t block_size, int64_t dil_factor,
+                                                      int64_t n_batch) {
+  (void)d;
+  (void)dtype;
+  if (n < 1 || block_size < 1 || dil_factor < 0) return 0;
+  return grad_layout(n, n_batch, uniform_items_bound(n, block_live_count(block_size, dil_factor + 1)), 0)
+      .total;
 }
 
 int spfa_local_2d_dilated_backward(const spfa_problem_t* p, const spfa_grads_t* g,
-                                   int64_t block_size, int64_t dil_factor, void* stream) {
+                                   int64_t block_size, int64_t dil_factor, void* workspace,
+                                   size_t workspace_bytes, void* stream) {
   int rc = check_problem(p);
   if (rc) return rc;
   if (block_size <= 0 || p->n_q % block_size != 0) return SPFA_ERR_BLOCK_DIVISOR;
@@ -797,9 +981,26 @@ int spfa_local_2d_dilated_backward(const spfa_problem_t* p, const spfa_grads_t* 
   if (block_size / (dil_factor + 1) < 1) return SPFA_ERR_BLOCK_DILATION;
   rc = check_grads(p, g);
   if (rc) return rc;
-  StrideMask mask{p->n_q, 0, dil_factor + 1, block_size,
-                  block_live_count(block_size, dil_factor + 1)};
-  return run_backward_stride(p->dtype, make_tensors(p), mask, make_grads(g), (hipStream_t)stream);
+  if (p->n_k != p->n_q) return SPFA_ERR_BAD_ARG;
+  const int64_t n = p->n_q;
+  if (n == 0) return SPFA_OK;
+  const int64_t cnt = block_live_count(block_size, dil_factor + 1);
+  const GradLayout lay = grad_layout(n, batch_of(p), uniform_items_bound(n, cnt), 0);
+  if (!lay.ok) return SPFA_ERR_BAD_ARG;
+  rc = check_workspace(workspace, workspace_bytes, lay.total);
+  if (rc) return rc;
+  StrideMask mask{n, 0, dil_factor + 1, block_size, cnt};
+  return stride_backward(p, g, mask, lay, workspace, (hipStream_t)stream);
+}
+
+size_t spfa_global_no_local_backward_workspace_bytes(int64_t n, int64_t d, int dtype,
+                                                     int64_t n_globals, int64_t local_size,
+                                                     int64_t n_batch) {
+  (void)d;
+  (void)dtype;
+  (void)local_size;
+  if (n < 1 || n_globals < 1) return 0;
+  return grad_layout(n, n_batch, global_items_bound(n, n_globals), global_mask_bytes(n, n_globals)).total;
 }
 
 int spfa_global_no_local_backward(const spfa_problem_t* p, const spfa_grads_t* g,
@@ -812,18 +1013,30 @@ int spfa_global_no_local_backward(const spfa_problem_t* p, const spfa_grads_t* g
   if (local_size < 0 || local_size > p->n_q - 1) return SPFA_ERR_LOCAL_SIZE;
   rc = check_grads(p, g);
   if (rc) return rc;
-  if (!global_inds) return SPFA_ERR_BAD_ARG;
+  if (!global_inds || p->n_k != p->n_q) return SPFA_ERR_BAD_ARG;
   const int64_t n = p->n_q;
-  const GlobalLayout lay = global_layout(n, n_globals, p->d, 1);
-  rc = check_workspace(workspace, workspace_bytes, lay.off_engine);  // the bit map and the row list
+  const GradLayout lay =
+      grad_layout(n, batch_of(p), global_items_bound(n, n_globals), global_mask_bytes(n, n_globals));
+  if (!lay.ok) return SPFA_ERR_BAD_ARG;
+  rc = check_workspace(workspace, workspace_bytes, lay.total);
   if (rc) return rc;
-  char* base = (char*)workspace;
-  uint32_t* bits = (uint32_t*)(base + lay.off_bits);
-  rc = prepare_global_rows(global_inds, n_globals, n, bits, (int32_t*)(base + lay.off_uq),
-                           (hipStream_t)stream);
+  char* mbase = (char*)workspace + lay.off_mask;
+  uint32_t* bits = (uint32_t*)mbase;
+  int32_t* uq = (int32_t*)(mbase + align_up(global_bits_words(n) * 4, 256));
+  rc = prepare_global_rows(global_inds, n_globals, n, bits, uq, (hipStream_t)stream);
   if (rc) return rc;
-  GlobalMask mask{n, local_size, global_inds, n_globals, bits};
-  return run_backward_global(p->dtype, make_tensors(p), mask, make_grads(g), (hipStream_t)stream);
+  GlobalMask rows{n, local_size, global_inds, n_globals, bits};
+  if (is_f64(p))
+    return run_backward_global(p->dtype, make_tensors(p), rows, make_grads(g), (hipStream_t)stream);
+  GlobalColMask cols{n, local_size, global_inds, n_globals, bits, uq, bits + (global_bits_words(n) - 1)};
+  const GradArgs a = make_grad_args(p, g, lay, workspace);
+  const Tensors t = make_tensors(p);
+  switch (p->dtype) {
+    case SPFA_DTYPE_F32: return run_grad_global<float>(t, a, rows, cols, (hipStream_t)stream);
+    case SPFA_DTYPE_F16: return run_grad_global<f16>(t, a, rows, cols, (hipStream_t)stream);
+    case SPFA_DTYPE_BF16: return run_grad_global<bf16>(t, a, rows, cols, (hipStream_t)stream);
+  }
+  return SPFA_ERR_UNSUPPORTED;
 }
 
 }  // extern "C"

@@ -1,0 +1,361 @@
+// Gradients of masked attention by two gather passes, no atomics on the hot path (the reference
+// has no backward pass; the m and l it leaves behind are the statistics one needs).
+//
+// With lse_i = m_i + log l_i, p_ij = exp(q_i.k_j / sqrt(d) - lse_i) on live positions,
+// delta_i = dO_i . O_i and dS_ij = p_ij (dO_i . v_j - delta_i) / sqrt(d):
+//     query pass, owner = query row i, candidates = its live columns j (gathers K_j, V_j):
+//         dQ_i += sum_j dS_ij k_j
+//     key pass, owner = key row j, candidates = the query rows i that attend it (gathers Q_i,
+//     dO_i, lse_i, delta_i):
+//         dK_j += sum_i dS_ij q_i          dV_j += sum_i p_ij dO_i
+// The key pass walks the mask by column: the implicit masks are symmetric and answer that with
+// the same functor (the global mask with a column functor that knows about repeated list
+// entries), an explicit mask is transposed first (spfa_api.hip).
+//
+// Both passes are one kernel template.  One wavefront per owner row: the row's two vectors sit in
+// registers, replicated in every lane group; each group of LPR lanes takes one candidate at a
+// time (16 bytes per lane of each of its two rows, U candidates in flight per group), does both
+// dot products with in-group reductions and adds the weighted candidate rows to its
+// accumulators; the groups are summed at the end.  Owners with more than `seg` candidates do
+// their first `seg` here and leave (owner, segment) items behind for grad_items_kernel, whose
+// results are added with floating-point atomics (a few rows only).
+#pragma once
+
+#include "spfa_engine.hpp"
+#include "spfa_masks.hpp"
+
+namespace spfa {
+
+struct GradArgs {
+  const void* q;      // element type T; [n_batch, n_q, d]
+  const void* k;      // [n_batch, n_k, d]
+  const void* v;
+  const void* d_out;  // [n_batch, n_q, d]
+  float* lse;         // [n_batch * n_q]  m + log l, +inf for rows that never saw a live column
+  float* delta;       // [n_batch * n_q]  dO . O (0 for those rows)
+  float* d_q;         // fp32 gradients, added to
+  float* d_k;
+  float* d_v;
+  int64_t n_q;
+  int64_t n_k;
+  int64_t n_batch;
+  int32_t d;
+  int32_t seg;          // candidates one wavefront takes of a row
+  uint32_t* n_items;    // [2] counters of the two item lists (query pass, key pass)
+  uint32_t* items;      // [2][cap_items] pairs (owner among all problems, segment)
+  uint32_t cap_items;
+};
+
+constexpr int kGradWaves = 4;        // owners per workgroup
+constexpr int kGradItemBlocks = 2048;
+
+template <class Lay>
+__device__ __forceinline__ int grad_elem_index(int c, int e) {
+  return (Lay::LPR == kWave) ? c + e * kWave : c * Lay::NE + e;
+}
+
+// lse and delta of every query row
+template <typename T>
+__global__ __launch_bounds__(256) void grad_prologue_kernel(Tensors t, GradArgs g) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= t.n_q * t.n_batch) return;
+  const bool sf = t.state_f32 != 0;
+  const float m = load_state<T>(t.m, row, sf);
+  const float l = load_state<T>(t.l, row, sf);
+  const bool live = l > 0.f;
+  float acc = 0.f;
+  if (live) {
+    const T* orow = (const T*)t.out + row * t.d;
+    const T* drow = (const T*)g.d_out + row * t.d;
+    for (int e = lane; e < t.d; e += kWave) acc += to_f32(orow[e]) * to_f32(drow[e]);
+  }
+  acc = group_sum<kWave>(acc);
+  if (lane == 0) {
+    g.lse[row] = live ? m + __logf(l) : __builtin_inff();
+    g.delta[row] = live ? acc : 0.f;
+  }
+}
+
+static __global__ void grad_reset_kernel(uint32_t* n_items) {
+  if (threadIdx.x < 2) n_items[threadIdx.x] = 0;
+}
+
+// Candidates t_begin .. t_end of one owner, walked by the whole wavefront.
+//   KEYS == false: owner is a query row, (a, b) = (q_i, dO_i), X = K, Y = V, and lse_o / delta_o
+//                  are the owner's; acc1 collects dQ_i.
+//   KEYS == true:  owner is a key row, (a, b) = (k_j, v_j), X = Q, Y = dO, lse / delta are read
+//                  per candidate; acc1 collects dK_j, acc2 dV_j.
+template <class Lay, class Mask, bool KEYS, int U_>
+__device__ __forceinline__ void grad_walk(const Mask& mask, const typename Mask::Row& rc,
+                                          const typename Lay::elem* __restrict__ X,
+                                          const typename Lay::elem* __restrict__ Y,
+                                          const float* __restrict__ lse_c,
+                                          const float* __restrict__ delta_c, float lse_o,
+                                          float delta_o, int d, float scale,
+                                          const float (&a)[Lay::NE], const float (&b)[Lay::NE],
+                                          int64_t t_begin, int64_t t_end, int lane,
+                                          float (&acc1)[Lay::NE], float (&acc2)[Lay::NE]) {
+  constexpr int NE = Lay::NE;
+  constexpr int LPR = Lay::LPR;
+  constexpr int GS = kWave / LPR;
+  constexpr int U = (U_ * GS > kWave) ? kWave / GS : U_;
+  constexpr int PER = U * GS;
+  constexpr int PARTS = kWave / PER;
+  const int gi = lane / LPR;
+  const int c = lane % LPR;
+
+  auto fetch = [&](int64_t t) -> int {
+    const int64_t tt = t + lane;
+    bool valid = tt < t_end;
+    int64_t col = 0;
+    if (valid) col = mask.col(rc, tt, valid);
+    return valid ? (int)col : -1;
+  };
+
+  int next = fetch(t_begin);
+  for (int64_t tb = t_begin; tb < t_end; tb += kWave) {
+    const int cur = next;
+    if (tb + kWave < t_end) next = fetch(tb + kWave);
+#pragma unroll 1
+    for (int part = 0; part < PARTS; part++) {
+      if (tb + part * PER >= t_end) break;
+      int cols[U];
+#pragma unroll
+      for (int u = 0; u < U; u++) cols[u] = shfl_i32(cur, part * PER + u * GS + gi);
+      typename Lay::raw xr[U], yr[U];
+      float ls[U], dl[U];
+#pragma unroll
+      for (int u = 0; u < U; u++) {
+        ls[u] = lse_o;
+        dl[u] = delta_o;
+        if (cols[u] >= 0) {
+          xr[u] = Lay::load_gather(X + (int64_t)cols[u] * d, c, d);
+          yr[u] = Lay::load_gather(Y + (int64_t)cols[u] * d, c, d);
+          if constexpr (KEYS) {
+            ls[u] = lse_c[cols[u]];
+            dl[u] = delta_c[cols[u]];
+          }
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < U; u++) {
+        float xf[NE], yf[NE];
+        float s = 0.f, t = 0.f;
+        if (cols[u] >= 0) {
+          Lay::unpack(xr[u], xf);
+          Lay::unpack(yr[u], yf);
+#pragma unroll
+          for (int e = 0; e < NE; e++) {
+            s += a[e] * xf[e];
+            t += b[e] * yf[e];
+          }
+        }
+        s = group_sum<LPR>(s);
+        t = group_sum<LPR>(t);
+        if (cols[u] >= 0) {
+          float p = __expf(s * scale - ls[u]);
+          if constexpr (Mask::kWeighted) p *= mask.weight(rc, (int64_t)cols[u]);
+          const float ds = p * (t - dl[u]) * scale;
+#pragma unroll
+          for (int e = 0; e < NE; e++) acc1[e] += ds * xf[e];
+          if constexpr (KEYS) {
+#pragma unroll
+            for (int e = 0; e < NE; e++) acc2[e] += p * yf[e];
+          }
+        }
+      }
+    }
+  }
+  // every group has walked its share: add the groups up (group 0 ends up with the total too)
+#pragma unroll
+  for (int off = LPR; off < kWave; off <<= 1) {
+#pragma unroll
+    for (int e = 0; e < NE; e++) {
+      acc1[e] += shfl_xor_f32(acc1[e], off);
+      if constexpr (KEYS) acc2[e] += shfl_xor_f32(acc2[e], off);
+    }
+  }
+}
+
+// What one owner (row `r` among all problems) needs: pointers of its pass.
+template <class Lay, bool KEYS>
+struct GradOwner {
+  using T = typename Lay::elem;
+  const T* X;
+  const T* Y;
+  const float* lse_c;
+  const float* delta_c;
+  float lse_o, delta_o;
+  float a[Lay::NE], b[Lay::NE];
+  float* out1;
+  float* out2;
+  int64_t ri;  // row inside its problem
+  __device__ __forceinline__ void load(const GradArgs& g, int64_t r, int c) {
+    const int d = g.d;
+    const int64_t n_own = KEYS ? g.n_k : g.n_q;
+    int64_t bb = 0;
+    ri = r;
+    if (g.n_batch > 1) {
+      bb = r / n_own;
+      ri = r - bb * n_own;
+    }
+    const T* arow;
+    const T* brow;
+    if constexpr (KEYS) {
+      arow = (const T*)g.k + r * d;
+      brow = (const T*)g.v + r * d;
+      X = (const T*)g.q + bb * g.n_q * d;
+      Y = (const T*)g.d_out + bb * g.n_q * d;
+      lse_c = g.lse + bb * g.n_q;
+      delta_c = g.delta + bb * g.n_q;
+      lse_o = 0.f;
+      delta_o = 0.f;
+      out1 = g.d_k + r * d;
+      out2 = g.d_v + r * d;
+    } else {
+      arow = (const T*)g.q + r * d;
+      brow = (const T*)g.d_out + r * d;
+      X = (const T*)g.k + bb * g.n_k * d;
+      Y = (const T*)g.v + bb * g.n_k * d;
+      lse_c = nullptr;
+      delta_c = nullptr;
+      lse_o = g.lse[r];
+      delta_o = g.delta[r];
+      out1 = g.d_q + r * d;
+      out2 = nullptr;
+    }
+    Lay::unpack(Lay::load(arow, c, d), a);
+    Lay::unpack(Lay::load(brow, c, d), b);
+  }
+};
+
+template <class Lay, class Mask, bool KEYS>
+__global__ __launch_bounds__(kGradWaves* kWave) void grad_rows_kernel(GradArgs g, Mask mask) {
+  constexpr int NE = Lay::NE;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int c = lane % Lay::LPR;
+  const int64_t n_own = KEYS ? g.n_k : g.n_q;
+  const int64_t r = (int64_t)blockIdx.x * kGradWaves + (threadIdx.x >> 6);
+  if (r >= n_own * g.n_batch) return;
+  GradOwner<Lay, KEYS> o;
+  o.load(g, r, c);
+  const typename Mask::Row rc = mask.row(o.ri);
+  const int64_t deg = rc.deg;
+  if (deg <= 0) return;
+  if (!KEYS && o.lse_o == __builtin_inff()) return;  // the row never saw a live column
+  const int64_t seg = g.seg;
+  if (deg > seg && lane == 0) {  // leave the rest of the row to the item kernel
+    const uint32_t extra = (uint32_t)((deg - 1) / seg);
+    uint32_t* cnt = g.n_items + (KEYS ? 1 : 0);
+    uint32_t* list = g.items + (size_t)(KEYS ? 2 : 0) * g.cap_items;
+    const uint32_t base = atomicAdd(cnt, extra);
+    for (uint32_t s = 0; s < extra; s++) {
+      if (base + s < g.cap_items) {
+        list[2 * (size_t)(base + s)] = (uint32_t)r;
+        list[2 * (size_t)(base + s) + 1] = s + 1;
+      }
+    }
+  }
+  float acc1[NE], acc2[NE];
+#pragma unroll
+  for (int e = 0; e < NE; e++) {
+    acc1[e] = 0.f;
+    acc2[e] = 0.f;
+  }
+  const float scale = 1.0f / sqrtf((float)g.d);
+  grad_walk<Lay, Mask, KEYS, Lay::U_MEDIUM>(mask, rc, o.X, o.Y, o.lse_c, o.delta_c, o.lse_o, o.delta_o,
+                                            g.d, scale, o.a, o.b, 0, deg < seg ? deg : seg, lane,
+                                            acc1, acc2);
+  if (lane < Lay::LPR) {  // this wavefront is the only one that touches the row in this launch
+    float cur[NE];
+    Lay::load_f32(o.out1, c, g.d, cur);
+#pragma unroll
+    for (int e = 0; e < NE; e++) cur[e] += acc1[e];
+    Lay::store_f32(o.out1, c, g.d, cur);
+    if constexpr (KEYS) {
+      Lay::load_f32(o.out2, c, g.d, cur);
+#pragma unroll
+      for (int e = 0; e < NE; e++) cur[e] += acc2[e];
+      Lay::store_f32(o.out2, c, g.d, cur);
+    }
+  }
+}
+
+// The segments grad_rows_kernel left behind, a wavefront per item, results added atomically.
+template <class Lay, class Mask, bool KEYS>
+__global__ __launch_bounds__(kGradWaves* kWave) void grad_items_kernel(GradArgs g, Mask mask) {
+  constexpr int NE = Lay::NE;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int c = lane % Lay::LPR;
+  uint32_t n = g.n_items[KEYS ? 1 : 0];
+  if (n > g.cap_items) n = g.cap_items;
+  const uint32_t* list = g.items + (size_t)(KEYS ? 2 : 0) * g.cap_items;
+  const uint32_t stride = gridDim.x * kGradWaves;
+  const float scale = 1.0f / sqrtf((float)g.d);
+  for (uint32_t it = blockIdx.x * kGradWaves + (threadIdx.x >> 6); it < n; it += stride) {
+    const int64_t r = (int64_t)list[2 * (size_t)it];
+    const int64_t s = (int64_t)list[2 * (size_t)it + 1];
+    GradOwner<Lay, KEYS> o;
+    o.load(g, r, c);
+    const typename Mask::Row rc = mask.row(o.ri);
+    const int64_t t0 = s * g.seg;
+    const int64_t t1 = rc.deg < t0 + g.seg ? rc.deg : t0 + g.seg;
+    float acc1[NE], acc2[NE];
+#pragma unroll
+    for (int e = 0; e < NE; e++) {
+      acc1[e] = 0.f;
+      acc2[e] = 0.f;
+    }
+    grad_walk<Lay, Mask, KEYS, Lay::U_MEDIUM>(mask, rc, o.X, o.Y, o.lse_c, o.delta_c, o.lse_o,
+                                              o.delta_o, g.d, scale, o.a, o.b, t0, t1, lane, acc1,
+                                              acc2);
+    if (lane < Lay::LPR) {
+#pragma unroll
+      for (int e = 0; e < NE; e++) {
+        const int idx = grad_elem_index<Lay>(c, e);
+        if (idx < g.d) {
+          unsafeAtomicAdd(o.out1 + idx, acc1[e]);
+          if constexpr (KEYS) unsafeAtomicAdd(o.out2 + idx, acc2[e]);
+        }
+      }
+    }
+  }
+}
+
+template <class Lay, class RowMask, class ColMask>
+int launch_grad(const Tensors& t, const GradArgs& g, const RowMask& rows, const ColMask& cols,
+                hipStream_t stream) {
+  using T = typename Lay::elem;
+  const int64_t nq = g.n_q * g.n_batch, nk = g.n_k * g.n_batch;
+  if (nq == 0 || nk == 0) return 0;
+  if (nq >= ((int64_t)1 << 32) || nk >= ((int64_t)1 << 32)) return 1;  // items hold 32-bit owners
+  const dim3 block(kGradWaves * kWave);
+  hipLaunchKernelGGL(grad_reset_kernel, dim3(1), dim3(64), 0, stream, g.n_items);
+  hipLaunchKernelGGL((grad_prologue_kernel<T>), dim3((unsigned)((nq + 3) / 4)), dim3(256), 0, stream,
+                     t, g);
+  hipLaunchKernelGGL((grad_rows_kernel<Lay, RowMask, false>),
+                     dim3((unsigned)((nq + kGradWaves - 1) / kGradWaves)), block, 0, stream, g, rows);
+  hipLaunchKernelGGL((grad_items_kernel<Lay, RowMask, false>), dim3(kGradItemBlocks), block, 0, stream,
+                     g, rows);
+  hipLaunchKernelGGL((grad_rows_kernel<Lay, ColMask, true>),
+                     dim3((unsigned)((nk + kGradWaves - 1) / kGradWaves)), block, 0, stream, g, cols);
+  hipLaunchKernelGGL((grad_items_kernel<Lay, ColMask, true>), dim3(kGradItemBlocks), block, 0, stream,
+                     g, cols);
+  return hipGetLastError() == hipSuccess ? 0 : 4;
+}
+
+template <typename T, class RowMask, class ColMask>
+int run_grad(const Tensors& t, const GradArgs& g, const RowMask& rows, const ColMask& cols,
+             hipStream_t stream) {
+  const int64_t row_bytes = (int64_t)t.d * (int64_t)sizeof(T);
+  if (row_bytes == 64) return launch_grad<VecLay<T, 4>>(t, g, rows, cols, stream);
+  if (row_bytes == 128) return launch_grad<VecLay<T, 8>>(t, g, rows, cols, stream);
+  if (row_bytes == 256) return launch_grad<VecLay<T, 16>>(t, g, rows, cols, stream);
+  if (row_bytes == 512) return launch_grad<VecLay<T, 32>>(t, g, rows, cols, stream);
+  if (t.d <= 128) return launch_grad<GenLay<T, 2>>(t, g, rows, cols, stream);
+  if (t.d <= 1024) return launch_grad<GenLay<T, 16>>(t, g, rows, cols, stream);
+  return 5;
+}
+
+}  // namespace spfa

@@ -25,7 +25,19 @@ template <typename T>
 int run_global(const Tensors& t, const GlobalMask& mask, const EngineSizing& s, int use_nan,
                void* ws, hipStream_t stream);
 
-// Gradients (spfa_backward.hpp); dtype is the C enum of the element type.
+// Gradients by two gather passes (spfa_grad.hpp): `rows` walks the mask by query row, `cols` by
+// key row.
+struct GradArgs;
+template <typename T>
+int run_grad_csr(const Tensors& t, const GradArgs& g, const CsrMask& rows, const CsrMask& cols,
+                 hipStream_t stream);
+template <typename T>
+int run_grad_stride(const Tensors& t, const GradArgs& g, const StrideMask& mask, hipStream_t stream);
+template <typename T>
+int run_grad_global(const Tensors& t, const GradArgs& g, const GlobalMask& rows,
+                    const GlobalColMask& cols, hipStream_t stream);
+
+// fp64 gradients: one plain kernel with atomics (spfa_backward.hpp); dtype is the C enum.
 struct Grads;
 int run_backward_csr(int dtype, const Tensors& t, const CsrMask& mask, const Grads& g,
                      hipStream_t stream);

@@ -10,6 +10,7 @@ namespace spfa {
 // Explicit CSR adjacency: row i owns col_ind[row_off[i] .. row_off[i+1])
 // (reference: Sparse_FlashAttention_CSR/sp_flatt_csr_kernel.cu:29-33,117).
 struct CsrMask {
+  static constexpr bool kWeighted = false;  // every candidate counts once
   const void* row_off;
   const uint32_t* cols;
   int32_t off64;  // row_off entries are 8 bytes wide (else 4)
@@ -49,6 +50,7 @@ struct CsrMask {
 //               only when (i - low) mod s == 0, then deg = cnt = min(block, (block-1)/s + 1)
 //               (Sparse_FlashAttention_Local_2D_Dilated/sp_flatt_local_2d_dilated_kernel.cu:26-39,123).
 struct StrideMask {
+  static constexpr bool kWeighted = false;
   int64_t n;
   int64_t w;
   int64_t s;
@@ -81,6 +83,7 @@ struct StrideMask {
 //   (Sparse_FlashAttention_Global_No_Local/sp_flatt_global_no_local_kernel.cu:38-64,134-162).
 // Bit i of gbits marks the listed rows.
 struct GlobalMask {
+  static constexpr bool kWeighted = false;
   int64_t n;
   int64_t w;
   const int32_t* globs;
@@ -105,6 +108,52 @@ struct GlobalMask {
     int64_t c = (int64_t)globs[t];
     valid = (c < r.low) || (c >= r.up);
     return c;
+  }
+};
+
+// The global-minus-local mask read by COLUMN (the gradient's key-side pass): which query rows
+// attend column j, and how often.  The window test is symmetric, so
+//   listed column j:  every row outside the window; a listed row attends j once, any other row
+//                     once per occurrence of j in the list (it walks the list, duplicates and all);
+//   other columns:    the distinct listed rows outside the window, once each.
+struct GlobalColMask {
+  static constexpr bool kWeighted = true;
+  int64_t n;
+  int64_t w;
+  const int32_t* globs;   // the list as given (duplicates allowed)
+  int64_t n_globs;
+  const uint32_t* gbits;
+  const int32_t* uq;      // distinct listed rows
+  const uint32_t* n_uq;   // how many
+  struct Row {
+    int64_t low;
+    int64_t up;
+    int64_t deg;
+    bool glob;
+    float mult;  // occurrences of this column in the list
+  };
+  __device__ __forceinline__ Row row(int64_t j) const {
+    int64_t low = j - w;
+    if (low < 0) low = 0;
+    int64_t up = j + w + 1;
+    if (up > n) up = n;
+    const bool glob = bit_is_set(gbits, j);
+    float mult = 1.f;
+    if (glob) {
+      int cnt = 0;
+      for (int64_t t = 0; t < n_globs; t++) cnt += (globs[t] == (int32_t)j) ? 1 : 0;
+      mult = (float)cnt;
+    }
+    return Row{low, up, glob ? n - (up - low) : (int64_t)*n_uq, glob, mult};
+  }
+  __device__ __forceinline__ int64_t col(const Row& r, int64_t t, bool& valid) const {
+    if (r.glob) return t < r.low ? t : t + (r.up - r.low);
+    int64_t c = (int64_t)uq[t];
+    valid = (c < r.low) || (c >= r.up);
+    return c;
+  }
+  __device__ __forceinline__ float weight(const Row& r, int64_t c) const {
+    return (r.glob && !bit_is_set(gbits, c)) ? r.mult : 1.f;
   }
 };
 

@@ -332,6 +332,24 @@ __global__ __launch_bounds__(kPartRowsThreads) void coo_part_rows_kernel(
   }
 }
 
+// one wavefront per row: lanes stride over the row's entries
+__global__ __launch_bounds__(256) void csr_entry_list_kernel(const void* row_off, int off64,
+                                                             const uint32_t* cols,
+                                                             const uint32_t* alt_cols,
+                                                             const uint32_t* use_alt, int64_t n_rows,
+                                                             uint32_t* rows_out, uint32_t* cols_out) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int64_t stride = (int64_t)gridDim.x * 4;
+  const uint32_t* cp = (use_alt != nullptr && *use_alt != 0u) ? alt_cols : cols;
+  for (int64_t r = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6); r < n_rows; r += stride) {
+    const int64_t a = load_index(row_off, r, off64), b = load_index(row_off, r + 1, off64);
+    for (int64_t e = a + lane; e < b; e += kWave) {
+      rows_out[e] = (uint32_t)r;
+      cols_out[e] = cp[e];
+    }
+  }
+}
+
 inline unsigned grid_for(int64_t n, int threads, int64_t cap) {
   int64_t g = (n + threads - 1) / threads;
   if (g > cap) g = cap;
@@ -431,6 +449,15 @@ int coo_to_csr(const void* row_ind, int row_wide, const uint32_t* col_ind, int64
   out->row_off = row_off;
   out->cols = cols;
   out->unsorted = flag;
+  return hipGetLastError() == hipSuccess ? 0 : 4;
+}
+
+int csr_entry_list(const void* row_off, int off64, const uint32_t* cols, const uint32_t* alt_cols,
+                   const uint32_t* use_alt, int64_t n_rows, uint32_t* rows_out, uint32_t* cols_out,
+                   hipStream_t stream) {
+  if (n_rows <= 0) return 0;
+  hipLaunchKernelGGL(csr_entry_list_kernel, dim3(grid_for(n_rows, 4, 1 << 20)), dim3(256), 0, stream,
+                     row_off, off64, cols, alt_cols, use_alt, n_rows, rows_out, cols_out);
   return hipGetLastError() == hipSuccess ? 0 : 4;
 }
 

@@ -42,6 +42,13 @@ struct CooCsr {
 int coo_to_csr(const void* row_ind, int row_wide, const uint32_t* col_ind, int64_t nnz,
                int64_t n_rows, void* keep, void* scratch, hipStream_t stream, CooCsr* out);
 
+// The entry list of a CSR mask: rows[e], cols[e] for every entry e of row_off / col_ind (cols
+// from alt_cols when *use_alt != 0, as CsrMask reads them).  Feeding (cols, rows) back into
+// coo_to_csr gives the transposed mask.
+int csr_entry_list(const void* row_off, int off64, const uint32_t* cols, const uint32_t* alt_cols,
+                   const uint32_t* use_alt, int64_t n_rows, uint32_t* rows_out, uint32_t* cols_out,
+                   hipStream_t stream);
+
 // Global-row bookkeeping for the global-minus-local mask.  `bits` holds (n+31)/32 bitmap words
 // followed by one counter word; afterwards bit i is set for every listed i in [0, n), `uq` holds
 // the distinct listed rows (any order) and the counter word their number.

@@ -119,7 +119,8 @@ std::tuple<torch::Tensor, torch::Tensor, torch::Tensor> spfa_coo_backward_py(tor
   const int row_bytes = spfa_ext::index_bytes(W_row_ind, "W_row_ind", true);
   spfa_ext::index_bytes(W_col_ind, "W_col_ind", false);
   const int64_t nnz = W_col_ind.size(0);
-  torch::Tensor ws = spfa_ext::make_workspace(spfa_coo_workspace_bytes(p.n_q, nnz, p.d, p.dtype), Q);
+  torch::Tensor ws = spfa_ext::make_workspace(
+      spfa_coo_backward_workspace_bytes(p.n_q, p.n_k, nnz, p.d, p.dtype, p.n_batch), Q);
   spfa_ext::raise_on_error(spfa_coo_backward(&p, &g, W_row_ind.data_ptr(), row_bytes, W_col_ind.data_ptr(),
                                              nnz, ws.data_ptr(), (size_t)ws.numel(),
                                              spfa_ext::current_stream(Q)));

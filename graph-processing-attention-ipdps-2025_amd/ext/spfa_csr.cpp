@@ -115,8 +115,12 @@ std::tuple<torch::Tensor, torch::Tensor, torch::Tensor> spfa_csr_backward_py(tor
   (void)W_val;
   const int off_bytes = spfa_ext::index_bytes(W_row_off, "W_row_off", true);
   spfa_ext::index_bytes(W_col_ind, "W_col_ind", false);
+  const int64_t nnz = W_col_ind.size(0);
+  torch::Tensor ws = spfa_ext::make_workspace(
+      spfa_csr_backward_workspace_bytes(p.n_q, p.n_k, nnz, p.d, p.dtype, p.n_batch), Q);
   spfa_ext::raise_on_error(spfa_csr_backward(&p, &g, W_row_off.data_ptr(), off_bytes, W_col_ind.data_ptr(),
-                                             W_col_ind.size(0), spfa_ext::current_stream(Q)));
+                                             nnz, ws.data_ptr(), (size_t)ws.numel(),
+                                             spfa_ext::current_stream(Q)));
   return std::make_tuple(dQ, dK, dV);
 }
 

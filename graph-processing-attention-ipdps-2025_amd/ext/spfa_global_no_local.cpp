@@ -53,7 +53,8 @@ std::tuple<torch::Tensor, torch::Tensor, torch::Tensor> spfa_global_no_local_bac
   TORCH_CHECK(global_inds.scalar_type() == torch::kInt32, "global_inds must be an int32 tensor");
   const int64_t n_globs = global_inds.size(0);
   torch::Tensor ws = spfa_ext::make_workspace(
-      spfa_global_no_local_workspace_bytes(p.n_q, p.d, p.dtype, n_globs, local_size_each_dir), Q);
+      spfa_global_no_local_backward_workspace_bytes(p.n_q, p.d, p.dtype, n_globs, local_size_each_dir,
+                                                    p.n_batch), Q);
   spfa_ext::raise_on_error(spfa_global_no_local_backward(
       &p, &g, (const int32_t*)global_inds.data_ptr(), n_globs, local_size_each_dir, ws.data_ptr(),
       (size_t)ws.numel(), spfa_ext::current_stream(Q)));

@@ -41,7 +41,10 @@ std::tuple<torch::Tensor, torch::Tensor, torch::Tensor> spfa_local_backward_py(t
   spfa_problem_t p = spfa_ext::make_problem(Q, K, V, m, l, O);
   spfa_grads_t g = spfa_ext::make_grads(Q, K, dO, dQ, dK, dV);
   TORCH_CHECK(p.n_k == p.n_q, "Q, K and V must have the same number of rows");
-  spfa_ext::raise_on_error(spfa_local_backward(&p, &g, local_size_each_dir, spfa_ext::current_stream(Q)));
+  torch::Tensor ws = spfa_ext::make_workspace(
+      spfa_local_backward_workspace_bytes(p.n_q, p.d, p.dtype, local_size_each_dir, p.n_batch), Q);
+  spfa_ext::raise_on_error(spfa_local_backward(&p, &g, local_size_each_dir, ws.data_ptr(),
+                                               (size_t)ws.numel(), spfa_ext::current_stream(Q)));
   return std::make_tuple(dQ, dK, dV);
 }
 

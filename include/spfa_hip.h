@@ -206,8 +206,9 @@ int spfa_global_no_local_forward(const spfa_problem_t* p, const int32_t* global_
  * (never any live column) carry no gradient.
  *   d_out        [n_batch * n_q, d], element type of the problem
  *   d_q          [n_batch * n_q, d]  fp32 (fp64 for F64 problems); the caller zeroes it
- *   d_k, d_v     [n_batch * n_k, d]  likewise; added to with floating-point atomics, so two runs
- *                                    may differ in the last bits
+ *   d_k, d_v     [n_batch * n_k, d]  likewise.  Rows with more than 1024 live positions are
+ *                                    split and their pieces added with floating-point atomics, so
+ *                                    two runs may differ in the last bits there (F64: everywhere)
  * Parameter checks and their codes are those of the matching forward call. */
 typedef struct spfa_grads {
   const void* d_out;
@@ -216,19 +217,38 @@ typedef struct spfa_grads {
   void* d_v;
 } spfa_grads_t;
 
+/* workspace: scratch of at least *_backward_workspace_bytes(...) bytes, 256-byte aligned (the
+ * softmax statistics of every row, the work list of long rows and, for explicit masks, the mask
+ * transposed); n_batch as in spfa_problem_t. */
+size_t spfa_csr_backward_workspace_bytes(int64_t n_q, int64_t n_k, int64_t nnz, int64_t d, int dtype,
+                                         int64_t n_batch);
 int spfa_csr_backward(const spfa_problem_t* p, const spfa_grads_t* g, const void* row_off,
-                      int row_off_bytes, const void* col_ind, int64_t nnz, void* stream);
-/* workspace: at least spfa_coo_workspace_bytes(n_q, nnz, d, dtype) */
+                      int row_off_bytes, const void* col_ind, int64_t nnz, void* workspace,
+                      size_t workspace_bytes, void* stream);
+size_t spfa_coo_backward_workspace_bytes(int64_t n_q, int64_t n_k, int64_t nnz, int64_t d, int dtype,
+                                         int64_t n_batch);
 int spfa_coo_backward(const spfa_problem_t* p, const spfa_grads_t* g, const void* row_ind,
                       int row_ind_bytes, const void* col_ind, int64_t nnz, void* workspace,
                       size_t workspace_bytes, void* stream);
+size_t spfa_local_backward_workspace_bytes(int64_t n, int64_t d, int dtype, int64_t local_size,
+                                           int64_t n_batch);
 int spfa_local_backward(const spfa_problem_t* p, const spfa_grads_t* g, int64_t local_size,
-                        void* stream);
+                        void* workspace, size_t workspace_bytes, void* stream);
+size_t spfa_local_1d_dilated_backward_workspace_bytes(int64_t n, int64_t d, int dtype,
+                                                      int64_t local_size, int64_t dil_factor,
+                                                      int64_t n_batch);
 int spfa_local_1d_dilated_backward(const spfa_problem_t* p, const spfa_grads_t* g,
-                                   int64_t local_size, int64_t dil_factor, void* stream);
+                                   int64_t local_size, int64_t dil_factor, void* workspace,
+                                   size_t workspace_bytes, void* stream);
+size_t spfa_local_2d_dilated_backward_workspace_bytes(int64_t n, int64_t d, int dtype,
+                                                      int64_t block_size, int64_t dil_factor,
+                                                      int64_t n_batch);
 int spfa_local_2d_dilated_backward(const spfa_problem_t* p, const spfa_grads_t* g,
-                                   int64_t block_size, int64_t dil_factor, void* stream);
-/* workspace: at least spfa_global_no_local_workspace_bytes(n, d, dtype, n_globals, local_size) */
+                                   int64_t block_size, int64_t dil_factor, void* workspace,
+                                   size_t workspace_bytes, void* stream);
+size_t spfa_global_no_local_backward_workspace_bytes(int64_t n, int64_t d, int dtype,
+                                                     int64_t n_globals, int64_t local_size,
+                                                     int64_t n_batch);
 int spfa_global_no_local_backward(const spfa_problem_t* p, const spfa_grads_t* g,
                                   const int32_t* global_inds, int64_t n_globals,
                                   int64_t local_size, void* workspace, size_t workspace_bytes,

@@ -118,6 +118,52 @@ def test_chained_parts_are_differentiated_as_their_union(mods, dtype):
     assert np.abs(np64(out) - ref_out).max() <= (1e-11 if dtype == torch.float64 else 1e-4)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_rows_and_columns_longer_than_one_segment(mods, dtype):
+    """Owners with more than 1024 live positions are split over several wavefronts: a query row
+    and a key column with ~2500 entries (explicit mask), a band of 1401, the rows and columns of
+    listed global tokens."""
+    n, d = 2600, 64
+    rng = np.random.default_rng(61)
+    dense = rng.random((n, n)) < 0.01
+    dense[7, rng.permutation(n)[:2500]] = True
+    dense[rng.permutation(n)[:2500], 11] = True
+    q, k, v, d_out = _problem(n, d, dtype, 62)
+    for parts, mask in [([_csr_part(dense)], dense), ([_coo_part(dense, 63)], dense),
+                        ([("local", 700)], so.mask_local_dense(n, 700)),
+                        ([("global_no_local", torch.tensor([3, 1300], dtype=torch.int32, device=DEV), 4)],
+                         so.mask_global_no_local_dense(n, [3, 1300], 4))]:
+        ref = so.dense_masked_attention_backward(np64(q), np64(k), np64(v), mask, np64(d_out))
+        _, got = _grads_of(q, k, v, d_out, parts)
+        _check_grads(got, ref, dtype, parts[0][0])
+
+
+@pytest.mark.parametrize("dtype", [torch.float64, torch.float32])
+def test_repeated_global_indices_count_as_often_as_in_the_forward_pass(mods, dtype):
+    """A token listed twice is walked twice by every ordinary row
+    (sp_flatt_global_no_local_kernel.cu:134-162 reads the list as given) and once by listed rows.
+    The dense statement of that: one extra key/value column per repetition, live for the ordinary
+    rows outside their window; the gradient of the repeated token is the sum over its copies."""
+    n, d, w = 300, 32, 6
+    globs = [40, 200, 40, 7]
+    q, k, v, d_out = _problem(n, d, dtype, 71)
+    base = so.mask_global_no_local_dense(n, sorted(set(globs)), w)
+    extra = np.zeros((n, 1), dtype=bool)
+    for i in range(n):
+        extra[i, 0] = (i not in globs) and abs(i - 40) > w
+    mask = np.concatenate([base, extra], axis=1)
+    k2 = np.concatenate([np64(k), np64(k)[40:41]])
+    v2 = np.concatenate([np64(v), np64(v)[40:41]])
+    dq, dk2, dv2 = so.dense_masked_attention_backward(np64(q), k2, v2, mask, np64(d_out))
+    dk, dv = dk2[:n].copy(), dv2[:n].copy()
+    dk[40] += dk2[n]
+    dv[40] += dv2[n]
+    out, got = _grads_of(q, k, v, d_out, [("global_no_local", torch.tensor(globs, dtype=torch.int32, device=DEV), w)])
+    ref_out = so.dense_masked_attention(np64(q), k2, v2, mask)[0]
+    assert np.abs(np64(out) - ref_out).max() <= (1e-11 if dtype == torch.float64 else 1e-4)
+    _check_grads(got, (dq, dk, dv), dtype, "repeated globals")
+
+
 def test_batch_of_heads_shares_the_mask(mods):
     n, d, lead = 200, 64, (2, 3)
     q, k, v, d_out = _problem(n, d, torch.float32, 31, lead=lead)
