@@ -807,24 +807,38 @@ GradArgs make_grad_args(const spfa_problem_t* p, const spfa_grads_t* g, const Gr
   return a;
 }
 
-// Gradients through an explicit mask given as a CsrMask over the query rows: transpose it (entry
-// list -> bucketed by column), then the two passes.
-int explicit_backward(const spfa_problem_t* p, const spfa_grads_t* g, const CsrMask& rows, int64_t nnz,
-                      const GradLayout& lay, void* workspace, hipStream_t stream) {
-  if (is_f64(p)) return run_backward_csr(p->dtype, make_tensors(p), rows, make_grads(g), stream);
-  char* mbase = (char*)workspace + lay.off_mask;
-  const TransposeLayout tl = transpose_layout(p->n_k, nnz);
+// The transposed mask of `rows` (a CsrMask over n_q query rows) built in `mbase`
+// (transpose_layout() bytes): on return `out` reads it by key row.
+int transpose_mask(const CsrMask& rows, int64_t n_q, int64_t n_k, int64_t nnz, char* mbase,
+                   hipStream_t stream, CooCsr* tr, const uint32_t** entry_rows) {
+  const TransposeLayout tl = transpose_layout(n_k, nnz);
   uint32_t* e_rows = (uint32_t*)(mbase + tl.off_rows);
   uint32_t* e_cols = (uint32_t*)(mbase + tl.off_cols);
-  int rc = csr_entry_list(rows.row_off, rows.off64, rows.cols, rows.alt_cols, rows.use_alt, p->n_q,
-                          e_rows, e_cols, stream);
+  int rc = csr_entry_list(rows.row_off, rows.off64, rows.cols, rows.alt_cols, rows.use_alt, n_q, e_rows,
+                          e_cols, stream);
   if (rc) return rc;
-  const CooWorkspace cw = coo_workspace(p->n_k, nnz);
-  CooCsr tr{};
-  rc = coo_to_csr(e_cols, 0, e_rows, nnz, p->n_k, mbase + tl.off_coo, mbase + tl.off_coo + cw.keep_total,
-                  stream, &tr);
-  if (rc) return rc;
-  CsrMask cols{tr.row_off, e_rows, 0, tr.cols, tr.unsorted};
+  const CooWorkspace cw = coo_workspace(n_k, nnz);
+  *entry_rows = e_rows;
+  return coo_to_csr(e_cols, 0, e_rows, nnz, n_k, mbase + tl.off_coo, mbase + tl.off_coo + cw.keep_total,
+                    stream, tr);
+}
+
+// Gradients through an explicit mask given as a CsrMask over the query rows: the two passes, the
+// key pass over `given_cols` when the caller brought the transposed mask, else over one built here.
+int explicit_backward(const spfa_problem_t* p, const spfa_grads_t* g, const CsrMask& rows, int64_t nnz,
+                      const CsrMask* given_cols, const GradLayout& lay, void* workspace,
+                      hipStream_t stream) {
+  if (is_f64(p)) return run_backward_csr(p->dtype, make_tensors(p), rows, make_grads(g), stream);
+  CsrMask cols{};
+  if (given_cols != nullptr) {
+    cols = *given_cols;
+  } else {
+    CooCsr tr{};
+    const uint32_t* e_rows = nullptr;
+    int rc = transpose_mask(rows, p->n_q, p->n_k, nnz, (char*)workspace + lay.off_mask, stream, &tr, &e_rows);
+    if (rc) return rc;
+    cols = CsrMask{tr.row_off, e_rows, 0, tr.cols, tr.unsorted};
+  }
   const GradArgs a = make_grad_args(p, g, lay, workspace);
   const Tensors t = make_tensors(p);
   switch (p->dtype) {
@@ -863,23 +877,49 @@ size_t spfa_csr_backward_workspace_bytes(int64_t n_q, int64_t n_k, int64_t nnz, 
 }
 
 int spfa_csr_backward(const spfa_problem_t* p, const spfa_grads_t* g, const void* row_off,
-                      int row_off_bytes, const void* col_ind, int64_t nnz, void* workspace,
-                      size_t workspace_bytes, void* stream) {
+                      int row_off_bytes, const void* col_ind, int64_t nnz, const uint32_t* t_row_off,
+                      const uint32_t* t_col_ind, void* workspace, size_t workspace_bytes, void* stream) {
   int rc = check_problem(p);
   if (rc) return rc;
   if (nnz < 0 || nnz >= (int64_t)1 << 31 || (row_off_bytes != 4 && row_off_bytes != 8))
     return SPFA_ERR_BAD_ARG;
+  if ((t_row_off == nullptr) != (t_col_ind == nullptr)) return SPFA_ERR_BAD_ARG;
   rc = check_grads(p, g);
   if (rc) return rc;
   if (p->n_q == 0 || nnz == 0) return SPFA_OK;
   if (!row_off || !col_ind) return SPFA_ERR_BAD_ARG;
-  const GradLayout lay =
-      grad_layout(p->n_q, batch_of(p), explicit_items_bound(nnz), transpose_layout(p->n_k, nnz).total);
+  const bool given = t_row_off != nullptr;
+  const GradLayout lay = grad_layout(p->n_q, batch_of(p), explicit_items_bound(nnz),
+                                     given ? 0 : transpose_layout(p->n_k, nnz).total);
   if (!lay.ok) return SPFA_ERR_BAD_ARG;
   rc = check_workspace(workspace, workspace_bytes, lay.total);
   if (rc) return rc;
   CsrMask rows{row_off, (const uint32_t*)col_ind, row_off_bytes == 8 ? 1 : 0, nullptr, nullptr};
-  return explicit_backward(p, g, rows, nnz, lay, workspace, (hipStream_t)stream);
+  CsrMask cols{t_row_off, t_col_ind, 0, nullptr, nullptr};
+  return explicit_backward(p, g, rows, nnz, given ? &cols : nullptr, lay, workspace,
+                           (hipStream_t)stream);
+}
+
+size_t spfa_csr_transpose_workspace_bytes(int64_t n_q, int64_t n_k, int64_t nnz) {
+  if (n_q < 0 || n_k < 0 || nnz < 0) return 0;
+  return transpose_layout(n_k, nnz).total;
+}
+
+int spfa_csr_transpose(int64_t n_q, int64_t n_k, const void* row_off, int row_off_bytes,
+                       const void* col_ind, int64_t nnz, uint32_t* t_row_off, uint32_t* t_col_ind,
+                       void* workspace, size_t workspace_bytes, void* stream) {
+  if (n_q < 0 || n_k < 0 || n_k >= (int64_t)1 << 31 || n_q >= (int64_t)1 << 31 || nnz < 0 ||
+      nnz >= (int64_t)1 << 31 || (row_off_bytes != 4 && row_off_bytes != 8))
+    return SPFA_ERR_BAD_ARG;
+  if (!t_row_off || (nnz > 0 && (!row_off || !col_ind || !t_col_ind))) return SPFA_ERR_BAD_ARG;
+  int rc = check_workspace(workspace, workspace_bytes, transpose_layout(n_k, nnz).total);
+  if (rc) return rc;
+  CsrMask rows{row_off, (const uint32_t*)col_ind, row_off_bytes == 8 ? 1 : 0, nullptr, nullptr};
+  CooCsr tr{};
+  const uint32_t* e_rows = nullptr;
+  rc = transpose_mask(rows, n_q, n_k, nnz, (char*)workspace, (hipStream_t)stream, &tr, &e_rows);
+  if (rc) return rc;
+  return coo_csr_export(tr, e_rows, n_k, nnz, t_row_off, t_col_ind, (hipStream_t)stream);
 }
 
 size_t spfa_coo_backward_workspace_bytes(int64_t n_q, int64_t n_k, int64_t nnz, int64_t d, int dtype,
@@ -917,7 +957,7 @@ int spfa_coo_backward(const spfa_problem_t* p, const spfa_grads_t* g, const void
   if (rc) return rc;
   CsrMask rows{csr.row_off, (const uint32_t*)col_ind, 0, csr.cols, csr.unsorted};
   lay.off_mask += fwd_bytes;
-  return explicit_backward(p, g, rows, nnz, lay, workspace, (hipStream_t)stream);
+  return explicit_backward(p, g, rows, nnz, nullptr, lay, workspace, (hipStream_t)stream);
 }
 
 size_t spfa_local_backward_workspace_bytes(int64_t n, int64_t d, int dtype, int64_t local_size,

@@ -350,6 +350,17 @@ __global__ __launch_bounds__(256) void csr_entry_list_kernel(const void* row_off
   }
 }
 
+__global__ void coo_csr_export_kernel(const uint32_t* row_off, const uint32_t* bucketed,
+                                      const uint32_t* given, const uint32_t* unsorted, int64_t n_rows,
+                                      int64_t nnz, uint32_t* row_off_out, uint32_t* cols_out) {
+  const uint32_t* src = *unsorted ? bucketed : given;
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < nnz + n_rows + 1; i += stride) {
+    if (i < nnz) cols_out[i] = src[i];
+    else row_off_out[i - nnz] = row_off[i - nnz];
+  }
+}
+
 inline unsigned grid_for(int64_t n, int threads, int64_t cap) {
   int64_t g = (n + threads - 1) / threads;
   if (g > cap) g = cap;
@@ -458,6 +469,14 @@ int csr_entry_list(const void* row_off, int off64, const uint32_t* cols, const u
   if (n_rows <= 0) return 0;
   hipLaunchKernelGGL(csr_entry_list_kernel, dim3(grid_for(n_rows, 4, 1 << 20)), dim3(256), 0, stream,
                      row_off, off64, cols, alt_cols, use_alt, n_rows, rows_out, cols_out);
+  return hipGetLastError() == hipSuccess ? 0 : 4;
+}
+
+int coo_csr_export(const CooCsr& csr, const uint32_t* given_cols, int64_t n_rows, int64_t nnz,
+                   uint32_t* row_off_out, uint32_t* cols_out, hipStream_t stream) {
+  hipLaunchKernelGGL(coo_csr_export_kernel, dim3(grid_for(nnz + n_rows + 1, 256, 16384)), dim3(256), 0,
+                     stream, csr.row_off, csr.cols, given_cols, csr.unsorted, n_rows, nnz, row_off_out,
+                     cols_out);
   return hipGetLastError() == hipSuccess ? 0 : 4;
 }
 

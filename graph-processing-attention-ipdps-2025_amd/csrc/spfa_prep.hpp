@@ -49,6 +49,11 @@ int csr_entry_list(const void* row_off, int off64, const uint32_t* cols, const u
                    const uint32_t* use_alt, int64_t n_rows, uint32_t* rows_out, uint32_t* cols_out,
                    hipStream_t stream);
 
+// A CooCsr result as two plain arrays: row_off_out[0..n_rows] and cols_out[0..nnz) (the bucketed
+// columns, or `given_cols` unchanged when the entries came sorted).
+int coo_csr_export(const CooCsr& csr, const uint32_t* given_cols, int64_t n_rows, int64_t nnz,
+                   uint32_t* row_off_out, uint32_t* cols_out, hipStream_t stream);
+
 // Global-row bookkeeping for the global-minus-local mask.  `bits` holds (n+31)/32 bitmap words
 // followed by one counter word; afterwards bit i is set for every listed i in [0, n), `uq` holds
 // the distinct listed rows (any order) and the counter word their number.

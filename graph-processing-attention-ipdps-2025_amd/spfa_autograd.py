@@ -11,7 +11,8 @@ into the same gradients.
     out.sum().backward()
 
 Parts (their masks must not overlap, as with chained forward calls):
-    ("csr", w_row_off, w_col_ind)           ("coo", w_row_ind, w_col_ind)
+    ("csr", w_row_off, w_col_ind[, t_row_off, t_col_ind])   - see csr_part()
+    ("coo", w_row_ind, w_col_ind)
     ("local", w)                            ("local_1d_dilated", w, dilation)
     ("local_2d_dilated", block, dilation)   ("global_no_local", global_inds int32, w)
 Rows that no part gives a live column come out as zeros and carry no gradient.
@@ -44,7 +45,7 @@ def _run_backward(kind, args, q, k, v, m, l, out, d_out, d_q, d_k, d_v):
     mod = _module(kind)
     if kind in ("csr", "coo"):
         val = torch.empty(0, dtype=q.dtype, device=q.device)
-        mod.backward(q, k, v, args[0], args[1], val, m, l, out, d_out, d_q, d_k, d_v)
+        mod.backward(q, k, v, args[0], args[1], val, m, l, out, d_out, d_q, d_k, d_v, *args[2:])
     else:
         mod.backward(q, k, v, m, l, out, *args, d_out, d_q, d_k, d_v)
 
@@ -75,6 +76,13 @@ class _MaskedAttention(torch.autograd.Function):
         for part in ctx.parts:
             _run_backward(part[0], part[1:], q, k, v, m, l, out, d_out, d_q, d_k, d_v)
         return d_q.to(q.dtype), d_k.to(k.dtype), d_v.to(v.dtype), None
+
+
+def csr_part(w_row_off, w_col_ind, n_cols):
+    """A "csr" part that carries the mask read by column as well, so that backward passes do not
+    rebuild it: transpose once, reuse for every step that uses the mask."""
+    t_row_off, t_col_ind = importlib.import_module("spfa_csr").transpose(w_row_off, w_col_ind, n_cols)
+    return ("csr", w_row_off, w_col_ind, t_row_off, t_col_ind)
 
 
 def attention(q, k, v, parts, return_state=False):

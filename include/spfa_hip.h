@@ -222,9 +222,19 @@ typedef struct spfa_grads {
  * transposed); n_batch as in spfa_problem_t. */
 size_t spfa_csr_backward_workspace_bytes(int64_t n_q, int64_t n_k, int64_t nnz, int64_t d, int dtype,
                                          int64_t n_batch);
+/* t_row_off / t_col_ind: the mask read by key row, as spfa_csr_transpose writes it, or both NULL
+ * (it is then built inside the call; *_backward_workspace_bytes covers both cases). */
 int spfa_csr_backward(const spfa_problem_t* p, const spfa_grads_t* g, const void* row_off,
-                      int row_off_bytes, const void* col_ind, int64_t nnz, void* workspace,
-                      size_t workspace_bytes, void* stream);
+                      int row_off_bytes, const void* col_ind, int64_t nnz, const uint32_t* t_row_off,
+                      const uint32_t* t_col_ind, void* workspace, size_t workspace_bytes, void* stream);
+/* A CSR mask of n_q rows over n_k columns read by column: afterwards
+ * t_col_ind[t_row_off[j] .. t_row_off[j+1]) are the rows whose CSR row holds column j, in no
+ * particular order (t_row_off: n_k + 1 entries, t_col_ind: nnz).  A mask that is used for many
+ * backward calls is transposed once with this. */
+size_t spfa_csr_transpose_workspace_bytes(int64_t n_q, int64_t n_k, int64_t nnz);
+int spfa_csr_transpose(int64_t n_q, int64_t n_k, const void* row_off, int row_off_bytes,
+                       const void* col_ind, int64_t nnz, uint32_t* t_row_off, uint32_t* t_col_ind,
+                       void* workspace, size_t workspace_bytes, void* stream);
 size_t spfa_coo_backward_workspace_bytes(int64_t n_q, int64_t n_k, int64_t nnz, int64_t d, int dtype,
                                          int64_t n_batch);
 int spfa_coo_backward(const spfa_problem_t* p, const spfa_grads_t* g, const void* row_ind,

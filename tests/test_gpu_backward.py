@@ -164,6 +164,40 @@ def test_repeated_global_indices_count_as_often_as_in_the_forward_pass(mods, dty
     _check_grads(got, (dq, dk, dv), dtype, "repeated globals")
 
 
+def test_transposed_mask_is_exact_and_reusable(mods):
+    """spfa_csr.transpose against a CPU transposition (bit-exact offsets, the rows of every column
+    as a set), for a rectangular mask with empty rows and columns, both offset widths; and the
+    gradients with the transposed mask handed in equal those that rebuild it."""
+    n, n_k, d = 500, 700, 64
+    rng = np.random.default_rng(81)
+    dense = rng.random((n, n_k)) < 0.05
+    dense[9] = False
+    dense[:, 13] = False
+    dense[20] = True
+    ro, ci = so.csr_from_dense(dense)
+    t_ro_ref, t_ci_ref = so.csr_from_dense(dense.T)
+    for off_dtype in (torch.uint64, torch.int32):
+        ro_t = torch.as_tensor(ro).to(off_dtype).to(DEV)
+        ci_t = torch.as_tensor(ci).to(torch.uint32).to(DEV)
+        t_ro, t_ci = mods["spfa_csr"].transpose(ro_t, ci_t, n_k)
+        torch.cuda.synchronize()
+        assert t_ro.dtype == torch.uint32 and t_ci.dtype == torch.uint32
+        t_ro, t_ci = t_ro.cpu().numpy().astype(np.int64), t_ci.cpu().numpy().astype(np.int64)
+        assert np.array_equal(t_ro, t_ro_ref)
+        for j in range(n_k):
+            assert np.array_equal(np.sort(t_ci[t_ro[j]:t_ro[j + 1]]), t_ci_ref[t_ro_ref[j]:t_ro_ref[j + 1]]), j
+    q, k, v, d_out = _problem(n, d, torch.float32, 82, n_k)
+    part = _csr_part(dense)
+    ref = so.dense_masked_attention_backward(np64(q), np64(k), np64(v), dense, np64(d_out))
+    _, got = _grads_of(q, k, v, d_out, [spfa_autograd.csr_part(part[1], part[2], n_k)])
+    _check_grads(got, ref, torch.float32, "csr with transposed mask")
+    # an empty mask transposes to empty columns
+    z_ro, z_ci = mods["spfa_csr"].transpose(torch.zeros(5, dtype=torch.int64, device=DEV),
+                                            torch.zeros(0, dtype=torch.int32, device=DEV), 6)
+    torch.cuda.synchronize()
+    assert z_ro.cpu().tolist() == [0] * 7 and z_ci.numel() == 0
+
+
 def test_batch_of_heads_shares_the_mask(mods):
     n, d, lead = 200, 64, (2, 3)
     q, k, v, d_out = _problem(n, d, torch.float32, 31, lead=lead)
