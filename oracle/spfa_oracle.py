@@ -37,6 +37,7 @@ How each function is pinned (none of them is checked against itself):
                                finite differences of dense_masked_attention, and
                                the closed forms "one live column => dq = dk = 0,
                                dv = d_out" and "sum_j dS_ij == 0".
+  * rowwise_query_gradient   - dense_masked_attention_backward on the same mask.
 """
 from __future__ import annotations
 
@@ -171,6 +172,32 @@ def rowwise_attention(q, k, v, row_off, col_ind, m=None, l=None, out=None, use_n
         ob = (p @ v[cols]) / lb
         m[i], l[i], out[i] = merge_state(m[i], l[i], out[i], mb, lb, ob)
     return out, m, l
+
+
+def rowwise_query_gradient(q, k, v, d_out, row_off, col_ind):
+    """``dQ`` of attention over adjacency lists, row by row (each row only needs its own live
+    columns, so a sample of rows of a large problem can be checked).  Same mathematics as
+    ``dense_masked_attention_backward``; checked against it in the tests."""
+    q = np.asarray(q, dtype=np.float64)
+    k = np.asarray(k, dtype=np.float64)
+    v = np.asarray(v, dtype=np.float64)
+    d_out = np.asarray(d_out, dtype=np.float64)
+    row_off = np.asarray(row_off).astype(np.int64)
+    col_ind = np.asarray(col_ind).astype(np.int64)
+    n, d = q.shape
+    inv = 1.0 / math.sqrt(float(d))
+    d_q = np.zeros((n, d))
+    for i in range(n):
+        cols = col_ind[row_off[i]:row_off[i + 1]]
+        if len(cols) == 0:
+            continue
+        s = (k[cols] @ q[i]) * inv
+        p = np.exp(s - s.max())
+        p /= p.sum()
+        d_p = v[cols] @ d_out[i]
+        d_s = p * (d_p - p @ d_p)
+        d_q[i] = (d_s @ k[cols]) * inv
+    return d_q
 
 
 # --------------------------------------------------------------------------

@@ -187,3 +187,111 @@ def test_coo_zipf_n1m_50m_entries(mods):
     empty = torch.nonzero(deg == 0)[:4, 0].cpu().numpy()
     rows = np.unique(np.concatenate([heavy, empty, rand_rows(n, 40, 8)]))
     sample_check(q, k, v, o, m, l, rows, lambda i: c[r == i].cpu().numpy(), torch.float32)
+
+
+# ------------------------------------------------------------------ gradients at the full sizes
+def _grad_properties(q, k, v, d_out, l, dq, dk, dv, dtype):
+    """Two identities that hold for any mask: every live row's weights sum to one, so the columns
+    of dV add up to those of dO over the live rows; and sum_i q_i.dQ_i == sum_j k_j.dK_j (both are
+    sum_ij dS_ij s_ij)."""
+    live = (l > 0).double().unsqueeze(-1)
+    want = (d_out.double() * live).sum(dim=-2)
+    got = dv.double().sum(dim=-2)
+    scale = float(d_out.double().abs().sum(dim=-2).max())
+    tol = 1e-6 if dtype == torch.float32 else 3e-3
+    assert float((got - want).abs().max()) <= tol * scale
+    a = float((q.double() * dq.double()).sum())
+    b = float((k.double() * dk.double()).sum())
+    ref = float((q.double() * dq.double()).abs().sum())
+    assert abs(a - b) <= (1e-5 if dtype == torch.float32 else 2e-2) * ref
+
+
+def _dq_sample_check(q, k, v, d_out, dq, rows, live_fn, dtype):
+    rows = np.asarray(rows, dtype=np.int64)
+    cols = [np.asarray(live_fn(int(i)), dtype=np.int64) for i in rows]
+    off = np.zeros(len(rows) + 1, dtype=np.int64)
+    np.cumsum([len(c) for c in cols], out=off[1:])
+    ci = np.concatenate(cols)
+    sel = torch.as_tensor(rows).to(DEV)
+    ref = so.rowwise_query_gradient(np64(q[sel]), np64(k), np64(v), np64(d_out[sel]), off, ci)
+    err = np.abs(np64(dq[sel]) - ref).max()
+    assert err <= (2e-4 if dtype == torch.float32 else 3e-2) * max(1.0, np.abs(ref).max()), err
+
+
+def test_backward_csr_zipf_n131072(mods):
+    n, d = 131072, 64
+    q, k, v = syn.qkv(n, d, device=DEV, seed=0)
+    ro, ci = syn.zipf_csr(n, 1.5, 1, 4096, device=DEV, seed=0)
+    ro_t, ci_t = ro.to(torch.uint64), ci.to(torch.uint32)
+    val = torch.empty(0, device=DEV)
+    m, l, o = syn.fresh_state(n, d, device=DEV)
+    mods["spfa_csr"].forward(q, k, v, ro_t, ci_t, val, m, l, o, False)
+    d_out = torch.randn(n, d, device=DEV, generator=torch.Generator(device=DEV).manual_seed(5))
+    dq, dk, dv = (torch.zeros(n, d, device=DEV) for _ in range(3))
+    mods["spfa_csr"].backward(q, k, v, ro_t, ci_t, val, m, l, o, d_out, dq, dk, dv)
+    torch.cuda.synchronize()
+    _grad_properties(q, k, v, d_out, l, dq, dk, dv, torch.float32)
+    ro_c, ci_c = ro.cpu().numpy(), ci.cpu().numpy()
+    deg = ro_c[1:] - ro_c[:-1]
+    rows = np.concatenate([np.nonzero(deg == 1)[0][:10], np.nonzero(deg == 4096)[0][:6],
+                           np.nonzero((deg > 1000) & (deg < 1100))[0][:6], rand_rows(n, 60, 6)])
+    _dq_sample_check(q, k, v, d_out, dq, rows, lambda i: ci_c[ro_c[i]:ro_c[i + 1]], torch.float32)
+    # key side on a sample of columns: the rows that attend column j, weighted with the forward
+    # pass's own statistics, in float64
+    rows_of = torch.repeat_interleave(torch.arange(n, device=DEV), ro[1:] - ro[:-1])
+    lse = (m.double() + l.double().log())
+    delta = (d_out.double() * o.double()).sum(dim=1)
+    for j in rand_rows(n, 12, 7):
+        att = rows_of[ci == int(j)]
+        s = (q[att].double() @ k[j].double()) / math.sqrt(d)
+        p = torch.exp(s - lse[att])
+        ds = p * (d_out[att].double() @ v[j].double() - delta[att]) / math.sqrt(d)
+        assert float((dv[j].double() - p @ d_out[att].double()).abs().max()) <= 2e-4
+        assert float((dk[j].double() - ds @ q[att].double()).abs().max()) <= 2e-4
+    # the mask transposed once and handed in gives the same gradients (up to summation order)
+    t_ro, t_ci = mods["spfa_csr"].transpose(ro_t, ci_t, n)
+    dq2, dk2, dv2 = (torch.zeros(n, d, device=DEV) for _ in range(3))
+    mods["spfa_csr"].backward(q, k, v, ro_t, ci_t, val, m, l, o, d_out, dq2, dk2, dv2, t_ro, t_ci)
+    # (rows longer than a segment are added up in whatever order their pieces finish)
+    assert torch.allclose(dq2, dq, atol=1e-4)
+    assert torch.allclose(dk2, dk, atol=1e-4) and torch.allclose(dv2, dv, atol=1e-4)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_backward_local_n65536(mods, dtype):
+    n, d, w = 65536, 64, 128
+    q, k, v = syn.qkv(n, d, dtype=dtype, device=DEV, seed=0)
+    m, l, o = syn.fresh_state(n, d, dtype=dtype, device=DEV, state_dtype=torch.float32)
+    mods["spfa_local"].forward(q, k, v, m, l, o, w)
+    d_out = torch.randn(n, d, device=DEV, generator=torch.Generator(device=DEV).manual_seed(8)).to(dtype)
+    dq, dk, dv = (torch.zeros(n, d, device=DEV) for _ in range(3))
+    mods["spfa_local"].backward(q, k, v, m, l, o, w, d_out, dq, dk, dv)
+    torch.cuda.synchronize()
+    _grad_properties(q, k, v, d_out, l, dq, dk, dv, dtype)
+    rows = np.concatenate([[0, 1, w, n - 1, n - w - 1], rand_rows(n, 60, 9)])
+    _dq_sample_check(q, k, v, d_out, dq, rows, lambda i: so.live_local(n, w, i), dtype)
+    # the mask is symmetric: swapping the roles (q <-> k, d_out -> v's place) is not an identity,
+    # but window 0 is a closed form: p == 1, so dV == dO and dQ == dK == 0
+    m0, l0, o0 = syn.fresh_state(n, d, dtype=dtype, device=DEV, state_dtype=torch.float32)
+    mods["spfa_local"].forward(q, k, v, m0, l0, o0, 0)
+    dq0, dk0, dv0 = (torch.zeros(n, d, device=DEV) for _ in range(3))
+    mods["spfa_local"].backward(q, k, v, m0, l0, o0, 0, d_out, dq0, dk0, dv0)
+    assert torch.allclose(dv0, d_out.float(), atol=1e-5)
+    assert float(dq0.abs().max()) <= (1e-4 if dtype == torch.float32 else 0.3) and float(dk0.abs().max()) <= (
+        1e-4 if dtype == torch.float32 else 0.3)
+
+
+def test_backward_global_no_local_n1m(mods):
+    n, d, g, w = 1 << 20, 64, 64, 64
+    q, k, v = syn.qkv(n, d, device=DEV, seed=0)
+    globs = syn.global_indices(n, g, device=DEV, seed=0)
+    m, l, o = syn.fresh_state(n, d, device=DEV)
+    mods["spfa_global_no_local"].forward(q, k, v, m, l, o, globs, w)
+    d_out = torch.randn(n, d, device=DEV, generator=torch.Generator(device=DEV).manual_seed(10))
+    dq, dk, dv = (torch.zeros(n, d, device=DEV) for _ in range(3))
+    mods["spfa_global_no_local"].backward(q, k, v, m, l, o, globs, w, d_out, dq, dk, dv)
+    torch.cuda.synchronize()
+    _grad_properties(q, k, v, d_out, l, dq, dk, dv, torch.float32)
+    gl = globs.cpu().tolist()
+    rows = np.concatenate([np.asarray(gl[:3]), rand_rows(n, 40, 11)])
+    _dq_sample_check(q, k, v, d_out, dq, rows, lambda i: so.live_global_no_local(n, gl, w, i), torch.float32)

@@ -139,6 +139,18 @@ def test_backward_closed_forms():
     np.testing.assert_allclose(d_v.sum(axis=0), d_out.sum(axis=0), atol=1e-12)
 
 
+def test_rowwise_query_gradient_matches_the_dense_backward():
+    n, n_k, d = 60, 45, 8
+    q, k, v = _rand(n, d, 13, n_k)
+    rng = np.random.default_rng(14)
+    mask = rng.random((n, n_k)) < 0.3
+    mask[2] = False
+    d_out = rng.standard_normal((n, d))
+    ro, ci = so.csr_from_dense(mask)
+    ref = so.dense_masked_attention_backward(q, k, v, mask, d_out)[0]
+    np.testing.assert_allclose(so.rowwise_query_gradient(q, k, v, d_out, ro, ci), ref, rtol=0, atol=1e-13)
+
+
 def test_scale_rule_is_one_over_sqrt_d():
     # one query, two keys with a known score gap: weights must be sigmoid(gap / sqrt(d))
     d = 16
