@@ -101,6 +101,7 @@ def make_workload(name, dtype, torch, syn, inline_limit=32, planned=False, heads
             nnz = int(c.numel())
             r_t, c_t = r.to(torch.uint64), c.to(torch.uint32)
             val = torch.empty(nnz, device=dev, dtype=dtype)
+            w["bwd"] = lambda st, do, g: spfa_coo.backward(q, k, v, r_t, c_t, val, st[0], st[1], st[2], do, *g)
             if planned:
                 plan = spfa_coo.plan(r_t, c_t, n)  # mask pre-pass, outside the timed region
                 w["call"] = lambda st: spfa_coo.forward_planned(q, k, v, r_t, c_t, val, st[0], st[1], st[2],
@@ -115,6 +116,13 @@ def make_workload(name, dtype, torch, syn, inline_limit=32, planned=False, heads
             nnz = int(ci.numel())
             ro_t, ci_t = ro.to(torch.uint64), ci.to(torch.uint32)
             val = torch.empty(nnz, device=dev, dtype=dtype)
+            if planned:
+                tr = spfa_csr.transpose(ro_t, ci_t, n)  # the mask by column, for the gradients
+                w["bwd"] = lambda st, do, g: spfa_csr.backward(q, k, v, ro_t, ci_t, val, st[0], st[1], st[2],
+                                                               do, *g, *tr)
+            else:
+                w["bwd"] = lambda st, do, g: spfa_csr.backward(q, k, v, ro_t, ci_t, val, st[0], st[1], st[2],
+                                                               do, *g)
             if planned:
                 plan = spfa_csr.plan(ro_t, ci_t)  # mask pre-pass, outside the timed region
                 w["call"] = lambda st: spfa_csr.forward_planned(q, k, v, ro_t, ci_t, val, st[0], st[1], st[2],
@@ -154,6 +162,7 @@ def make_workload(name, dtype, torch, syn, inline_limit=32, planned=False, heads
                            for j in range(3)]
             nnz = syn.local_nnz(n, wsz)
             w["call"] = lambda st: spfa_local.forward(q, k, v, st[0], st[1], st[2], wsz)
+            w["bwd"] = lambda st, do, g: spfa_local.backward(q, k, v, st[0], st[1], st[2], wsz, do, *g)
             if heads > 1 and loop_heads:
                 def looped(st):
                     for h in range(heads):
@@ -167,6 +176,8 @@ def make_workload(name, dtype, torch, syn, inline_limit=32, planned=False, heads
             q, k, v = syn.qkv(n, d, dtype=dtype, device=dev, seed=0, scale=0.5)
             nnz = syn.local_1d_dilated_nnz(n, wsz, dil)
             w["call"] = lambda st: spfa_local_1d_dilated.forward(q, k, v, st[0], st[1], st[2], wsz, dil)
+            w["bwd"] = lambda st, do, g: spfa_local_1d_dilated.backward(q, k, v, st[0], st[1], st[2], wsz, dil,
+                                                                        do, *g)
             w["params"] = {"LOCAL_SIZE": wsz, "DILATE_FACTOR": dil}
             live = n
         elif name == "local_2d":
@@ -175,6 +186,8 @@ def make_workload(name, dtype, torch, syn, inline_limit=32, planned=False, heads
             q, k, v = syn.qkv(n, d, dtype=dtype, device=dev, seed=0, scale=0.5)
             nnz = syn.local_2d_dilated_nnz(n, blk, dil)
             w["call"] = lambda st: spfa_local_2d_dilated.forward(q, k, v, st[0], st[1], st[2], blk, dil, False)
+            w["bwd"] = lambda st, do, g: spfa_local_2d_dilated.backward(q, k, v, st[0], st[1], st[2], blk, dil,
+                                                                        do, *g)
             w["params"] = {"BLOCK_SIZE": blk, "DILATE_FACTOR": dil}
             live = (n // blk) * min(blk, (blk - 1) // (dil + 1) + 1)
         elif name == "bigbird":
@@ -211,6 +224,11 @@ def make_workload(name, dtype, torch, syn, inline_limit=32, planned=False, heads
                 w["call"] = chained
             else:
                 w["call"] = lambda st: spfa_bigbird.forward(q, k, v, st[0], st[1], st[2], wsz, globs, ro_t, ci_t, val)
+            def bwd_chain(st, do, gr):
+                spfa_local.backward(q, k, v, st[0], st[1], st[2], wsz, do, *gr)
+                spfa_global_no_local.backward(q, k, v, st[0], st[1], st[2], globs, wsz, do, *gr)
+                spfa_csr.backward(q, k, v, ro_t, ci_t, val, st[0], st[1], st[2], do, *gr)
+            w["bwd"] = bwd_chain
             w["params"] = {"n_globals": g, "LOCAL_SIZE": wsz, "csr_nnz": nnz_csr}
             w["globs"] = globs
             w["csr"] = (ro, ci)
@@ -224,6 +242,8 @@ def make_workload(name, dtype, torch, syn, inline_limit=32, planned=False, heads
             globs = syn.global_indices(n, g, device=dev, seed=0)
             nnz = syn.global_no_local_nnz(n, globs, wsz)
             w["call"] = lambda st: spfa_global_no_local.forward(q, k, v, st[0], st[1], st[2], globs, wsz)
+            w["bwd"] = lambda st, do, gr: spfa_global_no_local.backward(q, k, v, st[0], st[1], st[2], globs, wsz,
+                                                                        do, *gr)
             w["params"] = {"n_globals": g, "LOCAL_SIZE": wsz}
             w["globs"] = globs
             live = n
@@ -237,8 +257,9 @@ def make_workload(name, dtype, torch, syn, inline_limit=32, planned=False, heads
     return w
 
 
-def verify_sample(w, state, torch, rows=192):
-    """Max-abs error of `rows` sampled output rows against the float64 CPU oracle."""
+def verify_sample(w, state, torch, rows=192, d_out=None, d_q=None):
+    """Max-abs error of `rows` sampled output rows against the float64 CPU oracle; with d_out and
+    d_q, of the sampled rows of the query gradient instead (relative to its largest entry)."""
     import numpy as np
     from oracle import c_oracle
     from oracle import spfa_oracle as so
@@ -246,6 +267,8 @@ def verify_sample(w, state, torch, rows=192):
     if w.get("heads", 1) > 1:  # a batch of heads: the last one is checked
         w = dict(w, q=w["q"][-1], k=w["k"][-1], v=w["v"][-1])
         state = [x[-1] for x in state]
+        if d_out is not None:
+            d_out, d_q = d_out[-1], d_q[-1]
     g = torch.Generator().manual_seed(123)
     idx = torch.sort(torch.randperm(n, generator=g)[:rows])[0]
     qs = w["q"][idx.to("cuda")].float().cpu().numpy().astype(np.float64)
@@ -302,8 +325,12 @@ def verify_sample(w, state, torch, rows=192):
     off = np.zeros(len(lists) + 1, dtype=np.int64)
     np.cumsum([len(x) for x in lists], out=off[1:])
     cols = np.concatenate(lists).astype(np.int64) if len(lists) else np.zeros(0, np.int64)
-    ref_out, ref_m, ref_l = c_oracle.csr(qs, kk, vv, off, cols)
     sel = torch.as_tensor(idx_np).to("cuda")
+    if d_out is not None:
+        ref = so.rowwise_query_gradient(qs, kk, vv, d_out[sel].float().cpu().numpy().astype(np.float64), off, cols)
+        got = d_q[sel].float().cpu().numpy().astype(np.float64)
+        return float(np.abs(got - ref).max() / max(1.0, np.abs(ref).max())), len(idx_np)
+    ref_out, ref_m, ref_l = c_oracle.csr(qs, kk, vv, off, cols)
     got = state[2][sel].float().cpu().numpy().astype(np.float64)
     live_rows = ref_l > 0
     err = float(np.abs(got[live_rows] - ref_out[live_rows]).max()) if live_rows.any() else 0.0
@@ -403,6 +430,65 @@ def measured_traffic(workload, dtype_name):
     return None
 
 
+def bench_backward(a, w, st, dtype, torch, syn):
+    """--backward: one forward call builds the state, then K timed gradient calls (they add into
+    the same dQ, dK, dV; the parity check afterwards starts from zeroed gradients)."""
+    if a.loop_heads:
+        sys.exit("bench.py: --backward times the batched / single call only")
+    n, d, nnz = w["n"], w["d"], w["nnz"]
+    es = torch.tensor([], dtype=dtype).element_size()
+    w["call"](st)
+    gen = torch.Generator(device="cuda").manual_seed(1)
+    d_out = torch.randn(w["q"].shape, device="cuda", generator=gen).to(dtype)
+    grads = tuple(torch.zeros(x.shape, device="cuda", dtype=torch.float32) for x in (w["q"], w["k"], w["v"]))
+    for _ in range(a.warmup):
+        w["bwd"](st, d_out, grads)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(a.steps):
+        w["bwd"](st, d_out, grads)
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) / a.steps * 1e3
+    for g in grads:
+        g.zero_()
+    w["bwd"](st, d_out, grads)
+    torch.cuda.synchronize()
+    err, checked = verify_sample(w, st, torch, rows=64, d_out=d_out, d_q=grads[0])
+    tol = 2e-4 if dtype == torch.float32 else 3e-2
+    # every live row's weights sum to one: the columns of dV add up to those of dO
+    live = (st[1] > 0).double().unsqueeze(-1)
+    col_err = float(((grads[2].double().sum(dim=-2) - (d_out.double() * live).sum(dim=-2)).abs().max()
+                     / d_out.double().abs().sum(dim=-2).max()))
+    # algorithmic work: five products of length d per live position (scores, dO.V, dQ, dK, dV);
+    # bytes: K, V rows for the query pass and Q, dO rows for the key pass per live position, the
+    # dense tensors once (q, k, v, out, dO read; dQ, dK, dV read and written in fp32)
+    heads = w.get("heads", 1)
+    flops = 10.0 * d * nnz
+    dense = heads * n * d * (5 * es + 6 * 4)
+    gathered = nnz * 4 * d * es
+    index = nnz * 8 if w["name"].startswith(("csr", "coo", "bigbird")) else 0
+    total = dense + gathered + index
+    out = {
+        "metric": "masked-attn backward GFLOP/s (10*d per live position) + algorithmic GB/s",
+        "value": flops / (ms_per_step * 1e-3) / 1e9, "unit": "GFLOP/s",
+        "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": ms_per_step,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": a.dtype, "data": "synthetic",
+        "config": {"workload": w["desc"] + " (gradients)", "n": n, "d": d, "nnz": nnz, "seed": 0, "heads": heads,
+                   "transposed_mask": ("reused (built outside the timed region)" if a.planned else
+                                       "rebuilt every call") if w["name"].startswith("csr") else None},
+        "algorithmic_GBs": total / (ms_per_step * 1e-3) / 1e9,
+        "roofline": {"bound": "hbm", "achieved": total / (ms_per_step * 1e-3) / 1e9, "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": total / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": None,
+                     "kernel": "whole call (query pass + key pass)", "algorithmic_bytes": total,
+                     "gathered_bytes": gathered},
+        "parity": {"dq_rel_err": err, "rows_checked": checked, "tolerance": tol,
+                   "dv_column_sum_rel_err": col_err, "ok": bool(err <= tol and col_err <= (1e-5 if es == 4 else 3e-3))},
+    }
+    print(json.dumps(out))
+    if not out["parity"]["ok"]:
+        sys.exit("parity check of the gradients failed")
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -420,6 +506,9 @@ def main():
     ap.add_argument("--planned", action="store_true",
                     help="explicit masks: build the mask plan once, outside the timed region, and time "
                          "forward_planned (a mask reused across calls)")
+    ap.add_argument("--backward", action="store_true",
+                    help="time the gradient call (dQ, dK, dV from a finished forward state) instead of the "
+                         "forward call; with --planned the transposed CSR mask is built outside the timed region")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="after the timed region, run one plain 256 MiB device copy (a kernel of known "
                          "traffic that counter runs use to scale FETCH_SIZE / WRITE_SIZE)")
@@ -460,6 +549,9 @@ def main():
             st[0].fill_(-float("inf"))
             st[1].zero_()
         return st
+
+    if a.backward:
+        return bench_backward(a, w, states[0], dtype, torch, syn)
 
     ev = HipEvents()
     for i in range(a.warmup):
