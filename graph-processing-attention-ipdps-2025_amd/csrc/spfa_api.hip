@@ -196,8 +196,10 @@ int dispatch_stride(const spfa_problem_t* p, const StrideMask& mask, const Engin
 }
 
 // Band / block masks whose rows are long enough go to the dense-tile kernel.
-int dispatch_band(const spfa_problem_t* p, int64_t w, int64_t stride, int64_t block, int64_t cnt,
-                  int use_nan, hipStream_t stream) {
+// The tile problem of a band / block mask; false when it does not fit the tile kernels' index
+// arithmetic.
+bool band_tile_args(const spfa_problem_t* p, int64_t w, int64_t stride, int64_t block, int64_t cnt,
+                    TileArgs* out) {
   TileArgs a{};
   a.t = make_tensors(p);
   a.n = p->n_q;
@@ -216,8 +218,16 @@ int dispatch_band(const spfa_problem_t* p, int64_t w, int64_t stride, int64_t bl
   }
   a.tiles_per_sub = (len_max + 127) / 128;
   a.n_tiles = n_sub * a.tiles_per_sub;
-  if (a.n_tiles * a.t.n_batch + 8 >= ((int64_t)1 << 31)) return -1;
-  if (p->n_q * a.t.n_batch * p->d >= ((int64_t)1 << 40)) return -1;
+  if (a.n_tiles * a.t.n_batch + 8 >= ((int64_t)1 << 31)) return false;
+  if (p->n_q * a.t.n_batch * p->d >= ((int64_t)1 << 40)) return false;
+  *out = a;
+  return true;
+}
+
+int dispatch_band(const spfa_problem_t* p, int64_t w, int64_t stride, int64_t block, int64_t cnt,
+                  int use_nan, hipStream_t stream) {
+  TileArgs a{};
+  if (!band_tile_args(p, w, stride, block, cnt, &a)) return -1;
   switch (p->dtype) {
     case SPFA_DTYPE_F32: return run_band<float>(a, use_nan, stream);
     case SPFA_DTYPE_F16: return run_band<f16>(a, use_nan, stream);
@@ -849,11 +859,22 @@ int explicit_backward(const spfa_problem_t* p, const spfa_grads_t* g, const CsrM
   return SPFA_ERR_UNSUPPORTED;
 }
 
-int stride_backward(const spfa_problem_t* p, const spfa_grads_t* g, const StrideMask& mask,
+// tiles: whether the rows are long enough for the dense-tile kernels (the forward call's rule)
+int stride_backward(const spfa_problem_t* p, const spfa_grads_t* g, const StrideMask& mask, bool tiles,
                     const GradLayout& lay, void* workspace, hipStream_t stream) {
   if (is_f64(p)) return run_backward_stride(p->dtype, make_tensors(p), mask, make_grads(g), stream);
   const GradArgs a = make_grad_args(p, g, lay, workspace);
   const Tensors t = make_tensors(p);
+  TileArgs ta{};
+  if (tiles && band_tile_args(p, mask.w, mask.s, mask.block, mask.cnt, &ta)) {
+    int rc = -1;
+    switch (p->dtype) {
+      case SPFA_DTYPE_F32: rc = run_band_grad<float>(ta, a, stream); break;
+      case SPFA_DTYPE_F16: rc = run_band_grad<f16>(ta, a, stream); break;
+      case SPFA_DTYPE_BF16: rc = run_band_grad<bf16>(ta, a, stream); break;
+    }
+    if (rc >= 0) return rc;
+  }
   switch (p->dtype) {
     case SPFA_DTYPE_F32: return run_grad_stride<float>(t, a, mask, stream);
     case SPFA_DTYPE_F16: return run_grad_stride<f16>(t, a, mask, stream);
@@ -998,7 +1019,10 @@ int spfa_local_1d_dilated_backward(const spfa_problem_t* p, const spfa_grads_t* 
   rc = check_workspace(workspace, workspace_bytes, lay.total);
   if (rc) return rc;
   StrideMask mask{n, local_size, dil_factor + 1, 0, 0};
-  return stride_backward(p, g, mask, lay, workspace, (hipStream_t)stream);
+  const int64_t len_max = (n + dil_factor) / (dil_factor + 1);
+  const int64_t span = 2 * local_size + 1 < len_max ? 2 * local_size + 1 : len_max;
+  const bool tiles = span >= kBandTileMinRow && local_size <= kTileMaxWindow;
+  return stride_backward(p, g, mask, tiles, lay, workspace, (hipStream_t)stream);
 }
 
 size_t spfa_local_2d_dilated_backward_workspace_bytes(int64_t n, int64_t d, int dtype,
@@ -1030,7 +1054,7 @@ int spfa_local_2d_dilated_backward(const spfa_problem_t* p, const spfa_grads_t* 
   rc = check_workspace(workspace, workspace_bytes, lay.total);
   if (rc) return rc;
   StrideMask mask{n, 0, dil_factor + 1, block_size, cnt};
-  return stride_backward(p, g, mask, lay, workspace, (hipStream_t)stream);
+  return stride_backward(p, g, mask, cnt >= kBandTileMinRow, lay, workspace, (hipStream_t)stream);
 }
 
 size_t spfa_global_no_local_backward_workspace_bytes(int64_t n, int64_t d, int dtype,

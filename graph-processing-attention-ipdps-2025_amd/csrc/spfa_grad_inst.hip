@@ -1,6 +1,7 @@
 // One (mask kind, element type) instantiation of the gradient passes per object file:
 // compiled with -DSPFA_INST_MASK={0,1,2} -DSPFA_INST_T={float,spfa::f16,spfa::bf16}.
 #include "spfa_grad.hpp"
+#include "spfa_grad_tiles.hpp"
 #include "spfa_kernels.hpp"
 
 namespace spfa {
@@ -16,6 +17,10 @@ template <>
 int run_grad_stride<SPFA_INST_T>(const Tensors& t, const GradArgs& g, const StrideMask& mask,
                                  hipStream_t stream) {
   return run_grad<SPFA_INST_T>(t, g, mask, mask, stream);  // symmetric: rows and columns alike
+}
+template <>
+int run_band_grad<SPFA_INST_T>(const TileArgs& a, const GradArgs& g, hipStream_t stream) {
+  return run_band_grad_tiles<SPFA_INST_T>(a, g, stream);
 }
 #elif SPFA_INST_MASK == 2
 template <>

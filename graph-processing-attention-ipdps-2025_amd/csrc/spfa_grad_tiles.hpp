@@ -1,0 +1,336 @@
+// Gradients of band / block masks on the matrix cores: the dense-tile counterpart of the two
+// gather passes of spfa_grad.hpp, for the shapes the forward tile kernels cover.
+//
+// The masks are symmetric inside a subsequence (|t - u| <= w), so both passes are the same tile
+// problem with the roles swapped: 128 consecutive OWNER positions per workgroup (32 per
+// wavefront, one per lane column), the positions within w of them STREAMED through LDS in tiles.
+//   query pass: owner = query (q_i, dO_i in registers, lse_i, delta_i per lane), streamed = keys
+//               (K, V tiles);  dQ_i += sum_j dS_ij k_j
+//   key pass:   owner = key (k_j, v_j in registers), streamed = queries (Q, dO tiles, lse and
+//               delta of the tile in LDS);  dK_j += sum_i dS_ij q_i,  dV_j += sum_i p_ij dO_i
+// Everything is computed transposed, as in the forward tiles (streamed index on the rows of a
+// 32x32 result, owner on the columns):
+//     S^T = X A^T,  dP^T = Y B^T            (X, Y the streamed tiles; A, B the owner's vectors)
+//     P^T = exp2(S^T sc - lse),  dS^T = P^T (dP^T - delta) / sqrt(d)
+//     G1^T += X^T dS^T,  G2^T += Y^T P^T    (G2 in the key pass only)
+// The streamed tiles are row-major in LDS and serve as both operands: by rows for the first two
+// products, transposed (8-byte transposing reads for the half types, scalar reads for fp32) for
+// the last two.  No atomics: an owner row belongs to one wavefront.
+#pragma once
+
+#include "spfa_grad.hpp"
+#include "spfa_tiles.hpp"
+
+namespace spfa {
+
+template <typename T, int D>
+struct GradTileCfg {
+  static constexpr bool kF32 = sizeof(T) == 4;
+  static constexpr int BM = 128;
+  static constexpr int BN = (kF32 && D > 64) ? 32 : 64;  // streamed positions per tile
+  static constexpr int NB = BN / 32;
+  // row stride in elements: fp32 rows land on distinct banks for the by-row reads (2r + h),
+  // half rows are 16-byte aligned and 4 banks apart
+  static constexpr int STRIDE = kF32 ? D + 2 : D + 8;
+  static constexpr int TILE = BN * STRIDE;
+  static constexpr int EB = D / 32;
+  static constexpr int AREGS = kF32 ? D / 2 : D / 16;
+};
+
+template <typename T, int D, bool KEYS>
+__global__ __launch_bounds__(256, 2) void band_grad_kernel(TileArgs a, GradArgs g) {
+  using C = GradTileCfg<T, D>;
+  constexpr bool kF32 = C::kF32;
+  constexpr int BM = C::BM, BN = C::BN, EB = C::EB, NB = C::NB, ST = C::STRIDE;
+  __shared__ __attribute__((aligned(16))) T lds[2 * C::TILE];
+  __shared__ float lse_s[BN], delta_s[BN];
+  T* Xs = lds;
+  T* Ys = lds + C::TILE;
+
+  // the tile list of the forward band kernels: [problem][subsequence][tile], dealt to the XCDs
+  // in contiguous runs
+  const int64_t n_all = a.n_tiles * a.t.n_batch;
+  const int64_t per_xcd = (n_all + 7) / 8;
+  int64_t lt = (int64_t)(blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+  if (lt >= n_all) return;
+  const int64_t pb = lt / a.n_tiles;
+  lt -= pb * a.n_tiles;
+  const int64_t sub = lt / a.tiles_per_sub;
+  const int64_t tile = lt - sub * a.tiles_per_sub;
+  int64_t base, len;
+  if (a.block > 0) {
+    base = sub * a.block + pb * a.n;
+    len = a.cnt;
+  } else {
+    base = sub + pb * a.n;
+    len = (a.n - sub + a.s - 1) / a.s;
+  }
+  const int64_t t0 = tile * BM;
+  if (t0 >= len) return;
+  int64_t u_lo = t0 - a.w;
+  if (u_lo < 0) u_lo = 0;
+  int64_t u_hi = t0 + BM + a.w;
+  if (u_hi > len || u_hi < 0) u_hi = len;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int r = lane & 31, h = lane >> 5;
+  const T* Ap = (const T*)(KEYS ? g.k : g.q);      // owner vectors
+  const T* Bp = (const T*)(KEYS ? g.v : g.d_out);
+  const T* Xp = (const T*)(KEYS ? g.q : g.k);      // streamed rows
+  const T* Yp = (const T*)(KEYS ? g.d_out : g.v);
+  const float scale = 1.0f / sqrtf((float)D);
+  const float sc = 1.4426950408889634f * scale;
+
+  const int64_t tw0 = t0 + 32 * wave;  // first owner of this wavefront
+  const int64_t tq = tw0 + r;          // this lane's owner position
+  const bool own_ok = tq < len;
+  const int64_t own_tok = base + (own_ok ? tq : len - 1) * a.s;  // row of the stacked tensors
+
+  // ---- the owner's two vectors as B operands, kept in registers
+  uint4v ah[kF32 ? 1 : C::AREGS], bh[kF32 ? 1 : C::AREGS];
+  float af[kF32 ? C::AREGS : 1], bf[kF32 ? C::AREGS : 1];
+  {
+    const T* arow = Ap + own_tok * D;
+    const T* brow = Bp + own_tok * D;
+    if constexpr (kF32) {
+#pragma unroll
+      for (int c4 = 0; c4 < D / 4; c4++) {
+        const float4v x = *reinterpret_cast<const float4v*>(arow + 4 * c4);
+        const float4v y = *reinterpret_cast<const float4v*>(brow + 4 * c4);
+        af[2 * c4] = h ? x[1] : x[0];
+        af[2 * c4 + 1] = h ? x[3] : x[2];
+        bf[2 * c4] = h ? y[1] : y[0];
+        bf[2 * c4 + 1] = h ? y[3] : y[2];
+      }
+    } else {
+#pragma unroll
+      for (int ks = 0; ks < C::AREGS; ks++) {
+        ah[ks] = *reinterpret_cast<const uint4v*>(arow + 16 * ks + 8 * h);
+        bh[ks] = *reinterpret_cast<const uint4v*>(brow + 16 * ks + 8 * h);
+      }
+    }
+  }
+  // query pass: the owner's statistics (log2 units for the exponent)
+  float lse_o = 0.f, delta_o = 0.f;
+  if constexpr (!KEYS) {
+    lse_o = g.lse[own_tok] * 1.4426950408889634f;
+    delta_o = g.delta[own_tok];
+  }
+
+  f32x16 g1[EB], g2[KEYS ? EB : 1];
+#pragma unroll
+  for (int eb = 0; eb < EB; eb++)
+#pragma unroll
+    for (int v = 0; v < 16; v++) {
+      g1[eb][v] = 0.f;
+      if constexpr (KEYS) g2[eb][v] = 0.f;
+    }
+
+  // ---- streamed tiles, fetched one ahead through registers
+  constexpr int CH = kF32 ? D / 4 : D / 8;  // 16-byte chunks per row
+  constexpr int KIT = BN * CH / 256;        // chunks per thread, tile and matrix
+  uint4v xreg[KIT], yreg[KIT];
+  float lse_reg = 0.f, delta_reg = 0.f;
+
+  auto fetch = [&](int64_t ut) {
+#pragma unroll
+    for (int it = 0; it < KIT; it++) {
+      const int idx = it * 256 + tid;
+      const int j = idx / CH, c = idx % CH;
+      const int64_t u = ut + j;
+      uint4v xx = {0u, 0u, 0u, 0u}, yy = {0u, 0u, 0u, 0u};
+      if (u < u_hi) {
+        const int64_t off = (base + u * a.s) * D + (16 / (int)sizeof(T)) * c;
+        xx = *reinterpret_cast<const uint4v*>(Xp + off);
+        yy = *reinterpret_cast<const uint4v*>(Yp + off);
+      }
+      xreg[it] = xx;
+      yreg[it] = yy;
+    }
+    if constexpr (KEYS) {
+      if (tid < BN) {
+        const bool ok = ut + tid < u_hi;
+        lse_reg = ok ? g.lse[base + (ut + tid) * a.s] * 1.4426950408889634f : __builtin_inff();
+        delta_reg = ok ? g.delta[base + (ut + tid) * a.s] : 0.f;
+      }
+    }
+  };
+  auto stash = [&]() {
+#pragma unroll
+    for (int it = 0; it < KIT; it++) {
+      const int idx = it * 256 + tid;
+      const int j = idx / CH, c = idx % CH;
+      if constexpr (kF32) {
+        // rows are only 8-byte aligned
+        const float4v xx = __builtin_bit_cast(float4v, xreg[it]);
+        const float4v yy = __builtin_bit_cast(float4v, yreg[it]);
+        float* xd = (float*)Xs + j * ST + 4 * c;
+        float* yd = (float*)Ys + j * ST + 4 * c;
+        xd[0] = xx[0]; xd[1] = xx[1]; xd[2] = xx[2]; xd[3] = xx[3];
+        yd[0] = yy[0]; yd[1] = yy[1]; yd[2] = yy[2]; yd[3] = yy[3];
+      } else {
+        *reinterpret_cast<uint4v*>(Xs + j * ST + 8 * c) = xreg[it];
+        *reinterpret_cast<uint4v*>(Ys + j * ST + 8 * c) = yreg[it];
+      }
+    }
+    if constexpr (KEYS) {
+      if (tid < BN) {
+        lse_s[tid] = lse_reg;
+        delta_s[tid] = delta_reg;
+      }
+    }
+  };
+
+  // transposing reads (half types): lane 4*x + y of a group of 16 points at streamed row
+  // 4*h + x, columns 16*r_hi + 4*y .. +3 of a 32-column block; lane i of the group receives
+  // column i of the four rows
+  const int tx = (lane & 15) >> 2, ty = lane & 3, r_hi = (lane >> 4) & 1;
+  const int tadr = (4 * h + tx) * ST + 16 * r_hi + 4 * ty;  // elements
+
+  if (u_lo < u_hi) fetch(u_lo);
+  for (int64_t ut = u_lo; ut < u_hi; ut += BN) {
+    __syncthreads();  // the previous tile has been consumed
+    stash();
+    __syncthreads();
+    if (ut + BN < u_hi) fetch(ut + BN);
+
+    const uint32_t w32 = (uint32_t)a.w, w2 = 2u * (uint32_t)a.w;
+    const int rem = (int)((u_hi - ut) < BN ? (u_hi - ut) : BN);
+    const uint32_t d0 = (uint32_t)(int32_t)(ut - tq) + w32;
+#pragma unroll
+    for (int jb = 0; jb < NB; jb++) {
+      const int64_t ub = ut + 32 * jb;
+      // the block matters iff it overlaps the band of this wavefront's owners
+      const bool need = (tw0 < len) && (ub < u_hi) && (ub <= tw0 + 31 + a.w) && (ub + 31 + a.w >= tw0);
+      if (!need) continue;
+      const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+      f32x16 s = zero16, dp = zero16;
+      if constexpr (kF32) {
+        const float* xrow = (const float*)Xs + (32 * jb + r) * ST + h;
+        const float* yrow = (const float*)Ys + (32 * jb + r) * ST + h;
+#pragma unroll
+        for (int ks = 0; ks < D / 2; ks++) {
+          s = __builtin_amdgcn_mfma_f32_32x32x2f32(xrow[2 * ks], af[ks], s, 0, 0, 0);
+          dp = __builtin_amdgcn_mfma_f32_32x32x2f32(yrow[2 * ks], bf[ks], dp, 0, 0, 0);
+        }
+      } else {
+        const T* xrow = Xs + (32 * jb + r) * ST + 8 * h;
+        const T* yrow = Ys + (32 * jb + r) * ST + 8 * h;
+#pragma unroll
+        for (int ks = 0; ks < D / 16; ks++) {
+          s = mfma16<T>(*reinterpret_cast<const uint4v*>(xrow + 16 * ks), ah[ks], s);
+          dp = mfma16<T>(*reinterpret_cast<const uint4v*>(yrow + 16 * ks), bh[ks], dp);
+        }
+      }
+      // ---- weights: p (kept in s) and dS (kept in dp)
+      const bool full = (ub + 31 < u_hi) && (ub + a.w >= tw0 + 31) && (ub + 31 <= tw0 + a.w);
+#pragma unroll
+      for (int v = 0; v < 16; v++) {
+        const int j = 32 * jb + 8 * (v / 4) + 4 * h + (v % 4);
+        float ls = lse_o, dl = delta_o;
+        if constexpr (KEYS) {
+          ls = lse_s[j];
+          dl = delta_s[j];
+        }
+        float p = __builtin_amdgcn_exp2f(__builtin_fmaf(s[v], sc, -ls));
+        if (!full) {
+          const bool ok = (d0 + (uint32_t)j <= w2) && (j < rem);
+          p = ok ? p : 0.f;
+        }
+        s[v] = p;
+        dp[v] = p * (dp[v] - dl) * scale;
+      }
+      // ---- G1^T += X^T dS^T,  G2^T += Y^T P^T
+      if constexpr (kF32) {
+#pragma unroll
+        for (int v = 0; v < 16; v++) {
+          const int j = 32 * jb + 8 * (v / 4) + 4 * h + (v % 4);
+          const float* xcol = (const float*)Xs + j * ST + r;
+          const float* ycol = (const float*)Ys + j * ST + r;
+#pragma unroll
+          for (int eb = 0; eb < EB; eb++) {
+            g1[eb] = __builtin_amdgcn_mfma_f32_32x32x2f32(xcol[32 * eb], dp[v], g1[eb], 0, 0, 0);
+            if constexpr (KEYS)
+              g2[eb] = __builtin_amdgcn_mfma_f32_32x32x2f32(ycol[32 * eb], s[v], g2[eb], 0, 0, 0);
+          }
+        }
+      } else {
+        typedef short s16x4 __attribute__((ext_vector_type(4)));
+        typedef short s16x8 __attribute__((ext_vector_type(8)));
+        typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+#pragma unroll
+        for (int sl = 0; sl < 2; sl++) {
+          uint4v dsb, pb;
+#pragma unroll
+          for (int x = 0; x < 4; x++) {
+            dsb[x] = pack2<T>(dp[8 * sl + 2 * x], dp[8 * sl + 2 * x + 1]);
+            pb[x] = pack2<T>(s[8 * sl + 2 * x], s[8 * sl + 2 * x + 1]);
+          }
+          const T* xt = Xs + (32 * jb + 16 * sl) * ST + tadr;
+          const T* yt = Ys + (32 * jb + 16 * sl) * ST + tadr;
+#pragma unroll
+          for (int eb = 0; eb < EB; eb++) {
+            const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(xt + 32 * eb));
+            const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(xt + 32 * eb + 8 * ST));
+            const s16x8 both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+            g1[eb] = mfma16<T>(__builtin_bit_cast(uint4v, both), dsb, g1[eb]);
+            if constexpr (KEYS) {
+              const s16x4 lo2 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(yt + 32 * eb));
+              const s16x4 hi2 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(yt + 32 * eb + 8 * ST));
+              const s16x8 both2 = {lo2[0], lo2[1], lo2[2], lo2[3], hi2[0], hi2[1], hi2[2], hi2[3]};
+              g2[eb] = mfma16<T>(__builtin_bit_cast(uint4v, both2), pb, g2[eb]);
+            }
+          }
+        }
+      }
+    }
+  }
+
+  // ---- add into the owner's gradient rows (element 32*eb + 8*(v/4) + 4*h + v%4 in g[eb][v])
+  if (!own_ok) return;
+  float* out1 = (KEYS ? g.d_k : g.d_q) + own_tok * D;
+  float* out2 = KEYS ? g.d_v + own_tok * D : nullptr;
+#pragma unroll
+  for (int eb = 0; eb < EB; eb++)
+#pragma unroll
+    for (int g4 = 0; g4 < 4; g4++) {
+      const int e = 32 * eb + 8 * g4 + 4 * h;
+      float4v x = *reinterpret_cast<const float4v*>(out1 + e);
+#pragma unroll
+      for (int i = 0; i < 4; i++) x[i] += g1[eb][4 * g4 + i];
+      *reinterpret_cast<float4v*>(out1 + e) = x;
+      if constexpr (KEYS) {
+        float4v y = *reinterpret_cast<const float4v*>(out2 + e);
+#pragma unroll
+        for (int i = 0; i < 4; i++) y[i] += g2[eb][4 * g4 + i];
+        *reinterpret_cast<float4v*>(out2 + e) = y;
+      }
+    }
+}
+
+// Both passes of a band / block mask described by `a` (as the forward tile kernels take it).
+template <typename T, int D>
+int launch_band_grad(const TileArgs& a, const GradArgs& g, hipStream_t stream) {
+  const int64_t rows = g.n_q * g.n_batch;
+  if (rows == 0 || a.n_tiles == 0) return 0;
+  hipLaunchKernelGGL((grad_prologue_kernel<T>), dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, stream,
+                     a.t, g);
+  const int64_t grid = (a.n_tiles * a.t.n_batch + 7) / 8 * 8;
+  hipLaunchKernelGGL((band_grad_kernel<T, D, false>), dim3((unsigned)grid), dim3(256), 0, stream, a, g);
+  hipLaunchKernelGGL((band_grad_kernel<T, D, true>), dim3((unsigned)grid), dim3(256), 0, stream, a, g);
+  return hipGetLastError() == hipSuccess ? 0 : 4;
+}
+
+// Returns -1 when the shape is not covered (the caller then runs the gather passes).
+template <typename T>
+int run_band_grad_tiles(const TileArgs& a, const GradArgs& g, hipStream_t stream) {
+  if (!tile_shape_ok(a.t, sizeof(T))) return -1;
+  if (((uintptr_t)g.d_out | (uintptr_t)g.d_q | (uintptr_t)g.d_k | (uintptr_t)g.d_v) & 15) return -1;
+  if (a.t.d == 64) return launch_band_grad<T, 64>(a, g, stream);
+  if (a.t.d == 128) return launch_band_grad<T, 128>(a, g, stream);
+  return -1;
+}
+
+}  // namespace spfa

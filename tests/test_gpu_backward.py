@@ -99,6 +99,36 @@ def test_implicit_masks_match_the_oracle(mods, dtype):
         _check_grads(got, ref, dtype, parts[0][0])
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("d", [64, 128])
+def test_band_masks_on_the_tile_path(mods, dtype, d):
+    """d = 64 / 128 with rows of 32 and more live positions go to the dense-tile gradient kernels:
+    windows below, at and above a tile, sequence ends inside a tile, dilation (several
+    subsequences of unequal length), blocks with and without dilation, a stacked batch."""
+    cases = [
+        (517, [("local", 16)], lambda n: so.mask_local_dense(n, 16)),
+        (700, [("local", 150)], lambda n: so.mask_local_dense(n, 150)),
+        (300, [("local", 299)], lambda n: so.mask_local_dense(n, 299)),
+        (1000, [("local_1d_dilated", 40, 2)], lambda n: so.mask_local_1d_dilated_dense(n, 40, 2)),
+        (640, [("local_2d_dilated", 160, 0)], lambda n: so.mask_local_2d_dilated_dense(n, 160, 0)),
+        (768, [("local_2d_dilated", 256, 1)], lambda n: so.mask_local_2d_dilated_dense(n, 256, 1)),
+    ]
+    for n, parts, mask_fn in cases:
+        q, k, v, d_out = _problem(n, d, dtype, 91)
+        dense = mask_fn(n)
+        ref = so.dense_masked_attention_backward(np64(q), np64(k), np64(v), dense, np64(d_out))
+        _, got = _grads_of(q, k, v, d_out, parts)
+        _check_grads(got, ref, dtype, "%s n=%d" % (parts[0], n))
+    # a batch of problems sharing the mask
+    n, lead = 400, (3,)
+    q, k, v, d_out = _problem(n, d, dtype, 92, lead=lead)
+    dense = so.mask_local_dense(n, 50)
+    _, got = _grads_of(q, k, v, d_out, [("local", 50)])
+    for b in range(lead[0]):
+        ref = so.dense_masked_attention_backward(np64(q[b]), np64(k[b]), np64(v[b]), dense, np64(d_out[b]))
+        _check_grads([x[b] for x in got], ref, dtype, "batch %d" % b)
+
+
 @pytest.mark.parametrize("dtype", [torch.float64, torch.float32])
 def test_chained_parts_are_differentiated_as_their_union(mods, dtype):
     """window + global + random, the chain of verification/verify.py:337-352: one backward call
