@@ -37,8 +37,10 @@ struct GradTileCfg {
   static constexpr int AREGS = kF32 ? D / 2 : D / 16;
 };
 
+// d = 128 needs more than 256 registers per lane (owner vectors plus two accumulators): one
+// workgroup per CU there, two otherwise.
 template <typename T, int D, bool KEYS>
-__global__ __launch_bounds__(256, 2) void band_grad_kernel(TileArgs a, GradArgs g) {
+__global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void band_grad_kernel(TileArgs a, GradArgs g) {
   using C = GradTileCfg<T, D>;
   constexpr bool kF32 = C::kF32;
   constexpr int BM = C::BM, BN = C::BN, EB = C::EB, NB = C::NB, ST = C::STRIDE;
