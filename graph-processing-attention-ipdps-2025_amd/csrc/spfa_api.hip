@@ -1095,6 +1095,34 @@ int spfa_global_no_local_backward(const spfa_problem_t* p, const spfa_grads_t* g
   GlobalColMask cols{n, local_size, global_inds, n_globals, bits, uq, bits + (global_bits_words(n) - 1)};
   const GradArgs a = make_grad_args(p, g, lay, workspace);
   const Tensors t = make_tensors(p);
+  {
+    // dense tiles when the shape allows it (the forward call's rule); the streamed range of the
+    // listed tokens' pass is split as in the forward pass
+    const GlobalLayout fl = global_layout(n, n_globals, p->d, 1);
+    TileArgs ta{};
+    ta.t = t;
+    ta.n = n;
+    ta.w = local_size;
+    ta.s = 1;
+    ta.globs = global_inds;
+    ta.n_globs = n_globals;
+    ta.gbits = bits;
+    ta.uq = uq;
+    ta.n_uq = bits + (global_bits_words(n) - 1);
+    ta.key_run = fl.key_run;
+    ta.n_split = fl.n_split;
+    const int64_t q_tiles = (n_globals + 127) / 128;
+    if (q_tiles * fl.n_split * batch_of(p) < ((int64_t)1 << 31) && batch_of(p) < 65536 &&
+        local_size <= kTileMaxWindow && n * batch_of(p) * p->d < ((int64_t)1 << 40)) {
+      rc = -1;
+      switch (p->dtype) {
+        case SPFA_DTYPE_F32: rc = run_global_grad_dense<float>(ta, a, (hipStream_t)stream); break;
+        case SPFA_DTYPE_F16: rc = run_global_grad_dense<f16>(ta, a, (hipStream_t)stream); break;
+        case SPFA_DTYPE_BF16: rc = run_global_grad_dense<bf16>(ta, a, (hipStream_t)stream); break;
+      }
+      if (rc >= 0) return rc;
+    }
+  }
   switch (p->dtype) {
     case SPFA_DTYPE_F32: return run_grad_global<float>(t, a, rows, cols, (hipStream_t)stream);
     case SPFA_DTYPE_F16: return run_grad_global<f16>(t, a, rows, cols, (hipStream_t)stream);

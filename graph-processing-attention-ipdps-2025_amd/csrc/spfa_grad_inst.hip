@@ -28,6 +28,10 @@ int run_grad_global<SPFA_INST_T>(const Tensors& t, const GradArgs& g, const Glob
                                  const GlobalColMask& cols, hipStream_t stream) {
   return run_grad<SPFA_INST_T>(t, g, rows, cols, stream);
 }
+template <>
+int run_global_grad_dense<SPFA_INST_T>(const TileArgs& a, const GradArgs& g, hipStream_t stream) {
+  return run_global_grad_tiles<SPFA_INST_T>(a, g, stream);
+}
 #else
 #error "SPFA_INST_MASK must be 0 (csr), 1 (stride) or 2 (global)"
 #endif

@@ -16,6 +16,16 @@
 // The streamed tiles are row-major in LDS and serve as both operands: by rows for the first two
 // products, transposed (8-byte transposing reads for the half types, scalar reads for fp32) for
 // the last two.  No atomics: an owner row belongs to one wavefront.
+//
+// The global-minus-local mask is two more tile problems of the same kind (the window test
+// |i - j| > w is symmetric as well):
+//   kTileGlobalRows: owners = the distinct listed tokens, streamed = every token, the streamed
+//                    range split over workgroups (results added with atomics: a few rows only);
+//   kTileGlobalCols: owners = every token that is not listed, streamed = the listed tokens (the
+//                    list as given for the query pass - an ordinary row walks repeated entries
+//                    repeatedly - and the distinct ones for the key pass).
+// In the key pass over the listed tokens an ordinary query row counts once per occurrence of the
+// owner in the list, a listed one once.
 #pragma once
 
 #include "spfa_grad.hpp"
@@ -39,40 +49,67 @@ struct GradTileCfg {
 
 // d = 128 needs more than 256 registers per lane (owner vectors plus two accumulators): one
 // workgroup per CU there, two otherwise.
-template <typename T, int D, bool KEYS>
-__global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void band_grad_kernel(TileArgs a, GradArgs g) {
+template <typename T, int D, bool KEYS, int MODE>
+__global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void tile_grad_kernel(TileArgs a, GradArgs g) {
   using C = GradTileCfg<T, D>;
   constexpr bool kF32 = C::kF32;
   constexpr int BM = C::BM, BN = C::BN, EB = C::EB, NB = C::NB, ST = C::STRIDE;
   __shared__ __attribute__((aligned(16))) T lds[2 * C::TILE];
   __shared__ float lse_s[BN], delta_s[BN];
+  __shared__ int ktok_s[BN];    // GlobalCols: token of every streamed row of the tile
+  __shared__ float once_s[BN];  // GlobalRows key pass: 1 when the streamed query is a listed token
   T* Xs = lds;
   T* Ys = lds + C::TILE;
 
-  // the tile list of the forward band kernels: [problem][subsequence][tile], dealt to the XCDs
-  // in contiguous runs
-  const int64_t n_all = a.n_tiles * a.t.n_batch;
-  const int64_t per_xcd = (n_all + 7) / 8;
-  int64_t lt = (int64_t)(blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
-  if (lt >= n_all) return;
-  const int64_t pb = lt / a.n_tiles;
-  lt -= pb * a.n_tiles;
-  const int64_t sub = lt / a.tiles_per_sub;
-  const int64_t tile = lt - sub * a.tiles_per_sub;
-  int64_t base, len;
-  if (a.block > 0) {
-    base = sub * a.block + pb * a.n;
-    len = a.cnt;
+  // len: owner positions; [u_lo, u_hi): streamed positions of this workgroup; tok_off: first row
+  // of the problem in the stacked tensors (band mode folds it into base)
+  int64_t base = 0, len, t0, u_lo, u_hi, tok_off = 0;
+  if constexpr (MODE == kTileBand) {
+    // the tile list of the forward band kernels: [problem][subsequence][tile], dealt to the XCDs
+    // in contiguous runs
+    const int64_t n_all = a.n_tiles * a.t.n_batch;
+    const int64_t per_xcd = (n_all + 7) / 8;
+    int64_t lt = (int64_t)(blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+    if (lt >= n_all) return;
+    const int64_t pb = lt / a.n_tiles;
+    lt -= pb * a.n_tiles;
+    const int64_t sub = lt / a.tiles_per_sub;
+    const int64_t tile = lt - sub * a.tiles_per_sub;
+    if (a.block > 0) {
+      base = sub * a.block + pb * a.n;
+      len = a.cnt;
+    } else {
+      base = sub + pb * a.n;
+      len = (a.n - sub + a.s - 1) / a.s;
+    }
+    t0 = tile * BM;
+    if (t0 >= len) return;
+    u_lo = t0 - a.w;
+    if (u_lo < 0) u_lo = 0;
+    u_hi = t0 + BM + a.w;
+    if (u_hi > len || u_hi < 0) u_hi = len;
+  } else if constexpr (MODE == kTileGlobalRows) {
+    // grid: [problem][owner tile][split of the streamed range]
+    const int64_t per_problem = (int64_t)gridDim.x / a.t.n_batch;
+    const int64_t bb = blockIdx.x / per_problem;
+    const int64_t in_problem = blockIdx.x - bb * per_problem;
+    const int64_t qt = in_problem / a.n_split;
+    const int64_t split = in_problem - qt * a.n_split;
+    tok_off = bb * a.n;
+    len = (int64_t)*a.n_uq;
+    t0 = qt * BM;
+    if (t0 >= len) return;
+    u_lo = split * a.key_run;
+    u_hi = u_lo + a.key_run;
+    if (u_hi > a.n) u_hi = a.n;
   } else {
-    base = sub + pb * a.n;
-    len = (a.n - sub + a.s - 1) / a.s;
+    tok_off = (int64_t)blockIdx.y * a.n;  // one grid row per problem
+    len = a.n;
+    t0 = (int64_t)blockIdx.x * BM;
+    if (t0 >= len) return;
+    u_lo = 0;
+    u_hi = KEYS ? (int64_t)*a.n_uq : a.n_globs;
   }
-  const int64_t t0 = tile * BM;
-  if (t0 >= len) return;
-  int64_t u_lo = t0 - a.w;
-  if (u_lo < 0) u_lo = 0;
-  int64_t u_hi = t0 + BM + a.w;
-  if (u_hi > len || u_hi < 0) u_hi = len;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -87,15 +124,31 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void band_grad_kernel(TileAr
 
   const int64_t tw0 = t0 + 32 * wave;  // first owner of this wavefront
   const int64_t tq = tw0 + r;          // this lane's owner position
-  const bool own_ok = tq < len;
-  const int64_t own_tok = base + (own_ok ? tq : len - 1) * a.s;  // row of the stacked tensors
+  bool own_ok = tq < len;
+  int64_t own_tok;  // the owner's token (band: already its row of the stacked tensors)
+  if constexpr (MODE == kTileBand) {
+    own_tok = base + (own_ok ? tq : len - 1) * a.s;
+  } else if constexpr (MODE == kTileGlobalRows) {
+    own_tok = a.uq[own_ok ? tq : len - 1];
+  } else {
+    own_tok = own_ok ? tq : len - 1;
+    if (own_ok && bit_is_set(a.gbits, own_tok)) own_ok = false;  // listed tokens belong to GlobalRows
+  }
+  const int64_t own_row = own_tok + tok_off;
+  // GlobalRows key pass: how often the owner is listed (what an ordinary query row counts it as)
+  float mult_o = 1.f;
+  if constexpr (MODE == kTileGlobalRows && KEYS) {
+    int cnt = 0;
+    for (int64_t t = 0; t < a.n_globs; t++) cnt += (a.globs[t] == (int32_t)own_tok) ? 1 : 0;
+    mult_o = (float)cnt;
+  }
 
   // ---- the owner's two vectors as B operands, kept in registers
   uint4v ah[kF32 ? 1 : C::AREGS], bh[kF32 ? 1 : C::AREGS];
   float af[kF32 ? C::AREGS : 1], bf[kF32 ? C::AREGS : 1];
   {
-    const T* arow = Ap + own_tok * D;
-    const T* brow = Bp + own_tok * D;
+    const T* arow = Ap + own_row * D;
+    const T* brow = Bp + own_row * D;
     if constexpr (kF32) {
 #pragma unroll
       for (int c4 = 0; c4 < D / 4; c4++) {
@@ -117,8 +170,8 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void band_grad_kernel(TileAr
   // query pass: the owner's statistics (log2 units for the exponent)
   float lse_o = 0.f, delta_o = 0.f;
   if constexpr (!KEYS) {
-    lse_o = g.lse[own_tok] * 1.4426950408889634f;
-    delta_o = g.delta[own_tok];
+    lse_o = g.lse[own_row] * 1.4426950408889634f;
+    delta_o = g.delta[own_row];
   }
 
   f32x16 g1[EB], g2[KEYS ? EB : 1];
@@ -134,8 +187,15 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void band_grad_kernel(TileAr
   constexpr int CH = kF32 ? D / 4 : D / 8;  // 16-byte chunks per row
   constexpr int KIT = BN * CH / 256;        // chunks per thread, tile and matrix
   uint4v xreg[KIT], yreg[KIT];
-  float lse_reg = 0.f, delta_reg = 0.f;
+  float lse_reg = 0.f, delta_reg = 0.f, once_reg = 0.f;
+  int ktok_reg = 0;
 
+  // row of the stacked tensors of streamed position u
+  auto streamed_row = [&](int64_t u) -> int64_t {
+    if constexpr (MODE == kTileBand) return base + u * a.s;
+    else if constexpr (MODE == kTileGlobalRows) return u + tok_off;
+    else return (int64_t)(KEYS ? a.uq[u] : a.globs[u]) + tok_off;
+  };
   auto fetch = [&](int64_t ut) {
 #pragma unroll
     for (int it = 0; it < KIT; it++) {
@@ -144,19 +204,23 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void band_grad_kernel(TileAr
       const int64_t u = ut + j;
       uint4v xx = {0u, 0u, 0u, 0u}, yy = {0u, 0u, 0u, 0u};
       if (u < u_hi) {
-        const int64_t off = (base + u * a.s) * D + (16 / (int)sizeof(T)) * c;
+        const int64_t off = streamed_row(u) * D + (16 / (int)sizeof(T)) * c;
         xx = *reinterpret_cast<const uint4v*>(Xp + off);
         yy = *reinterpret_cast<const uint4v*>(Yp + off);
       }
       xreg[it] = xx;
       yreg[it] = yy;
     }
-    if constexpr (KEYS) {
-      if (tid < BN) {
-        const bool ok = ut + tid < u_hi;
-        lse_reg = ok ? g.lse[base + (ut + tid) * a.s] * 1.4426950408889634f : __builtin_inff();
-        delta_reg = ok ? g.delta[base + (ut + tid) * a.s] : 0.f;
+    if (tid < BN) {
+      const bool ok = ut + tid < u_hi;
+      const int64_t row = ok ? streamed_row(ut + tid) : 0;
+      if constexpr (KEYS) {
+        lse_reg = ok ? g.lse[row] * 1.4426950408889634f : __builtin_inff();
+        delta_reg = ok ? g.delta[row] : 0.f;
       }
+      if constexpr (MODE == kTileGlobalCols) ktok_reg = ok ? (int)(row - tok_off) : 0;
+      if constexpr (MODE == kTileGlobalRows && KEYS)
+        once_reg = (ok && bit_is_set(a.gbits, row - tok_off)) ? 1.f : 0.f;
     }
   };
   auto stash = [&]() {
@@ -177,11 +241,13 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void band_grad_kernel(TileAr
         *reinterpret_cast<uint4v*>(Ys + j * ST + 8 * c) = yreg[it];
       }
     }
-    if constexpr (KEYS) {
-      if (tid < BN) {
+    if (tid < BN) {
+      if constexpr (KEYS) {
         lse_s[tid] = lse_reg;
         delta_s[tid] = delta_reg;
       }
+      if constexpr (MODE == kTileGlobalCols) ktok_s[tid] = ktok_reg;
+      if constexpr (MODE == kTileGlobalRows && KEYS) once_s[tid] = once_reg;
     }
   };
 
@@ -200,12 +266,18 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void band_grad_kernel(TileAr
 
     const uint32_t w32 = (uint32_t)a.w, w2 = 2u * (uint32_t)a.w;
     const int rem = (int)((u_hi - ut) < BN ? (u_hi - ut) : BN);
-    const uint32_t d0 = (uint32_t)(int32_t)(ut - tq) + w32;
+    // a streamed row is live iff (unsigned)(delta + w) <= 2w (band; delta in positions) or > 2w
+    // (global; delta in tokens)
+    uint32_t d0;
+    if constexpr (MODE == kTileBand) d0 = (uint32_t)(int32_t)(ut - tq) + w32;
+    else if constexpr (MODE == kTileGlobalRows) d0 = (uint32_t)(int32_t)(ut - own_tok) + w32;
+    else d0 = w32 - (uint32_t)(int32_t)own_tok;
 #pragma unroll
     for (int jb = 0; jb < NB; jb++) {
       const int64_t ub = ut + 32 * jb;
-      // the block matters iff it overlaps the band of this wavefront's owners
-      const bool need = (tw0 < len) && (ub < u_hi) && (ub <= tw0 + 31 + a.w) && (ub + 31 + a.w >= tw0);
+      // band: the block matters iff it overlaps the band of this wavefront's owners
+      bool need = (tw0 < len) && (ub < u_hi);
+      if constexpr (MODE == kTileBand) need = need && (ub <= tw0 + 31 + a.w) && (ub + 31 + a.w >= tw0);
       if (!need) continue;
       const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
       f32x16 s = zero16, dp = zero16;
@@ -227,7 +299,13 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void band_grad_kernel(TileAr
         }
       }
       // ---- weights: p (kept in s) and dS (kept in dp)
-      const bool full = (ub + 31 < u_hi) && (ub + a.w >= tw0 + 31) && (ub + 31 <= tw0 + a.w);
+      bool full = false;  // every (streamed, owner) pair of the block is live
+      if constexpr (MODE == kTileBand) {
+        full = (ub + 31 < u_hi) && (ub + a.w >= tw0 + 31) && (ub + 31 <= tw0 + a.w);
+      } else if constexpr (MODE == kTileGlobalRows) {
+        const bool hit = (ub + 31 + a.w >= own_tok) && (ub <= own_tok + a.w);
+        full = (ub + 31 < u_hi) && (__builtin_amdgcn_ballot_w64(hit) == 0);
+      }
 #pragma unroll
       for (int v = 0; v < 16; v++) {
         const int j = 32 * jb + 8 * (v / 4) + 4 * h + (v % 4);
@@ -237,9 +315,13 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void band_grad_kernel(TileAr
           dl = delta_s[j];
         }
         float p = __builtin_amdgcn_exp2f(__builtin_fmaf(s[v], sc, -ls));
+        if constexpr (MODE == kTileGlobalRows && KEYS) p *= (once_s[j] != 0.f) ? 1.f : mult_o;
         if (!full) {
-          const bool ok = (d0 + (uint32_t)j <= w2) && (j < rem);
-          p = ok ? p : 0.f;
+          bool ok;
+          if constexpr (MODE == kTileBand) ok = (d0 + (uint32_t)j <= w2);
+          else if constexpr (MODE == kTileGlobalRows) ok = (d0 + (uint32_t)j > w2);
+          else ok = (d0 + (uint32_t)ktok_s[j] > w2);
+          p = (ok && j < rem) ? p : 0.f;
         }
         s[v] = p;
         dp[v] = p * (dp[v] - dl) * scale;
@@ -292,22 +374,31 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void band_grad_kernel(TileAr
 
   // ---- add into the owner's gradient rows (element 32*eb + 8*(v/4) + 4*h + v%4 in g[eb][v])
   if (!own_ok) return;
-  float* out1 = (KEYS ? g.d_k : g.d_q) + own_tok * D;
-  float* out2 = KEYS ? g.d_v + own_tok * D : nullptr;
+  float* out1 = (KEYS ? g.d_k : g.d_q) + own_row * D;
+  float* out2 = KEYS ? g.d_v + own_row * D : nullptr;
 #pragma unroll
   for (int eb = 0; eb < EB; eb++)
 #pragma unroll
     for (int g4 = 0; g4 < 4; g4++) {
       const int e = 32 * eb + 8 * g4 + 4 * h;
-      float4v x = *reinterpret_cast<const float4v*>(out1 + e);
+      if constexpr (MODE == kTileGlobalRows) {
+        // several workgroups (splits of the streamed range) add to the same row
 #pragma unroll
-      for (int i = 0; i < 4; i++) x[i] += g1[eb][4 * g4 + i];
-      *reinterpret_cast<float4v*>(out1 + e) = x;
-      if constexpr (KEYS) {
-        float4v y = *reinterpret_cast<const float4v*>(out2 + e);
+        for (int i = 0; i < 4; i++) {
+          unsafeAtomicAdd(out1 + e + i, g1[eb][4 * g4 + i]);
+          if constexpr (KEYS) unsafeAtomicAdd(out2 + e + i, g2[eb][4 * g4 + i]);
+        }
+      } else {
+        float4v x = *reinterpret_cast<const float4v*>(out1 + e);
 #pragma unroll
-        for (int i = 0; i < 4; i++) y[i] += g2[eb][4 * g4 + i];
-        *reinterpret_cast<float4v*>(out2 + e) = y;
+        for (int i = 0; i < 4; i++) x[i] += g1[eb][4 * g4 + i];
+        *reinterpret_cast<float4v*>(out1 + e) = x;
+        if constexpr (KEYS) {
+          float4v y = *reinterpret_cast<const float4v*>(out2 + e);
+#pragma unroll
+          for (int i = 0; i < 4; i++) y[i] += g2[eb][4 * g4 + i];
+          *reinterpret_cast<float4v*>(out2 + e) = y;
+        }
       }
     }
 }
@@ -320,8 +411,29 @@ int launch_band_grad(const TileArgs& a, const GradArgs& g, hipStream_t stream) {
   hipLaunchKernelGGL((grad_prologue_kernel<T>), dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, stream,
                      a.t, g);
   const int64_t grid = (a.n_tiles * a.t.n_batch + 7) / 8 * 8;
-  hipLaunchKernelGGL((band_grad_kernel<T, D, false>), dim3((unsigned)grid), dim3(256), 0, stream, a, g);
-  hipLaunchKernelGGL((band_grad_kernel<T, D, true>), dim3((unsigned)grid), dim3(256), 0, stream, a, g);
+  hipLaunchKernelGGL((tile_grad_kernel<T, D, false, kTileBand>), dim3((unsigned)grid), dim3(256), 0, stream,
+                     a, g);
+  hipLaunchKernelGGL((tile_grad_kernel<T, D, true, kTileBand>), dim3((unsigned)grid), dim3(256), 0, stream,
+                     a, g);
+  return hipGetLastError() == hipSuccess ? 0 : 4;
+}
+
+// Both passes of the global-minus-local mask: the ordinary tokens against the listed ones, then
+// the listed ones against everything (a: globs, n_globs, gbits, uq, n_uq, key_run, n_split set).
+template <typename T, int D>
+int launch_global_grad(const TileArgs& a, const GradArgs& g, hipStream_t stream) {
+  const int64_t rows = g.n_q * g.n_batch;
+  if (rows == 0) return 0;
+  hipLaunchKernelGGL((grad_prologue_kernel<T>), dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, stream,
+                     a.t, g);
+  const unsigned nb = (unsigned)a.t.n_batch;
+  const dim3 grid_cols((unsigned)((a.n + 127) / 128), nb);
+  hipLaunchKernelGGL((tile_grad_kernel<T, D, false, kTileGlobalCols>), grid_cols, dim3(256), 0, stream, a, g);
+  hipLaunchKernelGGL((tile_grad_kernel<T, D, true, kTileGlobalCols>), grid_cols, dim3(256), 0, stream, a, g);
+  const int64_t q_tiles = (a.n_globs + 127) / 128;
+  const dim3 grid_rows((unsigned)(q_tiles * a.n_split * nb));
+  hipLaunchKernelGGL((tile_grad_kernel<T, D, false, kTileGlobalRows>), grid_rows, dim3(256), 0, stream, a, g);
+  hipLaunchKernelGGL((tile_grad_kernel<T, D, true, kTileGlobalRows>), grid_rows, dim3(256), 0, stream, a, g);
   return hipGetLastError() == hipSuccess ? 0 : 4;
 }
 
@@ -332,6 +444,15 @@ int run_band_grad_tiles(const TileArgs& a, const GradArgs& g, hipStream_t stream
   if (((uintptr_t)g.d_out | (uintptr_t)g.d_q | (uintptr_t)g.d_k | (uintptr_t)g.d_v) & 15) return -1;
   if (a.t.d == 64) return launch_band_grad<T, 64>(a, g, stream);
   if (a.t.d == 128) return launch_band_grad<T, 128>(a, g, stream);
+  return -1;
+}
+
+template <typename T>
+int run_global_grad_tiles(const TileArgs& a, const GradArgs& g, hipStream_t stream) {
+  if (!tile_shape_ok(a.t, sizeof(T))) return -1;
+  if (((uintptr_t)g.d_out | (uintptr_t)g.d_q | (uintptr_t)g.d_k | (uintptr_t)g.d_v) & 15) return -1;
+  if (a.t.d == 64) return launch_global_grad<T, 64>(a, g, stream);
+  if (a.t.d == 128) return launch_global_grad<T, 128>(a, g, stream);
   return -1;
 }
 

@@ -36,6 +36,9 @@ int run_grad_stride(const Tensors& t, const GradArgs& g, const StrideMask& mask,
 // Dense-tile gradients of band / block masks; -1 when the shape is not covered.
 template <typename T>
 int run_band_grad(const TileArgs& a, const GradArgs& g, hipStream_t stream);
+// ... of the global-minus-local mask
+template <typename T>
+int run_global_grad_dense(const TileArgs& a, const GradArgs& g, hipStream_t stream);
 template <typename T>
 int run_grad_global(const Tensors& t, const GradArgs& g, const GlobalMask& rows,
                     const GlobalColMask& cols, hipStream_t stream);

@@ -112,6 +112,11 @@ def test_band_masks_on_the_tile_path(mods, dtype, d):
         (1000, [("local_1d_dilated", 40, 2)], lambda n: so.mask_local_1d_dilated_dense(n, 40, 2)),
         (640, [("local_2d_dilated", 160, 0)], lambda n: so.mask_local_2d_dilated_dense(n, 160, 0)),
         (768, [("local_2d_dilated", 256, 1)], lambda n: so.mask_local_2d_dilated_dense(n, 256, 1)),
+        (700, [("global_no_local", torch.tensor([3, 350, 699], dtype=torch.int32, device=DEV), 5)],
+         lambda n: so.mask_global_no_local_dense(n, [3, 350, 699], 5)),
+        # more listed tokens than one tile of owners (128) or of streamed rows (64)
+        (900, [("global_no_local", torch.arange(2, 900, 6, dtype=torch.int32, device=DEV), 0)],
+         lambda n: so.mask_global_no_local_dense(n, list(range(2, 900, 6)), 0)),
     ]
     for n, parts, mask_fn in cases:
         q, k, v, d_out = _problem(n, d, dtype, 91)
@@ -122,11 +127,14 @@ def test_band_masks_on_the_tile_path(mods, dtype, d):
     # a batch of problems sharing the mask
     n, lead = 400, (3,)
     q, k, v, d_out = _problem(n, d, dtype, 92, lead=lead)
-    dense = so.mask_local_dense(n, 50)
-    _, got = _grads_of(q, k, v, d_out, [("local", 50)])
-    for b in range(lead[0]):
-        ref = so.dense_masked_attention_backward(np64(q[b]), np64(k[b]), np64(v[b]), dense, np64(d_out[b]))
-        _check_grads([x[b] for x in got], ref, dtype, "batch %d" % b)
+    gl = [7, 120, 399]
+    for parts, dense in [([("local", 50)], so.mask_local_dense(n, 50)),
+                         ([("global_no_local", torch.tensor(gl, dtype=torch.int32, device=DEV), 20)],
+                          so.mask_global_no_local_dense(n, gl, 20))]:
+        _, got = _grads_of(q, k, v, d_out, parts)
+        for b in range(lead[0]):
+            ref = so.dense_masked_attention_backward(np64(q[b]), np64(k[b]), np64(v[b]), dense, np64(d_out[b]))
+            _check_grads([x[b] for x in got], ref, dtype, "%s batch %d" % (parts[0][0], b))
 
 
 @pytest.mark.parametrize("dtype", [torch.float64, torch.float32])
@@ -168,13 +176,14 @@ def test_rows_and_columns_longer_than_one_segment(mods, dtype):
         _check_grads(got, ref, dtype, parts[0][0])
 
 
+@pytest.mark.parametrize("d", [32, 64])
 @pytest.mark.parametrize("dtype", [torch.float64, torch.float32])
-def test_repeated_global_indices_count_as_often_as_in_the_forward_pass(mods, dtype):
+def test_repeated_global_indices_count_as_often_as_in_the_forward_pass(mods, dtype, d):
     """A token listed twice is walked twice by every ordinary row
     (sp_flatt_global_no_local_kernel.cu:134-162 reads the list as given) and once by listed rows.
     The dense statement of that: one extra key/value column per repetition, live for the ordinary
     rows outside their window; the gradient of the repeated token is the sum over its copies."""
-    n, d, w = 300, 32, 6
+    n, w = 300, 6  # (d = 32: gather passes, d = 64: dense tiles)
     globs = [40, 200, 40, 7]
     q, k, v, d_out = _problem(n, d, dtype, 71)
     base = so.mask_global_no_local_dense(n, sorted(set(globs)), w)
