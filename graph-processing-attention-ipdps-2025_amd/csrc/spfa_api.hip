@@ -883,8 +883,15 @@ int stride_backward(const spfa_problem_t* p, const spfa_grads_t* g, const Stride
   return SPFA_ERR_UNSUPPORTED;
 }
 
-size_t global_mask_bytes(int64_t n, int64_t n_globals) {
-  return align_up(global_bits_words(n) * 4, 256) + align_up((size_t)n_globals * 4, 256);
+// bit map of listed tokens, their distinct list, and the partial sums of the listed tokens'
+// passes: [problem][split][half][dK or dV][listed token][d] floats
+size_t global_grad_partial_bytes(int64_t n, int64_t n_globals, int64_t d, int64_t n_batch) {
+  const GlobalLayout fl = global_layout(n, n_globals, d, 1);
+  return (size_t)(n_batch > 1 ? n_batch : 1) * (size_t)fl.n_split * 4 * (size_t)n_globals * (size_t)d * 4;
+}
+size_t global_mask_bytes(int64_t n, int64_t n_globals, int64_t d, int64_t n_batch) {
+  return align_up(global_bits_words(n) * 4, 256) + align_up((size_t)n_globals * 4, 256) +
+         align_up(global_grad_partial_bytes(n, n_globals, d, n_batch), 256);
 }
 
 }  // namespace
@@ -1060,11 +1067,11 @@ int spfa_local_2d_dilated_backward(const spfa_problem_t* p, const spfa_grads_t* 
 size_t spfa_global_no_local_backward_workspace_bytes(int64_t n, int64_t d, int dtype,
                                                      int64_t n_globals, int64_t local_size,
                                                      int64_t n_batch) {
-  (void)d;
   (void)dtype;
   (void)local_size;
-  if (n < 1 || n_globals < 1) return 0;
-  return grad_layout(n, n_batch, global_items_bound(n, n_globals), global_mask_bytes(n, n_globals)).total;
+  if (n < 1 || n_globals < 1 || d < 1) return 0;
+  return grad_layout(n, n_batch, global_items_bound(n, n_globals), global_mask_bytes(n, n_globals, d, n_batch))
+      .total;
 }
 
 int spfa_global_no_local_backward(const spfa_problem_t* p, const spfa_grads_t* g,
@@ -1079,8 +1086,8 @@ int spfa_global_no_local_backward(const spfa_problem_t* p, const spfa_grads_t* g
   if (rc) return rc;
   if (!global_inds || p->n_k != p->n_q) return SPFA_ERR_BAD_ARG;
   const int64_t n = p->n_q;
-  const GradLayout lay =
-      grad_layout(n, batch_of(p), global_items_bound(n, n_globals), global_mask_bytes(n, n_globals));
+  const GradLayout lay = grad_layout(n, batch_of(p), global_items_bound(n, n_globals),
+                                     global_mask_bytes(n, n_globals, p->d, batch_of(p)));
   if (!lay.ok) return SPFA_ERR_BAD_ARG;
   rc = check_workspace(workspace, workspace_bytes, lay.total);
   if (rc) return rc;
@@ -1111,6 +1118,7 @@ int spfa_global_no_local_backward(const spfa_problem_t* p, const spfa_grads_t* g
     ta.n_uq = bits + (global_bits_words(n) - 1);
     ta.key_run = fl.key_run;
     ta.n_split = fl.n_split;
+    ta.pacc = (float*)(mbase + align_up(global_bits_words(n) * 4, 256) + align_up((size_t)n_globals * 4, 256));
     const int64_t q_tiles = (n_globals + 127) / 128;
     if (q_tiles * fl.n_split * batch_of(p) < ((int64_t)1 << 31) && batch_of(p) < 65536 &&
         local_size <= kTileMaxWindow && n * batch_of(p) * p->d < ((int64_t)1 << 40)) {

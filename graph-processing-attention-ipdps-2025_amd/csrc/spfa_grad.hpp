@@ -54,11 +54,13 @@ __device__ __forceinline__ int grad_elem_index(int c, int e) {
   return (Lay::LPR == kWave) ? c + e * kWave : c * Lay::NE + e;
 }
 
-// lse and delta of every query row
+// lse and delta of every query row: 16 lanes per row, 16 bytes per lane and step
 template <typename T>
 __global__ __launch_bounds__(256) void grad_prologue_kernel(Tensors t, GradArgs g) {
-  const int lane = threadIdx.x & (kWave - 1);
-  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  constexpr int V = 16 / (int)sizeof(T);
+  typedef T vec __attribute__((ext_vector_type(V)));
+  const int c = threadIdx.x & 15;
+  const int64_t row = (int64_t)blockIdx.x * 16 + (threadIdx.x >> 4);
   if (row >= t.n_q * t.n_batch) return;
   const bool sf = t.state_f32 != 0;
   const float m = load_state<T>(t.m, row, sf);
@@ -68,10 +70,19 @@ __global__ __launch_bounds__(256) void grad_prologue_kernel(Tensors t, GradArgs 
   if (live) {
     const T* orow = (const T*)t.out + row * t.d;
     const T* drow = (const T*)g.d_out + row * t.d;
-    for (int e = lane; e < t.d; e += kWave) acc += to_f32(orow[e]) * to_f32(drow[e]);
+    if ((t.d % V) == 0 && (((uintptr_t)t.out | (uintptr_t)g.d_out) & 15) == 0) {
+      for (int e = c * V; e < t.d; e += 16 * V) {
+        const vec a = *reinterpret_cast<const vec*>(orow + e);
+        const vec b = *reinterpret_cast<const vec*>(drow + e);
+#pragma unroll
+        for (int x = 0; x < V; x++) acc += to_f32((T)a[x]) * to_f32((T)b[x]);
+      }
+    } else {
+      for (int e = c; e < t.d; e += 16) acc += to_f32(orow[e]) * to_f32(drow[e]);
+    }
   }
-  acc = group_sum<kWave>(acc);
-  if (lane == 0) {
+  acc = group_sum<16>(acc);
+  if (c == 0) {
     g.lse[row] = live ? m + __logf(l) : __builtin_inff();
     g.delta[row] = live ? acc : 0.f;
   }
@@ -332,7 +343,7 @@ int launch_grad(const Tensors& t, const GradArgs& g, const RowMask& rows, const 
   if (nq >= ((int64_t)1 << 32) || nk >= ((int64_t)1 << 32)) return 1;  // items hold 32-bit owners
   const dim3 block(kGradWaves * kWave);
   hipLaunchKernelGGL(grad_reset_kernel, dim3(1), dim3(64), 0, stream, g.n_items);
-  hipLaunchKernelGGL((grad_prologue_kernel<T>), dim3((unsigned)((nq + 3) / 4)), dim3(256), 0, stream,
+  hipLaunchKernelGGL((grad_prologue_kernel<T>), dim3((unsigned)((nq + 15) / 16)), dim3(256), 0, stream,
                      t, g);
   hipLaunchKernelGGL((grad_rows_kernel<Lay, RowMask, false>),
                      dim3((unsigned)((nq + kGradWaves - 1) / kGradWaves)), block, 0, stream, g, rows);

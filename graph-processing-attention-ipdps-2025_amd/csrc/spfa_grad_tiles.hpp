@@ -20,7 +20,9 @@
 // The global-minus-local mask is two more tile problems of the same kind (the window test
 // |i - j| > w is symmetric as well):
 //   kTileGlobalRows: owners = the distinct listed tokens, streamed = every token, the streamed
-//                    range split over workgroups (results added with atomics: a few rows only);
+//                    range split over workgroups; every workgroup writes partial sums, which
+//                    global_grad_merge_kernel adds up (atomic adds of all the splits into the
+//                    same few rows were measured: they took longer than the products);
 //   kTileGlobalCols: owners = every token that is not listed, streamed = the listed tokens (the
 //                    list as given for the query pass - an ordinary row walks repeated entries
 //                    repeatedly - and the distinct ones for the key pass).
@@ -64,6 +66,7 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void tile_grad_kernel(TileAr
   // len: owner positions; [u_lo, u_hi): streamed positions of this workgroup; tok_off: first row
   // of the problem in the stacked tensors (band mode folds it into base)
   int64_t base = 0, len, t0, u_lo, u_hi, tok_off = 0;
+  int64_t part_bb = 0, part_split = 0;  // GlobalRows: where this workgroup's partial sums go
   if constexpr (MODE == kTileBand) {
     // the tile list of the forward band kernels: [problem][subsequence][tile], dealt to the XCDs
     // in contiguous runs
@@ -96,6 +99,8 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void tile_grad_kernel(TileAr
     const int64_t qt = in_problem / a.n_split;
     const int64_t split = in_problem - qt * a.n_split;
     tok_off = bb * a.n;
+    part_bb = bb;
+    part_split = split;
     len = (int64_t)*a.n_uq;
     t0 = qt * BM;
     if (t0 >= len) return;
@@ -122,7 +127,13 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void tile_grad_kernel(TileAr
   const float scale = 1.0f / sqrtf((float)D);
   const float sc = 1.4426950408889634f * scale;
 
-  const int64_t tw0 = t0 + 32 * wave;  // first owner of this wavefront
+  // GlobalRows with at most 64 listed tokens: only two wavefronts would have owners.  Wavefronts
+  // 0, 1 then take the first 32 streamed rows of every tile and wavefronts 2, 3 the second 32, for
+  // the same two owner blocks (two partial sums per split).
+  const bool pair_split = (MODE == kTileGlobalRows) && NB == 2 && len <= 64;
+  const int wave_q = pair_split ? (wave & 1) : wave;
+  const int wave_k = pair_split ? (wave >> 1) : -1;  // streamed block it is restricted to (-1: all)
+  const int64_t tw0 = t0 + 32 * wave_q;  // first owner of this wavefront
   const int64_t tq = tw0 + r;          // this lane's owner position
   bool own_ok = tq < len;
   int64_t own_tok;  // the owner's token (band: already its row of the stacked tensors)
@@ -276,7 +287,7 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void tile_grad_kernel(TileAr
     for (int jb = 0; jb < NB; jb++) {
       const int64_t ub = ut + 32 * jb;
       // band: the block matters iff it overlaps the band of this wavefront's owners
-      bool need = (tw0 < len) && (ub < u_hi);
+      bool need = (tw0 < len) && (ub < u_hi) && (wave_k < 0 || wave_k == jb);
       if constexpr (MODE == kTileBand) need = need && (ub <= tw0 + 31 + a.w) && (ub + 31 + a.w >= tw0);
       if (!need) continue;
       const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
@@ -382,11 +393,14 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void tile_grad_kernel(TileAr
     for (int g4 = 0; g4 < 4; g4++) {
       const int e = 32 * eb + 8 * g4 + 4 * h;
       if constexpr (MODE == kTileGlobalRows) {
-        // several workgroups (splits of the streamed range) add to the same row
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-          unsafeAtomicAdd(out1 + e + i, g1[eb][4 * g4 + i]);
-          if constexpr (KEYS) unsafeAtomicAdd(out2 + e + i, g2[eb][4 * g4 + i]);
+        // partial sums of this split (and half): [problem][split][half][which][listed token][D]
+        const int64_t slot0 = ((part_bb * a.n_split + part_split) * 2 + (wave_k > 0 ? 1 : 0)) * (KEYS ? 2 : 1);
+        float* p1 = a.pacc + (slot0 * a.n_globs + tq) * D + e;
+        const float4v x = {g1[eb][4 * g4], g1[eb][4 * g4 + 1], g1[eb][4 * g4 + 2], g1[eb][4 * g4 + 3]};
+        *reinterpret_cast<float4v*>(p1) = x;
+        if constexpr (KEYS) {
+          const float4v y = {g2[eb][4 * g4], g2[eb][4 * g4 + 1], g2[eb][4 * g4 + 2], g2[eb][4 * g4 + 3]};
+          *reinterpret_cast<float4v*>(p1 + a.n_globs * D) = y;
         }
       } else {
         float4v x = *reinterpret_cast<const float4v*>(out1 + e);
@@ -408,7 +422,7 @@ template <typename T, int D>
 int launch_band_grad(const TileArgs& a, const GradArgs& g, hipStream_t stream) {
   const int64_t rows = g.n_q * g.n_batch;
   if (rows == 0 || a.n_tiles == 0) return 0;
-  hipLaunchKernelGGL((grad_prologue_kernel<T>), dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, stream,
+  hipLaunchKernelGGL((grad_prologue_kernel<T>), dim3((unsigned)((rows + 15) / 16)), dim3(256), 0, stream,
                      a.t, g);
   const int64_t grid = (a.n_tiles * a.t.n_batch + 7) / 8 * 8;
   hipLaunchKernelGGL((tile_grad_kernel<T, D, false, kTileBand>), dim3((unsigned)grid), dim3(256), 0, stream,
@@ -418,13 +432,36 @@ int launch_band_grad(const TileArgs& a, const GradArgs& g, hipStream_t stream) {
   return hipGetLastError() == hipSuccess ? 0 : 4;
 }
 
+// Adds the partial sums of the GlobalRows passes into the gradient rows of the listed tokens: one
+// workgroup per (problem, listed token), a thread per element of (g1, g2).
+template <typename T, int D>
+__global__ __launch_bounds__(2 * D) void global_grad_merge_kernel(TileArgs a, GradArgs g, int keys) {
+  const int64_t n_uq = (int64_t)*a.n_uq;
+  const int64_t bb = blockIdx.x / a.n_globs;
+  const int64_t t = blockIdx.x - bb * a.n_globs;
+  if (t >= n_uq) return;
+  const int which = threadIdx.x / D, e = threadIdx.x % D;
+  const int n_which = keys ? 2 : 1;
+  if (which >= n_which) return;
+  const int halves = (GradTileCfg<T, D>::NB == 2 && n_uq <= 64) ? 2 : 1;  // the tile kernel's pair split
+  float acc = 0.f;
+  for (int64_t sp = 0; sp < a.n_split; sp++)
+    for (int hf = 0; hf < halves; hf++) {
+      const int64_t slot = (((bb * a.n_split + sp) * 2 + hf) * n_which + which) * a.n_globs + t;
+      acc += a.pacc[slot * D + e];
+    }
+  const int64_t row = (int64_t)a.uq[t] + bb * a.n;
+  float* out = (keys ? (which ? g.d_v : g.d_k) : g.d_q) + row * D + e;
+  *out += acc;
+}
+
 // Both passes of the global-minus-local mask: the ordinary tokens against the listed ones, then
 // the listed ones against everything (a: globs, n_globs, gbits, uq, n_uq, key_run, n_split set).
 template <typename T, int D>
 int launch_global_grad(const TileArgs& a, const GradArgs& g, hipStream_t stream) {
   const int64_t rows = g.n_q * g.n_batch;
   if (rows == 0) return 0;
-  hipLaunchKernelGGL((grad_prologue_kernel<T>), dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, stream,
+  hipLaunchKernelGGL((grad_prologue_kernel<T>), dim3((unsigned)((rows + 15) / 16)), dim3(256), 0, stream,
                      a.t, g);
   const unsigned nb = (unsigned)a.t.n_batch;
   const dim3 grid_cols((unsigned)((a.n + 127) / 128), nb);
@@ -432,8 +469,11 @@ int launch_global_grad(const TileArgs& a, const GradArgs& g, hipStream_t stream)
   hipLaunchKernelGGL((tile_grad_kernel<T, D, true, kTileGlobalCols>), grid_cols, dim3(256), 0, stream, a, g);
   const int64_t q_tiles = (a.n_globs + 127) / 128;
   const dim3 grid_rows((unsigned)(q_tiles * a.n_split * nb));
+  const dim3 grid_merge((unsigned)(a.n_globs * nb));
   hipLaunchKernelGGL((tile_grad_kernel<T, D, false, kTileGlobalRows>), grid_rows, dim3(256), 0, stream, a, g);
+  hipLaunchKernelGGL((global_grad_merge_kernel<T, D>), grid_merge, dim3(2 * D), 0, stream, a, g, 0);
   hipLaunchKernelGGL((tile_grad_kernel<T, D, true, kTileGlobalRows>), grid_rows, dim3(256), 0, stream, a, g);
+  hipLaunchKernelGGL((global_grad_merge_kernel<T, D>), grid_merge, dim3(2 * D), 0, stream, a, g, 1);
   return hipGetLastError() == hipSuccess ? 0 : 4;
 }
 
