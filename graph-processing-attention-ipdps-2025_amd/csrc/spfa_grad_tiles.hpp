@@ -432,8 +432,9 @@ int launch_band_grad(const TileArgs& a, const GradArgs& g, hipStream_t stream) {
   return hipGetLastError() == hipSuccess ? 0 : 4;
 }
 
-// Adds the partial sums of the GlobalRows passes into the gradient rows of the listed tokens: one
-// workgroup per (problem, listed token), a thread per element of (g1, g2).
+// Adds the partial sums of the GlobalRows passes into the gradient rows of the listed tokens.
+// Grid: x = (problem, listed token), y = a chunk of the splits; a thread per element of (g1, g2)
+// sums its chunk and adds it to the row with one atomic (gridDim.y adds per address).
 template <typename T, int D>
 __global__ __launch_bounds__(2 * D) void global_grad_merge_kernel(TileArgs a, GradArgs g, int keys) {
   const int64_t n_uq = (int64_t)*a.n_uq;
@@ -444,15 +445,19 @@ __global__ __launch_bounds__(2 * D) void global_grad_merge_kernel(TileArgs a, Gr
   const int n_which = keys ? 2 : 1;
   if (which >= n_which) return;
   const int halves = (GradTileCfg<T, D>::NB == 2 && n_uq <= 64) ? 2 : 1;  // the tile kernel's pair split
+  const int64_t per = (a.n_split + gridDim.y - 1) / gridDim.y;
+  const int64_t sp0 = (int64_t)blockIdx.y * per;
+  const int64_t sp1 = sp0 + per < a.n_split ? sp0 + per : a.n_split;
   float acc = 0.f;
-  for (int64_t sp = 0; sp < a.n_split; sp++)
+  for (int64_t sp = sp0; sp < sp1; sp++)
     for (int hf = 0; hf < halves; hf++) {
       const int64_t slot = (((bb * a.n_split + sp) * 2 + hf) * n_which + which) * a.n_globs + t;
       acc += a.pacc[slot * D + e];
     }
+  if (sp0 >= sp1) return;
   const int64_t row = (int64_t)a.uq[t] + bb * a.n;
   float* out = (keys ? (which ? g.d_v : g.d_k) : g.d_q) + row * D + e;
-  *out += acc;
+  unsafeAtomicAdd(out, acc);
 }
 
 // Both passes of the global-minus-local mask: the ordinary tokens against the listed ones, then
@@ -469,7 +474,11 @@ int launch_global_grad(const TileArgs& a, const GradArgs& g, hipStream_t stream)
   hipLaunchKernelGGL((tile_grad_kernel<T, D, true, kTileGlobalCols>), grid_cols, dim3(256), 0, stream, a, g);
   const int64_t q_tiles = (a.n_globs + 127) / 128;
   const dim3 grid_rows((unsigned)(q_tiles * a.n_split * nb));
-  const dim3 grid_merge((unsigned)(a.n_globs * nb));
+  // enough workgroups to fill the device, at least 8 splits each
+  int64_t chunks = 4096 / (a.n_globs * nb);
+  if (chunks > a.n_split / 8) chunks = a.n_split / 8;
+  if (chunks < 1) chunks = 1;
+  const dim3 grid_merge((unsigned)(a.n_globs * nb), (unsigned)chunks);
   hipLaunchKernelGGL((tile_grad_kernel<T, D, false, kTileGlobalRows>), grid_rows, dim3(256), 0, stream, a, g);
   hipLaunchKernelGGL((global_grad_merge_kernel<T, D>), grid_merge, dim3(2 * D), 0, stream, a, g, 0);
   hipLaunchKernelGGL((tile_grad_kernel<T, D, true, kTileGlobalRows>), grid_rows, dim3(256), 0, stream, a, g);
