@@ -162,3 +162,35 @@ def test_mask_arrays_from_torch_sparse_tensors():
         spfa_masks.csr_arrays(mask.to_sparse_coo())
     with pytest.raises(ValueError):
         spfa_masks.coo_arrays(mask)
+
+
+def test_autograd_layer_rejects_unknown_parts_before_touching_a_device():
+    import spfa_autograd
+    q = torch.zeros(4, 4)
+    with pytest.raises(ValueError, match="unknown mask part"):
+        spfa_autograd.attention(q, q, q, [("banded", 3)])
+    with pytest.raises(ValueError, match="at least one"):
+        spfa_autograd.attention(q, q, q, [])
+
+
+def test_backward_workspace_sizes_and_checks(lib):
+    i64 = ctypes.c_int64
+    for name in ("spfa_csr_backward_workspace_bytes", "spfa_coo_backward_workspace_bytes",
+                 "spfa_local_backward_workspace_bytes", "spfa_global_no_local_backward_workspace_bytes",
+                 "spfa_csr_transpose_workspace_bytes"):
+        getattr(lib, name).restype = ctypes.c_size_t
+    n, nnz, d = 131072, 13_000_000, 64
+    csr = lib.spfa_csr_backward_workspace_bytes(i64(n), i64(n), i64(nnz), i64(d), 0, i64(1))
+    coo = lib.spfa_coo_backward_workspace_bytes(i64(n), i64(n), i64(nnz), i64(d), 0, i64(1))
+    tr = lib.spfa_csr_transpose_workspace_bytes(i64(n), i64(n), i64(nnz))
+    assert 8 * n < tr < csr < coo < (1 << 30)
+    assert lib.spfa_local_backward_workspace_bytes(i64(n), i64(d), 0, i64(128), i64(4)) >= 4 * 8 * n
+    assert lib.spfa_global_no_local_backward_workspace_bytes(i64(n), i64(d), 0, i64(64), i64(64), i64(1)) > 8 * n
+    # parameter checks come first, as in the forward calls; a null gradient block is a bad argument
+    p = _problem()
+    r = ctypes.byref(p)
+    assert lib.spfa_local_backward(r, None, i64(16), None, 0, None) == 6
+    assert lib.spfa_local_2d_dilated_backward(r, None, i64(3), i64(0), None, 0, None) == 8
+    assert lib.spfa_global_no_local_backward(r, None, None, i64(0), i64(1), None, 0, None) == 10
+    assert lib.spfa_local_backward(r, None, i64(3), None, 0, None) == 1
+    assert lib.spfa_csr_backward(r, None, None, 5, None, i64(0), None, None, None, 0, None) == 1
