@@ -1,5 +1,6 @@
-// Gradients of masked attention for every mask functor (the reference has no backward pass; the
-// m and l it leaves behind are exactly the log-sum-exp statistics one needs).
+// fp64 gradients of masked attention: one plain kernel for every mask functor, double arithmetic,
+// for parity checks (torch.autograd.gradcheck) rather than speed.  The fp32 / half problems go
+// through the two gather passes of spfa_grad.hpp and the tile kernels of spfa_grad_tiles.hpp.
 //
 // With lse_i = m_i + log l_i, p_ij = exp(q_i.k_j / sqrt(d) - lse_i) on live positions and
 // delta_i = dO_i . O_i:
@@ -13,7 +14,9 @@
 // One wavefront per query row.  Candidates are taken 64 at a time: lane j holds candidate j and
 // computes both of its dot products (q_i.k_j and dO_i.v_j) from the row's q and dO kept in LDS;
 // then, candidate after candidate, lane e adds to dQ in registers and to dK_j, dV_j with
-// hardware floating-point atomics (consecutive lanes, consecutive addresses).
+// hardware floating-point atomics (consecutive lanes, consecutive addresses).  (The same kernel
+// in fp32 spent its time in those atomics - 7.8 ms at 12.8 M positions - which is why the fp32
+// path walks the mask twice instead.)
 #pragma once
 
 #include "spfa_engine.hpp"
@@ -181,17 +184,12 @@ int run_backward(const Tensors& t, const Mask& mask, const Grads& g, hipStream_t
   return hipGetLastError() == hipSuccess ? 0 : 4;
 }
 
-// element type by the C enum (0 fp32, 1 fp16, 2 bf16, 3 fp64)
+// dtype: the C enum of the element type (3 = fp64, the only one served here)
 template <class Mask>
 int run_backward_any(int dtype, const Tensors& t, const Mask& mask, const Grads& g,
                      hipStream_t stream) {
-  switch (dtype) {
-    case 0: return run_backward<float, float, Mask>(t, mask, g, stream);
-    case 1: return run_backward<f16, float, Mask>(t, mask, g, stream);
-    case 2: return run_backward<bf16, float, Mask>(t, mask, g, stream);
-    case 3: return run_backward<double, double, Mask>(t, mask, g, stream);
-  }
-  return 2;
+  if (dtype == 3) return run_backward<double, double, Mask>(t, mask, g, stream);
+  return 2;  // the other element types have kernels of their own
 }
 
 }  // namespace spfa
