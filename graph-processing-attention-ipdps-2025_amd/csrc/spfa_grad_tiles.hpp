@@ -49,10 +49,18 @@ struct GradTileCfg {
   static constexpr int AREGS = kF32 ? D / 2 : D / 16;
 };
 
-// d = 128 needs more than 256 registers per lane (owner vectors plus two accumulators): one
-// workgroup per CU there, two otherwise.
+// d = 128 needs more than 256 registers per lane (owner vectors plus accumulators) except for the
+// query pass of the half types: one workgroup per CU there, two otherwise.  (Splitting the d = 128
+// key pass into a dK and a dV launch, each at two workgroups per CU, was measured: 308 + 206 us
+// against 512 us for the combined one - no gain for 25 % more products.)
+template <typename T, int D, bool KEYS>
+constexpr int grad_tile_min_blocks() {
+  return (D > 64 && (KEYS || sizeof(T) == 4)) ? 1 : 2;
+}
+
 template <typename T, int D, bool KEYS, int MODE>
-__global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void tile_grad_kernel(TileArgs a, GradArgs g) {
+__global__ __launch_bounds__(256, (grad_tile_min_blocks<T, D, KEYS>())) void tile_grad_kernel(TileArgs a,
+                                                                                             GradArgs g) {
   using C = GradTileCfg<T, D>;
   constexpr bool kF32 = C::kF32;
   constexpr int BM = C::BM, BN = C::BN, EB = C::EB, NB = C::NB, ST = C::STRIDE;
