@@ -502,6 +502,23 @@ def bench_backward(a, w, st, dtype, torch, syn):
         sys.exit("parity check of the gradients failed")
 
 
+def measured_copy_bandwidth(torch, mib=1024, reps=5):
+    """Bytes read + written per second by a plain device-to-device copy of `mib` MiB on this box:
+    what the memory system delivers to the simplest streaming kernel, beside the vendor's 8 TB/s."""
+    src = torch.empty(mib * 1024 * 1024 // 4, dtype=torch.float32, device="cuda").normal_()
+    dst = torch.empty_like(src)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    dst.copy_(src)
+    best = float("inf")
+    for _ in range(reps):
+        e0.record()
+        dst.copy_(src)
+        e1.record()
+        torch.cuda.synchronize()
+        best = min(best, e0.elapsed_time(e1))
+    return 2.0 * src.numel() * 4 / (best * 1e-3) / 1e9
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -581,18 +598,24 @@ def main():
     ms_per_step = dt / a.steps * 1e3
 
     # dominant-kernel time: HIP events recorded inside the library around that kernel only
-    kernel_ms = []
+    kernel_ms, call_ms = [], []
     lib.spfa_set_kernel_events(ev.start, ev.stop)
+    c0, c1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     for i in range(min(a.steps, 10)):
         st = states[i % n_alloc]
         st[0].fill_(-float("inf"))
         st[1].zero_()
         torch.cuda.synchronize()
+        c0.record()
         w["call"](st)
+        c1.record()
+        c1.synchronize()
         kernel_ms.append(ev.elapsed_ms())
+        call_ms.append(c0.elapsed_time(c1))
     lib.spfa_set_kernel_events(None, None)
     torch.cuda.synchronize()
     k_avg = sum(kernel_ms) / len(kernel_ms)
+    copy_gbs = measured_copy_bandwidth(torch)
 
     if a.copy_calibration:
         src = torch.empty(64 * 1024 * 1024, dtype=torch.float32, device="cuda").normal_()
@@ -634,6 +657,13 @@ def main():
                     "kernel": "tile_kernel (global rows)" if a.workload == "global" else "tile_kernel",
                     "hbm_time_ms": w["bytes_total"] / (HBM_PEAK_GBS * 1e9) * 1e3,
                     "mfma_time_ms": flops / (peak * 1e12) * 1e3}
+    if roofline["bound"] == "hbm":
+        roofline["measured_copy_GBs"] = copy_gbs
+        roofline["frac_of_measured_copy"] = roofline["achieved"] / copy_gbs
+    else:
+        roofline["measured_copy_GBs"] = copy_gbs
+        roofline["hbm_time_at_measured_copy_ms"] = w["bytes_total"] / (copy_gbs * 1e9) * 1e3
+    call_sorted = sorted(call_ms)
     roofline.update({"kernel_ms_avg": k_avg, "kernel_ms_min": min(kernel_ms),
                      "algorithmic_bytes": w["kernel_bytes"], "kernel_nnz": w["kernel_nnz"],
                      "kernel_rows": w["kernel_rows"], "call_algorithmic_bytes": w["bytes_total"],
@@ -652,6 +682,7 @@ def main():
                    "heads_call": ("one call per head" if a.loop_heads else "one batched call") if a.heads > 1 else "single",
                    "composite_call": (("three chained calls" if a.loop_heads else "one call (spfa_bigbird)")
                                       if a.workload == "bigbird" else None)},
+        "call_ms_median": call_sorted[len(call_sorted) // 2], "call_ms_min": call_sorted[0],
         "effective_gathered_GBs": w["bytes_gathered"] / (ms_per_step * 1e-3) / 1e9,
         "algorithmic_GBs": w["bytes_total"] / (ms_per_step * 1e-3) / 1e9,
         "roofline": roofline,
