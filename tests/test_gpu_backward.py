@@ -282,3 +282,43 @@ def test_backward_adds_to_the_given_gradients_and_checks_parameters(mods):
         mods["spfa_local"].backward(q, k, v, m, l, o, 3, d_out, dq.half(), dk, dv)
     with pytest.raises(RuntimeError, match="dO must have the shape"):
         mods["spfa_local"].backward(q, k, v, m, l, o, 3, d_out[:-1].contiguous(), dq, dk, dv)
+
+
+@pytest.mark.parametrize("d", [1, 3, 512, 1024])
+def test_extreme_embedding_sizes(mods, d):
+    """d = 1 .. 1024 (the limit the forward calls accept) through the general lane layouts."""
+    n = 96
+    q, k, v, d_out = _problem(n, d, torch.float32, 101)
+    dense = np.random.default_rng(102).random((n, n)) < 0.2
+    dense[np.arange(n), np.arange(n)] = True
+    ref = so.dense_masked_attention_backward(np64(q), np64(k), np64(v), dense, np64(d_out))
+    _, got = _grads_of(q, k, v, d_out, [_csr_part(dense)])
+    _check_grads(got, ref, torch.float32, "csr d=%d" % d)
+    ref = so.dense_masked_attention_backward(np64(q), np64(k), np64(v), so.mask_local_dense(n, 40), np64(d_out))
+    _, got = _grads_of(q, k, v, d_out, [("local", 40)])
+    _check_grads(got, ref, torch.float32, "local d=%d" % d)
+
+
+def test_empty_masks_and_dead_rows_leave_gradients_alone(mods):
+    n, d = 50, 16
+    q, k, v, d_out = _problem(n, d, torch.float32, 111)
+    empty = np.zeros((n, n), dtype=bool)
+    out, got = _grads_of(q, k, v, d_out, [_csr_part(empty)])
+    assert not np64(out).any()
+    for x in got:
+        assert not np64(x).any()
+    # use_nan forward leaves NaN rows in out; the backward call must not spread them
+    dense = np.random.default_rng(112).random((n, n)) < 0.1
+    dense[7] = False
+    part = _csr_part(dense)
+    m = torch.full((n,), -float("inf"), device=DEV)
+    l = torch.zeros(n, device=DEV)
+    o = torch.zeros(n, d, device=DEV)
+    val = torch.empty(0, device=DEV)
+    mods["spfa_csr"].forward(q, k, v, part[1], part[2], val, m, l, o, True)
+    assert torch.isnan(o[7]).all()
+    dq, dk, dv = (torch.zeros(n, d, device=DEV) for _ in range(3))
+    mods["spfa_csr"].backward(q, k, v, part[1], part[2], val, m, l, o, d_out, dq, dk, dv)
+    torch.cuda.synchronize()
+    ref = so.dense_masked_attention_backward(np64(q), np64(k), np64(v), dense, np64(d_out))
+    _check_grads((dq, dk, dv), ref, torch.float32, "NaN rows in out")
