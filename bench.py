@@ -224,11 +224,9 @@ def make_workload(name, dtype, torch, syn, inline_limit=32, planned=False, heads
                 w["call"] = chained
             else:
                 w["call"] = lambda st: spfa_bigbird.forward(q, k, v, st[0], st[1], st[2], wsz, globs, ro_t, ci_t, val)
-            def bwd_chain(st, do, gr):
-                spfa_local.backward(q, k, v, st[0], st[1], st[2], wsz, do, *gr)
-                spfa_global_no_local.backward(q, k, v, st[0], st[1], st[2], globs, wsz, do, *gr)
-                spfa_csr.backward(q, k, v, ro_t, ci_t, val, st[0], st[1], st[2], do, *gr)
-            w["bwd"] = bwd_chain
+            tr = spfa_csr.transpose(ro_t, ci_t, n) if planned else ()  # the random part by column
+            w["bwd"] = lambda st, do, gr: spfa_bigbird.backward(q, k, v, st[0], st[1], st[2], wsz, globs, ro_t,
+                                                                ci_t, val, do, *gr, *tr)
             w["params"] = {"n_globals": g, "LOCAL_SIZE": wsz, "csr_nnz": nnz_csr}
             w["globs"] = globs
             w["csr"] = (ro, ci)
@@ -491,7 +489,7 @@ def bench_backward(a, w, st, dtype, torch, syn):
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": a.dtype, "data": "synthetic",
         "config": {"workload": w["desc"] + " (gradients)", "n": n, "d": d, "nnz": nnz, "seed": 0, "heads": heads,
                    "transposed_mask": ("reused (built outside the timed region)" if a.planned else
-                                       "rebuilt every call") if w["name"].startswith("csr") else None},
+                                       "rebuilt every call") if w["name"].startswith(("csr", "bigbird")) else None},
         "algorithmic_GBs": total / (ms_per_step * 1e-3) / 1e9,
         "roofline": roofline,
         "parity": {"dq_rel_err": err, "rows_checked": checked, "tolerance": tol,
@@ -554,8 +552,8 @@ def main():
     torch.cuda.set_device(0)
     dtype = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}[a.dtype]
     lib = load_library()
-    if a.planned and not (a.workload.startswith("csr") or a.workload.startswith("coo")):
-        sys.exit("bench.py: --planned applies to the explicit-mask workloads (csr_*, coo_*)")
+    if a.planned and not (a.workload.startswith(("csr", "coo")) or (a.workload == "bigbird" and a.backward)):
+        sys.exit("bench.py: --planned applies to the explicit-mask workloads (csr_*, coo_*; bigbird with --backward)")
     if a.heads > 1 and not (a.workload.startswith("csr") or a.workload == "local"):
         sys.exit("bench.py: --heads applies to the csr_* and local workloads")
     w = make_workload(a.workload, dtype, torch, syn, int(lib.spfa_explicit_inline_row_limit()), a.planned,

@@ -1139,4 +1139,54 @@ int spfa_global_no_local_backward(const spfa_problem_t* p, const spfa_grads_t* g
   return SPFA_ERR_UNSUPPORTED;
 }
 
+/* window + global + CSR: the three gradient calls behind one entry point, like the forward one */
+size_t spfa_window_global_csr_backward_workspace_bytes(int64_t n, int64_t d, int dtype,
+                                                       int64_t local_size, int64_t n_globals,
+                                                       int64_t nnz, int64_t n_batch) {
+  size_t need = spfa_local_backward_workspace_bytes(n, d, dtype, local_size, n_batch);
+  if (n_globals > 0) {
+    const size_t g = spfa_global_no_local_backward_workspace_bytes(n, d, dtype, n_globals, local_size, n_batch);
+    if (g > need) need = g;
+  }
+  if (nnz > 0) {
+    const size_t c = spfa_csr_backward_workspace_bytes(n, n, nnz, d, dtype, n_batch);
+    if (c > need) need = c;
+  }
+  return need;
+}
+
+int spfa_window_global_csr_backward(const spfa_problem_t* p, const spfa_grads_t* g, int64_t local_size,
+                                    const int32_t* global_inds, int64_t n_globals, const void* row_off,
+                                    int row_off_bytes, const void* col_ind, int64_t nnz,
+                                    const uint32_t* t_row_off, const uint32_t* t_col_ind, void* workspace,
+                                    size_t workspace_bytes, void* stream) {
+  // every parameter check of the three parts, before anything is enqueued
+  int rc = check_problem(p);
+  if (rc) return rc;
+  if (p->n_k != p->n_q) return SPFA_ERR_BAD_ARG;
+  if (local_size < 0 || local_size > p->n_q - 1) return SPFA_ERR_LOCAL_SIZE;
+  if (n_globals < 0 || n_globals > p->n_q) return SPFA_ERR_GLOBAL_COUNT;
+  if (nnz < 0 || (nnz > 0 && row_off_bytes != 4 && row_off_bytes != 8)) return SPFA_ERR_BAD_ARG;
+  if ((t_row_off == nullptr) != (t_col_ind == nullptr)) return SPFA_ERR_BAD_ARG;
+  rc = check_grads(p, g);
+  if (rc) return rc;
+  if (p->n_q == 0) return SPFA_OK;
+  if ((n_globals > 0 && !global_inds) || (nnz > 0 && (!row_off || !col_ind))) return SPFA_ERR_BAD_ARG;
+  rc = check_workspace(workspace, workspace_bytes,
+                       spfa_window_global_csr_backward_workspace_bytes(p->n_q, p->d, p->dtype, local_size,
+                                                                       n_globals, nnz, batch_of(p)));
+  if (rc) return rc;
+  rc = spfa_local_backward(p, g, local_size, workspace, workspace_bytes, stream);
+  if (rc) return rc;
+  if (n_globals > 0) {
+    rc = spfa_global_no_local_backward(p, g, global_inds, n_globals, local_size, workspace, workspace_bytes,
+                                       stream);
+    if (rc) return rc;
+  }
+  if (nnz > 0)
+    rc = spfa_csr_backward(p, g, row_off, row_off_bytes, col_ind, nnz, t_row_off, t_col_ind, workspace,
+                           workspace_bytes, stream);
+  return rc;
+}
+
 }  // extern "C"

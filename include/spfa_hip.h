@@ -264,6 +264,17 @@ int spfa_global_no_local_backward(const spfa_problem_t* p, const spfa_grads_t* g
                                   int64_t local_size, void* workspace, size_t workspace_bytes,
                                   void* stream);
 
+/* The gradients of spfa_window_global_csr_forward: the three parts' gradient calls in sequence on
+ * one workspace (t_row_off / t_col_ind as in spfa_csr_backward, may be NULL). */
+size_t spfa_window_global_csr_backward_workspace_bytes(int64_t n, int64_t d, int dtype,
+                                                       int64_t local_size, int64_t n_globals,
+                                                       int64_t nnz, int64_t n_batch);
+int spfa_window_global_csr_backward(const spfa_problem_t* p, const spfa_grads_t* g, int64_t local_size,
+                                    const int32_t* global_inds, int64_t n_globals, const void* row_off,
+                                    int row_off_bytes, const void* col_ind, int64_t nnz,
+                                    const uint32_t* t_row_off, const uint32_t* t_col_ind, void* workspace,
+                                    size_t workspace_bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -322,3 +322,34 @@ def test_empty_masks_and_dead_rows_leave_gradients_alone(mods):
     torch.cuda.synchronize()
     ref = so.dense_masked_attention_backward(np64(q), np64(k), np64(v), dense, np64(d_out))
     _check_grads((dq, dk, dv), ref, torch.float32, "NaN rows in out")
+
+
+def test_composite_backward_equals_dense_union(mods):
+    """spfa_bigbird.backward == gradients of dense attention over window | global | random, with
+    and without the transposed CSR part handed in; parts may be empty."""
+    n, d, w = 600, 64, 9
+    globs = [4, 333]
+    rng = np.random.default_rng(121)
+    union = so.mask_local_dense(n, w) | so.mask_global_no_local_dense(n, globs, w)
+    rand = (rng.random((n, n)) < 0.02) & ~union
+    ro, ci = so.csr_from_dense(rand)
+    ro_t = torch.as_tensor(ro).to(torch.uint64).to(DEV)
+    ci_t = torch.as_tensor(ci).to(torch.uint32).to(DEV)
+    gl = torch.tensor(globs, dtype=torch.int32, device=DEV)
+    q, k, v, d_out = _problem(n, d, torch.float32, 122)
+    val = torch.empty(0, device=DEV)
+    tr = mods["spfa_csr"].transpose(ro_t, ci_t, n)
+    none_i = torch.zeros(0, dtype=torch.int32, device=DEV)
+    none_o = torch.zeros(0, dtype=torch.int64, device=DEV)
+    for gl_arg, csr_arg, dense, extra in [(gl, (ro_t, ci_t), union | rand, ()), (gl, (ro_t, ci_t), union | rand, tr),
+                                          (none_i, (none_o, none_i), so.mask_local_dense(n, w), ())]:
+        m = torch.full((n,), -float("inf"), device=DEV)
+        l = torch.zeros(n, device=DEV)
+        o = torch.zeros(n, d, device=DEV)
+        mods["spfa_bigbird"].forward(q, k, v, m, l, o, w, gl_arg, csr_arg[0], csr_arg[1], val)
+        dq, dk, dv = (torch.zeros(n, d, device=DEV) for _ in range(3))
+        mods["spfa_bigbird"].backward(q, k, v, m, l, o, w, gl_arg, csr_arg[0], csr_arg[1], val, d_out, dq, dk, dv,
+                                      *extra)
+        torch.cuda.synchronize()
+        ref = so.dense_masked_attention_backward(np64(q), np64(k), np64(v), dense, np64(d_out))
+        _check_grads((dq, dk, dv), ref, torch.float32, "composite")
