@@ -622,16 +622,18 @@ KernelEvents& kernel_events();
 
 constexpr int kSegmentWorkgroupsPerCu = 1;
 
+// compute units of the current device (looked up once per device)
 inline int device_cu_count() {
-  static int cus = 0;
-  if (cus == 0) {
-    int dev = 0;
-    hipDeviceProp_t prop;
-    if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
-      cus = prop.multiProcessorCount;
-    if (cus <= 0) cus = 256;
+  constexpr int kMaxDevices = 64;
+  static int cus[kMaxDevices];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return 256;
+  if (cus[dev] == 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    cus[dev] = n;
   }
-  return cus;
+  return cus[dev];
 }
 
 // What a call does: the whole thing, only the work list of the mask (a "plan": counters, items,

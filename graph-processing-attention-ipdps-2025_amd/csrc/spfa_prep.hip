@@ -422,14 +422,18 @@ int coo_to_csr(const void* row_ind, int row_wide, const uint32_t* col_ind, int64
   if (nnz > 0 && w.partition) {
     uint32_t* hist = (uint32_t*)(base + w.off_hist);
     uint64_t* tmp_pairs = (uint64_t*)(base + w.off_tmp_pairs);
-    static bool lds_attr_set = false;
-    if (!lds_attr_set) {
-      // 88 KB of LDS per workgroup: above the 64 KB a kernel gets without asking
+    // 88 KB of LDS per workgroup: above the 64 KB a kernel gets without asking (set once per
+    // device: the attribute belongs to the device's copy of the kernel)
+    constexpr int kMaxDevices = 64;
+    static bool lds_attr_set[kMaxDevices];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return 4;
+    if (dev < 0 || dev >= kMaxDevices || !lds_attr_set[dev]) {
       if (hipFuncSetAttribute(reinterpret_cast<const void*>(coo_part_scatter_kernel),
                               hipFuncAttributeMaxDynamicSharedMemorySize,
                               (int)kPartScatterLds) != hipSuccess)
         return 4;
-      lds_attr_set = true;
+      if (dev >= 0 && dev < kMaxDevices) lds_attr_set[dev] = true;
     }
     const int64_t n_hist = w.n_hi * w.n_tiles1;
     const int64_t hist_tiles = (n_hist + kScanTile - 1) / kScanTile;
