@@ -534,6 +534,9 @@ def main():
     ap.add_argument("--planned", action="store_true",
                     help="explicit masks: build the mask plan once, outside the timed region, and time "
                          "forward_planned (a mask reused across calls)")
+    ap.add_argument("--graph", action="store_true",
+                    help="capture one step (state reset + the call) in a HIP graph and time K replays "
+                         "(for the launch-bound small workloads)")
     ap.add_argument("--backward", action="store_true",
                     help="time the gradient call (dQ, dK, dV from a finished forward state) instead of the "
                          "forward call; with --planned the transposed CSR mask is built outside the timed region")
@@ -586,13 +589,34 @@ def main():
         w["call"](fresh(i))
     torch.cuda.synchronize()
 
-    # timed region: exactly K steps
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for i in range(a.steps):
-        w["call"](fresh(a.warmup + i))
-    torch.cuda.synchronize()
-    dt = time.perf_counter() - t0
+    if a.graph:
+        # one step = reset of (m, l) + the call, captured once; the timed region replays it K times
+        gst = states[0]
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            w["call"](gst)
+        torch.cuda.current_stream().wait_stream(side)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            gst[0].fill_(-float("inf"))
+            gst[1].zero_()
+            w["call"](gst)
+        graph.replay()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(a.steps):
+            graph.replay()
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+    else:
+        # timed region: exactly K steps
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(a.steps):
+            w["call"](fresh(a.warmup + i))
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
     ms_per_step = dt / a.steps * 1e3
 
     # dominant-kernel time: HIP events recorded inside the library around that kernel only
@@ -676,7 +700,7 @@ def main():
         "config": {"workload": w["desc"], "n": n, "d": d, "nnz": nnz, "seed": 0,
                    "index_dtypes": "uint64 offsets / uint32 columns", "state": "fresh m=-inf l=0 each step",
                    "mask_plan": "reused (built outside the timed region)" if a.planned else "rebuilt every call",
-                   "heads": max(1, a.heads),
+                   "heads": max(1, a.heads), "hip_graph": bool(a.graph),
                    "heads_call": ("one call per head" if a.loop_heads else "one batched call") if a.heads > 1 else "single",
                    "composite_call": (("three chained calls" if a.loop_heads else "one call (spfa_bigbird)")
                                       if a.workload == "bigbird" else None)},
