@@ -40,3 +40,33 @@ def coo_arrays(sparse_coo, value_dtype=None):
     if value_dtype is not None:
         w_val = w_val.to(value_dtype)
     return w_row_ind, w_col_ind, w_val.contiguous()
+
+
+def stack_csr_masks(masks, n_cols):
+    """One CSR mask for several problems that each have a mask of their own (heads with different
+    masks): problem b's rows and columns are shifted by b * n_rows and b * n_cols, so the masks
+    form a block diagonal and
+
+        row_off, col_ind = stack_csr_masks([(ro_0, ci_0), (ro_1, ci_1), ...], n_cols)
+        spfa_csr.forward(q.reshape(-1, d), k.reshape(-1, d), v.reshape(-1, d), row_off, col_ind, w_val,
+                         m.reshape(-1), l.reshape(-1), out.reshape(-1, d), use_nan)
+
+    runs all of them in one call on the stacked [B * n, d] tensors (the batched call with leading
+    dimensions is for problems that SHARE a mask).  masks: sequence of (w_row_off, w_col_ind), all
+    with the same number of rows; returns (uint64 offsets, uint32 columns)."""
+    masks = list(masks)
+    if not masks:
+        raise ValueError("no masks given")
+    n_rows = masks[0][0].numel() - 1
+    offs, cols = [], []
+    base = 0
+    for b, (ro, ci) in enumerate(masks):
+        if ro.numel() - 1 != n_rows:
+            raise ValueError("all masks must have the same number of rows")
+        ro64 = ro.to(torch.int64)
+        offs.append(ro64[:-1] + base if b + 1 < len(masks) else ro64 + base)
+        cols.append(ci.to(torch.int64) + b * n_cols)
+        base += int(ro64[-1])
+    if len(masks) * n_cols >= 1 << 32:
+        raise ValueError("stacked column indices do not fit 32 bits")
+    return torch.cat(offs).to(torch.uint64).contiguous(), torch.cat(cols).to(torch.uint32).contiguous()

@@ -194,3 +194,25 @@ def test_backward_workspace_sizes_and_checks(lib):
     assert lib.spfa_global_no_local_backward(r, None, None, i64(0), i64(1), None, 0, None) == 10
     assert lib.spfa_local_backward(r, None, i64(3), None, 0, None) == 1
     assert lib.spfa_csr_backward(r, None, None, 5, None, i64(0), None, None, None, 0, None) == 1
+
+
+def test_stacked_per_head_masks_form_a_block_diagonal():
+    import numpy as np
+    import spfa_masks
+    from oracle import spfa_oracle as so
+    rng = np.random.default_rng(9)
+    n, n_k = 11, 7
+    dense = [rng.random((n, n_k)) < p for p in (0.0, 0.3, 0.9)]
+    parts = []
+    for dm in dense:
+        ro, ci = so.csr_from_dense(dm)
+        parts.append((torch.as_tensor(ro).to(torch.uint64), torch.as_tensor(ci).to(torch.uint32)))
+    ro, ci = spfa_masks.stack_csr_masks(parts, n_k)
+    big = np.zeros((3 * n, 3 * n_k), dtype=bool)
+    for b, dm in enumerate(dense):
+        big[b * n:(b + 1) * n, b * n_k:(b + 1) * n_k] = dm
+    ro_ref, ci_ref = so.csr_from_dense(big)
+    assert ro.dtype == torch.uint64 and ci.dtype == torch.uint32
+    assert np.array_equal(ro.to(torch.int64).numpy(), ro_ref) and np.array_equal(ci.to(torch.int64).numpy(), ci_ref)
+    with pytest.raises(ValueError):
+        spfa_masks.stack_csr_masks([], n_k)

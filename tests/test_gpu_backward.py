@@ -353,3 +353,25 @@ def test_composite_backward_equals_dense_union(mods):
         torch.cuda.synchronize()
         ref = so.dense_masked_attention_backward(np64(q), np64(k), np64(v), dense, np64(d_out))
         _check_grads((dq, dk, dv), ref, torch.float32, "composite")
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_statistics_stored_in_the_element_type(mods, dtype):
+    """m and l in the element type (the reference's convention) instead of float32: the gradient
+    calls read them the same way the forward calls wrote them.  m is then rounded to 8 / 11 bits,
+    so the bar is the statistics' own (1e-1 on m + log l, as in the forward tests)."""
+    n, d, w = 300, 64, 20
+    q, k, v, d_out = _problem(n, d, dtype, 131)
+    for name, args, dense in [("spfa_local", (w,), so.mask_local_dense(n, w)),
+                              ("spfa_local_1d_dilated", (5, 1), so.mask_local_1d_dilated_dense(n, 5, 1))]:
+        m = torch.full((n,), -float("inf"), device=DEV, dtype=dtype)
+        l = torch.zeros(n, device=DEV, dtype=dtype)
+        o = torch.zeros(n, d, device=DEV, dtype=dtype)
+        mods[name].forward(q, k, v, m, l, o, *args)
+        dq, dk, dv = (torch.zeros(n, d, device=DEV) for _ in range(3))
+        mods[name].backward(q, k, v, m, l, o, *args, d_out, dq, dk, dv)
+        torch.cuda.synchronize()
+        ref = so.dense_masked_attention_backward(np64(q), np64(k), np64(v), dense, np64(d_out))
+        for nm, a, b in zip(("dq", "dk", "dv"), (dq, dk, dv), ref):
+            err = float(np.abs(np64(a) - b).max())
+            assert err <= 0.15 * max(1.0, float(np.abs(b).max())), "%s %s: %.3e" % (name, nm, err)

@@ -485,6 +485,34 @@ def test_fp64_chained_calls_accumulate(mods):
     check(o, m, l, *so.dense_masked_attention(np64(q), np64(k), np64(v), dense), torch.float64)
 
 
+def test_heads_with_masks_of_their_own_in_one_call(mods):
+    """spfa_masks.stack_csr_masks: heads whose masks differ run as one block-diagonal problem on the
+    stacked tensors (the batched call is for heads that share a mask)."""
+    import spfa_masks
+    n, n_k, d, heads = 200, 260, 64, 3
+    rng = np.random.default_rng(141)
+    dense = [rng.random((n, n_k)) < p for p in (0.05, 0.3, 0.01)]
+    parts = []
+    for dm in dense:
+        ro, ci = so.csr_from_dense(dm)
+        parts.append(csr_tensors(ro, ci))
+    ro_t, ci_t = spfa_masks.stack_csr_masks(parts, n_k)
+    g = torch.Generator().manual_seed(142)
+    q = torch.randn(heads, n, d, generator=g).to(DEV)
+    k = torch.randn(heads, n_k, d, generator=g).to(DEV)
+    v = torch.randn(heads, n_k, d, generator=g).to(DEV)
+    m = torch.full((heads, n), -float("inf"), device=DEV)
+    l = torch.zeros(heads, n, device=DEV)
+    o = torch.zeros(heads, n, d, device=DEV)
+    val = torch.empty(0, device=DEV)
+    mods["spfa_csr"].forward(q.view(-1, d), k.view(-1, d), v.view(-1, d), ro_t, ci_t, val, m.view(-1), l.view(-1),
+                             o.view(-1, d), False)
+    sync()
+    for h in range(heads):
+        check(o[h], m[h], l[h], *so.dense_masked_attention(np64(q[h]), np64(k[h]), np64(v[h]), dense[h]),
+              torch.float32)
+
+
 # ------------------------------------------------------------------ window + global + CSR in one call
 @pytest.mark.parametrize("dtype,d", [(torch.float32, 64), (torch.bfloat16, 64), (torch.float16, 128),
                                       (torch.float32, 40)])
