@@ -11,7 +11,8 @@
 // Everything is computed transposed, as in the forward tiles (streamed index on the rows of a
 // 32x32 result, owner on the columns):
 //     S^T = X A^T,  dP^T = Y B^T            (X, Y the streamed tiles; A, B the owner's vectors)
-//     P^T = exp2(S^T sc - lse),  dS^T = P^T (dP^T - delta) / sqrt(d)
+//     P^T = exp2(S^T sc - lse),  dS^T = P^T (dP^T - delta)      (the 1/sqrt(d) of dS is applied once,
+//                                                               to G1, at the end)
 //     G1^T += X^T dS^T,  G2^T += Y^T P^T    (G2 in the key pass only)
 // The streamed tiles are row-major in LDS and serve as both operands: by rows for the first two
 // products, transposed (8-byte transposing reads for the half types, scalar reads for fp32) for
@@ -285,9 +286,16 @@ __global__ __launch_bounds__(256, (grad_tile_min_blocks<T, D, KEYS>())) void til
 
     const uint32_t w32 = (uint32_t)a.w, w2 = 2u * (uint32_t)a.w;
     const int rem = (int)((u_hi - ut) < BN ? (u_hi - ut) : BN);
+    (void)rem;
     // a streamed row is live iff (unsigned)(delta + w) <= 2w (band; delta in positions) or > 2w
     // (global; delta in tokens)
-    uint32_t d0;
+    // band: the end of the subsequence is folded into the same comparison (a streamed position u
+    // is past the end iff u - tq + w > u_hi - 1 - tq + w, which is not negative for a valid owner)
+    uint32_t d0, band_hi = w2;
+    if constexpr (MODE == kTileBand) {
+      const uint32_t end_hi = (uint32_t)(int32_t)(u_hi - 1 - tq) + w32;
+      band_hi = own_ok && end_hi < w2 ? end_hi : w2;
+    }
     if constexpr (MODE == kTileBand) d0 = (uint32_t)(int32_t)(ut - tq) + w32;
     else if constexpr (MODE == kTileGlobalRows) d0 = (uint32_t)(int32_t)(ut - own_tok) + w32;
     else d0 = w32 - (uint32_t)(int32_t)own_tok;
@@ -299,7 +307,13 @@ __global__ __launch_bounds__(256, (grad_tile_min_blocks<T, D, KEYS>())) void til
       if constexpr (MODE == kTileBand) need = need && (ub <= tw0 + 31 + a.w) && (ub + 31 + a.w >= tw0);
       if (!need) continue;
       const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-      f32x16 s = zero16, dp = zero16;
+      // the dO.V product starts at -delta, so that it comes out as (dP - delta)
+      f32x16 s = zero16, dp;
+#pragma unroll
+      for (int v = 0; v < 16; v++) {
+        if constexpr (KEYS) dp[v] = -delta_s[32 * jb + 8 * (v / 4) + 4 * h + (v % 4)];
+        else dp[v] = -delta_o;
+      }
       if constexpr (kF32) {
         const float* xrow = (const float*)Xs + (32 * jb + r) * ST + h;
         const float* yrow = (const float*)Ys + (32 * jb + r) * ST + h;
@@ -328,22 +342,19 @@ __global__ __launch_bounds__(256, (grad_tile_min_blocks<T, D, KEYS>())) void til
 #pragma unroll
       for (int v = 0; v < 16; v++) {
         const int j = 32 * jb + 8 * (v / 4) + 4 * h + (v % 4);
-        float ls = lse_o, dl = delta_o;
-        if constexpr (KEYS) {
-          ls = lse_s[j];
-          dl = delta_s[j];
-        }
+        float ls = lse_o;
+        if constexpr (KEYS) ls = lse_s[j];
         float p = __builtin_amdgcn_exp2f(__builtin_fmaf(s[v], sc, -ls));
         if constexpr (MODE == kTileGlobalRows && KEYS) p *= (once_s[j] != 0.f) ? 1.f : mult_o;
         if (!full) {
           bool ok;
-          if constexpr (MODE == kTileBand) ok = (d0 + (uint32_t)j <= w2);
-          else if constexpr (MODE == kTileGlobalRows) ok = (d0 + (uint32_t)j > w2);
-          else ok = (d0 + (uint32_t)ktok_s[j] > w2);
-          p = (ok && j < rem) ? p : 0.f;
+          if constexpr (MODE == kTileBand) ok = (d0 + (uint32_t)j <= band_hi);
+          else if constexpr (MODE == kTileGlobalRows) ok = (d0 + (uint32_t)j > w2) && (j < rem);
+          else ok = (d0 + (uint32_t)ktok_s[j] > w2) && (j < rem);
+          p = ok ? p : 0.f;
         }
         s[v] = p;
-        dp[v] = p * (dp[v] - dl) * scale;
+        dp[v] *= p;  // dS without its 1/sqrt(d), which the write-out applies
       }
       // ---- G1^T += X^T dS^T,  G2^T += Y^T P^T
       if constexpr (kF32) {
@@ -404,7 +415,8 @@ __global__ __launch_bounds__(256, (grad_tile_min_blocks<T, D, KEYS>())) void til
         // partial sums of this split (and half): [problem][split][half][which][listed token][D]
         const int64_t slot0 = ((part_bb * a.n_split + part_split) * 2 + (wave_k > 0 ? 1 : 0)) * (KEYS ? 2 : 1);
         float* p1 = a.pacc + (slot0 * a.n_globs + tq) * D + e;
-        const float4v x = {g1[eb][4 * g4], g1[eb][4 * g4 + 1], g1[eb][4 * g4 + 2], g1[eb][4 * g4 + 3]};
+        const float4v x = {g1[eb][4 * g4] * scale, g1[eb][4 * g4 + 1] * scale, g1[eb][4 * g4 + 2] * scale,
+                           g1[eb][4 * g4 + 3] * scale};
         *reinterpret_cast<float4v*>(p1) = x;
         if constexpr (KEYS) {
           const float4v y = {g2[eb][4 * g4], g2[eb][4 * g4 + 1], g2[eb][4 * g4 + 2], g2[eb][4 * g4 + 3]};
@@ -413,7 +425,7 @@ __global__ __launch_bounds__(256, (grad_tile_min_blocks<T, D, KEYS>())) void til
       } else {
         float4v x = *reinterpret_cast<const float4v*>(out1 + e);
 #pragma unroll
-        for (int i = 0; i < 4; i++) x[i] += g1[eb][4 * g4 + i];
+        for (int i = 0; i < 4; i++) x[i] += g1[eb][4 * g4 + i] * scale;
         *reinterpret_cast<float4v*>(out1 + e) = x;
         if constexpr (KEYS) {
           float4v y = *reinterpret_cast<const float4v*>(out2 + e);
