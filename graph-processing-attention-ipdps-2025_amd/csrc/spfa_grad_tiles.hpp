@@ -56,6 +56,7 @@ struct GradTileCfg {
 // against 512 us for the combined one - no gain for 25 % more products.)
 template <typename T, int D, bool KEYS>
 constexpr int grad_tile_min_blocks() {
+  if (D <= 64 && sizeof(T) == 2 && !KEYS) return 3;
   return (D > 64 && (KEYS || sizeof(T) == 4)) ? 1 : 2;
 }
 
