@@ -42,9 +42,9 @@ struct GradTileCfg {
   static constexpr int BM = 128;
   static constexpr int BN = (kF32 && D > 64) ? 32 : 64;  // streamed positions per tile
   static constexpr int NB = BN / 32;
-  // row stride in elements: fp32 rows land on distinct banks for the by-row reads (2r + h),
-  // half rows are 16-byte aligned and 4 banks apart
-  static constexpr int STRIDE = kF32 ? D + 2 : D + 8;
+  // row stride in elements: rows are 16-byte aligned and 4 banks apart (a 16-byte read by 16
+  // consecutive rows then covers every bank once)
+  static constexpr int STRIDE = kF32 ? D + 4 : D + 8;
   static constexpr int TILE = BN * STRIDE;
   static constexpr int EB = D / 32;
   static constexpr int AREGS = kF32 ? D / 2 : D / 16;
@@ -171,14 +171,18 @@ __global__ __launch_bounds__(256, (grad_tile_min_blocks<T, D, KEYS>())) void til
     const T* arow = Ap + own_row * D;
     const T* brow = Bp + own_row * D;
     if constexpr (kF32) {
+      // the 32x32x2 product takes two k per instruction, one per half of the wavefront: half h
+      // takes k = h * D/2 + ks in step ks (any pairing works as long as both operands use it),
+      // so that a lane's operands are consecutive in memory and in LDS
 #pragma unroll
-      for (int c4 = 0; c4 < D / 4; c4++) {
-        const float4v x = *reinterpret_cast<const float4v*>(arow + 4 * c4);
-        const float4v y = *reinterpret_cast<const float4v*>(brow + 4 * c4);
-        af[2 * c4] = h ? x[1] : x[0];
-        af[2 * c4 + 1] = h ? x[3] : x[2];
-        bf[2 * c4] = h ? y[1] : y[0];
-        bf[2 * c4 + 1] = h ? y[3] : y[2];
+      for (int c4 = 0; c4 < D / 8; c4++) {
+        const float4v x = *reinterpret_cast<const float4v*>(arow + h * (D / 2) + 4 * c4);
+        const float4v y = *reinterpret_cast<const float4v*>(brow + h * (D / 2) + 4 * c4);
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+          af[4 * c4 + i] = x[i];
+          bf[4 * c4 + i] = y[i];
+        }
       }
     } else {
 #pragma unroll
@@ -250,13 +254,8 @@ __global__ __launch_bounds__(256, (grad_tile_min_blocks<T, D, KEYS>())) void til
       const int idx = it * 256 + tid;
       const int j = idx / CH, c = idx % CH;
       if constexpr (kF32) {
-        // rows are only 8-byte aligned
-        const float4v xx = __builtin_bit_cast(float4v, xreg[it]);
-        const float4v yy = __builtin_bit_cast(float4v, yreg[it]);
-        float* xd = (float*)Xs + j * ST + 4 * c;
-        float* yd = (float*)Ys + j * ST + 4 * c;
-        xd[0] = xx[0]; xd[1] = xx[1]; xd[2] = xx[2]; xd[3] = xx[3];
-        yd[0] = yy[0]; yd[1] = yy[1]; yd[2] = yy[2]; yd[3] = yy[3];
+        *reinterpret_cast<uint4v*>((float*)Xs + j * ST + 4 * c) = xreg[it];
+        *reinterpret_cast<uint4v*>((float*)Ys + j * ST + 4 * c) = yreg[it];
       } else {
         *reinterpret_cast<uint4v*>(Xs + j * ST + 8 * c) = xreg[it];
         *reinterpret_cast<uint4v*>(Ys + j * ST + 8 * c) = yreg[it];
@@ -316,12 +315,17 @@ __global__ __launch_bounds__(256, (grad_tile_min_blocks<T, D, KEYS>())) void til
         else dp[v] = -delta_o;
       }
       if constexpr (kF32) {
-        const float* xrow = (const float*)Xs + (32 * jb + r) * ST + h;
-        const float* yrow = (const float*)Ys + (32 * jb + r) * ST + h;
+        const float* xrow = (const float*)Xs + (32 * jb + r) * ST + h * (D / 2);
+        const float* yrow = (const float*)Ys + (32 * jb + r) * ST + h * (D / 2);
 #pragma unroll
-        for (int ks = 0; ks < D / 2; ks++) {
-          s = __builtin_amdgcn_mfma_f32_32x32x2f32(xrow[2 * ks], af[ks], s, 0, 0, 0);
-          dp = __builtin_amdgcn_mfma_f32_32x32x2f32(yrow[2 * ks], bf[ks], dp, 0, 0, 0);
+        for (int k4 = 0; k4 < D / 8; k4++) {
+          const float4v xa = *reinterpret_cast<const float4v*>(xrow + 4 * k4);
+          const float4v ya = *reinterpret_cast<const float4v*>(yrow + 4 * k4);
+#pragma unroll
+          for (int i = 0; i < 4; i++) {
+            s = __builtin_amdgcn_mfma_f32_32x32x2f32(xa[i], af[4 * k4 + i], s, 0, 0, 0);
+            dp = __builtin_amdgcn_mfma_f32_32x32x2f32(ya[i], bf[4 * k4 + i], dp, 0, 0, 0);
+          }
         }
       } else {
         const T* xrow = Xs + (32 * jb + r) * ST + 8 * h;
