@@ -184,8 +184,11 @@ __global__ void mark_globals_kernel(const int32_t* globs, int64_t n_globs, int64
 }
 
 // ---- two-pass partition of unsorted COO entries by row -----------------------------------
-constexpr int kPartThreads = 256;
-constexpr int kPartTile = 8192;      // entries per workgroup in pass 1
+// Pass 1 stages a whole tile in LDS (152 KB with the bucket tables: one workgroup per CU), so the
+// workgroup is as large as it can be: 1024 threads and 16384 entries measured 0.35 ms for 50 M
+// entries against 0.78 ms with 256 threads and 8192 entries (and longer runs per bucket).
+constexpr int kPartThreads = 1024;
+constexpr int kPartTile = 16384;     // entries per workgroup in pass 1
 constexpr int kPartMaxBuckets = 2048;
 
 // pass 1a: per-tile histogram of the high digit, stored bucket-major: hist[b * n_tiles + tile]
@@ -422,7 +425,7 @@ int coo_to_csr(const void* row_ind, int row_wide, const uint32_t* col_ind, int64
   if (nnz > 0 && w.partition) {
     uint32_t* hist = (uint32_t*)(base + w.off_hist);
     uint64_t* tmp_pairs = (uint64_t*)(base + w.off_tmp_pairs);
-    // 88 KB of LDS per workgroup: above the 64 KB a kernel gets without asking (set once per
+    // 152 KB of LDS per workgroup: above the 64 KB a kernel gets without asking (set once per
     // device: the attribute belongs to the device's copy of the kernel)
     constexpr int kMaxDevices = 64;
     static bool lds_attr_set[kMaxDevices];
