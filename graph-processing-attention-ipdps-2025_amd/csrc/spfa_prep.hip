@@ -299,8 +299,19 @@ __global__ __launch_bounds__(kPartRowsThreads) void coo_part_rows_kernel(
   for (int i = threadIdx.x; i < n_lo; i += kPartRowsThreads) cnt[i] = 0;
   __syncthreads();
   const uint32_t lo_mask = (uint32_t)n_lo - 1u;
-  for (uint32_t e = beg + threadIdx.x; e < end; e += kPartRowsThreads)
-    atomicAdd(&cnt[(uint32_t)(tmp_pairs[e] >> 32) & lo_mask], 1u);
+  // (four loads in flight per thread: the loop is bound by their latency)
+  constexpr uint32_t kStep = 4 * kPartRowsThreads;
+  for (uint32_t e0 = beg; e0 < end; e0 += kStep) {
+    uint64_t x[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      const uint32_t e = e0 + i * kPartRowsThreads + threadIdx.x;
+      x[i] = e < end ? tmp_pairs[e] : ~0ull;
+    }
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+      if (x[i] != ~0ull) atomicAdd(&cnt[(uint32_t)(x[i] >> 32) & lo_mask], 1u);
+  }
   __syncthreads();
   // exclusive scan of cnt[0 .. n_lo) in place, kPartRowsThreads values at a time
   const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
@@ -328,10 +339,20 @@ __global__ __launch_bounds__(kPartRowsThreads) void coo_part_rows_kernel(
     __syncthreads();
   }
   if (b == n_hi - 1 && threadIdx.x == 0) row_off[n_rows] = end;
-  for (uint32_t e = beg + threadIdx.x; e < end; e += kPartRowsThreads) {
-    const uint64_t x = tmp_pairs[e];
-    const uint32_t pos = atomicAdd(&cnt[(uint32_t)(x >> 32) & lo_mask], 1u);
-    cols_out[pos] = (uint32_t)x;
+  for (uint32_t e0 = beg; e0 < end; e0 += kStep) {
+    uint64_t x[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      const uint32_t e = e0 + i * kPartRowsThreads + threadIdx.x;
+      x[i] = e < end ? tmp_pairs[e] : ~0ull;
+    }
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      if (x[i] != ~0ull) {
+        const uint32_t pos = atomicAdd(&cnt[(uint32_t)(x[i] >> 32) & lo_mask], 1u);
+        cols_out[pos] = (uint32_t)x[i];
+      }
+    }
   }
 }
 
