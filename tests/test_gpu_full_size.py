@@ -295,3 +295,36 @@ def test_backward_global_no_local_n1m(mods):
     gl = globs.cpu().tolist()
     rows = np.concatenate([np.asarray(gl[:3]), rand_rows(n, 40, 11)])
     _dq_sample_check(q, k, v, d_out, dq, rows, lambda i: so.live_global_no_local(n, gl, w, i), torch.float32)
+
+
+def test_backward_coo_zipf_n1m_50m_entries(mods):
+    """Unsorted COO at the bench size: two bucketing pre-passes (by row, by column); columns are
+    uniform, rows are not, so the heaviest rows leave segment items behind."""
+    n, d = 1 << 20, 64
+    q, k, v = syn.qkv(n, d, device=DEV, seed=0)
+    r, c = syn.zipf_coo(n, 50_000_000, 1.3, device=DEV, seed=0)
+    r_t, c_t = r.to(torch.uint64), c.to(torch.uint32)
+    val = torch.empty(0, device=DEV)
+    m, l, o = syn.fresh_state(n, d, device=DEV)
+    mods["spfa_coo"].forward(q, k, v, r_t, c_t, val, m, l, o, False)
+    d_out = torch.randn(n, d, device=DEV, generator=torch.Generator(device=DEV).manual_seed(12))
+    dq, dk, dv = (torch.zeros(n, d, device=DEV) for _ in range(3))
+    mods["spfa_coo"].backward(q, k, v, r_t, c_t, val, m, l, o, d_out, dq, dk, dv)
+    torch.cuda.synchronize()
+    _grad_properties(q, k, v, d_out, l, dq, dk, dv, torch.float32)
+    deg = torch.bincount(r, minlength=n)
+    heavy = torch.topk(deg, 3)[1].cpu().numpy()
+    empty = torch.nonzero(deg == 0)[:3, 0].cpu().numpy()
+    rows = np.unique(np.concatenate([heavy, empty, rand_rows(n, 30, 13)]))
+    _dq_sample_check(q, k, v, d_out, dq, rows, lambda i: c[r == i].cpu().numpy(), torch.float32)
+    assert not dq[torch.as_tensor(empty).to(DEV)].any()
+    # key side on a few columns, weighted with the forward pass's own statistics
+    lse = m.double() + l.double().log()
+    delta = (d_out.double() * o.double()).sum(dim=1)
+    for j in rand_rows(n, 6, 14):
+        att = r[c == int(j)]
+        s = (q[att].double() @ k[j].double()) / math.sqrt(d)
+        p = torch.exp(s - lse[att])
+        ds = p * (d_out[att].double() @ v[j].double() - delta[att]) / math.sqrt(d)
+        assert float((dv[j].double() - p @ d_out[att].double()).abs().max()) <= 2e-4
+        assert float((dk[j].double() - ds @ q[att].double()).abs().max()) <= 2e-4
