@@ -950,6 +950,28 @@ int spfa_csr_transpose(int64_t n_q, int64_t n_k, const void* row_off, int row_of
   return coo_csr_export(tr, e_rows, n_k, nnz, t_row_off, t_col_ind, (hipStream_t)stream);
 }
 
+size_t spfa_coo_to_csr_workspace_bytes(int64_t n_rows, int64_t nnz) {
+  if (n_rows < 0 || nnz < 0) return 0;
+  return coo_workspace(n_rows, nnz).total;
+}
+
+int spfa_coo_to_csr(int64_t n_rows, const void* row_ind, int row_ind_bytes, const void* col_ind, int64_t nnz,
+                    uint32_t* row_off, uint32_t* csr_col_ind, void* workspace, size_t workspace_bytes,
+                    void* stream) {
+  if (n_rows < 0 || n_rows >= (int64_t)1 << 31 || nnz < 0 || nnz >= (int64_t)1 << 31 ||
+      (row_ind_bytes != 4 && row_ind_bytes != 8))
+    return SPFA_ERR_BAD_ARG;
+  if (!row_off || (nnz > 0 && (!row_ind || !col_ind || !csr_col_ind))) return SPFA_ERR_BAD_ARG;
+  const CooWorkspace cw = coo_workspace(n_rows, nnz);
+  int rc = check_workspace(workspace, workspace_bytes, cw.total);
+  if (rc) return rc;
+  CooCsr csr{};
+  rc = coo_to_csr(row_ind, row_ind_bytes == 8 ? 1 : 0, (const uint32_t*)col_ind, nnz, n_rows, workspace,
+                  (char*)workspace + cw.keep_total, (hipStream_t)stream, &csr);
+  if (rc) return rc;
+  return coo_csr_export(csr, (const uint32_t*)col_ind, n_rows, nnz, row_off, csr_col_ind, (hipStream_t)stream);
+}
+
 size_t spfa_coo_backward_workspace_bytes(int64_t n_q, int64_t n_k, int64_t nnz, int64_t d, int dtype,
                                          int64_t n_batch) {
   (void)d;

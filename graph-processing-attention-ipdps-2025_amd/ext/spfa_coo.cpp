@@ -127,10 +127,35 @@ std::tuple<torch::Tensor, torch::Tensor, torch::Tensor> spfa_coo_backward_py(tor
   return std::make_tuple(dQ, dK, dV);
 }
 
+// to_csr(w_row_ind, w_col_ind, n_rows) -> (row_off, col_ind), uint32: the entries as a CSR mask (columns
+// of a row in no particular order), for the spfa_csr entry points (plans, transpose, backward).
+std::tuple<torch::Tensor, torch::Tensor> spfa_coo_to_csr_py(torch::Tensor W_row_ind, torch::Tensor W_col_ind,
+                                                            int64_t n_rows) {
+  CHECK_INPUT(W_row_ind);
+  CHECK_INPUT(W_col_ind);
+  c10::DeviceGuard guard(W_row_ind.device());
+  TORCH_CHECK(W_row_ind.dim() == 1 && W_col_ind.dim() == 1 && W_row_ind.size(0) == W_col_ind.size(0),
+              "W_row_ind and W_col_ind must be 1-D and of equal length");
+  TORCH_CHECK(n_rows >= 0, "n_rows must not be negative");
+  const int row_bytes = spfa_ext::index_bytes(W_row_ind, "W_row_ind", true);
+  spfa_ext::index_bytes(W_col_ind, "W_col_ind", false);
+  const int64_t nnz = W_col_ind.size(0);
+  auto opt = torch::TensorOptions().dtype(torch::kUInt32).device(W_row_ind.device());
+  torch::Tensor row_off = torch::empty({n_rows + 1}, opt);
+  torch::Tensor cols = torch::empty({nnz}, opt);
+  torch::Tensor ws = spfa_ext::make_workspace(spfa_coo_to_csr_workspace_bytes(n_rows, nnz), W_row_ind);
+  spfa_ext::raise_on_error(spfa_coo_to_csr(n_rows, W_row_ind.data_ptr(), row_bytes, W_col_ind.data_ptr(), nnz,
+                                           (uint32_t*)row_off.data_ptr(), (uint32_t*)cols.data_ptr(),
+                                           ws.data_ptr(), (size_t)ws.numel(),
+                                           spfa_ext::current_stream(W_row_ind)));
+  return std::make_tuple(row_off, cols);
+}
+
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, mod) {
   mod.def("forward", &spfa_coo_forward_py, "Sparse-FlashAttention forward, COO mask (HIP, gfx950)");
   mod.def("plan", &spfa_coo_plan_py, "Mask pre-pass of a COO mask, for forward_planned");
   mod.def("forward_planned", &spfa_coo_forward_planned_py,
           "forward(...) with the mask pre-pass taken from plan(...)");
   mod.def("backward", &spfa_coo_backward_py, "Gradients of forward(...), added to dQ, dK, dV");
+  mod.def("to_csr", &spfa_coo_to_csr_py, "The COO entries as a CSR mask (uint32 offsets and columns)");
 }

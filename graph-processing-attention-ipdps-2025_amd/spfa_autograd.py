@@ -85,6 +85,13 @@ def csr_part(w_row_off, w_col_ind, n_cols):
     return ("csr", w_row_off, w_col_ind, t_row_off, t_col_ind)
 
 
+def coo_part(w_row_ind, w_col_ind, n_rows, n_cols):
+    """COO entries (any order) as a "csr" part with the mask by column attached: converted and
+    transposed once, so that no forward or backward pass buckets the entries again."""
+    row_off, col_ind = importlib.import_module("spfa_coo").to_csr(w_row_ind, w_col_ind, n_rows)
+    return csr_part(row_off, col_ind, n_cols)
+
+
 def attention(q, k, v, parts, return_state=False):
     """Masked attention over the union of `parts` (see the module text), differentiable in q, k, v.
 

@@ -235,6 +235,15 @@ size_t spfa_csr_transpose_workspace_bytes(int64_t n_q, int64_t n_k, int64_t nnz)
 int spfa_csr_transpose(int64_t n_q, int64_t n_k, const void* row_off, int row_off_bytes,
                        const void* col_ind, int64_t nnz, uint32_t* t_row_off, uint32_t* t_col_ind,
                        void* workspace, size_t workspace_bytes, void* stream);
+/* COO entries in any order as a CSR mask: row_off (n_rows + 1 entries) and csr_col_ind (nnz; the
+ * columns of a row in no particular order), both uint32 - the conversion every spfa_coo_* call does
+ * internally (Sparse_FlashAttention_COO/sp_flatt_coo_kernel.cu:47-84 locates a row's range by a
+ * scan instead), for callers that keep a mask for many calls and want the CSR entry points, their
+ * plans and spfa_csr_transpose. */
+size_t spfa_coo_to_csr_workspace_bytes(int64_t n_rows, int64_t nnz);
+int spfa_coo_to_csr(int64_t n_rows, const void* row_ind, int row_ind_bytes, const void* col_ind, int64_t nnz,
+                    uint32_t* row_off, uint32_t* csr_col_ind, void* workspace, size_t workspace_bytes,
+                    void* stream);
 size_t spfa_coo_backward_workspace_bytes(int64_t n_q, int64_t n_k, int64_t nnz, int64_t d, int dtype,
                                          int64_t n_batch);
 int spfa_coo_backward(const spfa_problem_t* p, const spfa_grads_t* g, const void* row_ind,

@@ -375,3 +375,28 @@ def test_statistics_stored_in_the_element_type(mods, dtype):
         for nm, a, b in zip(("dq", "dk", "dv"), (dq, dk, dv), ref):
             err = float(np.abs(np64(a) - b).max())
             assert err <= 0.15 * max(1.0, float(np.abs(b).max())), "%s %s: %.3e" % (name, nm, err)
+
+
+def test_coo_entries_converted_once(mods):
+    """spfa_coo.to_csr against a CPU conversion (exact offsets, every row's columns as a set, both
+    row index widths, sorted and shuffled entries), and spfa_autograd.coo_part == the coo part."""
+    n, n_k, d = 300, 410, 64
+    rng = np.random.default_rng(151)
+    dense = rng.random((n, n_k)) < 0.06
+    dense[17] = False
+    r, c = so.coo_from_dense(dense)
+    ro_ref, ci_ref = so.csr_from_dense(dense)
+    for perm, rdt in ((np.arange(len(r)), torch.uint64), (rng.permutation(len(r)), torch.int32)):
+        r_t = torch.as_tensor(r[perm]).to(rdt).to(DEV)
+        c_t = torch.as_tensor(c[perm]).to(torch.uint32).to(DEV)
+        ro, ci = mods["spfa_coo"].to_csr(r_t, c_t, n)
+        torch.cuda.synchronize()
+        ro, ci = ro.cpu().numpy().astype(np.int64), ci.cpu().numpy().astype(np.int64)
+        assert np.array_equal(ro, ro_ref)
+        for i in range(n):
+            assert np.array_equal(np.sort(ci[ro[i]:ro[i + 1]]), ci_ref[ro_ref[i]:ro_ref[i + 1]]), i
+    q, k, v, d_out = _problem(n, d, torch.float32, 152, n_k)
+    ref = so.dense_masked_attention_backward(np64(q), np64(k), np64(v), dense, np64(d_out))
+    out, got = _grads_of(q, k, v, d_out, [spfa_autograd.coo_part(r_t, c_t, n, n_k)])
+    _check_grads(got, ref, torch.float32, "coo_part")
+    assert np.abs(np64(out) - np.nan_to_num(so.dense_masked_attention(np64(q), np64(k), np64(v), dense)[0])).max() <= 1e-4
