@@ -15,8 +15,10 @@
 //                                                               to G1, at the end)
 //     G1^T += X^T dS^T,  G2^T += Y^T P^T    (G2 in the key pass only)
 // The streamed tiles are row-major in LDS and serve as both operands: by rows for the first two
-// products, transposed (8-byte transposing reads for the half types, scalar reads for fp32) for
-// the last two.  No atomics: an owner row belongs to one wavefront.
+// products, transposed for the last two: 8-byte transposing reads for the half types; for fp32
+// row i of result block eb stands for element (D/32) * i + eb of the gradient row, so that the
+// D/32 values a lane feeds to the blocks for one streamed row are adjacent in LDS (one 8- or
+// 16-byte read for D/32 instructions).  No atomics: an owner row belongs to one wavefront.
 //
 // The global-minus-local mask is two more tile problems of the same kind (the window test
 // |i - j| > w is symmetric as well):
@@ -377,17 +379,26 @@ __global__ __launch_bounds__(256, (grad_tile_min_blocks<T, D, KEYS>())) void til
       }
       // ---- G1^T += X^T dS^T,  G2^T += Y^T P^T
       if constexpr (kF32) {
+        typedef float vecE __attribute__((ext_vector_type(EB)));
+        const float* xbase = (const float*)Xs + (32 * jb + 4 * h) * ST + EB * r;
+        const float* ybase = (const float*)Ys + (32 * jb + 4 * h) * ST + EB * r;
+        vecE xv = *reinterpret_cast<const vecE*>(xbase), yv = xv;
+        if constexpr (KEYS) yv = *reinterpret_cast<const vecE*>(ybase);
 #pragma unroll
         for (int v = 0; v < 16; v++) {
-          const int j = 32 * jb + 8 * (v / 4) + 4 * h + (v % 4);
-          const float* xcol = (const float*)Xs + j * ST + r;
-          const float* ycol = (const float*)Ys + j * ST + r;
+          vecE xn = xv, yn = yv;
+          if (v + 1 < 16) {
+            const int jn = (8 * ((v + 1) / 4) + ((v + 1) % 4)) * ST;
+            xn = *reinterpret_cast<const vecE*>(xbase + jn);
+            if constexpr (KEYS) yn = *reinterpret_cast<const vecE*>(ybase + jn);
+          }
 #pragma unroll
           for (int eb = 0; eb < EB; eb++) {
-            g1[eb] = __builtin_amdgcn_mfma_f32_32x32x2f32(xcol[32 * eb], dp[v], g1[eb], 0, 0, 0);
-            if constexpr (KEYS)
-              g2[eb] = __builtin_amdgcn_mfma_f32_32x32x2f32(ycol[32 * eb], s[v], g2[eb], 0, 0, 0);
+            g1[eb] = __builtin_amdgcn_mfma_f32_32x32x2f32(xv[eb], dp[v], g1[eb], 0, 0, 0);
+            if constexpr (KEYS) g2[eb] = __builtin_amdgcn_mfma_f32_32x32x2f32(yv[eb], s[v], g2[eb], 0, 0, 0);
           }
+          xv = xn;
+          yv = yn;
         }
       } else {
         typedef short s16x4 __attribute__((ext_vector_type(4)));
@@ -421,36 +432,41 @@ __global__ __launch_bounds__(256, (grad_tile_min_blocks<T, D, KEYS>())) void til
     }
   }
 
-  // ---- add into the owner's gradient rows (element 32*eb + 8*(v/4) + 4*h + v%4 in g[eb][v])
+  // ---- add into the owner's gradient rows.  g[eb][v] is element 32*eb + i of the row for the half
+  // types and (D/32)*i + eb for fp32, i = 8*(v/4) + 4*h + v%4: four registers of one block, or of
+  // all blocks, are four adjacent elements
   if (!own_ok) return;
   float* out1 = (KEYS ? g.d_k : g.d_q) + own_row * D;
   float* out2 = KEYS ? g.d_v + own_row * D : nullptr;
 #pragma unroll
-  for (int eb = 0; eb < EB; eb++)
+  for (int oc = 0; oc < EB; oc++)
 #pragma unroll
     for (int g4 = 0; g4 < 4; g4++) {
-      const int e = 32 * eb + 8 * g4 + 4 * h;
+      const int e = kF32 ? EB * (8 * g4 + 4 * h) + 4 * oc : 32 * oc + 8 * g4 + 4 * h;
+      float4v x, y = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int u = 0; u < 4; u++) {
+        const int eb = kF32 ? (4 * oc + u) % EB : oc;
+        const int v = kF32 ? 4 * g4 + (4 * oc + u) / EB : 4 * g4 + u;
+        x[u] = g1[eb][v] * scale;
+        if constexpr (KEYS) y[u] = g2[eb][v];
+      }
       if constexpr (MODE == kTileGlobalRows) {
         // partial sums of this split (and half): [problem][split][half][which][listed token][D]
         const int64_t slot0 = ((part_bb * a.n_split + part_split) * 2 + (wave_k > 0 ? 1 : 0)) * (KEYS ? 2 : 1);
         float* p1 = a.pacc + (slot0 * a.n_globs + tq) * D + e;
-        const float4v x = {g1[eb][4 * g4] * scale, g1[eb][4 * g4 + 1] * scale, g1[eb][4 * g4 + 2] * scale,
-                           g1[eb][4 * g4 + 3] * scale};
         *reinterpret_cast<float4v*>(p1) = x;
-        if constexpr (KEYS) {
-          const float4v y = {g2[eb][4 * g4], g2[eb][4 * g4 + 1], g2[eb][4 * g4 + 2], g2[eb][4 * g4 + 3]};
-          *reinterpret_cast<float4v*>(p1 + a.n_globs * D) = y;
-        }
+        if constexpr (KEYS) *reinterpret_cast<float4v*>(p1 + a.n_globs * D) = y;
       } else {
-        float4v x = *reinterpret_cast<const float4v*>(out1 + e);
+        float4v x0 = *reinterpret_cast<const float4v*>(out1 + e);
 #pragma unroll
-        for (int i = 0; i < 4; i++) x[i] += g1[eb][4 * g4 + i] * scale;
-        *reinterpret_cast<float4v*>(out1 + e) = x;
+        for (int u = 0; u < 4; u++) x0[u] += x[u];
+        *reinterpret_cast<float4v*>(out1 + e) = x0;
         if constexpr (KEYS) {
-          float4v y = *reinterpret_cast<const float4v*>(out2 + e);
+          float4v y0 = *reinterpret_cast<const float4v*>(out2 + e);
 #pragma unroll
-          for (int i = 0; i < 4; i++) y[i] += g2[eb][4 * g4 + i];
-          *reinterpret_cast<float4v*>(out2 + e) = y;
+          for (int u = 0; u < 4; u++) y0[u] += y[u];
+          *reinterpret_cast<float4v*>(out2 + e) = y0;
         }
       }
     }

@@ -20,6 +20,17 @@
 //     that product is the key, and any key order works as long as V^T uses the same one).
 // Half types use v_mfma_f32_32x32x16 (8 consecutive k per lane), fp32 uses v_mfma_f32_32x32x2
 // (no down-cast of fp32 inputs).
+//
+// fp32 operands come out of LDS 16 bytes at a time, one read for four (K) or D/32 (V) matrix
+// instructions, which takes two free choices of index order:
+//   - first product: the instruction sums over two k, one per half of the wavefront.  Half h
+//     takes k = 8g + 4h + i in instruction 4g + i, so its four values of a group g are adjacent
+//     in the K row (and in the Q row, which is loaded into registers the same way);
+//   - second product: row i of result block eb is element e = (D/32) * i + eb of the output
+//     row, so the D/32 values a lane feeds to the blocks for one key are adjacent in the V row.
+//     tile_write_row and the partial results of the global rows undo that order when they write.
+// (With one 4-byte read per instruction the compiler, short of registers, ran read - wait - two
+// instructions in strict sequence and the matrix pipe idled through every LDS round trip.)
 #pragma once
 
 #include "spfa_engine.hpp"
@@ -46,6 +57,9 @@ struct TileArgs {
   int64_t cnt;            // block mode: live positions per block
   int64_t tiles_per_sub;  // query tiles per subsequence (of the longest subsequence)
   int64_t n_tiles;
+  int64_t n_tail;         // band: the last n_tail tiles (over all problems) are each shared by four
+                          // workgroups of 32 queries whose wavefronts deal the key blocks among
+                          // themselves; they fill the last, partly empty round of the grid
   // global modes
   const int32_t* globs;   // listed global tokens (keys of GlobalCols)
   int64_t n_globs;
@@ -74,7 +88,7 @@ struct TileCfg {
   // K tile: [key][k] rows padded so that the 32 keys read by one operand fetch spread over the
   // banks.  V tile: half types are stored transposed [e][key'] (16-byte operand reads), fp32
   // row-major [key][e].
-  static constexpr int K_STRIDE = kF32 ? D + 2 : D + 8;
+  static constexpr int K_STRIDE = kF32 ? D + 4 : D + 8;
   static constexpr int V_STRIDE = kF32 ? D + 8 : BN + 8;
   static constexpr int K_ELEMS = BN * K_STRIDE;
   static constexpr int V_ELEMS = kF32 ? BN * V_STRIDE : D * V_STRIDE;
@@ -112,8 +126,8 @@ struct BoolConst {
 };
 
 // Fold the incoming state of row `row` into a finished tile result and write the row back.
-// o holds O^T in the 32x32 result layout (element e = 32*eb + 8*(v/4) + 4*h + v%4 of the row in
-// o[eb][v]); m is the running max in log2 units, l the row sum (already summed over both halves
+// o holds O^T in the 32x32 result layout: o[eb][v] is element e = 32*eb + i of the row for the
+// half types and e = (D/32)*i + eb for fp32, i = 8*(v/4) + 4*h + v%4; m is the running max in log2 units, l the row sum (already summed over both halves
 // of the wavefront); o * o_scale is the accumulator that goes with (m, l).
 template <typename T, int D>
 __device__ __forceinline__ void tile_write_row(const Tensors& t, int64_t row, int h, float m, float l,
@@ -136,18 +150,20 @@ __device__ __forceinline__ void tile_write_row(const Tensors& t, int64_t row, in
   wa *= inv;
   T* orow = (T*)t.out + row * D;
   if constexpr (kF32) {
+    // registers 4*g4 .. 4*g4+3 of all blocks: 4*EB consecutive elements from EB * (8*g4 + 4*h)
+    constexpr int EB = D / 32;
 #pragma unroll
-    for (int eb = 0; eb < D / 32; eb++) {
+    for (int g4 = 0; g4 < 4; g4++) {
 #pragma unroll
-      for (int g4 = 0; g4 < 4; g4++) {
-        const int e = 32 * eb + 8 * g4 + 4 * h;
+      for (int c = 0; c < EB; c++) {
+        const int e = EB * (8 * g4 + 4 * h) + 4 * c;
         float x[4];
 #pragma unroll
-        for (int i = 0; i < 4; i++) x[i] = o[eb][4 * g4 + i] * wb;
+        for (int u = 0; u < 4; u++) x[u] = o[(4 * c + u) % EB][4 * g4 + (4 * c + u) / EB] * wb;
         if (wa != 0.f) {
           float4v oi = *reinterpret_cast<const float4v*>(orow + e);
 #pragma unroll
-          for (int i = 0; i < 4; i++) x[i] += wa * oi[i];
+          for (int u = 0; u < 4; u++) x[u] += wa * oi[u];
         }
         float4v y = {x[0], x[1], x[2], x[3]};
         *reinterpret_cast<float4v*>(orow + e) = y;
@@ -211,14 +227,23 @@ __global__ __launch_bounds__(256, 2) void tile_kernel(TileArgs a) {
   // position counts; [u_lo, u_hi): key positions this workgroup walks
   int64_t base = 0, qlen, klen, t0, u_lo, u_hi, split = 0;
   int64_t bb = 0;  // problem of the batch (global modes; band mode folds it into base)
+  int quarter = -1;  // band: which 32 queries of a shared tail tile (-1: a whole tile)
   if constexpr (MODE == kTileBand) {
     // workgroups are dealt round-robin to the 8 XCDs: give each XCD a contiguous run of tiles
     // so that neighbouring query tiles (which share most of their keys) meet in one L2
     // (the tiles of all problems of a batch form one list; problem pb starts at token pb * n)
     const int64_t n_all = a.n_tiles * a.t.n_batch;
-    const int64_t per_xcd = (n_all + 7) / 8;
-    int64_t lt = (int64_t)(blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
-    if (lt >= n_all) return;
+    const int64_t n_main = n_all - a.n_tail;
+    const int64_t per_xcd = (n_main + 7) / 8;
+    int64_t lt;
+    if ((int64_t)blockIdx.x < 8 * per_xcd) {
+      lt = (int64_t)(blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+      if (lt >= n_main) return;
+    } else {
+      const int64_t qid = (int64_t)blockIdx.x - 8 * per_xcd;
+      lt = n_main + qid / 4;
+      quarter = (int)(qid & 3);
+    }
     const int64_t pb = lt / a.n_tiles;
     lt -= pb * a.n_tiles;
     const int64_t sub = lt / a.tiles_per_sub;
@@ -231,11 +256,11 @@ __global__ __launch_bounds__(256, 2) void tile_kernel(TileArgs a) {
       qlen = (a.n - sub + a.s - 1) / a.s;
     }
     klen = qlen;
-    t0 = tile * BM;
+    t0 = tile * BM + (quarter >= 0 ? 32 * quarter : 0);
     if (t0 >= qlen) return;
     u_lo = t0 - a.w;
     if (u_lo < 0) u_lo = 0;
-    u_hi = t0 + BM + a.w;
+    u_hi = t0 + (quarter >= 0 ? 32 : BM) + a.w;
     if (u_hi > klen || u_hi < 0) u_hi = klen;
   } else if constexpr (MODE == kTileGlobalRows) {
     // grid: [problem][query tile][key split]
@@ -281,8 +306,10 @@ __global__ __launch_bounds__(256, 2) void tile_kernel(TileArgs a) {
   for (;; t0 += (int64_t)gridDim.x * BM) {
   if (t0 >= qlen) break;
   const bool pair_split = (MODE == kTileGlobalRows) && NB == 2 && a.pair_split != 0;
-  const int wave_q = pair_split ? (wave & 1) : wave;  // query block of this wavefront
-  const int wave_k = pair_split ? (wave >> 1) : -1;   // key block it is restricted to (-1: all)
+  const bool quad_split = (MODE == kTileBand) && quarter >= 0;
+  // query block of this wavefront, and the share of the key blocks it is restricted to (-1: all)
+  const int wave_q = quad_split ? 0 : pair_split ? (wave & 1) : wave;
+  const int wave_k = quad_split ? wave : pair_split ? (wave >> 1) : -1;
   const int64_t tw0 = t0 + 32 * wave_q;  // first query of this wavefront
   const int64_t tq = tw0 + r;          // this lane's query position
   bool q_ok = tq < qlen;
@@ -303,10 +330,12 @@ __global__ __launch_bounds__(256, 2) void tile_kernel(TileArgs a) {
     const T* qrow = Qp + (q_tok + tok_off) * D;
     if constexpr (kF32) {
 #pragma unroll
-      for (int c4 = 0; c4 < D / 4; c4++) {
-        float4v x = *reinterpret_cast<const float4v*>(qrow + 4 * c4);
-        qf[2 * c4] = h ? x[1] : x[0];
-        qf[2 * c4 + 1] = h ? x[3] : x[2];
+      for (int g = 0; g < D / 8; g++) {
+        float4v x = *reinterpret_cast<const float4v*>(qrow + 8 * g + 4 * h);
+        qf[4 * g] = x[0];
+        qf[4 * g + 1] = x[1];
+        qf[4 * g + 2] = x[2];
+        qf[4 * g + 3] = x[3];
       }
     } else {
 #pragma unroll
@@ -377,9 +406,7 @@ __global__ __launch_bounds__(256, 2) void tile_kernel(TileArgs a) {
       const int idx = it * 256 + tid;
       const int j = idx / CH, c = idx % CH;
       if constexpr (kF32) {
-        float4v kx = __builtin_bit_cast(float4v, kreg[it]);
-        float* kd = (float*)Ks + j * C::K_STRIDE + 4 * c;  // rows are only 8-byte aligned
-        kd[0] = kx[0]; kd[1] = kx[1]; kd[2] = kx[2]; kd[3] = kx[3];
+        *reinterpret_cast<uint4v*>((float*)Ks + j * C::K_STRIDE + 4 * c) = kreg[it];
         *reinterpret_cast<uint4v*>((float*)Vs + j * C::V_STRIDE + 4 * c) = vreg[it];
       } else {
         *reinterpret_cast<uint4v*>(Ks + j * C::K_STRIDE + 8 * c) = kreg[it];
@@ -425,7 +452,8 @@ __global__ __launch_bounds__(256, 2) void tile_kernel(TileArgs a) {
     for (int jb = 0; jb < NB; jb++) {
       const int64_t ub = ut + 32 * jb;
       if constexpr (MODE == kTileBand)
-        need[jb] = (tw0 < qlen) && (ub < u_hi) && (ub <= tw0 + 31 + a.w) && (ub + 31 + a.w >= tw0);
+        need[jb] = (tw0 < qlen) && (ub < u_hi) && (ub <= tw0 + 31 + a.w) && (ub + 31 + a.w >= tw0) &&
+                   (wave_k < 0 || (int)(((ub - u_lo) >> 5) & 3) == wave_k);
       else
         need[jb] = (tw0 < qlen) && (ub < u_hi) && (wave_k < 0 || wave_k == jb);
       any_need = any_need || need[jb];
@@ -438,11 +466,18 @@ __global__ __launch_bounds__(256, 2) void tile_kernel(TileArgs a) {
     for (int jb = 0; jb < NB; jb++) {
       if (!need[jb]) continue;  // (filled with -inf below)
       if constexpr (kF32) {
-        const float* krow = (const float*)Ks + (32 * jb + r) * C::K_STRIDE + h;
-        sreg[jb] = __builtin_amdgcn_mfma_f32_32x32x2f32(krow[0], qf[0], zero16, 0, 0, 0);
+        const float* krow = (const float*)Ks + (32 * jb + r) * C::K_STRIDE + 4 * h;
+        float4v kx = *reinterpret_cast<const float4v*>(krow);
+        sreg[jb] = zero16;
 #pragma unroll
-        for (int ks = 1; ks < D / 2; ks++)
-          sreg[jb] = __builtin_amdgcn_mfma_f32_32x32x2f32(krow[2 * ks], qf[ks], sreg[jb], 0, 0, 0);
+        for (int g = 0; g < D / 8; g++) {
+          float4v kn = kx;
+          if (g + 1 < D / 8) kn = *reinterpret_cast<const float4v*>(krow + 8 * (g + 1));
+#pragma unroll
+          for (int i = 0; i < 4; i++)
+            sreg[jb] = __builtin_amdgcn_mfma_f32_32x32x2f32(kx[i], qf[4 * g + i], sreg[jb], 0, 0, 0);
+          kx = kn;
+        }
       } else {
         const T* krow = Ks + (32 * jb + r) * C::K_STRIDE + 8 * h;
         sreg[jb] = mfma16<T>(*reinterpret_cast<const uint4v*>(krow), qh[0], zero16);
@@ -532,12 +567,18 @@ __global__ __launch_bounds__(256, 2) void tile_kernel(TileArgs a) {
     for (int jb = 0; jb < NB; jb++) {
       if (!need[jb]) continue;
       if constexpr (kF32) {
+        typedef float vecE __attribute__((ext_vector_type(EB)));
+        const float* vbase = (const float*)Vs + (32 * jb + 4 * h) * C::V_STRIDE + EB * r;
+        vecE vx = *reinterpret_cast<const vecE*>(vbase);
 #pragma unroll
         for (int v = 0; v < 16; v++) {
-          const float* vrow = (const float*)Vs + (32 * jb + 8 * (v / 4) + 4 * h + (v % 4)) * C::V_STRIDE + r;
+          vecE vn = vx;
+          if (v + 1 < 16)
+            vn = *reinterpret_cast<const vecE*>(vbase + (8 * ((v + 1) / 4) + ((v + 1) % 4)) * C::V_STRIDE);
 #pragma unroll
           for (int eb = 0; eb < EB; eb++)
-            o[eb] = __builtin_amdgcn_mfma_f32_32x32x2f32(vrow[32 * eb], sreg[jb][v], o[eb], 0, 0, 0);
+            o[eb] = __builtin_amdgcn_mfma_f32_32x32x2f32(vx[eb], sreg[jb][v], o[eb], 0, 0, 0);
+          vx = vn;
         }
       } else {
 #pragma unroll
@@ -559,34 +600,44 @@ __global__ __launch_bounds__(256, 2) void tile_kernel(TileArgs a) {
 
   // ---- finish: combine the two key halves, fold the incoming state in, write back
   l += shfl_xor_f32(l, 32);
-  if constexpr (MODE == kTileGlobalRows && NB == 2) {
-    if (pair_split) {
-      // fold wavefront (q, 1) into wavefront (q, 0) through LDS (the tiles are no longer needed)
+  if constexpr ((MODE == kTileGlobalRows && NB == 2) || MODE == kTileBand) {
+    if (pair_split || quad_split) {
+      // fold the wavefronts that share a query block, upper half into lower half, through LDS
+      // (the tiles are no longer needed): (q, 1) into (q, 0) for the pairs; 2, 3 into 0, 1 and
+      // then 1 into 0 for the four wavefronts of a shared tail tile
       constexpr int XR = EB * 16 + 2;
       static_assert(2 * XR * kWave * 4 <= C::LDS_BYTES, "exchange area does not fit the tile buffers");
-      float* xs = reinterpret_cast<float*>(lds) + (size_t)wave_q * XR * kWave + lane;
-      __syncthreads();
-      if (wave_k == 1) {
+      const int nq = quad_split ? 1 : 2;
+      for (int step = quad_split ? 2 : 1; step >= 1; step >>= 1) {
+        const bool gives = wave_k >= step && wave_k < 2 * step;
+        const bool takes = wave_k < step;
+        float* xs = reinterpret_cast<float*>(lds) +
+                    (size_t)(wave_q + nq * (gives ? wave_k - step : wave_k)) * XR * kWave + lane;
+        __syncthreads();
+        if (gives) {
 #pragma unroll
-        for (int eb = 0; eb < EB; eb++)
+          for (int eb = 0; eb < EB; eb++)
 #pragma unroll
-          for (int v = 0; v < 16; v++) xs[(eb * 16 + v) * kWave] = o[eb][v];
-        xs[(EB * 16) * kWave] = m;
-        xs[(EB * 16 + 1) * kWave] = l;
+            for (int v = 0; v < 16; v++) xs[(eb * 16 + v) * kWave] = o[eb][v];
+          xs[(EB * 16) * kWave] = m;
+          xs[(EB * 16 + 1) * kWave] = l;
+        }
+        __syncthreads();
+        if (takes) {
+          const float m2 = xs[(EB * 16) * kWave], l2 = xs[(EB * 16 + 1) * kWave];
+          const float m_new = fmaxf(m, m2);
+          if (m_new > kNegInf) {
+            const float fa = __builtin_amdgcn_exp2f(m - m_new), fb = __builtin_amdgcn_exp2f(m2 - m_new);
+            l = l * fa + l2 * fb;
+#pragma unroll
+            for (int eb = 0; eb < EB; eb++)
+#pragma unroll
+              for (int v = 0; v < 16; v++) o[eb][v] = o[eb][v] * fa + xs[(eb * 16 + v) * kWave] * fb;
+            m = m_new;
+          }
+        }
       }
-      __syncthreads();
-      if (wave_k == 1) return;
-      const float m2 = xs[(EB * 16) * kWave], l2 = xs[(EB * 16 + 1) * kWave];
-      const float m_new = fmaxf(m, m2);
-      if (m_new > kNegInf) {
-        const float fa = __builtin_amdgcn_exp2f(m - m_new), fb = __builtin_amdgcn_exp2f(m2 - m_new);
-        l = l * fa + l2 * fb;
-#pragma unroll
-        for (int eb = 0; eb < EB; eb++)
-#pragma unroll
-          for (int v = 0; v < 16; v++) o[eb][v] = o[eb][v] * fa + xs[(eb * 16 + v) * kWave] * fb;
-        m = m_new;
-      }
+      if (wave_k != 0) return;  // (both modes make a single trip)
     }
   }
   if constexpr (MODE == kTileGlobalRows) {
@@ -595,16 +646,30 @@ __global__ __launch_bounds__(256, 2) void tile_kernel(TileArgs a) {
     const int64_t slot = (bb * a.n_globs + tq) * a.n_split + split;
     const bool any = l > 0.f;
     float* prow = a.pacc + slot * D;
+    if constexpr (kF32) {
 #pragma unroll
-    for (int eb = 0; eb < EB; eb++)
+      for (int g4 = 0; g4 < 4; g4++)
 #pragma unroll
-      for (int g4 = 0; g4 < 4; g4++) {
-        float4v y = {0.f, 0.f, 0.f, 0.f};
-        if (any) {
-          y[0] = o[eb][4 * g4]; y[1] = o[eb][4 * g4 + 1]; y[2] = o[eb][4 * g4 + 2]; y[3] = o[eb][4 * g4 + 3];
+        for (int c = 0; c < EB; c++) {
+          float4v y = {0.f, 0.f, 0.f, 0.f};
+          if (any) {
+#pragma unroll
+            for (int u = 0; u < 4; u++) y[u] = o[(4 * c + u) % EB][4 * g4 + (4 * c + u) / EB];
+          }
+          *reinterpret_cast<float4v*>(prow + EB * (8 * g4 + 4 * h) + 4 * c) = y;
         }
-        *reinterpret_cast<float4v*>(prow + 32 * eb + 8 * g4 + 4 * h) = y;
-      }
+    } else {
+#pragma unroll
+      for (int eb = 0; eb < EB; eb++)
+#pragma unroll
+        for (int g4 = 0; g4 < 4; g4++) {
+          float4v y = {0.f, 0.f, 0.f, 0.f};
+          if (any) {
+            y[0] = o[eb][4 * g4]; y[1] = o[eb][4 * g4 + 1]; y[2] = o[eb][4 * g4 + 2]; y[3] = o[eb][4 * g4 + 3];
+          }
+          *reinterpret_cast<float4v*>(prow + 32 * eb + 8 * g4 + 4 * h) = y;
+        }
+    }
     if (h == 0) {
       a.pm[slot] = any ? m * 0.6931471805599453f : kNegInf;
       a.pl[slot] = any ? l : 0.f;
@@ -1019,7 +1084,20 @@ int launch_band_tiles(const TileArgs& a, int use_nan, hipStream_t stream) {
       else
         hipLaunchKernelGGL((tile_kernel<T, D, kTileBand>), dim3((unsigned)grid), dim3(256), 0, stream, a);
     } else {
-      hipLaunchKernelGGL((tile_kernel<T, D, kTileBand>), dim3((unsigned)grid), dim3(256), 0, stream, a);
+      // Two workgroups fit a CU, and tiles take about the same time, so the grid runs in rounds
+      // of `resident` tiles and the tiles of a last, sparsely filled round keep the chip
+      // waiting for a whole round (0.14 ms for a single tile left over at d = 128, window 256).
+      // When four workgroups for each of those tiles still fit one round, the tiles are shared
+      // out that way: such a workgroup takes two thirds of the time of a whole tile (its
+      // wavefronts take turns, one key block per LDS tile), and all of them together cost about
+      // twice the time per tile, hence not for fuller rounds.
+      TileArgs at = a;
+      const int64_t n_all = a.n_tiles * a.t.n_batch;
+      const int64_t resident = (int64_t)device_cu_count() * 2;
+      const int64_t rem = n_all % resident;
+      at.n_tail = (4 * rem <= resident) ? rem : 0;
+      const int64_t grid_t = (n_all - at.n_tail + 7) / 8 * 8 + 4 * at.n_tail;
+      hipLaunchKernelGGL((tile_kernel<T, D, kTileBand>), dim3((unsigned)grid_t), dim3(256), 0, stream, at);
     }
     if (timed) (void)hipEventRecord(ev.stop, stream);
   }

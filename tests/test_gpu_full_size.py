@@ -128,6 +128,36 @@ def test_local_1d_dilated_n262144(mods):
     assert int(l.double().sum().item()) == so.nnz_local_1d_dilated(n, w, dil)
 
 
+@pytest.mark.parametrize("case", ["local_d64", "dilated_d128"])
+def test_band_fp32_shared_tail_tiles(mods, case):
+    """fp32 band masks whose tile count is a few over a multiple of the resident workgroups: the
+    left-over tiles are shared by four workgroups each.  Rows of those tiles (the end of the last
+    subsequence) and of ordinary ones, against the oracle."""
+    dtype = torch.float32
+    if case == "local_d64":
+        n, d, w = 128 * 515 + 40, 64, 96
+        call = lambda q, k, v, m, l, o: mods["spfa_local"].forward(q, k, v, m, l, o, w)
+        live = lambda i: so.live_local(n, w, i)
+        nnz = so.nnz_local(n, w)
+    else:
+        n, d, w, dil = 262144, 128, 256, 2
+        call = lambda q, k, v, m, l, o: mods["spfa_local_1d_dilated"].forward(q, k, v, m, l, o, w, dil)
+        live = lambda i: so.live_local_1d_dilated(n, w, dil, i)
+        nnz = so.nnz_local_1d_dilated(n, w, dil)
+    q, k, v = syn.qkv(n, d, dtype=dtype, device=DEV, seed=3, scale=0.5)
+    m, l, o = syn.fresh_state(n, d, dtype=dtype, device=DEV, state_dtype=torch.float32)
+    call(q, k, v, m, l, o)
+    rows = np.concatenate([np.arange(n - 600, n, 7), [0, 1, 2, n - 3, n - 2, n - 1], rand_rows(n, 60, 9)])
+    sample_check(q, k, v, o, m, l, np.unique(rows), live, dtype)
+    # a second call on top of the first doubles l and leaves out where it was
+    m2, l2, o2 = m.clone(), l.clone(), o.clone()
+    call(q, k, v, m2, l2, o2)
+    assert torch.allclose(l2, 2 * l, rtol=1e-5) and torch.allclose(o2, o, atol=2e-5)
+    m, l, o = syn.fresh_state(n, d, dtype=dtype, device=DEV, state_dtype=torch.float32)
+    call(torch.zeros_like(q), k, v, m, l, o)
+    assert torch.all(m == 0) and int(l.double().sum().item()) == nnz
+
+
 @pytest.mark.parametrize("use_nan", [True, False])
 def test_local_2d_dilated_n262144(mods, use_nan):
     n, d, block, dil = 262144, 128, 256, 2
