@@ -131,15 +131,17 @@ struct BoolConst {
 // of the wavefront); o * o_scale is the accumulator that goes with (m, l).
 template <typename T, int D>
 __device__ __forceinline__ void tile_write_row(const Tensors& t, int64_t row, int h, float m, float l,
-                                               const f32x16 (&o)[D / 32], float o_scale = 1.f) {
+                                               const f32x16 (&o)[D / 32], float o_scale = 1.f,
+                                               bool have_in = false, float l_pre = 0.f, float m_pre = 0.f) {
   constexpr bool kF32 = sizeof(T) == 4;
   const bool sf = t.state_f32 != 0;
   const float m_nat = m * 0.6931471805599453f;
   float m_out = m_nat, l_out = l;
   float wa = 0.f, wb = 1.f;
-  const float l_in = load_state<T>(t.l, row, sf);
+  // (have_in: the caller has read the incoming state already, while it worked on the tile)
+  const float l_in = have_in ? l_pre : load_state<T>(t.l, row, sf);
   if (l_in != 0.f) {
-    const float m_in = load_state<T>(t.m, row, sf);
+    const float m_in = have_in ? m_pre : load_state<T>(t.m, row, sf);
     m_out = fmaxf(m_nat, m_in);
     wa = l_in * __expf(m_in - m_out);
     wb = __expf(m_nat - m_out);
@@ -302,6 +304,29 @@ __global__ __launch_bounds__(256, 2) void tile_kernel(TileArgs a) {
   const int64_t tok_off = (MODE == kTileBand) ? 0 : bb * a.n;
   bool staged = false;  // persist: the key tile is already in LDS
 
+  // Q^T operand of a query tile, kept in registers.  A persistent workgroup asks for the rows of
+  // its next query tile before it works on the current one (where the registers allow it).
+  constexpr bool kNextQ = (MODE == kTileGlobalCols) && D <= 64;
+  uint4v qh[kF32 ? 1 : C::QREGS], qh_next[(kNextQ && !kF32) ? C::QREGS : 1];
+  float qf[kF32 ? C::QREGS : 1], qf_next[(kNextQ && kF32) ? C::QREGS : 1];
+  auto load_q = [&](const T* qrow, uint4v* dh, float* df) {
+    if constexpr (kF32) {
+#pragma unroll
+      for (int g = 0; g < D / 8; g++) {
+        float4v x = *reinterpret_cast<const float4v*>(qrow + 8 * g + 4 * h);
+        df[4 * g] = x[0];
+        df[4 * g + 1] = x[1];
+        df[4 * g + 2] = x[2];
+        df[4 * g + 3] = x[3];
+      }
+    } else {
+#pragma unroll
+      for (int ks = 0; ks < C::QREGS; ks++)
+        dh[ks] = *reinterpret_cast<const uint4v*>(qrow + 16 * ks + 8 * h);
+    }
+  };
+  bool have_q = false;  // the rows of this trip were asked for during the previous one
+
   // One trip per query tile.  Only a persistent GlobalCols workgroup makes more than one.
   for (;; t0 += (int64_t)gridDim.x * BM) {
   if (t0 >= qlen) break;
@@ -323,24 +348,20 @@ __global__ __launch_bounds__(256, 2) void tile_kernel(TileArgs a) {
     if (q_ok && bit_is_set(a.gbits, q_tok)) q_ok = false;  // global rows belong to GlobalRows
   }
 
-  // ---- Q^T operand, kept in registers
-  uint4v qh[kF32 ? 1 : C::QREGS];
-  float qf[kF32 ? C::QREGS : 1];
-  {
-    const T* qrow = Qp + (q_tok + tok_off) * D;
-    if constexpr (kF32) {
-#pragma unroll
-      for (int g = 0; g < D / 8; g++) {
-        float4v x = *reinterpret_cast<const float4v*>(qrow + 8 * g + 4 * h);
-        qf[4 * g] = x[0];
-        qf[4 * g + 1] = x[1];
-        qf[4 * g + 2] = x[2];
-        qf[4 * g + 3] = x[3];
-      }
-    } else {
-#pragma unroll
-      for (int ks = 0; ks < C::QREGS; ks++)
-        qh[ks] = *reinterpret_cast<const uint4v*>(qrow + 16 * ks + 8 * h);
+  if (!have_q) load_q(Qp + (q_tok + tok_off) * D, qh, qf);
+  // a persistent workgroup finishes a row every few microseconds: its incoming state is read
+  // here, long before the write-back needs it
+  float l_pre = 0.f, m_pre = 0.f;
+  if constexpr (MODE == kTileGlobalCols) {
+    l_pre = load_state<T>(a.t.l, q_tok + tok_off, a.t.state_f32 != 0);
+    m_pre = load_state<T>(a.t.m, q_tok + tok_off, a.t.state_f32 != 0);
+  }
+  if constexpr (kNextQ) {
+    const int64_t t0n = t0 + (int64_t)gridDim.x * BM;
+    have_q = persist && t0n < qlen;
+    if (have_q) {
+      const int64_t tqn = t0n + 32 * wave_q + r;
+      load_q(Qp + ((tqn < qlen ? tqn : qlen - 1) + tok_off) * D, qh_next, qf_next);
     }
   }
 
@@ -466,17 +487,24 @@ __global__ __launch_bounds__(256, 2) void tile_kernel(TileArgs a) {
     for (int jb = 0; jb < NB; jb++) {
       if (!need[jb]) continue;  // (filled with -inf below)
       if constexpr (kF32) {
+        // operand reads run two groups of four instructions ahead (order pinned: left to
+        // itself the compiler issues a read, waits for it and only then starts the four)
         const float* krow = (const float*)Ks + (32 * jb + r) * C::K_STRIDE + 4 * h;
-        float4v kx = *reinterpret_cast<const float4v*>(krow);
+        float4v kx[3];
+        kx[0] = *reinterpret_cast<const float4v*>(krow);
+        kx[1] = *reinterpret_cast<const float4v*>(krow + 8);
         sreg[jb] = zero16;
+        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
 #pragma unroll
         for (int g = 0; g < D / 8; g++) {
-          float4v kn = kx;
-          if (g + 1 < D / 8) kn = *reinterpret_cast<const float4v*>(krow + 8 * (g + 1));
+          if (g + 2 < D / 8) {
+            kx[(g + 2) % 3] = *reinterpret_cast<const float4v*>(krow + 8 * (g + 2));
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+          }
 #pragma unroll
           for (int i = 0; i < 4; i++)
-            sreg[jb] = __builtin_amdgcn_mfma_f32_32x32x2f32(kx[i], qf[4 * g + i], sreg[jb], 0, 0, 0);
-          kx = kn;
+            sreg[jb] = __builtin_amdgcn_mfma_f32_32x32x2f32(kx[g % 3][i], qf[4 * g + i], sreg[jb], 0, 0, 0);
+          __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
         }
       } else {
         const T* krow = Ks + (32 * jb + r) * C::K_STRIDE + 8 * h;
@@ -569,16 +597,24 @@ __global__ __launch_bounds__(256, 2) void tile_kernel(TileArgs a) {
       if constexpr (kF32) {
         typedef float vecE __attribute__((ext_vector_type(EB)));
         const float* vbase = (const float*)Vs + (32 * jb + 4 * h) * C::V_STRIDE + EB * r;
-        vecE vx = *reinterpret_cast<const vecE*>(vbase);
+        // reads run PD keys ahead of the instructions that use them (order pinned, as above)
+        constexpr int PD = 8 / EB;
+        vecE vx[PD + 1];
+#pragma unroll
+        for (int v = 0; v < PD; v++)
+          vx[v] = *reinterpret_cast<const vecE*>(vbase + (8 * (v / 4) + (v % 4)) * C::V_STRIDE);
+        __builtin_amdgcn_sched_group_barrier(0x100, PD, 0);
 #pragma unroll
         for (int v = 0; v < 16; v++) {
-          vecE vn = vx;
-          if (v + 1 < 16)
-            vn = *reinterpret_cast<const vecE*>(vbase + (8 * ((v + 1) / 4) + ((v + 1) % 4)) * C::V_STRIDE);
+          if (v + PD < 16) {
+            vx[(v + PD) % (PD + 1)] =
+                *reinterpret_cast<const vecE*>(vbase + (8 * ((v + PD) / 4) + ((v + PD) % 4)) * C::V_STRIDE);
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+          }
 #pragma unroll
           for (int eb = 0; eb < EB; eb++)
-            o[eb] = __builtin_amdgcn_mfma_f32_32x32x2f32(vx[eb], sreg[jb][v], o[eb], 0, 0, 0);
-          vx = vn;
+            o[eb] = __builtin_amdgcn_mfma_f32_32x32x2f32(vx[v % (PD + 1)][eb], sreg[jb][v], o[eb], 0, 0, 0);
+          __builtin_amdgcn_sched_group_barrier(0x008, EB, 0);
         }
       } else {
 #pragma unroll
@@ -676,8 +712,20 @@ __global__ __launch_bounds__(256, 2) void tile_kernel(TileArgs a) {
     }
     return;
   }
-  if (q_ok && l > 0.f) tile_write_row<T, D>(a.t, q_tok + tok_off, h, m, l, o);
+  if (q_ok && l > 0.f && wave_k <= 0)
+    tile_write_row<T, D>(a.t, q_tok + tok_off, h, m, l, o, 1.f, MODE == kTileGlobalCols, l_pre, m_pre);
   if (!persist) break;
+  if constexpr (kNextQ) {
+    if (have_q) {
+      if constexpr (kF32) {
+#pragma unroll
+        for (int i = 0; i < C::QREGS; i++) qf[i] = qf_next[i];
+      } else {
+#pragma unroll
+        for (int i = 0; i < C::QREGS; i++) qh[i] = qh_next[i];
+      }
+    }
+  }
   }  // query tiles
 }
 
