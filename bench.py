@@ -676,7 +676,8 @@ def main():
         achieved_tf = kernel_flops / (k_avg * 1e-3) / 1e12
         roofline = {"bound": "mfma", "achieved": achieved_tf, "peak": peak, "unit": "TFLOP/s",
                     "frac": achieved_tf / peak, "traffic": None,
-                    "kernel": "tile_kernel (global rows)" if a.workload == "global" else "tile_kernel",
+                    "kernel": "tile_kernel (global rows)" if a.workload == "global" else
+                              ("band_dma_f32_kernel" if a.dtype == "f32" else "band_dma_kernel"),
                     "hbm_time_ms": w["bytes_total"] / (HBM_PEAK_GBS * 1e9) * 1e3,
                     "mfma_time_ms": flops / (peak * 1e12) * 1e3}
     if roofline["bound"] == "hbm":

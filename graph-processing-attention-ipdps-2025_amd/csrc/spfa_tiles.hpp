@@ -60,6 +60,7 @@ struct TileArgs {
   int64_t n_tail;         // band: the last n_tail tiles (over all problems) are each shared by four
                           // workgroups of 32 queries whose wavefronts deal the key blocks among
                           // themselves; they fill the last, partly empty round of the grid
+  int32_t tail_only;      // band: the launch holds the shared tail tiles only
   // global modes
   const int32_t* globs;   // listed global tokens (keys of GlobalCols)
   int64_t n_globs;
@@ -238,7 +239,10 @@ __global__ __launch_bounds__(256, 2) void tile_kernel(TileArgs a) {
     const int64_t n_main = n_all - a.n_tail;
     const int64_t per_xcd = (n_main + 7) / 8;
     int64_t lt;
-    if ((int64_t)blockIdx.x < 8 * per_xcd) {
+    if (a.tail_only) {
+      lt = n_main + blockIdx.x / 4;
+      quarter = (int)(blockIdx.x & 3);
+    } else if ((int64_t)blockIdx.x < 8 * per_xcd) {
       lt = (int64_t)(blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
       if (lt >= n_main) return;
     } else {
@@ -1030,6 +1034,268 @@ __global__ __launch_bounds__(256, 2) void band_dma_kernel(TileArgs a) {
   }
 }
 
+// ---------------------------------------------------------------------------------------
+// Band masks, fp32: tiles go from global memory straight into LDS
+// ---------------------------------------------------------------------------------------
+// The fp32 counterpart of band_dma_kernel: the same plumbing (two 32-KB tile buffers filled by the
+// load instructions, one barrier per tile, reference maximum with slack) around the fp32
+// products of tile_kernel (k pairing and permuted output rows, 16-byte operand reads).  A tile is
+// 4096 floats of K and of V: 64 keys at d = 64, 32 keys at d = 128.  Rows are 256 or 512 bytes,
+// so chunk c of row j sits at chunk position c ^ (j mod 16): the 16 rows read by a quarter of a
+// wavefront for one K operand, and the 16 consecutive chunks of one row read for a V operand,
+// then cover every bank once.
+template <int D>
+struct BandDmaF32Cfg {
+  static constexpr int BM = 128;
+  static constexpr int BN = 4096 / D;           // keys per tile
+  static constexpr int NB = BN / 32;            // 32-key blocks per tile
+  static constexpr int ROWB = D * 4;            // bytes per K / V row
+  static constexpr int TILE_B = BN * ROWB;      // bytes of one K (or V) tile: 16 KB
+  static constexpr int BUF_B = 2 * TILE_B;      // K tile then V tile
+  static constexpr int NI = TILE_B / 4096;      // load instructions per wavefront, tile and matrix
+  static constexpr int EB = D / 32, QREGS = D / 2;
+};
+
+template <int D>
+__global__ __launch_bounds__(256, 2) void band_dma_f32_kernel(TileArgs a) {
+  using C = BandDmaF32Cfg<D>;
+  constexpr int BM = C::BM, BN = C::BN, NB = C::NB, EB = C::EB, ROWB = C::ROWB;
+  constexpr int TILE_B = C::TILE_B, BUF_B = C::BUF_B, NI = C::NI;
+  static_assert(D == 64 || D == 128, "d = 64 or 128");
+  __shared__ __attribute__((aligned(1024))) char lds_even[BUF_B];
+  __shared__ __attribute__((aligned(1024))) char lds_odd[BUF_B];
+
+  auto uni = [](int x) { return __builtin_amdgcn_readfirstlane(x); };
+  // the whole tiles of the list (the shared tail tiles have a launch of their own)
+  const int64_t n_main = a.n_tiles * a.t.n_batch - a.n_tail;
+  const int64_t per_xcd = (n_main + 7) / 8;
+  int64_t lt = (int64_t)(blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+  if (lt >= n_main) return;
+  const int64_t bb = lt / a.n_tiles;
+  lt -= bb * a.n_tiles;
+  const int64_t sub = lt / a.tiles_per_sub;
+  const int tile = uni((int)(lt - sub * a.tiles_per_sub));
+  int64_t base;
+  int qlen;
+  if (a.block > 0) {
+    base = sub * a.block + bb * a.n;
+    qlen = (int)a.cnt;
+  } else {
+    base = sub + bb * a.n;
+    qlen = uni((int)((a.n - sub + a.s - 1) / a.s));
+  }
+  const int wlim = (int)(a.w < (int64_t)0x3fffffff ? a.w : (int64_t)0x3fffffff);  // window, clamped
+  const int t0 = tile * BM;
+  if (t0 >= qlen) return;
+  const int u_lo = t0 > wlim ? t0 - wlim : 0;
+  const int u_hi = (qlen - BM - wlim > t0) ? t0 + BM + wlim : qlen;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int r = lane & 31, h = lane >> 5;
+  const char* Kp = (const char*)a.t.k;
+  const char* Vp = (const char*)a.t.v;
+  const float sc = 1.4426950408889634f / sqrtf((float)D);
+
+  const int tw0 = t0 + 32 * wave;  // first query of this wavefront
+  const int tq = tw0 + r;          // this lane's query position
+  const bool q_ok = tq < qlen;
+  const int64_t q_tok = base + (int64_t)(q_ok ? tq : qlen - 1) * a.s;
+
+  // ---- Q^T operand, kept in registers: half h holds k = 8g + 4h + i in qf[4g + i]
+  float qf[C::QREGS];
+  {
+    const float* qrow = (const float*)a.t.q + q_tok * D;
+#pragma unroll
+    for (int g = 0; g < D / 8; g++) {
+      const float4v x = *reinterpret_cast<const float4v*>(qrow + 8 * g + 4 * h);
+      qf[4 * g] = x[0];
+      qf[4 * g + 1] = x[1];
+      qf[4 * g + 2] = x[2];
+      qf[4 * g + 3] = x[3];
+    }
+  }
+
+  // ---- tile loads: instruction `it` of this wavefront fills the 1-KB segment 4*it + wave of a
+  // tile; this lane's 16 bytes are row j, chunk position p of it (K and V alike)
+  uint32_t toff[NI];  // byte offset of the lane's source chunk from the tile's first row
+  const uint32_t row_step = (uint32_t)a.s * (uint32_t)ROWB;  // bytes between consecutive keys
+#pragma unroll
+  for (int it = 0; it < NI; it++) {
+    const int at = (4 * it + wave) * 1024 + lane * 16;
+    const int j = at / ROWB, p = (at % ROWB) / 16;
+    toff[it] = (uint32_t)j * row_step + (uint32_t)((p ^ (j & 15)) * 16);
+  }
+  auto request = [&](int ut, char* dst_buf) {
+    const int64_t tile_byte = (base + (int64_t)ut * a.s) * (int64_t)ROWB;  // scalar
+    const bool whole = ut + BN <= u_hi;
+#pragma unroll
+    for (int it = 0; it < NI; it++) {
+      uint32_t off = toff[it];
+      if (!whole) {
+        // rows past the last key repeat the last key (finite values; they are masked out)
+        const int last = u_hi - 1 - ut;
+        const int j = ((4 * it + wave) * 1024 + lane * 16) / ROWB;
+        if (j > last) {
+          // (the chunk permutation depends on the row's slot in the tile, not on the key)
+          off -= (uint32_t)(j - last) * row_step;
+        }
+      }
+      char* dst = dst_buf + (4 * it + wave) * 1024;
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(Kp + tile_byte + off),
+                                       (__attribute__((address_space(3))) void*)dst, 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(Vp + tile_byte + off),
+                                       (__attribute__((address_space(3))) void*)(dst + TILE_B), 16, 0, 0);
+    }
+  };
+
+  // ---- operand addresses inside a tile buffer (bytes).  A chunk index is compile-time bits
+  // XOR a per-lane value, so eight addresses (the low three variable bits) serve every operand
+  // and the rest is a constant offset.
+  // K, block jb, group g: row 32*jb + r, chunk 2*g + h, at position (2*g) ^ (h ^ (r mod 16))
+  int kadr[8];
+#pragma unroll
+  for (int gl = 0; gl < 8; gl++) kadr[gl] = r * ROWB + (((2 * gl) ^ (h ^ (r & 15))) * 16);
+  // V, register v: row 8*(v/4) + 4*h + v%4 (+ 32*jb), the lane's EB floats from element EB*r:
+  // chunk (EB*r)/4, at position that ^ (row mod 16) = ((EB*r)/4 ^ 4*h) ^ cv, cv = 8*((v/4)%2) + v%4
+  int vadr[8];
+#pragma unroll
+  for (int x = 0; x < 8; x++) {
+    const int cv = 8 * (x / 4) + (x % 4);
+    vadr[x] = TILE_B + (4 * h + cv) * ROWB + (((((EB * r) / 4) ^ (4 * h)) ^ cv) * 16) + ((EB * r) % 4) * 4;
+  }
+
+  f32x16 o[EB];
+#pragma unroll
+  for (int eb = 0; eb < EB; eb++)
+#pragma unroll
+    for (int v = 0; v < 16; v++) o[eb][v] = 0.f;
+  constexpr float kSlack = 8.f;
+  float m = kNegInf;   // reference maximum of the exponentials, log2 units
+  float mt = kNegInf;  // true running maximum
+  float l = 0.f;       // running sum (relative to m) over this lane's half of the keys
+
+  auto step = [&](int ut, const char* tb, char* other) __attribute__((always_inline)) {
+    __builtin_amdgcn_s_waitcnt(0);  // this wavefront's part of the tile has landed
+    __syncthreads();                // everyone's has, and everyone is done with the other buffer
+    if (ut + BN < u_hi) request(ut + BN, other);
+
+    const bool all_full = (ut + BN <= u_hi) && (ut >= tw0 + 31 - wlim) && (ut + BN - 1 - wlim <= tw0);
+    const bool none = (tw0 >= qlen) || (ut - wlim > tw0 + 31) || (ut + BN - 1 < tw0 - wlim);
+    if (none) return;
+
+    // key slot j of the tile is live for this lane's query iff jlo <= j <= jhi; the slots this
+    // lane holds are c + 4*h for compile-time c, so the bounds are shifted by 4*h once
+    const int live_slots = (u_hi - ut) < BN ? (u_hi - ut) : BN;
+    const int jlo = (tq - wlim - ut) - 4 * h;
+    const int jhi_band = tq + wlim - ut;
+    const int jhi = (jhi_band < live_slots - 1 ? jhi_band : live_slots - 1) - 4 * h;
+    const uint32_t span = (uint32_t)(jhi - jlo);  // jhi < jlo: wraps to a huge value, handled below
+    const bool any_live = jhi >= jlo;
+
+    // one online-softmax step over a 32-key block (reference maximum with slack, as in
+    // band_dma_kernel); leaves the exponentials in s
+    auto soft = [&](f32x16& s, int jb) {
+      if (!all_full) {
+#pragma unroll
+        for (int v = 0; v < 16; v++) {
+          const int c = 32 * jb + 8 * (v / 4) + (v % 4);
+          const bool ok = any_live && ((uint32_t)(c - jlo) <= span);
+          s[v] = ok ? s[v] : kNegInf;
+        }
+      }
+      float mx = s[0];
+#pragma unroll
+      for (int v = 1; v < 16; v++) mx = fmaxf(mx, s[v]);
+      mx = fmaxf(mx, shfl_xor_f32(mx, 32)) * sc;
+      mt = fmaxf(mt, mx);
+      if (__builtin_expect(__builtin_amdgcn_ballot_w64(mx > m + kSlack) != 0, 0)) {
+        const float m_new = (mx > m + kSlack) ? mx : m;
+        const float alpha = (m > kNegInf) ? __builtin_amdgcn_exp2f(m - m_new) : 0.f;
+        m = m_new;
+        l *= alpha;
+#pragma unroll
+        for (int eb = 0; eb < EB; eb++)
+#pragma unroll
+          for (int v = 0; v < 16; v++) o[eb][v] *= alpha;
+      }
+      const float neg_m = (m > kNegInf) ? -m : 0.f;
+      float lsum = 0.f;
+#pragma unroll
+      for (int v = 0; v < 16; v++) {
+        const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(s[v], sc, neg_m));  // exp2(-inf) = 0
+        s[v] = p;
+        lsum += p;
+      }
+      l += lsum;
+    };
+
+    const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    f32x16 s[NB];
+    // ---- S^T = K Q^T, operand reads two groups of four instructions ahead (order pinned)
+#pragma unroll
+    for (int jb = 0; jb < NB; jb++) {
+      const char* kb = tb + 32 * jb * ROWB;
+      float4v kx[3];
+      kx[0] = *reinterpret_cast<const float4v*>(kb + kadr[0]);
+      kx[1] = *reinterpret_cast<const float4v*>(kb + kadr[1]);
+      s[jb] = zero16;
+      __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+#pragma unroll
+      for (int g = 0; g < D / 8; g++) {
+        if (g + 2 < D / 8) {
+          kx[(g + 2) % 3] = *reinterpret_cast<const float4v*>(kb + kadr[(g + 2) % 8] + 256 * ((g + 2) / 8));
+          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+          s[jb] = __builtin_amdgcn_mfma_f32_32x32x2f32(kx[g % 3][i], qf[4 * g + i], s[jb], 0, 0, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+      }
+    }
+    // ---- softmax and O^T += V^T P^T per block, V reads PD keys ahead (order pinned)
+    typedef float vecE __attribute__((ext_vector_type(EB)));
+    constexpr int PD = 8 / EB;
+#pragma unroll
+    for (int jb = 0; jb < NB; jb++) {
+      const char* vb = tb + 32 * jb * ROWB;
+      soft(s[jb], jb);
+      __builtin_amdgcn_sched_barrier(0);
+      vecE vx[PD + 1];
+#pragma unroll
+      for (int v = 0; v < PD; v++)
+        vx[v] = *reinterpret_cast<const vecE*>(vb + vadr[v % 8] + 16 * ROWB * (v / 8));
+      __builtin_amdgcn_sched_group_barrier(0x100, PD, 0);
+#pragma unroll
+      for (int v = 0; v < 16; v++) {
+        if (v + PD < 16) {
+          vx[(v + PD) % (PD + 1)] =
+              *reinterpret_cast<const vecE*>(vb + vadr[(v + PD) % 8] + 16 * ROWB * ((v + PD) / 8));
+          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        }
+#pragma unroll
+        for (int eb = 0; eb < EB; eb++)
+          o[eb] = __builtin_amdgcn_mfma_f32_32x32x2f32(vx[v % (PD + 1)][eb], s[jb][v], o[eb], 0, 0, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, EB, 0);
+      }
+    }
+  };
+
+  if (u_lo < u_hi) request(u_lo, lds_even);
+  for (int ut = u_lo; ut < u_hi; ut += 2 * BN) {
+    step(ut, lds_even, lds_odd);
+    if (ut + BN < u_hi) step(ut + BN, lds_odd, lds_even);
+  }
+
+  l += shfl_xor_f32(l, 32);
+  if (q_ok && l > 0.f) {
+    // hand the row over relative to its true maximum: (m, l, o) -> (mt, l * 2^(m - mt), o)
+    const float shrink = __builtin_amdgcn_exp2f(m - mt);
+    tile_write_row<float, D>(a.t, q_tok, h, mt, l * shrink, o, shrink);
+  }
+}
+
 // rows of a block mask that have no live column: out := NaN (m, l untouched)
 template <typename T>
 __global__ void band_dead_rows_kernel(T* out, int64_t n, int d, int64_t block, int64_t s) {
@@ -1144,8 +1410,26 @@ int launch_band_tiles(const TileArgs& a, int use_nan, hipStream_t stream) {
       const int64_t resident = (int64_t)device_cu_count() * 2;
       const int64_t rem = n_all % resident;
       at.n_tail = (4 * rem <= resident) ? rem : 0;
-      const int64_t grid_t = (n_all - at.n_tail + 7) / 8 * 8 + 4 * at.n_tail;
-      hipLaunchKernelGGL((tile_kernel<T, D, kTileBand>), dim3((unsigned)grid_t), dim3(256), 0, stream, at);
+      // whole tiles: loads write LDS directly where a tile's rows can be addressed with 32-bit
+      // offsets and positions fit 32-bit arithmetic; the shared tail tiles go through the
+      // register-staged kernel either way
+      const int64_t max_len = a.block > 0 ? a.cnt : (a.n + a.s - 1) / a.s;
+      const bool dma = a.s * (int64_t)(4 * D) * BandDmaF32Cfg<D>::BN < ((int64_t)1 << 31) &&
+                       (a.w <= (int64_t)0x3fffffff || max_len <= (int64_t)0x3fffffff);
+      const int64_t n_main = n_all - at.n_tail;
+      if (dma) {
+        if (n_main > 0)
+          hipLaunchKernelGGL((band_dma_f32_kernel<D>), dim3((unsigned)((n_main + 7) / 8 * 8)), dim3(256), 0,
+                             stream, at);
+        if (at.n_tail > 0) {
+          at.tail_only = 1;
+          hipLaunchKernelGGL((tile_kernel<T, D, kTileBand>), dim3((unsigned)(4 * at.n_tail)), dim3(256), 0,
+                             stream, at);
+        }
+      } else {
+        const int64_t grid_t = (n_main + 7) / 8 * 8 + 4 * at.n_tail;
+        hipLaunchKernelGGL((tile_kernel<T, D, kTileBand>), dim3((unsigned)grid_t), dim3(256), 0, stream, at);
+      }
     }
     if (timed) (void)hipEventRecord(ev.stop, stream);
   }

@@ -751,6 +751,35 @@ def test_local_2d_dilated(mods, dtype, d, n, block, dil, use_nan):
     check(o, m, l, *ref, dtype, state_dtype=torch.float32, dead_expect="nan" if use_nan else None)
 
 
+@pytest.mark.parametrize("dtype,d", [(torch.float32, 64), (torch.float32, 128), (torch.bfloat16, 64),
+                                     (torch.float16, 128)])
+@pytest.mark.parametrize("kind,n,p1,p2", [("local", 20011, 33, 0), ("local", 20011, 0, 0), ("local", 17000, 700, 0),
+                                          ("d1", 20011, 70, 2), ("d1", 20000, 1500, 1), ("d1", 33333, 129, 4),
+                                          ("d2", 20480, 128, 1), ("d2", 42000, 300, 2), ("d2", 30000, 200, 0)])
+def test_band_masks_with_a_few_hundred_tiles(mods, dtype, d, kind, n, p1, p2):
+    """Band masks with 130 .. 500 query tiles: whole tiles only (the kernels whose loads write LDS directly),
+    sequence ends inside a tile, windows narrower and wider than a tile; then a second call on top of the first."""
+    q, k, v = dev_qkv(n, d, dtype, 41, scale=0.5)
+    m, l, o = state(n, d, dtype, torch.float32)
+    if kind == "local":
+        call = lambda: mods["spfa_local"].forward(q, k, v, m, l, o, p1)
+        ref = c_oracle.local(np64(q), np64(k), np64(v), p1)
+    elif kind == "d1":
+        call = lambda: mods["spfa_local_1d_dilated"].forward(q, k, v, m, l, o, p1, p2)
+        ref = c_oracle.local_1d_dilated(np64(q), np64(k), np64(v), p1, p2)
+    else:
+        call = lambda: mods["spfa_local_2d_dilated"].forward(q, k, v, m, l, o, p1, p2, False)
+        ref = c_oracle.local_2d_dilated(np64(q), np64(k), np64(v), p1, p2, use_nan=False)
+    call()
+    sync()
+    check(o, m, l, *ref, dtype, state_dtype=torch.float32)
+    l1, o1 = l.clone(), o.clone()
+    call()
+    sync()
+    assert torch.allclose(l, 2 * l1, rtol=1e-5)
+    assert torch.allclose(o.float(), o1.float(), atol=2e-5 if dtype == torch.float32 else 2e-2)
+
+
 @pytest.mark.parametrize("dtype,d", [(torch.float32, 64), (torch.bfloat16, 64), (torch.float16, 128),
                                      (torch.float32, 128), (torch.float32, 32)])
 @pytest.mark.parametrize("n,n_globs,w", [(1024, 4, 10), (1024, 1, 0), (1024, 64, 64), (1500, 100, 1499),
