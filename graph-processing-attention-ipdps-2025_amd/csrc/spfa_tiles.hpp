@@ -8,8 +8,8 @@
 // so all three are the same tile problem.  One workgroup (4 wavefronts) owns 128 consecutive
 // query positions, one wavefront 32 of them; keys are streamed in tiles of 64 (32 for fp32 at
 // d = 128) through LDS and shared by the four wavefronts.  tile_kernel stages the tiles through
-// registers (fp32 band masks, every type of the global mask); band_dma_kernel lets the loads
-// write LDS directly (bf16 / fp16 band masks).
+// registers (every type of the global mask, the shared tail tiles of fp32 band masks);
+// band_dma_kernel (bf16 / fp16) and band_dma_f32_kernel let the loads write LDS directly.
 //
 // Everything is computed transposed, S^T = K Q^T and O^T = V^T P^T, with 32x32 MFMA tiles.  In
 // the 32x32 result layout lane (r, h) = (lane % 32, lane / 32) holds column r, rows
