@@ -780,6 +780,20 @@ def test_band_masks_with_a_few_hundred_tiles(mods, dtype, d, kind, n, p1, p2):
     assert torch.allclose(o.float(), o1.float(), atol=2e-5 if dtype == torch.float32 else 2e-2)
 
 
+@pytest.mark.parametrize("dtype,d", [(torch.float32, 64), (torch.float32, 128), (torch.bfloat16, 128)])
+def test_band_masks_batch_with_a_few_hundred_tiles(mods, dtype, d):
+    """Three heads of 9000 tokens in one call: 213 whole tiles over the stacked problems."""
+    n, shape = 9000, (3,)
+    cases = [("spfa_local", (50,), lambda a, b, c: c_oracle.local(a, b, c, 50)),
+             ("spfa_local_1d_dilated", (200, 2), lambda a, b, c: c_oracle.local_1d_dilated(a, b, c, 200, 2)),
+             ("spfa_local_2d_dilated", (250, 1, False), lambda a, b, c: c_oracle.local_2d_dilated(a, b, c, 250, 1, use_nan=False))]
+    for name, args, ref_fn in cases:
+        q, k, v, m, l, o = _stacked(n, d, dtype, shape, 57)
+        mods[name].forward(q, k, v, m, l, o, *args)
+        sync()
+        _check_heads(q, k, v, o, m, l, ref_fn, dtype)
+
+
 @pytest.mark.parametrize("dtype,d", [(torch.float32, 64), (torch.bfloat16, 64), (torch.float16, 128),
                                      (torch.float32, 128), (torch.float32, 32)])
 @pytest.mark.parametrize("n,n_globs,w", [(1024, 4, 10), (1024, 1, 0), (1024, 64, 64), (1500, 100, 1499),
