@@ -116,7 +116,8 @@ def _source_loop_depth(kname: str) -> int:
         # key-tile loop; the global-columns mode (third template argument 2) also loops over
         # query tiles
         return 2 if re.search(r"Li2EEEv", kname) else 1
-    med = "18medium_rows_kernelI" in kname
+    whole = "17whole_rows_kernelI" in kname  # (a medium-row walk inside its loop over long rows)
+    med = "18medium_rows_kernelI" in kname or whole
     if "15segments_kernelI" not in kname and "11rows_kernelI" not in kname and not med:
         return 1
     seg = "15segments_kernelI" in kname
@@ -130,7 +131,7 @@ def _source_loop_depth(kname: str) -> int:
     groups = span // lpr
     unroll = min(unroll, span // groups)
     parts = span // (unroll * groups)
-    return (2 if seg else 1) + (1 if parts > 2 else 0)
+    return (2 if (seg or whole) else 1) + (1 if parts > 2 else 0)
 
 
 def check_loop_nests(workers: int | None = None) -> None:

@@ -525,6 +525,121 @@ __global__ __launch_bounds__(256) void medium_rows_kernel(Tensors t, Mask mask, 
   if (g == 0) finish_row<Lay>(t, row, c, m, l, acc);
 }
 
+// Small problems in one launch: one wavefront per row and problem (empty rows included), eight
+// rows per workgroup.  The general path is five launches and a work list; below a few tens of
+// thousands of rows those cost more than the attention (4096 rows of ~83 entries: 37 us, against
+// 13 us here).  A row of more than kWholeRowsLong candidates is left for a second phase in which
+// the eight wavefronts of the workgroup share it (a contiguous run of candidates each) and fold
+// their partial results through LDS, so that one very long row costs an eighth of what a single
+// wavefront would take.
+constexpr int kWholeRowsWaves = 8;
+constexpr int64_t kWholeRowsLong = 1024;
+
+template <class Lay, class Mask>
+__global__ __launch_bounds__(kWholeRowsWaves* kWave) void whole_rows_kernel(Tensors t, Mask mask, int use_nan) {
+  using T = typename Lay::elem;
+  constexpr int NE = Lay::NE;
+  constexpr int LPR = Lay::LPR;
+  constexpr int W = kWholeRowsWaves;
+  constexpr int DP = NE * LPR;  // padded row length
+  __shared__ float part_acc[W * DP];
+  __shared__ float part_m[W], part_l[W];
+  __shared__ int long_rows[W];
+  __shared__ int n_long_s;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x >> 6;
+  const int g = lane / LPR;
+  const int c = lane % LPR;
+  const int64_t total = t.n_q * t.n_batch;
+  const int64_t row0 = (int64_t)blockIdx.x * W;
+  const float scale = 1.0f / sqrtf((float)t.d);
+  if (threadIdx.x == 0) n_long_s = 0;
+  __syncthreads();
+
+  // the gather over candidates [t0, t1) of row `row`, folded over the groups of the wavefront
+  auto walk = [&](int64_t row, int64_t t0, int64_t t1, float& m, float& l, float (&acc)[NE]) {
+    int64_t b, ri;
+    split_row(t, row, b, ri);
+    const typename Mask::Row rc = mask.row(ri);
+    float q[NE];
+    load_q<Lay>(t, row, c, q);
+    m = kNegInf;
+    l = 0.f;
+#pragma unroll
+    for (int e = 0; e < NE; e++) acc[e] = 0.f;
+    if (t1 > rc.deg) t1 = rc.deg;
+    if (t0 < t1)
+      attend<Lay, Mask, Lay::U_MEDIUM, kWave>(mask, rc, (const T*)t.k + b * t.kv_stride,
+                                              (const T*)t.v + b * t.kv_stride, t.d, scale, q, t0, t1, lane,
+                                              m, l, acc);
+#pragma unroll
+    for (int off = LPR; off < kWave; off <<= 1) {
+      float m2 = shfl_xor_f32(m, off);
+      float l2 = shfl_xor_f32(l, off);
+      float acc2[NE];
+#pragma unroll
+      for (int e = 0; e < NE; e++) acc2[e] = shfl_xor_f32(acc[e], off);
+      merge_partial<NE>(m, l, acc, m2, l2, acc2);
+    }
+  };
+
+  // ---- phase 1: a wavefront per row
+  {
+    const int64_t row = row0 + wave;
+    if (row < total) {
+      int64_t b, ri;
+      split_row(t, row, b, ri);
+      const int64_t deg = mask.row(ri).deg;
+      if (deg <= 0) {
+        if (use_nan && g == 0) {
+          float nanv[NE];
+#pragma unroll
+          for (int e = 0; e < NE; e++) nanv[e] = __builtin_nanf("");
+          Lay::store((T*)t.out + row * t.d, c, t.d, nanv);
+        }
+      } else if (deg > kWholeRowsLong) {
+        if (lane == 0) long_rows[atomicAdd(&n_long_s, 1)] = wave;
+      } else {
+        float m, l, acc[NE];
+        walk(row, 0, deg, m, l, acc);
+        if (g == 0) finish_row<Lay>(t, row, c, m, l, acc);
+      }
+    }
+  }
+  __syncthreads();
+
+  // ---- phase 2: the workgroup's long rows, one after the other, shared by all wavefronts
+  const int n_long = n_long_s;
+  for (int i = 0; i < n_long; i++) {
+    const int64_t row = row0 + long_rows[i];
+    int64_t b, ri;
+    split_row(t, row, b, ri);
+    const int64_t deg = mask.row(ri).deg;
+    int64_t per = (deg + W - 1) / W;
+    per = (per + kWave - 1) / kWave * kWave;
+    float m, l, acc[NE];
+    walk(row, wave * per, (wave + 1) * per, m, l, acc);
+    if (g == 0) {
+      Lay::store_f32(part_acc + wave * DP, c, t.d, acc);
+      if (c == 0) {
+        part_m[wave] = m;
+        part_l[wave] = l;
+      }
+    }
+    __syncthreads();
+    if (wave == 0 && g == 0) {
+      // (wavefront 0 still holds its own partial in registers)
+      for (int w2 = 1; w2 < W; w2++) {
+        float acc2[NE];
+        Lay::load_f32(part_acc + w2 * DP, c, t.d, acc2);
+        merge_partial<NE>(m, l, acc, part_m[w2], part_l[w2], acc2);
+      }
+      finish_row<Lay>(t, row, c, m, l, acc);
+    }
+    __syncthreads();
+  }
+}
+
 template <class Lay>
 __global__ __launch_bounds__(256) void merge_kernel(Tensors t, Plan plan) {
   constexpr int NE = Lay::NE;
@@ -621,6 +736,15 @@ struct KernelEvents {
 KernelEvents& kernel_events();
 
 constexpr int kSegmentWorkgroupsPerCu = 1;
+// whole_rows_kernel takes a call of at most this many rows (over all problems), keys and
+// candidates.  What it cannot do is share one very long row over the device, so the limits keep
+// such a row short: K and V of 16384 keys stay in the caches, a row of distinct columns is at
+// most 16384 long (8 wavefronts x 32 trips); only repeated columns can make a row longer, up to
+// all the candidates (measured: 500 K candidates in one row of 64, K and V of 512 K rows, 4.8 ms
+// here against 1.5 ms on the general path - hence the limit on keys).
+constexpr int64_t kWholeRowsMaxRows = 16384;
+constexpr int64_t kWholeRowsMaxKeys = 16384;
+constexpr int64_t kWholeRowsMaxEntries = (int64_t)1 << 19;
 
 // compute units of the current device (looked up once per device)
 inline int device_cu_count() {
@@ -668,6 +792,17 @@ int launch_engine(const Tensors& t, const Mask& mask, const EngineSizing& s, int
   if (t.n_q == 0) return 0;
 
   const bool has_long = s.max_deg > s.short_max;
+  const KernelEvents ev = kernel_events();
+  const bool timed = ev.start != nullptr && ev.stop != nullptr;
+  if (has_long && phase == kEngineAll && t.n_q * t.n_batch <= kWholeRowsMaxRows &&
+      t.kv_stride <= kWholeRowsMaxKeys * (int64_t)t.d && s.nnz_bound <= kWholeRowsMaxEntries) {
+    const int64_t grid = (t.n_q * t.n_batch + kWholeRowsWaves - 1) / kWholeRowsWaves;
+    if (timed) (void)hipEventRecord(ev.start, stream);
+    hipLaunchKernelGGL((whole_rows_kernel<Lay, Mask>), dim3((unsigned)grid), dim3(kWholeRowsWaves * kWave), 0,
+                       stream, t, mask, use_nan);
+    if (timed) (void)hipEventRecord(ev.stop, stream);
+    return hipGetLastError() == hipSuccess ? 0 : 4;
+  }
   if (has_long && phase != kEngineRunOnly) {
     hipLaunchKernelGGL(reset_counters_kernel, dim3(1), dim3(64), 0, stream, plan.cnt);
     hipLaunchKernelGGL((plan_kernel<Mask>), dim3((unsigned)((t.n_q + kPlanThreads - 1) / kPlanThreads)),
@@ -677,8 +812,6 @@ int launch_engine(const Tensors& t, const Mask& mask, const EngineSizing& s, int
   if (has_long && phase == kEngineRunOnly)
     hipLaunchKernelGGL(reset_cursor_kernel, dim3(1), dim3(64), 0, stream, plan.cursor);
 
-  const KernelEvents ev = kernel_events();
-  const bool timed = ev.start != nullptr && ev.stop != nullptr;
   const int64_t rows_per_wg = 4 * Lay::GROUPS;
   const int64_t grid1 = (t.n_q * t.n_batch + rows_per_wg - 1) / rows_per_wg;
   if (timed && !has_long) (void)hipEventRecord(ev.start, stream);

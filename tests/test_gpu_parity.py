@@ -42,10 +42,28 @@ def run_csr(mods, q, k, v, ro, ci, use_nan, st=None, off_dtype=torch.uint64, col
     m, l, o = st if st is not None else state(n, d, q.dtype, state_dtype)
     ro_t, ci_t = csr_tensors(ro, ci, off_dtype, col_dtype)
     val = torch.ones(ci_t.numel(), device=DEV, dtype=q.dtype)
+    fresh = st is None
     ret = mods["spfa_csr"].forward(q, k, v, ro_t, ci_t, val, m, l, o, use_nan)
     sync()
     assert ret.data_ptr() == o.data_ptr()
+    if fresh and q.dim() == 2:
+        # Small problems take a single-launch path in a plain call; a planned call always takes the
+        # general one (work list, short / medium / segmented rows).  Both must agree.
+        m2, l2, o2 = state(n, d, q.dtype, state_dtype)
+        plan = mods["spfa_csr"].plan(ro_t, ci_t)
+        mods["spfa_csr"].forward_planned(q, k, v, ro_t, ci_t, val, m2, l2, o2, use_nan, plan)
+        sync()
+        tol = 2e-5 if q.dtype in (torch.float32, torch.float64) else 2e-2
+        assert torch.allclose(torch.nan_to_num(o).float(), torch.nan_to_num(o2).float(), atol=tol)
+        assert torch.equal(torch.isnan(o), torch.isnan(o2))
+        assert torch.allclose(lse_t(m, l), lse_t(m2, l2), atol=1e-3 if tol > 1e-3 else 1e-5, equal_nan=True)
     return o, m, l
+
+
+def lse_t(m, l):
+    with torch.no_grad():
+        x = m.float() + torch.log(l.float())
+    return torch.where(l.float() > 0, x, torch.zeros_like(x))
 
 
 # ------------------------------------------------------------------ the reference's own checks
@@ -226,6 +244,24 @@ def test_csr_row_lengths_around_every_threshold(mods, dtype, d):
     lengths = [0, 1, 2, 31, 32, 33, 63, 64, 65, 255, 256, 257, 511, 512, 513, 768, 1024, 2048, 0, 7]
     ro, ci = _special_rows_csr(n, rng, lengths)
     q, k, v = dev_qkv(n, d, dtype, 21)
+    o, m, l = run_csr(mods, q, k, v, ro, ci, True, state_dtype=torch.float32)
+    ref = c_oracle.csr(np64(q), np64(k), np64(v), ro, ci, use_nan=True)
+    check(o, m, l, *ref, dtype, state_dtype=torch.float32, dead_expect="nan")
+
+
+@pytest.mark.parametrize("dtype,d", [(torch.float32, 64), (torch.bfloat16, 128), (torch.float32, 200)])
+def test_csr_small_problem_with_very_long_rows(mods, dtype, d):
+    """Few rows, some of them longer than the single-launch path gives one wavefront: whole key range, repeated
+    columns, lengths around the hand-over."""
+    n_q, n_k = 37, 8192
+    rng = np.random.default_rng(77)
+    lengths = [8192, 0, 2048, 2049, 5000, 3, 12000, 1, 2047, 4097] + [int(x) for x in rng.integers(0, 40, n_q - 10)]
+    cols, off = [], [0]
+    for ln in lengths:
+        cols.append(rng.integers(0, n_k, ln) if ln > n_k else rng.choice(n_k, ln, replace=False))
+        off.append(off[-1] + ln)
+    ro, ci = np.array(off, np.int64), np.concatenate(cols).astype(np.int64)
+    q, k, v = dev_qkv(n_q, d, dtype, 78, n_k=n_k)
     o, m, l = run_csr(mods, q, k, v, ro, ci, True, state_dtype=torch.float32)
     ref = c_oracle.csr(np64(q), np64(k), np64(v), ro, ci, use_nan=True)
     check(o, m, l, *ref, dtype, state_dtype=torch.float32, dead_expect="nan")
