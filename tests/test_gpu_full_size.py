@@ -311,6 +311,50 @@ def test_backward_local_n65536(mods, dtype):
         1e-4 if dtype == torch.float32 else 0.3)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("kind", ["d1", "d2"])
+def test_backward_dilated_d128(mods, kind, dtype):
+    """Gradient tiles at d = 128 (one workgroup per CU, accumulators beyond 256 registers) on a few hundred tiles:
+    sampled dQ rows against the oracle, dK / dV of sampled columns from the forward pass's own statistics in float64
+    (the masks are symmetric: the rows that attend column j are live(j)), and the two identities."""
+    d = 128
+    if kind == "d1":
+        n, w, dil = 40000, 200, 2
+        fwd = lambda *a: mods["spfa_local_1d_dilated"].forward(*a, w, dil)
+        bwd = lambda q, k, v, m, l, o, *g: mods["spfa_local_1d_dilated"].backward(q, k, v, m, l, o, w, dil, *g)
+        live = lambda i: so.live_local_1d_dilated(n, w, dil, i)
+    else:
+        n, block, dil = 40000, 400, 1
+        fwd = lambda *a: mods["spfa_local_2d_dilated"].forward(*a, block, dil, False)
+        bwd = lambda q, k, v, m, l, o, *g: mods["spfa_local_2d_dilated"].backward(q, k, v, m, l, o, block, dil, *g)
+        live = lambda i: so.live_local_2d_dilated(n, block, dil, i)
+    q, k, v = syn.qkv(n, d, dtype=dtype, device=DEV, seed=2, scale=0.5)
+    m, l, o = syn.fresh_state(n, d, dtype=dtype, device=DEV, state_dtype=torch.float32)
+    fwd(q, k, v, m, l, o)
+    d_out = torch.randn(n, d, device=DEV, generator=torch.Generator(device=DEV).manual_seed(12)).to(dtype)
+    dq, dk, dv = (torch.zeros(n, d, device=DEV) for _ in range(3))
+    bwd(q, k, v, m, l, o, d_out, dq, dk, dv)
+    torch.cuda.synchronize()
+    _grad_properties(q, k, v, d_out, l, dq, dk, dv, dtype)
+    rows = np.concatenate([[0, 2, 3, n - 3, n - 1], rand_rows(n, 40, 13)])
+    rows = np.asarray([i for i in rows if len(live(int(i)))])
+    _dq_sample_check(q, k, v, d_out, dq, rows, live, dtype)
+    lse = m.double() + l.double().log()
+    delta = (d_out.double() * o.double()).sum(dim=1)
+    tol = 2e-4 if dtype == torch.float32 else 3e-2
+    for j in rand_rows(n, 10, 14):
+        att = torch.as_tensor(np.asarray(live(int(j)), dtype=np.int64)).to(DEV)
+        if att.numel() == 0:
+            assert float(dk[j].abs().max()) == 0 and float(dv[j].abs().max()) == 0
+            continue
+        sco = (q[att].double() @ k[j].double()) / math.sqrt(d)
+        pw = torch.exp(sco - lse[att])
+        ds = pw * (d_out[att].double() @ v[j].double() - delta[att]) / math.sqrt(d)
+        want_v, want_k = pw @ d_out[att].double(), ds @ q[att].double()
+        assert float((dv[j].double() - want_v).abs().max()) <= tol * max(1.0, float(want_v.abs().max()))
+        assert float((dk[j].double() - want_k).abs().max()) <= tol * max(1.0, float(want_k.abs().max()))
+
+
 def test_backward_global_no_local_n1m(mods):
     n, d, g, w = 1 << 20, 64, 64, 64
     q, k, v = syn.qkv(n, d, device=DEV, seed=0)
