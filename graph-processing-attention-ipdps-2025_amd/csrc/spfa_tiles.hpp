@@ -8,8 +8,9 @@
 // so all three are the same tile problem.  One workgroup (4 wavefronts) owns 128 consecutive
 // query positions, one wavefront 32 of them; keys are streamed in tiles of 64 (32 for fp32 at
 // d = 128) through LDS and shared by the four wavefronts.  tile_kernel stages the tiles through
-// registers (every type of the global mask, the shared tail tiles of fp32 band masks);
-// band_dma_kernel (bf16 / fp16) and band_dma_f32_kernel let the loads write LDS directly.
+// registers (every type of the global mask; band masks only when a tile's rows are too far apart
+// for 32-bit offsets); band_dma_kernel (bf16 / fp16) and band_dma_f32_kernel let the loads write
+// LDS directly.
 //
 // Everything is computed transposed, S^T = K Q^T and O^T = V^T P^T, with 32x32 MFMA tiles.  In
 // the 32x32 result layout lane (r, h) = (lane % 32, lane / 32) holds column r, rows
@@ -60,7 +61,6 @@ struct TileArgs {
   int64_t n_tail;         // band: the last n_tail tiles (over all problems) are each shared by four
                           // workgroups of 32 queries whose wavefronts deal the key blocks among
                           // themselves; they fill the last, partly empty round of the grid
-  int32_t tail_only;      // band: the launch holds the shared tail tiles only
   // global modes
   const int32_t* globs;   // listed global tokens (keys of GlobalCols)
   int64_t n_globs;
@@ -239,10 +239,7 @@ __global__ __launch_bounds__(256, 2) void tile_kernel(TileArgs a) {
     const int64_t n_main = n_all - a.n_tail;
     const int64_t per_xcd = (n_main + 7) / 8;
     int64_t lt;
-    if (a.tail_only) {
-      lt = n_main + blockIdx.x / 4;
-      quarter = (int)(blockIdx.x & 3);
-    } else if ((int64_t)blockIdx.x < 8 * per_xcd) {
+    if ((int64_t)blockIdx.x < 8 * per_xcd) {
       lt = (int64_t)(blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
       if (lt >= n_main) return;
     } else {
@@ -1066,11 +1063,20 @@ __global__ __launch_bounds__(256, 2) void band_dma_f32_kernel(TileArgs a) {
   __shared__ __attribute__((aligned(1024))) char lds_odd[BUF_B];
 
   auto uni = [](int x) { return __builtin_amdgcn_readfirstlane(x); };
-  // the whole tiles of the list (the shared tail tiles have a launch of their own)
+  // whole tiles first (a contiguous run per XCD), then four workgroups for each shared tail tile
   const int64_t n_main = a.n_tiles * a.t.n_batch - a.n_tail;
   const int64_t per_xcd = (n_main + 7) / 8;
-  int64_t lt = (int64_t)(blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
-  if (lt >= n_main) return;
+  int64_t lt;
+  int quarter = -1;  // which 32 queries of a shared tail tile (-1: a whole tile)
+  if ((int64_t)blockIdx.x < 8 * per_xcd) {
+    lt = (int64_t)(blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+    if (lt >= n_main) return;
+  } else {
+    const int64_t qid = (int64_t)blockIdx.x - 8 * per_xcd;
+    lt = n_main + qid / 4;
+    quarter = uni((int)(qid & 3));
+  }
+  const bool quad = quarter >= 0;
   const int64_t bb = lt / a.n_tiles;
   lt -= bb * a.n_tiles;
   const int64_t sub = lt / a.tiles_per_sub;
@@ -1085,10 +1091,13 @@ __global__ __launch_bounds__(256, 2) void band_dma_f32_kernel(TileArgs a) {
     qlen = uni((int)((a.n - sub + a.s - 1) / a.s));
   }
   const int wlim = (int)(a.w < (int64_t)0x3fffffff ? a.w : (int64_t)0x3fffffff);  // window, clamped
-  const int t0 = tile * BM;
+  // a shared tail tile: this workgroup has 32 of its queries, all four wavefronts work on them
+  // and take the key tiles in turn
+  const int t0 = tile * BM + (quad ? 32 * quarter : 0);
+  const int qspan = quad ? 32 : BM;
   if (t0 >= qlen) return;
   const int u_lo = t0 > wlim ? t0 - wlim : 0;
-  const int u_hi = (qlen - BM - wlim > t0) ? t0 + BM + wlim : qlen;
+  const int u_hi = (qlen - qspan - wlim > t0) ? t0 + qspan + wlim : qlen;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -1098,7 +1107,7 @@ __global__ __launch_bounds__(256, 2) void band_dma_f32_kernel(TileArgs a) {
   const char* Vp = (const char*)a.t.v;
   const float sc = 1.4426950408889634f / sqrtf((float)D);
 
-  const int tw0 = t0 + 32 * wave;  // first query of this wavefront
+  const int tw0 = t0 + (quad ? 0 : 32 * wave);  // first query of this wavefront
   const int tq = tw0 + r;          // this lane's query position
   const bool q_ok = tq < qlen;
   const int64_t q_tok = base + (int64_t)(q_ok ? tq : qlen - 1) * a.s;
@@ -1182,7 +1191,8 @@ __global__ __launch_bounds__(256, 2) void band_dma_f32_kernel(TileArgs a) {
     if (ut + BN < u_hi) request(ut + BN, other);
 
     const bool all_full = (ut + BN <= u_hi) && (ut >= tw0 + 31 - wlim) && (ut + BN - 1 - wlim <= tw0);
-    const bool none = (tw0 >= qlen) || (ut - wlim > tw0 + 31) || (ut + BN - 1 < tw0 - wlim);
+    const bool none = (tw0 >= qlen) || (ut - wlim > tw0 + 31) || (ut + BN - 1 < tw0 - wlim) ||
+                      (quad && (((ut - u_lo) / BN) & 3) != wave);
     if (none) return;
 
     // key slot j of the tile is live for this lane's query iff jlo <= j <= jhi; the slots this
@@ -1289,6 +1299,45 @@ __global__ __launch_bounds__(256, 2) void band_dma_f32_kernel(TileArgs a) {
   }
 
   l += shfl_xor_f32(l, 32);
+  if (quad) {
+    // fold the four wavefronts (same queries, different key tiles) through LDS, 2, 3 into 0, 1
+    // and then 1 into 0; the tile buffers are no longer needed
+    constexpr int XR = EB * 16 + 3;
+    static_assert(XR * kWave * 4 <= BUF_B, "exchange area does not fit a tile buffer");
+    for (int step = 2; step >= 1; step >>= 1) {
+      const bool gives = wave >= step && wave < 2 * step;
+      const bool takes = wave < step;
+      // (one exchange slot in each of the two buffers)
+      float* xs = reinterpret_cast<float*>((gives ? wave - step : wave) ? lds_odd : lds_even) + lane;
+      __builtin_amdgcn_s_waitcnt(0);
+      __syncthreads();
+      if (gives) {
+#pragma unroll
+        for (int eb = 0; eb < EB; eb++)
+#pragma unroll
+          for (int v = 0; v < 16; v++) xs[(eb * 16 + v) * kWave] = o[eb][v];
+        xs[(EB * 16) * kWave] = m;
+        xs[(EB * 16 + 1) * kWave] = l;
+        xs[(EB * 16 + 2) * kWave] = mt;
+      }
+      __syncthreads();
+      if (takes) {
+        const float m2 = xs[(EB * 16) * kWave], l2 = xs[(EB * 16 + 1) * kWave];
+        mt = fmaxf(mt, xs[(EB * 16 + 2) * kWave]);
+        const float m_new = fmaxf(m, m2);
+        if (m_new > kNegInf) {
+          const float fa = __builtin_amdgcn_exp2f(m - m_new), fb = __builtin_amdgcn_exp2f(m2 - m_new);
+          l = l * fa + l2 * fb;
+#pragma unroll
+          for (int eb = 0; eb < EB; eb++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) o[eb][v] = o[eb][v] * fa + xs[(eb * 16 + v) * kWave] * fb;
+          m = m_new;
+        }
+      }
+    }
+    if (wave != 0) return;
+  }
   if (q_ok && l > 0.f) {
     // hand the row over relative to its true maximum: (m, l, o) -> (mt, l * 2^(m - mt), o)
     const float shrink = __builtin_amdgcn_exp2f(m - mt);
@@ -1410,22 +1459,15 @@ int launch_band_tiles(const TileArgs& a, int use_nan, hipStream_t stream) {
       const int64_t resident = (int64_t)device_cu_count() * 2;
       const int64_t rem = n_all % resident;
       at.n_tail = (4 * rem <= resident) ? rem : 0;
-      // whole tiles: loads write LDS directly where a tile's rows can be addressed with 32-bit
-      // offsets and positions fit 32-bit arithmetic; the shared tail tiles go through the
-      // register-staged kernel either way
+      // loads write LDS directly where a tile's rows can be addressed with 32-bit offsets and
+      // positions fit 32-bit arithmetic
       const int64_t max_len = a.block > 0 ? a.cnt : (a.n + a.s - 1) / a.s;
       const bool dma = a.s * (int64_t)(4 * D) * BandDmaF32Cfg<D>::BN < ((int64_t)1 << 31) &&
                        (a.w <= (int64_t)0x3fffffff || max_len <= (int64_t)0x3fffffff);
       const int64_t n_main = n_all - at.n_tail;
       if (dma) {
-        if (n_main > 0)
-          hipLaunchKernelGGL((band_dma_f32_kernel<D>), dim3((unsigned)((n_main + 7) / 8 * 8)), dim3(256), 0,
-                             stream, at);
-        if (at.n_tail > 0) {
-          at.tail_only = 1;
-          hipLaunchKernelGGL((tile_kernel<T, D, kTileBand>), dim3((unsigned)(4 * at.n_tail)), dim3(256), 0,
-                             stream, at);
-        }
+        const int64_t grid_d = (n_main + 7) / 8 * 8 + 4 * at.n_tail;
+        hipLaunchKernelGGL((band_dma_f32_kernel<D>), dim3((unsigned)grid_d), dim3(256), 0, stream, at);
       } else {
         const int64_t grid_t = (n_main + 7) / 8 * 8 + 4 * at.n_tail;
         hipLaunchKernelGGL((tile_kernel<T, D, kTileBand>), dim3((unsigned)grid_t), dim3(256), 0, stream, at);
