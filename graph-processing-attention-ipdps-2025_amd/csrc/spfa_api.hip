@@ -329,6 +329,9 @@ const char* spfa_status_string(int status) {
     case SPFA_ERR_BLOCK_DILATION: return "The dilation factor must be less than the block/window size.";
     case SPFA_ERR_GLOBAL_COUNT:
       return "There are either no global tokens provided or there are more than the sequence length given.";
+    case SPFA_ERR_STATIC_LIMIT:
+      return "spfa: the mask needs more scratch than the library's static buffer "
+             "(SPFA_STATIC_SCRATCH_BYTES) holds; use spfa_csr_forward with a workspace";
   }
   return "spfa: unknown status";
 }

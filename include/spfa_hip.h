@@ -59,7 +59,9 @@ enum {
   SPFA_ERR_DILATION_NEG = 7,  /* sp_flatt_local_1d_dilated_kernel.cu:259-261 */
   SPFA_ERR_BLOCK_DIVISOR = 8, /* sp_flatt_local_2d_dilated_kernel.cu:274-276 */
   SPFA_ERR_BLOCK_DILATION = 9,/* sp_flatt_local_2d_dilated_kernel.cu:284-286 */
-  SPFA_ERR_GLOBAL_COUNT = 10  /* sp_flatt_global_no_local_kernel.cu:325-327 */
+  SPFA_ERR_GLOBAL_COUNT = 10, /* sp_flatt_global_no_local_kernel.cu:325-327 */
+  SPFA_ERR_STATIC_LIMIT = 11  /* spfa_csr_forward_static: the mask needs more scratch than
+                                 SPFA_STATIC_SCRATCH_BYTES */
 };
 
 typedef struct spfa_problem {
@@ -105,6 +107,23 @@ size_t spfa_csr_workspace_bytes(int64_t n_q, int64_t nnz, int64_t d, int dtype);
 int spfa_csr_forward(const spfa_problem_t* p, const void* row_off, int row_off_bytes,
                      const void* col_ind, int64_t nnz, int use_nan, void* workspace,
                      size_t workspace_bytes, void* stream);
+
+/* spfa_csr_forward without a workspace argument and without any allocation.  No counterpart in
+ * the reference (its kernel needs no scratch, sp_flatt_csr_kernel.cu:271-287); it is for callers
+ * that cannot allocate device memory: code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc.  Same arguments, checks, kernels and results as
+ * spfa_csr_forward; the scratch is a device array of SPFA_STATIC_SCRATCH_BYTES bytes inside the
+ * library (one per device, held until the process ends), and a call calls neither hipMalloc nor
+ * hipFree nor any allocating routine.
+ *   - Limit: n_batch * spfa_csr_workspace_bytes(n_q, nnz, d, dtype) <= SPFA_STATIC_SCRATCH_BYTES,
+ *     else SPFA_ERR_STATIC_LIMIT and nothing is enqueued (16 MiB holds a mask of 131072 rows and
+ *     12.8 M entries at d = 64).
+ *   - All calls on one device share that device's array: calls that overlap in time on one
+ *     device (two streams, two host threads) race; calls in stream order do not.  Nothing needs
+ *     clearing between calls. */
+#define SPFA_STATIC_SCRATCH_BYTES (16u << 20)
+int spfa_csr_forward_static(const spfa_problem_t* p, const void* row_off, int row_off_bytes,
+                            const void* col_ind, int64_t nnz, int use_nan, void* stream);
 
 /* COO: row i attends {col_ind[e] : row_ind[e] == i}.  Entries may come in any order (the
  * reference needs them sorted by row, sp_flatt_coo_kernel.cu:47-79); they are bucketed by

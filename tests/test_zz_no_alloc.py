@@ -1,0 +1,132 @@
+"""spfa_csr_forward_static (the CSR call whose scratch is a device array inside the library) against
+spfa_csr_forward, both through the C ABI with ctypes: two calls in a row, the second on a smaller
+mask, plus the limit check.  Collected last (file name) so that a failure here hides nothing."""
+import ctypes
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import spfa_synth as syn
+from helpers import OUT_TOL, lse, np64, oracle_rows
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+LIB = os.path.join(ROOT, "graph-processing-attention-ipdps-2025_amd", "libspfa_hip.so")
+STATIC_BYTES = 16 << 20  # SPFA_STATIC_SCRATCH_BYTES of include/spfa_hip.h
+SPFA_ERR_STATIC_LIMIT = 11
+
+
+class Problem(ctypes.Structure):
+    _fields_ = [("q", ctypes.c_void_p), ("k", ctypes.c_void_p), ("v", ctypes.c_void_p),
+                ("m", ctypes.c_void_p), ("l", ctypes.c_void_p), ("out", ctypes.c_void_p),
+                ("n_q", ctypes.c_int64), ("n_k", ctypes.c_int64), ("d", ctypes.c_int64),
+                ("dtype", ctypes.c_int32), ("state_dtype", ctypes.c_int32), ("n_batch", ctypes.c_int64)]
+
+
+@pytest.fixture(scope="module")
+def lib():
+    L = ctypes.CDLL(LIB)
+    L.spfa_csr_workspace_bytes.restype = ctypes.c_size_t
+    L.spfa_csr_workspace_bytes.argtypes = [ctypes.c_int64, ctypes.c_int64, ctypes.c_int64, ctypes.c_int]
+    L.spfa_csr_forward.argtypes = [ctypes.POINTER(Problem), ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p,
+                                   ctypes.c_int64, ctypes.c_int, ctypes.c_void_p, ctypes.c_size_t,
+                                   ctypes.c_void_p]
+    L.spfa_csr_forward_static.argtypes = [ctypes.POINTER(Problem), ctypes.c_void_p, ctypes.c_int,
+                                          ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_void_p]
+    return L
+
+
+def test_header_and_test_agree_on_the_limit():
+    text = open(os.path.join(ROOT, "include", "spfa_hip.h")).read()
+    assert "#define SPFA_STATIC_SCRATCH_BYTES (16u << 20)" in text
+    assert "SPFA_ERR_STATIC_LIMIT = 11" in text
+
+
+def _problem(q, k, v, state):
+    m, l, out = state
+    n, d = q.shape
+    return Problem(q.data_ptr(), k.data_ptr(), v.data_ptr(), m.data_ptr(), l.data_ptr(), out.data_ptr(),
+                   n, k.shape[0], d, 0, 0, 1)
+
+
+def _run_both(lib, n, d, kmax, seed, use_nan):
+    dev = "cuda:0"
+    q, k, v = syn.qkv(n, d, device=dev, seed=seed)
+    ro, ci = syn.zipf_csr(n, 1.5, 1, kmax, device=dev, seed=seed)
+    # a few empty rows, so that the NaN / untouched rule is exercised too
+    deg = (ro[1:] - ro[:-1]).clone()
+    keep = torch.ones(ci.numel(), dtype=torch.bool, device=dev)
+    for r in (3, n // 2, n - 1):
+        keep[int(ro[r]):int(ro[r + 1])] = False
+        deg[r] = 0
+    ci = ci[keep].contiguous()
+    ro = torch.zeros(n + 1, dtype=torch.int64, device=dev)
+    ro[1:] = torch.cumsum(deg, 0)
+    nnz = ci.numel()
+    ro32, ci32 = ro.to(torch.int32), ci.to(torch.int32)
+    stream = torch.cuda.current_stream().cuda_stream
+
+    need = lib.spfa_csr_workspace_bytes(n, nnz, d, 0)
+    assert 0 < need <= STATIC_BYTES
+    ws = torch.empty(need + 256, dtype=torch.uint8, device=dev)
+    ws_ptr = (ws.data_ptr() + 255) // 256 * 256
+    ref = syn.fresh_state(n, d, device=dev)
+    p = _problem(q, k, v, ref)
+    rc = lib.spfa_csr_forward(ctypes.byref(p), ro32.data_ptr(), 4, ci32.data_ptr(), nnz, use_nan, ws_ptr,
+                              need, stream)
+    assert rc == 0
+
+    got = syn.fresh_state(n, d, device=dev)
+    p = _problem(q, k, v, got)
+    torch.cuda.synchronize()
+    before = torch.cuda.memory_allocated()
+    rc = lib.spfa_csr_forward_static(ctypes.byref(p), ro32.data_ptr(), 4, ci32.data_ptr(), nnz, use_nan,
+                                     stream)
+    assert rc == 0
+    torch.cuda.synchronize()
+    assert torch.cuda.memory_allocated() == before
+
+    # the same kernels on the same inputs: identical results, NaN rows included
+    for a, b, name in zip(got, ref, ("m", "l", "out")):
+        assert torch.equal(torch.nan_to_num(a, nan=12345.0), torch.nan_to_num(b, nan=12345.0)), name
+    dead = torch.tensor([3, n // 2, n - 1], device=dev)
+    if use_nan:
+        assert torch.isnan(got[2][dead]).all()
+    else:
+        assert (got[2][dead] == 0).all()
+    assert (got[1][dead] == 0).all()
+
+    # and both agree with the float64 oracle on a sample of rows
+    rows = np.unique(np.concatenate([np.random.default_rng(seed).integers(0, n, 48),
+                                     [0, 1, n - 2, int(torch.argmax(deg))]]))
+    rows = rows[deg.cpu().numpy()[rows] > 0]
+    ro_n, ci_n = ro.cpu().numpy(), ci.cpu().numpy()
+    ref_out, ref_m, ref_l = oracle_rows(q, k, v, rows, lambda i: ci_n[ro_n[i]:ro_n[i + 1]])
+    err = np.abs(np64(got[2])[rows] - ref_out).max()
+    assert err <= OUT_TOL[torch.float32], err
+    lerr = np.abs(lse(np64(got[0])[rows], np64(got[1])[rows]) - lse(ref_m, ref_l)).max()
+    assert lerr <= 1e-4, lerr
+
+
+@pytest.mark.gpu
+def test_static_entry_matches_workspace_entry_twice_in_a_row(lib):
+    # long rows (segments and merges: every region of the scratch is used), then a smaller
+    # problem that reuses the array with the first call's contents still in it
+    _run_both(lib, 40000, 64, 4096, seed=11, use_nan=1)
+    _run_both(lib, 20000, 64, 2048, seed=12, use_nan=0)
+
+
+@pytest.mark.gpu
+def test_static_entry_rejects_masks_beyond_its_buffer(lib):
+    dev = "cuda:0"
+    n, d = 64, 64
+    q, k, v = syn.qkv(n, d, device=dev, seed=1)
+    st = syn.fresh_state(n, d, device=dev)
+    p = _problem(q, k, v, st)
+    nnz = 1 << 30  # sizes only: the call must return before it reads a pointer
+    assert lib.spfa_csr_workspace_bytes(n, nnz, d, 0) > STATIC_BYTES
+    rc = lib.spfa_csr_forward_static(ctypes.byref(p), None, 4, None, nnz, 0, None)
+    assert rc == SPFA_ERR_STATIC_LIMIT
+    torch.cuda.synchronize()
+    assert torch.isinf(st[0]).all() and (st[1] == 0).all()
