@@ -110,6 +110,9 @@ def make_workload(name, dtype, torch, syn, inline_limit=32, planned=False, heads
                 w["call"] = lambda st: spfa_coo.forward(q, k, v, r_t, c_t, val, st[0], st[1], st[2], False)
             w["csr"] = None
             w["coo"] = (r, c)
+            # the columns in the order the attention kernel walks them (row by row)
+            w["probe_idx"] = c[torch.argsort(r, stable=True)].to(torch.int32).contiguous()
+            w["probe_sorted_rows"] = True
             off_b = 8
         else:
             import spfa_csr
@@ -135,6 +138,7 @@ def make_workload(name, dtype, torch, syn, inline_limit=32, planned=False, heads
                         spfa_csr.forward(q[h], k[h], v[h], ro_t, ci_t, val, st[0][h], st[1][h], st[2][h], False)
                 w["call"] = looped
             w["csr"] = (ro, ci)
+            w["probe_idx"] = ci.to(torch.int32).contiguous()
             off_b = 8
         gathered, total = syn.explicit_mask_bytes(nnz, n, d, es, off_bytes=off_b)
         if name.startswith("coo"):
@@ -145,6 +149,8 @@ def make_workload(name, dtype, torch, syn, inline_limit=32, planned=False, heads
         # the dominant (segment) kernel owns the rows longer than the library's in-place limit
         long_rows = deg > inline_limit
         nnz_long, rows_long = int(deg[long_rows].sum()), int(long_rows.sum())
+        if nnz_long > 0:  # the ceiling probe walks what the segment kernel walks: the long rows' columns
+            w["probe_idx"] = w["probe_idx"][torch.repeat_interleave(long_rows, deg)].contiguous()
         _, kernel_bytes = syn.explicit_mask_bytes(nnz_long, rows_long, d, es, off_bytes=off_b)
         w.update(n=n, d=d, nnz=nnz * heads, bytes_total=total * heads, bytes_gathered=gathered * heads,
                  bound="hbm", kernel_bytes=kernel_bytes * heads, kernel_nnz=nnz_long * heads,
@@ -230,6 +236,7 @@ def make_workload(name, dtype, torch, syn, inline_limit=32, planned=False, heads
             w["params"] = {"n_globals": g, "LOCAL_SIZE": wsz, "csr_nnz": nnz_csr}
             w["globs"] = globs
             w["csr"] = (ro, ci)
+            w["probe_idx"] = ci.to(torch.int32).contiguous()
             w["whole_call"] = True
             live = n
             w["extra_bytes"] = syn.explicit_mask_bytes(nnz_csr, n, d, es, off_bytes=8)[1]
@@ -255,6 +262,49 @@ def make_workload(name, dtype, torch, syn, inline_limit=32, planned=False, heads
     return w
 
 
+def live_columns_fn(w, torch):
+    """i -> numpy array of the live columns of query row i of the workload's mask."""
+    import numpy as np
+    from oracle import spfa_oracle as so
+    n, name = w["n"], w["name"]
+    if name.startswith("csr"):
+        ro, ci = w["csr"]
+        ro_c = ro.cpu().numpy()
+        return lambda i: ci[ro_c[i]:ro_c[i + 1]].cpu().numpy()
+    if name.startswith("coo"):
+        r, c = w["coo"]
+        return lambda i: c[r == int(i)].cpu().numpy()
+    if name == "local":
+        return lambda i: so.live_local(n, w["params"]["LOCAL_SIZE"], int(i))
+    if name == "local_1d":
+        p = w["params"]
+        return lambda i: so.live_local_1d_dilated(n, p["LOCAL_SIZE"], p["DILATE_FACTOR"], int(i))
+    if name == "local_2d":
+        p = w["params"]
+        return lambda i: so.live_local_2d_dilated(n, p["BLOCK_SIZE"], p["DILATE_FACTOR"], int(i))
+    gl = w["globs"].cpu().numpy()
+    gset = set(int(x) for x in gl)
+    wsz = w["params"]["LOCAL_SIZE"]
+    if name == "bigbird":
+        ro, ci = w["csr"]
+        ro_c = ro.cpu().numpy()
+
+        def live_bb(i):
+            low, up = max(0, i - wsz), min(n, i + wsz + 1)
+            if i in gset:
+                return np.arange(0, n)
+            outside = np.array([x for x in gl if x < low or x >= up], dtype=np.int64)
+            return np.concatenate([np.arange(low, up), outside, ci[ro_c[i]:ro_c[i + 1]].cpu().numpy()])
+        return live_bb
+
+    def live_global(i):
+        low, up = max(0, i - wsz), min(n, i + wsz + 1)
+        if i in gset:
+            return np.concatenate([np.arange(0, low), np.arange(up, n)])
+        return np.array([x for x in gl if x < low or x >= up], dtype=np.int64)
+    return live_global
+
+
 def verify_sample(w, state, torch, rows=192, d_out=None, d_q=None):
     """Max-abs error of `rows` sampled output rows against the float64 CPU oracle; with d_out and
     d_q, of the sampled rows of the query gradient instead (relative to its largest entry)."""
@@ -268,58 +318,18 @@ def verify_sample(w, state, torch, rows=192, d_out=None, d_q=None):
         if d_out is not None:
             d_out, d_q = d_out[-1], d_q[-1]
     g = torch.Generator().manual_seed(123)
-    idx = torch.sort(torch.randperm(n, generator=g)[:rows])[0]
-    qs = w["q"][idx.to("cuda")].float().cpu().numpy().astype(np.float64)
+    idx_np = torch.sort(torch.randperm(n, generator=g)[:rows])[0].numpy()
+    name = w["name"]
+    if name.startswith("coo"):
+        idx_np = idx_np[:32]
+    elif name in ("bigbird", "global"):
+        # one global row is enough (each is an n-column row for the CPU)
+        idx_np = np.concatenate([idx_np[:63], w["globs"].cpu().numpy()[:1].astype(np.int64)])
+    qs = w["q"][torch.as_tensor(idx_np).to("cuda")].float().cpu().numpy().astype(np.float64)
     kk = w["k"].float().cpu().numpy().astype(np.float64)
     vv = w["v"].float().cpu().numpy().astype(np.float64)
-    name = w["name"]
-    idx_np = idx.numpy()
-    if name.startswith("csr"):
-        ro, ci = w["csr"]
-        ro_c = ro.cpu().numpy()
-        lists = [ci[ro_c[i]:ro_c[i + 1]].cpu().numpy() for i in idx_np]
-    elif name.startswith("coo"):
-        r, c = w["coo"]
-        lists = [c[r == int(i)].cpu().numpy() for i in idx_np[:32]]
-        idx_np, qs = idx_np[:32], qs[:32]
-    elif name == "local":
-        lists = [so.live_local(n, w["params"]["LOCAL_SIZE"], int(i)) for i in idx_np]
-    elif name == "local_1d":
-        p = w["params"]
-        lists = [so.live_local_1d_dilated(n, p["LOCAL_SIZE"], p["DILATE_FACTOR"], int(i)) for i in idx_np]
-    elif name == "local_2d":
-        p = w["params"]
-        lists = [so.live_local_2d_dilated(n, p["BLOCK_SIZE"], p["DILATE_FACTOR"], int(i)) for i in idx_np]
-    elif name == "bigbird":
-        gl = w["globs"].cpu().numpy()
-        gset = set(int(x) for x in gl)
-        wsz = w["params"]["LOCAL_SIZE"]
-        ro, ci = w["csr"]
-        ro_c = ro.cpu().numpy()
-        idx_np = np.concatenate([idx_np[:63], gl[:1].astype(np.int64)])
-        qs = w["q"][torch.as_tensor(idx_np).to("cuda")].float().cpu().numpy().astype(np.float64)
-
-        def live_bb(i):
-            low, up = max(0, i - wsz), min(n, i + wsz + 1)
-            if i in gset:
-                return np.arange(0, n)
-            outside = np.array([x for x in gl if x < low or x >= up], dtype=np.int64)
-            return np.concatenate([np.arange(low, up), outside, ci[ro_c[i]:ro_c[i + 1]].cpu().numpy()])
-        lists = [live_bb(int(i)) for i in idx_np]
-    else:
-        gl = w["globs"].cpu().numpy()
-        # one global row is enough (each is a 1M-column row for the CPU)
-        idx_np = np.concatenate([idx_np[:63], gl[:1].astype(np.int64)])
-        qs = w["q"][torch.as_tensor(idx_np).to("cuda")].float().cpu().numpy().astype(np.float64)
-        gset = set(int(x) for x in gl)
-        wsz = w["params"]["LOCAL_SIZE"]
-
-        def live(i):
-            low, up = max(0, i - wsz), min(n, i + wsz + 1)
-            if i in gset:
-                return np.concatenate([np.arange(0, low), np.arange(up, n)])
-            return np.array([x for x in gl if x < low or x >= up], dtype=np.int64)
-        lists = [live(int(i)) for i in idx_np]
+    live = live_columns_fn(w, torch)
+    lists = [live(int(i)) for i in idx_np]
     off = np.zeros(len(lists) + 1, dtype=np.int64)
     np.cumsum([len(x) for x in lists], out=off[1:])
     cols = np.concatenate(lists).astype(np.int64) if len(lists) else np.zeros(0, np.int64)
@@ -337,50 +347,50 @@ def verify_sample(w, state, torch, rows=192, d_out=None, d_q=None):
 
 def cpu_baseline(w, torch, target_s=12.0):
     """The reference's verification formulation on host cores: dense masked
-    scaled_dot_product_attention in fp32 over a block of query rows against all keys."""
-    import numpy as np
-    name = w["name"]
-    if not name.startswith("csr"):
-        return None
+    scaled_dot_product_attention in fp32 over blocks of query rows against all keys
+    (verification/verify.py:61-63).  The dense formulation costs the same for every query row
+    whatever its mask, so the whole job is the sampled blocks' time scaled to all n rows, and the
+    nnz-counted rate credits it with the workload's live positions."""
     n, d = w["n"], w["d"]
-    ro, ci = w["csr"]
-    ro_c, ci_c = ro.cpu(), ci.cpu()
+    heads = w.get("heads", 1)
+    if heads > 1:
+        w = dict(w, q=w["q"][-1], k=w["k"][-1], v=w["v"][-1])
     k = w["k"].float().cpu()
     v = w["v"].float().cpu()
     q = w["q"].float().cpu()
-    block = min(1024, n)
+    # scores of a block are block x n floats (twice, with the softmax) plus the boolean mask
+    block = int(min(1024, n, max(64, (1 << 28) // n)))
     g = torch.Generator().manual_seed(7)
+    live = live_columns_fn(w, torch)
 
     def one_block():
         rows = torch.sort(torch.randperm(n, generator=g)[:block])[0]
         mask = torch.zeros(block, n, dtype=torch.bool)
-        nnz = 0
         for j, i in enumerate(rows.tolist()):
-            cols = ci_c[ro_c[i]:ro_c[i + 1]]
+            cols = torch.as_tensor(live(i), dtype=torch.int64)
             mask[j, cols] = True
-            nnz += cols.numel()
         qb = q[rows]
         t0 = time.perf_counter()
         torch.nn.functional.scaled_dot_product_attention(qb, k, v, attn_mask=mask)
-        return time.perf_counter() - t0, nnz
+        return time.perf_counter() - t0
 
     one_block()  # warm-up
-    t_tot, nnz_tot, blocks = 0.0, 0, 0
+    t_tot, blocks = 0.0, 0
     t_begin = time.perf_counter()
     while (time.perf_counter() - t_begin) < target_s and blocks < 64:
-        t, z = one_block()
-        t_tot += t
-        nnz_tot += z
+        t_tot += one_block()
         blocks += 1
-    gflops = 4.0 * d * nnz_tot / t_tot / 1e9
-    dense_gflops = 4.0 * d * block * blocks * n / t_tot / 1e9
+    job_s = t_tot / blocks * (n / block)  # one head
+    nnz_head = w["nnz"] / heads
     return {
-        "value": gflops, "unit": "GFLOP/s (nnz-counted)", "cores": torch.get_num_threads(),
-        "kind": "port",
+        "value": 4.0 * d * nnz_head / job_s / 1e9, "unit": "GFLOP/s (nnz-counted)",
+        "cores": torch.get_num_threads(), "kind": "port",
         "sample": "%d blocks of %d random query rows x all %d keys, torch CPU dense masked "
-                  "scaled_dot_product_attention fp32 (the reference's verification formulation); "
-                  "%.2f s of SDPA time, %d live positions" % (blocks, block, n, t_tot, nnz_tot),
-        "dense_gflops": dense_gflops, "host_cpus": os.cpu_count(),
+                  "scaled_dot_product_attention fp32 (the reference's verification formulation), "
+                  "%.2f s of SDPA time; scaled to all %d rows (%.1f s for the whole mask) and "
+                  "credited with its %d live positions" % (blocks, block, n, t_tot, n, job_s, nnz_head),
+        "dense_gflops": 4.0 * d * block * blocks * n / t_tot / 1e9, "host_cpus": os.cpu_count(),
+        "whole_job_s": job_s,
     }
 
 
@@ -517,6 +527,46 @@ def measured_copy_bandwidth(torch, mib=1024, reps=5):
     return 2.0 * src.numel() * 4 / (best * 1e-3) / 1e9
 
 
+def measured_gather_ceiling(lib, w, torch, min_entries=8_000_000, reps=5):
+    """What the memory system delivers to the explicit-mask access pattern at this working set:
+    spfa_probe_gather (the gather of segments_kernel without any arithmetic) over the workload's
+    own K, V and column list (the list is repeated up to min_entries so that the launch is long
+    enough to time).  Best of a few launch shapes.  None when the row size has no probe."""
+    k, v = w["k"], w["v"]
+    if k.dim() != 2:
+        k, v = k[-1], v[-1]
+    row_bytes = k.shape[1] * k.element_size()
+    idx = w.get("probe_idx")
+    if idx is None or row_bytes not in (64, 128, 256, 512) or idx.numel() == 0:
+        return None
+    if idx.numel() < min_entries:
+        idx = idx.repeat((min_entries + idx.numel() - 1) // idx.numel())
+    lib.spfa_probe_gather.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64,
+                                      ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64, ctypes.c_int, ctypes.c_int,
+                                      ctypes.c_void_p, ctypes.c_void_p]
+    cursor = torch.zeros(64, dtype=torch.int32, device="cuda")
+    stream = torch.cuda.current_stream().cuda_stream
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    best, best_shape = float("inf"), None
+    shapes = ((1, 16), (1, 32), (2, 16), (2, 32), (4, 32))
+    for wg, fl in shapes:
+        for _ in range(reps):
+            e0.record()
+            rc = lib.spfa_probe_gather(k.data_ptr(), v.data_ptr(), k.shape[0], row_bytes, idx.data_ptr(),
+                                       idx.numel(), 1024, wg, fl, cursor.data_ptr(), stream)
+            assert rc == 0, "spfa_probe_gather rc=%d" % rc
+            e1.record()
+            torch.cuda.synchronize()
+            ms = e0.elapsed_time(e1)
+            if ms < best:
+                best, best_shape = ms, (wg, fl)
+    bytes_moved = idx.numel() * (2 * row_bytes + 4)
+    return {"GBs": bytes_moved / (best * 1e-3) / 1e9,
+            "how": "%d list entries x (2 rows of %d B + 4 B index) in %.3f ms; best of %d launches each of "
+                   "(workgroups per CU, rows in flight) %s: (%d,%d)"
+                   % (idx.numel(), row_bytes, best, reps, " ".join("(%d,%d)" % x for x in shapes), *best_shape)}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -584,7 +634,8 @@ def main():
     if a.backward:
         return bench_backward(a, w, states[0], dtype, torch, syn)
 
-    ev = HipEvents()
+    n_ev = min(a.steps, 10)
+    evs = [HipEvents() for _ in range(n_ev)]
     for i in range(a.warmup):
         w["call"](fresh(i))
     torch.cuda.synchronize()
@@ -609,19 +660,32 @@ def main():
             graph.replay()
         torch.cuda.synchronize()
         dt = time.perf_counter() - t0
+        # (events cannot be recorded inside a captured graph: one eager step is timed for the kernel)
+        lib.spfa_set_kernel_events(evs[0].start, evs[0].stop)
+        w["call"](fresh(0))
+        lib.spfa_set_kernel_events(None, None)
+        torch.cuda.synchronize()
+        evs = evs[:1]
     else:
-        # timed region: exactly K steps
+        # timed region: exactly K steps, back to back on the stream.  In the last n_ev of them the
+        # library records an event pair around its dominant kernel (no host synchronisation), so the
+        # kernel times come out of the very steps that ms_per_step averages over.
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         for i in range(a.steps):
+            j = i - (a.steps - n_ev)
+            if j >= 0:
+                lib.spfa_set_kernel_events(evs[j].start, evs[j].stop)
             w["call"](fresh(a.warmup + i))
         torch.cuda.synchronize()
         dt = time.perf_counter() - t0
+        lib.spfa_set_kernel_events(None, None)
     ms_per_step = dt / a.steps * 1e3
+    kernel_ms = [e.elapsed_ms() for e in evs]
+    k_avg = sum(kernel_ms) / len(kernel_ms)
 
-    # dominant-kernel time: HIP events recorded inside the library around that kernel only
-    kernel_ms, call_ms = [], []
-    lib.spfa_set_kernel_events(ev.start, ev.stop)
+    # one call at a time (synchronised before and after): latency of a single call
+    call_ms = []
     c0, c1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     for i in range(min(a.steps, 10)):
         st = states[i % n_alloc]
@@ -632,11 +696,8 @@ def main():
         w["call"](st)
         c1.record()
         c1.synchronize()
-        kernel_ms.append(ev.elapsed_ms())
         call_ms.append(c0.elapsed_time(c1))
-    lib.spfa_set_kernel_events(None, None)
     torch.cuda.synchronize()
-    k_avg = sum(kernel_ms) / len(kernel_ms)
     copy_gbs = measured_copy_bandwidth(torch)
 
     if a.copy_calibration:
@@ -651,43 +712,79 @@ def main():
     tol = 1e-4 if dtype == torch.float32 else 2e-2
 
     flops = syn.attention_flops(nnz, d)
-    achieved_gbs = w["kernel_bytes"] / (k_avg * 1e-3) / 1e9
+    es = torch.tensor([], dtype=dtype).element_size()
     explicit = a.workload.startswith(("csr", "coo"))
-    if w.get("whole_call") or (explicit and w["kernel_nnz"] == 0):
-        # no row is long enough for the segment kernel (all of them go to the row kernels): the
-        # whole call stands in, with the call's algorithmic bytes
-        k_avg = ms_per_step
-        kernel_ms = [ms_per_step]
-        achieved_gbs = w["bytes_total"] / (ms_per_step * 1e-3) / 1e9
-        roofline = {"bound": "hbm", "achieved": achieved_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                    "frac": achieved_gbs / HBM_PEAK_GBS, "traffic": None,
-                    "kernel": "whole call (several kernels, none dominant)"}
-        w = dict(w, kernel_bytes=w["bytes_total"], kernel_nnz=w["nnz"], kernel_rows=w["n"] * w.get("heads", 1))
-    elif explicit:
-        # gather work: bound by memory, algorithmic bytes of the segment kernel over its time
-        roofline = {"bound": "hbm", "achieved": achieved_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                    "frac": achieved_gbs / HBM_PEAK_GBS, "traffic": measured_traffic(a.workload, a.dtype),
-                    "kernel": "segments_kernel"}
-    else:
-        # dense tiles: the matrix pipe bounds these (compulsory bytes / 8 TB/s is the smaller time);
-        # flops of the timed kernel = 4*d per live position it covers
-        peak = FP32_PEAK_TFLOPS if a.dtype == "f32" else HALF_PEAK_TFLOPS
-        kernel_flops = flops if a.workload != "global" else 4.0 * d * w["n_global_rows_nnz"]
-        achieved_tf = kernel_flops / (k_avg * 1e-3) / 1e12
-        roofline = {"bound": "mfma", "achieved": achieved_tf, "peak": peak, "unit": "TFLOP/s",
-                    "frac": achieved_tf / peak, "traffic": None,
-                    "kernel": "tile_kernel (global rows)" if a.workload == "global" else
-                              ("band_dma_f32_kernel" if a.dtype == "f32" else "band_dma_kernel"),
-                    "hbm_time_ms": w["bytes_total"] / (HBM_PEAK_GBS * 1e9) * 1e3,
-                    "mfma_time_ms": flops / (peak * 1e12) * 1e3}
-    if roofline["bound"] == "hbm":
+    if explicit or w.get("whole_call"):
+        # Gather work: bound by the memory system.  Which level binds depends on where K and V
+        # live: every XCD's 4 MiB L2, the 256 MiB memory-side cache, or HBM.  The 8 TB/s HBM figure
+        # is only a ceiling when K and V do not fit the memory-side cache; below that the ceiling
+        # is what the same gather without arithmetic sustains at this working set (measured here).
+        kernel_name = "segments_kernel"
+        if w.get("whole_call") or w["kernel_nnz"] == 0:
+            # no row is long enough for the segment kernel, or several kernels share the call: the
+            # whole call stands in, with the call's algorithmic bytes
+            k_avg, kernel_ms = ms_per_step, [ms_per_step]
+            kernel_name = "whole call (several kernels, none dominant)"
+            w = dict(w, kernel_bytes=w["bytes_total"], kernel_nnz=w["nnz"],
+                     kernel_rows=w["n"] * w.get("heads", 1))
+        achieved_gbs = w["kernel_bytes"] / (k_avg * 1e-3) / 1e9
+        kv_bytes = 2 * w["k"].numel() * es
+        gather = measured_gather_ceiling(lib, w, torch)
+        if kv_bytes <= 4 << 20:
+            bound = "l2"
+        elif kv_bytes <= 256 << 20:
+            bound = "infinity_cache"
+        else:
+            bound = "hbm"
+        peak = HBM_PEAK_GBS if bound == "hbm" or gather is None else gather["GBs"]
+        roofline = {"bound": bound, "achieved": achieved_gbs, "peak": peak, "unit": "GB/s",
+                    "frac": achieved_gbs / peak,
+                    "peak_source": "MI355X HBM3E, published" if peak == HBM_PEAK_GBS else
+                                   "measured on this device: the same gather without arithmetic "
+                                   "(spfa_probe_gather) over this K and V and this column list",
+                    "traffic": measured_traffic(a.workload, a.dtype), "kernel": kernel_name,
+                    "kv_working_set_bytes": kv_bytes,
+                    "hbm_peak_GBs": HBM_PEAK_GBS, "achieved_over_hbm_peak": achieved_gbs / HBM_PEAK_GBS}
+        if gather is not None:
+            roofline["measured_gather_GBs"] = gather["GBs"]
+            roofline["frac_of_measured_gather"] = achieved_gbs / gather["GBs"]
+            roofline["measured_gather"] = gather["how"]
         roofline["measured_copy_GBs"] = copy_gbs
-        roofline["frac_of_measured_copy"] = roofline["achieved"] / copy_gbs
     else:
-        roofline["measured_copy_GBs"] = copy_gbs
-        roofline["hbm_time_at_measured_copy_ms"] = w["bytes_total"] / (copy_gbs * 1e9) * 1e3
+        # dense tiles: the roofline time is the larger of the HBM time of the compulsory bytes and
+        # the matrix-pipe time of the live flops; whichever is larger names the bound.  The global
+        # mask runs two tile kernels; the timed one (global rows against every key) reads K and V
+        # once and computes the global rows' positions.
+        mfma_peak = FP32_PEAK_TFLOPS if a.dtype == "f32" else HALF_PEAK_TFLOPS
+        if a.workload == "global":
+            kernel_flops = 4.0 * d * w["n_global_rows_nnz"]
+            kernel_bytes = 2 * n * d * es
+            kernel_name = "tile_kernel (global rows)"
+            w = dict(w, kernel_bytes=kernel_bytes, kernel_nnz=w["n_global_rows_nnz"],
+                     kernel_rows=w["params"]["n_globals"])
+        else:
+            kernel_flops, kernel_bytes = flops, w["bytes_total"]
+            kernel_name = "band_dma_f32_kernel" if a.dtype == "f32" else "band_dma_kernel"
+        hbm_ms = kernel_bytes / (HBM_PEAK_GBS * 1e9) * 1e3
+        mfma_ms = kernel_flops / (mfma_peak * 1e12) * 1e3
+        if hbm_ms >= mfma_ms:
+            achieved, peak, unit, bound = kernel_bytes / (k_avg * 1e-3) / 1e9, HBM_PEAK_GBS, "GB/s", "hbm"
+        else:
+            achieved, peak, unit, bound = kernel_flops / (k_avg * 1e-3) / 1e12, mfma_peak, "TFLOP/s", "mfma"
+        roofline = {"bound": bound, "achieved": achieved, "peak": peak, "unit": unit,
+                    "frac": achieved / peak, "traffic": None, "kernel": kernel_name,
+                    "hbm_time_ms": hbm_ms, "mfma_time_ms": mfma_ms, "roofline_time_ms": max(hbm_ms, mfma_ms),
+                    "kernel_TFLOPs": kernel_flops / (k_avg * 1e-3) / 1e12,
+                    "kernel_compulsory_GBs": kernel_bytes / (k_avg * 1e-3) / 1e9,
+                    "call_hbm_time_ms": w["bytes_total"] / (HBM_PEAK_GBS * 1e9) * 1e3,
+                    "call_mfma_time_ms": flops / (mfma_peak * 1e12) * 1e3,
+                    "measured_copy_GBs": copy_gbs,
+                    "hbm_time_at_measured_copy_ms": kernel_bytes / (copy_gbs * 1e9) * 1e3}
+    roofline["frac_above_one"] = bool(roofline["frac"] > 1.0)
     call_sorted = sorted(call_ms)
     roofline.update({"kernel_ms_avg": k_avg, "kernel_ms_min": min(kernel_ms),
+                     "kernel_ms_from": "event pairs around the kernel in the last %d steps of the timed loop"
+                                       % len(kernel_ms),
                      "algorithmic_bytes": w["kernel_bytes"], "kernel_nnz": w["kernel_nnz"],
                      "kernel_rows": w["kernel_rows"], "call_algorithmic_bytes": w["bytes_total"],
                      "call_gathered_bytes": w["bytes_gathered"]})
@@ -707,6 +804,7 @@ def main():
                                       if a.workload == "bigbird" else None)},
         "call_ms_median": call_sorted[len(call_sorted) // 2], "call_ms_min": call_sorted[0],
         "effective_gathered_GBs": w["bytes_gathered"] / (ms_per_step * 1e-3) / 1e9,
+        "effective_gathered_over_hbm_peak": w["bytes_gathered"] / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS,
         "algorithmic_GBs": w["bytes_total"] / (ms_per_step * 1e-3) / 1e9,
         "roofline": roofline,
         "parity": {"max_abs_err": err, "rows_checked": checked, "tolerance": tol, "ok": bool(err <= tol)},

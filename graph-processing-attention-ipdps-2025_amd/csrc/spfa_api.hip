@@ -3,6 +3,7 @@
 #include "spfa_hip.h"
 
 #include <limits>
+#include <mutex>
 
 #include "spfa_backward.hpp"
 #include "spfa_grad.hpp"
@@ -14,6 +15,7 @@ using namespace spfa;
 namespace {
 
 constexpr int64_t kInlineAll = std::numeric_limits<int64_t>::max();
+constexpr int64_t kAnyColumn = std::numeric_limits<int64_t>::max();  // a mask used for its row lengths only
 
 
 
@@ -294,10 +296,32 @@ GlobalLayout global_layout(int64_t n, int64_t n_globs, int64_t d, int64_t n_batc
 
 }  // namespace
 
+// One word per device that kernels OR bits into when mask arrays turn out inconsistent (see
+// spfa_device_status).  Its name is only a host-side handle: the device address comes from the
+// runtime, once per device.
+static __device__ uint32_t spfa_status_word;
+
 namespace spfa {
 KernelEvents& kernel_events() {
   static KernelEvents ev;
   return ev;
+}
+
+uint32_t* device_status_word() {
+  constexpr int kMaxDevices = 64;
+  static uint32_t* ptrs[kMaxDevices];
+  static bool tried[kMaxDevices];
+  static std::mutex mu;
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return nullptr;
+  std::lock_guard<std::mutex> lock(mu);
+  if (!tried[dev]) {
+    tried[dev] = true;
+    void* ptr = nullptr;
+    if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(spfa_status_word)) == hipSuccess) ptrs[dev] = (uint32_t*)ptr;
+    else (void)hipGetLastError();
+  }
+  return ptrs[dev];
 }
 }  // namespace spfa
 
@@ -306,6 +330,18 @@ extern "C" {
 int spfa_version(void) { return 1; }
 
 int64_t spfa_explicit_inline_row_limit(void) { return kExplicitMediumRowLimit; }
+
+int spfa_device_status(int reset) {
+  uint32_t* word = device_status_word();
+  if (word == nullptr) return -1;
+  uint32_t bits = 0;
+  if (hipMemcpy(&bits, word, sizeof(bits), hipMemcpyDeviceToHost) != hipSuccess) return -1;
+  if (reset && bits != 0) {
+    const uint32_t zero = 0;
+    if (hipMemcpy(word, &zero, sizeof(zero), hipMemcpyHostToDevice) != hipSuccess) return -1;
+  }
+  return (int)bits;
+}
 
 void spfa_set_kernel_events(void* start, void* stop) {
   kernel_events().start = (hipEvent_t)start;
@@ -343,6 +379,18 @@ size_t spfa_csr_workspace_bytes(int64_t n_q, int64_t nnz, int64_t d, int dtype) 
   return engine_workspace(size_csr(n_q, nnz), n_q, d).total;
 }
 
+size_t spfa_csr_workspace_bytes_batched(int64_t n_q, int64_t nnz, int64_t d, int dtype, int64_t n_batch) {
+  (void)dtype;
+  if (n_q < 0 || nnz < 0 || d < 1) return 0;
+  const EngineSizing s = size_csr(n_q, nnz);
+  spfa_problem_t p{};
+  p.n_q = n_q;
+  p.d = d;
+  p.n_batch = n_batch;
+  // (a batch too large for the engine's 32-bit work cursor is walked problem by problem)
+  return engine_workspace(s, n_q, d, batch_fits_engine(s, &p) ? batch_of(&p) : 1).total;
+}
+
 int spfa_csr_forward(const spfa_problem_t* p, const void* row_off, int row_off_bytes,
                      const void* col_ind, int64_t nnz, int use_nan, void* workspace,
                      size_t workspace_bytes, void* stream) {
@@ -354,7 +402,7 @@ int spfa_csr_forward(const spfa_problem_t* p, const void* row_off, int row_off_b
   if (p->n_q == 0) return SPFA_OK;
   if (!row_off || (nnz > 0 && !col_ind)) return SPFA_ERR_BAD_ARG;
   if (is_f64(p)) {
-    CsrMask mask{row_off, (const uint32_t*)col_ind, row_off_bytes == 8 ? 1 : 0, nullptr, nullptr};
+    CsrMask mask{row_off, (const uint32_t*)col_ind, row_off_bytes == 8 ? 1 : 0, nullptr, nullptr, nnz, p->n_k};
     return run_f64(make_tensors(p), mask, use_nan ? 1 : 0, (hipStream_t)stream);
   }
   EngineSizing s = size_csr(p->n_q, nnz);
@@ -370,7 +418,7 @@ int spfa_csr_forward(const spfa_problem_t* p, const void* row_off, int row_off_b
   rc = check_workspace(workspace, workspace_bytes,
                        engine_workspace(s, p->n_q, p->d, batch_of(p)).total);
   if (rc) return rc;
-  CsrMask mask{row_off, (const uint32_t*)col_ind, row_off_bytes == 8 ? 1 : 0, nullptr, nullptr};
+  CsrMask mask{row_off, (const uint32_t*)col_ind, row_off_bytes == 8 ? 1 : 0, nullptr, nullptr, nnz, p->n_k};
   return dispatch_csr(p, mask, s, use_nan ? 1 : 0, workspace, (hipStream_t)stream);
 }
 
@@ -387,7 +435,7 @@ int spfa_csr_plan(int64_t n_q, const void* row_off, int row_off_bytes, const voi
   if (!row_off || (nnz > 0 && !col_ind)) return SPFA_ERR_BAD_ARG;
   int rc = check_workspace(plan, plan_bytes, work_list_bytes(n_q, nnz));
   if (rc) return rc;
-  CsrMask mask{row_off, (const uint32_t*)col_ind, row_off_bytes == 8 ? 1 : 0, nullptr, nullptr};
+  CsrMask mask{row_off, (const uint32_t*)col_ind, row_off_bytes == 8 ? 1 : 0, nullptr, nullptr, nnz, kAnyColumn};
   return build_work_list(n_q, mask, size_csr(n_q, nnz), plan, (hipStream_t)stream);
 }
 
@@ -403,7 +451,7 @@ int spfa_csr_forward_planned(const spfa_problem_t* p, const void* row_off, int r
   if (p->n_q == 0) return SPFA_OK;
   if (!row_off || (nnz > 0 && !col_ind)) return SPFA_ERR_BAD_ARG;
   if (is_f64(p)) {  // (the fp64 kernel needs no work list)
-    CsrMask mask{row_off, (const uint32_t*)col_ind, row_off_bytes == 8 ? 1 : 0, nullptr, nullptr};
+    CsrMask mask{row_off, (const uint32_t*)col_ind, row_off_bytes == 8 ? 1 : 0, nullptr, nullptr, nnz, p->n_k};
     return run_f64(make_tensors(p), mask, use_nan ? 1 : 0, (hipStream_t)stream);
   }
   EngineSizing s = size_csr(p->n_q, nnz);
@@ -421,7 +469,7 @@ int spfa_csr_forward_planned(const spfa_problem_t* p, const void* row_off, int r
   rc = check_workspace(workspace, workspace_bytes,
                        engine_workspace(s, p->n_q, p->d, batch_of(p)).total);
   if (rc) return rc;
-  CsrMask mask{row_off, (const uint32_t*)col_ind, row_off_bytes == 8 ? 1 : 0, nullptr, nullptr};
+  CsrMask mask{row_off, (const uint32_t*)col_ind, row_off_bytes == 8 ? 1 : 0, nullptr, nullptr, nnz, p->n_k};
   return dispatch_csr(p, mask, s, use_nan ? 1 : 0, workspace, (hipStream_t)stream, kEngineRunOnly,
                       plan);
 }
@@ -431,6 +479,11 @@ size_t spfa_coo_workspace_bytes(int64_t n_q, int64_t nnz, int64_t d, int dtype) 
   (void)dtype;
   if (n_q < 0 || nnz < 0 || d < 1) return 0;
   return coo_workspace(n_q, nnz).total + engine_workspace(size_csr(n_q, nnz), n_q, d).total;
+}
+
+size_t spfa_coo_workspace_bytes_batched(int64_t n_q, int64_t nnz, int64_t d, int dtype, int64_t n_batch) {
+  if (n_q < 0 || nnz < 0 || d < 1) return 0;
+  return coo_workspace(n_q, nnz).total + spfa_csr_workspace_bytes_batched(n_q, nnz, d, dtype, n_batch);
 }
 
 int spfa_coo_forward(const spfa_problem_t* p, const void* row_ind, int row_ind_bytes,
@@ -455,7 +508,7 @@ int spfa_coo_forward(const spfa_problem_t* p, const void* row_ind, int row_ind_b
   rc = coo_to_csr(row_ind, row_ind_bytes == 8 ? 1 : 0, (const uint32_t*)col_ind, nnz, p->n_q,
                   workspace, (char*)workspace + cw.keep_total, (hipStream_t)stream, &csr);
   if (rc) return rc;
-  CsrMask mask{csr.row_off, (const uint32_t*)col_ind, 0, csr.cols, csr.unsorted};
+  CsrMask mask{csr.row_off, (const uint32_t*)col_ind, 0, csr.cols, csr.unsorted, nnz, p->n_k};
   if (is_f64(p)) return run_f64(make_tensors(p), mask, use_nan ? 1 : 0, (hipStream_t)stream);
   if (!batched) {  // one conversion, then problem after problem
     for (int64_t b = 0; b < batch_of(p); b++) {
@@ -498,7 +551,7 @@ int spfa_coo_plan(int64_t n_q, const void* row_ind, int row_ind_bytes, const voi
   rc = coo_to_csr(row_ind, row_ind_bytes == 8 ? 1 : 0, (const uint32_t*)col_ind, nnz, n_q, plan,
                   workspace, (hipStream_t)stream, &csr);
   if (rc) return rc;
-  CsrMask mask{csr.row_off, (const uint32_t*)col_ind, 0, csr.cols, csr.unsorted};
+  CsrMask mask{csr.row_off, (const uint32_t*)col_ind, 0, csr.cols, csr.unsorted, nnz, kAnyColumn};
   return build_work_list(n_q, mask, size_csr(n_q, nnz), (char*)plan + w.keep_total,
                          (hipStream_t)stream);
 }
@@ -531,7 +584,7 @@ int spfa_coo_forward_planned(const spfa_problem_t* p, const void* col_ind, int64
   if (rc) return rc;
   const char* pb = (const char*)plan;
   CsrMask mask{pb + w.off_row_off, (const uint32_t*)col_ind, 0, (const uint32_t*)(pb + w.off_cols),
-               (const uint32_t*)(pb + w.off_flag)};
+               (const uint32_t*)(pb + w.off_flag), nnz, p->n_k};
   if (is_f64(p)) return run_f64(make_tensors(p), mask, use_nan ? 1 : 0, (hipStream_t)stream);
   return dispatch_csr(p, mask, s, use_nan ? 1 : 0, workspace, (hipStream_t)stream, kEngineRunOnly,
                       pb + w.keep_total);
@@ -562,7 +615,7 @@ int spfa_local_1d_dilated_forward(const spfa_problem_t* p, int64_t local_size, i
   if (rc) return rc;
   if (local_size < 0 || local_size > p->n_q - 1) return SPFA_ERR_LOCAL_SIZE;
   if (dil_factor < 0) return SPFA_ERR_DILATION_NEG;
-  if (dil_factor >= (int64_t)1 << 31) return SPFA_ERR_BAD_ARG;
+  if (dil_factor >= (int64_t)1 << 31 || p->n_k != p->n_q) return SPFA_ERR_BAD_ARG;
   rc = check_pointers(p);
   if (rc) return rc;
   const int64_t n = p->n_q;
@@ -598,6 +651,7 @@ int spfa_local_2d_dilated_forward(const spfa_problem_t* p, int64_t block_size, i
   if (block_size <= 0 || p->n_q % block_size != 0) return SPFA_ERR_BLOCK_DIVISOR;
   if (dil_factor < 0) return SPFA_ERR_DILATION_NEG;
   if (block_size / (dil_factor + 1) < 1) return SPFA_ERR_BLOCK_DILATION;
+  if (p->n_k != p->n_q) return SPFA_ERR_BAD_ARG;
   rc = check_pointers(p);
   if (rc) return rc;
   const int64_t n = p->n_q;
@@ -631,6 +685,7 @@ int spfa_global_no_local_forward(const spfa_problem_t* p, const int32_t* global_
   if (rc) return rc;
   if (n_globals <= 0 || n_globals > p->n_q) return SPFA_ERR_GLOBAL_COUNT;
   if (local_size < 0 || local_size > p->n_q - 1) return SPFA_ERR_LOCAL_SIZE;
+  if (p->n_k != p->n_q) return SPFA_ERR_BAD_ARG;
   rc = check_pointers(p);
   if (rc) return rc;
   if (!global_inds) return SPFA_ERR_BAD_ARG;
@@ -850,7 +905,7 @@ int explicit_backward(const spfa_problem_t* p, const spfa_grads_t* g, const CsrM
     const uint32_t* e_rows = nullptr;
     int rc = transpose_mask(rows, p->n_q, p->n_k, nnz, (char*)workspace + lay.off_mask, stream, &tr, &e_rows);
     if (rc) return rc;
-    cols = CsrMask{tr.row_off, e_rows, 0, tr.cols, tr.unsorted};
+    cols = CsrMask{tr.row_off, e_rows, 0, tr.cols, tr.unsorted, nnz, p->n_q};
   }
   const GradArgs a = make_grad_args(p, g, lay, workspace);
   const Tensors t = make_tensors(p);
@@ -925,8 +980,8 @@ int spfa_csr_backward(const spfa_problem_t* p, const spfa_grads_t* g, const void
   if (!lay.ok) return SPFA_ERR_BAD_ARG;
   rc = check_workspace(workspace, workspace_bytes, lay.total);
   if (rc) return rc;
-  CsrMask rows{row_off, (const uint32_t*)col_ind, row_off_bytes == 8 ? 1 : 0, nullptr, nullptr};
-  CsrMask cols{t_row_off, t_col_ind, 0, nullptr, nullptr};
+  CsrMask rows{row_off, (const uint32_t*)col_ind, row_off_bytes == 8 ? 1 : 0, nullptr, nullptr, nnz, p->n_k};
+  CsrMask cols{t_row_off, t_col_ind, 0, nullptr, nullptr, nnz, p->n_q};
   return explicit_backward(p, g, rows, nnz, given ? &cols : nullptr, lay, workspace,
                            (hipStream_t)stream);
 }
@@ -945,7 +1000,7 @@ int spfa_csr_transpose(int64_t n_q, int64_t n_k, const void* row_off, int row_of
   if (!t_row_off || (nnz > 0 && (!row_off || !col_ind || !t_col_ind))) return SPFA_ERR_BAD_ARG;
   int rc = check_workspace(workspace, workspace_bytes, transpose_layout(n_k, nnz).total);
   if (rc) return rc;
-  CsrMask rows{row_off, (const uint32_t*)col_ind, row_off_bytes == 8 ? 1 : 0, nullptr, nullptr};
+  CsrMask rows{row_off, (const uint32_t*)col_ind, row_off_bytes == 8 ? 1 : 0, nullptr, nullptr, nnz, n_k};
   CooCsr tr{};
   const uint32_t* e_rows = nullptr;
   rc = transpose_mask(rows, n_q, n_k, nnz, (char*)workspace, (hipStream_t)stream, &tr, &e_rows);
@@ -1008,7 +1063,7 @@ int spfa_coo_backward(const spfa_problem_t* p, const spfa_grads_t* g, const void
   rc = coo_to_csr(row_ind, row_ind_bytes == 8 ? 1 : 0, (const uint32_t*)col_ind, nnz, p->n_q, fwd,
                   fwd + cw.keep_total, (hipStream_t)stream, &csr);
   if (rc) return rc;
-  CsrMask rows{csr.row_off, (const uint32_t*)col_ind, 0, csr.cols, csr.unsorted};
+  CsrMask rows{csr.row_off, (const uint32_t*)col_ind, 0, csr.cols, csr.unsorted, nnz, p->n_k};
   lay.off_mask += fwd_bytes;
   return explicit_backward(p, g, rows, nnz, nullptr, lay, workspace, (hipStream_t)stream);
 }

@@ -209,6 +209,12 @@ __device__ __forceinline__ bool bit_is_set(const uint32_t* bits, int64_t i) {
   return (bits[i >> 5] >> (i & 31)) & 1u;
 }
 
+// A listed (global) token as the kernels use it: itself when it names a row of the problem, else
+// -1 (such an entry is masked for every query and never used as an address).
+__device__ __forceinline__ int listed_token(int g, int64_t n) {
+  return ((int64_t)g >= 0 && (int64_t)g < n) ? g : -1;
+}
+
 __device__ __forceinline__ int lane_id() {
   return (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
 }

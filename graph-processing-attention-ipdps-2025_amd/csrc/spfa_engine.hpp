@@ -21,6 +21,8 @@
 // form one grid, the work list is shared, partial results are per problem.
 #pragma once
 
+#include <hip/hip_ext.h>
+
 #include "spfa_common.hpp"
 #include "spfa_prep.hpp"
 
@@ -90,11 +92,20 @@ struct Plan {
   uint32_t cap_partials;
   uint32_t cap_multi;
   uint32_t cap_medium;
+  uint32_t* status;  // the device's sticky status word (may be null): see device_status_word()
   int32_t use_nan;
   int64_t short_max;
   int64_t medium_max;  // == short_max: no medium rows
   int64_t seg;
 };
+
+// Bits of the device's sticky status word (spfa_device_status): what kernels found wrong with mask
+// arrays they could only look at on the device.
+constexpr uint32_t kStatusWorkListOverflow = 1u;  // more long-row segments than the nnz passed allows
+constexpr uint32_t kStatusRowOffsets = 2u;        // row offsets decreasing or beyond nnz
+
+// Device address of the current device's status word, or null when it cannot be looked up.
+uint32_t* device_status_word();
 
 static __global__ void reset_cursor_kernel(uint32_t* cursor) {
   if (threadIdx.x == 0) *cursor = 0;
@@ -293,7 +304,13 @@ __global__ __launch_bounds__(kPlanThreads) void plan_kernel(int64_t n_q, Mask ma
   const int wave = threadIdx.x / kWave;
   const int64_t row = (int64_t)blockIdx.x * kPlanThreads + threadIdx.x;
   int64_t deg = 0;
-  if (row < n_q) deg = mask.row(row).deg;
+  if (row < n_q) {
+    deg = mask.row(row).deg;
+    if constexpr (Mask::kExplicit) {
+      // offsets that run backwards or past the entry count: the row was cut to what exists
+      if (plan.status != nullptr && !mask.consistent(row)) atomicOr(plan.status, kStatusRowOffsets);
+    }
+  }
   const bool is_medium = deg > plan.short_max && deg <= plan.medium_max;
   const bool is_long = deg > plan.medium_max;
   const uint32_t nseg = is_long ? (uint32_t)((deg + plan.seg - 1) / plan.seg) : 0u;
@@ -328,6 +345,7 @@ __global__ __launch_bounds__(kPlanThreads) void plan_kernel(int64_t n_q, Mask ma
           block_base[2] + tot[2] > plan.cap_multi) {
         ok = 0;
         atomicOr(&plan.cnt->overflow, 1u);
+        if (plan.status != nullptr) atomicOr(plan.status, kStatusWorkListOverflow);
       }
     }
     if (tot[3]) {
@@ -335,6 +353,7 @@ __global__ __launch_bounds__(kPlanThreads) void plan_kernel(int64_t n_q, Mask ma
       if (block_base[3] + tot[3] > plan.cap_medium) {
         ok = 0;
         atomicOr(&plan.cnt->overflow, 1u);
+        if (plan.status != nullptr) atomicOr(plan.status, kStatusWorkListOverflow);
       }
     }
     block_ok = ok;
@@ -536,7 +555,8 @@ constexpr int kWholeRowsWaves = 8;
 constexpr int64_t kWholeRowsLong = 1024;
 
 template <class Lay, class Mask>
-__global__ __launch_bounds__(kWholeRowsWaves* kWave) void whole_rows_kernel(Tensors t, Mask mask, int use_nan) {
+__global__ __launch_bounds__(kWholeRowsWaves* kWave) void whole_rows_kernel(Tensors t, Mask mask, int use_nan,
+                                                                            uint32_t* status) {
   using T = typename Lay::elem;
   constexpr int NE = Lay::NE;
   constexpr int LPR = Lay::LPR;
@@ -590,6 +610,9 @@ __global__ __launch_bounds__(kWholeRowsWaves* kWave) void whole_rows_kernel(Tens
       int64_t b, ri;
       split_row(t, row, b, ri);
       const int64_t deg = mask.row(ri).deg;
+      if constexpr (Mask::kExplicit) {
+        if (status != nullptr && lane == 0 && !mask.consistent(ri)) atomicOr(status, kStatusRowOffsets);
+      }
       if (deg <= 0) {
         if (use_nan && g == 0) {
           float nanv[NE];
@@ -735,6 +758,18 @@ struct KernelEvents {
 };
 KernelEvents& kernel_events();
 
+// Launches `kernel`; with a pair of events set, the pair receives the start and end time stamps
+// of this very dispatch (no extra packets in the queue), so that their difference is the
+// kernel's own duration even when launches follow each other back to back on the stream.
+template <typename... KArgs, typename... Args>
+inline void launch_maybe_timed(const KernelEvents& ev, void (*kernel)(KArgs...), dim3 grid, dim3 block,
+                               hipStream_t stream, Args&&... args) {
+  if (ev.start != nullptr && ev.stop != nullptr)
+    hipExtLaunchKernelGGL(kernel, grid, block, 0, stream, ev.start, ev.stop, 0, static_cast<KArgs>(args)...);
+  else
+    hipLaunchKernelGGL(kernel, grid, block, 0, stream, static_cast<KArgs>(args)...);
+}
+
 constexpr int kSegmentWorkgroupsPerCu = 1;
 // whole_rows_kernel takes a call of at most this many rows (over all problems), keys and
 // candidates.  What it cannot do is share one very long row over the device, so the limits keep
@@ -785,6 +820,7 @@ int launch_engine(const Tensors& t, const Mask& mask, const EngineSizing& s, int
   plan.cap_partials = w.cap_partials;
   plan.cap_multi = w.cap_multi;
   plan.cap_medium = w.cap_medium;
+  plan.status = device_status_word();
   plan.use_nan = use_nan;
   plan.short_max = s.short_max;
   plan.medium_max = s.medium_max > s.short_max ? s.medium_max : s.short_max;
@@ -793,14 +829,11 @@ int launch_engine(const Tensors& t, const Mask& mask, const EngineSizing& s, int
 
   const bool has_long = s.max_deg > s.short_max;
   const KernelEvents ev = kernel_events();
-  const bool timed = ev.start != nullptr && ev.stop != nullptr;
   if (has_long && phase == kEngineAll && t.n_q * t.n_batch <= kWholeRowsMaxRows &&
       t.kv_stride <= kWholeRowsMaxKeys * (int64_t)t.d && s.nnz_bound <= kWholeRowsMaxEntries) {
     const int64_t grid = (t.n_q * t.n_batch + kWholeRowsWaves - 1) / kWholeRowsWaves;
-    if (timed) (void)hipEventRecord(ev.start, stream);
-    hipLaunchKernelGGL((whole_rows_kernel<Lay, Mask>), dim3((unsigned)grid), dim3(kWholeRowsWaves * kWave), 0,
-                       stream, t, mask, use_nan);
-    if (timed) (void)hipEventRecord(ev.stop, stream);
+    launch_maybe_timed(ev, whole_rows_kernel<Lay, Mask>, dim3((unsigned)grid), dim3(kWholeRowsWaves * kWave),
+                       stream, t, mask, use_nan, device_status_word());
     return hipGetLastError() == hipSuccess ? 0 : 4;
   }
   if (has_long && phase != kEngineRunOnly) {
@@ -814,10 +847,8 @@ int launch_engine(const Tensors& t, const Mask& mask, const EngineSizing& s, int
 
   const int64_t rows_per_wg = 4 * Lay::GROUPS;
   const int64_t grid1 = (t.n_q * t.n_batch + rows_per_wg - 1) / rows_per_wg;
-  if (timed && !has_long) (void)hipEventRecord(ev.start, stream);
-  hipLaunchKernelGGL((rows_kernel<Lay, Mask>), dim3((unsigned)grid1), dim3(256), 0, stream, t, mask,
-                     plan);
-  if (timed && !has_long) (void)hipEventRecord(ev.stop, stream);
+  launch_maybe_timed(has_long ? KernelEvents{} : ev, rows_kernel<Lay, Mask>, dim3((unsigned)grid1), dim3(256),
+                     stream, t, mask, plan);
   if (has_long && w.cap_medium > 0) {
     const int64_t gridm = ((int64_t)w.cap_medium * t.n_batch + 3) / 4;
     hipLaunchKernelGGL((medium_rows_kernel<Lay, Mask>), dim3((unsigned)gridm), dim3(256), 0, stream, t,
@@ -831,10 +862,8 @@ int launch_engine(const Tensors& t, const Mask& mask, const EngineSizing& s, int
     int64_t need = ((int64_t)w.cap_items * t.n_batch + 3) / 4;
     if (grid2 > need) grid2 = need;
     if (grid2 < 1) grid2 = 1;
-    if (timed) (void)hipEventRecord(ev.start, stream);
-    hipLaunchKernelGGL((segments_kernel<Lay, Mask>), dim3((unsigned)grid2), dim3(256), 0, stream, t,
-                       mask, plan);
-    if (timed) (void)hipEventRecord(ev.stop, stream);
+    launch_maybe_timed(ev, segments_kernel<Lay, Mask>, dim3((unsigned)grid2), dim3(256), stream, t, mask,
+                       plan);
     const int64_t grid3 = ((int64_t)w.cap_multi * t.n_batch + rows_per_wg - 1) / rows_per_wg;
     hipLaunchKernelGGL((merge_kernel<Lay>), dim3((unsigned)grid3), dim3(256), 0, stream, t, plan);
   }

@@ -221,7 +221,11 @@ __global__ __launch_bounds__(256, (grad_tile_min_blocks<T, D, KEYS>())) void til
   auto streamed_row = [&](int64_t u) -> int64_t {
     if constexpr (MODE == kTileBand) return base + u * a.s;
     else if constexpr (MODE == kTileGlobalRows) return u + tok_off;
-    else return (int64_t)(KEYS ? a.uq[u] : a.globs[u]) + tok_off;
+    else {
+      // (an out-of-range listed entry reads row 0 and is masked below)
+      const int g = KEYS ? a.uq[u] : listed_token(a.globs[u], a.n);
+      return (int64_t)(g < 0 ? 0 : g) + tok_off;
+    }
   };
   auto fetch = [&](int64_t ut) {
 #pragma unroll
@@ -245,7 +249,8 @@ __global__ __launch_bounds__(256, (grad_tile_min_blocks<T, D, KEYS>())) void til
         lse_reg = ok ? g.lse[row] * 1.4426950408889634f : __builtin_inff();
         delta_reg = ok ? g.delta[row] : 0.f;
       }
-      if constexpr (MODE == kTileGlobalCols) ktok_reg = ok ? (int)(row - tok_off) : 0;
+      if constexpr (MODE == kTileGlobalCols)
+        ktok_reg = ok ? (KEYS ? (int)(row - tok_off) : listed_token(a.globs[ut + tid], a.n)) : 0;
       if constexpr (MODE == kTileGlobalRows && KEYS)
         once_reg = (ok && bit_is_set(a.gbits, row - tok_off)) ? 1.f : 0.f;
     }
@@ -370,7 +375,7 @@ __global__ __launch_bounds__(256, (grad_tile_min_blocks<T, D, KEYS>())) void til
           if (!full) {
             bool ok;
             if constexpr (MODE == kTileGlobalRows) ok = (d0 + (uint32_t)j > w2) && (j < rem);
-            else ok = (d0 + (uint32_t)ktok_s[j] > w2) && (j < rem);
+            else ok = (d0 + (uint32_t)ktok_s[j] > w2) && (j < rem) && ktok_s[j] >= 0;
             p = ok ? p : 0.f;
           }
         }

@@ -11,12 +11,17 @@ namespace spfa {
 // (reference: Sparse_FlashAttention_CSR/sp_flatt_csr_kernel.cu:29-33,117).
 struct CsrMask {
   static constexpr bool kWeighted = false;  // every candidate counts once
+  static constexpr bool kExplicit = true;   // the mask lives in arrays that can be inconsistent
   const void* row_off;
   const uint32_t* cols;
   int32_t off64;  // row_off entries are 8 bytes wide (else 4)
   // COO only: when *use_alt != 0 the columns are read from alt_cols (the bucketed copy) instead
   const uint32_t* alt_cols;
   const uint32_t* use_alt;
+  // Bounds the arrays are held to, so that inconsistent mask arrays cannot send a load outside
+  // the tensors: a row's range is cut to [0, nnz) and a column >= n_cols is masked.
+  int64_t nnz;
+  int64_t n_cols;
   struct Row {
     int64_t start;
     int64_t deg;
@@ -35,10 +40,28 @@ struct CsrMask {
     }
     const uint32_t* cp = cols;
     if (use_alt != nullptr && *use_alt != 0u) cp = alt_cols;
+    if (b > nnz) b = nnz;
+    if (a > b) a = b;
     return Row{a, b - a, cp};
   }
-  __device__ __forceinline__ int64_t col(const Row& r, int64_t t, bool&) const {
-    return (int64_t)r.cols[r.start + t];
+  __device__ __forceinline__ int64_t col(const Row& r, int64_t t, bool& valid) const {
+    const int64_t c = (int64_t)r.cols[r.start + t];
+    valid = c < n_cols;
+    return c;
+  }
+  // the row's offsets as stored, for consistency checks: 0 <= start <= end <= nnz
+  __device__ __forceinline__ bool consistent(int64_t i) const {
+    int64_t a, b;
+    if (off64) {
+      const uint64_t* p = (const uint64_t*)row_off;
+      a = (int64_t)p[i];
+      b = (int64_t)p[i + 1];
+    } else {
+      const uint32_t* p = (const uint32_t*)row_off;
+      a = (int64_t)p[i];
+      b = (int64_t)p[i + 1];
+    }
+    return a >= 0 && a <= b && b <= nnz;
   }
 };
 
@@ -51,6 +74,7 @@ struct CsrMask {
 //               (Sparse_FlashAttention_Local_2D_Dilated/sp_flatt_local_2d_dilated_kernel.cu:26-39,123).
 struct StrideMask {
   static constexpr bool kWeighted = false;
+  static constexpr bool kExplicit = false;
   int64_t n;
   int64_t w;
   int64_t s;
@@ -84,6 +108,7 @@ struct StrideMask {
 // Bit i of gbits marks the listed rows.
 struct GlobalMask {
   static constexpr bool kWeighted = false;
+  static constexpr bool kExplicit = false;
   int64_t n;
   int64_t w;
   const int32_t* globs;
@@ -106,7 +131,7 @@ struct GlobalMask {
   __device__ __forceinline__ int64_t col(const Row& r, int64_t t, bool& valid) const {
     if (r.glob) return t < r.low ? t : t + (r.up - r.low);
     int64_t c = (int64_t)globs[t];
-    valid = (c < r.low) || (c >= r.up);
+    valid = c >= 0 && c < n && ((c < r.low) || (c >= r.up));  // (an out-of-range entry is masked)
     return c;
   }
 };
@@ -118,6 +143,7 @@ struct GlobalMask {
 //   other columns:    the distinct listed rows outside the window, once each.
 struct GlobalColMask {
   static constexpr bool kWeighted = true;
+  static constexpr bool kExplicit = false;
   int64_t n;
   int64_t w;
   const int32_t* globs;   // the list as given (duplicates allowed)

@@ -380,7 +380,10 @@ __global__ __launch_bounds__(256, 2) void tile_kernel(TileArgs a) {
   auto key_tok = [&](int64_t u) -> int64_t {
     if constexpr (MODE == kTileBand) return base + u * a.s;
     else if constexpr (MODE == kTileGlobalRows) return u + tok_off;
-    else return (int64_t)a.globs[u] + tok_off;
+    else {
+      const int g = listed_token(a.globs[u], a.n);  // (an out-of-range entry reads row 0, masked below)
+      return (int64_t)(g < 0 ? 0 : g) + tok_off;
+    }
   };
   constexpr int CH = kF32 ? D / 4 : D / 8;       // 16-byte chunks per row
   constexpr int KIT = BN * CH / 256;             // chunks of K per thread and tile
@@ -418,7 +421,7 @@ __global__ __launch_bounds__(256, 2) void tile_kernel(TileArgs a) {
       }
     }
     if constexpr (MODE == kTileGlobalCols) {
-      if (tid < BN) ktok_reg = (ut + tid < u_hi) ? a.globs[ut + tid] : 0;
+      if (tid < BN) ktok_reg = (ut + tid < u_hi) ? listed_token(a.globs[ut + tid], a.n) : 0;
     }
   };
 
@@ -550,7 +553,7 @@ __global__ __launch_bounds__(256, 2) void tile_kernel(TileArgs a) {
         // keys are listed tokens, queries the tokens tw0 .. tw0+31: live unless one of the
         // block's keys lies in the window of one of them
         const int64_t kt = (int64_t)ktok_s[32 * jb + r];
-        const bool hit = (kt + a.w >= tw0) && (kt <= tw0 + 31 + a.w);
+        const bool hit = kt < 0 || ((kt + a.w >= tw0) && (kt <= tw0 + 31 + a.w));
         full = (32 * jb + 31 < rem) && (__builtin_amdgcn_ballot_w64(hit) == 0);
       }
       if (!full) {
@@ -560,7 +563,7 @@ __global__ __launch_bounds__(256, 2) void tile_kernel(TileArgs a) {
           bool ok;
           if constexpr (MODE == kTileBand) ok = (d0 + (uint32_t)j <= w2);
           else if constexpr (MODE == kTileGlobalRows) ok = (d0 + (uint32_t)j > w2);
-          else ok = (d0 + (uint32_t)ktok_s[j] > w2);
+          else ok = (d0 + (uint32_t)ktok_s[j] > w2) && ktok_s[j] >= 0;
           if (!(ok && j < rem)) sreg[jb][v] = kNegInf;
         }
       }
@@ -1433,19 +1436,17 @@ __global__ __launch_bounds__(256) void global_rows_merge_kernel(TileArgs a) {
 template <typename T, int D>
 int launch_band_tiles(const TileArgs& a, int use_nan, hipStream_t stream) {
   const KernelEvents ev = kernel_events();
-  const bool timed = ev.start != nullptr && ev.stop != nullptr;
   if (a.n_tiles > 0) {
     const int64_t grid = (a.n_tiles * a.t.n_batch + 7) / 8 * 8;
-    if (timed) (void)hipEventRecord(ev.start, stream);
     if constexpr (sizeof(T) == 2) {
       // the direct-to-LDS kernel addresses a tile's rows with 32-bit offsets
       // and windows / positions with 32-bit arithmetic
       const int64_t max_len = a.block > 0 ? a.cnt : (a.n + a.s - 1) / a.s;
       if (a.s * (int64_t)(2 * D) * 64 < ((int64_t)1 << 31) &&
           (a.w <= (int64_t)0x3fffffff || max_len <= (int64_t)0x3fffffff))
-        hipLaunchKernelGGL((band_dma_kernel<T, D>), dim3((unsigned)grid), dim3(256), 0, stream, a);
+        launch_maybe_timed(ev, band_dma_kernel<T, D>, dim3((unsigned)grid), dim3(256), stream, a);
       else
-        hipLaunchKernelGGL((tile_kernel<T, D, kTileBand>), dim3((unsigned)grid), dim3(256), 0, stream, a);
+        launch_maybe_timed(ev, tile_kernel<T, D, kTileBand>, dim3((unsigned)grid), dim3(256), stream, a);
     } else {
       // Two workgroups fit a CU, and tiles take about the same time, so the grid runs in rounds
       // of `resident` tiles and the tiles of a last, sparsely filled round keep the chip
@@ -1467,13 +1468,12 @@ int launch_band_tiles(const TileArgs& a, int use_nan, hipStream_t stream) {
       const int64_t n_main = n_all - at.n_tail;
       if (dma) {
         const int64_t grid_d = (n_main + 7) / 8 * 8 + 4 * at.n_tail;
-        hipLaunchKernelGGL((band_dma_f32_kernel<D>), dim3((unsigned)grid_d), dim3(256), 0, stream, at);
+        launch_maybe_timed(ev, band_dma_f32_kernel<D>, dim3((unsigned)grid_d), dim3(256), stream, at);
       } else {
         const int64_t grid_t = (n_main + 7) / 8 * 8 + 4 * at.n_tail;
-        hipLaunchKernelGGL((tile_kernel<T, D, kTileBand>), dim3((unsigned)grid_t), dim3(256), 0, stream, at);
+        launch_maybe_timed(ev, tile_kernel<T, D, kTileBand>, dim3((unsigned)grid_t), dim3(256), stream, at);
       }
     }
-    if (timed) (void)hipEventRecord(ev.stop, stream);
   }
   if (a.block > 0 && use_nan && a.s > 1) {
     const int64_t rows = a.n * a.t.n_batch;
@@ -1489,7 +1489,6 @@ int launch_band_tiles(const TileArgs& a, int use_nan, hipStream_t stream) {
 template <typename T, int D>
 int launch_global_tiles(const TileArgs& a, hipStream_t stream) {
   const KernelEvents ev = kernel_events();
-  const bool timed = ev.start != nullptr && ev.stop != nullptr;
   int64_t grid_cols = (a.n + 127) / 128;
   TileArgs ac = a;
   ac.persist = (a.n_globs <= TileCfg<T, D>::BN) ? 1 : 0;
@@ -1507,10 +1506,8 @@ int launch_global_tiles(const TileArgs& a, hipStream_t stream) {
   const int64_t q_tiles = (a.n_globs + 127) / 128;
   TileArgs ar = a;
   ar.pair_split = (a.n_globs <= 64 && TileCfg<T, D>::NB == 2) ? 1 : 0;
-  if (timed) (void)hipEventRecord(ev.start, stream);
-  hipLaunchKernelGGL((tile_kernel<T, D, kTileGlobalRows>), dim3((unsigned)(q_tiles * a.n_split * nb)),
-                     dim3(256), 0, stream, ar);
-  if (timed) (void)hipEventRecord(ev.stop, stream);
+  launch_maybe_timed(ev, tile_kernel<T, D, kTileGlobalRows>, dim3((unsigned)(q_tiles * a.n_split * nb)),
+                     dim3(256), stream, ar);
   hipLaunchKernelGGL((global_rows_merge_kernel<T, D>), dim3((unsigned)(a.n_globs * nb)), dim3(256), 0,
                      stream, a);
   return hipGetLastError() == hipSuccess ? 0 : 4;

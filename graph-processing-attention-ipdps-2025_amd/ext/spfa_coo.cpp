@@ -28,7 +28,7 @@ torch::Tensor spfa_coo_forward_py(torch::Tensor Q, torch::Tensor K, torch::Tenso
   spfa_ext::index_bytes(W_col_ind, "W_col_ind", false);
   const int64_t nnz = W_col_ind.size(0);
 
-  const size_t ws_bytes = spfa_ext::batched(spfa_coo_workspace_bytes(p.n_q, nnz, p.d, p.dtype), p);
+  const size_t ws_bytes = spfa_coo_workspace_bytes_batched(p.n_q, nnz, p.d, p.dtype, p.n_batch);
   torch::Tensor ws = spfa_ext::make_workspace(ws_bytes, Q);
   spfa_ext::raise_on_error(spfa_coo_forward(&p, W_row_ind.data_ptr(), row_bytes, W_col_ind.data_ptr(),
                                             nnz, use_nan ? 1 : 0, ws.data_ptr(), (size_t)ws.numel(),
@@ -85,7 +85,7 @@ torch::Tensor spfa_coo_forward_planned_py(torch::Tensor Q, torch::Tensor K, torc
   const int64_t nnz = W_col_ind.size(0);
 
   // (the attention part of the plain call's workspace would do; the plain size is simply enough)
-  const size_t ws_bytes = spfa_ext::batched(spfa_csr_workspace_bytes(p.n_q, nnz, p.d, p.dtype), p);
+  const size_t ws_bytes = spfa_csr_workspace_bytes_batched(p.n_q, nnz, p.d, p.dtype, p.n_batch);
   torch::Tensor ws = spfa_ext::make_workspace(ws_bytes, Q);
   spfa_ext::raise_on_error(spfa_coo_forward_planned(
       &p, W_col_ind.data_ptr(), nnz, use_nan ? 1 : 0, plan.data_ptr(), (size_t)plan.numel(),

@@ -29,7 +29,7 @@ torch::Tensor spfa_csr_forward_py(torch::Tensor Q, torch::Tensor K, torch::Tenso
   spfa_ext::index_bytes(W_col_ind, "W_col_ind", false);
   const int64_t nnz = W_col_ind.size(0);
 
-  const size_t ws_bytes = spfa_ext::batched(spfa_csr_workspace_bytes(p.n_q, nnz, p.d, p.dtype), p);
+  const size_t ws_bytes = spfa_csr_workspace_bytes_batched(p.n_q, nnz, p.d, p.dtype, p.n_batch);
   torch::Tensor ws = spfa_ext::make_workspace(ws_bytes, Q);
   spfa_ext::raise_on_error(spfa_csr_forward(&p, W_row_off.data_ptr(), off_bytes, W_col_ind.data_ptr(),
                                             nnz, use_nan ? 1 : 0, ws.data_ptr(), (size_t)ws.numel(),
@@ -49,6 +49,9 @@ torch::Tensor spfa_csr_plan_py(torch::Tensor W_row_off, torch::Tensor W_col_ind)
   const int off_bytes = spfa_ext::index_bytes(W_row_off, "W_row_off", true);
   spfa_ext::index_bytes(W_col_ind, "W_col_ind", false);
   const int64_t n_q = W_row_off.size(0) - 1, nnz = W_col_ind.size(0);
+  // a plan is built once and used many times: worth one look at the data (this synchronises)
+  TORCH_CHECK(spfa_ext::index_value(W_row_off, n_q) == nnz,
+              "W_row_off must end at the number of entries of W_col_ind");
   torch::Tensor plan = spfa_ext::make_workspace(spfa_csr_plan_bytes(n_q, nnz), W_row_off);
   spfa_ext::raise_on_error(spfa_csr_plan(n_q, W_row_off.data_ptr(), off_bytes, W_col_ind.data_ptr(), nnz,
                                          plan.data_ptr(), (size_t)plan.numel(),
@@ -82,7 +85,7 @@ torch::Tensor spfa_csr_forward_planned_py(torch::Tensor Q, torch::Tensor K, torc
   spfa_ext::index_bytes(W_col_ind, "W_col_ind", false);
   const int64_t nnz = W_col_ind.size(0);
 
-  const size_t ws_bytes = spfa_ext::batched(spfa_csr_workspace_bytes(p.n_q, nnz, p.d, p.dtype), p);
+  const size_t ws_bytes = spfa_csr_workspace_bytes_batched(p.n_q, nnz, p.d, p.dtype, p.n_batch);
   torch::Tensor ws = spfa_ext::make_workspace(ws_bytes, Q);
   spfa_ext::raise_on_error(spfa_csr_forward_planned(
       &p, W_row_off.data_ptr(), off_bytes, W_col_ind.data_ptr(), nnz, use_nan ? 1 : 0, plan.data_ptr(),
@@ -177,4 +180,9 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, mod) {
           py::arg("m"), py::arg("l"), py::arg("O"), py::arg("dO"), py::arg("dQ"), py::arg("dK"),
           py::arg("dV"), py::arg("t_row_off") = py::none(), py::arg("t_col_ind") = py::none());
   mod.def("transpose", &spfa_csr_transpose_py, "The CSR mask read by column, for backward(...)");
+  mod.def("device_status", &spfa_ext::device_status,
+          "Bits the kernels set on the current device when mask arrays were inconsistent "
+          "(1: more long-row entries than W_col_ind holds, 2: row offsets decreasing or beyond its "
+          "size); synchronise first",
+          py::arg("reset") = false);
 }

@@ -120,6 +120,24 @@ inline spfa_grads_t make_grads(const torch::Tensor& Q, const torch::Tensor& K, c
   CHECK_INPUT(dK);               \
   CHECK_INPUT(dV)
 
+// Entry i of an integer index tensor on the device, read back to the host (synchronises).
+inline int64_t index_value(const torch::Tensor& t, int64_t i) {
+  const torch::Tensor x = t.narrow(0, i, 1).cpu();
+  switch (x.scalar_type()) {
+    case torch::kInt32: return (int64_t)*x.data_ptr<int32_t>();
+    case torch::kUInt32: return (int64_t)*(const uint32_t*)x.data_ptr();
+    case torch::kInt64: return *x.data_ptr<int64_t>();
+    default: return (int64_t)*(const uint64_t*)x.data_ptr();
+  }
+}
+
+// the status word of the current device (spfa_device_status)
+inline int64_t device_status(bool reset) {
+  const int bits = spfa_device_status(reset ? 1 : 0);
+  TORCH_CHECK(bits >= 0, "the device status word cannot be read");
+  return bits;
+}
+
 // workspace of a (possibly batched) call: the single-problem size times the batch count
 inline size_t batched(size_t bytes, const spfa_problem_t& p) {
   return bytes * (size_t)(p.n_batch > 1 ? p.n_batch : 1);

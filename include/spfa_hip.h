@@ -86,6 +86,24 @@ typedef struct spfa_problem {
 int spfa_version(void);
 const char* spfa_status_string(int status);
 
+/* What the kernels found wrong with mask arrays they can only look at on the device.  The
+ * reference checks nothing there (sp_flatt_csr_kernel.cu:271-287 launches on whatever row_off and
+ * col_ind hold, and reads out of bounds when they disagree).  Here the explicit-mask kernels hold
+ * the arrays to the sizes the call states - a row's range is cut to [0, nnz), a column >= n_k is
+ * masked, COO entries with a row >= n_q are dropped, listed global tokens outside [0, n) are
+ * masked - so inconsistent arrays cannot send a load outside the tensors; rows hit by an
+ * inconsistency are computed on what is left of them or left untouched, and the call still
+ * returns SPFA_OK because the host never sees device data.  Each device keeps a sticky word that
+ * the CSR / COO kernels OR these bits into (only calls with nnz > 32 look):
+ *   SPFA_STATUS_WORK_LIST_OVERFLOW  the row offsets describe more long-row entries than the nnz
+ *                                   passed; every long row of that call was left untouched
+ *   SPFA_STATUS_ROW_OFFSETS         some row's offsets decrease or end beyond nnz
+ * spfa_device_status returns the current device's word (>= 0; reset != 0 clears it), or -1 when it
+ * cannot be read.  It copies from the device: synchronise the streams of the calls in question
+ * first. */
+enum { SPFA_STATUS_WORK_LIST_OVERFLOW = 1, SPFA_STATUS_ROW_OFFSETS = 2 };
+int spfa_device_status(int reset);
+
 /* Measurement aid; no counterpart in the reference.  While both handles are non-NULL
  * (hipEvent_t passed as void*), every forward call records `start` on its stream immediately
  * before, and `stop` immediately after, the launch of the kernel that does the bulk of the
@@ -93,6 +111,19 @@ const char* spfa_status_string(int status);
  * benchmark can time that one kernel with hipEventElapsedTime.  Process-wide and not
  * thread-safe: set it, run, read the events, reset it with NULLs. */
 void spfa_set_kernel_events(void* start, void* stop);
+
+/* Measurement aid; no counterpart in the reference.  The gather of the explicit-mask kernels with
+ * the arithmetic taken out: for each of the n_idx entries of `idx` (values < n_rows; entries with
+ * the top bit set are skipped) one row of `row_bytes` (64, 128, 256 or 512) bytes is loaded from
+ * `k` and one from `v`, 16 bytes per lane, `in_flight` (4, 8, 16 or 32) rows of each per lane group
+ * issued back to back, by a persistent grid of wg_per_cu (1..8) four-wavefront workgroups per
+ * compute unit whose wavefronts pull runs of `chunk` (>= 64) entries off an atomic cursor
+ * (`cursor`: 4 bytes of device memory).  Nothing is computed or written.  Timed by the caller
+ * with events on `stream`, it gives the rate the memory system sustains for this access pattern
+ * at a given working-set size: the ceiling a gather-bound kernel is priced against. */
+int spfa_probe_gather(const void* k, const void* v, int64_t n_rows, int64_t row_bytes,
+                      const uint32_t* idx, int64_t n_idx, int64_t chunk, int wg_per_cu, int in_flight,
+                      void* cursor, void* stream);
 
 /* Rows of an explicit mask with at most this many entries are finished by the row kernels (a
  * lane group or a wavefront per row); longer rows go through the segment kernel.  Exposed so a
@@ -104,6 +135,10 @@ int64_t spfa_explicit_inline_row_limit(void);
  * index tensors are bit-identical in range.  The reference's value vector is never read
  * (sp_flatt_csr_kernel.cu:21) and is not part of this interface. */
 size_t spfa_csr_workspace_bytes(int64_t n_q, int64_t nnz, int64_t d, int dtype);
+/* ... of a call with p->n_batch == n_batch: the exact size (the work list is shared by the
+ * problems of a batch, only the partial results are per problem); n_batch times the
+ * single-problem size is always enough too. */
+size_t spfa_csr_workspace_bytes_batched(int64_t n_q, int64_t nnz, int64_t d, int dtype, int64_t n_batch);
 int spfa_csr_forward(const spfa_problem_t* p, const void* row_off, int row_off_bytes,
                      const void* col_ind, int64_t nnz, int use_nan, void* workspace,
                      size_t workspace_bytes, void* stream);
@@ -129,6 +164,8 @@ int spfa_csr_forward_static(const spfa_problem_t* p, const void* row_off, int ro
  * reference needs them sorted by row, sp_flatt_coo_kernel.cu:47-79); they are bucketed by
  * row on the device first.  row_ind entries are row_ind_bytes (4 or 8) bytes wide. */
 size_t spfa_coo_workspace_bytes(int64_t n_q, int64_t nnz, int64_t d, int dtype);
+/* ... of a batched call (the conversion's scratch is needed once, not per problem) */
+size_t spfa_coo_workspace_bytes_batched(int64_t n_q, int64_t nnz, int64_t d, int dtype, int64_t n_batch);
 int spfa_coo_forward(const spfa_problem_t* p, const void* row_ind, int row_ind_bytes,
                      const void* col_ind, int64_t nnz, int use_nan, void* workspace,
                      size_t workspace_bytes, void* stream);

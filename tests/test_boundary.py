@@ -216,3 +216,42 @@ def test_stacked_per_head_masks_form_a_block_diagonal():
     assert np.array_equal(ro.to(torch.int64).numpy(), ro_ref) and np.array_equal(ci.to(torch.int64).numpy(), ci_ref)
     with pytest.raises(ValueError):
         spfa_masks.stack_csr_masks([], n_k)
+
+
+def test_implicit_masks_need_as_many_keys_as_queries(lib):
+    """The band and global masks index K and V by query token: a problem with fewer K rows than Q
+    rows is refused on the host (after the reference's own parameter checks)."""
+    i64 = ctypes.c_int64
+    p = Problem(None, None, None, None, None, None, 16, 8, 8, 0, 0, 1)
+    r = ctypes.byref(p)
+    assert lib.spfa_local_forward(r, i64(3), None, 0, None) == 1
+    assert lib.spfa_local_1d_dilated_forward(r, i64(3), i64(1), None, 0, None) == 1
+    assert lib.spfa_local_2d_dilated_forward(r, i64(4), i64(1), 0, None, 0, None) == 1
+    assert lib.spfa_global_no_local_forward(r, None, i64(2), i64(1), None, 0, None) == 1
+    # the reference's checks still come first
+    assert lib.spfa_local_forward(r, i64(16), None, 0, None) == 6
+
+
+def test_batched_workspace_queries_share_the_mask_scratch(lib):
+    for name in ("spfa_csr_workspace_bytes_batched", "spfa_coo_workspace_bytes_batched"):
+        getattr(lib, name).restype = ctypes.c_size_t
+        getattr(lib, name).argtypes = [ctypes.c_int64, ctypes.c_int64, ctypes.c_int64, ctypes.c_int, ctypes.c_int64]
+    for name in ("spfa_csr_workspace_bytes", "spfa_coo_workspace_bytes"):
+        getattr(lib, name).argtypes = [ctypes.c_int64, ctypes.c_int64, ctypes.c_int64, ctypes.c_int]
+    n, nnz, d = 1 << 20, 50_000_000, 64
+    for kind in ("csr", "coo"):
+        one = getattr(lib, "spfa_%s_workspace_bytes" % kind)(n, nnz, d, 0)
+        assert getattr(lib, "spfa_%s_workspace_bytes_batched" % kind)(n, nnz, d, 0, 1) == one
+        eight = getattr(lib, "spfa_%s_workspace_bytes_batched" % kind)(n, nnz, d, 0, 8)
+        assert one < eight <= 8 * one
+    # COO: the conversion's scratch (about 0.65 GB here) is counted once, not per problem
+    coo1 = lib.spfa_coo_workspace_bytes(n, nnz, d, 0)
+    csr1 = lib.spfa_csr_workspace_bytes(n, nnz, d, 0)
+    assert lib.spfa_coo_workspace_bytes_batched(n, nnz, d, 0, 8) - lib.spfa_csr_workspace_bytes_batched(n, nnz, d, 0, 8) \
+        == coo1 - csr1
+
+
+def test_status_word_query_needs_a_device(lib):
+    import torch
+    if not torch.cuda.is_available():
+        assert lib.spfa_device_status(0) == -1
