@@ -427,7 +427,7 @@ def measured_traffic(workload, dtype_name):
     workload (profiles/<workload>..._pmc.md, line `traffic_bytes_per_launch = N`), else None."""
     import glob
     import re
-    names = {"csr_zipf": "csr_zipf_n131072_d64"}
+    names = {"csr_zipf": "csr_zipf_n131072_d64", "coo_zipf": "coo_zipf_unsorted_n1048576_d64"}
     stem = names.get(workload)
     if stem is None:
         return None
