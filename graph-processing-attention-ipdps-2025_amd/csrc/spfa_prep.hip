@@ -191,20 +191,26 @@ constexpr int kPartThreads = 1024;
 constexpr int kPartTile = 16384;     // entries per workgroup in pass 1
 constexpr int kPartMaxBuckets = 2048;
 
-// pass 1a: per-tile histogram of the high digit, stored bucket-major: hist[b * n_tiles + tile]
+// pass 1a: per-tile histogram of the high digit, stored bucket-major: hist[b * n_tiles + tile].
+// The same pass over the row indices decides whether the entries need bucketing at all: it sets
+// *flag when they are not sorted by row or hold a row outside [0, n_rows) (so the sortedness check
+// costs no pass of its own; for sorted entries the histogram is simply not used).
 __global__ __launch_bounds__(kPartThreads) void coo_part_count_kernel(
     const void* row_ind, int wide, int64_t nnz, int64_t n_rows, int lo_bits, int n_hi,
-    int64_t n_tiles, const uint32_t* flag, uint32_t* hist) {
+    int64_t n_tiles, uint32_t* flag, uint32_t* hist) {
   __shared__ uint32_t cnt[kPartMaxBuckets];
-  if (!*flag) return;
   for (int b = threadIdx.x; b < n_hi; b += kPartThreads) cnt[b] = 0;
   __syncthreads();
   const int64_t beg = (int64_t)blockIdx.x * kPartTile;
   const int64_t end = beg + kPartTile < nnz ? beg + kPartTile : nnz;
+  bool bad = false;
   for (int64_t e = beg + threadIdx.x; e < end; e += kPartThreads) {
     const int64_t r = load_index(row_ind, e, wide);
     if (r >= 0 && r < n_rows) atomicAdd(&cnt[r >> lo_bits], 1u);
+    else bad = true;
+    if (e > 0 && load_index(row_ind, e - 1, wide) > r) bad = true;
   }
+  if (bad) *flag = 1u;
   __syncthreads();
   for (int b = threadIdx.x; b < n_hi; b += kPartThreads) hist[(int64_t)b * n_tiles + blockIdx.x] = cnt[b];
 }
@@ -436,14 +442,20 @@ int coo_to_csr(const void* row_ind, int row_wide, const uint32_t* col_ind, int64
   hipLaunchKernelGGL(fill_u32_kernel, dim3(grid_for(n_rows + 1, 256, 4096)), dim3(256), 0, stream,
                      counts, n_rows + 1, 0u);
   hipLaunchKernelGGL(fill_u32_kernel, dim3(1), dim3(64), 0, stream, flag, (int64_t)1, 0u);
-  if (nnz > 0)
+  // sorted or not: decided on the device (by the first pass of the partition where there is one)
+  const bool part = nnz > 0 && w.partition;
+  if (part)
+    hipLaunchKernelGGL(coo_part_count_kernel, dim3((unsigned)w.n_tiles1), dim3(kPartThreads), 0, stream,
+                       row_ind, row_wide, nnz, n_rows, w.lo_bits, (int)w.n_hi, w.n_tiles1, flag,
+                       (uint32_t*)(base + w.off_hist));
+  else if (nnz > 0)
     hipLaunchKernelGGL(coo_check_sorted_kernel, dim3(grid_for(nnz, 256, 8192)), dim3(256), 0, stream,
                        row_ind, row_wide, nnz, n_rows, flag);
   // sorted: offsets straight from the row array
   hipLaunchKernelGGL(coo_sorted_offsets_kernel, dim3(grid_for(nnz + 1, 256, 16384)), dim3(256), 0,
                      stream, row_ind, row_wide, nnz, n_rows, flag, row_off);
   // unsorted: bucket by row
-  if (nnz > 0 && w.partition) {
+  if (part) {
     uint32_t* hist = (uint32_t*)(base + w.off_hist);
     uint64_t* tmp_pairs = (uint64_t*)(base + w.off_tmp_pairs);
     // 152 KB of LDS per workgroup: above the 64 KB a kernel gets without asking (set once per
@@ -461,8 +473,6 @@ int coo_to_csr(const void* row_ind, int row_wide, const uint32_t* col_ind, int64
     }
     const int64_t n_hist = w.n_hi * w.n_tiles1;
     const int64_t hist_tiles = (n_hist + kScanTile - 1) / kScanTile;
-    hipLaunchKernelGGL(coo_part_count_kernel, dim3((unsigned)w.n_tiles1), dim3(kPartThreads), 0, stream,
-                       row_ind, row_wide, nnz, n_rows, w.lo_bits, (int)w.n_hi, w.n_tiles1, flag, hist);
     hipLaunchKernelGGL(scan_tile_sums_kernel, dim3((unsigned)hist_tiles), dim3(kScanThreads), 0, stream,
                        hist, n_hist, tiles, flag);
     hipLaunchKernelGGL(scan_sums_kernel, dim3(1), dim3(kScanThreads), 0, stream, tiles, hist_tiles, flag);
