@@ -121,6 +121,20 @@ __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
   return __builtin_bit_cast(uint32_t, x);
 }
 
+// acc + lo + hi of a packed pair of half-type values
+template <typename T>
+__device__ __forceinline__ float dot2_ones(uint32_t pk, float acc) {
+  if constexpr (__is_same(T, bf16)) {
+    typedef __bf16 b2 __attribute__((ext_vector_type(2)));
+    const b2 ones = {(__bf16)1.0f, (__bf16)1.0f};
+    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(b2, pk), ones, acc, false);
+  } else {
+    typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+    const h2 ones = {(_Float16)1.0f, (_Float16)1.0f};
+    return __builtin_amdgcn_fdot2(__builtin_bit_cast(h2, pk), ones, acc, false);
+  }
+}
+
 template <bool B>
 struct BoolConst {
   static constexpr bool value = B;
@@ -739,8 +753,9 @@ __global__ __launch_bounds__(256, 2) void tile_kernel(TileArgs a) {
 // Same tile problem and register layouts as tile_kernel<T, D, kTileBand>, different plumbing:
 //   - K and V tiles are written to LDS by the load instructions themselves (16 bytes per lane,
 //     64 lanes = 1 KB of consecutive LDS per instruction), row-major and unpadded; no staging
-//     registers, no LDS store instructions.  Two tile buffers, one barrier per tile: tile n+1 is
-//     requested right after the barrier that publishes tile n.
+//     registers, no LDS store instructions.  A ring of NBUF tile buffers, one barrier per tile:
+//     tile n + NBUF - 1 is requested right after the barrier that publishes tile n, into the
+//     buffer that tile n - 1 has left.
 //   - Rows are 128 or 256 bytes, a multiple of the bank cycle, so bank conflicts are avoided by
 //     permuting the 16-byte chunks inside a row instead of padding: chunk c of row j is stored at
 //     chunk position c ^ f(j).  K is read with 16-byte operand fetches by 8 consecutive rows at a
@@ -761,40 +776,48 @@ struct BandDmaCfg {
   static constexpr int BUF_B = 2 * TILE_B;      // K tile then V tile
   static constexpr int NI = TILE_B / 4096;      // load instructions per wavefront, tile and matrix
   static constexpr int EB = D / 32, QREGS = D / 16;
+  // Tile buffers.  A tile is requested NBUF - 1 steps before it is consumed.  A request takes
+  // about 3500 clocks to land when the whole device streams tiles (measured with the cycle
+  // counter), a step of the tile loop about 3300: with two buffers every step waits for its
+  // data.  d = 64 has room for four buffers (64 KB, two workgroups per CU); d = 128 fills 64 KB
+  // with two.
+  static constexpr int NBUF = D == 64 ? 4 : 2;
 };
+
+// s_waitcnt vmcnt(N) alone (the other counters at their maximum), gfx9 encoding
+#define SPFA_WAIT_VMCNT(N) __builtin_amdgcn_s_waitcnt(((N) & 15) | (((N) >> 4) << 14) | 0x0f70)
 
 template <typename T, int D>
 __global__ __launch_bounds__(256, 2) void band_dma_kernel(TileArgs a) {
   using C = BandDmaCfg<T, D>;
   constexpr int BM = C::BM, BN = C::BN, EB = C::EB, ROWB = C::ROWB, CH = C::CH, RPC = C::RPC;
-  constexpr int TILE_B = C::TILE_B, BUF_B = C::BUF_B, NI = C::NI;
+  constexpr int TILE_B = C::TILE_B, BUF_B = C::BUF_B, NI = C::NI, NBUF = C::NBUF;
   static_assert(sizeof(T) == 2 && (D == 64 || D == 128), "half types, d = 64 or 128");
-  // two tile buffers as two separate arrays: the compiler can then tell the loads that fill one
-  // buffer from the operand reads of the other and does not wait for the former before the latter
-  __shared__ __attribute__((aligned(1024))) char lds_even[BUF_B];
-  __shared__ __attribute__((aligned(1024))) char lds_odd[BUF_B];
+  static_assert(2 * NI * (NBUF - 1) < 64, "outstanding tile loads must fit the vmcnt field");
+  __shared__ __attribute__((aligned(1024))) char lds[NBUF * BUF_B];
 
   // workgroups are dealt round-robin to the 8 XCDs: give each XCD a contiguous run of tiles.
-  // Positions inside a subsequence fit 32 bits (there are fewer than 2^31 tokens); everything
+  // Tile numbers and positions inside a subsequence fit 32 bits (the launcher checks); everything
   // that is the same for the whole workgroup is moved to scalar registers.
   auto uni = [](int x) { return __builtin_amdgcn_readfirstlane(x); };
   // (the tiles of all problems of a batch form one list; problem bb starts at token bb * n)
-  const int64_t n_all = a.n_tiles * a.t.n_batch;
-  const int64_t per_xcd = (n_all + 7) / 8;
-  int64_t lt = (int64_t)(blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+  const uint32_t n_tiles = (uint32_t)a.n_tiles, tiles_per_sub = (uint32_t)a.tiles_per_sub;
+  const uint32_t n_all = n_tiles * (uint32_t)a.t.n_batch;
+  const uint32_t per_xcd = (n_all + 7u) / 8u;
+  uint32_t lt = (blockIdx.x % 8u) * per_xcd + blockIdx.x / 8u;
   if (lt >= n_all) return;
-  const int64_t bb = lt / a.n_tiles;
-  lt -= bb * a.n_tiles;
-  const int64_t sub = lt / a.tiles_per_sub;
-  const int tile = uni((int)(lt - sub * a.tiles_per_sub));
+  const uint32_t bb = lt / n_tiles;
+  lt -= bb * n_tiles;
+  const uint32_t sub = lt / tiles_per_sub;
+  const int tile = uni((int)(lt - sub * tiles_per_sub));
   int64_t base;
   int qlen;
   if (a.block > 0) {
-    base = sub * a.block + bb * a.n;
+    base = (int64_t)sub * a.block + (int64_t)bb * a.n;
     qlen = (int)a.cnt;
   } else {
-    base = sub + bb * a.n;
-    qlen = uni((int)((a.n - sub + a.s - 1) / a.s));
+    base = (int64_t)sub + (int64_t)bb * a.n;
+    qlen = uni((int)(((uint32_t)a.n - sub + (uint32_t)a.s - 1u) / (uint32_t)a.s));
   }
   const int wlim = (int)(a.w < (int64_t)0x3fffffff ? a.w : (int64_t)0x3fffffff);  // window, clamped
   const int t0 = tile * BM;
@@ -810,12 +833,59 @@ __global__ __launch_bounds__(256, 2) void band_dma_kernel(TileArgs a) {
   const char* Vp = (const char*)a.t.v;
   const float sc = 1.4426950408889634f / sqrtf((float)D);
 
+  // ---- tile loads: instruction `it` of this wavefront fills the 1-KB segment 4*it + wave of a
+  // tile; this lane's 16 bytes are row j0 + it * RPI, chunk position p0 of it.  The chunk
+  // permutation repeats every CH rows and an instruction covers a multiple of CH rows, so the
+  // lane's offset for instruction `it` is that of instruction 0 plus whole rows, which go into
+  // the scalar base: two offset registers serve every load.
+  constexpr int RPI = 4096 / ROWB;  // rows per load instruction of the workgroup's four wavefronts
+  static_assert(RPI % CH == 0 && (RPI / RPC) % (CH / 4) == 0, "chunk permutation must repeat per instruction");
+  const uint32_t row_step = (uint32_t)a.s * (uint32_t)ROWB;  // bytes between consecutive keys
+  const int j0 = (wave * 1024 + lane * 16) / ROWB, p0 = ((wave * 1024 + lane * 16) % ROWB) / 16;
+  const uint32_t koff = (uint32_t)j0 * row_step + (uint32_t)((p0 ^ (j0 % CH)) * 16);
+  const uint32_t voff = (uint32_t)j0 * row_step + (uint32_t)((p0 ^ (4 * ((j0 / RPC) % (CH / 4)))) * 16);
+  const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)lds;
+  // The loads are written as instructions: scalar base + 32-bit lane offset, LDS address in M0.
+  // (Through the builtin the compiler forms a 64-bit address per lane and load, and it orders the
+  // loads against LDS reads it cannot tell apart from them; the waits for the tiles are explicit
+  // below, the compiler does not know of these loads.)
+  auto request = [&](int ut, int stage) __attribute__((always_inline)) {
+    const int64_t tile_byte = (base + (int64_t)ut * a.s) * (int64_t)ROWB;  // scalar
+    const bool whole = ut + BN <= u_hi;
+#pragma unroll
+    for (int it = 0; it < NI; it++) {
+      // whole tile: this instruction's rows are added to the scalar base; last tile of a
+      // subsequence: they stay in the lane offset, where rows past the last key are replaced by
+      // the last key (finite values; they are masked out)
+      uint32_t ko = koff, vo = voff;
+      int64_t it_byte = tile_byte + (int64_t)it * RPI * (int64_t)row_step;  // scalar
+      if (!whole) {
+        // (the opaque copy keeps the compiler from precomputing these products for every
+        // instruction outside the tile loop, where they would hold registers all the time)
+        int last = u_hi - 1 - ut;
+        asm volatile("" : "+s"(last));
+        const int j = j0 + it * RPI;
+        // source row min(j, last), relative to the row j0 that koff / voff stand for (the sum is
+        // non-negative; the unsigned arithmetic wraps to it when last < j0)
+        const uint32_t rel = (uint32_t)((j > last ? last : j) - j0) * row_step;
+        ko = koff + rel;
+        vo = voff + rel;
+        it_byte = tile_byte;
+      }
+      const uint32_t lds_k = lds_base + (uint32_t)(stage * BUF_B + (4 * it + wave) * 1024);
+      asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                   :: "v"(ko), "s"(Kp + it_byte), "s"(lds_k) : "memory", "m0");
+      asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                   :: "v"(vo), "s"(Vp + it_byte), "s"(lds_k + (uint32_t)TILE_B) : "memory", "m0");
+    }
+  };
   const int tw0 = t0 + 32 * wave;  // first query of this wavefront
   const int tq = tw0 + r;          // this lane's query position
   const bool q_ok = tq < qlen;
   const int64_t q_tok = base + (int64_t)(q_ok ? tq : qlen - 1) * a.s;
 
-  // ---- Q^T operand, kept in registers
+  // ---- Q^T operand, kept in registers; the row's incoming state is read here as well, long
+  // before the write-back needs it
   uint4v qh[C::QREGS];
   {
     const T* qrow = (const T*)a.t.q + q_tok * D;
@@ -823,41 +893,16 @@ __global__ __launch_bounds__(256, 2) void band_dma_kernel(TileArgs a) {
     for (int ks = 0; ks < C::QREGS; ks++)
       qh[ks] = *reinterpret_cast<const uint4v*>(qrow + 16 * ks + 8 * h);
   }
-
-  // ---- tile loads: instruction `it` of this wavefront fills the 1-KB segment 4*it + wave of a
-  // tile; this lane's 16 bytes are row j, chunk position p of it
-  uint32_t koff[NI], voff[NI];  // byte offset of the lane's source chunk from the tile's first row
-  const uint32_t row_step = (uint32_t)a.s * (uint32_t)ROWB;  // bytes between consecutive keys
+  const float l_pre = load_state<T>(a.t.l, q_tok, a.t.state_f32 != 0);
+  const float m_pre = load_state<T>(a.t.m, q_tok, a.t.state_f32 != 0);
+  // the first NBUF - 1 tiles
 #pragma unroll
-  for (int it = 0; it < NI; it++) {
-    const int at = (4 * it + wave) * 1024 + lane * 16;
-    const int j = at / ROWB, p = (at % ROWB) / 16;
-    koff[it] = (uint32_t)j * row_step + (uint32_t)((p ^ (j % CH)) * 16);
-    voff[it] = (uint32_t)j * row_step + (uint32_t)((p ^ (4 * ((j / RPC) % (CH / 4)))) * 16);
-  }
-  auto request = [&](int ut, char* dst_buf) {
-    const int64_t tile_byte = (base + (int64_t)ut * a.s) * (int64_t)ROWB;  // scalar
-    const bool whole = ut + BN <= u_hi;
-#pragma unroll
-    for (int it = 0; it < NI; it++) {
-      uint32_t ko = koff[it], vo = voff[it];
-      if (!whole) {
-        // rows past the last key repeat the last key (finite values; they are masked out)
-        const int last = u_hi - 1 - ut;
-        const int j = ((4 * it + wave) * 1024 + lane * 16) / ROWB;
-        if (j > last) {
-          const uint32_t back = (uint32_t)(j - last) * row_step;
-          ko -= back;
-          vo -= back;
-        }
-      }
-      char* dst = dst_buf + (4 * it + wave) * 1024;
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(Kp + tile_byte + ko),
-                                       (__attribute__((address_space(3))) void*)dst, 16, 0, 0);
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(Vp + tile_byte + vo),
-                                       (__attribute__((address_space(3))) void*)(dst + TILE_B), 16, 0, 0);
-    }
-  };
+  for (int i = 0; i < NBUF - 1; i++)
+    if (u_lo + i * BN < u_hi) request(u_lo + i * BN, i);
+  // Everything asked for so far is waited for here, once: the compiler keeps count of the loads
+  // it knows (Q, the state) and would otherwise wait for them inside the tile loop with counts
+  // that make the tile requests it does not know of complete as well.
+  SPFA_WAIT_VMCNT(0);
 
   // ---- operand addresses inside a tile buffer (bytes)
   // K block jb, step ks: row 32*jb + r, chunk 2*ks + h
@@ -888,19 +933,53 @@ __global__ __launch_bounds__(256, 2) void band_dma_kernel(TileArgs a) {
   float mt = kNegInf;  // true running maximum
   float l = 0.f;       // running sum (relative to m) over this lane's half of the keys
 
-  // one tile: wait for it, publish it, request the next one into the other buffer, consume it
-  auto step = [&](int ut, const char* tb, char* other) __attribute__((always_inline)) {
-    __builtin_amdgcn_s_waitcnt(0);  // this wavefront's part of the tile has landed
-    __syncthreads();                // everyone's has, and everyone is done with the other buffer
-    if (ut + BN < u_hi) request(ut + BN, other);
+  // one tile: wait for it, publish it, request the tile NBUF - 1 steps ahead into the buffer the
+  // previous step has freed, consume it
+  auto step = [&](int ut, int stage) __attribute__((always_inline)) {
+    const char* tb = lds + stage * BUF_B;
+    // this wavefront's part of the tile has landed: the loads complete in order, and the tiles
+    // requested after this one (at most NBUF - 2) may still be under way
+    if constexpr (NBUF > 2) {
+      const int after = (u_hi - ut - 1) / BN;  // tiles behind this one
+      if (after >= 2) SPFA_WAIT_VMCNT(2 * 2 * NI);
+      else if (after == 1) SPFA_WAIT_VMCNT(2 * NI);
+      else SPFA_WAIT_VMCNT(0);
+      static_assert(NBUF <= 4, "one more case per buffer");
+    } else {
+      SPFA_WAIT_VMCNT(0);
+    }
+    __syncthreads();  // everyone's has, and everyone is done with the buffer of the previous step
 
-    // Both 32-key blocks of the tile are always computed (a block outside this wavefront's
-    // band is masked out completely; the band is much wider than a block), which keeps the
-    // tile body one straight line of code.  all_full: every (query, key) pair of the tile is
-    // live for this wavefront, no per-element test needed.
+    // What the two 32-key blocks of the tile are to this wavefront's 32 queries (all of it the
+    // same for the whole wavefront, so the code below branches on scalars).  A block is dead when
+    // no (query, key) pair of it is live; a live block needs a per-element test at its lower
+    // end when some query's window starts after the block's first key, at its upper end when
+    // some query's window (or the subsequence) ends before its last key.
     // (positions and the clamped window are below 2^30, so the sums stay inside 32 bits)
-    const bool all_full = (ut + BN <= u_hi) && (ut >= tw0 + 31 - wlim) && (ut + BN - 1 - wlim <= tw0);
-    const bool none = (tw0 >= qlen) || (ut - wlim > tw0 + 31) || (ut + BN - 1 < tw0 - wlim);
+    bool dead[2], test[2];
+#pragma unroll
+    for (int jb = 0; jb < 2; jb++) {
+      const int ub = ut + 32 * jb;
+      dead[jb] = (tw0 >= qlen) || (ub >= u_hi) || (ub - wlim > tw0 + 31) || (ub + 31 < tw0 - wlim);
+      test[jb] = dead[jb] || (ub < tw0 + 31 - wlim) || (ub + 31 - wlim > tw0) || (ub + 32 > u_hi);
+    }
+    const bool none = dead[0] && dead[1];
+
+    // The K operands of the first live block are asked for before the next tile is requested:
+    // the four wavefronts issue their tile loads in one burst right after the barrier, and the
+    // operand reads come back while that burst drains.
+    typedef short s16x4 __attribute__((ext_vector_type(4)));
+    typedef short s16x8 __attribute__((ext_vector_type(8)));
+    typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+    constexpr int QR = C::QREGS;
+    uint4v ka[QR];
+    if (!none) {
+#pragma unroll
+      for (int ks = 0; ks < QR; ks++) ka[ks] = *reinterpret_cast<const uint4v*>(tb + kadr[ks]);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    if (ut + (NBUF - 1) * BN < u_hi) request(ut + (NBUF - 1) * BN, (stage + NBUF - 1) % NBUF);
+    __builtin_amdgcn_sched_barrier(0);
     if (none) return;
 
     // key slot j of the tile is live for this lane's query iff jlo <= j <= jhi; the slots this
@@ -909,8 +988,10 @@ __global__ __launch_bounds__(256, 2) void band_dma_kernel(TileArgs a) {
     const int jlo = (tq - wlim - ut) - 4 * h;
     const int jhi_band = tq + wlim - ut;
     const int jhi = (jhi_band < live_slots - 1 ? jhi_band : live_slots - 1) - 4 * h;
-    const uint32_t span = (uint32_t)(jhi - jlo);  // jhi < jlo: wraps to a huge value, handled below
-    const bool any_live = jhi >= jlo;
+    // both ends at once: (unsigned)(c - jlo) <= jhi - jlo; a query without a live key in the tile
+    // (jhi < jlo) gets bounds that no c meets
+    const int jlo_both = jhi >= jlo ? jlo : 0x40000000;
+    const uint32_t span = jhi >= jlo ? (uint32_t)(jhi - jlo) : 0u;
 
     // One online-softmax step over a 32-key block; leaves the exponentials in s.  The
     // exponentials are taken against a reference maximum m that is only moved (and the
@@ -918,13 +999,15 @@ __global__ __launch_bounds__(256, 2) void band_dma_kernel(TileArgs a) {
     // since the reference was set: the weights then stay below 2^kSlack, the final division by
     // l cancels the reference, and the rescale is rare instead of happening on every block
     // while the maxima are still settling.  mt keeps the true maximum for the row statistics.
-    auto soft = [&](f32x16& s, int jb) {
-      if (!all_full) {
+    // The row sum is taken over the weights as the second product sees them (rounded to T), two
+    // at a time.  Masking costs a compare and a select per element at one end of the band, one
+    // more instruction when a block meets both ends (windows narrower than a block).
+    auto soft = [&](f32x16& s, int jb, bool test) {
+      if (test) {
 #pragma unroll
         for (int v = 0; v < 16; v++) {
           const int c = 32 * jb + 8 * (v / 4) + (v % 4);
-          const bool ok = any_live && ((uint32_t)(c - jlo) <= span);
-          s[v] = ok ? s[v] : kNegInf;
+          s[v] = ((uint32_t)(c - jlo_both) <= span) ? s[v] : kNegInf;
         }
       }
       float mx = s[0];
@@ -946,39 +1029,12 @@ __global__ __launch_bounds__(256, 2) void band_dma_kernel(TileArgs a) {
       const float neg_m = (m > kNegInf) ? -m : 0.f;
       float lsum = 0.f;
 #pragma unroll
-      for (int v = 0; v < 16; v++) {
-        const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(s[v], sc, neg_m));  // exp2(-inf) = 0
-        s[v] = p;
-        lsum += p;
-      }
+      for (int v = 0; v < 16; v++)
+        s[v] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[v], sc, neg_m));  // exp2(-inf) = 0
+#pragma unroll
+      for (int x = 0; x < 8; x++) lsum = dot2_ones<T>(pack2<T>(s[2 * x], s[2 * x + 1]), lsum);
       l += lsum;
     };
-
-    // Operands are fetched from LDS well ahead of the products that use them, in an order
-    // the scheduler is told to keep: all K operands of block 0, then the K operands of block 1
-    // while the S product of block 0 runs, the V operands of a block before its softmax step.
-    typedef short s16x4 __attribute__((ext_vector_type(4)));
-    typedef short s16x8 __attribute__((ext_vector_type(8)));
-    typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
-    constexpr int QR = C::QREGS;
-    const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-    uint4v ka[QR], kb[QR];
-#pragma unroll
-    for (int ks = 0; ks < QR; ks++) ka[ks] = *reinterpret_cast<const uint4v*>(tb + kadr[ks]);
-    __builtin_amdgcn_sched_barrier(0);
-    f32x16 s0 = zero16, s1 = zero16;
-#pragma unroll
-    for (int ks = 0; ks < QR; ks++) {
-      kb[ks] = *reinterpret_cast<const uint4v*>(tb + 32 * ROWB + kadr[ks]);
-      s0 = mfma16<T>(ka[ks], qh[ks], s0);
-    }
-    // one LDS read behind every matrix instruction
-#pragma unroll
-    for (int ks = 0; ks < QR; ks++) {
-      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-    }
-    __builtin_amdgcn_sched_barrier(0);
 
     // V^T operands of block jb: [sl][eb], two transposing 8-byte reads each
     auto v_fetch = [&](int jb, uint4v (&va)[2 * EB]) {
@@ -1005,24 +1061,43 @@ __global__ __launch_bounds__(256, 2) void band_dma_kernel(TileArgs a) {
       }
     };
 
+    const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     uint4v va[2 * EB];
+    // Both blocks.  Operands are fetched from LDS well ahead of the products that use them, in
+    // an order the scheduler is told to keep: the K operands of block 1 while the S product of
+    // block 0 runs, the V operands of a block before its softmax step.
+    uint4v kb[QR];
+    f32x16 s0 = zero16, s1 = zero16;
+#pragma unroll
+    for (int ks = 0; ks < QR; ks++) {
+      kb[ks] = *reinterpret_cast<const uint4v*>(tb + 32 * ROWB + kadr[ks]);
+      s0 = mfma16<T>(ka[ks], qh[ks], s0);
+    }
+    // one LDS read behind every matrix instruction
+#pragma unroll
+    for (int ks = 0; ks < QR; ks++) {
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int ks = 0; ks < QR; ks++) s1 = mfma16<T>(kb[ks], qh[ks], s1);
     v_fetch(0, va);
     __builtin_amdgcn_sched_barrier(0);
-    soft(s0, 0);
+    soft(s0, 0, test[0]);
     pv(s0, va);
     __builtin_amdgcn_sched_barrier(0);
     v_fetch(1, va);
     __builtin_amdgcn_sched_barrier(0);
-    soft(s1, 1);
+    soft(s1, 1, test[1]);
     pv(s1, va);
   };
 
-  if (u_lo < u_hi) request(u_lo, lds_even);
-  for (int ut = u_lo; ut < u_hi; ut += 2 * BN) {
-    step(ut, lds_even, lds_odd);
-    if (ut + BN < u_hi) step(ut + BN, lds_odd, lds_even);
+  // (unrolled over the buffers, so that every LDS address is a register plus a constant)
+  for (int ut = u_lo; ut < u_hi; ut += NBUF * BN) {
+#pragma unroll
+    for (int sg = 0; sg < NBUF; sg++)
+      if (ut + sg * BN < u_hi) step(ut + sg * BN, sg);
   }
 
   l += shfl_xor_f32(l, 32);
@@ -1030,7 +1105,7 @@ __global__ __launch_bounds__(256, 2) void band_dma_kernel(TileArgs a) {
     // hand the row over relative to its true maximum: (m, l, o) -> (mt, l * 2^(m - mt), o)
     // (o is divided by l later, so only l changes)
     const float shrink = __builtin_amdgcn_exp2f(m - mt);
-    tile_write_row<T, D>(a.t, q_tok, h, mt, l * shrink, o, shrink);
+    tile_write_row<T, D>(a.t, q_tok, h, mt, l * shrink, o, shrink, true, l_pre, m_pre);
   }
 }
 
@@ -1439,10 +1514,11 @@ int launch_band_tiles(const TileArgs& a, int use_nan, hipStream_t stream) {
   if (a.n_tiles > 0) {
     const int64_t grid = (a.n_tiles * a.t.n_batch + 7) / 8 * 8;
     if constexpr (sizeof(T) == 2) {
-      // the direct-to-LDS kernel addresses a tile's rows with 32-bit offsets
-      // and windows / positions with 32-bit arithmetic
+      // the direct-to-LDS kernel addresses a tile's rows with 32-bit offsets, and tile numbers,
+      // windows and positions with 32-bit arithmetic
       const int64_t max_len = a.block > 0 ? a.cnt : (a.n + a.s - 1) / a.s;
-      if (a.s * (int64_t)(2 * D) * 64 < ((int64_t)1 << 31) &&
+      if (a.s * (int64_t)(2 * D) * 64 < ((int64_t)1 << 31) && a.n < ((int64_t)1 << 31) &&
+          a.n_tiles * a.t.n_batch < ((int64_t)1 << 31) &&
           (a.w <= (int64_t)0x3fffffff || max_len <= (int64_t)0x3fffffff))
         launch_maybe_timed(ev, band_dma_kernel<T, D>, dim3((unsigned)grid), dim3(256), stream, a);
       else
