@@ -28,6 +28,22 @@ template <typename T>
 __device__ __forceinline__ float load_state(const void* p, int64_t i, bool state_f32) {
   return state_f32 ? ((const float*)p)[i] : to_f32(((const T*)p)[i]);
 }
+// The same load in two parts, for a value that is asked for long before it is needed: the raw
+// bits stay in a register and are only turned into a float where the value is used (a load that
+// is converted at once is waited for at once).
+template <typename T>
+__device__ __forceinline__ uint32_t load_state_raw(const void* p, int64_t i, bool state_f32) {
+  uint32_t raw;
+  if (state_f32) raw = ((const uint32_t*)p)[i];
+  else raw = ((const uint16_t*)p)[i];
+  return raw;
+}
+template <typename T>
+__device__ __forceinline__ float state_from_raw(uint32_t raw, bool state_f32) {
+  static_assert(sizeof(T) == 2, "two-byte state types");
+  const uint16_t lo = (uint16_t)raw;
+  return state_f32 ? __builtin_bit_cast(float, raw) : to_f32(__builtin_bit_cast(T, lo));
+}
 template <typename T>
 __device__ __forceinline__ void store_state(void* p, int64_t i, float x, bool state_f32) {
   if (state_f32) ((float*)p)[i] = x;

@@ -766,9 +766,10 @@ __global__ __launch_bounds__(256, 2) void tile_kernel(TileArgs a) {
 //   - The softmax runs per 32-key block; both S products of a tile are issued before the first
 //     softmax step, so the matrix pipe works on the second block while the vector ALU is busy
 //     with the first.
-template <typename T, int D>
+template <typename T, int D, int BN_>
 struct BandDmaCfg {
-  static constexpr int BM = 128, BN = 64;
+  static constexpr int BM = 128, BN = BN_;      // queries per workgroup, keys per tile
+  static constexpr int NB = BN / 32;            // 32-key blocks per tile
   static constexpr int ROWB = D * 2;            // bytes per K / V row
   static constexpr int CH = D / 8;              // 16-byte chunks per row
   static constexpr int RPC = 256 / ROWB;        // rows per 256-byte bank cycle
@@ -778,19 +779,26 @@ struct BandDmaCfg {
   static constexpr int EB = D / 32, QREGS = D / 16;
   // Tile buffers.  A tile is requested NBUF - 1 steps before it is consumed.  A request takes
   // about 3500 clocks to land when the whole device streams tiles (measured with the cycle
-  // counter), a step of the tile loop about 3300: with two buffers every step waits for its
-  // data.  d = 64 has room for four buffers (64 KB, two workgroups per CU); d = 128 fills 64 KB
-  // with two.
-  static constexpr int NBUF = D == 64 ? 4 : 2;
+  // counter), a 64-key step of the tile loop about 3300 at d = 128: with two buffers every step
+  // waits for its data.  Four buffers fit 64 KB (two workgroups per CU) with 64-key tiles at
+  // d = 64 and with 32-key tiles at d = 128.
+  static constexpr int NBUF = 65536 / BUF_B < 4 ? 65536 / BUF_B : 4;
+  static_assert(BN == 32 || BN == 64, "one or two 32-key blocks per tile");
+  static_assert(NI >= 1 && NBUF >= 2, "tile too small or too large");
 };
+
+// keys per tile of band_dma_kernel
+#ifndef SPFA_BAND_BN
+#define SPFA_BAND_BN(D) 64
+#endif
 
 // s_waitcnt vmcnt(N) alone (the other counters at their maximum), gfx9 encoding
 #define SPFA_WAIT_VMCNT(N) __builtin_amdgcn_s_waitcnt(((N) & 15) | (((N) >> 4) << 14) | 0x0f70)
 
-template <typename T, int D>
+template <typename T, int D, int BN_>
 __global__ __launch_bounds__(256, 2) void band_dma_kernel(TileArgs a) {
-  using C = BandDmaCfg<T, D>;
-  constexpr int BM = C::BM, BN = C::BN, EB = C::EB, ROWB = C::ROWB, CH = C::CH, RPC = C::RPC;
+  using C = BandDmaCfg<T, D, BN_>;
+  constexpr int BM = C::BM, BN = C::BN, NB = C::NB, EB = C::EB, ROWB = C::ROWB, CH = C::CH, RPC = C::RPC;
   constexpr int TILE_B = C::TILE_B, BUF_B = C::BUF_B, NI = C::NI, NBUF = C::NBUF;
   static_assert(sizeof(T) == 2 && (D == 64 || D == 128), "half types, d = 64 or 128");
   static_assert(2 * NI * (NBUF - 1) < 64, "outstanding tile loads must fit the vmcnt field");
@@ -879,12 +887,17 @@ __global__ __launch_bounds__(256, 2) void band_dma_kernel(TileArgs a) {
                    :: "v"(vo), "s"(Vp + it_byte), "s"(lds_k + (uint32_t)TILE_B) : "memory", "m0");
     }
   };
+  // the first NBUF - 1 tiles are on their way before anything else is loaded
+#pragma unroll
+  for (int i = 0; i < NBUF - 1; i++)
+    if (u_lo + i * BN < u_hi) request(u_lo + i * BN, i);
+
   const int tw0 = t0 + 32 * wave;  // first query of this wavefront
   const int tq = tw0 + r;          // this lane's query position
   const bool q_ok = tq < qlen;
   const int64_t q_tok = base + (int64_t)(q_ok ? tq : qlen - 1) * a.s;
 
-  // ---- Q^T operand, kept in registers; the row's incoming state is read here as well, long
+  // ---- Q^T operand, kept in registers; the row's incoming state is asked for here as well, long
   // before the write-back needs it
   uint4v qh[C::QREGS];
   {
@@ -893,12 +906,8 @@ __global__ __launch_bounds__(256, 2) void band_dma_kernel(TileArgs a) {
     for (int ks = 0; ks < C::QREGS; ks++)
       qh[ks] = *reinterpret_cast<const uint4v*>(qrow + 16 * ks + 8 * h);
   }
-  const float l_pre = load_state<T>(a.t.l, q_tok, a.t.state_f32 != 0);
-  const float m_pre = load_state<T>(a.t.m, q_tok, a.t.state_f32 != 0);
-  // the first NBUF - 1 tiles
-#pragma unroll
-  for (int i = 0; i < NBUF - 1; i++)
-    if (u_lo + i * BN < u_hi) request(u_lo + i * BN, i);
+  const uint32_t l_raw = load_state_raw<T>(a.t.l, q_tok, a.t.state_f32 != 0);
+  const uint32_t m_raw = load_state_raw<T>(a.t.m, q_tok, a.t.state_f32 != 0);
   // Everything asked for so far is waited for here, once: the compiler keeps count of the loads
   // it knows (Q, the state) and would otherwise wait for them inside the tile loop with counts
   // that make the tile requests it does not know of complete as well.
@@ -950,22 +959,23 @@ __global__ __launch_bounds__(256, 2) void band_dma_kernel(TileArgs a) {
     }
     __syncthreads();  // everyone's has, and everyone is done with the buffer of the previous step
 
-    // What the two 32-key blocks of the tile are to this wavefront's 32 queries (all of it the
-    // same for the whole wavefront, so the code below branches on scalars).  A block is dead when
-    // no (query, key) pair of it is live; a live block needs a per-element test at its lower
-    // end when some query's window starts after the block's first key, at its upper end when
-    // some query's window (or the subsequence) ends before its last key.
+    // What the 32-key blocks of the tile are to this wavefront's 32 queries (all of it the same
+    // for the whole wavefront, so the code below branches on scalars).  A block is dead when no
+    // (query, key) pair of it is live; a live block needs a per-element test when some query's
+    // window starts after the block's first key, or some query's window (or the subsequence)
+    // ends before its last key.  A dead block beside a live one is computed and masked out.
     // (positions and the clamped window are below 2^30, so the sums stay inside 32 bits)
-    bool dead[2], test[2];
+    bool test[NB];
+    bool none = true;
 #pragma unroll
-    for (int jb = 0; jb < 2; jb++) {
+    for (int jb = 0; jb < NB; jb++) {
       const int ub = ut + 32 * jb;
-      dead[jb] = (tw0 >= qlen) || (ub >= u_hi) || (ub - wlim > tw0 + 31) || (ub + 31 < tw0 - wlim);
-      test[jb] = dead[jb] || (ub < tw0 + 31 - wlim) || (ub + 31 - wlim > tw0) || (ub + 32 > u_hi);
+      const bool dead = (tw0 >= qlen) || (ub >= u_hi) || (ub - wlim > tw0 + 31) || (ub + 31 < tw0 - wlim);
+      test[jb] = dead || (ub < tw0 + 31 - wlim) || (ub + 31 - wlim > tw0) || (ub + 32 > u_hi);
+      none = none && dead;
     }
-    const bool none = dead[0] && dead[1];
 
-    // The K operands of the first live block are asked for before the next tile is requested:
+    // The K operands of the first block are asked for before the next tile is requested:
     // the four wavefronts issue their tile loads in one burst right after the barrier, and the
     // operand reads come back while that burst drains.
     typedef short s16x4 __attribute__((ext_vector_type(4)));
@@ -1063,34 +1073,46 @@ __global__ __launch_bounds__(256, 2) void band_dma_kernel(TileArgs a) {
 
     const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     uint4v va[2 * EB];
-    // Both blocks.  Operands are fetched from LDS well ahead of the products that use them, in
-    // an order the scheduler is told to keep: the K operands of block 1 while the S product of
-    // block 0 runs, the V operands of a block before its softmax step.
-    uint4v kb[QR];
-    f32x16 s0 = zero16, s1 = zero16;
+    // Operands are fetched from LDS well ahead of the products that use them, in an order the
+    // scheduler is told to keep.
+    if constexpr (NB == 2) {
+      // the K operands of block 1 while the S product of block 0 runs, the V operands of a block
+      // before its softmax step
+      uint4v kb[QR];
+      f32x16 s0 = zero16, s1 = zero16;
 #pragma unroll
-    for (int ks = 0; ks < QR; ks++) {
-      kb[ks] = *reinterpret_cast<const uint4v*>(tb + 32 * ROWB + kadr[ks]);
-      s0 = mfma16<T>(ka[ks], qh[ks], s0);
+      for (int ks = 0; ks < QR; ks++) {
+        kb[ks] = *reinterpret_cast<const uint4v*>(tb + 32 * ROWB + kadr[ks]);
+        s0 = mfma16<T>(ka[ks], qh[ks], s0);
+      }
+      // one LDS read behind every matrix instruction
+#pragma unroll
+      for (int ks = 0; ks < QR; ks++) {
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int ks = 0; ks < QR; ks++) s1 = mfma16<T>(kb[ks], qh[ks], s1);
+      v_fetch(0, va);
+      __builtin_amdgcn_sched_barrier(0);
+      soft(s0, 0, test[0]);
+      pv(s0, va);
+      __builtin_amdgcn_sched_barrier(0);
+      v_fetch(1, va);
+      __builtin_amdgcn_sched_barrier(0);
+      soft(s1, 1, test[1]);
+      pv(s1, va);
+    } else {
+      // one block: its V operands are read while the S product runs
+      f32x16 s0 = zero16;
+      v_fetch(0, va);
+#pragma unroll
+      for (int ks = 0; ks < QR; ks++) s0 = mfma16<T>(ka[ks], qh[ks], s0);
+      __builtin_amdgcn_sched_barrier(0);
+      soft(s0, 0, test[0]);
+      pv(s0, va);
     }
-    // one LDS read behind every matrix instruction
-#pragma unroll
-    for (int ks = 0; ks < QR; ks++) {
-      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-    }
-    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int ks = 0; ks < QR; ks++) s1 = mfma16<T>(kb[ks], qh[ks], s1);
-    v_fetch(0, va);
-    __builtin_amdgcn_sched_barrier(0);
-    soft(s0, 0, test[0]);
-    pv(s0, va);
-    __builtin_amdgcn_sched_barrier(0);
-    v_fetch(1, va);
-    __builtin_amdgcn_sched_barrier(0);
-    soft(s1, 1, test[1]);
-    pv(s1, va);
   };
 
   // (unrolled over the buffers, so that every LDS address is a register plus a constant)
@@ -1105,7 +1127,8 @@ __global__ __launch_bounds__(256, 2) void band_dma_kernel(TileArgs a) {
     // hand the row over relative to its true maximum: (m, l, o) -> (mt, l * 2^(m - mt), o)
     // (o is divided by l later, so only l changes)
     const float shrink = __builtin_amdgcn_exp2f(m - mt);
-    tile_write_row<T, D>(a.t, q_tok, h, mt, l * shrink, o, shrink, true, l_pre, m_pre);
+    tile_write_row<T, D>(a.t, q_tok, h, mt, l * shrink, o, shrink, true,
+                         state_from_raw<T>(l_raw, a.t.state_f32 != 0), state_from_raw<T>(m_raw, a.t.state_f32 != 0));
   }
 }
 
@@ -1520,7 +1543,7 @@ int launch_band_tiles(const TileArgs& a, int use_nan, hipStream_t stream) {
       if (a.s * (int64_t)(2 * D) * 64 < ((int64_t)1 << 31) && a.n < ((int64_t)1 << 31) &&
           a.n_tiles * a.t.n_batch < ((int64_t)1 << 31) &&
           (a.w <= (int64_t)0x3fffffff || max_len <= (int64_t)0x3fffffff))
-        launch_maybe_timed(ev, band_dma_kernel<T, D>, dim3((unsigned)grid), dim3(256), stream, a);
+        launch_maybe_timed(ev, band_dma_kernel<T, D, SPFA_BAND_BN(D)>, dim3((unsigned)grid), dim3(256), stream, a);
       else
         launch_maybe_timed(ev, tile_kernel<T, D, kTileBand>, dim3((unsigned)grid), dim3(256), stream, a);
     } else {
