@@ -74,7 +74,7 @@ def load_library():
     return lib
 
 
-def make_workload(name, dtype, torch, syn, inline_limit=32, planned=False, heads=1, loop_heads=False):
+def make_workload(name, dtype, torch, syn, inline_limit=32, planned=False, heads=1, loop_heads=False, d_local=64):
     """Returns dict(call=fn(state) -> None, n, d, nnz, bytes_total, bytes_gathered, sample=fn())."""
     dev = "cuda"
     es = torch.tensor([], dtype=dtype).element_size()
@@ -158,10 +158,12 @@ def make_workload(name, dtype, torch, syn, inline_limit=32, planned=False, heads
     else:
         if name == "local":
             import spfa_local
-            n, d, wsz = 65536, 64, 128
+            n, d, wsz = 65536, d_local, 128
+            if d != 64:
+                w["desc"] = "Local N=65536 d=%d LOCAL_SIZE=128 (|i-j|<=128)" % d
             if heads > 1:  # many heads of a short sequence instead of one long one
                 n = 4096
-                w["desc"] = "Local N=4096 d=64 LOCAL_SIZE=128 (|i-j|<=128)"
+                w["desc"] = "Local N=4096 d=%d LOCAL_SIZE=128 (|i-j|<=128)" % d
             q, k, v = syn.qkv(n, d, dtype=dtype, device=dev, seed=0)
             if heads > 1:
                 q, k, v = [torch.stack([syn.qkv(n, d, dtype=dtype, device=dev, seed=h)[j] for h in range(heads)])
@@ -575,6 +577,9 @@ def main():
     ap.add_argument("--workload", default="csr_zipf", choices=sorted(WORKLOADS))
     ap.add_argument("--dtype", default="f32", choices=["f32", "f16", "bf16"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--d", type=int, default=64, choices=[32, 64, 128, 256],
+                    help="head dimension of the `local` workload (BASELINE config 2 has 64; the reference's own "
+                         "check runs at 32)")
     ap.add_argument("--heads", type=int, default=1,
                     help="csr_* and local workloads: this many independent problems sharing the mask, stacked "
                          "[heads, n, d] (local: of N=4096 tokens each)")
@@ -610,7 +615,7 @@ def main():
     if a.heads > 1 and not (a.workload.startswith("csr") or a.workload == "local"):
         sys.exit("bench.py: --heads applies to the csr_* and local workloads")
     w = make_workload(a.workload, dtype, torch, syn, int(lib.spfa_explicit_inline_row_limit()), a.planned,
-                      max(1, a.heads), a.loop_heads)
+                      max(1, a.heads), a.loop_heads, a.d)
     n, d, nnz = w["n"], w["d"], w["nnz"]
 
     n_states = a.steps + a.warmup

@@ -83,8 +83,9 @@ template <typename T, int D>
 struct TileCfg {
   static constexpr bool kF32 = sizeof(T) == 4;
   static constexpr int BM = 128;  // queries per workgroup
-  // keys per LDS tile (fp32 at d = 128 takes half tiles to stay inside 64 KB of LDS)
-  static constexpr int BN = (kF32 && D > 64) ? 32 : 64;
+  // keys per LDS tile (fp32 at d = 128 and the half types at d = 256 take half tiles to stay
+  // inside 64 KB of LDS)
+  static constexpr int BN = (kF32 ? D > 64 : D > 128) ? 32 : 64;
   static constexpr int NB = BN / 32;  // 32-key blocks per tile
   // K tile: [key][k] rows padded so that the 32 keys read by one operand fetch spread over the
   // banks.  V tile: half types are stored transposed [e][key'] (16-byte operand reads), fp32
@@ -231,7 +232,7 @@ __device__ __forceinline__ void tile_write_row(const Tensors& t, int64_t row, in
 }
 
 template <typename T, int D, int MODE>
-__global__ __launch_bounds__(256, 2) void tile_kernel(TileArgs a) {
+__global__ __launch_bounds__(256, D > 128 ? 1 : 2) void tile_kernel(TileArgs a) {
   using C = TileCfg<T, D>;
   constexpr bool kF32 = C::kF32;
   constexpr int BM = C::BM, BN = C::BN, EB = C::EB, NB = C::NB;
@@ -401,7 +402,12 @@ __global__ __launch_bounds__(256, 2) void tile_kernel(TileArgs a) {
   };
   constexpr int CH = kF32 ? D / 4 : D / 8;       // 16-byte chunks per row
   constexpr int KIT = BN * CH / 256;             // chunks of K per thread and tile
-  constexpr int VIT = kF32 ? KIT : (BN / 2) * CH / 256;
+  // half types, V: a lane stages the key pair jp = lane % (BN / 2) and 8 columns; the 64 / (BN / 2)
+  // lanes of a pair times four wavefronts take VCOLS chunks of 8 columns per trip (d = 32: half
+  // of the lanes have no columns to stage)
+  constexpr int PAIRS = BN / 2, LPP = kWave / PAIRS, VCOLS = 4 * LPP;
+  constexpr int VIT = kF32 ? KIT : (CH + VCOLS - 1) / VCOLS;
+  static_assert(KIT >= 1 && C::LDS_BYTES + BN * 4 <= 65536, "tile shape does not fit");
   uint4v kreg[KIT], vreg[kF32 ? KIT : 2 * VIT];
   int ktok_reg = 0;
 
@@ -424,12 +430,12 @@ __global__ __launch_bounds__(256, 2) void tile_kernel(TileArgs a) {
       // V: a lane takes the key pair (2*jp, 2*jp+1) and 8 columns e
 #pragma unroll
       for (int it = 0; it < VIT; it++) {
-        const int jp = lane & 31;
-        const int c = (lane >> 5) + 2 * (wave + 4 * it);
+        const int jp = lane % PAIRS;
+        const int c = lane / PAIRS + LPP * (wave + 4 * it);
         const int64_t u = ut + 2 * jp;
         uint4v v0 = {0u, 0u, 0u, 0u}, v1 = {0u, 0u, 0u, 0u};
-        if (u < u_hi) v0 = *reinterpret_cast<const uint4v*>(Vp + key_tok(u) * D + 8 * c);
-        if (u + 1 < u_hi) v1 = *reinterpret_cast<const uint4v*>(Vp + key_tok(u + 1) * D + 8 * c);
+        if (u < u_hi && c < CH) v0 = *reinterpret_cast<const uint4v*>(Vp + key_tok(u) * D + 8 * c);
+        if (u + 1 < u_hi && c < CH) v1 = *reinterpret_cast<const uint4v*>(Vp + key_tok(u + 1) * D + 8 * c);
         vreg[2 * it] = v0;
         vreg[2 * it + 1] = v1;
       }
@@ -455,16 +461,18 @@ __global__ __launch_bounds__(256, 2) void tile_kernel(TileArgs a) {
       // the 8 packed key pairs go down a column of the transposed tile
 #pragma unroll
       for (int it = 0; it < VIT; it++) {
-        const int jp = lane & 31;
-        const int c = (lane >> 5) + 2 * (wave + 4 * it);
+        const int jp = lane % PAIRS;
+        const int c = lane / PAIRS + LPP * (wave + 4 * it);
         const uint4v v0 = vreg[2 * it], v1 = vreg[2 * it + 1];
         const int slot = key_slot(2 * jp);
         uint32_t* col = reinterpret_cast<uint32_t*>(Vs + (8 * c) * C::V_STRIDE + slot);
+        if (c < CH) {
 #pragma unroll
         for (int x = 0; x < 4; x++) {
           // dword x of v0/v1 holds columns 2x, 2x+1
           col[(2 * x) * (C::V_STRIDE / 2)] = __builtin_amdgcn_perm(v1[x], v0[x], 0x05040100u);
           col[(2 * x + 1) * (C::V_STRIDE / 2)] = __builtin_amdgcn_perm(v1[x], v0[x], 0x07060302u);
+        }
         }
       }
     }
@@ -659,8 +667,10 @@ __global__ __launch_bounds__(256, 2) void tile_kernel(TileArgs a) {
       // fold the wavefronts that share a query block, upper half into lower half, through LDS
       // (the tiles are no longer needed): (q, 1) into (q, 0) for the pairs; 2, 3 into 0, 1 and
       // then 1 into 0 for the four wavefronts of a shared tail tile
+      // (a shape whose exchange area does not fit the tile buffers is never launched with shared
+      // query blocks: d = 256 has one key block per tile and no shared tail tiles)
       constexpr int XR = EB * 16 + 2;
-      static_assert(2 * XR * kWave * 4 <= C::LDS_BYTES, "exchange area does not fit the tile buffers");
+      if constexpr (2 * XR * kWave * 4 <= C::LDS_BYTES) {
       const int nq = quad_split ? 1 : 2;
       for (int step = quad_split ? 2 : 1; step >= 1; step >>= 1) {
         const bool gives = wave_k >= step && wave_k < 2 * step;
@@ -690,6 +700,7 @@ __global__ __launch_bounds__(256, 2) void tile_kernel(TileArgs a) {
             m = m_new;
           }
         }
+      }
       }
       if (wave_k != 0) return;  // (both modes make a single trip)
     }
@@ -772,7 +783,7 @@ struct BandDmaCfg {
   static constexpr int NB = BN / 32;            // 32-key blocks per tile
   static constexpr int ROWB = D * 2;            // bytes per K / V row
   static constexpr int CH = D / 8;              // 16-byte chunks per row
-  static constexpr int RPC = 256 / ROWB;        // rows per 256-byte bank cycle
+  static constexpr int RPC = ROWB < 256 ? 256 / ROWB : 1;  // rows per 256-byte bank cycle
   static constexpr int TILE_B = BN * ROWB;      // bytes of one K (or V) tile
   static constexpr int BUF_B = 2 * TILE_B;      // K tile then V tile
   static constexpr int NI = TILE_B / 4096;      // load instructions per wavefront, tile and matrix
@@ -785,22 +796,29 @@ struct BandDmaCfg {
   static constexpr int NBUF = 65536 / BUF_B < 4 ? 65536 / BUF_B : 4;
   static_assert(BN == 32 || BN == 64, "one or two 32-key blocks per tile");
   static_assert(NI >= 1 && NBUF >= 2, "tile too small or too large");
+  // K rows: chunk c of row j is stored at chunk position c ^ kperm(j).  A K operand fetch reads
+  // one 16-byte chunk of 16 consecutive rows; they cover the 16 chunk positions of a 256-byte
+  // bank cycle once when the rows that start at the same place in the cycle (every 16 / CH-th
+  // row for rows shorter than the cycle) get different positions.
+  static constexpr int KSHIFT = CH >= 16 ? 0 : (CH == 8 ? 1 : 2);
+  static constexpr int KMASK = (CH < 16 ? CH : 16) - 1;
+  __device__ static constexpr int kperm(int j) { return (j >> KSHIFT) & KMASK; }
 };
 
-// keys per tile of band_dma_kernel
+// keys per tile of band_dma_kernel (d = 256: two 32-KB buffers of 32 keys)
 #ifndef SPFA_BAND_BN
-#define SPFA_BAND_BN(D) 64
+#define SPFA_BAND_BN(D) ((D) > 128 ? 32 : 64)
 #endif
 
 // s_waitcnt vmcnt(N) alone (the other counters at their maximum), gfx9 encoding
 #define SPFA_WAIT_VMCNT(N) __builtin_amdgcn_s_waitcnt(((N) & 15) | (((N) >> 4) << 14) | 0x0f70)
 
 template <typename T, int D, int BN_>
-__global__ __launch_bounds__(256, 2) void band_dma_kernel(TileArgs a) {
+__global__ __launch_bounds__(256, D > 128 ? 1 : 2) void band_dma_kernel(TileArgs a) {
   using C = BandDmaCfg<T, D, BN_>;
   constexpr int BM = C::BM, BN = C::BN, NB = C::NB, EB = C::EB, ROWB = C::ROWB, CH = C::CH, RPC = C::RPC;
   constexpr int TILE_B = C::TILE_B, BUF_B = C::BUF_B, NI = C::NI, NBUF = C::NBUF;
-  static_assert(sizeof(T) == 2 && (D == 64 || D == 128), "half types, d = 64 or 128");
+  static_assert(sizeof(T) == 2 && (D == 32 || D == 64 || D == 128 || D == 256), "half types, d = 32 ... 256");
   static_assert(2 * NI * (NBUF - 1) < 64, "outstanding tile loads must fit the vmcnt field");
   __shared__ __attribute__((aligned(1024))) char lds[NBUF * BUF_B];
 
@@ -847,11 +865,15 @@ __global__ __launch_bounds__(256, 2) void band_dma_kernel(TileArgs a) {
   // lane's offset for instruction `it` is that of instruction 0 plus whole rows, which go into
   // the scalar base: two offset registers serve every load.
   constexpr int RPI = 4096 / ROWB;  // rows per load instruction of the workgroup's four wavefronts
-  static_assert(RPI % CH == 0 && (RPI / RPC) % (CH / 4) == 0, "chunk permutation must repeat per instruction");
+  // (d = 256: an instruction covers 8 rows, half a period of the K permutation; the other half
+  // differs by one bit of the chunk position, KXOR below)
+  static_assert((RPI % 16 == 0 || RPI == 8) && (RPI / RPC) % (CH / 4 > 0 ? CH / 4 : 1) == 0,
+                "chunk permutation must repeat per instruction");
   const uint32_t row_step = (uint32_t)a.s * (uint32_t)ROWB;  // bytes between consecutive keys
   const int j0 = (wave * 1024 + lane * 16) / ROWB, p0 = ((wave * 1024 + lane * 16) % ROWB) / 16;
-  const uint32_t koff = (uint32_t)j0 * row_step + (uint32_t)((p0 ^ (j0 % CH)) * 16);
-  const uint32_t voff = (uint32_t)j0 * row_step + (uint32_t)((p0 ^ (4 * ((j0 / RPC) % (CH / 4)))) * 16);
+  constexpr int VPER = CH / 4 > 0 ? CH / 4 : 1;  // period of the V permutation (in bank cycles)
+  const uint32_t koff = (uint32_t)j0 * row_step + (uint32_t)((p0 ^ C::kperm(j0)) * 16);
+  const uint32_t voff = (uint32_t)j0 * row_step + (uint32_t)((p0 ^ (4 * ((j0 / RPC) % VPER))) * 16);
   const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)lds;
   // The loads are written as instructions: scalar base + 32-bit lane offset, LDS address in M0.
   // (Through the builtin the compiler forms a 64-bit address per lane and load, and it orders the
@@ -881,6 +903,7 @@ __global__ __launch_bounds__(256, 2) void band_dma_kernel(TileArgs a) {
         it_byte = tile_byte;
       }
       const uint32_t lds_k = lds_base + (uint32_t)(stage * BUF_B + (4 * it + wave) * 1024);
+      if constexpr (RPI < 16) ko ^= (uint32_t)(C::kperm(it * RPI) * 16);  // (j0 < RPI: the bits do not overlap)
       asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
                    :: "v"(ko), "s"(Kp + it_byte), "s"(lds_k) : "memory", "m0");
       asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
@@ -917,7 +940,7 @@ __global__ __launch_bounds__(256, 2) void band_dma_kernel(TileArgs a) {
   // K block jb, step ks: row 32*jb + r, chunk 2*ks + h
   int kadr[C::QREGS];
 #pragma unroll
-  for (int ks = 0; ks < C::QREGS; ks++) kadr[ks] = r * ROWB + (((2 * ks + h) ^ (r % CH)) * 16);
+  for (int ks = 0; ks < C::QREGS; ks++) kadr[ks] = r * ROWB + (((2 * ks + h) ^ C::kperm(r)) * 16);
   // V: group of 16 lanes = (column half r_hi, key half h); lane 4*x + y of the group points at
   // key 4*h + x (+ 8 for the second half of an operand), columns 32*eb + 16*r_hi + 4*y .. +3,
   // i.e. chunk 4*eb + 2*r_hi + y/2, stored at that chunk ^ g with g = 4 * gx a whole number of
@@ -926,7 +949,7 @@ __global__ __launch_bounds__(256, 2) void band_dma_kernel(TileArgs a) {
   {
     const int x = (lane & 15) >> 2, y = lane & 3, r_hi = (lane >> 4) & 1;
     const int key = 4 * h + x;
-    const int gx = (key / RPC) % (CH / 4);
+    const int gx = (key / RPC) % VPER;
     const int common = TILE_B + key * ROWB + (2 * r_hi + (y >> 1)) * 16 + (y & 1) * 8;
 #pragma unroll
     for (int eb = 0; eb < EB; eb++) vadr[eb] = common + 64 * (eb ^ gx);
@@ -1562,12 +1585,16 @@ int launch_band_tiles(const TileArgs& a, int use_nan, hipStream_t stream) {
       // loads write LDS directly where a tile's rows can be addressed with 32-bit offsets and
       // positions fit 32-bit arithmetic
       const int64_t max_len = a.block > 0 ? a.cnt : (a.n + a.s - 1) / a.s;
-      const bool dma = a.s * (int64_t)(4 * D) * BandDmaF32Cfg<D>::BN < ((int64_t)1 << 31) &&
-                       (a.w <= (int64_t)0x3fffffff || max_len <= (int64_t)0x3fffffff);
+      bool dma = false;
+      if constexpr (D == 64 || D == 128)
+        dma = a.s * (int64_t)(4 * D) * BandDmaF32Cfg<D>::BN < ((int64_t)1 << 31) &&
+              (a.w <= (int64_t)0x3fffffff || max_len <= (int64_t)0x3fffffff);
       const int64_t n_main = n_all - at.n_tail;
       if (dma) {
-        const int64_t grid_d = (n_main + 7) / 8 * 8 + 4 * at.n_tail;
-        launch_maybe_timed(ev, band_dma_f32_kernel<D>, dim3((unsigned)grid_d), dim3(256), stream, at);
+        if constexpr (D == 64 || D == 128) {
+          const int64_t grid_d = (n_main + 7) / 8 * 8 + 4 * at.n_tail;
+          launch_maybe_timed(ev, band_dma_f32_kernel<D>, dim3((unsigned)grid_d), dim3(256), stream, at);
+        }
       } else {
         const int64_t grid_t = (n_main + 7) / 8 * 8 + 4 * at.n_tail;
         launch_maybe_timed(ev, tile_kernel<T, D, kTileBand>, dim3((unsigned)grid_t), dim3(256), stream, at);
@@ -1614,8 +1641,9 @@ int launch_global_tiles(const TileArgs& a, hipStream_t stream) {
 
 inline bool tile_shape_ok(const Tensors& t, size_t elem_bytes) {
   if (!aligned16(t.q) || !aligned16(t.k) || !aligned16(t.v) || !aligned16(t.out)) return false;
-  (void)elem_bytes;
-  return t.d == 64 || t.d == 128;
+  // (fp32 rows of 256 elements: a 32-key tile of K and V alone is 64 KB)
+  if (t.d == 32 || t.d == 64 || t.d == 128) return true;
+  return elem_bytes == 2 && t.d == 256;
 }
 
 // Returns -1 when the shape is not covered (caller falls back to the row-gather engine).
@@ -1624,6 +1652,10 @@ int run_band_tiles(const TileArgs& a, int use_nan, hipStream_t stream) {
   if (!tile_shape_ok(a.t, sizeof(T))) return -1;
   if (a.t.d == 64) return launch_band_tiles<T, 64>(a, use_nan, stream);
   if (a.t.d == 128) return launch_band_tiles<T, 128>(a, use_nan, stream);
+  if (a.t.d == 32) return launch_band_tiles<T, 32>(a, use_nan, stream);
+  if constexpr (sizeof(T) == 2) {
+    if (a.t.d == 256) return launch_band_tiles<T, 256>(a, use_nan, stream);
+  }
   return -1;
 }
 
@@ -1632,6 +1664,10 @@ int run_global_tiles(const TileArgs& a, hipStream_t stream) {
   if (!tile_shape_ok(a.t, sizeof(T))) return -1;
   if (a.t.d == 64) return launch_global_tiles<T, 64>(a, stream);
   if (a.t.d == 128) return launch_global_tiles<T, 128>(a, stream);
+  if (a.t.d == 32) return launch_global_tiles<T, 32>(a, stream);
+  if constexpr (sizeof(T) == 2) {
+    if (a.t.d == 256) return launch_global_tiles<T, 256>(a, stream);
+  }
   return -1;
 }
 
