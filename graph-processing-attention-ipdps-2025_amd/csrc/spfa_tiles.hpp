@@ -95,6 +95,9 @@ struct TileCfg {
   static constexpr int K_ELEMS = BN * K_STRIDE;
   static constexpr int V_ELEMS = kF32 ? BN * V_STRIDE : D * V_STRIDE;
   static constexpr int LDS_BYTES = (K_ELEMS + V_ELEMS) * (int)sizeof(T);
+  // more than the 64 KB a kernel can declare (fp32 at d = 256: 66 KB): the tile buffers are then
+  // dynamic LDS, sized at the launch
+  static constexpr bool kDynLds = LDS_BYTES + BN * 4 > 65536;
   static constexpr int EB = D / 32;                 // 32-row blocks of O^T
   static constexpr int QREGS = kF32 ? D / 2 : D / 16;
 };
@@ -236,7 +239,9 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void tile_kernel(TileArgs a) 
   using C = TileCfg<T, D>;
   constexpr bool kF32 = C::kF32;
   constexpr int BM = C::BM, BN = C::BN, EB = C::EB, NB = C::NB;
-  __shared__ __attribute__((aligned(16))) T lds[C::K_ELEMS + C::V_ELEMS];
+  __shared__ __attribute__((aligned(16))) T lds_fixed[C::kDynLds ? 4 : C::K_ELEMS + C::V_ELEMS];
+  extern __shared__ __attribute__((aligned(16))) char lds_dyn[];
+  T* const lds = C::kDynLds ? reinterpret_cast<T*>(lds_dyn) : lds_fixed;
   __shared__ int ktok_s[BN];  // GlobalCols: token of every key of the tile
   T* Ks = lds;
   T* Vs = lds + C::K_ELEMS;
@@ -407,7 +412,7 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void tile_kernel(TileArgs a) 
   // of the lanes have no columns to stage)
   constexpr int PAIRS = BN / 2, LPP = kWave / PAIRS, VCOLS = 4 * LPP;
   constexpr int VIT = kF32 ? KIT : (CH + VCOLS - 1) / VCOLS;
-  static_assert(KIT >= 1 && C::LDS_BYTES + BN * 4 <= 65536, "tile shape does not fit");
+  static_assert(KIT >= 1 && C::LDS_BYTES + BN * 4 <= 160 * 1024, "tile shape does not fit");
   uint4v kreg[KIT], vreg[kF32 ? KIT : 2 * VIT];
   int ktok_reg = 0;
 
@@ -1554,6 +1559,30 @@ __global__ __launch_bounds__(256) void global_rows_merge_kernel(TileArgs a) {
   }
 }
 
+// tile_kernel's launch: shapes whose tile buffers exceed 64 KB get them as dynamic LDS (the limit
+// of the kernel is raised once per device)
+template <typename T, int D, int MODE>
+void launch_tile_kernel(const KernelEvents& ev, dim3 grid, hipStream_t stream, const TileArgs& a) {
+  using C = TileCfg<T, D>;
+  if constexpr (C::kDynLds) {
+    constexpr int kMaxDevices = 64;
+    static bool raised[kMaxDevices];
+    int dev = 0;
+    (void)hipGetDevice(&dev);
+    if (dev >= 0 && dev < kMaxDevices && !raised[dev]) {
+      (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&tile_kernel<T, D, MODE>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES);
+      raised[dev] = true;
+    }
+    if (ev.start != nullptr && ev.stop != nullptr)
+      hipExtLaunchKernelGGL((tile_kernel<T, D, MODE>), grid, dim3(256), C::LDS_BYTES, stream, ev.start, ev.stop, 0, a);
+    else
+      hipLaunchKernelGGL((tile_kernel<T, D, MODE>), grid, dim3(256), C::LDS_BYTES, stream, a);
+  } else {
+    launch_maybe_timed(ev, tile_kernel<T, D, MODE>, grid, dim3(256), stream, a);
+  }
+}
+
 template <typename T, int D>
 int launch_band_tiles(const TileArgs& a, int use_nan, hipStream_t stream) {
   const KernelEvents ev = kernel_events();
@@ -1568,7 +1597,7 @@ int launch_band_tiles(const TileArgs& a, int use_nan, hipStream_t stream) {
           (a.w <= (int64_t)0x3fffffff || max_len <= (int64_t)0x3fffffff))
         launch_maybe_timed(ev, band_dma_kernel<T, D, SPFA_BAND_BN(D)>, dim3((unsigned)grid), dim3(256), stream, a);
       else
-        launch_maybe_timed(ev, tile_kernel<T, D, kTileBand>, dim3((unsigned)grid), dim3(256), stream, a);
+        launch_tile_kernel<T, D, kTileBand>(ev, dim3((unsigned)grid), stream, a);
     } else {
       // Two workgroups fit a CU, and tiles take about the same time, so the grid runs in rounds
       // of `resident` tiles and the tiles of a last, sparsely filled round keep the chip
@@ -1597,7 +1626,7 @@ int launch_band_tiles(const TileArgs& a, int use_nan, hipStream_t stream) {
         }
       } else {
         const int64_t grid_t = (n_main + 7) / 8 * 8 + 4 * at.n_tail;
-        launch_maybe_timed(ev, tile_kernel<T, D, kTileBand>, dim3((unsigned)grid_t), dim3(256), stream, at);
+        launch_tile_kernel<T, D, kTileBand>(ev, dim3((unsigned)grid_t), stream, at);
       }
     }
   }
@@ -1627,13 +1656,11 @@ int launch_global_tiles(const TileArgs& a, hipStream_t stream) {
     grid_cols = grid_cols / nb;
     if (grid_cols < 1) grid_cols = 1;
   }
-  hipLaunchKernelGGL((tile_kernel<T, D, kTileGlobalCols>), dim3((unsigned)grid_cols, nb), dim3(256), 0,
-                     stream, ac);
+  launch_tile_kernel<T, D, kTileGlobalCols>(KernelEvents{}, dim3((unsigned)grid_cols, nb), stream, ac);
   const int64_t q_tiles = (a.n_globs + 127) / 128;
   TileArgs ar = a;
   ar.pair_split = (a.n_globs <= 64 && TileCfg<T, D>::NB == 2) ? 1 : 0;
-  launch_maybe_timed(ev, tile_kernel<T, D, kTileGlobalRows>, dim3((unsigned)(q_tiles * a.n_split * nb)),
-                     dim3(256), stream, ar);
+  launch_tile_kernel<T, D, kTileGlobalRows>(ev, dim3((unsigned)(q_tiles * a.n_split * nb)), stream, ar);
   hipLaunchKernelGGL((global_rows_merge_kernel<T, D>), dim3((unsigned)(a.n_globs * nb)), dim3(256), 0,
                      stream, a);
   return hipGetLastError() == hipSuccess ? 0 : 4;
@@ -1641,9 +1668,8 @@ int launch_global_tiles(const TileArgs& a, hipStream_t stream) {
 
 inline bool tile_shape_ok(const Tensors& t, size_t elem_bytes) {
   if (!aligned16(t.q) || !aligned16(t.k) || !aligned16(t.v) || !aligned16(t.out)) return false;
-  // (fp32 rows of 256 elements: a 32-key tile of K and V alone is 64 KB)
-  if (t.d == 32 || t.d == 64 || t.d == 128) return true;
-  return elem_bytes == 2 && t.d == 256;
+  (void)elem_bytes;
+  return t.d == 32 || t.d == 64 || t.d == 128 || t.d == 256;
 }
 
 // Returns -1 when the shape is not covered (caller falls back to the row-gather engine).
@@ -1653,9 +1679,7 @@ int run_band_tiles(const TileArgs& a, int use_nan, hipStream_t stream) {
   if (a.t.d == 64) return launch_band_tiles<T, 64>(a, use_nan, stream);
   if (a.t.d == 128) return launch_band_tiles<T, 128>(a, use_nan, stream);
   if (a.t.d == 32) return launch_band_tiles<T, 32>(a, use_nan, stream);
-  if constexpr (sizeof(T) == 2) {
-    if (a.t.d == 256) return launch_band_tiles<T, 256>(a, use_nan, stream);
-  }
+  if (a.t.d == 256) return launch_band_tiles<T, 256>(a, use_nan, stream);
   return -1;
 }
 
@@ -1665,9 +1689,7 @@ int run_global_tiles(const TileArgs& a, hipStream_t stream) {
   if (a.t.d == 64) return launch_global_tiles<T, 64>(a, stream);
   if (a.t.d == 128) return launch_global_tiles<T, 128>(a, stream);
   if (a.t.d == 32) return launch_global_tiles<T, 32>(a, stream);
-  if constexpr (sizeof(T) == 2) {
-    if (a.t.d == 256) return launch_global_tiles<T, 256>(a, stream);
-  }
+  if (a.t.d == 256) return launch_global_tiles<T, 256>(a, stream);
   return -1;
 }
 
