@@ -505,7 +505,7 @@ int spfa_coo_forward(const spfa_problem_t* p, const void* row_ind, int row_ind_b
   if (rc) return rc;
   CooCsr csr{};
   const CooWorkspace cw = coo_workspace(p->n_q, nnz);
-  rc = coo_to_csr(row_ind, row_ind_bytes == 8 ? 1 : 0, (const uint32_t*)col_ind, nnz, p->n_q,
+  rc = coo_to_csr(row_ind, row_ind_bytes == 8 ? 1 : 0, (const uint32_t*)col_ind, nnz, p->n_q, p->n_k,
                   workspace, (char*)workspace + cw.keep_total, (hipStream_t)stream, &csr);
   if (rc) return rc;
   CsrMask mask{csr.row_off, (const uint32_t*)col_ind, 0, csr.cols, csr.unsorted, nnz, p->n_k};
@@ -548,7 +548,7 @@ int spfa_coo_plan(int64_t n_q, const void* row_ind, int row_ind_bytes, const voi
   rc = check_workspace(workspace, workspace_bytes, w.total - w.keep_total);
   if (rc) return rc;
   CooCsr csr{};
-  rc = coo_to_csr(row_ind, row_ind_bytes == 8 ? 1 : 0, (const uint32_t*)col_ind, nnz, n_q, plan,
+  rc = coo_to_csr(row_ind, row_ind_bytes == 8 ? 1 : 0, (const uint32_t*)col_ind, nnz, n_q, 0, plan,
                   workspace, (hipStream_t)stream, &csr);
   if (rc) return rc;
   CsrMask mask{csr.row_off, (const uint32_t*)col_ind, 0, csr.cols, csr.unsorted, nnz, kAnyColumn};
@@ -887,7 +887,7 @@ int transpose_mask(const CsrMask& rows, int64_t n_q, int64_t n_k, int64_t nnz, c
   if (rc) return rc;
   const CooWorkspace cw = coo_workspace(n_k, nnz);
   *entry_rows = e_rows;
-  return coo_to_csr(e_cols, 0, e_rows, nnz, n_k, mbase + tl.off_coo, mbase + tl.off_coo + cw.keep_total,
+  return coo_to_csr(e_cols, 0, e_rows, nnz, n_k, n_q, mbase + tl.off_coo, mbase + tl.off_coo + cw.keep_total,
                     stream, tr);
 }
 
@@ -1024,7 +1024,7 @@ int spfa_coo_to_csr(int64_t n_rows, const void* row_ind, int row_ind_bytes, cons
   int rc = check_workspace(workspace, workspace_bytes, cw.total);
   if (rc) return rc;
   CooCsr csr{};
-  rc = coo_to_csr(row_ind, row_ind_bytes == 8 ? 1 : 0, (const uint32_t*)col_ind, nnz, n_rows, workspace,
+  rc = coo_to_csr(row_ind, row_ind_bytes == 8 ? 1 : 0, (const uint32_t*)col_ind, nnz, n_rows, 0, workspace,
                   (char*)workspace + cw.keep_total, (hipStream_t)stream, &csr);
   if (rc) return rc;
   return coo_csr_export(csr, (const uint32_t*)col_ind, n_rows, nnz, row_off, csr_col_ind, (hipStream_t)stream);
@@ -1060,7 +1060,7 @@ int spfa_coo_backward(const spfa_problem_t* p, const spfa_grads_t* g, const void
   // the mask by query row first (as the forward call does), then as an explicit CSR mask
   char* fwd = (char*)workspace + lay.off_mask;
   CooCsr csr{};
-  rc = coo_to_csr(row_ind, row_ind_bytes == 8 ? 1 : 0, (const uint32_t*)col_ind, nnz, p->n_q, fwd,
+  rc = coo_to_csr(row_ind, row_ind_bytes == 8 ? 1 : 0, (const uint32_t*)col_ind, nnz, p->n_q, p->n_k, fwd,
                   fwd + cw.keep_total, (hipStream_t)stream, &csr);
   if (rc) return rc;
   CsrMask rows{csr.row_off, (const uint32_t*)col_ind, 0, csr.cols, csr.unsorted, nnz, p->n_k};

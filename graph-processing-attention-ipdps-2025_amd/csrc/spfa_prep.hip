@@ -204,11 +204,24 @@ __global__ __launch_bounds__(kPartThreads) void coo_part_count_kernel(
   const int64_t beg = (int64_t)blockIdx.x * kPartTile;
   const int64_t end = beg + kPartTile < nnz ? beg + kPartTile : nnz;
   bool bad = false;
-  for (int64_t e = beg + threadIdx.x; e < end; e += kPartThreads) {
-    const int64_t r = load_index(row_ind, e, wide);
-    if (r >= 0 && r < n_rows) atomicAdd(&cnt[r >> lo_bits], 1u);
-    else bad = true;
-    if (e > 0 && load_index(row_ind, e - 1, wide) > r) bad = true;
+  // (the tile's loads are issued together: one trip instead of sixteen dependent ones)
+  int64_t rows[kPartTile / kPartThreads], prev[kPartTile / kPartThreads];
+#pragma unroll
+  for (int i = 0; i < kPartTile / kPartThreads; i++) {
+    const int64_t e = beg + (int64_t)i * kPartThreads + threadIdx.x;
+    const int64_t ec = e < end ? e : end - 1;  // (end > beg: the grid has no empty tile)
+    rows[i] = load_index(row_ind, ec, wide);
+    prev[i] = load_index(row_ind, ec > 0 ? ec - 1 : 0, wide);
+  }
+#pragma unroll
+  for (int i = 0; i < kPartTile / kPartThreads; i++) {
+    const int64_t e = beg + (int64_t)i * kPartThreads + threadIdx.x;
+    if (e < end) {
+      const int64_t r = rows[i];
+      if (r >= 0 && r < n_rows) atomicAdd(&cnt[r >> lo_bits], 1u);
+      else bad = true;
+      if (e > 0 && prev[i] > r) bad = true;
+    }
   }
   if (bad) *flag = 1u;
   __syncthreads();
@@ -223,7 +236,8 @@ constexpr size_t kPartScatterLds = (size_t)kPartTile * 8 + 3 * (size_t)kPartMaxB
 
 __global__ __launch_bounds__(kPartThreads) void coo_part_scatter_kernel(
     const void* row_ind, int wide, const uint32_t* col_ind, int64_t nnz, int64_t n_rows, int lo_bits,
-    int n_hi, int64_t n_tiles, const uint32_t* flag, const uint32_t* hist, uint64_t* tmp_pairs) {
+    int n_hi, int64_t n_tiles, const uint32_t* flag, const uint32_t* hist, uint64_t* tmp_pairs,
+    int col_bits, uint32_t col_max) {
   extern __shared__ __attribute__((aligned(16))) unsigned char part_lds[];
   uint64_t* stage = reinterpret_cast<uint64_t*>(part_lds);
   uint32_t* cnt = reinterpret_cast<uint32_t*>(part_lds + (size_t)kPartTile * 8);
@@ -280,6 +294,19 @@ __global__ __launch_bounds__(kPartThreads) void coo_part_scatter_kernel(
       stage[lstart[rows[i] >> lo_bits] + rank[i]] = ((uint64_t)rows[i] << 32) | cols[i];
   }
   __syncthreads();
+  if (col_bits > 0) {
+    // (row inside the bucket, column) fit 32 bits: half the bytes to write here and to read in
+    // pass 2; a column past the last key (masked later whatever its value) becomes col_max
+    uint32_t* tmp_packed = reinterpret_cast<uint32_t*>(tmp_pairs);
+    const uint32_t lo_mask = (1u << lo_bits) - 1u;
+    for (uint32_t i = tid; i < kept; i += kPartThreads) {
+      const uint64_t x = stage[i];
+      const uint32_t row = (uint32_t)(x >> 32), col = (uint32_t)x;
+      const uint32_t b = row >> lo_bits;
+      tmp_packed[gstart[b] + (i - lstart[b])] = ((row & lo_mask) << col_bits) | (col < col_max ? col : col_max);
+    }
+    return;
+  }
   for (uint32_t i = tid; i < kept; i += kPartThreads) {
     const uint64_t x = stage[i];
     const uint32_t b = (uint32_t)(x >> 32) >> lo_bits;
@@ -291,10 +318,64 @@ __global__ __launch_bounds__(kPartThreads) void coo_part_scatter_kernel(
 // Count the low digit in LDS, scan, emit the row offsets of the bucket's rows and place the
 // columns.
 constexpr int kPartRowsThreads = 1024;
+constexpr int kPartKeep = 32;  // pairs per thread that pass 2 keeps in registers
 
-__global__ __launch_bounds__(kPartRowsThreads) void coo_part_rows_kernel(
+// LDS counters under skew: a row that holds a large share of its bucket's entries (power-law
+// masks) has most lanes of every wavefront adding to the same counter, which the LDS serialises
+// lane by lane.  The lanes that share the key of the first lane not dealt with yet are counted
+// with a ballot and added once; after kAggRounds such rounds the remaining lanes add one by one.
+constexpr int kAggRounds = 2;
+
+__device__ __forceinline__ int wave_lane() {
+  return (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+}
+
+// cnt[key] += 1 for every lane with valid set
+__device__ __forceinline__ void lds_count(uint32_t* cnt, uint32_t key, bool valid) {
+  const int lane = wave_lane();
+  uint64_t todo = __builtin_amdgcn_ballot_w64(valid);
+#pragma unroll
+  for (int round = 0; round < kAggRounds; round++) {
+    if (todo == 0) break;
+    const int leader = __builtin_ctzll(todo);
+    const uint32_t k0 = (uint32_t)__builtin_amdgcn_readlane((int)key, leader);
+    const uint64_t same = __builtin_amdgcn_ballot_w64(valid && key == k0) & todo;
+    if (lane == leader) atomicAdd(&cnt[k0], (uint32_t)__builtin_popcountll(same));
+    todo &= ~same;
+  }
+  if ((todo >> lane) & 1ull) atomicAdd(&cnt[key], 1u);
+}
+
+// the same, returning the counter's value before this lane's own increment (a distinct slot per
+// lane): pos = atomicAdd(&cnt[key], 1)
+__device__ __forceinline__ uint32_t lds_take_slot(uint32_t* cnt, uint32_t key, bool valid) {
+  const int lane = wave_lane();
+  uint64_t todo = __builtin_amdgcn_ballot_w64(valid);
+  uint32_t pos = 0;
+#pragma unroll
+  for (int round = 0; round < kAggRounds; round++) {
+    if (todo == 0) break;
+    const int leader = __builtin_ctzll(todo);
+    const uint32_t k0 = (uint32_t)__builtin_amdgcn_readlane((int)key, leader);
+    const uint64_t same = __builtin_amdgcn_ballot_w64(valid && key == k0) & todo;
+    uint32_t base = 0;
+    if (lane == leader) base = atomicAdd(&cnt[k0], (uint32_t)__builtin_popcountll(same));
+    base = (uint32_t)__builtin_amdgcn_readlane((int)base, leader);
+    if ((same >> lane) & 1ull) pos = base + (uint32_t)__builtin_popcountll(same & ((1ull << lane) - 1ull));
+    todo &= ~same;
+  }
+  if ((todo >> lane) & 1ull) pos = atomicAdd(&cnt[key], 1u);
+  return pos;
+}
+
+// PACKED: the entries are 32-bit (row inside the bucket << col_bits | column).  A bucket of up to
+// kPartKeep * kPartRowsThreads entries is then read once, all loads in flight together, and stays
+// in registers between the count and the placement (32 registers; two workgroups share a CU).
+// Larger buckets, and 64-bit (row, column) pairs, are walked twice, four loads in flight.
+template <bool PACKED>
+__global__ __launch_bounds__(kPartRowsThreads, PACKED ? 8 : 4) void coo_part_rows_kernel(
     int64_t n_rows, int lo_bits, int n_hi, int64_t n_tiles, int64_t n_hist, const uint32_t* flag,
-    const uint32_t* hist, const uint64_t* tmp_pairs, uint32_t* row_off, uint32_t* cols_out) {
+    const uint32_t* hist, const uint64_t* tmp_pairs, uint32_t* row_off, uint32_t* cols_out, int col_bits) {
   __shared__ uint32_t cnt[kPartMaxBuckets];
   __shared__ uint32_t wave_sums[kPartRowsThreads / kWave];
   if (!*flag) return;
@@ -305,59 +386,104 @@ __global__ __launch_bounds__(kPartRowsThreads) void coo_part_rows_kernel(
   for (int i = threadIdx.x; i < n_lo; i += kPartRowsThreads) cnt[i] = 0;
   __syncthreads();
   const uint32_t lo_mask = (uint32_t)n_lo - 1u;
-  // (four loads in flight per thread: the loop is bound by their latency)
+  const uint32_t col_mask = PACKED ? (1u << col_bits) - 1u : 0xffffffffu;
+  const uint32_t* tmp_packed = reinterpret_cast<const uint32_t*>(tmp_pairs);
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  // entry e as (row inside the bucket, column)
+  auto key_of = [&](uint64_t x) -> uint32_t {
+    return PACKED ? (uint32_t)x >> col_bits : (uint32_t)(x >> 32) & lo_mask;
+  };
+  auto load_entry = [&](uint32_t e) -> uint64_t {
+    if constexpr (PACKED) return tmp_packed[e];
+    else return tmp_pairs[e];
+  };
+  // exclusive scan of cnt[0 .. n_lo) in place, kPartRowsThreads values at a time; the scanned
+  // values are the row offsets of the bucket's rows and the cursors of the placement
+  auto scan_counts = [&]() {
+    uint32_t carry = beg;
+    for (int base = 0; base < n_lo; base += kPartRowsThreads) {
+      const int i = base + threadIdx.x;
+      const uint32_t x = i < n_lo ? cnt[i] : 0u;
+      const uint32_t inc = wave_inclusive_scan(x, lane);
+      if (lane == kWave - 1) wave_sums[wave] = inc;
+      __syncthreads();
+      uint32_t prefix = 0, total = 0;
+#pragma unroll
+      for (int w = 0; w < kPartRowsThreads / kWave; w++) {
+        const uint32_t sw = wave_sums[w];
+        if (w < wave) prefix += sw;
+        total += sw;
+      }
+      const uint32_t ex = carry + prefix + inc - x;
+      if (i < n_lo) {
+        cnt[i] = ex;  // becomes the cursor of this row
+        const int64_t row = ((int64_t)b << lo_bits) + i;
+        if (row < n_rows) row_off[row] = ex;
+      }
+      carry += total;
+      __syncthreads();
+    }
+    if (b == n_hi - 1 && threadIdx.x == 0) row_off[n_rows] = end;
+  };
+  if constexpr (PACKED) {
+    if (end - beg <= (uint32_t)(kPartKeep * kPartRowsThreads)) {
+      if (end == beg) {
+        scan_counts();  // (an empty bucket still owes its rows their offsets)
+        return;
+      }
+      // (every load reads a valid entry: past the end, the bucket's last one, which is not counted)
+      uint32_t x[kPartKeep];
+      const uint32_t* bp = tmp_packed + beg;
+      const uint32_t last = end - beg - 1;
+#pragma unroll
+      for (int i = 0; i < kPartKeep; i++) {
+        const uint32_t e = i * kPartRowsThreads + threadIdx.x;
+        x[i] = bp[e < last ? e : last];
+      }
+      // (a few entries at a time: with all of them unrolled into one stretch the slots that come
+      // back from LDS pile up in registers beside the entries)
+#pragma unroll
+      for (int i = 0; i < kPartKeep; i++) {
+        lds_count(cnt, x[i] >> col_bits, beg + i * kPartRowsThreads + threadIdx.x < end);
+        if (i % 4 == 3) __builtin_amdgcn_sched_barrier(0);
+      }
+      __syncthreads();
+      scan_counts();
+#pragma unroll
+      for (int i = 0; i < kPartKeep; i++) {
+        const bool valid = beg + i * kPartRowsThreads + threadIdx.x < end;
+        const uint32_t pos = lds_take_slot(cnt, x[i] >> col_bits, valid);
+        if (valid) cols_out[pos] = x[i] & col_mask;
+        if (i % 4 == 3) __builtin_amdgcn_sched_barrier(0);
+      }
+      return;
+    }
+  }
   constexpr uint32_t kStep = 4 * kPartRowsThreads;
   for (uint32_t e0 = beg; e0 < end; e0 += kStep) {
     uint64_t x[4];
 #pragma unroll
     for (int i = 0; i < 4; i++) {
       const uint32_t e = e0 + i * kPartRowsThreads + threadIdx.x;
-      x[i] = e < end ? tmp_pairs[e] : ~0ull;
+      x[i] = e < end ? load_entry(e) : 0ull;
     }
 #pragma unroll
-    for (int i = 0; i < 4; i++)
-      if (x[i] != ~0ull) atomicAdd(&cnt[(uint32_t)(x[i] >> 32) & lo_mask], 1u);
+    for (int i = 0; i < 4; i++) lds_count(cnt, key_of(x[i]), e0 + i * kPartRowsThreads + threadIdx.x < end);
   }
   __syncthreads();
-  // exclusive scan of cnt[0 .. n_lo) in place, kPartRowsThreads values at a time
-  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
-  uint32_t carry = beg;
-  for (int base = 0; base < n_lo; base += kPartRowsThreads) {
-    const int i = base + threadIdx.x;
-    const uint32_t x = i < n_lo ? cnt[i] : 0u;
-    const uint32_t inc = wave_inclusive_scan(x, lane);
-    if (lane == kWave - 1) wave_sums[wave] = inc;
-    __syncthreads();
-    uint32_t prefix = 0, total = 0;
-#pragma unroll
-    for (int w = 0; w < kPartRowsThreads / kWave; w++) {
-      const uint32_t sw = wave_sums[w];
-      if (w < wave) prefix += sw;
-      total += sw;
-    }
-    const uint32_t ex = carry + prefix + inc - x;
-    if (i < n_lo) {
-      cnt[i] = ex;  // becomes the cursor of this row
-      const int64_t row = ((int64_t)b << lo_bits) + i;
-      if (row < n_rows) row_off[row] = ex;
-    }
-    carry += total;
-    __syncthreads();
-  }
-  if (b == n_hi - 1 && threadIdx.x == 0) row_off[n_rows] = end;
+  scan_counts();
   for (uint32_t e0 = beg; e0 < end; e0 += kStep) {
     uint64_t x[4];
 #pragma unroll
     for (int i = 0; i < 4; i++) {
       const uint32_t e = e0 + i * kPartRowsThreads + threadIdx.x;
-      x[i] = e < end ? tmp_pairs[e] : ~0ull;
+      x[i] = e < end ? load_entry(e) : 0ull;
     }
 #pragma unroll
     for (int i = 0; i < 4; i++) {
-      if (x[i] != ~0ull) {
-        const uint32_t pos = atomicAdd(&cnt[(uint32_t)(x[i] >> 32) & lo_mask], 1u);
-        cols_out[pos] = (uint32_t)x[i];
-      }
+      const bool valid = e0 + i * kPartRowsThreads + threadIdx.x < end;
+      const uint32_t pos = lds_take_slot(cnt, key_of(x[i]), valid);
+      if (valid) cols_out[pos] = (uint32_t)x[i] & col_mask;
     }
   }
 }
@@ -427,7 +553,7 @@ CooWorkspace coo_workspace(int64_t n_rows, int64_t nnz) {
 }
 
 int coo_to_csr(const void* row_ind, int row_wide, const uint32_t* col_ind, int64_t nnz,
-               int64_t n_rows, void* keep, void* scratch, hipStream_t stream, CooCsr* out) {
+               int64_t n_rows, int64_t n_cols, void* keep, void* scratch, hipStream_t stream, CooCsr* out) {
   CooWorkspace w = coo_workspace(n_rows, nnz);
   char* kbase = (char*)keep;
   char* base = (char*)scratch - w.keep_total;  // scratch offsets are counted from the start of keep
@@ -478,12 +604,25 @@ int coo_to_csr(const void* row_ind, int row_wide, const uint32_t* col_ind, int64
     hipLaunchKernelGGL(scan_sums_kernel, dim3(1), dim3(kScanThreads), 0, stream, tiles, hist_tiles, flag);
     hipLaunchKernelGGL(scan_apply_kernel, dim3((unsigned)hist_tiles), dim3(kScanThreads), 0, stream,
                        hist, n_hist, tiles, hist, hist, flag);
+    // 32-bit entries between the passes when the columns leave room for the row inside its bucket
+    // (n_cols known and n_cols < 2^(32 - lo_bits)); columns >= n_cols are stored as n_cols
+    int col_bits = 0;
+    if (n_cols > 0) {
+      int need = 1;
+      while (need < 32 && ((int64_t)1 << need) <= n_cols) need++;  // n_cols itself must fit
+      if (need + w.lo_bits <= 32) col_bits = need;
+    }
     hipLaunchKernelGGL(coo_part_scatter_kernel, dim3((unsigned)w.n_tiles1), dim3(kPartThreads),
                        kPartScatterLds, stream, row_ind, row_wide, col_ind, nnz, n_rows, w.lo_bits,
-                       (int)w.n_hi, w.n_tiles1, flag, hist, tmp_pairs);
-    hipLaunchKernelGGL(coo_part_rows_kernel, dim3((unsigned)w.n_hi), dim3(kPartRowsThreads), 0, stream,
-                       n_rows, w.lo_bits, (int)w.n_hi, w.n_tiles1, n_hist, flag, hist, tmp_pairs, row_off,
-                       cols);
+                       (int)w.n_hi, w.n_tiles1, flag, hist, tmp_pairs, col_bits, (uint32_t)(col_bits ? n_cols : 0));
+    if (col_bits)
+      hipLaunchKernelGGL(coo_part_rows_kernel<true>, dim3((unsigned)w.n_hi), dim3(kPartRowsThreads), 0, stream,
+                         n_rows, w.lo_bits, (int)w.n_hi, w.n_tiles1, n_hist, flag, hist, tmp_pairs, row_off,
+                         cols, col_bits);
+    else
+      hipLaunchKernelGGL(coo_part_rows_kernel<false>, dim3((unsigned)w.n_hi), dim3(kPartRowsThreads), 0, stream,
+                         n_rows, w.lo_bits, (int)w.n_hi, w.n_tiles1, n_hist, flag, hist, tmp_pairs, row_off,
+                         cols, 0);
   } else if (nnz > 0) {
     hipLaunchKernelGGL(coo_histogram_kernel, dim3(grid_for(nnz, 256, 16384)), dim3(256), 0, stream,
                        row_ind, row_wide, nnz, n_rows, flag, counts);

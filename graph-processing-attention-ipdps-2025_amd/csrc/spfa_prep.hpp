@@ -39,8 +39,10 @@ struct CooCsr {
 // both sets of kernels are enqueued and the ones that are not needed return at once.
 // Entries with a row outside [0, n_rows) are dropped (and force the bucketing path).
 // `keep` receives the result (keep_total bytes), `scratch` is total - keep_total bytes.
+// n_cols: columns >= n_cols mean nothing to the caller (they may come back as n_cols); 0 when the
+// columns must come back exactly as given.
 int coo_to_csr(const void* row_ind, int row_wide, const uint32_t* col_ind, int64_t nnz,
-               int64_t n_rows, void* keep, void* scratch, hipStream_t stream, CooCsr* out);
+               int64_t n_rows, int64_t n_cols, void* keep, void* scratch, hipStream_t stream, CooCsr* out);
 
 // The entry list of a CSR mask: rows[e], cols[e] for every entry e of row_off / col_ind (cols
 // from alt_cols when *use_alt != 0, as CsrMask reads them).  Feeding (cols, rows) back into
