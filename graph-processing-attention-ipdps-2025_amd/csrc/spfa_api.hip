@@ -678,6 +678,38 @@ size_t spfa_global_no_local_workspace_bytes(int64_t n, int64_t d, int dtype, int
   return global_layout(n, n_globals, d).total;
 }
 
+namespace {
+
+// The dense-tile problem of the global-minus-local mask over a workspace laid out by
+// global_layout; false when it does not fit the tile kernels' index arithmetic.
+bool global_tile_args(const spfa_problem_t* p, const int32_t* global_inds, int64_t n_globals,
+                      int64_t local_size, const GlobalLayout& lay, char* base, TileArgs* out) {
+  const int64_t n = p->n_q;
+  uint32_t* bits = (uint32_t*)(base + lay.off_bits);
+  TileArgs a{};
+  a.t = make_tensors(p);
+  a.n = n;
+  a.w = local_size;
+  a.s = 1;
+  a.globs = global_inds;
+  a.n_globs = n_globals;
+  a.gbits = bits;
+  a.uq = (int32_t*)(base + lay.off_uq);
+  a.n_uq = bits + (global_bits_words(n) - 1);
+  a.key_run = lay.key_run;
+  a.n_split = lay.n_split;
+  a.pm = (float*)(base + lay.off_pm);
+  a.pl = (float*)(base + lay.off_pl);
+  a.pacc = (float*)(base + lay.off_pacc);
+  *out = a;
+  const int64_t q_tiles = (n_globals + 127) / 128;
+  return q_tiles * lay.n_split * batch_of(p) < ((int64_t)1 << 31) &&
+         n_globals * batch_of(p) < ((int64_t)1 << 31) && batch_of(p) < 65536 &&
+         local_size <= kTileMaxWindow;
+}
+
+}  // namespace
+
 int spfa_global_no_local_forward(const spfa_problem_t* p, const int32_t* global_inds,
                                  int64_t n_globals, int64_t local_size, void* workspace,
                                  size_t workspace_bytes, void* stream) {
@@ -705,24 +737,7 @@ int spfa_global_no_local_forward(const spfa_problem_t* p, const int32_t* global_
 
   // dense tiles when the shape allows it
   TileArgs a{};
-  a.t = make_tensors(p);
-  a.n = n;
-  a.w = local_size;
-  a.s = 1;
-  a.globs = global_inds;
-  a.n_globs = n_globals;
-  a.gbits = bits;
-  a.uq = uq;
-  a.n_uq = bits + (global_bits_words(n) - 1);
-  a.key_run = lay.key_run;
-  a.n_split = lay.n_split;
-  a.pm = (float*)(base + lay.off_pm);
-  a.pl = (float*)(base + lay.off_pl);
-  a.pacc = (float*)(base + lay.off_pacc);
-  const int64_t q_tiles = (n_globals + 127) / 128;
-  if (q_tiles * lay.n_split * batch_of(p) < ((int64_t)1 << 31) &&
-      n_globals * batch_of(p) < ((int64_t)1 << 31) && batch_of(p) < 65536 &&
-      local_size <= kTileMaxWindow) {
+  if (global_tile_args(p, global_inds, n_globals, local_size, lay, base, &a)) {
     rc = -1;
     switch (p->dtype) {
       case SPFA_DTYPE_F32: rc = run_global_dense<float>(a, (hipStream_t)stream); break;
@@ -736,6 +751,20 @@ int spfa_global_no_local_forward(const spfa_problem_t* p, const int32_t* global_
   GlobalMask mask{n, local_size, global_inds, n_globals, bits};
   return dispatch_global(p, mask, s, base + lay.off_engine, (hipStream_t)stream);
 }
+
+namespace {
+
+// The listed tokens' rows of a window + global call whose other rows have had the listed tokens as
+// keys inside the band kernel already.
+int global_rows_only(const spfa_problem_t* p, const TileArgs& a, hipStream_t stream) {
+  switch (p->dtype) {
+    case SPFA_DTYPE_F16: return run_global_dense<f16>(a, stream, true);
+    case SPFA_DTYPE_BF16: return run_global_dense<bf16>(a, stream, true);
+  }
+  return -1;
+}
+
+}  // namespace
 
 /* ------------------------------------------------------------------------------ window + global + CSR */
 size_t spfa_window_global_csr_workspace_bytes(int64_t n, int64_t d, int dtype, int64_t local_size,
@@ -775,12 +804,42 @@ int spfa_window_global_csr_forward(const spfa_problem_t* p, int64_t local_size,
                                                                       n_globals, nnz));
   if (rc) return rc;
 
-  rc = spfa_local_forward(p, local_size, workspace, workspace_bytes, stream);
-  if (rc) return rc;
-  if (n_globals > 0) {
-    rc = spfa_global_no_local_forward(p, global_inds, n_globals, local_size, workspace, workspace_bytes,
-                                      stream);
+  // Half types on the tile kernels: the band kernel takes the listed tokens as further keys of
+  // the rows that are not listed themselves, so those rows' state makes one round trip instead
+  // of two and Q is read once; the listed tokens' own rows follow.  (fp32 band tiles are bound by
+  // the matrix pipe, not by this traffic: there the parts run one after the other.)
+  bool fused = false;
+  if (n_globals > 0 && (p->dtype == SPFA_DTYPE_F16 || p->dtype == SPFA_DTYPE_BF16) &&
+      2 * local_size + 1 >= kBandTileMinRow && p->n_q >= kBandTileMinRow && local_size <= kTileMaxWindow) {
+    const GlobalLayout lay = global_layout(p->n_q, n_globals, p->d, batch_of(p));
+    char* base = (char*)workspace;
+    TileArgs ag{}, ab{};
+    if (global_tile_args(p, global_inds, n_globals, local_size, lay, base, &ag) &&
+        tile_shape_ok(ag.t, 2) && band_tile_args(p, local_size, 1, 0, 0, &ab)) {
+      rc = prepare_global_rows(global_inds, n_globals, p->n_q, (uint32_t*)ag.gbits, (int32_t*)ag.uq,
+                               (hipStream_t)stream);
+      if (rc) return rc;
+      ab.globs = global_inds;
+      ab.n_globs = n_globals;
+      ab.gbits = ag.gbits;
+      rc = p->dtype == SPFA_DTYPE_F16 ? run_band<f16>(ab, 0, (hipStream_t)stream)
+                                      : run_band<bf16>(ab, 0, (hipStream_t)stream);
+      if (rc > 0) return rc;
+      if (rc == 0) {
+        rc = global_rows_only(p, ag, (hipStream_t)stream);
+        if (rc != 0) return rc < 0 ? SPFA_ERR_LAUNCH : rc;
+        fused = true;
+      }
+    }
+  }
+  if (!fused) {
+    rc = spfa_local_forward(p, local_size, workspace, workspace_bytes, stream);
     if (rc) return rc;
+    if (n_globals > 0) {
+      rc = spfa_global_no_local_forward(p, global_inds, n_globals, local_size, workspace, workspace_bytes,
+                                        stream);
+      if (rc) return rc;
+    }
   }
   if (nnz > 0)
     rc = spfa_csr_forward(p, row_off, row_off_bytes, col_ind, nnz, 0, workspace, workspace_bytes, stream);

@@ -27,8 +27,8 @@ int run_global<SPFA_INST_T>(const Tensors& t, const GlobalMask& mask, const Engi
   return run_engine<SPFA_INST_T, GlobalMask>(t, mask, s, use_nan, ws, stream);
 }
 template <>
-int run_global_dense<SPFA_INST_T>(const TileArgs& a, hipStream_t stream) {
-  return run_global_tiles<SPFA_INST_T>(a, stream);
+int run_global_dense<SPFA_INST_T>(const TileArgs& a, hipStream_t stream, bool rows_only) {
+  return run_global_tiles<SPFA_INST_T>(a, stream, rows_only);
 }
 #else
 #error "SPFA_INST_MASK must be 0 (csr), 1 (stride) or 2 (global)"

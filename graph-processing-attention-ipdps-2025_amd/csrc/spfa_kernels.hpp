@@ -19,8 +19,9 @@ int run_stride(const Tensors& t, const StrideMask& mask, const EngineSizing& s, 
 template <typename T>
 int run_band(const TileArgs& a, int use_nan, hipStream_t stream);
 // Dense-tile path for the global-minus-local mask; -1 when the shape is not covered.
+// (rows_only: see launch_global_tiles)
 template <typename T>
-int run_global_dense(const TileArgs& a, hipStream_t stream);
+int run_global_dense(const TileArgs& a, hipStream_t stream, bool rows_only = false);
 template <typename T>
 int run_global(const Tensors& t, const GlobalMask& mask, const EngineSizing& s, int use_nan,
                void* ws, hipStream_t stream);

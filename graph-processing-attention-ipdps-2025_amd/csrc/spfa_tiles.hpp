@@ -970,6 +970,71 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void band_dma_kernel(TileArgs
   float mt = kNegInf;  // true running maximum
   float l = 0.f;       // running sum (relative to m) over this lane's half of the keys
 
+  typedef short s16x4 __attribute__((ext_vector_type(4)));
+  typedef short s16x8 __attribute__((ext_vector_type(8)));
+  typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+  constexpr int QR = C::QREGS;
+  const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+
+  // One online-softmax step over a 32-key block whose dead entries are -inf already; leaves the
+  // exponentials in s.  The exponentials are taken against a reference maximum m that is only
+  // moved (and the accumulators rescaled) when a row's maximum has grown by more than kSlack
+  // (log2 units) since the reference was set: the weights then stay below 2^kSlack, the final
+  // division by l cancels the reference, and the rescale is rare instead of happening on every
+  // block while the maxima are still settling.  mt keeps the true maximum for the row
+  // statistics.  The row sum is taken over the weights as the second product sees them (rounded
+  // to T), two at a time.
+  auto soft_core = [&](f32x16& s) __attribute__((always_inline)) {
+    float mx = s[0];
+#pragma unroll
+    for (int v = 1; v < 16; v++) mx = fmaxf(mx, s[v]);
+    mx = fmaxf(mx, shfl_xor_f32(mx, 32)) * sc;
+    mt = fmaxf(mt, mx);
+    if (__builtin_expect(__builtin_amdgcn_ballot_w64(mx > m + kSlack) != 0, 0)) {
+      // (m = -inf: first live block of a row, nothing accumulated yet)
+      const float m_new = (mx > m + kSlack) ? mx : m;
+      const float alpha = (m > kNegInf) ? __builtin_amdgcn_exp2f(m - m_new) : 0.f;
+      m = m_new;
+      l *= alpha;
+#pragma unroll
+      for (int eb = 0; eb < EB; eb++)
+#pragma unroll
+        for (int v = 0; v < 16; v++) o[eb][v] *= alpha;
+    }
+    const float neg_m = (m > kNegInf) ? -m : 0.f;
+    float lsum = 0.f;
+#pragma unroll
+    for (int v = 0; v < 16; v++)
+      s[v] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[v], sc, neg_m));  // exp2(-inf) = 0
+#pragma unroll
+    for (int x = 0; x < 8; x++) lsum = dot2_ones<T>(pack2<T>(s[2 * x], s[2 * x + 1]), lsum);
+    l += lsum;
+  };
+  // V^T operands of block jb of the tile at tb: [sl][eb], two transposing 8-byte reads each
+  auto v_fetch = [&](const char* tb, int jb, uint4v (&va)[2 * EB]) __attribute__((always_inline)) {
+#pragma unroll
+    for (int sl = 0; sl < 2; sl++)
+#pragma unroll
+      for (int eb = 0; eb < EB; eb++) {
+        const char* va_p = tb + (32 * jb + 16 * sl) * ROWB + vadr[eb];
+        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)va_p);
+        const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(va_p + 8 * ROWB));
+        const s16x8 both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        va[sl * EB + eb] = __builtin_bit_cast(uint4v, both);
+      }
+  };
+  // O^T += V_block^T P_block^T
+  auto pv = [&](const f32x16& s, const uint4v (&va)[2 * EB]) __attribute__((always_inline)) {
+#pragma unroll
+    for (int sl = 0; sl < 2; sl++) {
+      uint4v pb;
+#pragma unroll
+      for (int x = 0; x < 4; x++) pb[x] = pack2<T>(s[8 * sl + 2 * x], s[8 * sl + 2 * x + 1]);
+#pragma unroll
+      for (int eb = 0; eb < EB; eb++) o[eb] = mfma16<T>(va[sl * EB + eb], pb, o[eb]);
+    }
+  };
+
   // one tile: wait for it, publish it, request the tile NBUF - 1 steps ahead into the buffer the
   // previous step has freed, consume it
   auto step = [&](int ut, int stage) __attribute__((always_inline)) {
@@ -1006,10 +1071,6 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void band_dma_kernel(TileArgs
     // The K operands of the first block are asked for before the next tile is requested:
     // the four wavefronts issue their tile loads in one burst right after the barrier, and the
     // operand reads come back while that burst drains.
-    typedef short s16x4 __attribute__((ext_vector_type(4)));
-    typedef short s16x8 __attribute__((ext_vector_type(8)));
-    typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
-    constexpr int QR = C::QREGS;
     uint4v ka[QR];
     if (!none) {
 #pragma unroll
@@ -1031,16 +1092,8 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void band_dma_kernel(TileArgs
     const int jlo_both = jhi >= jlo ? jlo : 0x40000000;
     const uint32_t span = jhi >= jlo ? (uint32_t)(jhi - jlo) : 0u;
 
-    // One online-softmax step over a 32-key block; leaves the exponentials in s.  The
-    // exponentials are taken against a reference maximum m that is only moved (and the
-    // accumulators rescaled) when a row's maximum has grown by more than kSlack (log2 units)
-    // since the reference was set: the weights then stay below 2^kSlack, the final division by
-    // l cancels the reference, and the rescale is rare instead of happening on every block
-    // while the maxima are still settling.  mt keeps the true maximum for the row statistics.
-    // The row sum is taken over the weights as the second product sees them (rounded to T), two
-    // at a time.  Masking costs a compare and a select per element at one end of the band, one
-    // more instruction when a block meets both ends (windows narrower than a block).
-    auto soft = [&](f32x16& s, int jb, bool test) {
+    // the band test of a block (a compare and a select per element), then the softmax step
+    auto soft = [&](f32x16& s, int jb, bool test) __attribute__((always_inline)) {
       if (test) {
 #pragma unroll
         for (int v = 0; v < 16; v++) {
@@ -1048,58 +1101,9 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void band_dma_kernel(TileArgs
           s[v] = ((uint32_t)(c - jlo_both) <= span) ? s[v] : kNegInf;
         }
       }
-      float mx = s[0];
-#pragma unroll
-      for (int v = 1; v < 16; v++) mx = fmaxf(mx, s[v]);
-      mx = fmaxf(mx, shfl_xor_f32(mx, 32)) * sc;
-      mt = fmaxf(mt, mx);
-      if (__builtin_expect(__builtin_amdgcn_ballot_w64(mx > m + kSlack) != 0, 0)) {
-        // (m = -inf: first live block of a row, nothing accumulated yet)
-        const float m_new = (mx > m + kSlack) ? mx : m;
-        const float alpha = (m > kNegInf) ? __builtin_amdgcn_exp2f(m - m_new) : 0.f;
-        m = m_new;
-        l *= alpha;
-#pragma unroll
-        for (int eb = 0; eb < EB; eb++)
-#pragma unroll
-          for (int v = 0; v < 16; v++) o[eb][v] *= alpha;
-      }
-      const float neg_m = (m > kNegInf) ? -m : 0.f;
-      float lsum = 0.f;
-#pragma unroll
-      for (int v = 0; v < 16; v++)
-        s[v] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[v], sc, neg_m));  // exp2(-inf) = 0
-#pragma unroll
-      for (int x = 0; x < 8; x++) lsum = dot2_ones<T>(pack2<T>(s[2 * x], s[2 * x + 1]), lsum);
-      l += lsum;
+      soft_core(s);
     };
 
-    // V^T operands of block jb: [sl][eb], two transposing 8-byte reads each
-    auto v_fetch = [&](int jb, uint4v (&va)[2 * EB]) {
-#pragma unroll
-      for (int sl = 0; sl < 2; sl++)
-#pragma unroll
-        for (int eb = 0; eb < EB; eb++) {
-          const char* va_p = tb + (32 * jb + 16 * sl) * ROWB + vadr[eb];
-          const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)va_p);
-          const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(va_p + 8 * ROWB));
-          const s16x8 both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-          va[sl * EB + eb] = __builtin_bit_cast(uint4v, both);
-        }
-    };
-    // O^T += V_block^T P_block^T
-    auto pv = [&](const f32x16& s, const uint4v (&va)[2 * EB]) {
-#pragma unroll
-      for (int sl = 0; sl < 2; sl++) {
-        uint4v pb;
-#pragma unroll
-        for (int x = 0; x < 4; x++) pb[x] = pack2<T>(s[8 * sl + 2 * x], s[8 * sl + 2 * x + 1]);
-#pragma unroll
-        for (int eb = 0; eb < EB; eb++) o[eb] = mfma16<T>(va[sl * EB + eb], pb, o[eb]);
-      }
-    };
-
-    const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     uint4v va[2 * EB];
     // Operands are fetched from LDS well ahead of the products that use them, in an order the
     // scheduler is told to keep.
@@ -1122,19 +1126,19 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void band_dma_kernel(TileArgs
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int ks = 0; ks < QR; ks++) s1 = mfma16<T>(kb[ks], qh[ks], s1);
-      v_fetch(0, va);
+      v_fetch(tb, 0, va);
       __builtin_amdgcn_sched_barrier(0);
       soft(s0, 0, test[0]);
       pv(s0, va);
       __builtin_amdgcn_sched_barrier(0);
-      v_fetch(1, va);
+      v_fetch(tb, 1, va);
       __builtin_amdgcn_sched_barrier(0);
       soft(s1, 1, test[1]);
       pv(s1, va);
     } else {
       // one block: its V operands are read while the S product runs
       f32x16 s0 = zero16;
-      v_fetch(0, va);
+      v_fetch(tb, 0, va);
 #pragma unroll
       for (int ks = 0; ks < QR; ks++) s0 = mfma16<T>(ka[ks], qh[ks], s0);
       __builtin_amdgcn_sched_barrier(0);
@@ -1148,6 +1152,63 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void band_dma_kernel(TileArgs
 #pragma unroll
     for (int sg = 0; sg < NBUF; sg++)
       if (ut + sg * BN < u_hi) step(ut + sg * BN, sg);
+  }
+
+  // ---- listed global tokens as further keys (the window + global composite): a query that is
+  // not a listed token itself attends the listed tokens outside its window
+  // (Sparse_FlashAttention_Global_No_Local/sp_flatt_global_no_local_kernel.cu:38-64); the rows
+  // of the listed tokens are not touched here.  The listed tokens' K and V rows are gathered
+  // into the first tile buffer, BN of them at a time; a list entry counts every time it is
+  // listed, an entry outside [0, n) not at all.
+  if (a.globs != nullptr) {
+    __shared__ int gtok_s[BN];  // token of every key of the gathered tile (-1: no key)
+    const int64_t tok_base = (int64_t)bb * a.n;             // first row of this problem
+    const int64_t tq_tok = q_tok - tok_base;                // this lane's query token
+    const bool q_plain = q_ok && !bit_is_set(a.gbits, tq_tok);
+    const uint32_t w32 = (uint32_t)wlim, w2 = 2u * (uint32_t)wlim;
+    const uint32_t d0 = w32 - (uint32_t)(int32_t)tq_tok;    // key token + d0 > 2w: outside the window
+    const int ng = (int)a.n_globs;
+    for (int gt = 0; gt < ng; gt += BN) {
+      __syncthreads();  // everyone is done with the buffer (band tiles, or the previous gathered tile)
+#pragma unroll
+      for (int it = 0; it < NI; it++) {
+        const int j = j0 + it * RPI;  // key slot of the tile this lane loads a chunk of
+        int g = -1;
+        if (gt + j < ng) g = listed_token(a.globs[gt + j], a.n);
+        if (p0 == 0) gtok_s[j] = g;
+        const uint32_t row_byte = (uint32_t)((tok_base + (g < 0 ? 0 : g)) * (int64_t)ROWB);
+        const uint32_t ko = row_byte + (uint32_t)((p0 ^ C::kperm(j)) * 16);
+        const uint32_t vo = row_byte + (uint32_t)((p0 ^ (4 * ((j / RPC) % VPER))) * 16);
+        const uint32_t lds_k = lds_base + (uint32_t)((4 * it + wave) * 1024);
+        asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                     :: "v"(ko), "s"(Kp), "s"(lds_k) : "memory", "m0");
+        asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                     :: "v"(vo), "s"(Vp), "s"(lds_k + (uint32_t)TILE_B) : "memory", "m0");
+      }
+      SPFA_WAIT_VMCNT(0);
+      __syncthreads();
+      if (tw0 >= qlen) continue;
+      const char* tb = lds;
+#pragma unroll
+      for (int jb = 0; jb < NB; jb++) {
+        if (gt + 32 * jb >= ng) break;
+        uint4v ka[QR], va[2 * EB];
+#pragma unroll
+        for (int ks = 0; ks < QR; ks++) ka[ks] = *reinterpret_cast<const uint4v*>(tb + 32 * jb * ROWB + kadr[ks]);
+        v_fetch(tb, jb, va);
+        f32x16 s0 = zero16;
+#pragma unroll
+        for (int ks = 0; ks < QR; ks++) s0 = mfma16<T>(ka[ks], qh[ks], s0);
+#pragma unroll
+        for (int v = 0; v < 16; v++) {
+          const int tok = gtok_s[32 * jb + 8 * (v / 4) + 4 * h + (v % 4)];
+          const bool ok = q_plain && tok >= 0 && ((uint32_t)tok + d0 > w2);
+          s0[v] = ok ? s0[v] : kNegInf;
+        }
+        soft_core(s0);
+        pv(s0, va);
+      }
+    }
   }
 
   l += shfl_xor_f32(l, 32);
@@ -1559,6 +1620,10 @@ __global__ __launch_bounds__(256) void global_rows_merge_kernel(TileArgs a) {
   }
 }
 
+// most listed tokens band_dma_kernel takes as further keys (they are gathered one tile at a time,
+// without prefetch)
+constexpr int64_t kFusedMaxGlobals = 256;
+
 // tile_kernel's launch: shapes whose tile buffers exceed 64 KB get them as dynamic LDS (the limit
 // of the kernel is raised once per device)
 template <typename T, int D, int MODE>
@@ -1592,13 +1657,20 @@ int launch_band_tiles(const TileArgs& a, int use_nan, hipStream_t stream) {
       // the direct-to-LDS kernel addresses a tile's rows with 32-bit offsets, and tile numbers,
       // windows and positions with 32-bit arithmetic
       const int64_t max_len = a.block > 0 ? a.cnt : (a.n + a.s - 1) / a.s;
-      if (a.s * (int64_t)(2 * D) * 64 < ((int64_t)1 << 31) && a.n < ((int64_t)1 << 31) &&
-          a.n_tiles * a.t.n_batch < ((int64_t)1 << 31) &&
-          (a.w <= (int64_t)0x3fffffff || max_len <= (int64_t)0x3fffffff))
+      const bool dma = a.s * (int64_t)(2 * D) * 64 < ((int64_t)1 << 31) && a.n < ((int64_t)1 << 31) &&
+                       a.n_tiles * a.t.n_batch < ((int64_t)1 << 31) &&
+                       (a.w <= (int64_t)0x3fffffff || max_len <= (int64_t)0x3fffffff);
+      // listed global tokens as further keys: only the direct-to-LDS kernel takes them, and it
+      // gathers their rows with 32-bit byte offsets
+      if (a.globs != nullptr &&
+          !(dma && a.n * a.t.n_batch * (int64_t)(2 * D) < ((int64_t)1 << 31) && a.n_globs <= kFusedMaxGlobals))
+        return -1;
+      if (dma)
         launch_maybe_timed(ev, band_dma_kernel<T, D, SPFA_BAND_BN(D)>, dim3((unsigned)grid), dim3(256), stream, a);
       else
         launch_tile_kernel<T, D, kTileBand>(ev, dim3((unsigned)grid), stream, a);
     } else {
+      if (a.globs != nullptr) return -1;  // (fp32: the composite runs its parts one after the other)
       // Two workgroups fit a CU, and tiles take about the same time, so the grid runs in rounds
       // of `resident` tiles and the tiles of a last, sparsely filled round keep the chip
       // waiting for a whole round (0.14 ms for a single tile left over at d = 128, window 256).
@@ -1641,8 +1713,10 @@ int launch_band_tiles(const TileArgs& a, int use_nan, hipStream_t stream) {
 
 // Global minus local: non-global rows against the listed globals, then the global rows against
 // everything (key range split over workgroups), then the fold of the splits.
+// rows_only: the listed tokens' own rows only (the other rows have had the listed tokens as keys
+// already, inside band_dma_kernel)
 template <typename T, int D>
-int launch_global_tiles(const TileArgs& a, hipStream_t stream) {
+int launch_global_tiles(const TileArgs& a, hipStream_t stream, bool rows_only) {
   const KernelEvents ev = kernel_events();
   int64_t grid_cols = (a.n + 127) / 128;
   TileArgs ac = a;
@@ -1656,7 +1730,7 @@ int launch_global_tiles(const TileArgs& a, hipStream_t stream) {
     grid_cols = grid_cols / nb;
     if (grid_cols < 1) grid_cols = 1;
   }
-  launch_tile_kernel<T, D, kTileGlobalCols>(KernelEvents{}, dim3((unsigned)grid_cols, nb), stream, ac);
+  if (!rows_only) launch_tile_kernel<T, D, kTileGlobalCols>(KernelEvents{}, dim3((unsigned)grid_cols, nb), stream, ac);
   const int64_t q_tiles = (a.n_globs + 127) / 128;
   TileArgs ar = a;
   ar.pair_split = (a.n_globs <= 64 && TileCfg<T, D>::NB == 2) ? 1 : 0;
@@ -1684,12 +1758,12 @@ int run_band_tiles(const TileArgs& a, int use_nan, hipStream_t stream) {
 }
 
 template <typename T>
-int run_global_tiles(const TileArgs& a, hipStream_t stream) {
+int run_global_tiles(const TileArgs& a, hipStream_t stream, bool rows_only = false) {
   if (!tile_shape_ok(a.t, sizeof(T))) return -1;
-  if (a.t.d == 64) return launch_global_tiles<T, 64>(a, stream);
-  if (a.t.d == 128) return launch_global_tiles<T, 128>(a, stream);
-  if (a.t.d == 32) return launch_global_tiles<T, 32>(a, stream);
-  if (a.t.d == 256) return launch_global_tiles<T, 256>(a, stream);
+  if (a.t.d == 64) return launch_global_tiles<T, 64>(a, stream, rows_only);
+  if (a.t.d == 128) return launch_global_tiles<T, 128>(a, stream, rows_only);
+  if (a.t.d == 32) return launch_global_tiles<T, 32>(a, stream, rows_only);
+  if (a.t.d == 256) return launch_global_tiles<T, 256>(a, stream, rows_only);
   return -1;
 }
 

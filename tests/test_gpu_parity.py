@@ -572,6 +572,44 @@ def test_bigbird_one_call_equals_dense_union(mods, dtype, d, n, w, n_globs):
     check(o, m, l, *ref, dtype, state_dtype=torch.float32)
 
 
+@pytest.mark.parametrize("dtype,d", [(torch.bfloat16, 64), (torch.float16, 128), (torch.bfloat16, 32),
+                                     (torch.float16, 256)])
+@pytest.mark.parametrize("n,w,kind", [(3000, 16, "one"), (3000, 100, "tile"), (2500, 40, "tile+1"),
+                                      (4100, 64, "many"), (2048, 33, "repeats"), (1000, 999, "tile")])
+def test_bigbird_window_and_listed_tokens_in_one_kernel(mods, dtype, d, n, w, kind):
+    """Half types on the tile kernels: the band kernel takes the listed tokens as further keys.  Against
+    the dense union mask where every token is listed once, and against the two chained calls (which
+    count a token as often as it is listed and drop entries outside [0, n)) otherwise; three problems
+    in one call, on top of a state left by an earlier call."""
+    rng = np.random.default_rng(n + w)
+    count = {"one": 1, "tile": 64, "tile+1": 65, "many": 200, "repeats": 40}[kind]
+    globs = rng.choice(n, count, replace=False)
+    if kind == "repeats":
+        globs = np.concatenate([globs, globs[:7], [-3, n, n + 5]])
+        rng.shuffle(globs)
+    g_t = torch.tensor(globs, dtype=torch.int32, device=DEV)
+    e_u64 = torch.zeros(0, dtype=torch.uint64, device=DEV)
+    e_u32 = torch.zeros(0, dtype=torch.uint32, device=DEV)
+    q, k, v, m, l, o = _stacked(n, d, dtype, (3,), 64)
+    mods["spfa_bigbird"].forward(q, k, v, m, l, o, w, g_t, e_u64, e_u32, torch.zeros(0, device=DEV, dtype=dtype))
+    sync()
+    if kind != "repeats":
+        dense = so.mask_local_dense(n, w) | so.mask_global_no_local_dense(n, np.sort(globs), w)
+        _check_heads(q, k, v, o, m, l, lambda a, b, c: so.dense_masked_attention(a, b, c, dense), dtype)
+    m2, l2, o2 = torch.full_like(m, -float("inf")), torch.zeros_like(l), torch.zeros_like(o)
+    mods["spfa_local"].forward(q, k, v, m2, l2, o2, w)
+    mods["spfa_global_no_local"].forward(q, k, v, m2, l2, o2, g_t, w)
+    sync()
+    assert torch.allclose(o.float(), o2.float(), atol=2e-2)
+    assert torch.allclose(m + torch.log(l), m2 + torch.log(l2), atol=2e-2)
+    # a second call on the same state: every row has the same keys again
+    l1, o1 = l.clone(), o.clone()
+    mods["spfa_bigbird"].forward(q, k, v, m, l, o, w, g_t, e_u64, e_u32, torch.zeros(0, device=DEV, dtype=dtype))
+    sync()
+    assert torch.allclose(l, 2 * l1, rtol=2e-3)
+    assert torch.allclose(o.float(), o1.float(), atol=2e-2)
+
+
 def test_bigbird_parts_may_be_empty_and_batched(mods):
     n, d, w = 1024, 64, 16
     globs = [7, 300, 1000]
