@@ -769,7 +769,8 @@ def main():
                      kernel_rows=w["params"]["n_globals"])
         else:
             kernel_flops, kernel_bytes = flops, w["bytes_total"]
-            kernel_name = "band_dma_f32_kernel" if a.dtype == "f32" else "band_dma_kernel"
+            kernel_name = "band_dma_kernel" if a.dtype != "f32" else \
+                "band_dma_f32_kernel" if d in (64, 128) else "tile_kernel"  # fp32 tiles straight to LDS: d = 64, 128
         hbm_ms = kernel_bytes / (HBM_PEAK_GBS * 1e9) * 1e3
         mfma_ms = kernel_flops / (mfma_peak * 1e12) * 1e3
         if hbm_ms >= mfma_ms:

@@ -162,17 +162,23 @@ __device__ __forceinline__ void attend(const Mask& mask, const typename Mask::Ro
   const int c = lane % LPR;
 
   // column of candidate t + ls, or -1 (past the end / masked)
+  // (an explicit mask's column is range-checked when the chunk is used, one trip after its load)
   auto fetch = [&](int64_t t) -> int {
     const int64_t tt = t + ls;
     bool valid = tt < t_end;
     int64_t col = 0;
-    if (valid) col = mask.col(rc, tt, valid);
+    if constexpr (Mask::kExplicit) {
+      if (valid) col = mask.col_unchecked(rc, tt);
+    } else {
+      if (valid) col = mask.col(rc, tt, valid);
+    }
     return valid ? (int)col : -1;
   };
 
   int next = fetch(t_begin);
   for (int64_t tb = t_begin; tb < t_end; tb += SPAN) {
-    const int cur = next;
+    int cur = next;
+    if constexpr (Mask::kExplicit) cur = mask.in_range(cur) ? cur : -1;
     if (tb + SPAN < t_end) next = fetch(tb + SPAN);
 #pragma unroll(PARTS <= 2 ? PARTS : 1)
     for (int part = 0; part < PARTS; part++) {

@@ -116,17 +116,23 @@ __device__ __forceinline__ void grad_walk(const Mask& mask, const typename Mask:
   const int gi = lane / LPR;
   const int c = lane % LPR;
 
+  // (an explicit mask's column is range-checked when the chunk is used, one trip after its load)
   auto fetch = [&](int64_t t) -> int {
     const int64_t tt = t + lane;
     bool valid = tt < t_end;
     int64_t col = 0;
-    if (valid) col = mask.col(rc, tt, valid);
+    if constexpr (Mask::kExplicit) {
+      if (valid) col = mask.col_unchecked(rc, tt);
+    } else {
+      if (valid) col = mask.col(rc, tt, valid);
+    }
     return valid ? (int)col : -1;
   };
 
   int next = fetch(t_begin);
   for (int64_t tb = t_begin; tb < t_end; tb += kWave) {
-    const int cur = next;
+    int cur = next;
+    if constexpr (Mask::kExplicit) cur = mask.in_range(cur) ? cur : -1;
     if (tb + kWave < t_end) next = fetch(tb + kWave);
 #pragma unroll 1
     for (int part = 0; part < PARTS; part++) {

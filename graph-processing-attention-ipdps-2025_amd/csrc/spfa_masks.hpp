@@ -49,6 +49,13 @@ struct CsrMask {
     valid = c < n_cols;
     return c;
   }
+  // The same in two steps, for loops that ask for a column long before they use it: testing the
+  // column where it is loaded would make the loop wait for the load (and for every load issued
+  // before it) on the spot.
+  __device__ __forceinline__ int64_t col_unchecked(const Row& r, int64_t t) const {
+    return (int64_t)r.cols[r.start + t];
+  }
+  __device__ __forceinline__ bool in_range(int c) const { return c >= 0 && (int64_t)c < n_cols; }
   // the row's offsets as stored, for consistency checks: 0 <= start <= end <= nnz
   __device__ __forceinline__ bool consistent(int64_t i) const {
     int64_t a, b;
