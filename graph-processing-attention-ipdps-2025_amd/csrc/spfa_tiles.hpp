@@ -125,20 +125,6 @@ __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
   return __builtin_bit_cast(uint32_t, x);
 }
 
-// acc + lo + hi of a packed pair of half-type values
-template <typename T>
-__device__ __forceinline__ float dot2_ones(uint32_t pk, float acc) {
-  if constexpr (__is_same(T, bf16)) {
-    typedef __bf16 b2 __attribute__((ext_vector_type(2)));
-    const b2 ones = {(__bf16)1.0f, (__bf16)1.0f};
-    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(b2, pk), ones, acc, false);
-  } else {
-    typedef _Float16 h2 __attribute__((ext_vector_type(2)));
-    const h2 ones = {(_Float16)1.0f, (_Float16)1.0f};
-    return __builtin_amdgcn_fdot2(__builtin_bit_cast(h2, pk), ones, acc, false);
-  }
-}
-
 template <bool B>
 struct BoolConst {
   static constexpr bool value = B;
@@ -982,8 +968,11 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void band_dma_kernel(TileArgs
   // (log2 units) since the reference was set: the weights then stay below 2^kSlack, the final
   // division by l cancels the reference, and the rescale is rare instead of happening on every
   // block while the maxima are still settling.  mt keeps the true maximum for the row
-  // statistics.  The row sum is taken over the weights as the second product sees them (rounded
-  // to T), two at a time.
+  // statistics.  The row sum is a plain chain of additions: the dot-product instructions
+  // (v_dot2c_f32_bf16 with a vector of ones, half the instruction count) keep the matrix
+  // instructions of the SIMD's other wavefront from overlapping with this one's vector work
+  // (measured with a probe: a matrix wavefront beside a vector wavefront takes the sum of their
+  // times as soon as the vector stream holds such instructions, 0.65 of it without).
   auto soft_core = [&](f32x16& s) __attribute__((always_inline)) {
     float mx = s[0];
 #pragma unroll
@@ -1007,7 +996,7 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void band_dma_kernel(TileArgs
     for (int v = 0; v < 16; v++)
       s[v] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[v], sc, neg_m));  // exp2(-inf) = 0
 #pragma unroll
-    for (int x = 0; x < 8; x++) lsum = dot2_ones<T>(pack2<T>(s[2 * x], s[2 * x + 1]), lsum);
+    for (int v = 0; v < 16; v++) lsum += s[v];
     l += lsum;
   };
   // V^T operands of block jb of the tile at tb: [sl][eb], two transposing 8-byte reads each
