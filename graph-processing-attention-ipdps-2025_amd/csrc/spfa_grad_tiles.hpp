@@ -477,6 +477,325 @@ __global__ __launch_bounds__(256, (grad_tile_min_blocks<T, D, KEYS>())) void til
     }
 }
 
+// ---------------------------------------------------------------------------------------
+// Band / block masks, bf16 / fp16: the streamed tiles go from global memory straight into LDS
+// ---------------------------------------------------------------------------------------
+// tile_grad_kernel's band problem with the plumbing of band_dma_kernel: the X and Y tiles of 64
+// streamed rows are written into a ring of LDS stages by the loads themselves
+// (global_load_lds_dwordx4, row-major, unpadded), one barrier per tile, a tile asked for
+// NBUF - 1 steps before it is used.  A tile is read by rows (16-byte reads, first two products)
+// and transposed (ds_read_b64_tr_b16, last two), so one chunk permutation has to serve both:
+// chunk c of row j is stored at chunk position c ^ perm(j) with
+//   d = 128 (16 chunks, a row is a bank cycle):  perm = the two low bit pairs of j swapped - 16
+//            consecutive rows take 16 different positions (row reads), and the four rows a
+//            transposing read touches (j = 4a .. 4a+3) put their 4-chunk groups in four different
+//            quarters of the bank cycle;
+//   d = 64  (8 chunks, two rows to a bank cycle): with t = (j >> 1) mod 8, perm = t rotated left
+//            by two bits of three - rows of the same parity take 8 different positions, and rows
+//            4a, 4a+2 (4a+1, 4a+3) put their groups in different halves.
+// The key pass also needs lse and delta of the streamed rows: 64 + 64 floats per stage, loaded
+// the same way (4 bytes per lane; every wavefront issues them, so that all wavefronts have the
+// same number of loads in flight and one wait count serves all).
+template <typename T, int D, bool KEYS>
+struct BandGradDmaCfg {
+  static constexpr int BM = 128, BN = 64, NB = 2;
+  static constexpr int ROWB = D * 2, CH = D / 8;
+  static constexpr int TILE_B = BN * ROWB, BUF_B = 2 * TILE_B;  // X tile then Y tile
+  static constexpr int NI = TILE_B / 4096, RPI = 4096 / ROWB;
+  // the key pass at d = 128 holds two accumulators and two owner vectors (one workgroup per CU
+  // for its registers): four stages; otherwise what fits 64 KB
+  static constexpr int NBUF = (KEYS && D == 128) ? 4 : (65536 / BUF_B < 4 ? 65536 / BUF_B : 4);
+  static constexpr int STAT_B = KEYS ? 2 * BN * 4 : 0;          // lse then delta of a stage
+  static constexpr int LDS_BYTES = NBUF * (BUF_B + STAT_B);
+  static constexpr int LOADS = 2 * NI + (KEYS ? 2 : 0);         // load instructions per wavefront and tile
+  static constexpr int EB = D / 32, AREGS = D / 16;
+  static_assert(D == 64 || D == 128, "d = 64 or 128");
+  static_assert(RPI % 16 == 0, "the permutation must repeat per load instruction");
+  __device__ static constexpr int perm(int j) {
+    if (D == 128) return ((j & 3) << 2) | ((j >> 2) & 3);
+    const int t = (j >> 1) & 7;
+    return ((t & 1) << 2) | (t >> 1);
+  }
+};
+
+template <typename T, int D, bool KEYS>
+__global__ __launch_bounds__(256, (KEYS && D == 128) ? 1 : 2) void band_grad_dma_kernel(TileArgs a, GradArgs g) {
+  using C = BandGradDmaCfg<T, D, KEYS>;
+  constexpr int BM = C::BM, BN = C::BN, NB = C::NB, EB = C::EB, ROWB = C::ROWB, CH = C::CH;
+  constexpr int TILE_B = C::TILE_B, BUF_B = C::BUF_B, NI = C::NI, RPI = C::RPI, NBUF = C::NBUF, AR = C::AREGS;
+  constexpr int LOADS = C::LOADS;
+  static_assert(sizeof(T) == 2, "half types");
+  static_assert(LOADS * (NBUF - 1) < 64, "outstanding tile loads must fit the vmcnt field");
+  extern __shared__ __attribute__((aligned(1024))) char lds_dyn[];
+  char* const lds = lds_dyn;
+  char* const stat = lds + NBUF * BUF_B;  // [stage][lse 64 floats, delta 64 floats]
+
+  // the tile list of the forward band kernels (32-bit arithmetic; the launcher checks the sizes)
+  auto uni = [](int x) { return __builtin_amdgcn_readfirstlane(x); };
+  const uint32_t n_tiles = (uint32_t)a.n_tiles, tiles_per_sub = (uint32_t)a.tiles_per_sub;
+  const uint32_t n_all = n_tiles * (uint32_t)a.t.n_batch;
+  const uint32_t per_xcd = (n_all + 7u) / 8u;
+  uint32_t lt = (blockIdx.x % 8u) * per_xcd + blockIdx.x / 8u;
+  if (lt >= n_all) return;
+  const uint32_t pb_ = lt / n_tiles;
+  lt -= pb_ * n_tiles;
+  const uint32_t sub = lt / tiles_per_sub;
+  const int tile = uni((int)(lt - sub * tiles_per_sub));
+  int64_t base;
+  int len;
+  if (a.block > 0) {
+    base = (int64_t)sub * a.block + (int64_t)pb_ * a.n;
+    len = (int)a.cnt;
+  } else {
+    base = (int64_t)sub + (int64_t)pb_ * a.n;
+    len = uni((int)(((uint32_t)a.n - sub + (uint32_t)a.s - 1u) / (uint32_t)a.s));
+  }
+  const int wlim = (int)(a.w < (int64_t)0x3fffffff ? a.w : (int64_t)0x3fffffff);
+  const int t0 = tile * BM;
+  if (t0 >= len) return;
+  const int u_lo = t0 > wlim ? t0 - wlim : 0;
+  const int u_hi = (len - BM - wlim > t0) ? t0 + BM + wlim : len;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int r = lane & 31, h = lane >> 5;
+  const T* Ap = (const T*)(KEYS ? g.k : g.q);            // owner vectors
+  const T* Bp = (const T*)(KEYS ? g.v : g.d_out);
+  const char* Xp = (const char*)(KEYS ? g.q : g.k);      // streamed rows
+  const char* Yp = (const char*)(KEYS ? g.d_out : g.v);
+  const float scale = 1.0f / sqrtf((float)D);
+  const float sc = 1.4426950408889634f * scale;
+
+  // ---- tile loads (band_dma_kernel's scheme: two lane offsets, the rest in the scalar base)
+  const uint32_t row_step = (uint32_t)a.s * (uint32_t)ROWB;
+  const int j0 = (wave * 1024 + lane * 16) / ROWB, p0 = ((wave * 1024 + lane * 16) % ROWB) / 16;
+  const uint32_t xoff = (uint32_t)j0 * row_step + (uint32_t)((p0 ^ C::perm(j0)) * 16);
+  const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)lds;
+  auto request = [&](int ut, int stage) __attribute__((always_inline)) {
+    const int64_t tile_byte = (base + (int64_t)ut * a.s) * (int64_t)ROWB;  // scalar
+    const bool whole = ut + BN <= u_hi;
+#pragma unroll
+    for (int it = 0; it < NI; it++) {
+      uint32_t xo = xoff;
+      int64_t it_byte = tile_byte + (int64_t)it * RPI * (int64_t)row_step;  // scalar
+      if (!whole) {
+        // last tile of a subsequence: rows past the last position are replaced by the last one
+        // (finite values; they are masked out)
+        int last = u_hi - 1 - ut;
+        asm volatile("" : "+s"(last));
+        const int j = j0 + it * RPI;
+        xo = xoff + (uint32_t)((j > last ? last : j) - j0) * row_step;
+        it_byte = tile_byte;
+      }
+      const uint32_t lds_x = lds_base + (uint32_t)(stage * BUF_B + (4 * it + wave) * 1024);
+      asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                   :: "v"(xo), "s"(Xp + it_byte), "s"(lds_x) : "memory", "m0");
+      asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                   :: "v"(xo), "s"(Yp + it_byte), "s"(lds_x + (uint32_t)TILE_B) : "memory", "m0");
+    }
+    if constexpr (KEYS) {
+      // lse and delta of the tile's rows: lane l takes row ut + l (past the end: the last row)
+      int last = u_hi - 1 - ut;
+      asm volatile("" : "+s"(last));
+      const uint32_t so = (uint32_t)(lane > last ? last : lane) * (uint32_t)a.s * 4u;
+      const int64_t st_byte = (base + (int64_t)ut * a.s) * 4;
+      const uint32_t lds_s = lds_base + (uint32_t)(NBUF * BUF_B + stage * C::STAT_B);
+      asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1"
+                   :: "v"(so), "s"((const char*)g.lse + st_byte), "s"(lds_s) : "memory", "m0");
+      asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1"
+                   :: "v"(so), "s"((const char*)g.delta + st_byte), "s"(lds_s + (uint32_t)(BN * 4)) : "memory", "m0");
+    }
+  };
+#pragma unroll
+  for (int i = 0; i < NBUF - 1; i++)
+    if (u_lo + i * BN < u_hi) request(u_lo + i * BN, i);
+
+  const int tw0 = t0 + 32 * wave;  // first owner of this wavefront
+  const int tq = tw0 + r;          // this lane's owner position
+  const bool own_ok = tq < len;
+  const int64_t own_row = base + (int64_t)(own_ok ? tq : len - 1) * a.s;
+
+  // ---- the owner's two vectors as B operands, kept in registers
+  uint4v ah[AR], bh[AR];
+  {
+    const T* arow = Ap + own_row * D;
+    const T* brow = Bp + own_row * D;
+#pragma unroll
+    for (int ks = 0; ks < AR; ks++) {
+      ah[ks] = *reinterpret_cast<const uint4v*>(arow + 16 * ks + 8 * h);
+      bh[ks] = *reinterpret_cast<const uint4v*>(brow + 16 * ks + 8 * h);
+    }
+  }
+  float lse_o = 0.f, delta_o = 0.f;
+  if constexpr (!KEYS) {
+    lse_o = g.lse[own_row] * 1.4426950408889634f;
+    delta_o = g.delta[own_row];
+  }
+  SPFA_WAIT_VMCNT(0);  // (the owner's vectors and the first tiles, once; see band_dma_kernel)
+
+  // ---- operand addresses inside a stage (bytes)
+  // by rows: row 32*jb + r, chunk 2*ks + h
+  int radr[AR];
+#pragma unroll
+  for (int ks = 0; ks < AR; ks++) radr[ks] = r * ROWB + (((2 * ks + h) ^ C::perm(r)) * 16);
+  // transposed: lane 4*x + y of a group of 16 points at row 4*h + x (+ 8 for the second half of
+  // an operand), columns 32*eb + 16*r_hi + 4*y .. +3, i.e. chunk 4*eb + 2*r_hi + y/2, half y & 1
+  int tadr_lo[EB], tadr_hi[EB];
+  {
+    const int x = (lane & 15) >> 2, y = lane & 3, r_hi = (lane >> 4) & 1;
+    const int key = 4 * h + x;
+#pragma unroll
+    for (int eb = 0; eb < EB; eb++) {
+      const int c = 4 * eb + 2 * r_hi + (y >> 1);
+      tadr_lo[eb] = key * ROWB + ((c ^ C::perm(key)) * 16) + (y & 1) * 8;
+      tadr_hi[eb] = (key + 8) * ROWB + ((c ^ C::perm(key + 8)) * 16) + (y & 1) * 8;
+    }
+  }
+
+  f32x16 g1[EB], g2[KEYS ? EB : 1];
+#pragma unroll
+  for (int eb = 0; eb < EB; eb++)
+#pragma unroll
+    for (int v = 0; v < 16; v++) {
+      g1[eb][v] = 0.f;
+      if constexpr (KEYS) g2[eb][v] = 0.f;
+    }
+
+  typedef short s16x4 __attribute__((ext_vector_type(4)));
+  typedef short s16x8 __attribute__((ext_vector_type(8)));
+  typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+  const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  const uint32_t w32 = (uint32_t)wlim, w2 = 2u * (uint32_t)wlim;
+  // the end of the subsequence folded into the band test (see tile_grad_kernel)
+  const uint32_t end_hi = (uint32_t)(u_hi - 1 - tq) + w32;
+  const uint32_t band_hi = own_ok && end_hi < w2 ? end_hi : w2;
+
+  auto step = [&](int ut, int stage) __attribute__((always_inline)) {
+    const char* xs = lds + stage * BUF_B;
+    const char* ys = xs + TILE_B;
+    const float* lse_s = reinterpret_cast<const float*>(stat + stage * C::STAT_B);
+    const float* delta_s = lse_s + BN;
+    if constexpr (NBUF > 2) {
+      const int after = (u_hi - ut - 1) / BN;  // tiles behind this one
+      if (after >= 2) SPFA_WAIT_VMCNT(2 * LOADS);
+      else if (after == 1) SPFA_WAIT_VMCNT(LOADS);
+      else SPFA_WAIT_VMCNT(0);
+    } else {
+      SPFA_WAIT_VMCNT(0);
+    }
+    __syncthreads();  // the tile has landed for everyone, and everyone is done with the stage before it
+    if (ut + (NBUF - 1) * BN < u_hi) request(ut + (NBUF - 1) * BN, (stage + NBUF - 1) % NBUF);
+
+    const uint32_t d0 = (uint32_t)(ut - tq) + w32;
+#pragma unroll
+    for (int jb = 0; jb < NB; jb++) {
+      const int ub = ut + 32 * jb;
+      const bool need = (tw0 < len) && (ub < u_hi) && (ub <= tw0 + 31 + wlim) && (ub + 31 + wlim >= tw0);
+      if (!need) continue;
+      f32x16 s = zero16, dp;
+#pragma unroll
+      for (int v = 0; v < 16; v++) {
+        if constexpr (KEYS) dp[v] = -delta_s[32 * jb + 8 * (v / 4) + 4 * h + (v % 4)];
+        else dp[v] = -delta_o;
+      }
+#pragma unroll
+      for (int ks = 0; ks < AR; ks++) {
+        s = mfma16<T>(*reinterpret_cast<const uint4v*>(xs + 32 * jb * ROWB + radr[ks]), ah[ks], s);
+        dp = mfma16<T>(*reinterpret_cast<const uint4v*>(ys + 32 * jb * ROWB + radr[ks]), bh[ks], dp);
+      }
+      const bool full = (ub + 31 < u_hi) && (ub + wlim >= tw0 + 31) && (ub + 31 <= tw0 + wlim);
+      if (!full) {
+#pragma unroll
+        for (int v = 0; v < 16; v++) {
+          const int j = 32 * jb + 8 * (v / 4) + 4 * h + (v % 4);
+          s[v] = (d0 + (uint32_t)j <= band_hi) ? s[v] : kNegInf;  // exp2(-inf) = 0
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+#pragma unroll
+      for (int v = 0; v < 16; v++) {
+        float ls = lse_o;
+        if constexpr (KEYS) ls = lse_s[32 * jb + 8 * (v / 4) + 4 * h + (v % 4)] * 1.4426950408889634f;
+        const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(s[v], sc, -ls));
+        s[v] = p;
+        dp[v] *= p;  // dS without its 1/sqrt(d), which the write-out applies
+      }
+#pragma unroll
+      for (int sl = 0; sl < 2; sl++) {
+        uint4v dsb, pb;
+#pragma unroll
+        for (int x = 0; x < 4; x++) {
+          dsb[x] = pack2<T>(dp[8 * sl + 2 * x], dp[8 * sl + 2 * x + 1]);
+          pb[x] = pack2<T>(s[8 * sl + 2 * x], s[8 * sl + 2 * x + 1]);
+        }
+        const char* xt = xs + (32 * jb + 16 * sl) * ROWB;
+        const char* yt = ys + (32 * jb + 16 * sl) * ROWB;
+#pragma unroll
+        for (int eb = 0; eb < EB; eb++) {
+          const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(xt + tadr_lo[eb]));
+          const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(xt + tadr_hi[eb]));
+          const s16x8 both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+          g1[eb] = mfma16<T>(__builtin_bit_cast(uint4v, both), dsb, g1[eb]);
+          if constexpr (KEYS) {
+            const s16x4 lo2 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(yt + tadr_lo[eb]));
+            const s16x4 hi2 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(yt + tadr_hi[eb]));
+            const s16x8 both2 = {lo2[0], lo2[1], lo2[2], lo2[3], hi2[0], hi2[1], hi2[2], hi2[3]};
+            g2[eb] = mfma16<T>(__builtin_bit_cast(uint4v, both2), pb, g2[eb]);
+          }
+        }
+      }
+    }
+  };
+
+  for (int ut = u_lo; ut < u_hi; ut += NBUF * BN) {
+#pragma unroll
+    for (int sg = 0; sg < NBUF; sg++)
+      if (ut + sg * BN < u_hi) step(ut + sg * BN, sg);
+  }
+
+  // ---- add into the owner's gradient rows (g[eb][v] is element 32*eb + 8*(v/4) + 4*h + v%4)
+  if (!own_ok) return;
+  float* out1 = (KEYS ? g.d_k : g.d_q) + own_row * D;
+  float* out2 = KEYS ? g.d_v + own_row * D : nullptr;
+#pragma unroll
+  for (int oc = 0; oc < EB; oc++)
+#pragma unroll
+    for (int g4 = 0; g4 < 4; g4++) {
+      const int e = 32 * oc + 8 * g4 + 4 * h;
+      float4v x0 = *reinterpret_cast<const float4v*>(out1 + e);
+#pragma unroll
+      for (int u = 0; u < 4; u++) x0[u] += g1[oc][4 * g4 + u] * scale;
+      *reinterpret_cast<float4v*>(out1 + e) = x0;
+      if constexpr (KEYS) {
+        float4v y0 = *reinterpret_cast<const float4v*>(out2 + e);
+#pragma unroll
+        for (int u = 0; u < 4; u++) y0[u] += g2[oc][4 * g4 + u];
+        *reinterpret_cast<float4v*>(out2 + e) = y0;
+      }
+    }
+}
+
+// One pass of band_grad_dma_kernel (its LDS stages are dynamic LDS; the kernel's limit is raised
+// once per device).  False: not launched.
+template <typename T, int D, bool KEYS>
+bool launch_band_grad_dma(const TileArgs& a, const GradArgs& g, dim3 grid, hipStream_t stream) {
+  using C = BandGradDmaCfg<T, D, KEYS>;
+  constexpr int kMaxDevices = 64;
+  static bool raised[kMaxDevices];
+  int dev = 0;
+  (void)hipGetDevice(&dev);
+  if (dev < 0 || dev >= kMaxDevices) return false;
+  if (!raised[dev]) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&band_grad_dma_kernel<T, D, KEYS>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES) != hipSuccess)
+      return false;
+    raised[dev] = true;
+  }
+  hipLaunchKernelGGL((band_grad_dma_kernel<T, D, KEYS>), grid, dim3(256), C::LDS_BYTES, stream, a, g);
+  return true;
+}
+
 // Both passes of a band / block mask described by `a` (as the forward tile kernels take it).
 template <typename T, int D>
 int launch_band_grad(const TileArgs& a, const GradArgs& g, hipStream_t stream) {
@@ -485,6 +804,17 @@ int launch_band_grad(const TileArgs& a, const GradArgs& g, hipStream_t stream) {
   hipLaunchKernelGGL((grad_prologue_kernel<T>), dim3((unsigned)((rows + 15) / 16)), dim3(256), 0, stream,
                      a.t, g);
   const int64_t grid = (a.n_tiles * a.t.n_batch + 7) / 8 * 8;
+  if constexpr (sizeof(T) == 2) {
+    // the direct-to-LDS kernels address a tile's rows with 32-bit offsets, and tile numbers,
+    // windows and positions with 32-bit arithmetic (the forward kernel's conditions)
+    const int64_t max_len = a.block > 0 ? a.cnt : (a.n + a.s - 1) / a.s;
+    const bool dma = a.s * (int64_t)(2 * D) * 64 < ((int64_t)1 << 31) && a.n < ((int64_t)1 << 31) &&
+                     a.n_tiles * a.t.n_batch < ((int64_t)1 << 31) &&
+                     (a.w <= (int64_t)0x3fffffff || max_len <= (int64_t)0x3fffffff);
+    if (dma && launch_band_grad_dma<T, D, false>(a, g, dim3((unsigned)grid), stream) &&
+        launch_band_grad_dma<T, D, true>(a, g, dim3((unsigned)grid), stream))
+      return hipGetLastError() == hipSuccess ? 0 : 4;
+  }
   hipLaunchKernelGGL((tile_grad_kernel<T, D, false, kTileBand>), dim3((unsigned)grid), dim3(256), 0, stream,
                      a, g);
   hipLaunchKernelGGL((tile_grad_kernel<T, D, true, kTileBand>), dim3((unsigned)grid), dim3(256), 0, stream,
