@@ -496,7 +496,13 @@ __global__ __launch_bounds__(256, (grad_tile_min_blocks<T, D, KEYS>())) void til
 // The key pass also needs lse and delta of the streamed rows: 64 + 64 floats per stage, loaded
 // the same way (4 bytes per lane; every wavefront issues them, so that all wavefronts have the
 // same number of loads in flight and one wait count serves all).
-template <typename T, int D, bool KEYS>
+// PART (key pass): 0 both gradients in one launch, 1 dK only, 2 dV only.  At d = 128 the two
+// accumulators and two owner vectors of the combined pass need more than 256 registers: one
+// workgroup per CU, every matrix result in an AccVGPR and copied out for the vector work (a
+// third of the pass's vector instructions).  As two launches (dK: S, dP and one accumulator, the
+// query pass's shape; dV: S and one accumulator) both run two workgroups per CU from plain
+// registers, for a quarter more matrix instructions.
+template <typename T, int D, bool KEYS, int PART = 0>
 struct BandGradDmaCfg {
   static constexpr int BM = 128, BN = 64, NB = 2;
   static constexpr int ROWB = D * 2, CH = D / 8;
@@ -504,7 +510,7 @@ struct BandGradDmaCfg {
   static constexpr int NI = TILE_B / 4096, RPI = 4096 / ROWB;
   // the key pass at d = 128 holds two accumulators and two owner vectors (one workgroup per CU
   // for its registers): four stages; otherwise what fits 64 KB
-  static constexpr int NBUF = (KEYS && D == 128) ? 4 : (65536 / BUF_B < 4 ? 65536 / BUF_B : 4);
+  static constexpr int NBUF = (KEYS && D == 128 && PART == 0) ? 4 : (65536 / BUF_B < 4 ? 65536 / BUF_B : 4);
   static constexpr int STAT_B = KEYS ? 2 * BN * 4 : 0;          // lse then delta of a stage
   static constexpr int LDS_BYTES = NBUF * (BUF_B + STAT_B);
   static constexpr int LOADS = 2 * NI + (KEYS ? 2 : 0);         // load instructions per wavefront and tile
@@ -518,9 +524,12 @@ struct BandGradDmaCfg {
   }
 };
 
-template <typename T, int D, bool KEYS>
-__global__ __launch_bounds__(256, (KEYS && D == 128) ? 1 : 2) void band_grad_dma_kernel(TileArgs a, GradArgs g) {
-  using C = BandGradDmaCfg<T, D, KEYS>;
+template <typename T, int D, bool KEYS, int PART>
+__global__ __launch_bounds__(256, (KEYS && D == 128 && PART == 0) ? 1 : 2) void band_grad_dma_kernel(TileArgs a, GradArgs g) {
+  using C = BandGradDmaCfg<T, D, KEYS, PART>;
+  static_assert(KEYS || PART == 0, "the query pass has one gradient");
+  constexpr bool kG1 = PART != 2;           // dQ / dK: needs S, dP and the first accumulator
+  constexpr bool kG2 = KEYS && PART != 1;   // dV: needs S and the second accumulator
   constexpr int BM = C::BM, BN = C::BN, NB = C::NB, EB = C::EB, ROWB = C::ROWB, CH = C::CH;
   constexpr int TILE_B = C::TILE_B, BUF_B = C::BUF_B, NI = C::NI, RPI = C::RPI, NBUF = C::NBUF, AR = C::AREGS;
   constexpr int LOADS = C::LOADS;
@@ -617,14 +626,14 @@ __global__ __launch_bounds__(256, (KEYS && D == 128) ? 1 : 2) void band_grad_dma
   const int64_t own_row = base + (int64_t)(own_ok ? tq : len - 1) * a.s;
 
   // ---- the owner's two vectors as B operands, kept in registers
-  uint4v ah[AR], bh[AR];
+  uint4v ah[AR], bh[kG1 ? AR : 1];
   {
     const T* arow = Ap + own_row * D;
     const T* brow = Bp + own_row * D;
 #pragma unroll
     for (int ks = 0; ks < AR; ks++) {
       ah[ks] = *reinterpret_cast<const uint4v*>(arow + 16 * ks + 8 * h);
-      bh[ks] = *reinterpret_cast<const uint4v*>(brow + 16 * ks + 8 * h);
+      if constexpr (kG1) bh[ks] = *reinterpret_cast<const uint4v*>(brow + 16 * ks + 8 * h);
     }
   }
   float lse_o = 0.f, delta_o = 0.f;
@@ -653,13 +662,13 @@ __global__ __launch_bounds__(256, (KEYS && D == 128) ? 1 : 2) void band_grad_dma
     }
   }
 
-  f32x16 g1[EB], g2[KEYS ? EB : 1];
+  f32x16 g1[kG1 ? EB : 1], g2[kG2 ? EB : 1];
 #pragma unroll
   for (int eb = 0; eb < EB; eb++)
 #pragma unroll
     for (int v = 0; v < 16; v++) {
-      g1[eb][v] = 0.f;
-      if constexpr (KEYS) g2[eb][v] = 0.f;
+      if constexpr (kG1) g1[eb][v] = 0.f;
+      if constexpr (kG2) g2[eb][v] = 0.f;
     }
 
   typedef short s16x4 __attribute__((ext_vector_type(4)));
@@ -693,16 +702,19 @@ __global__ __launch_bounds__(256, (KEYS && D == 128) ? 1 : 2) void band_grad_dma
       const int ub = ut + 32 * jb;
       const bool need = (tw0 < len) && (ub < u_hi) && (ub <= tw0 + 31 + wlim) && (ub + 31 + wlim >= tw0);
       if (!need) continue;
-      f32x16 s = zero16, dp;
+      f32x16 s = zero16, dp = zero16;
+      if constexpr (kG1) {
 #pragma unroll
-      for (int v = 0; v < 16; v++) {
-        if constexpr (KEYS) dp[v] = -delta_s[32 * jb + 8 * (v / 4) + 4 * h + (v % 4)];
-        else dp[v] = -delta_o;
+        for (int v = 0; v < 16; v++) {
+          if constexpr (KEYS) dp[v] = -delta_s[32 * jb + 8 * (v / 4) + 4 * h + (v % 4)];
+          else dp[v] = -delta_o;
+        }
       }
 #pragma unroll
       for (int ks = 0; ks < AR; ks++) {
         s = mfma16<T>(*reinterpret_cast<const uint4v*>(xs + 32 * jb * ROWB + radr[ks]), ah[ks], s);
-        dp = mfma16<T>(*reinterpret_cast<const uint4v*>(ys + 32 * jb * ROWB + radr[ks]), bh[ks], dp);
+        if constexpr (kG1)
+          dp = mfma16<T>(*reinterpret_cast<const uint4v*>(ys + 32 * jb * ROWB + radr[ks]), bh[ks], dp);
       }
       const bool full = (ub + 31 < u_hi) && (ub + wlim >= tw0 + 31) && (ub + 31 <= tw0 + wlim);
       if (!full) {
@@ -719,25 +731,27 @@ __global__ __launch_bounds__(256, (KEYS && D == 128) ? 1 : 2) void band_grad_dma
         if constexpr (KEYS) ls = lse_s[32 * jb + 8 * (v / 4) + 4 * h + (v % 4)] * 1.4426950408889634f;
         const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(s[v], sc, -ls));
         s[v] = p;
-        dp[v] *= p;  // dS without its 1/sqrt(d), which the write-out applies
+        if constexpr (kG1) dp[v] *= p;  // dS without its 1/sqrt(d), which the write-out applies
       }
 #pragma unroll
       for (int sl = 0; sl < 2; sl++) {
-        uint4v dsb, pb;
+        uint4v dsb = {0u, 0u, 0u, 0u}, pb = {0u, 0u, 0u, 0u};
 #pragma unroll
         for (int x = 0; x < 4; x++) {
-          dsb[x] = pack2<T>(dp[8 * sl + 2 * x], dp[8 * sl + 2 * x + 1]);
-          pb[x] = pack2<T>(s[8 * sl + 2 * x], s[8 * sl + 2 * x + 1]);
+          if constexpr (kG1) dsb[x] = pack2<T>(dp[8 * sl + 2 * x], dp[8 * sl + 2 * x + 1]);
+          if constexpr (kG2) pb[x] = pack2<T>(s[8 * sl + 2 * x], s[8 * sl + 2 * x + 1]);
         }
         const char* xt = xs + (32 * jb + 16 * sl) * ROWB;
         const char* yt = ys + (32 * jb + 16 * sl) * ROWB;
 #pragma unroll
         for (int eb = 0; eb < EB; eb++) {
-          const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(xt + tadr_lo[eb]));
-          const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(xt + tadr_hi[eb]));
-          const s16x8 both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-          g1[eb] = mfma16<T>(__builtin_bit_cast(uint4v, both), dsb, g1[eb]);
-          if constexpr (KEYS) {
+          if constexpr (kG1) {
+            const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(xt + tadr_lo[eb]));
+            const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(xt + tadr_hi[eb]));
+            const s16x8 both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+            g1[eb] = mfma16<T>(__builtin_bit_cast(uint4v, both), dsb, g1[eb]);
+          }
+          if constexpr (kG2) {
             const s16x4 lo2 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(yt + tadr_lo[eb]));
             const s16x4 hi2 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(yt + tadr_hi[eb]));
             const s16x8 both2 = {lo2[0], lo2[1], lo2[2], lo2[3], hi2[0], hi2[1], hi2[2], hi2[3]};
@@ -763,11 +777,13 @@ __global__ __launch_bounds__(256, (KEYS && D == 128) ? 1 : 2) void band_grad_dma
 #pragma unroll
     for (int g4 = 0; g4 < 4; g4++) {
       const int e = 32 * oc + 8 * g4 + 4 * h;
-      float4v x0 = *reinterpret_cast<const float4v*>(out1 + e);
+      if constexpr (kG1) {
+        float4v x0 = *reinterpret_cast<const float4v*>(out1 + e);
 #pragma unroll
-      for (int u = 0; u < 4; u++) x0[u] += g1[oc][4 * g4 + u] * scale;
-      *reinterpret_cast<float4v*>(out1 + e) = x0;
-      if constexpr (KEYS) {
+        for (int u = 0; u < 4; u++) x0[u] += g1[oc][4 * g4 + u] * scale;
+        *reinterpret_cast<float4v*>(out1 + e) = x0;
+      }
+      if constexpr (kG2) {
         float4v y0 = *reinterpret_cast<const float4v*>(out2 + e);
 #pragma unroll
         for (int u = 0; u < 4; u++) y0[u] += g2[oc][4 * g4 + u];
@@ -778,21 +794,21 @@ __global__ __launch_bounds__(256, (KEYS && D == 128) ? 1 : 2) void band_grad_dma
 
 // One pass of band_grad_dma_kernel (its LDS stages are dynamic LDS; the kernel's limit is raised
 // once per device).  False: not launched.
-template <typename T, int D, bool KEYS>
+template <typename T, int D, bool KEYS, int PART = 0>
 bool launch_band_grad_dma(const TileArgs& a, const GradArgs& g, dim3 grid, hipStream_t stream) {
-  using C = BandGradDmaCfg<T, D, KEYS>;
+  using C = BandGradDmaCfg<T, D, KEYS, PART>;
   constexpr int kMaxDevices = 64;
   static bool raised[kMaxDevices];
   int dev = 0;
   (void)hipGetDevice(&dev);
   if (dev < 0 || dev >= kMaxDevices) return false;
   if (!raised[dev]) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&band_grad_dma_kernel<T, D, KEYS>),
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&band_grad_dma_kernel<T, D, KEYS, PART>),
                             hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES) != hipSuccess)
       return false;
     raised[dev] = true;
   }
-  hipLaunchKernelGGL((band_grad_dma_kernel<T, D, KEYS>), grid, dim3(256), C::LDS_BYTES, stream, a, g);
+  hipLaunchKernelGGL((band_grad_dma_kernel<T, D, KEYS, PART>), grid, dim3(256), C::LDS_BYTES, stream, a, g);
   return true;
 }
 
@@ -811,9 +827,18 @@ int launch_band_grad(const TileArgs& a, const GradArgs& g, hipStream_t stream) {
     const bool dma = a.s * (int64_t)(2 * D) * 64 < ((int64_t)1 << 31) && a.n < ((int64_t)1 << 31) &&
                      a.n_tiles * a.t.n_batch < ((int64_t)1 << 31) &&
                      (a.w <= (int64_t)0x3fffffff || max_len <= (int64_t)0x3fffffff);
-    if (dma && launch_band_grad_dma<T, D, false>(a, g, dim3((unsigned)grid), stream) &&
-        launch_band_grad_dma<T, D, true>(a, g, dim3((unsigned)grid), stream))
-      return hipGetLastError() == hipSuccess ? 0 : 4;
+#ifndef SPFA_GRAD_KEY_SPLIT
+#define SPFA_GRAD_KEY_SPLIT 1
+#endif
+    if (dma && launch_band_grad_dma<T, D, false>(a, g, dim3((unsigned)grid), stream)) {
+      bool ok;
+      if constexpr (D == 128 && SPFA_GRAD_KEY_SPLIT)
+        ok = launch_band_grad_dma<T, D, true, 1>(a, g, dim3((unsigned)grid), stream) &&
+             launch_band_grad_dma<T, D, true, 2>(a, g, dim3((unsigned)grid), stream);
+      else
+        ok = launch_band_grad_dma<T, D, true, 0>(a, g, dim3((unsigned)grid), stream);
+      return ok && hipGetLastError() == hipSuccess ? 0 : 4;
+    }
   }
   hipLaunchKernelGGL((tile_grad_kernel<T, D, false, kTileBand>), dim3((unsigned)grid), dim3(256), 0, stream,
                      a, g);
