@@ -760,6 +760,7 @@ int global_rows_only(const spfa_problem_t* p, const TileArgs& a, hipStream_t str
   switch (p->dtype) {
     case SPFA_DTYPE_F16: return run_global_dense<f16>(a, stream, true);
     case SPFA_DTYPE_BF16: return run_global_dense<bf16>(a, stream, true);
+    case SPFA_DTYPE_F32: return run_global_dense<float>(a, stream, true);
   }
   return -1;
 }
@@ -804,26 +805,27 @@ int spfa_window_global_csr_forward(const spfa_problem_t* p, int64_t local_size,
                                                                       n_globals, nnz));
   if (rc) return rc;
 
-  // Half types on the tile kernels: the band kernel takes the listed tokens as further keys of
+  // On the direct-to-LDS tile kernels the band kernel takes the listed tokens as further keys of
   // the rows that are not listed themselves, so those rows' state makes one round trip instead
-  // of two and Q is read once; the listed tokens' own rows follow.  (fp32 band tiles are bound by
-  // the matrix pipe, not by this traffic: there the parts run one after the other.)
+  // of two and Q is read once; the listed tokens' own rows follow.
   bool fused = false;
-  if (n_globals > 0 && (p->dtype == SPFA_DTYPE_F16 || p->dtype == SPFA_DTYPE_BF16) &&
+  if (n_globals > 0 &&
+      (p->dtype == SPFA_DTYPE_F16 || p->dtype == SPFA_DTYPE_BF16 || p->dtype == SPFA_DTYPE_F32) &&
       2 * local_size + 1 >= kBandTileMinRow && p->n_q >= kBandTileMinRow && local_size <= kTileMaxWindow) {
     const GlobalLayout lay = global_layout(p->n_q, n_globals, p->d, batch_of(p));
     char* base = (char*)workspace;
     TileArgs ag{}, ab{};
     if (global_tile_args(p, global_inds, n_globals, local_size, lay, base, &ag) &&
-        tile_shape_ok(ag.t, 2) && band_tile_args(p, local_size, 1, 0, 0, &ab)) {
+        tile_shape_ok(ag.t, p->dtype == SPFA_DTYPE_F32 ? 4 : 2) && band_tile_args(p, local_size, 1, 0, 0, &ab)) {
       rc = prepare_global_rows(global_inds, n_globals, p->n_q, (uint32_t*)ag.gbits, (int32_t*)ag.uq,
                                (hipStream_t)stream);
       if (rc) return rc;
       ab.globs = global_inds;
       ab.n_globs = n_globals;
       ab.gbits = ag.gbits;
-      rc = p->dtype == SPFA_DTYPE_F16 ? run_band<f16>(ab, 0, (hipStream_t)stream)
-                                      : run_band<bf16>(ab, 0, (hipStream_t)stream);
+      rc = p->dtype == SPFA_DTYPE_F16    ? run_band<f16>(ab, 0, (hipStream_t)stream)
+           : p->dtype == SPFA_DTYPE_BF16 ? run_band<bf16>(ab, 0, (hipStream_t)stream)
+                                         : run_band<float>(ab, 0, (hipStream_t)stream);
       if (rc > 0) return rc;
       if (rc == 0) {
         rc = global_rows_only(p, ag, (hipStream_t)stream);

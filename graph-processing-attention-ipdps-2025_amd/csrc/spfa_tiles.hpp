@@ -1364,6 +1364,79 @@ __global__ __launch_bounds__(256, 2) void band_dma_f32_kernel(TileArgs a) {
   float mt = kNegInf;  // true running maximum
   float l = 0.f;       // running sum (relative to m) over this lane's half of the keys
 
+  // one online-softmax step over a 32-key block whose dead entries are -inf already (reference
+  // maximum with slack, as in band_dma_kernel); leaves the exponentials in s
+  auto soft_core = [&](f32x16& s) __attribute__((always_inline)) {
+    float mx = s[0];
+#pragma unroll
+    for (int v = 1; v < 16; v++) mx = fmaxf(mx, s[v]);
+    mx = fmaxf(mx, shfl_xor_f32(mx, 32)) * sc;
+    mt = fmaxf(mt, mx);
+    if (__builtin_expect(__builtin_amdgcn_ballot_w64(mx > m + kSlack) != 0, 0)) {
+      const float m_new = (mx > m + kSlack) ? mx : m;
+      const float alpha = (m > kNegInf) ? __builtin_amdgcn_exp2f(m - m_new) : 0.f;
+      m = m_new;
+      l *= alpha;
+#pragma unroll
+      for (int eb = 0; eb < EB; eb++)
+#pragma unroll
+        for (int v = 0; v < 16; v++) o[eb][v] *= alpha;
+    }
+    const float neg_m = (m > kNegInf) ? -m : 0.f;
+    float lsum = 0.f;
+#pragma unroll
+    for (int v = 0; v < 16; v++) {
+      const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(s[v], sc, neg_m));  // exp2(-inf) = 0
+      s[v] = p;
+      lsum += p;
+    }
+    l += lsum;
+  };
+  const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  // S^T = K Q^T of the 32-key block at kb, operand reads two groups of four instructions ahead
+  // (order pinned)
+  auto s_product = [&](const char* kb) __attribute__((always_inline)) -> f32x16 {
+    float4v kx[3];
+    kx[0] = *reinterpret_cast<const float4v*>(kb + kadr[0]);
+    kx[1] = *reinterpret_cast<const float4v*>(kb + kadr[1]);
+    f32x16 sb = zero16;
+    __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+#pragma unroll
+    for (int g = 0; g < D / 8; g++) {
+      if (g + 2 < D / 8) {
+        kx[(g + 2) % 3] = *reinterpret_cast<const float4v*>(kb + kadr[(g + 2) % 8] + 256 * ((g + 2) / 8));
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      }
+#pragma unroll
+      for (int i = 0; i < 4; i++)
+        sb = __builtin_amdgcn_mfma_f32_32x32x2f32(kx[g % 3][i], qf[4 * g + i], sb, 0, 0, 0);
+      __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+    }
+    return sb;
+  };
+  // O^T += V^T P^T of the 32-key block at vb, V reads PD keys ahead (order pinned)
+  auto pv_product = [&](const char* vb, const f32x16& sb) __attribute__((always_inline)) {
+    typedef float vecE __attribute__((ext_vector_type(EB)));
+    constexpr int PD = 8 / EB;
+    vecE vx[PD + 1];
+#pragma unroll
+    for (int v = 0; v < PD; v++)
+      vx[v] = *reinterpret_cast<const vecE*>(vb + vadr[v % 8] + 16 * ROWB * (v / 8));
+    __builtin_amdgcn_sched_group_barrier(0x100, PD, 0);
+#pragma unroll
+    for (int v = 0; v < 16; v++) {
+      if (v + PD < 16) {
+        vx[(v + PD) % (PD + 1)] =
+            *reinterpret_cast<const vecE*>(vb + vadr[(v + PD) % 8] + 16 * ROWB * ((v + PD) / 8));
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      }
+#pragma unroll
+      for (int eb = 0; eb < EB; eb++)
+        o[eb] = __builtin_amdgcn_mfma_f32_32x32x2f32(vx[v % (PD + 1)][eb], sb[v], o[eb], 0, 0, 0);
+      __builtin_amdgcn_sched_group_barrier(0x008, EB, 0);
+    }
+  };
+
   auto step = [&](int ut, const char* tb, char* other) __attribute__((always_inline)) {
     __builtin_amdgcn_s_waitcnt(0);  // this wavefront's part of the tile has landed
     __syncthreads();                // everyone's has, and everyone is done with the other buffer
@@ -1383,8 +1456,7 @@ __global__ __launch_bounds__(256, 2) void band_dma_f32_kernel(TileArgs a) {
     const uint32_t span = (uint32_t)(jhi - jlo);  // jhi < jlo: wraps to a huge value, handled below
     const bool any_live = jhi >= jlo;
 
-    // one online-softmax step over a 32-key block (reference maximum with slack, as in
-    // band_dma_kernel); leaves the exponentials in s
+    // the band test of a block, then the softmax step
     auto soft = [&](f32x16& s, int jb) {
       if (!all_full) {
 #pragma unroll
@@ -1394,80 +1466,18 @@ __global__ __launch_bounds__(256, 2) void band_dma_f32_kernel(TileArgs a) {
           s[v] = ok ? s[v] : kNegInf;
         }
       }
-      float mx = s[0];
-#pragma unroll
-      for (int v = 1; v < 16; v++) mx = fmaxf(mx, s[v]);
-      mx = fmaxf(mx, shfl_xor_f32(mx, 32)) * sc;
-      mt = fmaxf(mt, mx);
-      if (__builtin_expect(__builtin_amdgcn_ballot_w64(mx > m + kSlack) != 0, 0)) {
-        const float m_new = (mx > m + kSlack) ? mx : m;
-        const float alpha = (m > kNegInf) ? __builtin_amdgcn_exp2f(m - m_new) : 0.f;
-        m = m_new;
-        l *= alpha;
-#pragma unroll
-        for (int eb = 0; eb < EB; eb++)
-#pragma unroll
-          for (int v = 0; v < 16; v++) o[eb][v] *= alpha;
-      }
-      const float neg_m = (m > kNegInf) ? -m : 0.f;
-      float lsum = 0.f;
-#pragma unroll
-      for (int v = 0; v < 16; v++) {
-        const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(s[v], sc, neg_m));  // exp2(-inf) = 0
-        s[v] = p;
-        lsum += p;
-      }
-      l += lsum;
+      soft_core(s);
     };
 
-    const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     f32x16 s[NB];
-    // ---- S^T = K Q^T, operand reads two groups of four instructions ahead (order pinned)
+#pragma unroll
+    for (int jb = 0; jb < NB; jb++) s[jb] = s_product(tb + 32 * jb * ROWB);
+    // ---- softmax and O^T += V^T P^T per block
 #pragma unroll
     for (int jb = 0; jb < NB; jb++) {
-      const char* kb = tb + 32 * jb * ROWB;
-      float4v kx[3];
-      kx[0] = *reinterpret_cast<const float4v*>(kb + kadr[0]);
-      kx[1] = *reinterpret_cast<const float4v*>(kb + kadr[1]);
-      s[jb] = zero16;
-      __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-#pragma unroll
-      for (int g = 0; g < D / 8; g++) {
-        if (g + 2 < D / 8) {
-          kx[(g + 2) % 3] = *reinterpret_cast<const float4v*>(kb + kadr[(g + 2) % 8] + 256 * ((g + 2) / 8));
-          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-        }
-#pragma unroll
-        for (int i = 0; i < 4; i++)
-          s[jb] = __builtin_amdgcn_mfma_f32_32x32x2f32(kx[g % 3][i], qf[4 * g + i], s[jb], 0, 0, 0);
-        __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
-      }
-    }
-    // ---- softmax and O^T += V^T P^T per block, V reads PD keys ahead (order pinned)
-    typedef float vecE __attribute__((ext_vector_type(EB)));
-    constexpr int PD = 8 / EB;
-#pragma unroll
-    for (int jb = 0; jb < NB; jb++) {
-      const char* vb = tb + 32 * jb * ROWB;
       soft(s[jb], jb);
       __builtin_amdgcn_sched_barrier(0);
-      vecE vx[PD + 1];
-#pragma unroll
-      for (int v = 0; v < PD; v++)
-        vx[v] = *reinterpret_cast<const vecE*>(vb + vadr[v % 8] + 16 * ROWB * (v / 8));
-      __builtin_amdgcn_sched_group_barrier(0x100, PD, 0);
-#pragma unroll
-      for (int v = 0; v < 16; v++) {
-        if (v + PD < 16) {
-          vx[(v + PD) % (PD + 1)] =
-              *reinterpret_cast<const vecE*>(vb + vadr[(v + PD) % 8] + 16 * ROWB * ((v + PD) / 8));
-          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-        }
-#pragma unroll
-        for (int eb = 0; eb < EB; eb++)
-          o[eb] = __builtin_amdgcn_mfma_f32_32x32x2f32(vx[v % (PD + 1)][eb], s[jb][v], o[eb], 0, 0, 0);
-        __builtin_amdgcn_sched_group_barrier(0x008, EB, 0);
-      }
+      pv_product(tb + 32 * jb * ROWB, s[jb]);
     }
   };
 
@@ -1475,6 +1485,55 @@ __global__ __launch_bounds__(256, 2) void band_dma_f32_kernel(TileArgs a) {
   for (int ut = u_lo; ut < u_hi; ut += 2 * BN) {
     step(ut, lds_even, lds_odd);
     if (ut + BN < u_hi) step(ut + BN, lds_odd, lds_even);
+  }
+
+  // ---- listed global tokens as further keys (the window + global composite), as in
+  // band_dma_kernel: a query that is not a listed token itself attends the listed tokens outside
+  // its window; their K and V rows are gathered into the first tile buffer, BN at a time.  (Never
+  // together with shared tail tiles: the launcher makes none for such a call.)
+  if (a.globs != nullptr) {
+    __shared__ int gtok_s[BN];  // token of every key of the gathered tile (-1: no key)
+    const int64_t tok_base = bb * a.n;        // first row of this problem
+    const int64_t tq_tok = q_tok - tok_base;  // this lane's query token
+    const bool q_plain = q_ok && !bit_is_set(a.gbits, tq_tok);
+    const uint32_t w32 = (uint32_t)wlim, w2 = 2u * (uint32_t)wlim;
+    const uint32_t d0 = w32 - (uint32_t)(int32_t)tq_tok;  // key token + d0 > 2w: outside the window
+    const int ng = (int)a.n_globs;
+    for (int gt = 0; gt < ng; gt += BN) {
+      __builtin_amdgcn_s_waitcnt(0);
+      __syncthreads();  // everyone is done with the buffer (band tiles, or the previous gathered tile)
+#pragma unroll
+      for (int it = 0; it < NI; it++) {
+        const int at = (4 * it + wave) * 1024 + lane * 16;
+        const int j = at / ROWB, p = (at % ROWB) / 16;  // key slot and chunk position this lane fills
+        int g = -1;
+        if (gt + j < ng) g = listed_token(a.globs[gt + j], a.n);
+        if (p == 0) gtok_s[j] = g;
+        const int64_t src = (tok_base + (g < 0 ? 0 : g)) * (int64_t)ROWB + (int64_t)((p ^ (j & 15)) * 16);
+        char* dst = lds_even + (4 * it + wave) * 1024;
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(Kp + src),
+                                         (__attribute__((address_space(3))) void*)dst, 16, 0, 0);
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(Vp + src),
+                                         (__attribute__((address_space(3))) void*)(dst + TILE_B), 16, 0, 0);
+      }
+      __builtin_amdgcn_s_waitcnt(0);
+      __syncthreads();
+      if (tw0 >= qlen) continue;
+#pragma unroll
+      for (int jb = 0; jb < NB; jb++) {
+        if (gt + 32 * jb >= ng) break;
+        f32x16 sg = s_product(lds_even + 32 * jb * ROWB);
+#pragma unroll
+        for (int v = 0; v < 16; v++) {
+          const int tok = gtok_s[32 * jb + 8 * (v / 4) + 4 * h + (v % 4)];
+          const bool ok = q_plain && tok >= 0 && ((uint32_t)tok + d0 > w2);
+          sg[v] = ok ? sg[v] : kNegInf;
+        }
+        soft_core(sg);
+        __builtin_amdgcn_sched_barrier(0);
+        pv_product(lds_even + 32 * jb * ROWB, sg);
+      }
+    }
   }
 
   l += shfl_xor_f32(l, 32);
@@ -1659,7 +1718,8 @@ int launch_band_tiles(const TileArgs& a, int use_nan, hipStream_t stream) {
       else
         launch_tile_kernel<T, D, kTileBand>(ev, dim3((unsigned)grid), stream, a);
     } else {
-      if (a.globs != nullptr) return -1;  // (fp32: the composite runs its parts one after the other)
+      // listed global tokens as further keys: only the direct-to-LDS kernel takes them
+      if (a.globs != nullptr && !((D == 64 || D == 128) && a.n_globs <= kFusedMaxGlobals)) return -1;
       // Two workgroups fit a CU, and tiles take about the same time, so the grid runs in rounds
       // of `resident` tiles and the tiles of a last, sparsely filled round keep the chip
       // waiting for a whole round (0.14 ms for a single tile left over at d = 128, window 256).
@@ -1671,7 +1731,7 @@ int launch_band_tiles(const TileArgs& a, int use_nan, hipStream_t stream) {
       const int64_t n_all = a.n_tiles * a.t.n_batch;
       const int64_t resident = (int64_t)device_cu_count() * 2;
       const int64_t rem = n_all % resident;
-      at.n_tail = (4 * rem <= resident) ? rem : 0;
+      at.n_tail = (4 * rem <= resident && a.globs == nullptr) ? rem : 0;
       // loads write LDS directly where a tile's rows can be addressed with 32-bit offsets and
       // positions fit 32-bit arithmetic
       const int64_t max_len = a.block > 0 ? a.cnt : (a.n + a.s - 1) / a.s;
@@ -1685,6 +1745,8 @@ int launch_band_tiles(const TileArgs& a, int use_nan, hipStream_t stream) {
           const int64_t grid_d = (n_main + 7) / 8 * 8 + 4 * at.n_tail;
           launch_maybe_timed(ev, band_dma_f32_kernel<D>, dim3((unsigned)grid_d), dim3(256), stream, at);
         }
+      } else if (a.globs != nullptr) {
+        return -1;
       } else {
         const int64_t grid_t = (n_main + 7) / 8 * 8 + 4 * at.n_tail;
         launch_tile_kernel<T, D, kTileBand>(ev, dim3((unsigned)grid_t), stream, at);

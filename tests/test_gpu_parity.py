@@ -573,7 +573,7 @@ def test_bigbird_one_call_equals_dense_union(mods, dtype, d, n, w, n_globs):
 
 
 @pytest.mark.parametrize("dtype,d", [(torch.bfloat16, 64), (torch.float16, 128), (torch.bfloat16, 32),
-                                     (torch.float16, 256)])
+                                     (torch.float16, 256), (torch.float32, 64), (torch.float32, 128)])
 @pytest.mark.parametrize("n,w,kind", [(3000, 16, "one"), (3000, 100, "tile"), (2500, 40, "tile+1"),
                                       (4100, 64, "many"), (2048, 33, "repeats"), (1000, 999, "tile")])
 def test_bigbird_window_and_listed_tokens_in_one_kernel(mods, dtype, d, n, w, kind):
