@@ -818,11 +818,24 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void band_dma_kernel(TileArgs
   // that is the same for the whole workgroup is moved to scalar registers.
   auto uni = [](int x) { return __builtin_amdgcn_readfirstlane(x); };
   // (the tiles of all problems of a batch form one list; problem bb starts at token bb * n)
+  // Whole tiles first, then four workgroups for each of the last a.n_tail tiles (the tiles of a
+  // sparsely filled last round): such a workgroup has 32 of the tile's queries, all four
+  // wavefronts work on them and take the key tiles in turn (folded through LDS at the end).
   const uint32_t n_tiles = (uint32_t)a.n_tiles, tiles_per_sub = (uint32_t)a.tiles_per_sub;
   const uint32_t n_all = n_tiles * (uint32_t)a.t.n_batch;
-  const uint32_t per_xcd = (n_all + 7u) / 8u;
-  uint32_t lt = (blockIdx.x % 8u) * per_xcd + blockIdx.x / 8u;
-  if (lt >= n_all) return;
+  const uint32_t n_main = n_all - (uint32_t)a.n_tail;
+  const uint32_t per_xcd = (n_main + 7u) / 8u;
+  uint32_t lt;
+  int quarter = -1;  // which 32 queries of a shared tail tile (-1: a whole tile)
+  if (blockIdx.x < 8u * per_xcd) {
+    lt = (blockIdx.x % 8u) * per_xcd + blockIdx.x / 8u;
+    if (lt >= n_main) return;
+  } else {
+    const uint32_t qid = blockIdx.x - 8u * per_xcd;
+    lt = n_main + qid / 4u;
+    quarter = uni((int)(qid & 3u));
+  }
+  const bool quad = quarter >= 0;
   const uint32_t bb = lt / n_tiles;
   lt -= bb * n_tiles;
   const uint32_t sub = lt / tiles_per_sub;
@@ -837,10 +850,11 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void band_dma_kernel(TileArgs
     qlen = uni((int)(((uint32_t)a.n - sub + (uint32_t)a.s - 1u) / (uint32_t)a.s));
   }
   const int wlim = (int)(a.w < (int64_t)0x3fffffff ? a.w : (int64_t)0x3fffffff);  // window, clamped
-  const int t0 = tile * BM;
+  const int t0 = tile * BM + (quad ? 32 * quarter : 0);
+  const int qspan = quad ? 32 : BM;
   if (t0 >= qlen) return;
   const int u_lo = t0 > wlim ? t0 - wlim : 0;
-  const int u_hi = (qlen - BM - wlim > t0) ? t0 + BM + wlim : qlen;
+  const int u_hi = (qlen - qspan - wlim > t0) ? t0 + qspan + wlim : qlen;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -906,8 +920,8 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void band_dma_kernel(TileArgs
   for (int i = 0; i < NBUF - 1; i++)
     if (u_lo + i * BN < u_hi) request(u_lo + i * BN, i);
 
-  const int tw0 = t0 + 32 * wave;  // first query of this wavefront
-  const int tq = tw0 + r;          // this lane's query position
+  const int tw0 = t0 + (quad ? 0 : 32 * wave);  // first query of this wavefront
+  const int tq = tw0 + r;                       // this lane's query position
   const bool q_ok = tq < qlen;
   const int64_t q_tok = base + (int64_t)(q_ok ? tq : qlen - 1) * a.s;
 
@@ -1056,6 +1070,8 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void band_dma_kernel(TileArgs
       test[jb] = dead || (ub < tw0 + 31 - wlim) || (ub + 31 - wlim > tw0) || (ub + 32 > u_hi);
       none = none && dead;
     }
+    // (a shared tail tile: the wavefronts take the key tiles in turn)
+    if (quad && (((ut - u_lo) / BN) & 3) != wave) none = true;
 
     // The K operands of the first block are asked for before the next tile is requested:
     // the four wavefronts issue their tile loads in one burst right after the barrier, and the
@@ -1201,6 +1217,44 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void band_dma_kernel(TileArgs
   }
 
   l += shfl_xor_f32(l, 32);
+  if (quad) {
+    // fold the four wavefronts (same queries, different key tiles) through LDS, 2, 3 into 0, 1
+    // and then 1 into 0; the tile buffers are no longer needed
+    constexpr int XR = EB * 16 + 3;
+    if constexpr (2 * XR * kWave * 4 <= NBUF * BUF_B) {
+      for (int fs = 2; fs >= 1; fs >>= 1) {
+        const bool gives = wave >= fs && wave < 2 * fs;
+        const bool takes = wave < fs;
+        float* xs = reinterpret_cast<float*>(lds) + (size_t)(gives ? wave - fs : wave) * XR * kWave + lane;
+        __syncthreads();
+        if (gives) {
+#pragma unroll
+          for (int eb = 0; eb < EB; eb++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) xs[(eb * 16 + v) * kWave] = o[eb][v];
+          xs[(EB * 16) * kWave] = m;
+          xs[(EB * 16 + 1) * kWave] = l;
+          xs[(EB * 16 + 2) * kWave] = mt;
+        }
+        __syncthreads();
+        if (takes) {
+          const float m2 = xs[(EB * 16) * kWave], l2 = xs[(EB * 16 + 1) * kWave];
+          mt = fmaxf(mt, xs[(EB * 16 + 2) * kWave]);
+          const float m_new = fmaxf(m, m2);
+          if (m_new > kNegInf) {
+            const float fa = __builtin_amdgcn_exp2f(m - m_new), fb = __builtin_amdgcn_exp2f(m2 - m_new);
+            l = l * fa + l2 * fb;
+#pragma unroll
+            for (int eb = 0; eb < EB; eb++)
+#pragma unroll
+              for (int v = 0; v < 16; v++) o[eb][v] = o[eb][v] * fa + xs[(eb * 16 + v) * kWave] * fb;
+            m = m_new;
+          }
+        }
+      }
+    }
+    if (wave != 0) return;
+  }
   if (q_ok && l > 0.f) {
     // hand the row over relative to its true maximum: (m, l, o) -> (mt, l * 2^(m - mt), o)
     // (o is divided by l later, so only l changes)
@@ -1713,10 +1767,21 @@ int launch_band_tiles(const TileArgs& a, int use_nan, hipStream_t stream) {
       if (a.globs != nullptr &&
           !(dma && a.n * a.t.n_batch * (int64_t)(2 * D) < ((int64_t)1 << 31) && a.n_globs <= kFusedMaxGlobals))
         return -1;
-      if (dma)
-        launch_maybe_timed(ev, band_dma_kernel<T, D, SPFA_BAND_BN(D)>, dim3((unsigned)grid), dim3(256), stream, a);
-      else
+      if (dma) {
+        // the tiles of a sparsely filled last round are shared out to four workgroups each (see
+        // the fp32 branch below); not with listed tokens, and not where the fold does not fit
+        TileArgs at = a;
+        using BC = BandDmaCfg<T, D, SPFA_BAND_BN(D)>;
+        const int64_t n_all = a.n_tiles * a.t.n_batch;
+        const int64_t resident = (int64_t)device_cu_count() * (D > 128 ? 1 : 2);
+        const int64_t rem = n_all % resident;
+        constexpr bool kFoldFits = 2 * (BC::EB * 16 + 3) * kWave * 4 <= BC::NBUF * BC::BUF_B;
+        at.n_tail = (kFoldFits && a.globs == nullptr && n_all > resident && 4 * rem <= resident) ? rem : 0;
+        const int64_t grid_d = (n_all - at.n_tail + 7) / 8 * 8 + 4 * at.n_tail;
+        launch_maybe_timed(ev, band_dma_kernel<T, D, SPFA_BAND_BN(D)>, dim3((unsigned)grid_d), dim3(256), stream, at);
+      } else {
         launch_tile_kernel<T, D, kTileBand>(ev, dim3((unsigned)grid), stream, a);
+      }
     } else {
       // listed global tokens as further keys: only the direct-to-LDS kernel takes them
       if (a.globs != nullptr && !((D == 64 || D == 128) && a.n_globs <= kFusedMaxGlobals)) return -1;

@@ -859,6 +859,32 @@ def test_band_masks_with_a_few_hundred_tiles(mods, dtype, d, kind, n, p1, p2):
     assert torch.allclose(o.float(), o1.float(), atol=2e-5 if dtype == torch.float32 else 2e-2)
 
 
+@pytest.mark.parametrize("dtype,d", [(torch.bfloat16, 64), (torch.float16, 128), (torch.float16, 32), (torch.float32, 64)])
+@pytest.mark.parametrize("kind,n,p1,p2", [("local", 66098, 40, 0), ("local", 65700, 300, 0), ("d1", 131500, 70, 1),
+                                          ("d1", 66000, 20, 2)])
+def test_band_masks_with_a_few_tiles_beyond_a_full_round(mods, dtype, d, kind, n, p1, p2):
+    """Query tiles a few more than the device holds at once (512 at two workgroups per CU of 256): the
+    tiles of the last, sparsely filled round are shared out to four workgroups each, whose wavefronts
+    deal the key tiles among themselves and fold their partial results.  The last tile of a
+    subsequence is partly filled; then a second call on top of the first."""
+    q, k, v = dev_qkv(n, d, dtype, 43, scale=0.5)
+    m, l, o = state(n, d, dtype, torch.float32)
+    if kind == "local":
+        call = lambda: mods["spfa_local"].forward(q, k, v, m, l, o, p1)
+        ref = c_oracle.local(np64(q), np64(k), np64(v), p1)
+    else:
+        call = lambda: mods["spfa_local_1d_dilated"].forward(q, k, v, m, l, o, p1, p2)
+        ref = c_oracle.local_1d_dilated(np64(q), np64(k), np64(v), p1, p2)
+    call()
+    sync()
+    check(o, m, l, *ref, dtype, state_dtype=torch.float32)
+    l1, o1 = l.clone(), o.clone()
+    call()
+    sync()
+    assert torch.allclose(l, 2 * l1, rtol=1e-5)
+    assert torch.allclose(o.float(), o1.float(), atol=2e-5 if dtype == torch.float32 else 2e-2)
+
+
 @pytest.mark.parametrize("dtype,d", [(torch.float32, 64), (torch.float32, 128), (torch.bfloat16, 128)])
 def test_band_masks_batch_with_a_few_hundred_tiles(mods, dtype, d):
     """Three heads of 9000 tokens in one call: 213 whole tiles over the stacked problems."""
