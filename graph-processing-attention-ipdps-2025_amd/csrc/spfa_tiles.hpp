@@ -1796,7 +1796,11 @@ int launch_band_tiles(const TileArgs& a, int use_nan, hipStream_t stream) {
       const int64_t n_all = a.n_tiles * a.t.n_batch;
       const int64_t resident = (int64_t)device_cu_count() * 2;
       const int64_t rem = n_all % resident;
-      at.n_tail = (4 * rem <= resident && a.globs == nullptr) ? rem : 0;
+      // (a problem of less than a round: only while every such workgroup gets a CU to itself -
+      // 64 tiles, i.e. N = 8192, took 30 / 48 us instead of 33 / 58 at d = 64 / 128, but 128 tiles
+      // 44 / 201 us instead of 33 / 152 at d = 64, w = 128 / 1024)
+      const bool few = n_all > resident ? 4 * rem <= resident : 8 * rem <= resident;
+      at.n_tail = (few && a.globs == nullptr) ? rem : 0;
       // loads write LDS directly where a tile's rows can be addressed with 32-bit offsets and
       // positions fit 32-bit arithmetic
       const int64_t max_len = a.block > 0 ? a.cnt : (a.n + a.s - 1) / a.s;
