@@ -95,10 +95,13 @@ __device__ __forceinline__ float group_sum(float x) {
 // ---------------------------------------------------------------------------------------
 // VecLay: d * sizeof(T) == LPR * 16 bytes.  Lane c of a group owns 16 contiguous bytes of the
 // row, so one wave-wide load instruction fetches 64/LPR whole rows with full 16-byte lanes.
-template <typename T, int LPR_>
+// PAD: rows of any multiple of 16 bytes up to LPR * 16 - the lanes past the end of a row hold
+// zeros and neither load nor store (a row of 96 floats takes 24 of a group's 32 lanes).
+template <typename T, int LPR_, bool PAD_ = false>
 struct VecLay {
   using elem = T;
   static constexpr int LPR = LPR_;
+  static constexpr bool PAD = PAD_;
   static constexpr int GROUPS = kWave / LPR;
   static constexpr int NE = 16 / (int)sizeof(T);  // floats held per lane
   static constexpr int D = LPR * NE;
@@ -107,12 +110,15 @@ struct VecLay {
   static constexpr int U_MEDIUM = 8; // ... in the medium-row kernel
   using raw = uint4v;
 
-  __device__ static __forceinline__ raw load(const T* row_ptr, int c, int) {
+  __device__ static __forceinline__ raw load(const T* row_ptr, int c, int d) {
+    if constexpr (PAD) {
+      if (c * NE >= d) return raw{0u, 0u, 0u, 0u};
+    }
     return *reinterpret_cast<const raw*>(reinterpret_cast<const char*>(row_ptr) + c * 16);
   }
   // gathered K / V rows
-  __device__ static __forceinline__ raw load_gather(const T* row_ptr, int c, int) {
-    return *reinterpret_cast<const raw*>(reinterpret_cast<const char*>(row_ptr) + c * 16);
+  __device__ static __forceinline__ raw load_gather(const T* row_ptr, int c, int d) {
+    return load(row_ptr, c, d);
   }
   __device__ static __forceinline__ void unpack(const raw& r, float (&f)[NE]) {
     if constexpr (sizeof(T) == 4) {
@@ -132,7 +138,10 @@ struct VecLay {
       }
     }
   }
-  __device__ static __forceinline__ void store(T* row_ptr, int c, int, const float (&f)[NE]) {
+  __device__ static __forceinline__ void store(T* row_ptr, int c, int d, const float (&f)[NE]) {
+    if constexpr (PAD) {
+      if (c * NE >= d) return;
+    }
     raw r;
     if constexpr (sizeof(T) == 4) {
       float4v x;
@@ -153,19 +162,98 @@ struct VecLay {
     *reinterpret_cast<raw*>(reinterpret_cast<char*>(row_ptr) + c * 16) = r;
   }
   // fp32 partial rows in the workspace: element e of lane c is at c*NE + e
-  __device__ static __forceinline__ void load_f32(const float* row_ptr, int c, int, float (&f)[NE]) {
+  __device__ static __forceinline__ void load_f32(const float* row_ptr, int c, int d, float (&f)[NE]) {
+    if constexpr (PAD) {
+      if (c * NE >= d) {
+#pragma unroll
+        for (int e = 0; e < NE; e++) f[e] = 0.f;
+        return;
+      }
+    }
 #pragma unroll
     for (int e = 0; e < NE; e += 4) {
       float4v x = *reinterpret_cast<const float4v*>(row_ptr + c * NE + e);
       f[e] = x[0]; f[e + 1] = x[1]; f[e + 2] = x[2]; f[e + 3] = x[3];
     }
   }
-  __device__ static __forceinline__ void store_f32(float* row_ptr, int c, int, const float (&f)[NE]) {
+  __device__ static __forceinline__ void store_f32(float* row_ptr, int c, int d, const float (&f)[NE]) {
+    if constexpr (PAD) {
+      if (c * NE >= d) return;
+    }
 #pragma unroll
     for (int e = 0; e < NE; e += 4) {
       float4v x = {f[e], f[e + 1], f[e + 2], f[e + 3]};
       *reinterpret_cast<float4v*>(row_ptr + c * NE + e) = x;
     }
+  }
+};
+
+// WideLay: rows of more than 512 and at most 1024 bytes (a multiple of 16).  Half a wavefront per
+// row; lane c owns the 16-byte chunks c and c + 32 of it (two load instructions per row, each
+// 512 contiguous bytes), lanes past the end of a row hold zeros.
+template <typename T>
+struct WideLay {
+  using elem = T;
+  static constexpr int LPR = 32;
+  static constexpr bool PAD = true;
+  static constexpr int GROUPS = kWave / LPR;
+  static constexpr int NC = 16 / (int)sizeof(T);  // elements per chunk
+  static constexpr int NE = 2 * NC;               // floats held per lane
+  static constexpr int U = 8;  // (twice the bytes per neighbour of VecLay)
+  static constexpr int U_SHORT = 2;
+  static constexpr int U_MEDIUM = 4;
+  struct raw { uint4v x[2]; };
+
+  __device__ static __forceinline__ raw load(const T* row_ptr, int c, int d) {
+    raw r;
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+      const int ch = c + 32 * j;
+      r.x[j] = uint4v{0u, 0u, 0u, 0u};
+      if (ch * NC < d) r.x[j] = *reinterpret_cast<const uint4v*>(reinterpret_cast<const char*>(row_ptr) + ch * 16);
+    }
+    return r;
+  }
+  __device__ static __forceinline__ raw load_gather(const T* row_ptr, int c, int d) { return load(row_ptr, c, d); }
+  __device__ static __forceinline__ void unpack(const raw& r, float (&f)[NE]) {
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+      float g[NC];
+      VecLay<T, 32>::unpack(r.x[j], g);
+#pragma unroll
+      for (int e = 0; e < NC; e++) f[j * NC + e] = g[e];
+    }
+  }
+  __device__ static __forceinline__ void store(T* row_ptr, int c, int d, const float (&f)[NE]) {
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+      float g[NC];
+#pragma unroll
+      for (int e = 0; e < NC; e++) g[e] = f[j * NC + e];
+      VecLay<T, 64, true>::store(row_ptr, c + 32 * j, d, g);
+    }
+  }
+  // fp32 partial rows in the workspace: the row's own element order
+  __device__ static __forceinline__ void load_f32(const float* row_ptr, int c, int d, float (&f)[NE]) {
+#pragma unroll
+    for (int j = 0; j < 2; j++)
+#pragma unroll
+      for (int e = 0; e < NC; e += 4) {
+        const int idx = (c + 32 * j) * NC + e;
+        float4v x = {0.f, 0.f, 0.f, 0.f};
+        if (idx < d) x = *reinterpret_cast<const float4v*>(row_ptr + idx);
+        f[j * NC + e] = x[0]; f[j * NC + e + 1] = x[1]; f[j * NC + e + 2] = x[2]; f[j * NC + e + 3] = x[3];
+      }
+  }
+  __device__ static __forceinline__ void store_f32(float* row_ptr, int c, int d, const float (&f)[NE]) {
+#pragma unroll
+    for (int j = 0; j < 2; j++)
+#pragma unroll
+      for (int e = 0; e < NC; e += 4) {
+        const int idx = (c + 32 * j) * NC + e;
+        float4v x = {f[j * NC + e], f[j * NC + e + 1], f[j * NC + e + 2], f[j * NC + e + 3]};
+        if (idx < d) *reinterpret_cast<float4v*>(row_ptr + idx) = x;
+      }
   }
 };
 

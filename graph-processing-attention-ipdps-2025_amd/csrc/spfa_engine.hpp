@@ -889,6 +889,15 @@ int run_engine(const Tensors& t, const Mask& mask, const EngineSizing& s, int us
     if (row_bytes == 128) return launch_engine<VecLay<T, 8>, Mask>(t, mask, s, use_nan, ws, stream, phase, plan_buf);
     if (row_bytes == 256) return launch_engine<VecLay<T, 16>, Mask>(t, mask, s, use_nan, ws, stream, phase, plan_buf);
     if (row_bytes == 512) return launch_engine<VecLay<T, 32>, Mask>(t, mask, s, use_nan, ws, stream, phase, plan_buf);
+    // other multiples of 16 bytes: the next layout up with its last lanes idle, then two chunks
+    // per lane up to 1024 bytes
+    if (row_bytes % 16 == 0) {
+      if (row_bytes < 64) return launch_engine<VecLay<T, 4, true>, Mask>(t, mask, s, use_nan, ws, stream, phase, plan_buf);
+      if (row_bytes < 128) return launch_engine<VecLay<T, 8, true>, Mask>(t, mask, s, use_nan, ws, stream, phase, plan_buf);
+      if (row_bytes < 256) return launch_engine<VecLay<T, 16, true>, Mask>(t, mask, s, use_nan, ws, stream, phase, plan_buf);
+      if (row_bytes < 512) return launch_engine<VecLay<T, 32, true>, Mask>(t, mask, s, use_nan, ws, stream, phase, plan_buf);
+      if (row_bytes <= 1024) return launch_engine<WideLay<T>, Mask>(t, mask, s, use_nan, ws, stream, phase, plan_buf);
+    }
   }
   if (t.d <= 128) return launch_engine<GenLay<T, 2>, Mask>(t, mask, s, use_nan, ws, stream, phase, plan_buf);
   if (t.d <= 1024) return launch_engine<GenLay<T, 16>, Mask>(t, mask, s, use_nan, ws, stream, phase, plan_buf);
