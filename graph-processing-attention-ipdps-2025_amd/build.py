@@ -124,6 +124,8 @@ def _source_loop_depth(kname: str) -> int:
     m = re.search(r"6VecLayI\w+?Li(\d+)E", kname)
     if m:
         lpr, unroll = int(m.group(1)), (16 if seg else 8 if med else 4)
+    elif "7WideLayI" in kname:
+        lpr, unroll = 32, (8 if seg else 4 if med else 2)
     else:
         m = re.search(r"6GenLayI\w+?Li(\d+)E", kname)
         lpr, unroll = 64, (8 if int(m.group(1)) <= 2 else 2)

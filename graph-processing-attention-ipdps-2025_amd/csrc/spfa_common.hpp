@@ -109,6 +109,8 @@ struct VecLay {
   static constexpr int U_SHORT = 4;  // ... in the row kernel
   static constexpr int U_MEDIUM = 8; // ... in the medium-row kernel
   using raw = uint4v;
+  // which element of the row lane c holds in slot e (may lie past the end of a padded row)
+  __device__ static __forceinline__ int elem_index(int c, int e) { return c * NE + e; }
 
   __device__ static __forceinline__ raw load(const T* row_ptr, int c, int d) {
     if constexpr (PAD) {
@@ -203,6 +205,7 @@ struct WideLay {
   static constexpr int U_SHORT = 2;
   static constexpr int U_MEDIUM = 4;
   struct raw { uint4v x[2]; };
+  __device__ static __forceinline__ int elem_index(int c, int e) { return (c + 32 * (e / NC)) * NC + e % NC; }
 
   __device__ static __forceinline__ raw load(const T* row_ptr, int c, int d) {
     raw r;
@@ -269,6 +272,7 @@ struct GenLay {
   static constexpr int U_SHORT = U;
   static constexpr int U_MEDIUM = U;
   struct raw { T x[EPL]; };
+  __device__ static __forceinline__ int elem_index(int c, int e) { return c + e * kWave; }
 
   __device__ static __forceinline__ raw load(const T* row_ptr, int c, int d) {
     raw r;

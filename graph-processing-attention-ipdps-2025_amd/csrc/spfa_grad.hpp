@@ -51,7 +51,7 @@ constexpr int kGradItemBlocks = 2048;
 
 template <class Lay>
 __device__ __forceinline__ int grad_elem_index(int c, int e) {
-  return (Lay::LPR == kWave) ? c + e * kWave : c * Lay::NE + e;
+  return Lay::elem_index(c, e);
 }
 
 // lse and delta of every query row: 16 lanes per row, 16 bytes per lane and step
@@ -370,6 +370,13 @@ int run_grad(const Tensors& t, const GradArgs& g, const RowMask& rows, const Col
   if (row_bytes == 128) return launch_grad<VecLay<T, 8>>(t, g, rows, cols, stream);
   if (row_bytes == 256) return launch_grad<VecLay<T, 16>>(t, g, rows, cols, stream);
   if (row_bytes == 512) return launch_grad<VecLay<T, 32>>(t, g, rows, cols, stream);
+  if (row_bytes % 16 == 0) {  // (the padded layouts of the forward engine)
+    if (row_bytes < 64) return launch_grad<VecLay<T, 4, true>>(t, g, rows, cols, stream);
+    if (row_bytes < 128) return launch_grad<VecLay<T, 8, true>>(t, g, rows, cols, stream);
+    if (row_bytes < 256) return launch_grad<VecLay<T, 16, true>>(t, g, rows, cols, stream);
+    if (row_bytes < 512) return launch_grad<VecLay<T, 32, true>>(t, g, rows, cols, stream);
+    if (row_bytes <= 1024) return launch_grad<WideLay<T>>(t, g, rows, cols, stream);
+  }
   if (t.d <= 128) return launch_grad<GenLay<T, 2>>(t, g, rows, cols, stream);
   if (t.d <= 1024) return launch_grad<GenLay<T, 16>>(t, g, rows, cols, stream);
   return 5;
