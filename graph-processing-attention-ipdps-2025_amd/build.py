@@ -125,7 +125,9 @@ def _source_loop_depth(kname: str) -> int:
     if m:
         lpr, unroll = int(m.group(1)), (16 if seg else 8 if med else 4)
     elif "7WideLayI" in kname:
-        lpr, unroll = 32, (8 if seg else 4 if med else 2)
+        nch = int(re.search(r"7WideLayI\w+?Li(\d+)E", kname).group(1))
+        u = 16 // nch
+        lpr, unroll = 32, (u if seg else max(u // 2, 1) if med else max(u // 4, 1))
     else:
         m = re.search(r"6GenLayI\w+?Li(\d+)E", kname)
         lpr, unroll = 64, (8 if int(m.group(1)) <= 2 else 2)

@@ -190,27 +190,29 @@ struct VecLay {
   }
 };
 
-// WideLay: rows of more than 512 and at most 1024 bytes (a multiple of 16).  Half a wavefront per
-// row; lane c owns the 16-byte chunks c and c + 32 of it (two load instructions per row, each
+// WideLay: rows of more than 512 bytes, up to NCH * 512 (a multiple of 16).  Half a wavefront per
+// row; lane c owns the 16-byte chunks c, c + 32, ... of it (NCH load instructions per row, each
 // 512 contiguous bytes), lanes past the end of a row hold zeros.
-template <typename T>
+template <typename T, int NCH_>
 struct WideLay {
   using elem = T;
   static constexpr int LPR = 32;
+  static constexpr int NCH = NCH_;
   static constexpr bool PAD = true;
   static constexpr int GROUPS = kWave / LPR;
   static constexpr int NC = 16 / (int)sizeof(T);  // elements per chunk
-  static constexpr int NE = 2 * NC;               // floats held per lane
-  static constexpr int U = 8;  // (twice the bytes per neighbour of VecLay)
-  static constexpr int U_SHORT = 2;
-  static constexpr int U_MEDIUM = 4;
-  struct raw { uint4v x[2]; };
+  static constexpr int NE = NCH * NC;             // floats held per lane
+  static constexpr int U = 16 / NCH;  // (the bytes in flight per lane of VecLay)
+  static constexpr int U_SHORT = U >= 4 ? U / 4 : 1;
+  static constexpr int U_MEDIUM = U >= 2 ? U / 2 : 1;
+  static_assert(NCH == 2 || NCH == 4 || NCH == 8, "two to eight chunks per lane");
+  struct raw { uint4v x[NCH]; };
   __device__ static __forceinline__ int elem_index(int c, int e) { return (c + 32 * (e / NC)) * NC + e % NC; }
 
   __device__ static __forceinline__ raw load(const T* row_ptr, int c, int d) {
     raw r;
 #pragma unroll
-    for (int j = 0; j < 2; j++) {
+    for (int j = 0; j < NCH; j++) {
       const int ch = c + 32 * j;
       r.x[j] = uint4v{0u, 0u, 0u, 0u};
       if (ch * NC < d) r.x[j] = *reinterpret_cast<const uint4v*>(reinterpret_cast<const char*>(row_ptr) + ch * 16);
@@ -220,7 +222,7 @@ struct WideLay {
   __device__ static __forceinline__ raw load_gather(const T* row_ptr, int c, int d) { return load(row_ptr, c, d); }
   __device__ static __forceinline__ void unpack(const raw& r, float (&f)[NE]) {
 #pragma unroll
-    for (int j = 0; j < 2; j++) {
+    for (int j = 0; j < NCH; j++) {
       float g[NC];
       VecLay<T, 32>::unpack(r.x[j], g);
 #pragma unroll
@@ -229,7 +231,7 @@ struct WideLay {
   }
   __device__ static __forceinline__ void store(T* row_ptr, int c, int d, const float (&f)[NE]) {
 #pragma unroll
-    for (int j = 0; j < 2; j++) {
+    for (int j = 0; j < NCH; j++) {
       float g[NC];
 #pragma unroll
       for (int e = 0; e < NC; e++) g[e] = f[j * NC + e];
@@ -239,7 +241,7 @@ struct WideLay {
   // fp32 partial rows in the workspace: the row's own element order
   __device__ static __forceinline__ void load_f32(const float* row_ptr, int c, int d, float (&f)[NE]) {
 #pragma unroll
-    for (int j = 0; j < 2; j++)
+    for (int j = 0; j < NCH; j++)
 #pragma unroll
       for (int e = 0; e < NC; e += 4) {
         const int idx = (c + 32 * j) * NC + e;
@@ -250,7 +252,7 @@ struct WideLay {
   }
   __device__ static __forceinline__ void store_f32(float* row_ptr, int c, int d, const float (&f)[NE]) {
 #pragma unroll
-    for (int j = 0; j < 2; j++)
+    for (int j = 0; j < NCH; j++)
 #pragma unroll
       for (int e = 0; e < NC; e += 4) {
         const int idx = (c + 32 * j) * NC + e;

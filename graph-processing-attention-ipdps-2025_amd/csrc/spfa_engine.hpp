@@ -896,7 +896,11 @@ int run_engine(const Tensors& t, const Mask& mask, const EngineSizing& s, int us
       if (row_bytes < 128) return launch_engine<VecLay<T, 8, true>, Mask>(t, mask, s, use_nan, ws, stream, phase, plan_buf);
       if (row_bytes < 256) return launch_engine<VecLay<T, 16, true>, Mask>(t, mask, s, use_nan, ws, stream, phase, plan_buf);
       if (row_bytes < 512) return launch_engine<VecLay<T, 32, true>, Mask>(t, mask, s, use_nan, ws, stream, phase, plan_buf);
-      if (row_bytes <= 1024) return launch_engine<WideLay<T>, Mask>(t, mask, s, use_nan, ws, stream, phase, plan_buf);
+      if (row_bytes <= 1024) return launch_engine<WideLay<T, 2>, Mask>(t, mask, s, use_nan, ws, stream, phase, plan_buf);
+      if (row_bytes <= 2048) return launch_engine<WideLay<T, 4>, Mask>(t, mask, s, use_nan, ws, stream, phase, plan_buf);
+      if constexpr (sizeof(T) == 4) {  // (d <= 1024: only fp32 rows get this long)
+        if (row_bytes <= 4096) return launch_engine<WideLay<T, 8>, Mask>(t, mask, s, use_nan, ws, stream, phase, plan_buf);
+      }
     }
   }
   if (t.d <= 128) return launch_engine<GenLay<T, 2>, Mask>(t, mask, s, use_nan, ws, stream, phase, plan_buf);

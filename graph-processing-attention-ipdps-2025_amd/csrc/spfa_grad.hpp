@@ -375,7 +375,11 @@ int run_grad(const Tensors& t, const GradArgs& g, const RowMask& rows, const Col
     if (row_bytes < 128) return launch_grad<VecLay<T, 8, true>>(t, g, rows, cols, stream);
     if (row_bytes < 256) return launch_grad<VecLay<T, 16, true>>(t, g, rows, cols, stream);
     if (row_bytes < 512) return launch_grad<VecLay<T, 32, true>>(t, g, rows, cols, stream);
-    if (row_bytes <= 1024) return launch_grad<WideLay<T>>(t, g, rows, cols, stream);
+    if (row_bytes <= 1024) return launch_grad<WideLay<T, 2>>(t, g, rows, cols, stream);
+    if (row_bytes <= 2048) return launch_grad<WideLay<T, 4>>(t, g, rows, cols, stream);
+    if constexpr (sizeof(T) == 4) {  // (d <= 1024: only fp32 rows get this long)
+      if (row_bytes <= 4096) return launch_grad<WideLay<T, 8>>(t, g, rows, cols, stream);
+    }
   }
   if (t.d <= 128) return launch_grad<GenLay<T, 2>>(t, g, rows, cols, stream);
   if (t.d <= 1024) return launch_grad<GenLay<T, 16>>(t, g, rows, cols, stream);
