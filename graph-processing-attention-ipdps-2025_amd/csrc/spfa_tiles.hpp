@@ -83,9 +83,9 @@ template <typename T, int D>
 struct TileCfg {
   static constexpr bool kF32 = sizeof(T) == 4;
   static constexpr int BM = 128;  // queries per workgroup
-  // keys per LDS tile (fp32 at d = 128 and the half types at d = 256 take half tiles to stay
+  // keys per LDS tile (fp32 above d = 64 and the half types at d = 256 take half tiles to stay
   // inside 64 KB of LDS)
-  static constexpr int BN = (kF32 ? D > 64 : D > 128) ? 32 : 64;
+  static constexpr int BN = (kF32 ? D > 64 : D >= 256) ? 32 : 64;
   static constexpr int NB = BN / 32;  // 32-key blocks per tile
   // K tile: [key][k] rows padded so that the 32 keys read by one operand fetch spread over the
   // banks.  V tile: half types are stored transposed [e][key'] (16-byte operand reads), fp32
@@ -128,6 +128,14 @@ __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
 template <bool B>
 struct BoolConst {
   static constexpr bool value = B;
+};
+
+// N adjacent floats of an LDS row, read as one piece where N is a power of two (8 or 16 bytes,
+// aligned as such), as single floats otherwise (d = 96, 160, 192, 224: 3, 5, 6, 7 floats)
+template <int N>
+struct alignas((N & (N - 1)) == 0 ? 4 * N : 4) RowPiece {
+  float x[N];
+  __device__ __forceinline__ float operator[](int i) const { return x[i]; }
 };
 
 // Fold the incoming state of row `row` into a finished tile result and write the row back.
@@ -612,7 +620,7 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void tile_kernel(TileArgs a) 
     for (int jb = 0; jb < NB; jb++) {
       if (!need[jb]) continue;
       if constexpr (kF32) {
-        typedef float vecE __attribute__((ext_vector_type(EB)));
+        typedef RowPiece<EB> vecE;
         const float* vbase = (const float*)Vs + (32 * jb + 4 * h) * C::V_STRIDE + EB * r;
         // reads run PD keys ahead of the instructions that use them (order pinned, as above)
         constexpr int PD = 8 / EB;
@@ -1680,9 +1688,10 @@ __global__ __launch_bounds__(256) void global_rows_merge_kernel(TileArgs a) {
   __syncthreads();
   lsum = (red[0] + red[1]) + (red[2] + red[3]);
 
+  // (d that does not divide 256: the threads past NSUB * d have no element)
   const int e = tid % D, sub = tid / D;
   float acc = 0.f;
-  int64_t k = sub;
+  int64_t k = sub < NSUB ? sub : a.n_split;
   for (; k + 3 * NSUB < a.n_split; k += 4 * NSUB) {
     float x[4], wgt[4];
 #pragma unroll
@@ -1759,7 +1768,8 @@ int launch_band_tiles(const TileArgs& a, int use_nan, hipStream_t stream) {
       // the direct-to-LDS kernel addresses a tile's rows with 32-bit offsets, and tile numbers,
       // windows and positions with 32-bit arithmetic
       const int64_t max_len = a.block > 0 ? a.cnt : (a.n + a.s - 1) / a.s;
-      const bool dma = a.s * (int64_t)(2 * D) * 64 < ((int64_t)1 << 31) && a.n < ((int64_t)1 << 31) &&
+      constexpr bool kDmaShape = D == 32 || D == 64 || D == 128 || D == 256;  // (rows a power of two long)
+      const bool dma = kDmaShape && a.s * (int64_t)(2 * D) * 64 < ((int64_t)1 << 31) && a.n < ((int64_t)1 << 31) &&
                        a.n_tiles * a.t.n_batch < ((int64_t)1 << 31) &&
                        (a.w <= (int64_t)0x3fffffff || max_len <= (int64_t)0x3fffffff);
       // listed global tokens as further keys: only the direct-to-LDS kernel takes them, and it
@@ -1767,7 +1777,7 @@ int launch_band_tiles(const TileArgs& a, int use_nan, hipStream_t stream) {
       if (a.globs != nullptr &&
           !(dma && a.n * a.t.n_batch * (int64_t)(2 * D) < ((int64_t)1 << 31) && a.n_globs <= kFusedMaxGlobals))
         return -1;
-      if (dma) {
+      if constexpr (kDmaShape) if (dma) {
         // the tiles of a sparsely filled last round are shared out to four workgroups each (see
         // the fp32 branch below); not with listed tokens, and not where the fold does not fit
         TileArgs at = a;
@@ -1779,9 +1789,8 @@ int launch_band_tiles(const TileArgs& a, int use_nan, hipStream_t stream) {
         at.n_tail = (kFoldFits && a.globs == nullptr && n_all > resident && 4 * rem <= resident) ? rem : 0;
         const int64_t grid_d = (n_all - at.n_tail + 7) / 8 * 8 + 4 * at.n_tail;
         launch_maybe_timed(ev, band_dma_kernel<T, D, SPFA_BAND_BN(D)>, dim3((unsigned)grid_d), dim3(256), stream, at);
-      } else {
-        launch_tile_kernel<T, D, kTileBand>(ev, dim3((unsigned)grid), stream, a);
       }
+      if (!dma) launch_tile_kernel<T, D, kTileBand>(ev, dim3((unsigned)grid), stream, a);
     } else {
       // listed global tokens as further keys: only the direct-to-LDS kernel takes them
       if (a.globs != nullptr && !((D == 64 || D == 128) && a.n_globs <= kFusedMaxGlobals)) return -1;
@@ -1863,7 +1872,7 @@ int launch_global_tiles(const TileArgs& a, hipStream_t stream, bool rows_only) {
 inline bool tile_shape_ok(const Tensors& t, size_t elem_bytes) {
   if (!aligned16(t.q) || !aligned16(t.k) || !aligned16(t.v) || !aligned16(t.out)) return false;
   (void)elem_bytes;
-  return t.d == 32 || t.d == 64 || t.d == 128 || t.d == 256;
+  return t.d % 32 == 0 && t.d >= 32 && t.d <= 256;
 }
 
 // Returns -1 when the shape is not covered (caller falls back to the row-gather engine).
@@ -1874,6 +1883,10 @@ int run_band_tiles(const TileArgs& a, int use_nan, hipStream_t stream) {
   if (a.t.d == 128) return launch_band_tiles<T, 128>(a, use_nan, stream);
   if (a.t.d == 32) return launch_band_tiles<T, 32>(a, use_nan, stream);
   if (a.t.d == 256) return launch_band_tiles<T, 256>(a, use_nan, stream);
+  if (a.t.d == 96) return launch_band_tiles<T, 96>(a, use_nan, stream);
+  if (a.t.d == 160) return launch_band_tiles<T, 160>(a, use_nan, stream);
+  if (a.t.d == 192) return launch_band_tiles<T, 192>(a, use_nan, stream);
+  if (a.t.d == 224) return launch_band_tiles<T, 224>(a, use_nan, stream);
   return -1;
 }
 
@@ -1884,6 +1897,10 @@ int run_global_tiles(const TileArgs& a, hipStream_t stream, bool rows_only = fal
   if (a.t.d == 128) return launch_global_tiles<T, 128>(a, stream, rows_only);
   if (a.t.d == 32) return launch_global_tiles<T, 32>(a, stream, rows_only);
   if (a.t.d == 256) return launch_global_tiles<T, 256>(a, stream, rows_only);
+  if (a.t.d == 96) return launch_global_tiles<T, 96>(a, stream, rows_only);
+  if (a.t.d == 160) return launch_global_tiles<T, 160>(a, stream, rows_only);
+  if (a.t.d == 192) return launch_global_tiles<T, 192>(a, stream, rows_only);
+  if (a.t.d == 224) return launch_global_tiles<T, 224>(a, stream, rows_only);
   return -1;
 }
 

@@ -789,7 +789,10 @@ def test_coo_empty_mask(mods):
 @pytest.mark.parametrize("dtype,d", [(torch.float32, 64), (torch.bfloat16, 64), (torch.float16, 32),
                                      (torch.bfloat16, 128), (torch.float32, 48), (torch.float32, 128),
                                      (torch.bfloat16, 32), (torch.bfloat16, 256), (torch.float16, 256),
-                                     (torch.float32, 32), (torch.float32, 256)])
+                                     (torch.float32, 32), (torch.float32, 256), (torch.float32, 96),
+                                     (torch.bfloat16, 96), (torch.float16, 160), (torch.float32, 160),
+                                     (torch.bfloat16, 192), (torch.float32, 192), (torch.float16, 224),
+                                     (torch.float32, 224)])
 @pytest.mark.parametrize("n,w", [(1000, 0), (1000, 1), (1000, 128), (777, 776), (4096, 300), (130, 20)])
 def test_local(mods, dtype, d, n, w):
     q, k, v = dev_qkv(n, d, dtype, 30)
@@ -802,7 +805,8 @@ def test_local(mods, dtype, d, n, w):
 
 @pytest.mark.parametrize("dtype,d", [(torch.float32, 64), (torch.bfloat16, 128), (torch.float16, 64),
                                      (torch.float32, 128), (torch.float16, 32), (torch.bfloat16, 256),
-                                     (torch.float32, 32)])
+                                     (torch.float32, 32), (torch.float32, 96), (torch.bfloat16, 160),
+                                     (torch.float16, 192), (torch.float32, 224)])
 @pytest.mark.parametrize("n,w,dil", [(1000, 10, 2), (1000, 0, 3), (1000, 999, 0), (1001, 100, 1),
                                      (2048, 256, 2), (300, 299, 6), (5000, 40, 4)])
 def test_local_1d_dilated(mods, dtype, d, n, w, dil):
@@ -816,7 +820,8 @@ def test_local_1d_dilated(mods, dtype, d, n, w, dil):
 
 @pytest.mark.parametrize("dtype,d", [(torch.float32, 64), (torch.bfloat16, 128), (torch.float16, 64),
                                      (torch.float32, 128), (torch.bfloat16, 32), (torch.float16, 256),
-                                     (torch.float32, 32)])
+                                     (torch.float32, 32), (torch.bfloat16, 96), (torch.float32, 160),
+                                     (torch.float32, 192), (torch.float16, 224)])
 @pytest.mark.parametrize("n,block,dil", [(1024, 16, 0), (1024, 16, 1), (1024, 256, 2), (1000, 1000, 3),
                                          (1024, 1, 0), (960, 32, 31), (2048, 2048, 0), (1200, 300, 1)])
 @pytest.mark.parametrize("use_nan", [True, False])
@@ -831,7 +836,7 @@ def test_local_2d_dilated(mods, dtype, d, n, block, dil, use_nan):
 
 @pytest.mark.parametrize("dtype,d", [(torch.float32, 64), (torch.float32, 128), (torch.bfloat16, 64),
                                      (torch.float16, 128), (torch.float16, 32), (torch.bfloat16, 256),
-                                     (torch.float32, 32)])
+                                     (torch.float32, 32), (torch.float32, 96), (torch.bfloat16, 192)])
 @pytest.mark.parametrize("kind,n,p1,p2", [("local", 20011, 33, 0), ("local", 20011, 0, 0), ("local", 17000, 700, 0),
                                           ("d1", 20011, 70, 2), ("d1", 20000, 1500, 1), ("d1", 33333, 129, 4),
                                           ("d2", 20480, 128, 1), ("d2", 42000, 300, 2), ("d2", 30000, 200, 0)])
@@ -901,7 +906,9 @@ def test_band_masks_batch_with_a_few_hundred_tiles(mods, dtype, d):
 
 @pytest.mark.parametrize("dtype,d", [(torch.float32, 64), (torch.bfloat16, 64), (torch.float16, 128),
                                      (torch.float32, 128), (torch.float32, 32), (torch.bfloat16, 32),
-                                     (torch.float16, 256), (torch.bfloat16, 256), (torch.float32, 256)])
+                                     (torch.float16, 256), (torch.bfloat16, 256), (torch.float32, 256),
+                                     (torch.float32, 96), (torch.bfloat16, 96), (torch.float16, 160),
+                                     (torch.float32, 192), (torch.bfloat16, 224), (torch.float32, 224)])
 @pytest.mark.parametrize("n,n_globs,w", [(1024, 4, 10), (1024, 1, 0), (1024, 64, 64), (1500, 100, 1499),
                                          (1024, 1024, 3), (8192, 16, 100), (3000, 200, 7)])
 def test_global_no_local(mods, dtype, d, n, n_globs, w):
