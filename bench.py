@@ -577,7 +577,7 @@ def main():
     ap.add_argument("--workload", default="csr_zipf", choices=sorted(WORKLOADS))
     ap.add_argument("--dtype", default="f32", choices=["f32", "f16", "bf16"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--d", type=int, default=64, choices=[32, 64, 128, 256],
+    ap.add_argument("--d", type=int, default=64, choices=[32, 64, 96, 128, 160, 192, 224, 256],
                     help="head dimension of the `local` workload (BASELINE config 2 has 64; the reference's own "
                          "check runs at 32)")
     ap.add_argument("--heads", type=int, default=1,
@@ -769,8 +769,9 @@ def main():
                      kernel_rows=w["params"]["n_globals"])
         else:
             kernel_flops, kernel_bytes = flops, w["bytes_total"]
-            kernel_name = "band_dma_kernel" if a.dtype != "f32" else \
-                "band_dma_f32_kernel" if d in (64, 128) else "tile_kernel"  # fp32 tiles straight to LDS: d = 64, 128
+            # tiles straight to LDS: half types at d = 32, 64, 128, 256, fp32 at d = 64, 128
+            kernel_name = ("band_dma_kernel" if d in (32, 64, 128, 256) else "tile_kernel") if a.dtype != "f32" else \
+                "band_dma_f32_kernel" if d in (64, 128) else "tile_kernel"
         hbm_ms = kernel_bytes / (HBM_PEAK_GBS * 1e9) * 1e3
         mfma_ms = kernel_flops / (mfma_peak * 1e12) * 1e3
         if hbm_ms >= mfma_ms:
