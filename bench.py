@@ -548,20 +548,23 @@ def measured_gather_ceiling(lib, w, torch, min_entries=8_000_000, reps=5):
                                       ctypes.c_void_p, ctypes.c_void_p]
     cursor = torch.zeros(64, dtype=torch.int32, device="cuda")
     stream = torch.cuda.current_stream().cuda_stream
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    # timed like the kernel it is compared with: the dispatch's own start and end stamps
+    ev = HipEvents()
     best, best_shape = float("inf"), None
     shapes = ((1, 16), (1, 32), (2, 16), (2, 32), (4, 32))
-    for wg, fl in shapes:
-        for _ in range(reps):
-            e0.record()
-            rc = lib.spfa_probe_gather(k.data_ptr(), v.data_ptr(), k.shape[0], row_bytes, idx.data_ptr(),
-                                       idx.numel(), 1024, wg, fl, cursor.data_ptr(), stream)
-            assert rc == 0, "spfa_probe_gather rc=%d" % rc
-            e1.record()
-            torch.cuda.synchronize()
-            ms = e0.elapsed_time(e1)
-            if ms < best:
-                best, best_shape = ms, (wg, fl)
+    try:
+        for wg, fl in shapes:
+            for _ in range(reps):
+                lib.spfa_set_kernel_events(ev.start, ev.stop)
+                rc = lib.spfa_probe_gather(k.data_ptr(), v.data_ptr(), k.shape[0], row_bytes, idx.data_ptr(),
+                                           idx.numel(), 1024, wg, fl, cursor.data_ptr(), stream)
+                assert rc == 0, "spfa_probe_gather rc=%d" % rc
+                torch.cuda.synchronize()
+                ms = ev.elapsed_ms()
+                if ms < best:
+                    best, best_shape = ms, (wg, fl)
+    finally:
+        lib.spfa_set_kernel_events(None, None)
     bytes_moved = idx.numel() * (2 * row_bytes + 4)
     return {"GBs": bytes_moved / (best * 1e-3) / 1e9,
             "how": "%d list entries x (2 rows of %d B + 4 B index) in %.3f ms; best of %d launches each of "

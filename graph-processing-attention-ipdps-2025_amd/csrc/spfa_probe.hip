@@ -11,6 +11,7 @@
 #include "spfa_hip.h"
 
 #include "spfa_common.hpp"
+#include "spfa_engine.hpp"
 
 namespace spfa {
 namespace {
@@ -127,23 +128,25 @@ int launch_probe(const void* k, const void* v, int64_t row_bytes, const uint32_t
     (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
   const dim3 grid((unsigned)(cus * wg_per_cu)), block(256);
   hipLaunchKernelGGL(probe_reset_kernel, dim3(1), dim3(64), 0, stream, cursor);
+  // the gather itself takes the caller's event pair, as the kernel it stands in for does
+  const KernelEvents ev = kernel_events();
   constexpr int UMAX = LPR;  // a batch of U rows per group covers at most one 64-entry chunk
   if constexpr (LPR <= 16) {
     if (in_flight >= 2 * UMAX) {
-      hipLaunchKernelGGL((gather_probe_deep_kernel<LPR>), grid, block, 0, stream, (const char*)k,
-                         (const char*)v, row_bytes, idx, n_idx, chunk, cursor);
+      launch_maybe_timed(ev, gather_probe_deep_kernel<LPR>, grid, block, stream, (const char*)k, (const char*)v,
+                         row_bytes, idx, n_idx, chunk, cursor);
       return hipGetLastError() == hipSuccess ? SPFA_OK : SPFA_ERR_LAUNCH;
     }
   }
   if (in_flight >= 16 && UMAX >= 16)
-    hipLaunchKernelGGL((gather_probe_kernel<LPR, (UMAX >= 16 ? 16 : UMAX)>), grid, block, 0, stream,
+    launch_maybe_timed(ev, gather_probe_kernel<LPR, (UMAX >= 16 ? 16 : UMAX)>, grid, block, stream,
                        (const char*)k, (const char*)v, row_bytes, idx, n_idx, chunk, cursor);
   else if (in_flight >= 8 && UMAX >= 8)
-    hipLaunchKernelGGL((gather_probe_kernel<LPR, (UMAX >= 8 ? 8 : UMAX)>), grid, block, 0, stream,
+    launch_maybe_timed(ev, gather_probe_kernel<LPR, (UMAX >= 8 ? 8 : UMAX)>, grid, block, stream,
                        (const char*)k, (const char*)v, row_bytes, idx, n_idx, chunk, cursor);
   else
-    hipLaunchKernelGGL((gather_probe_kernel<LPR, 4>), grid, block, 0, stream, (const char*)k,
-                       (const char*)v, row_bytes, idx, n_idx, chunk, cursor);
+    launch_maybe_timed(ev, gather_probe_kernel<LPR, 4>, grid, block, stream, (const char*)k, (const char*)v,
+                       row_bytes, idx, n_idx, chunk, cursor);
   return hipGetLastError() == hipSuccess ? SPFA_OK : SPFA_ERR_LAUNCH;
 }
 
