@@ -3,6 +3,8 @@
 //   - global-token list -> per-row flag bytes.
 #include "spfa_prep.hpp"
 
+#include <type_traits>
+
 #include "spfa_common.hpp"
 
 namespace spfa {
@@ -195,49 +197,70 @@ constexpr int kPartMaxBuckets = 2048;
 // The same pass over the row indices decides whether the entries need bucketing at all: it sets
 // *flag when they are not sorted by row or hold a row outside [0, n_rows) (so the sortedness check
 // costs no pass of its own; for sorted entries the histogram is simply not used).
-__global__ __launch_bounds__(kPartThreads) void coo_part_count_kernel(
-    const void* row_ind, int wide, int64_t nnz, int64_t n_rows, int lo_bits, int n_hi,
-    int64_t n_tiles, uint32_t* flag, uint32_t* hist) {
+// The kernels of pass 1 take the row type as a template argument: a run-time choice between a
+// 32-bit and a 64-bit load puts a branch, and with it a wait for the data, between every two
+// loads of a thread, and the sixteen loads of a thread become sixteen round trips.
+constexpr int kPartPerThread = kPartTile / kPartThreads;
+constexpr uint32_t kPartBadRow = 0xffffffffu;  // a row outside [0, n_rows)
+
+template <typename RowT>
+__global__ __launch_bounds__(kPartThreads, 8) void coo_part_count_kernel(
+    const RowT* row_ind, int64_t nnz, int64_t n_rows, int lo_bits, int n_hi, int64_t n_tiles,
+    uint32_t* flag, uint32_t* hist) {
   __shared__ uint32_t cnt[kPartMaxBuckets];
-  for (int b = threadIdx.x; b < n_hi; b += kPartThreads) cnt[b] = 0;
-  __syncthreads();
+  __shared__ uint32_t last_of[kPartPerThread][kPartThreads / kWave];
+  const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+  for (int b = tid; b < n_hi; b += kPartThreads) cnt[b] = 0;
   const int64_t beg = (int64_t)blockIdx.x * kPartTile;
-  const int64_t end = beg + kPartTile < nnz ? beg + kPartTile : nnz;
-  bool bad = false;
-  // (the tile's loads are issued together: one trip instead of sixteen dependent ones)
-  int64_t rows[kPartTile / kPartThreads], prev[kPartTile / kPartThreads];
+  const uint32_t n_tile = (uint32_t)(nnz - beg < kPartTile ? nnz - beg : kPartTile);  // (> 0)
+  const RowT* rp = row_ind + beg;
+  RowT raw[kPartPerThread];
 #pragma unroll
-  for (int i = 0; i < kPartTile / kPartThreads; i++) {
-    const int64_t e = beg + (int64_t)i * kPartThreads + threadIdx.x;
-    const int64_t ec = e < end ? e : end - 1;  // (end > beg: the grid has no empty tile)
-    rows[i] = load_index(row_ind, ec, wide);
-    prev[i] = load_index(row_ind, ec > 0 ? ec - 1 : 0, wide);
+  for (int i = 0; i < kPartPerThread; i++) {
+    const uint32_t idx = (uint32_t)(i * kPartThreads + tid);
+    raw[i] = rp[idx < n_tile ? idx : n_tile - 1];
   }
+  // the row of the entry before the tile (thread 0 compares its first entry with it)
+  uint32_t before = 0;
+  if (tid == 0 && beg > 0) {
+    const RowT pr = rp[-1];
+    before = pr < (RowT)n_rows ? (uint32_t)pr : kPartBadRow;
+  }
+  uint32_t row[kPartPerThread];
 #pragma unroll
-  for (int i = 0; i < kPartTile / kPartThreads; i++) {
-    const int64_t e = beg + (int64_t)i * kPartThreads + threadIdx.x;
-    if (e < end) {
-      const int64_t r = rows[i];
-      if (r >= 0 && r < n_rows) atomicAdd(&cnt[r >> lo_bits], 1u);
-      else bad = true;
-      if (e > 0 && prev[i] > r) bad = true;
+  for (int i = 0; i < kPartPerThread; i++) {
+    row[i] = raw[i] < (RowT)n_rows ? (uint32_t)raw[i] : kPartBadRow;
+    if (lane == kWave - 1) last_of[i][wave] = row[i];
+  }
+  __syncthreads();
+  // entry idx follows entry idx - 1: the lane before, the last lane of the wavefront before, or
+  // the last thread's previous entry
+  bool bad = false;
+#pragma unroll
+  for (int i = 0; i < kPartPerThread; i++) {
+    const uint32_t idx = (uint32_t)(i * kPartThreads + tid);
+    uint32_t prev = (uint32_t)__builtin_amdgcn_ds_bpermute(((lane - 1) & 63) << 2, (int)row[i]);
+    if (lane == 0) prev = wave > 0 ? last_of[i][wave - 1] : i > 0 ? last_of[i > 0 ? i - 1 : 0][kPartThreads / kWave - 1] : before;
+    if (idx < n_tile) {
+      if (row[i] == kPartBadRow) bad = true;
+      else atomicAdd(&cnt[row[i] >> lo_bits], 1u);
+      if (prev > row[i]) bad = true;  // (a bad row before this one has raised the flag already)
     }
   }
   if (bad) *flag = 1u;
   __syncthreads();
-  for (int b = threadIdx.x; b < n_hi; b += kPartThreads) hist[(int64_t)b * n_tiles + blockIdx.x] = cnt[b];
+  for (int b = tid; b < n_hi; b += kPartThreads) hist[(int64_t)b * n_tiles + blockIdx.x] = cnt[b];
 }
 
 // pass 1b: hist now holds exclusive prefixes.  The tile is first sorted by high digit inside LDS,
 // then written out, so that the entries a tile sends to one bucket leave as one contiguous run
 // of (row, col) pairs instead of as isolated 4-byte stores.
-constexpr int kPartPerThread = kPartTile / kPartThreads;
 constexpr size_t kPartScatterLds = (size_t)kPartTile * 8 + 3 * (size_t)kPartMaxBuckets * 4;
 
+template <typename RowT>
 __global__ __launch_bounds__(kPartThreads) void coo_part_scatter_kernel(
-    const void* row_ind, int wide, const uint32_t* col_ind, int64_t nnz, int64_t n_rows, int lo_bits,
-    int n_hi, int64_t n_tiles, const uint32_t* flag, const uint32_t* hist, uint64_t* tmp_pairs,
-    int col_bits, uint32_t col_max) {
+    const RowT* row_ind, const uint32_t* col_ind, int64_t nnz, int64_t n_rows, int lo_bits,
+    int n_hi, int64_t n_tiles, const uint32_t* flag, const uint32_t* hist, uint64_t* tmp_pairs) {
   extern __shared__ __attribute__((aligned(16))) unsigned char part_lds[];
   uint64_t* stage = reinterpret_cast<uint64_t*>(part_lds);
   uint32_t* cnt = reinterpret_cast<uint32_t*>(part_lds + (size_t)kPartTile * 8);
@@ -252,19 +275,24 @@ __global__ __launch_bounds__(kPartThreads) void coo_part_scatter_kernel(
   }
   __syncthreads();
   const int64_t beg = (int64_t)blockIdx.x * kPartTile;
-  const int64_t end = beg + kPartTile < nnz ? beg + kPartTile : nnz;
+  const uint32_t n_tile = (uint32_t)(nnz - beg < kPartTile ? nnz - beg : kPartTile);  // (> 0)
+  const RowT* rp = row_ind + beg;
+  const uint32_t* cp = col_ind + beg;
+  RowT raw[kPartPerThread];
   uint32_t rows[kPartPerThread], cols[kPartPerThread], rank[kPartPerThread];
 #pragma unroll
   for (int i = 0; i < kPartPerThread; i++) {
-    const int64_t e = beg + (int64_t)i * kPartThreads + tid;
-    rows[i] = 0xffffffffu;  // dropped
-    if (e < end) {
-      const int64_t r = load_index(row_ind, e, wide);
-      if (r >= 0 && r < n_rows) {
-        rows[i] = (uint32_t)r;
-        cols[i] = col_ind[e];
-        rank[i] = atomicAdd(&cnt[r >> lo_bits], 1u);
-      }
+    const uint32_t idx = (uint32_t)(i * kPartThreads + tid);
+    raw[i] = rp[idx < n_tile ? idx : n_tile - 1];
+    cols[i] = cp[idx < n_tile ? idx : n_tile - 1];
+  }
+#pragma unroll
+  for (int i = 0; i < kPartPerThread; i++) {
+    const uint32_t idx = (uint32_t)(i * kPartThreads + tid);
+    rows[i] = kPartBadRow;  // dropped
+    if (idx < n_tile && raw[i] < (RowT)n_rows) {
+      rows[i] = (uint32_t)raw[i];
+      rank[i] = atomicAdd(&cnt[rows[i] >> lo_bits], 1u);
     }
   }
   __syncthreads();
@@ -290,23 +318,10 @@ __global__ __launch_bounds__(kPartThreads) void coo_part_scatter_kernel(
   const uint32_t kept = carry;
 #pragma unroll
   for (int i = 0; i < kPartPerThread; i++) {
-    if (rows[i] != 0xffffffffu)
+    if (rows[i] != kPartBadRow)
       stage[lstart[rows[i] >> lo_bits] + rank[i]] = ((uint64_t)rows[i] << 32) | cols[i];
   }
   __syncthreads();
-  if (col_bits > 0) {
-    // (row inside the bucket, column) fit 32 bits: half the bytes to write here and to read in
-    // pass 2; a column past the last key (masked later whatever its value) becomes col_max
-    uint32_t* tmp_packed = reinterpret_cast<uint32_t*>(tmp_pairs);
-    const uint32_t lo_mask = (1u << lo_bits) - 1u;
-    for (uint32_t i = tid; i < kept; i += kPartThreads) {
-      const uint64_t x = stage[i];
-      const uint32_t row = (uint32_t)(x >> 32), col = (uint32_t)x;
-      const uint32_t b = row >> lo_bits;
-      tmp_packed[gstart[b] + (i - lstart[b])] = ((row & lo_mask) << col_bits) | (col < col_max ? col : col_max);
-    }
-    return;
-  }
   for (uint32_t i = tid; i < kept; i += kPartThreads) {
     const uint64_t x = stage[i];
     const uint32_t b = (uint32_t)(x >> 32) >> lo_bits;
@@ -314,70 +329,198 @@ __global__ __launch_bounds__(kPartThreads) void coo_part_scatter_kernel(
   }
 }
 
+// pass 1b when an entry leaves as one 32-bit word (row inside the bucket << col_bits | column;
+// a column past the last key, masked later whatever its value, becomes col_max): half the bytes to
+// write here and to read in pass 2, and a staged tile of 64 KB, so that two workgroups share a CU
+// and one loads while the other sorts.  Where the tile's entries of a bucket go inside the staged
+// tile follows from the scanned histogram alone (the tile's count of bucket b is the distance to
+// the next element of hist), so an entry is staged as soon as it is loaded and nothing is kept in
+// registers across a barrier.  The staged words no longer say which bucket they belong to, so
+// the tile leaves bucket by bucket: a group of 16 lanes copies the run of one bucket (16 entries
+// on average); runs of more than kPartLongRun entries are left to the whole workgroup.
+constexpr int kPartLongRun = 256;
+constexpr int kPartMaxLongRuns = kPartTile / kPartLongRun;
+
+inline size_t part_scatter_packed_lds(int64_t n_hi) { return (size_t)kPartTile * 4 + (size_t)n_hi * 4; }
+
+template <typename RowT>
+__global__ __launch_bounds__(kPartThreads, 8) void coo_part_scatter_packed_kernel(
+    const RowT* row_ind, const uint32_t* col_ind, int64_t nnz, int64_t n_rows, int lo_bits,
+    int n_hi, int64_t n_tiles, const uint32_t* flag, const uint32_t* hist, uint32_t* tmp_packed,
+    int col_bits, uint32_t col_max) {
+  extern __shared__ __attribute__((aligned(16))) uint32_t packed_lds[];
+  uint32_t* stage = packed_lds;              // kPartTile words
+  uint32_t* cursor = packed_lds + kPartTile;  // n_hi: next free staged position of each bucket
+  __shared__ uint32_t wave_sums[kPartThreads / kWave];
+  __shared__ uint32_t long_runs[kPartMaxLongRuns];
+  __shared__ uint32_t n_long;
+  if (!*flag) return;
+  const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+  if (tid == 0) n_long = 0;
+  const int64_t beg = (int64_t)blockIdx.x * kPartTile;
+  const uint32_t n_tile = (uint32_t)(nnz - beg < kPartTile ? nnz - beg : kPartTile);  // (> 0)
+  const RowT* rp = row_ind + beg;
+  const uint32_t* cp = col_ind + beg;
+  const uint32_t lo_mask = (1u << lo_bits) - 1u;
+  // (half of the thread's entries at a time: 64 registers)
+  constexpr int kHalf = kPartPerThread / 2;
+  RowT r[kHalf];
+  uint32_t c[kHalf];
+  auto load_half = [&](int h) {
+#pragma unroll
+    for (int i = 0; i < kHalf; i++) {
+      const uint32_t idx = (uint32_t)((h * kHalf + i) * kPartThreads + tid);
+      r[i] = rp[idx < n_tile ? idx : n_tile - 1];
+      c[i] = cp[idx < n_tile ? idx : n_tile - 1];
+    }
+  };
+  auto stage_half = [&](int h) {
+#pragma unroll
+    for (int i = 0; i < kHalf; i++) {
+      const uint32_t idx = (uint32_t)((h * kHalf + i) * kPartThreads + tid);
+      if (idx < n_tile && r[i] < (RowT)n_rows) {
+        const uint32_t row = (uint32_t)r[i];
+        stage[atomicAdd(&cursor[row >> lo_bits], 1u)] =
+            ((row & lo_mask) << col_bits) | (c[i] < col_max ? c[i] : col_max);
+      }
+    }
+  };
+  // cursor[b] = number of entries the tile holds of the buckets before b
+  uint32_t carry = 0;
+  for (int base = 0; base < n_hi; base += kPartThreads) {
+    const int i = base + tid;
+    uint32_t x = 0;
+    if (i < n_hi) {
+      const uint32_t* h = hist + (int64_t)i * n_tiles + blockIdx.x;
+      x = h[1] - h[0];
+    }
+    const uint32_t inc = wave_inclusive_scan(x, lane);
+    if (lane == kWave - 1) wave_sums[wave] = inc;
+    __syncthreads();
+    uint32_t prefix = 0, total = 0;
+#pragma unroll
+    for (int w = 0; w < kPartThreads / kWave; w++) {
+      const uint32_t sw = wave_sums[w];
+      if (w < wave) prefix += sw;
+      total += sw;
+    }
+    if (i < n_hi) {
+      cursor[i] = carry + prefix + inc - x;
+      if (x > (uint32_t)kPartLongRun) long_runs[atomicAdd(&n_long, 1u)] = (uint32_t)i;
+    }
+    carry += total;
+    __syncthreads();
+  }
+  load_half(0);
+  stage_half(0);
+  load_half(1);
+  stage_half(1);
+  __syncthreads();
+  // (cursor[b] is now the end of bucket b's run, and the start of the next bucket's)
+  // short runs: bucket b to the 16-lane group b % 64 of the workgroup
+  const int group = tid >> 4, sub = tid & 15;
+  for (int b = group; b < n_hi; b += kPartThreads / 16) {
+    const uint32_t s = b > 0 ? cursor[b - 1] : 0u, n = cursor[b] - s;
+    if (n == 0 || n > (uint32_t)kPartLongRun) continue;
+    uint32_t* out = tmp_packed + hist[(int64_t)b * n_tiles + blockIdx.x];
+    for (uint32_t j = sub; j < n; j += 16) out[j] = stage[s + j];
+  }
+  const uint32_t longs = n_long;
+  for (uint32_t q = 0; q < longs; q++) {
+    const int b = (int)long_runs[q];
+    const uint32_t s = b > 0 ? cursor[b - 1] : 0u, n = cursor[b] - s;
+    uint32_t* out = tmp_packed + hist[(int64_t)b * n_tiles + blockIdx.x];
+    for (uint32_t j = tid; j < n; j += kPartThreads) out[j] = stage[s + j];
+  }
+}
+
 // pass 2: one workgroup per high bucket; its (row, col) pairs are contiguous in tmp_pairs.
 // Count the low digit in LDS, scan, emit the row offsets of the bucket's rows and place the
 // columns.
 constexpr int kPartRowsThreads = 1024;
-constexpr int kPartKeep = 32;  // pairs per thread that pass 2 keeps in registers
+constexpr int kPartKeep = 64;        // entries per thread that pass 2 keeps in registers
+constexpr int kPartWindow = 36864;   // positions of a bucket's output staged in LDS at a time
+constexpr int kPartMaxWindows = 8;
+constexpr size_t kPartRowsLds = (size_t)kPartWindow * 4;
 
-// LDS counters under skew: a row that holds a large share of its bucket's entries (power-law
-// masks) has most lanes of every wavefront adding to the same counter, which the LDS serialises
-// lane by lane.  The lanes that share the key of the first lane not dealt with yet are counted
-// with a ballot and added once; after kAggRounds such rounds the remaining lanes add one by one.
+// LDS counters under skew: when one row holds most of its bucket's entries, most lanes of every
+// wavefront add to the same counter, which the LDS serialises lane by lane.  With ROUNDS > 0 the
+// lanes that share the key of the first lane not dealt with yet are counted with a ballot and
+// added once; after ROUNDS such rounds the remaining lanes add one by one.  The rounds cost about
+// forty dependent instructions per 64 entries, more than the serialised adds of a mask whose rows
+// hold up to a tenth of a bucket each (measured, 20 M entries in 1024 buckets: rows of 20 entries
+// 89 against 159 us with two rounds, rows of 20000 entries 142 against 191 us; a quarter of all
+// entries in one row 8.4 against 3.0 ms), so only a bucket that a sample shows to be dominated by
+// one row takes them.
 constexpr int kAggRounds = 2;
+constexpr int kAggSampleLanes = 16;  // lanes of a wavefront on one key that make a bucket "skewed"
 
-__device__ __forceinline__ int wave_lane() {
-  return (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+// number of set bits of `mask` below this lane
+__device__ __forceinline__ uint32_t bits_below_lane(uint64_t mask) {
+  return __builtin_amdgcn_mbcnt_hi((uint32_t)(mask >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0u));
 }
 
 // cnt[key] += 1 for every lane with valid set
+template <int ROUNDS>
 __device__ __forceinline__ void lds_count(uint32_t* cnt, uint32_t key, bool valid) {
-  const int lane = wave_lane();
-  uint64_t todo = __builtin_amdgcn_ballot_w64(valid);
+  bool pending = valid;
 #pragma unroll
-  for (int round = 0; round < kAggRounds; round++) {
+  for (int round = 0; round < ROUNDS; round++) {
+    const uint64_t todo = __builtin_amdgcn_ballot_w64(pending);
     if (todo == 0) break;
-    const int leader = __builtin_ctzll(todo);
-    const uint32_t k0 = (uint32_t)__builtin_amdgcn_readlane((int)key, leader);
-    const uint64_t same = __builtin_amdgcn_ballot_w64(valid && key == k0) & todo;
-    if (lane == leader) atomicAdd(&cnt[k0], (uint32_t)__builtin_popcountll(same));
-    todo &= ~same;
+    const uint32_t k0 = (uint32_t)__builtin_amdgcn_readlane((int)key, __builtin_ctzll(todo));
+    const bool hit = pending && key == k0;
+    const uint64_t same = __builtin_amdgcn_ballot_w64(hit);
+    // (the lowest lane of `same` is the leader)
+    if (hit && bits_below_lane(same) == 0) atomicAdd(&cnt[k0], (uint32_t)__builtin_popcountll(same));
+    pending = pending && !hit;
   }
-  if ((todo >> lane) & 1ull) atomicAdd(&cnt[key], 1u);
+  if (pending) atomicAdd(&cnt[key], 1u);
 }
 
 // the same, returning the counter's value before this lane's own increment (a distinct slot per
 // lane): pos = atomicAdd(&cnt[key], 1)
+template <int ROUNDS>
 __device__ __forceinline__ uint32_t lds_take_slot(uint32_t* cnt, uint32_t key, bool valid) {
-  const int lane = wave_lane();
-  uint64_t todo = __builtin_amdgcn_ballot_w64(valid);
+  bool pending = valid;
   uint32_t pos = 0;
 #pragma unroll
-  for (int round = 0; round < kAggRounds; round++) {
+  for (int round = 0; round < ROUNDS; round++) {
+    const uint64_t todo = __builtin_amdgcn_ballot_w64(pending);
     if (todo == 0) break;
     const int leader = __builtin_ctzll(todo);
     const uint32_t k0 = (uint32_t)__builtin_amdgcn_readlane((int)key, leader);
-    const uint64_t same = __builtin_amdgcn_ballot_w64(valid && key == k0) & todo;
+    const bool hit = pending && key == k0;
+    const uint64_t same = __builtin_amdgcn_ballot_w64(hit);
+    const uint32_t below = bits_below_lane(same);
     uint32_t base = 0;
-    if (lane == leader) base = atomicAdd(&cnt[k0], (uint32_t)__builtin_popcountll(same));
+    if (hit && below == 0) base = atomicAdd(&cnt[k0], (uint32_t)__builtin_popcountll(same));
     base = (uint32_t)__builtin_amdgcn_readlane((int)base, leader);
-    if ((same >> lane) & 1ull) pos = base + (uint32_t)__builtin_popcountll(same & ((1ull << lane) - 1ull));
-    todo &= ~same;
+    if (hit) pos = base + below;
+    pending = pending && !hit;
   }
-  if ((todo >> lane) & 1ull) pos = atomicAdd(&cnt[key], 1u);
+  if (pending) pos = atomicAdd(&cnt[key], 1u);
   return pos;
 }
 
-// PACKED: the entries are 32-bit (row inside the bucket << col_bits | column).  A bucket of up to
-// kPartKeep * kPartRowsThreads entries is then read once, all loads in flight together, and stays
-// in registers between the count and the placement (32 registers; two workgroups share a CU).
-// Larger buckets, and 64-bit (row, column) pairs, are walked twice, four loads in flight.
+// PACKED: the entries are 32-bit (row inside the bucket << col_bits | column).  The first
+// kPartKeep * kPartRowsThreads of them are read once, all loads in flight together, and stay in
+// registers from the count to the placement; what a larger bucket holds beyond them is walked
+// again from memory.  The columns do not leave as isolated 4-byte stores (one memory request
+// each: 50 M of them take longer than everything else in this kernel): the bucket's output is
+// cut into windows of kPartWindow positions, a window takes the rows that start inside it, their
+// columns are placed in LDS and leave as contiguous runs.  The tail of a row that runs past its
+// window's end is stored directly.  Buckets of more than kPartMaxWindows windows, and 64-bit
+// (row, column) pairs, are walked twice with direct stores.
+// (One workgroup per CU: the staged window and 64 entries per thread in 128 registers.)
 template <bool PACKED>
-__global__ __launch_bounds__(kPartRowsThreads, PACKED ? 8 : 4) void coo_part_rows_kernel(
+__global__ __launch_bounds__(kPartRowsThreads, 4) void coo_part_rows_kernel(
     int64_t n_rows, int lo_bits, int n_hi, int64_t n_tiles, int64_t n_hist, const uint32_t* flag,
     const uint32_t* hist, const uint64_t* tmp_pairs, uint32_t* row_off, uint32_t* cols_out, int col_bits) {
+  extern __shared__ __attribute__((aligned(16))) uint32_t rows_stage[];  // PACKED: kPartWindow words
   __shared__ uint32_t cnt[kPartMaxBuckets];
   __shared__ uint32_t wave_sums[kPartRowsThreads / kWave];
+  __shared__ uint32_t win_row[kPartMaxWindows + 1], win_pos[kPartMaxWindows + 1];
   if (!*flag) return;
   const int b = blockIdx.x;
   const int n_lo = 1 << lo_bits;
@@ -425,67 +568,157 @@ __global__ __launch_bounds__(kPartRowsThreads, PACKED ? 8 : 4) void coo_part_row
     }
     if (b == n_hi - 1 && threadIdx.x == 0) row_off[n_rows] = end;
   };
+  constexpr uint32_t kStep = 4 * kPartRowsThreads;
   if constexpr (PACKED) {
-    if (end - beg <= (uint32_t)(kPartKeep * kPartRowsThreads)) {
-      if (end == beg) {
-        scan_counts();  // (an empty bucket still owes its rows their offsets)
-        return;
-      }
-      // (every load reads a valid entry: past the end, the bucket's last one, which is not counted)
+    const uint32_t size = end - beg;
+    if (size == 0) {
+      scan_counts();  // (an empty bucket still owes its rows their offsets)
+      return;
+    }
+    constexpr uint32_t kKept = (uint32_t)kPartKeep * kPartRowsThreads;
+    constexpr uint32_t kWin = (uint32_t)kPartWindow;
+    if (size <= kWin * (uint32_t)kPartMaxWindows) {
+      const uint32_t n_win = (size + kWin - 1) / kWin;
+      const uint32_t kept = size < kKept ? size : kKept;
+      // This thread keeps the entries threadIdx.x + i * kPartRowsThreads, i < n_mine.  (The loads
+      // are not clamped to the bucket, so that they need no register per address: the buffer is
+      // padded by what a bucket's loads can run past its end; what they read there is not used.)
       uint32_t x[kPartKeep];
       const uint32_t* bp = tmp_packed + beg;
-      const uint32_t last = end - beg - 1;
+      const uint32_t n_mine = threadIdx.x < kept ? (kept - threadIdx.x + kPartRowsThreads - 1) / kPartRowsThreads : 0u;
+#pragma unroll
+      for (int i = 0; i < kPartKeep; i++) x[i] = bp[i * kPartRowsThreads + threadIdx.x];
 #pragma unroll
       for (int i = 0; i < kPartKeep; i++) {
-        const uint32_t e = i * kPartRowsThreads + threadIdx.x;
-        x[i] = bp[e < last ? e : last];
-      }
-      // (a few entries at a time: with all of them unrolled into one stretch the slots that come
-      // back from LDS pile up in registers beside the entries)
-#pragma unroll
-      for (int i = 0; i < kPartKeep; i++) {
-        lds_count(cnt, x[i] >> col_bits, beg + i * kPartRowsThreads + threadIdx.x < end);
+        lds_count<0>(cnt, x[i] >> col_bits, (uint32_t)i < n_mine);
         if (i % 4 == 3) __builtin_amdgcn_sched_barrier(0);
+      }
+      for (uint32_t e0 = kKept; e0 < size; e0 += kStep) {
+        uint32_t y[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+          const uint32_t e = e0 + i * kPartRowsThreads + threadIdx.x;
+          y[i] = bp[e < size ? e : size - 1];
+        }
+#pragma unroll
+        for (int i = 0; i < 4; i++) lds_count<0>(cnt, y[i] >> col_bits, e0 + i * kPartRowsThreads + threadIdx.x < size);
       }
       __syncthreads();
       scan_counts();
+      // window k takes the rows [win_row[k], win_row[k + 1]): those whose first position lies in
+      // [k * kWin, (k + 1) * kWin); win_pos[k] is the first position of row win_row[k]
+      for (int i = threadIdx.x; i < n_lo; i += kPartRowsThreads) {
+        const uint32_t start = cnt[i] - beg;
+        uint32_t wi = start / kWin;
+        if (wi > n_win) wi = n_win;
+        uint32_t k = i > 0 ? (cnt[i - 1] - beg) / kWin + 1 : 0u;
+        for (; k <= wi; k++) {
+          win_row[k] = (uint32_t)i;
+          win_pos[k] = start;
+        }
+        if (i == n_lo - 1)
+          for (k = wi + 1; k <= n_win; k++) {
+            win_row[k] = (uint32_t)n_lo;
+            win_pos[k] = size;
+          }
+      }
+      __syncthreads();
+      uint32_t* outp = cols_out + beg;
+      for (uint32_t k = 0; k < n_win; k++) {
+        const uint32_t first = win_row[k], n_in = win_row[k + 1] - first;
+        if (n_in == 0) continue;  // (the same for every thread)
+        const uint32_t lo = k * kWin;
+        // (the entries and their number are made opaque in every trip, or the compiler keeps the
+        // 64 row numbers and the 64 validity masks of the trip-invariant part in registers)
+        uint32_t n_mine_k = n_mine;
+        asm volatile("" : "+v"(n_mine_k));
 #pragma unroll
-      for (int i = 0; i < kPartKeep; i++) {
-        const bool valid = beg + i * kPartRowsThreads + threadIdx.x < end;
-        const uint32_t pos = lds_take_slot(cnt, x[i] >> col_bits, valid);
-        if (valid) cols_out[pos] = x[i] & col_mask;
-        if (i % 4 == 3) __builtin_amdgcn_sched_barrier(0);
+        for (int i = 0; i < kPartKeep; i++) {
+          uint32_t xi = x[i];
+          asm volatile("" : "+v"(xi));
+          const uint32_t r = xi >> col_bits;
+          const bool in = (uint32_t)i < n_mine_k && r - first < n_in;
+          const uint32_t pos = lds_take_slot<0>(cnt, r, in) - beg;
+          if (in) {
+            if (pos - lo < kWin) rows_stage[pos - lo] = xi & col_mask;
+            else outp[pos] = xi & col_mask;
+          }
+          if (i % 4 == 3) __builtin_amdgcn_sched_barrier(0);
+        }
+        for (uint32_t e0 = kKept; e0 < size; e0 += kStep) {
+          uint32_t y[4];
+#pragma unroll
+          for (int i = 0; i < 4; i++) {
+            const uint32_t e = e0 + i * kPartRowsThreads + threadIdx.x;
+            y[i] = bp[e < size ? e : size - 1];
+          }
+#pragma unroll
+          for (int i = 0; i < 4; i++) {
+            const uint32_t r = y[i] >> col_bits;
+            const bool in = e0 + i * kPartRowsThreads + threadIdx.x < size && r - first < n_in;
+            const uint32_t pos = lds_take_slot<0>(cnt, r, in) - beg;
+            if (in) {
+              if (pos - lo < kWin) rows_stage[pos - lo] = y[i] & col_mask;
+              else outp[pos] = y[i] & col_mask;
+            }
+          }
+        }
+        __syncthreads();
+        const uint32_t stop = win_pos[k + 1] < lo + kWin ? win_pos[k + 1] : lo + kWin;
+        for (uint32_t p = win_pos[k] + threadIdx.x; p < stop; p += kPartRowsThreads) outp[p] = rows_stage[p - lo];
+        __syncthreads();
       }
       return;
     }
   }
-  constexpr uint32_t kStep = 4 * kPartRowsThreads;
-  for (uint32_t e0 = beg; e0 < end; e0 += kStep) {
-    uint64_t x[4];
+  // the bucket's first entries as a sample: is one row on a quarter of a wavefront's lanes?
+  bool heavy = false;
+  {
+    const uint32_t e = beg + threadIdx.x;
+    const bool valid = e < end;
+    const uint32_t key = valid ? key_of(load_entry(e)) : 0u;
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
-      const uint32_t e = e0 + i * kPartRowsThreads + threadIdx.x;
-      x[i] = e < end ? load_entry(e) : 0ull;
+    for (int j = 0; j < 4; j++) {
+      const uint32_t k0 = (uint32_t)__builtin_amdgcn_readlane((int)key, 16 * j);
+      heavy |= __builtin_popcountll(__builtin_amdgcn_ballot_w64(valid && key == k0)) >= kAggSampleLanes;
     }
-#pragma unroll
-    for (int i = 0; i < 4; i++) lds_count(cnt, key_of(x[i]), e0 + i * kPartRowsThreads + threadIdx.x < end);
   }
+  const bool skewed = __syncthreads_or(heavy) != 0;
+  auto count_all = [&](auto rounds) {
+    for (uint32_t e0 = beg; e0 < end; e0 += kStep) {
+      uint64_t x[4];
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        const uint32_t e = e0 + i * kPartRowsThreads + threadIdx.x;
+        x[i] = e < end ? load_entry(e) : 0ull;
+      }
+#pragma unroll
+      for (int i = 0; i < 4; i++)
+        lds_count<decltype(rounds)::value>(cnt, key_of(x[i]), e0 + i * kPartRowsThreads + threadIdx.x < end);
+    }
+  };
+  auto place_all = [&](auto rounds) {
+    for (uint32_t e0 = beg; e0 < end; e0 += kStep) {
+      uint64_t x[4];
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        const uint32_t e = e0 + i * kPartRowsThreads + threadIdx.x;
+        x[i] = e < end ? load_entry(e) : 0ull;
+      }
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        const bool valid = e0 + i * kPartRowsThreads + threadIdx.x < end;
+        const uint32_t pos = lds_take_slot<decltype(rounds)::value>(cnt, key_of(x[i]), valid);
+        if (valid) cols_out[pos] = (uint32_t)x[i] & col_mask;
+      }
+    }
+  };
+  if (skewed) count_all(std::integral_constant<int, kAggRounds>{});
+  else count_all(std::integral_constant<int, 0>{});
   __syncthreads();
   scan_counts();
-  for (uint32_t e0 = beg; e0 < end; e0 += kStep) {
-    uint64_t x[4];
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-      const uint32_t e = e0 + i * kPartRowsThreads + threadIdx.x;
-      x[i] = e < end ? load_entry(e) : 0ull;
-    }
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-      const bool valid = e0 + i * kPartRowsThreads + threadIdx.x < end;
-      const uint32_t pos = lds_take_slot(cnt, key_of(x[i]), valid);
-      if (valid) cols_out[pos] = (uint32_t)x[i] & col_mask;
-    }
-  }
+  if (skewed) place_all(std::integral_constant<int, kAggRounds>{});
+  else place_all(std::integral_constant<int, 0>{});
 }
 
 // one wavefront per row: lanes stride over the row's entries
@@ -547,7 +780,10 @@ CooWorkspace coo_workspace(int64_t n_rows, int64_t nnz) {
   w.off_cursor = off;  off = align_up(off + (size_t)(n_rows + 1) * 4, 256);
   w.off_tiles = off;   off = align_up(off + (size_t)n_tiles * 4, 256);
   w.off_hist = off;    off = align_up(off + (size_t)(n_hist + 1) * 4, 256);
-  w.off_tmp_pairs = off; off = align_up(off + (size_t)(w.partition ? nnz : 0) * 8, 256);
+  // (pass 2 reads kPartKeep * kPartRowsThreads packed entries from a bucket's start whatever the
+  // bucket's size: the padding keeps the last buckets' loads inside the buffer)
+  w.off_tmp_pairs = off;
+  off = align_up(off + (w.partition ? (size_t)nnz * 8 + (size_t)kPartKeep * kPartRowsThreads * 4 : 0), 256);
   w.total = off;
   return w;
 }
@@ -570,10 +806,16 @@ int coo_to_csr(const void* row_ind, int row_wide, const uint32_t* col_ind, int64
   hipLaunchKernelGGL(fill_u32_kernel, dim3(1), dim3(64), 0, stream, flag, (int64_t)1, 0u);
   // sorted or not: decided on the device (by the first pass of the partition where there is one)
   const bool part = nnz > 0 && w.partition;
-  if (part)
-    hipLaunchKernelGGL(coo_part_count_kernel, dim3((unsigned)w.n_tiles1), dim3(kPartThreads), 0, stream,
-                       row_ind, row_wide, nnz, n_rows, w.lo_bits, (int)w.n_hi, w.n_tiles1, flag,
-                       (uint32_t*)(base + w.off_hist));
+  if (part) {
+    if (row_wide)
+      hipLaunchKernelGGL(coo_part_count_kernel<uint64_t>, dim3((unsigned)w.n_tiles1), dim3(kPartThreads), 0,
+                         stream, (const uint64_t*)row_ind, nnz, n_rows, w.lo_bits, (int)w.n_hi, w.n_tiles1,
+                         flag, (uint32_t*)(base + w.off_hist));
+    else
+      hipLaunchKernelGGL(coo_part_count_kernel<uint32_t>, dim3((unsigned)w.n_tiles1), dim3(kPartThreads), 0,
+                         stream, (const uint32_t*)row_ind, nnz, n_rows, w.lo_bits, (int)w.n_hi, w.n_tiles1,
+                         flag, (uint32_t*)(base + w.off_hist));
+  }
   else if (nnz > 0)
     hipLaunchKernelGGL(coo_check_sorted_kernel, dim3(grid_for(nnz, 256, 8192)), dim3(256), 0, stream,
                        row_ind, row_wide, nnz, n_rows, flag);
@@ -584,17 +826,24 @@ int coo_to_csr(const void* row_ind, int row_wide, const uint32_t* col_ind, int64
   if (part) {
     uint32_t* hist = (uint32_t*)(base + w.off_hist);
     uint64_t* tmp_pairs = (uint64_t*)(base + w.off_tmp_pairs);
-    // 152 KB of LDS per workgroup: above the 64 KB a kernel gets without asking (set once per
-    // device: the attribute belongs to the device's copy of the kernel)
+    // 152 KB of LDS per workgroup in both passes: above the 64 KB a kernel gets without asking
+    // (set once per device: the attribute belongs to the device's copy of the kernel)
     constexpr int kMaxDevices = 64;
     static bool lds_attr_set[kMaxDevices];
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess) return 4;
     if (dev < 0 || dev >= kMaxDevices || !lds_attr_set[dev]) {
-      if (hipFuncSetAttribute(reinterpret_cast<const void*>(coo_part_scatter_kernel),
-                              hipFuncAttributeMaxDynamicSharedMemorySize,
-                              (int)kPartScatterLds) != hipSuccess)
-        return 4;
+      const int packed_max = (int)part_scatter_packed_lds(kPartMaxBuckets);
+      const struct { const void* kernel; int bytes; } big_lds[] = {
+          {reinterpret_cast<const void*>(coo_part_scatter_kernel<uint64_t>), (int)kPartScatterLds},
+          {reinterpret_cast<const void*>(coo_part_scatter_kernel<uint32_t>), (int)kPartScatterLds},
+          {reinterpret_cast<const void*>(coo_part_scatter_packed_kernel<uint64_t>), packed_max},
+          {reinterpret_cast<const void*>(coo_part_scatter_packed_kernel<uint32_t>), packed_max},
+          {reinterpret_cast<const void*>(coo_part_rows_kernel<true>), (int)kPartRowsLds},
+      };
+      for (const auto& k : big_lds)
+        if (hipFuncSetAttribute(k.kernel, hipFuncAttributeMaxDynamicSharedMemorySize, k.bytes) != hipSuccess)
+          return 4;
       if (dev >= 0 && dev < kMaxDevices) lds_attr_set[dev] = true;
     }
     const int64_t n_hist = w.n_hi * w.n_tiles1;
@@ -612,11 +861,28 @@ int coo_to_csr(const void* row_ind, int row_wide, const uint32_t* col_ind, int64
       while (need < 32 && ((int64_t)1 << need) <= n_cols) need++;  // n_cols itself must fit
       if (need + w.lo_bits <= 32) col_bits = need;
     }
-    hipLaunchKernelGGL(coo_part_scatter_kernel, dim3((unsigned)w.n_tiles1), dim3(kPartThreads),
-                       kPartScatterLds, stream, row_ind, row_wide, col_ind, nnz, n_rows, w.lo_bits,
-                       (int)w.n_hi, w.n_tiles1, flag, hist, tmp_pairs, col_bits, (uint32_t)(col_bits ? n_cols : 0));
+    const dim3 grid1((unsigned)w.n_tiles1), block1(kPartThreads);
+    const size_t packed_lds = part_scatter_packed_lds(w.n_hi);
+    uint32_t* tmp_packed = (uint32_t*)tmp_pairs;
+    const uint32_t col_max = (uint32_t)n_cols;
+    if (col_bits && row_wide)
+      hipLaunchKernelGGL(coo_part_scatter_packed_kernel<uint64_t>, grid1, block1, packed_lds, stream,
+                         (const uint64_t*)row_ind, col_ind, nnz, n_rows, w.lo_bits, (int)w.n_hi, w.n_tiles1,
+                         flag, hist, tmp_packed, col_bits, col_max);
+    else if (col_bits)
+      hipLaunchKernelGGL(coo_part_scatter_packed_kernel<uint32_t>, grid1, block1, packed_lds, stream,
+                         (const uint32_t*)row_ind, col_ind, nnz, n_rows, w.lo_bits, (int)w.n_hi, w.n_tiles1,
+                         flag, hist, tmp_packed, col_bits, col_max);
+    else if (row_wide)
+      hipLaunchKernelGGL(coo_part_scatter_kernel<uint64_t>, grid1, block1, kPartScatterLds, stream,
+                         (const uint64_t*)row_ind, col_ind, nnz, n_rows, w.lo_bits, (int)w.n_hi, w.n_tiles1,
+                         flag, hist, tmp_pairs);
+    else
+      hipLaunchKernelGGL(coo_part_scatter_kernel<uint32_t>, grid1, block1, kPartScatterLds, stream,
+                         (const uint32_t*)row_ind, col_ind, nnz, n_rows, w.lo_bits, (int)w.n_hi, w.n_tiles1,
+                         flag, hist, tmp_pairs);
     if (col_bits)
-      hipLaunchKernelGGL(coo_part_rows_kernel<true>, dim3((unsigned)w.n_hi), dim3(kPartRowsThreads), 0, stream,
+      hipLaunchKernelGGL(coo_part_rows_kernel<true>, dim3((unsigned)w.n_hi), dim3(kPartRowsThreads), kPartRowsLds, stream,
                          n_rows, w.lo_bits, (int)w.n_hi, w.n_tiles1, n_hist, flag, hist, tmp_pairs, row_off,
                          cols, col_bits);
     else
