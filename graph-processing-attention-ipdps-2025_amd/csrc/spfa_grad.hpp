@@ -47,6 +47,17 @@ struct GradArgs {
 };
 
 constexpr int kGradWaves = 4;        // owners per workgroup
+
+// Candidates in flight per lane group in grad_rows_kernel.  One wavefront per owner row makes the
+// kernel live on the number of rows in flight, not on the loads in flight per row: with 2 instead
+// of 8 (57 / 78 registers instead of 108 / 131 in the query / key pass at fp32 d = 64, 8 / 6
+// wavefronts per SIMD instead of 4 / 3) the two passes of the Zipf masks take 1.48 ms instead of
+// 1.66 (131 K rows, 12.8 M positions) and 9.7 ms instead of 10.9 (1 M rows, 50 M positions);
+// 16 in flight: 1.95 and 11.2 ms; forcing 8 wavefronts per SIMD on 4 in flight spills: 3.3 ms.
+template <class Lay>
+constexpr int grad_rows_unroll() {
+  return Lay::U_SHORT >= 2 ? Lay::U_SHORT / 2 : 1;
+}
 constexpr int kGradItemBlocks = 2048;
 
 template <class Lay>
@@ -281,7 +292,7 @@ __global__ __launch_bounds__(kGradWaves* kWave) void grad_rows_kernel(GradArgs g
     acc2[e] = 0.f;
   }
   const float scale = 1.0f / sqrtf((float)g.d);
-  grad_walk<Lay, Mask, KEYS, Lay::U_MEDIUM>(mask, rc, o.X, o.Y, o.lse_c, o.delta_c, o.lse_o, o.delta_o,
+  grad_walk<Lay, Mask, KEYS, grad_rows_unroll<Lay>()>(mask, rc, o.X, o.Y, o.lse_c, o.delta_c, o.lse_o, o.delta_o,
                                             g.d, scale, o.a, o.b, 0, deg < seg ? deg : seg, lane,
                                             acc1, acc2);
   if (lane < Lay::LPR) {  // this wavefront is the only one that touches the row in this launch
