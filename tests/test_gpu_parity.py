@@ -774,6 +774,55 @@ def test_coo_power_law_with_many_empty_rows(mods):
     check(o, m, l, *ref, torch.float32)
 
 
+@pytest.mark.parametrize("case,n,n_k,nnz,d,dtype", [
+    ("two_windows", 2048, 2048, 3_000_000, 64, torch.float32),       # 64 buckets of ~47 K entries
+    ("beyond_registers", 2048, 2048, 8_000_000, 64, torch.float32),  # ~125 K entries per bucket
+    ("direct", 256, 256, 6_000_000, 64, torch.float32),              # 16 buckets of ~375 K entries
+    ("one_heavy_row", 2048, 2048, 3_000_000, 64, torch.float32),     # 60 % of the entries in one row
+    # 1465 buckets of 2048 rows; row in bucket and column do not fit 32 bits together
+    ("many_buckets_pairs", 3_000_000, 3_000_000, 2_000_000, 32, torch.bfloat16),
+    # 1465 buckets of 1024 rows, 32-bit entries between the passes
+    ("many_buckets_packed", 1_500_000, 65536, 2_000_000, 32, torch.bfloat16),
+])
+def test_coo_unsorted_bucket_shapes(mods, case, n, n_k, nnz, d, dtype):
+    """Unsorted entries whose row buckets have the sizes that the bucketing pre-pass treats
+    differently (one or several staged windows, entries beyond those kept in registers, buckets too
+    large to stage, a bucket dominated by one row, the largest number of buckets), a number of
+    entries that is no multiple of a tile, repeated entries: the attention result against the
+    same mask sorted by torch and given as CSR, and to_csr against that sort entry by entry."""
+    g = torch.Generator(device=DEV)
+    g.manual_seed(61)
+    nnz += 12345
+    r = torch.randint(0, n, (nnz,), generator=g, device=DEV, dtype=torch.int64)
+    c = torch.randint(0, n_k, (nnz,), generator=g, device=DEV, dtype=torch.int64)
+    if case == "one_heavy_row":
+        r[torch.rand(nnz, generator=g, device=DEV) < 0.6] = 5
+    q, k, v = dev_qkv(n, d, dtype, 61, n_k=n_k)
+    r_t, c_t = r.to(torch.uint64), c.to(torch.uint32)
+    val = torch.ones(nnz, device=DEV, dtype=dtype)
+    m, l, o = state(n, d, dtype, torch.float32)
+    mods["spfa_coo"].forward(q, k, v, r_t, c_t, val, m, l, o, False)
+    sync()
+    order = torch.argsort(r, stable=True)
+    deg = torch.bincount(r, minlength=n)
+    ro = torch.zeros(n + 1, dtype=torch.int64, device=DEV)
+    ro[1:] = torch.cumsum(deg, 0)
+    m2, l2, o2 = state(n, d, dtype, torch.float32)
+    mods["spfa_csr"].forward(q, k, v, ro.to(torch.uint64), c[order].to(torch.uint32).contiguous(), val, m2, l2, o2,
+                             False)
+    sync()
+    assert torch.equal(m, m2)
+    assert torch.allclose(l, l2, rtol=1e-4, atol=0)
+    # (the order of a row's columns differs, and with it the rounding: one unit of a bf16 output)
+    atol, rtol = (2e-5, 1e-3) if dtype == torch.float32 else (2e-3, 8e-3)
+    assert torch.allclose(o.float(), o2.float(), atol=atol, rtol=rtol)
+    ro3, ci3 = mods["spfa_coo"].to_csr(r_t, c_t, n)
+    sync()
+    assert torch.equal(ro3.to(torch.int64), ro)
+    rows3 = torch.repeat_interleave(torch.arange(n, device=DEV), deg)
+    assert torch.equal(torch.sort(rows3 * n_k + ci3.to(torch.int64))[0], torch.sort(r * n_k + c)[0])
+
+
 def test_coo_empty_mask(mods):
     n, d = 64, 64
     q, k, v = dev_qkv(n, d, torch.float32, 18)
