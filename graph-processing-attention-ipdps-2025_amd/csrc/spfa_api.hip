@@ -865,10 +865,10 @@ int check_grads(const spfa_problem_t* p, const spfa_grads_t* g) {
 
 Grads make_grads(const spfa_grads_t* g) { return Grads{g->d_out, g->d_q, g->d_k, g->d_v}; }
 
-// Workspace of a gradient call: lse and delta of every query row, the two lists of (owner,
+// Workspace of a gradient call: lse and delta of every query row (apart and side by side), the two lists of (owner,
 // segment) items of long rows, then whatever the mask needs (`mask_bytes`).
 struct GradLayout {
-  size_t off_lse, off_delta, off_cnt, off_items, off_mask, total;
+  size_t off_lse, off_delta, off_stat, off_cnt, off_items, off_mask, total;
   uint32_t cap_items;
   bool ok;
 };
@@ -883,6 +883,7 @@ GradLayout grad_layout(int64_t n_q, int64_t n_batch, int64_t items_bound, size_t
   size_t off = 0;
   g.off_lse = off;   off = align_up(off + (size_t)(n_q * b) * 4, 256);
   g.off_delta = off; off = align_up(off + (size_t)(n_q * b) * 4, 256);
+  g.off_stat = off;  off = align_up(off + (size_t)(n_q * b) * 8, 256);
   g.off_cnt = off;   off += 256;
   g.off_items = off; off = align_up(off + (size_t)g.cap_items * 16, 256);  // two lists of pairs
   g.off_mask = off;  off = align_up(off + mask_bytes, 256);
@@ -922,6 +923,7 @@ GradArgs make_grad_args(const spfa_problem_t* p, const spfa_grads_t* g, const Gr
   a.d_out = g->d_out;
   a.lse = (float*)(base + lay.off_lse);
   a.delta = (float*)(base + lay.off_delta);
+  a.stat = (float2*)(base + lay.off_stat);
   a.d_q = (float*)g->d_q;
   a.d_k = (float*)g->d_k;
   a.d_v = (float*)g->d_v;

@@ -33,6 +33,9 @@ struct GradArgs {
   const void* d_out;  // [n_batch, n_q, d]
   float* lse;         // [n_batch * n_q]  m + log l, +inf for rows that never saw a live column
   float* delta;       // [n_batch * n_q]  dO . O (0 for those rows)
+  float2* stat;       // [n_batch * n_q]  (lse, delta) side by side, for the gather engine's key pass:
+                      // a candidate's two numbers then cost one cache line, not two (measured, 50 M
+                      // candidates of 1 M rows: as many line fills went to the two arrays as to Q)
   float* d_q;         // fp32 gradients, added to
   float* d_k;
   float* d_v;
@@ -94,8 +97,11 @@ __global__ __launch_bounds__(256) void grad_prologue_kernel(Tensors t, GradArgs 
   }
   acc = group_sum<16>(acc);
   if (c == 0) {
-    g.lse[row] = live ? m + __logf(l) : __builtin_inff();
-    g.delta[row] = live ? acc : 0.f;
+    const float lse = live ? m + __logf(l) : __builtin_inff();
+    const float delta = live ? acc : 0.f;
+    g.lse[row] = lse;
+    g.delta[row] = delta;
+    g.stat[row] = make_float2(lse, delta);
   }
 }
 
@@ -106,14 +112,13 @@ static __global__ void grad_reset_kernel(uint32_t* n_items) {
 // Candidates t_begin .. t_end of one owner, walked by the whole wavefront.
 //   KEYS == false: owner is a query row, (a, b) = (q_i, dO_i), X = K, Y = V, and lse_o / delta_o
 //                  are the owner's; acc1 collects dQ_i.
-//   KEYS == true:  owner is a key row, (a, b) = (k_j, v_j), X = Q, Y = dO, lse / delta are read
+//   KEYS == true:  owner is a key row, (a, b) = (k_j, v_j), X = Q, Y = dO, (lse, delta) are read
 //                  per candidate; acc1 collects dK_j, acc2 dV_j.
 template <class Lay, class Mask, bool KEYS, int U_>
 __device__ __forceinline__ void grad_walk(const Mask& mask, const typename Mask::Row& rc,
                                           const typename Lay::elem* __restrict__ X,
                                           const typename Lay::elem* __restrict__ Y,
-                                          const float* __restrict__ lse_c,
-                                          const float* __restrict__ delta_c, float lse_o,
+                                          const float2* __restrict__ stat_c, float lse_o,
                                           float delta_o, int d, float scale,
                                           const float (&a)[Lay::NE], const float (&b)[Lay::NE],
                                           int64_t t_begin, int64_t t_end, int lane,
@@ -161,8 +166,13 @@ __device__ __forceinline__ void grad_walk(const Mask& mask, const typename Mask:
           xr[u] = Lay::load_gather(X + (int64_t)cols[u] * d, c, d);
           yr[u] = Lay::load_gather(Y + (int64_t)cols[u] * d, c, d);
           if constexpr (KEYS) {
-            ls[u] = lse_c[cols[u]];
-            dl[u] = delta_c[cols[u]];
+            // (two 4-byte loads of the one line: as one 8-byte load the key pass of 131 K rows
+            // took 533 us instead of 440)
+            const float* sp = reinterpret_cast<const float*>(stat_c + cols[u]);
+            ls[u] = sp[0];
+            const float* sp1 = sp + 1;
+            asm volatile("" : "+v"(sp1));
+            dl[u] = *sp1;
           }
         }
       }
@@ -212,8 +222,7 @@ struct GradOwner {
   using T = typename Lay::elem;
   const T* X;
   const T* Y;
-  const float* lse_c;
-  const float* delta_c;
+  const float2* stat_c;
   float lse_o, delta_o;
   float a[Lay::NE], b[Lay::NE];
   float* out1;
@@ -235,8 +244,7 @@ struct GradOwner {
       brow = (const T*)g.v + r * d;
       X = (const T*)g.q + bb * g.n_q * d;
       Y = (const T*)g.d_out + bb * g.n_q * d;
-      lse_c = g.lse + bb * g.n_q;
-      delta_c = g.delta + bb * g.n_q;
+      stat_c = g.stat + bb * g.n_q;
       lse_o = 0.f;
       delta_o = 0.f;
       out1 = g.d_k + r * d;
@@ -246,8 +254,7 @@ struct GradOwner {
       brow = (const T*)g.d_out + r * d;
       X = (const T*)g.k + bb * g.n_k * d;
       Y = (const T*)g.v + bb * g.n_k * d;
-      lse_c = nullptr;
-      delta_c = nullptr;
+      stat_c = nullptr;
       lse_o = g.lse[r];
       delta_o = g.delta[r];
       out1 = g.d_q + r * d;
@@ -292,7 +299,7 @@ __global__ __launch_bounds__(kGradWaves* kWave) void grad_rows_kernel(GradArgs g
     acc2[e] = 0.f;
   }
   const float scale = 1.0f / sqrtf((float)g.d);
-  grad_walk<Lay, Mask, KEYS, grad_rows_unroll<Lay>()>(mask, rc, o.X, o.Y, o.lse_c, o.delta_c, o.lse_o, o.delta_o,
+  grad_walk<Lay, Mask, KEYS, grad_rows_unroll<Lay>()>(mask, rc, o.X, o.Y, o.stat_c, o.lse_o, o.delta_o,
                                             g.d, scale, o.a, o.b, 0, deg < seg ? deg : seg, lane,
                                             acc1, acc2);
   if (lane < Lay::LPR) {  // this wavefront is the only one that touches the row in this launch
@@ -335,7 +342,7 @@ __global__ __launch_bounds__(kGradWaves* kWave) void grad_items_kernel(GradArgs 
       acc1[e] = 0.f;
       acc2[e] = 0.f;
     }
-    grad_walk<Lay, Mask, KEYS, Lay::U_MEDIUM>(mask, rc, o.X, o.Y, o.lse_c, o.delta_c, o.lse_o,
+    grad_walk<Lay, Mask, KEYS, Lay::U_MEDIUM>(mask, rc, o.X, o.Y, o.stat_c, o.lse_o,
                                               o.delta_o, g.d, scale, o.a, o.b, t0, t1, lane, acc1,
                                               acc2);
     if (lane < Lay::LPR) {
