@@ -61,7 +61,8 @@ struct Counters {
   uint32_t next_item;
   uint32_t overflow;
   uint32_t n_medium;
-  uint32_t pad[2];
+  uint32_t n_short;
+  uint32_t pad[1];
 };
 
 struct Item {
@@ -85,6 +86,7 @@ struct Plan {
   Item* items;
   MultiRow* multi;
   int32_t* medium;   // rows with short_max < deg <= medium_max: one wavefront each, no queue
+  int32_t* shorts;   // rows with 0 < deg <= short_max (null: no list was made)
   float* pm;
   float* pl;
   float* pacc;
@@ -119,6 +121,7 @@ static __global__ void reset_counters_kernel(Counters* cnt) {
     cnt->next_item = 0;
     cnt->overflow = 0;
     cnt->n_medium = 0;
+    cnt->n_short = 0;
   }
 }
 
@@ -303,8 +306,8 @@ constexpr int kPlanThreads = 1024;
 template <class Mask>
 __global__ __launch_bounds__(kPlanThreads) void plan_kernel(int64_t n_q, Mask mask, Plan plan) {
   constexpr int NW = kPlanThreads / kWave;
-  __shared__ uint32_t wave_tot[NW][4];
-  __shared__ uint32_t block_base[4];
+  __shared__ uint32_t wave_tot[NW][5];
+  __shared__ uint32_t block_base[5];
   __shared__ uint32_t block_ok;
   const int lane = lane_id();
   const int wave = threadIdx.x / kWave;
@@ -323,21 +326,24 @@ __global__ __launch_bounds__(kPlanThreads) void plan_kernel(int64_t n_q, Mask ma
   const uint32_t multi = nseg > 1 ? 1u : 0u;
   const uint32_t npart = multi ? nseg : 0u;
   const uint32_t med = is_medium ? 1u : 0u;
+  const uint32_t sht = (deg > 0 && deg <= plan.short_max) ? 1u : 0u;
   const uint32_t inc_items = wave_inclusive_sum(nseg, lane);
   const uint32_t inc_part = wave_inclusive_sum(npart, lane);
   const uint32_t inc_multi = wave_inclusive_sum(multi, lane);
   const uint32_t inc_med = wave_inclusive_sum(med, lane);
+  const uint32_t inc_sht = wave_inclusive_sum(sht, lane);
   if (lane == kWave - 1) {
     wave_tot[wave][0] = inc_items;
     wave_tot[wave][1] = inc_part;
     wave_tot[wave][2] = inc_multi;
     wave_tot[wave][3] = inc_med;
+    wave_tot[wave][4] = inc_sht;
   }
   __syncthreads();
   if (threadIdx.x == 0) {
-    uint32_t tot[4] = {0u, 0u, 0u, 0u};
+    uint32_t tot[5] = {0u, 0u, 0u, 0u, 0u};
     for (int w = 0; w < NW; w++)
-      for (int k = 0; k < 4; k++) {
+      for (int k = 0; k < 5; k++) {
         const uint32_t x = wave_tot[w][k];
         wave_tot[w][k] = tot[k];  // exclusive prefix over the wavefronts
         tot[k] += x;
@@ -362,9 +368,11 @@ __global__ __launch_bounds__(kPlanThreads) void plan_kernel(int64_t n_q, Mask ma
         if (plan.status != nullptr) atomicOr(plan.status, kStatusWorkListOverflow);
       }
     }
+    if (tot[4]) block_base[4] = atomicAdd(&plan.cnt->n_short, tot[4]);  // (as many slots as rows)
     block_ok = ok;
   }
   __syncthreads();
+  if (sht) plan.shorts[block_base[4] + wave_tot[wave][4] + inc_sht - 1] = (int32_t)row;
   if (!block_ok) return;
   if (is_medium) plan.medium[block_base[3] + wave_tot[wave][3] + inc_med - 1] = (int32_t)row;
   if (!is_long) return;
@@ -397,10 +405,22 @@ __global__ __launch_bounds__(256) void rows_kernel(Tensors t, Mask mask, Plan pl
   const int wave = threadIdx.x >> 6;
   const int g = lane / LPR;
   const int c = lane % LPR;
-  const int64_t row = ((int64_t)blockIdx.x * 4 + wave) * Lay::GROUPS + g;  // among all problems
-  if (row >= t.n_q * t.n_batch) return;
-  int64_t b, ri;
-  split_row(t, row, b, ri);
+  const int64_t idx = ((int64_t)blockIdx.x * 4 + wave) * Lay::GROUPS + g;
+  // A mask whose rows are mostly empty (and stay untouched) would spend a lane group on every
+  // empty row and a wavefront on every four rows that hold one short row among them: the rows are
+  // then taken from the list of non-empty short rows that plan_kernel made.
+  int64_t row, b, ri;  // row among all problems, problem, row inside the problem
+  const uint32_t n_short = plan.shorts != nullptr ? plan.cnt->n_short : 0u;
+  if (plan.shorts != nullptr && !plan.use_nan && !plan.cnt->overflow && (int64_t)n_short * 2 <= t.n_q) {
+    if (idx >= (int64_t)n_short * t.n_batch) return;
+    b = idx / n_short;
+    ri = plan.shorts[idx - b * n_short];
+    row = b * t.n_q + ri;
+  } else {
+    row = idx;
+    if (row >= t.n_q * t.n_batch) return;
+    split_row(t, row, b, ri);
+  }
 
   const typename Mask::Row rc = mask.row(ri);
   const int64_t deg = rc.deg;
@@ -713,8 +733,8 @@ struct EngineSizing {
 };
 
 struct WorkspaceLayout {
-  size_t off_cnt, off_items, off_multi, off_medium, off_pm, off_pl, off_pacc, total;
-  uint32_t cap_items, cap_partials, cap_multi, cap_medium;
+  size_t off_cnt, off_items, off_multi, off_medium, off_short, off_pm, off_pl, off_pacc, total;
+  uint32_t cap_items, cap_partials, cap_multi, cap_medium, cap_short;
 };
 
 
@@ -727,8 +747,9 @@ inline int64_t pow2_ceil(int64_t x) {
 inline WorkspaceLayout engine_workspace(const EngineSizing& s, int64_t n_q, int64_t d,
                                         int64_t n_batch = 1) {
   WorkspaceLayout w{};
-  int64_t cap_items = 0, cap_partials = 0, cap_multi = 0, cap_medium = 0;
+  int64_t cap_items = 0, cap_partials = 0, cap_multi = 0, cap_medium = 0, cap_short = 0;
   if (s.max_deg > s.short_max) {
+    cap_short = n_q;
     int64_t n_long = s.nnz_bound / (s.short_max + 1);
     if (n_long > n_q) n_long = n_q;
     if (n_long > s.n_long_bound) n_long = s.n_long_bound;
@@ -743,11 +764,13 @@ inline WorkspaceLayout engine_workspace(const EngineSizing& s, int64_t n_q, int6
   w.cap_partials = (uint32_t)cap_partials;
   w.cap_multi = (uint32_t)cap_multi;
   w.cap_medium = (uint32_t)cap_medium;
+  w.cap_short = (uint32_t)cap_short;
   size_t off = 0;
   w.off_cnt = off;      off = align_up(off + sizeof(Counters), 256);
   w.off_items = off;    off = align_up(off + (size_t)cap_items * sizeof(Item), 256);
   w.off_multi = off;    off = align_up(off + (size_t)cap_multi * sizeof(MultiRow), 256);
   w.off_medium = off;   off = align_up(off + (size_t)cap_medium * sizeof(int32_t), 256);
+  w.off_short = off;    off = align_up(off + (size_t)cap_short * sizeof(int32_t), 256);
   // (the work list is shared by the problems of a batch, the partial results are not)
   const size_t nb = (size_t)(n_batch > 1 ? n_batch : 1);
   w.off_pm = off;       off = align_up(off + nb * (size_t)cap_partials * sizeof(float), 256);
@@ -818,6 +841,7 @@ int launch_engine(const Tensors& t, const Mask& mask, const EngineSizing& s, int
   plan.items = (Item*)(pbase + w.off_items);
   plan.multi = (MultiRow*)(pbase + w.off_multi);
   plan.medium = (int32_t*)(pbase + w.off_medium);
+  plan.shorts = w.cap_short > 0 ? (int32_t*)(pbase + w.off_short) : nullptr;
   plan.cursor = &((Counters*)(base + w.off_cnt))->next_item;
   plan.pm = (float*)(base + w.off_pm);
   plan.pl = (float*)(base + w.off_pl);
