@@ -945,7 +945,7 @@ int transpose_mask(const CsrMask& rows, int64_t n_q, int64_t n_k, int64_t nnz, c
   const TransposeLayout tl = transpose_layout(n_k, nnz);
   uint32_t* e_rows = (uint32_t*)(mbase + tl.off_rows);
   uint32_t* e_cols = (uint32_t*)(mbase + tl.off_cols);
-  int rc = csr_entry_list(rows.row_off, rows.off64, rows.cols, rows.alt_cols, rows.use_alt, n_q, e_rows,
+  int rc = csr_entry_list(rows.row_off, rows.off64, rows.cols, rows.alt_cols, rows.use_alt, n_q, nnz, e_rows,
                           e_cols, stream);
   if (rc) return rc;
   const CooWorkspace cw = coo_workspace(n_k, nnz);

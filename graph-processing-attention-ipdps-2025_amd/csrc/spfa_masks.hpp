@@ -41,6 +41,7 @@ struct CsrMask {
     const uint32_t* cp = cols;
     if (use_alt != nullptr && *use_alt != 0u) cp = alt_cols;
     if (b > nnz) b = nnz;
+    if (a < 0) a = 0;  // (an offset of 2^63 or more)
     if (a > b) a = b;
     return Row{a, b - a, cp};
   }

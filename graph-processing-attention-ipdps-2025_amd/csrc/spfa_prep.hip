@@ -743,22 +743,69 @@ __global__ __launch_bounds__(kPartRowsThreads, 4) void coo_part_rows_kernel(
   else place_all(std::integral_constant<int, 0>{});
 }
 
-// one wavefront per row: lanes stride over the row's entries
+// (row, column) of every entry of a CSR mask.  A wavefront takes `rpw` (16 or 64) consecutive
+// rows, one pair of offsets per lane; the rows' entries are one contiguous range, which the
+// wavefront walks 64 entries at a time, every lane finding the row of its entry by a binary search
+// among the wavefront's row ends (six cross-lane reads).  (A wavefront per row spends most of
+// its time on the empty rows of a mask that has many: 360 us for 50 M entries in 1 M rows.)
+// Row ranges are held to [0, nnz) as in CsrMask::row; entries before the first row's range or
+// after the last row's belong to no row and get a column that the bucketing drops.  Offsets that
+// are not in ascending order give entries of the wrong row or none, never a store outside
+// [0, nnz).
 __global__ __launch_bounds__(256) void csr_entry_list_kernel(const void* row_off, int off64,
-                                                             const uint32_t* cols,
-                                                             const uint32_t* alt_cols,
+                                                             const uint32_t* __restrict__ cols,
+                                                             const uint32_t* __restrict__ alt_cols,
                                                              const uint32_t* use_alt, int64_t n_rows,
-                                                             uint32_t* rows_out, uint32_t* cols_out) {
+                                                             int64_t nnz, int rpw,
+                                                             uint32_t* __restrict__ rows_out,
+                                                             uint32_t* __restrict__ cols_out) {
   const int lane = threadIdx.x & (kWave - 1);
-  const int64_t stride = (int64_t)gridDim.x * 4;
-  const uint32_t* cp = (use_alt != nullptr && *use_alt != 0u) ? alt_cols : cols;
-  for (int64_t r = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6); r < n_rows; r += stride) {
-    const int64_t a = load_index(row_off, r, off64), b = load_index(row_off, r + 1, off64);
-    for (int64_t e = a + lane; e < b; e += kWave) {
-      rows_out[e] = (uint32_t)r;
-      cols_out[e] = cp[e];
+  const uint32_t* __restrict__ cp = (use_alt != nullptr && *use_alt != 0u) ? alt_cols : cols;
+  const int64_t r0 = ((int64_t)blockIdx.x * 4 + (threadIdx.x >> 6)) * rpw;
+  if (r0 >= n_rows) return;
+  const int n_here = n_rows - r0 < rpw ? (int)(n_rows - r0) : rpw;
+  // lane l < n_here: the range of row r0 + l; the other lanes: an empty range at the end
+  const int64_t r = r0 + (lane < n_here ? lane : n_here - 1);
+  int64_t a = load_index(row_off, r, off64);
+  int64_t b = load_index(row_off, r + 1, off64);
+  if (b > nnz) b = nnz;
+  if (a < 0) a = 0;
+  if (a > b) a = b;
+  if (lane >= n_here) a = b;
+  // (nnz < 2^32: the offsets of the bucketed mask are 32 bits wide)
+  const uint32_t end32 = (uint32_t)b;
+  const uint32_t first = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)a, 0);
+  const uint32_t last = (uint32_t)__builtin_amdgcn_readlane((int)end32, kWave - 1);
+  // (eight loads in flight per lane: one load per trip makes a row of 4096 entries a chain of 64
+  // memory round trips, which was the whole of the kernel's time on a power-law mask)
+  constexpr int kInFlight = 8;
+  for (uint32_t e0 = first; e0 < last; e0 += kInFlight * kWave) {
+    uint32_t col[kInFlight];
+#pragma unroll
+    for (int u = 0; u < kInFlight; u++) {
+      const uint32_t e = e0 + u * kWave + lane;
+      col[u] = e < last ? cp[e] : 0u;
+    }
+#pragma unroll
+    for (int u = 0; u < kInFlight; u++) {
+      const uint32_t e = e0 + u * kWave + lane;
+      // number of rows of this wavefront that end at or before e
+      int lo = 0;
+#pragma unroll
+      for (int step = kWave / 2; step >= 1; step >>= 1) {
+        const uint32_t end_v = (uint32_t)__builtin_amdgcn_ds_bpermute((lo + step - 1) << 2, (int)end32);
+        if (end_v <= e) lo += step;
+      }
+      if (e < last) {
+        rows_out[e] = (uint32_t)(r0 + lo);
+        cols_out[e] = col[u];
+      }
     }
   }
+  if (r0 == 0)
+    for (uint32_t e = lane; e < first; e += kWave) cols_out[e] = 0xffffffffu;
+  if (r0 + rpw >= n_rows)
+    for (int64_t e = (int64_t)last + lane; e < nnz; e += kWave) cols_out[e] = 0xffffffffu;
 }
 
 __global__ void coo_csr_export_kernel(const uint32_t* row_off, const uint32_t* bucketed,
@@ -930,11 +977,13 @@ int coo_to_csr(const void* row_ind, int row_wide, const uint32_t* col_ind, int64
 }
 
 int csr_entry_list(const void* row_off, int off64, const uint32_t* cols, const uint32_t* alt_cols,
-                   const uint32_t* use_alt, int64_t n_rows, uint32_t* rows_out, uint32_t* cols_out,
-                   hipStream_t stream) {
+                   const uint32_t* use_alt, int64_t n_rows, int64_t nnz, uint32_t* rows_out,
+                   uint32_t* cols_out, hipStream_t stream) {
   if (n_rows <= 0) return 0;
-  hipLaunchKernelGGL(csr_entry_list_kernel, dim3(grid_for(n_rows, 4, 1 << 20)), dim3(256), 0, stream,
-                     row_off, off64, cols, alt_cols, use_alt, n_rows, rows_out, cols_out);
+  // (64 rows per wavefront when that still leaves a few wavefronts for every SIMD)
+  const int rpw = n_rows >= ((int64_t)1 << 19) ? kWave : 16;
+  hipLaunchKernelGGL(csr_entry_list_kernel, dim3((unsigned)((n_rows + 4 * rpw - 1) / (4 * rpw))), dim3(256), 0,
+                     stream, row_off, off64, cols, alt_cols, use_alt, n_rows, nnz, rpw, rows_out, cols_out);
   return hipGetLastError() == hipSuccess ? 0 : 4;
 }
 

@@ -48,8 +48,8 @@ int coo_to_csr(const void* row_ind, int row_wide, const uint32_t* col_ind, int64
 // from alt_cols when *use_alt != 0, as CsrMask reads them).  Feeding (cols, rows) back into
 // coo_to_csr gives the transposed mask.
 int csr_entry_list(const void* row_off, int off64, const uint32_t* cols, const uint32_t* alt_cols,
-                   const uint32_t* use_alt, int64_t n_rows, uint32_t* rows_out, uint32_t* cols_out,
-                   hipStream_t stream);
+                   const uint32_t* use_alt, int64_t n_rows, int64_t nnz, uint32_t* rows_out,
+                   uint32_t* cols_out, hipStream_t stream);
 
 // A CooCsr result as two plain arrays: row_off_out[0..n_rows] and cols_out[0..nnz) (the bucketed
 // columns, or `given_cols` unchanged when the entries came sorted).
