@@ -158,3 +158,26 @@ def test_coo_rows_by_the_atomic_path_beyond_four_million_rows(mods):
     got = torch.sort(got_rows * (1 << 20) + ci)[0]
     want = torch.sort(rows * (1 << 20) + cols)[0]
     assert torch.equal(got, want)
+
+
+@pytest.mark.parametrize("n,nnz", [(3000, 40_000), (40_000, 900_000)])
+def test_coo_entries_outside_the_mask_are_dropped(mods, n, nnz):
+    """Unsorted COO entries whose row is not a query row (at or beyond n, or a 64-bit pattern far
+    beyond) are dropped by the row-bucketing pre-pass, entries whose column is not a key are
+    masked: the result is that of the entries left."""
+    d, n_k = 64, n - 100
+    q, k, v = _qkv(n, d, 12, n_k=n_k)
+    rng = np.random.default_rng(12)
+    rows = rng.integers(0, n, nnz).astype(np.uint64)
+    cols = rng.integers(0, n_k + n_k // 5, nnz).astype(np.int64)  # one in six past the keys
+    bad = rng.random(nnz) < 0.1
+    rows[bad] = rng.choice(np.array([n, n + 7, 2 ** 31, 2 ** 40 + 3, 2 ** 63 + 5, 2 ** 64 - 1], dtype=np.uint64),
+                           int(bad.sum()))
+    m, l, o = _state(n, d)
+    r_t = torch.as_tensor(rows.view(np.int64)).view(torch.uint64).to(DEV)
+    c_t = torch.as_tensor(cols).to(torch.uint32).to(DEV)
+    mods["spfa_coo"].forward(q, k, v, r_t, c_t, torch.ones(nnz, device=DEV), m, l, o, False)
+    torch.cuda.synchronize()
+    keep = ~bad & (cols < n_k)
+    ref = c_oracle.coo(np64(q), np64(k), np64(v), rows[keep].astype(np.int64), cols[keep])
+    check(o, m, l, *ref, torch.float32)
