@@ -59,6 +59,7 @@ struct GradTileCfg {
 template <typename T, int D, bool KEYS>
 constexpr int grad_tile_min_blocks() {
   if (D <= 64 && sizeof(T) == 2 && !KEYS) return 3;
+  if (D > 128) return 1;
   return (D > 64 && (KEYS || sizeof(T) == 4)) ? 1 : 2;
 }
 
@@ -820,7 +821,7 @@ int launch_band_grad(const TileArgs& a, const GradArgs& g, hipStream_t stream) {
   hipLaunchKernelGGL((grad_prologue_kernel<T>), dim3((unsigned)((rows + 15) / 16)), dim3(256), 0, stream,
                      a.t, g);
   const int64_t grid = (a.n_tiles * a.t.n_batch + 7) / 8 * 8;
-  if constexpr (sizeof(T) == 2) {
+  if constexpr (sizeof(T) == 2 && (D == 64 || D == 128)) {
     // the direct-to-LDS kernels address a tile's rows with 32-bit offsets, and tile numbers,
     // windows and positions with 32-bit arithmetic (the forward kernel's conditions)
     const int64_t max_len = a.block > 0 ? a.cnt : (a.n + a.s - 1) / a.s;
@@ -908,6 +909,13 @@ int run_band_grad_tiles(const TileArgs& a, const GradArgs& g, hipStream_t stream
   if (((uintptr_t)g.d_out | (uintptr_t)g.d_q | (uintptr_t)g.d_k | (uintptr_t)g.d_v) & 15) return -1;
   if (a.t.d == 64) return launch_band_grad<T, 64>(a, g, stream);
   if (a.t.d == 128) return launch_band_grad<T, 128>(a, g, stream);
+  if (a.t.d == 32) return launch_band_grad<T, 32>(a, g, stream);
+  if (a.t.d == 96) return launch_band_grad<T, 96>(a, g, stream);
+  // (fp32 beyond d = 128: the key pass no longer fits 512 registers)
+  if constexpr (sizeof(T) == 2) {
+    if (a.t.d == 160) return launch_band_grad<T, 160>(a, g, stream);
+    if (a.t.d == 192) return launch_band_grad<T, 192>(a, g, stream);
+  }
   return -1;
 }
 
