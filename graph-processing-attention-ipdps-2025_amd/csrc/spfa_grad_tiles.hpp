@@ -925,6 +925,8 @@ int run_global_grad_tiles(const TileArgs& a, const GradArgs& g, hipStream_t stre
   if (((uintptr_t)g.d_out | (uintptr_t)g.d_q | (uintptr_t)g.d_k | (uintptr_t)g.d_v) & 15) return -1;
   if (a.t.d == 64) return launch_global_grad<T, 64>(a, g, stream);
   if (a.t.d == 128) return launch_global_grad<T, 128>(a, g, stream);
+  if (a.t.d == 32) return launch_global_grad<T, 32>(a, g, stream);
+  if (a.t.d == 96) return launch_global_grad<T, 96>(a, g, stream);
   return -1;
 }
 

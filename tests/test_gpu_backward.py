@@ -102,8 +102,8 @@ def test_implicit_masks_match_the_oracle(mods, dtype):
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("d", [64, 128, 32, 96, 160, 192])
 def test_band_masks_on_the_tile_path(mods, dtype, d):
-    """Band and block masks at d = 32 / 64 / 96 / 128 (half types also 160 / 192), the global mask at
-    d = 64 / 128, with rows of 32 and more live positions go to the dense-tile gradient kernels:
+    """Band, block and global masks at d = 32 / 64 / 96 / 128 (band and block masks of the half types
+    also at 160 / 192) with rows of 32 and more live positions go to the dense-tile gradient kernels:
     windows below, at and above a tile, sequence ends inside a tile, dilation (several
     subsequences of unequal length), blocks with and without dilation, a stacked batch."""
     cases = [
