@@ -428,6 +428,37 @@ def test_coo_batch_rectangular_keys(mods):
                  torch.float32)
 
 
+@pytest.mark.parametrize("use_nan", [False, True])
+@pytest.mark.parametrize("shape", [(), (3,)])
+def test_csr_mostly_empty_rows(mods, shape, use_nan):
+    """Seven rows in ten empty, the others short (1 - 25 columns) with a few medium and long ones:
+    the short rows are then taken from a list instead of row by row (when empty rows are left
+    untouched), one problem and a batch sharing the mask, plain and planned calls."""
+    n, d = 40_000, 64
+    g = torch.Generator().manual_seed(53)
+    deg = torch.randint(1, 26, (n,), generator=g)
+    deg[torch.rand(n, generator=g) < 0.7] = 0
+    deg[torch.randperm(n, generator=g)[:60]] = 150
+    deg[torch.randperm(n, generator=g)[:5]] = 3000
+    ro, ci = syn.csr_from_degrees(deg, n, g, "cpu", force_diagonal=False)
+    ro_t, ci_t = csr_tensors(ro, ci)
+    q, k, v, m, l, o = _stacked(n, d, torch.float32, shape, 53)
+    val = torch.ones(ci_t.numel(), device=DEV)
+    mods["spfa_csr"].forward(q, k, v, ro_t, ci_t, val, m, l, o, use_nan)
+    sync()
+    ref_fn = lambda a, b, c: c_oracle.csr(a, b, c, ro.numpy(), ci.numpy(), use_nan=use_nan)
+    if shape:
+        _check_heads(q, k, v, o, m, l, ref_fn, torch.float32, dead_expect="nan" if use_nan else "zero")
+    else:
+        check(o, m, l, *ref_fn(np64(q), np64(k), np64(v)), torch.float32, dead_expect="nan" if use_nan else "zero")
+    plan = mods["spfa_csr"].plan(ro_t, ci_t)
+    m2, l2, o2 = torch.full_like(m, -float("inf")), torch.zeros_like(l), torch.zeros_like(o)
+    mods["spfa_csr"].forward_planned(q, k, v, ro_t, ci_t, val, m2, l2, o2, use_nan, plan)
+    sync()
+    assert torch.allclose(torch.nan_to_num(o), torch.nan_to_num(o2), atol=2e-6)
+    assert torch.equal(m, m2) and torch.allclose(l, l2, rtol=1e-5)
+
+
 @pytest.mark.parametrize("dtype,d", [(torch.float32, 64), (torch.bfloat16, 64), (torch.float32, 40)])
 def test_implicit_masks_batch_of_heads(mods, dtype, d):
     """d = 64 runs the dense-tile kernels, d = 40 the row-gather engine."""
