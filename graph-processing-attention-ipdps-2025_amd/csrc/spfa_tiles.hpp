@@ -863,6 +863,19 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void band_dma_kernel(TileArgs
   if (t0 >= qlen) return;
   const int u_lo = t0 > wlim ? t0 - wlim : 0;
   const int u_hi = (qlen - qspan - wlim > t0) ? t0 + qspan + wlim : qlen;
+  // Key tiles are visited in a rotated order: the workgroups of neighbouring query tiles (the
+  // same XCD has them, at the same time) walk ranges that overlap in all but BM / BN tiles, and
+  // started at their own first tile they would ask for any one tile BM / BN steps apart, after
+  // the L2 has seen a whole round of other tiles.  Visit number `it` is therefore the tile whose
+  // number, counted along the subsequence, is it modulo the tile count, so that all of them ask
+  // for the same tile at about the same time.  (The online softmax does not care about order.)
+  const int nk = (u_hi - u_lo + BN - 1) / BN;
+  const int rot0 = uni((nk - (int)(((uint32_t)tile * (uint32_t)(BM / BN)) % (uint32_t)nk)) % nk);
+  auto tile_start = [&](int it) __attribute__((always_inline)) {
+    int j = rot0 + it;
+    j = j >= nk ? j - nk : j;
+    return u_lo + j * BN;
+  };
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -926,7 +939,7 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void band_dma_kernel(TileArgs
   // the first NBUF - 1 tiles are on their way before anything else is loaded
 #pragma unroll
   for (int i = 0; i < NBUF - 1; i++)
-    if (u_lo + i * BN < u_hi) request(u_lo + i * BN, i);
+    if (i < nk) request(tile_start(i), i);
 
   const int tw0 = t0 + (quad ? 0 : 32 * wave);  // first query of this wavefront
   const int tq = tw0 + r;                       // this lane's query position
@@ -974,9 +987,26 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void band_dma_kernel(TileArgs
 #pragma unroll
     for (int v = 0; v < 16; v++) o[eb][v] = 0.f;
   constexpr float kSlack = 8.f;
-  float m = kNegInf;   // reference maximum of the exponentials, log2 units
-  float mt = kNegInf;  // true running maximum
-  float l = 0.f;       // running sum (relative to m) over this lane's half of the keys
+  float m = kNegInf;        // reference maximum of the exponentials, log2 units
+  float neg_m = 0.f;        // -m (0 while m is -inf), the addend of the exponent
+  float thr_raw = kNegInf;  // (m + kSlack) / sc: a raw score above it moves the reference
+  float mt_raw = kNegInf;   // true running maximum of this lane's raw scores (its half of the keys)
+  // Row sums of P: one more result block of the second product whose A operand is all ones, so
+  // every row of it is the sum over all keys (both halves of the wavefront) of the ROUNDED
+  // weights, the ones the numerator is built from; only lsum[0] is ever read.  (Not at d = 256,
+  // where the registers are all taken: there the sum is a chain of additions, l_add, over this
+  // lane's half of the keys.)
+#ifndef SPFA_BAND_MFMA_SUM
+#define SPFA_BAND_MFMA_SUM(D) ((D) <= 64)
+#endif
+  constexpr bool kMfmaSum = SPFA_BAND_MFMA_SUM(D);
+  float l_add = 0.f;
+  f32x16 lsum;
+#pragma unroll
+  for (int v = 0; v < 16; v++) lsum[v] = 0.f;
+  const uint32_t one2 = sizeof(T) == 2 && __is_same(T, bf16) ? 0x3f803f80u : 0x3c003c00u;
+  const uint4v ones = {one2, one2, one2, one2};
+  const float inv_sc = sqrtf((float)D) * 0.6931471805599453f;
 
   typedef short s16x4 __attribute__((ext_vector_type(4)));
   typedef short s16x8 __attribute__((ext_vector_type(8)));
@@ -988,38 +1018,51 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void band_dma_kernel(TileArgs
   // exponentials in s.  The exponentials are taken against a reference maximum m that is only
   // moved (and the accumulators rescaled) when a row's maximum has grown by more than kSlack
   // (log2 units) since the reference was set: the weights then stay below 2^kSlack, the final
-  // division by l cancels the reference, and the rescale is rare instead of happening on every
-  // block while the maxima are still settling.  mt keeps the true maximum for the row
-  // statistics.  The row sum is a plain chain of additions: the dot-product instructions
-  // (v_dot2c_f32_bf16 with a vector of ones, half the instruction count) keep the matrix
-  // instructions of the SIMD's other wavefront from overlapping with this one's vector work
-  // (measured with a probe: a matrix wavefront beside a vector wavefront takes the sum of their
-  // times as soon as the vector stream holds such instructions, 0.65 of it without).
-  auto soft_core = [&](f32x16& s) __attribute__((always_inline)) {
-    float mx = s[0];
+  // division by the row sum cancels the reference, and the rescale is rare instead of happening
+  // on every block while the maxima are still settling.  The common path is 8 three-input
+  // maxima, one compare, and a multiply-add + exponential per score: the running maximum stays
+  // per lane and in raw units (the two lanes of a query only meet when the reference moves, and
+  // once at the end for the row statistics), and the row sum comes out of the matrix pipe.
+  auto soft_max = [&](const f32x16& s) __attribute__((always_inline)) {
+    float mx = mt_raw;
 #pragma unroll
-    for (int v = 1; v < 16; v++) mx = fmaxf(mx, s[v]);
-    mx = fmaxf(mx, shfl_xor_f32(mx, 32)) * sc;
-    mt = fmaxf(mt, mx);
-    if (__builtin_expect(__builtin_amdgcn_ballot_w64(mx > m + kSlack) != 0, 0)) {
+    for (int v = 0; v < 16; v += 2) mx = fmaxf(fmaxf(mx, s[v]), s[v + 1]);
+    mt_raw = mx;
+    if (__builtin_expect(__builtin_amdgcn_ballot_w64(mx > thr_raw) != 0, 0)) {
       // (m = -inf: first live block of a row, nothing accumulated yet)
-      const float m_new = (mx > m + kSlack) ? mx : m;
+      const float mp = fmaxf(mx, shfl_xor_f32(mx, 32)) * sc;
+      const float m_new = (mp > m + kSlack) ? mp : m;
       const float alpha = (m > kNegInf) ? __builtin_amdgcn_exp2f(m - m_new) : 0.f;
       m = m_new;
-      l *= alpha;
+      neg_m = (m > kNegInf) ? -m : 0.f;
+      thr_raw = (m + kSlack) * inv_sc;
+      lsum[0] *= alpha;
+      l_add *= alpha;
 #pragma unroll
       for (int eb = 0; eb < EB; eb++)
 #pragma unroll
         for (int v = 0; v < 16; v++) o[eb][v] *= alpha;
     }
-    const float neg_m = (m > kNegInf) ? -m : 0.f;
-    float lsum = 0.f;
+  };
+  // ... and its second half: the exponentials, packed as the B operands of the second product
+  auto soft_exp = [&](f32x16& s, uint4v (&pb)[2]) __attribute__((always_inline)) {
 #pragma unroll
     for (int v = 0; v < 16; v++)
       s[v] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[v], sc, neg_m));  // exp2(-inf) = 0
+    if constexpr (!kMfmaSum) {
+      float part = 0.f;
 #pragma unroll
-    for (int v = 0; v < 16; v++) lsum += s[v];
-    l += lsum;
+      for (int v = 0; v < 16; v++) part += s[v];
+      l_add += part;
+    }
+#pragma unroll
+    for (int sl = 0; sl < 2; sl++)
+#pragma unroll
+      for (int x = 0; x < 4; x++) pb[sl][x] = pack2<T>(s[8 * sl + 2 * x], s[8 * sl + 2 * x + 1]);
+  };
+  auto soft_core = [&](f32x16& s, uint4v (&pb)[2]) __attribute__((always_inline)) {
+    soft_max(s);
+    soft_exp(s, pb);
   };
   // V^T operands of block jb of the tile at tb: [sl][eb], two transposing 8-byte reads each
   auto v_fetch = [&](const char* tb, int jb, uint4v (&va)[2 * EB]) __attribute__((always_inline)) {
@@ -1035,25 +1078,24 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void band_dma_kernel(TileArgs
       }
   };
   // O^T += V_block^T P_block^T
-  auto pv = [&](const f32x16& s, const uint4v (&va)[2 * EB]) __attribute__((always_inline)) {
+  auto pv = [&](const uint4v (&pb)[2], const uint4v (&va)[2 * EB]) __attribute__((always_inline)) {
 #pragma unroll
     for (int sl = 0; sl < 2; sl++) {
-      uint4v pb;
 #pragma unroll
-      for (int x = 0; x < 4; x++) pb[x] = pack2<T>(s[8 * sl + 2 * x], s[8 * sl + 2 * x + 1]);
-#pragma unroll
-      for (int eb = 0; eb < EB; eb++) o[eb] = mfma16<T>(va[sl * EB + eb], pb, o[eb]);
+      for (int eb = 0; eb < EB; eb++) o[eb] = mfma16<T>(va[sl * EB + eb], pb[sl], o[eb]);
+      if constexpr (kMfmaSum) lsum = mfma16<T>(ones, pb[sl], lsum);
     }
   };
 
   // one tile: wait for it, publish it, request the tile NBUF - 1 steps ahead into the buffer the
   // previous step has freed, consume it
-  auto step = [&](int ut, int stage) __attribute__((always_inline)) {
+  auto step = [&](int it, int stage) __attribute__((always_inline)) {
+    const int ut = tile_start(it);
     const char* tb = lds + stage * BUF_B;
     // this wavefront's part of the tile has landed: the loads complete in order, and the tiles
     // requested after this one (at most NBUF - 2) may still be under way
     if constexpr (NBUF > 2) {
-      const int after = (u_hi - ut - 1) / BN;  // tiles behind this one
+      const int after = nk - 1 - it;  // tiles behind this one
       if (after >= 2) SPFA_WAIT_VMCNT(2 * 2 * NI);
       else if (after == 1) SPFA_WAIT_VMCNT(2 * NI);
       else SPFA_WAIT_VMCNT(0);
@@ -1079,7 +1121,7 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void band_dma_kernel(TileArgs
       none = none && dead;
     }
     // (a shared tail tile: the wavefronts take the key tiles in turn)
-    if (quad && (((ut - u_lo) / BN) & 3) != wave) none = true;
+    if (quad && (it & 3) != wave) none = true;
 
     // The K operands of the first block are asked for before the next tile is requested:
     // the four wavefronts issue their tile loads in one burst right after the barrier, and the
@@ -1090,7 +1132,7 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void band_dma_kernel(TileArgs
       for (int ks = 0; ks < QR; ks++) ka[ks] = *reinterpret_cast<const uint4v*>(tb + kadr[ks]);
     }
     __builtin_amdgcn_sched_barrier(0);
-    if (ut + (NBUF - 1) * BN < u_hi) request(ut + (NBUF - 1) * BN, (stage + NBUF - 1) % NBUF);
+    if (it + NBUF - 1 < nk) request(tile_start(it + NBUF - 1), (stage + NBUF - 1) % NBUF);
     __builtin_amdgcn_sched_barrier(0);
     if (none) return;
 
@@ -1106,7 +1148,7 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void band_dma_kernel(TileArgs
     const uint32_t span = jhi >= jlo ? (uint32_t)(jhi - jlo) : 0u;
 
     // the band test of a block (a compare and a select per element), then the softmax step
-    auto soft = [&](f32x16& s, int jb, bool test) __attribute__((always_inline)) {
+    auto band_test = [&](f32x16& s, int jb, bool test) __attribute__((always_inline)) {
       if (test) {
 #pragma unroll
         for (int v = 0; v < 16; v++) {
@@ -1114,7 +1156,6 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void band_dma_kernel(TileArgs
           s[v] = ((uint32_t)(c - jlo_both) <= span) ? s[v] : kNegInf;
         }
       }
-      soft_core(s);
     };
 
     uint4v va[2 * EB];
@@ -1141,13 +1182,16 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void band_dma_kernel(TileArgs
       for (int ks = 0; ks < QR; ks++) s1 = mfma16<T>(kb[ks], qh[ks], s1);
       v_fetch(tb, 0, va);
       __builtin_amdgcn_sched_barrier(0);
-      soft(s0, 0, test[0]);
-      pv(s0, va);
+      uint4v pb[2];
+      band_test(s0, 0, test[0]);
+      soft_core(s0, pb);
+      pv(pb, va);
       __builtin_amdgcn_sched_barrier(0);
       v_fetch(tb, 1, va);
       __builtin_amdgcn_sched_barrier(0);
-      soft(s1, 1, test[1]);
-      pv(s1, va);
+      band_test(s1, 1, test[1]);
+      soft_core(s1, pb);
+      pv(pb, va);
     } else {
       // one block: its V operands are read while the S product runs
       f32x16 s0 = zero16;
@@ -1155,16 +1199,18 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void band_dma_kernel(TileArgs
 #pragma unroll
       for (int ks = 0; ks < QR; ks++) s0 = mfma16<T>(ka[ks], qh[ks], s0);
       __builtin_amdgcn_sched_barrier(0);
-      soft(s0, 0, test[0]);
-      pv(s0, va);
+      uint4v pb[2];
+      band_test(s0, 0, test[0]);
+      soft_core(s0, pb);
+      pv(pb, va);
     }
   };
 
   // (unrolled over the buffers, so that every LDS address is a register plus a constant)
-  for (int ut = u_lo; ut < u_hi; ut += NBUF * BN) {
+  for (int it = 0; it < nk; it += NBUF) {
 #pragma unroll
     for (int sg = 0; sg < NBUF; sg++)
-      if (ut + sg * BN < u_hi) step(ut + sg * BN, sg);
+      if (it + sg < nk) step(it + sg, sg);
   }
 
   // ---- listed global tokens as further keys (the window + global composite): a query that is
@@ -1218,13 +1264,16 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void band_dma_kernel(TileArgs
           const bool ok = q_plain && tok >= 0 && ((uint32_t)tok + d0 > w2);
           s0[v] = ok ? s0[v] : kNegInf;
         }
-        soft_core(s0);
-        pv(s0, va);
+        uint4v pb[2];
+        soft_core(s0, pb);
+        pv(pb, va);
       }
     }
   }
 
-  l += shfl_xor_f32(l, 32);
+  // (the matrix product has summed over both halves of the wavefront)
+  float l = kMfmaSum ? lsum[0] : l_add + shfl_xor_f32(l_add, 32);
+  float mt = fmaxf(mt_raw, shfl_xor_f32(mt_raw, 32)) * sc;  // true maximum, log2 units
   if (quad) {
     // fold the four wavefronts (same queries, different key tiles) through LDS, 2, 3 into 0, 1
     // and then 1 into 0; the tile buffers are no longer needed
@@ -1339,6 +1388,15 @@ __global__ __launch_bounds__(256, 2) void band_dma_f32_kernel(TileArgs a) {
   if (t0 >= qlen) return;
   const int u_lo = t0 > wlim ? t0 - wlim : 0;
   const int u_hi = (qlen - qspan - wlim > t0) ? t0 + qspan + wlim : qlen;
+  // key tiles are visited in a rotated order, so that the workgroups of neighbouring query tiles
+  // ask for the same tile at about the same time (see band_dma_kernel)
+  const int nk = (u_hi - u_lo + BN - 1) / BN;
+  const int rot0 = uni((nk - (int)(((uint32_t)tile * (uint32_t)(BM / BN)) % (uint32_t)nk)) % nk);
+  auto tile_start = [&](int it) __attribute__((always_inline)) {
+    int j = rot0 + it;
+    j = j >= nk ? j - nk : j;
+    return u_lo + j * BN;
+  };
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -1499,14 +1557,15 @@ __global__ __launch_bounds__(256, 2) void band_dma_f32_kernel(TileArgs a) {
     }
   };
 
-  auto step = [&](int ut, const char* tb, char* other) __attribute__((always_inline)) {
+  auto step = [&](int it, const char* tb, char* other) __attribute__((always_inline)) {
+    const int ut = tile_start(it);
     __builtin_amdgcn_s_waitcnt(0);  // this wavefront's part of the tile has landed
     __syncthreads();                // everyone's has, and everyone is done with the other buffer
-    if (ut + BN < u_hi) request(ut + BN, other);
+    if (it + 1 < nk) request(tile_start(it + 1), other);
 
     const bool all_full = (ut + BN <= u_hi) && (ut >= tw0 + 31 - wlim) && (ut + BN - 1 - wlim <= tw0);
     const bool none = (tw0 >= qlen) || (ut - wlim > tw0 + 31) || (ut + BN - 1 < tw0 - wlim) ||
-                      (quad && (((ut - u_lo) / BN) & 3) != wave);
+                      (quad && (it & 3) != wave);
     if (none) return;
 
     // key slot j of the tile is live for this lane's query iff jlo <= j <= jhi; the slots this
@@ -1531,22 +1590,32 @@ __global__ __launch_bounds__(256, 2) void band_dma_f32_kernel(TileArgs a) {
       soft_core(s);
     };
 
+    // a 32-key block without a live pair beside a live one (the first and the last tile of a
+    // wavefront's band) is left out: here the matrix instructions are the time
+    bool live[NB];
+#pragma unroll
+    for (int jb = 0; jb < NB; jb++) {
+      const int ub = ut + 32 * jb;
+      live[jb] = NB == 1 || !((ub >= u_hi) || (ub - wlim > tw0 + 31) || (ub + 31 < tw0 - wlim));
+    }
     f32x16 s[NB];
 #pragma unroll
-    for (int jb = 0; jb < NB; jb++) s[jb] = s_product(tb + 32 * jb * ROWB);
+    for (int jb = 0; jb < NB; jb++)
+      if (live[jb]) s[jb] = s_product(tb + 32 * jb * ROWB);
     // ---- softmax and O^T += V^T P^T per block
 #pragma unroll
     for (int jb = 0; jb < NB; jb++) {
+      if (!live[jb]) continue;
       soft(s[jb], jb);
       __builtin_amdgcn_sched_barrier(0);
       pv_product(tb + 32 * jb * ROWB, s[jb]);
     }
   };
 
-  if (u_lo < u_hi) request(u_lo, lds_even);
-  for (int ut = u_lo; ut < u_hi; ut += 2 * BN) {
-    step(ut, lds_even, lds_odd);
-    if (ut + BN < u_hi) step(ut + BN, lds_odd, lds_even);
+  request(tile_start(0), lds_even);
+  for (int it = 0; it < nk; it += 2) {
+    step(it, lds_even, lds_odd);
+    if (it + 1 < nk) step(it + 1, lds_odd, lds_even);
   }
 
   // ---- listed global tokens as further keys (the window + global composite), as in
