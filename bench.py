@@ -32,6 +32,8 @@ HALF_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 / fp16 matrix
 
 WORKLOADS = {
     "csr_zipf": "CSR N=131072 d=64 Zipf(1.5) degrees clipped [1,4096], uniform sorted columns + diagonal",
+    "csr_zipf_hbm": "CSR N=4194304 d=64 Zipf(1.5) degrees clipped [1,4096], uniform sorted columns + diagonal "
+                    "(the headline generator at a size whose K and V, 2 GiB, do not fit the 256 MiB memory-side cache)",
     "csr_bernoulli": "CSR N=4096 d=64 Bernoulli(2%) + diagonal",
     "coo_zipf": "COO N=1048576 d=64 ~50M unsorted entries, row weights Zipf(1.3), uniform columns",
     "coo_zipf_sorted": "COO N=1048576 d=64 ~50M entries sorted by row, row weights Zipf(1.3), uniform columns",
@@ -74,14 +76,29 @@ def load_library():
     return lib
 
 
+def load_probe_library():
+    """libspfa_probe.so: the gather without arithmetic (include/spfa_probe.h), a measurement aid kept
+    apart from the attention library."""
+    path = os.path.join(os.environ.get("SPFA_LIB_DIR", PKG), "libspfa_probe.so")
+    if not os.path.exists(path):
+        path = os.path.join(PKG, "libspfa_probe.so")
+    if not os.path.exists(path):
+        raise RuntimeError("libspfa_probe.so is not built: run `python -c 'import __graft_entry__ as g; g.build()'`")
+    probe = ctypes.CDLL(path)
+    probe.spfa_probe_gather.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64,
+                                        ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64, ctypes.c_int, ctypes.c_int,
+                                        ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]
+    return probe
+
+
 def make_workload(name, dtype, torch, syn, inline_limit=32, planned=False, heads=1, loop_heads=False, d_local=64):
     """Returns dict(call=fn(state) -> None, n, d, nnz, bytes_total, bytes_gathered, sample=fn())."""
     dev = "cuda"
     es = torch.tensor([], dtype=dtype).element_size()
     w = {"name": name, "desc": WORKLOADS[name]}
-    if name in ("csr_zipf", "csr_bernoulli", "coo_zipf", "coo_zipf_sorted"):
-        if name == "csr_zipf":
-            n, d = 131072, 64
+    if name in ("csr_zipf", "csr_zipf_hbm", "csr_bernoulli", "coo_zipf", "coo_zipf_sorted"):
+        if name in ("csr_zipf", "csr_zipf_hbm"):
+            n, d = (131072 if name == "csr_zipf" else 1 << 22), 64
             ro, ci = syn.zipf_csr(n, 1.5, 1, 4096, device=dev, seed=0)
         elif name == "csr_bernoulli":
             n, d = 4096, 64
@@ -274,8 +291,14 @@ def live_columns_fn(w, torch):
         ro_c = ro.cpu().numpy()
         return lambda i: ci[ro_c[i]:ro_c[i + 1]].cpu().numpy()
     if name.startswith("coo"):
+        # (the entries are bucketed by row once; a compare over all of them per sampled row would
+        # take minutes for a block of the CPU baseline)
         r, c = w["coo"]
-        return lambda i: c[r == int(i)].cpu().numpy()
+        order = torch.argsort(r, stable=True)
+        c_sorted = c[order]
+        off = torch.searchsorted(r[order].contiguous(), torch.arange(n + 1, device=r.device)).cpu().numpy()
+        del order
+        return lambda i: c_sorted[off[i]:off[i + 1]].cpu().numpy()
     if name == "local":
         return lambda i: so.live_local(n, w["params"]["LOCAL_SIZE"], int(i))
     if name == "local_1d":
@@ -429,18 +452,19 @@ def measured_traffic(workload, dtype_name):
     workload (profiles/<workload>..._pmc.md, line `traffic_bytes_per_launch = N`), else None."""
     import glob
     import re
-    names = {"csr_zipf": "csr_zipf_n131072_d64", "coo_zipf": "coo_zipf_unsorted_n1048576_d64"}
+    names = {"csr_zipf": "csr_zipf_n131072_d64", "coo_zipf": "coo_zipf_unsorted_n1048576_d64",
+             "csr_zipf_hbm": "csr_zipf_hbm_n4194304_d64"}
     stem = names.get(workload)
     if stem is None:
         return None
     for path in glob.glob(os.path.join(ROOT, "profiles", "%s_%s_pmc.md" % (stem, {"f32": "f32"}.get(dtype_name, dtype_name)))):
         m = re.search(r"^traffic_bytes_per_launch\s*=\s*(\d+)", open(path).read(), re.M)
         if m:
-            return int(m.group(1))
-    return None
+            return int(m.group(1)), os.path.relpath(path, ROOT)
+    return None, None
 
 
-def bench_backward(a, w, st, dtype, torch, syn):
+def bench_backward(a, w, st, dtype, torch, syn, lib):
     """--backward: one forward call builds the state, then K timed gradient calls (they add into
     the same dQ, dK, dV; the parity check afterwards starts from zeroed gradients)."""
     if a.loop_heads:
@@ -469,31 +493,74 @@ def bench_backward(a, w, st, dtype, torch, syn):
     live = (st[1] > 0).double().unsqueeze(-1)
     col_err = float(((grads[2].double().sum(dim=-2) - (d_out.double() * live).sum(dim=-2)).abs().max()
                      / d_out.double().abs().sum(dim=-2).max()))
-    # algorithmic work: five products of length d per live position (scores, dO.V, dQ, dK, dV);
-    # bytes: K, V rows for the query pass and Q, dO rows for the key pass per live position, the
-    # dense tensors once (q, k, v, out, dO read; dQ, dK, dV read and written in fp32)
+    # Algorithmic work: five products of length d per live position (scores, dO.V, dQ, dK, dV).
+    # Bytes: the dense tensors once (q, k, v, out, dO read; dQ, dK, dV read and written in fp32);
+    # a position that a GATHER pass processes also fetches K, V rows (query pass) and Q, dO rows
+    # (key pass) and two index words; a position that a TILE kernel processes is matrix work on
+    # streamed tiles and fetches nothing of its own.  The composite's window and listed-token
+    # positions are tile work, only its random (CSR) part is gathered.
     heads = w.get("heads", 1)
+    name = w["name"]
+    explicit = name.startswith(("csr", "coo"))
     flops = 10.0 * d * nnz
     dense = heads * n * d * (5 * es + 6 * 4)
-    gathered = nnz * 4 * d * es
-    index = nnz * 8 if w["name"].startswith(("csr", "coo", "bigbird")) else 0
+    nnz_gather = nnz if explicit else (w["params"]["csr_nnz"] if name == "bigbird" else 0)
+    nnz_tiles = nnz - nnz_gather
+    gathered = nnz_gather * 4 * d * es
+    index = nnz_gather * 8
     total = dense + gathered + index
-    if w["name"].startswith(("csr", "coo", "bigbird")):
-        # gather passes: bound by memory
-        roofline = {"bound": "hbm", "achieved": total / (ms_per_step * 1e-3) / 1e9, "peak": HBM_PEAK_GBS,
-                    "unit": "GB/s", "frac": total / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": None,
-                    "kernel": "whole call (query pass + key pass)", "algorithmic_bytes": total,
-                    "gathered_bytes": gathered}
+    t_s = ms_per_step * 1e-3
+    mfma_peak = FP32_PEAK_TFLOPS if a.dtype == "f32" else HALF_PEAK_TFLOPS
+    # what the gather passes can be served at: the published HBM rate when Q, K, V, dO together do
+    # not fit the 256 MiB memory-side cache, else what the same gather without arithmetic
+    # sustains over this K, V and this column list on this device (as for the forward call)
+    ws_bytes = 4 * w["k"].numel() * es
+    gather = measured_gather_ceiling(lib, w, torch) if nnz_gather else None
+    if nnz_gather and ws_bytes > (256 << 20) or gather is None:
+        gather_peak, gather_src = HBM_PEAK_GBS, "MI355X HBM3E, published"
+        gather_bound = "hbm"
     else:
-        # dense tiles: bound by the matrix pipe; both passes recompute the scores and dO.V, so 14*d
-        # flops per live position are executed for the 10*d counted
-        peak = FP32_PEAK_TFLOPS if a.dtype == "f32" else HALF_PEAK_TFLOPS
-        achieved_tf = flops / (ms_per_step * 1e-3) / 1e12
-        roofline = {"bound": "mfma", "achieved": achieved_tf, "peak": peak, "unit": "TFLOP/s",
-                    "frac": achieved_tf / peak, "traffic": None,
-                    "kernel": "whole call (tile_grad_kernel, query pass + key pass)",
-                    "executed_over_counted_flops": 1.4,
-                    "hbm_time_ms": dense / (HBM_PEAK_GBS * 1e9) * 1e3, "mfma_time_ms": flops / (peak * 1e12) * 1e3}
+        gather_peak = gather["GBs"]
+        gather_src = "measured on this device: the same gather without arithmetic (spfa_probe_gather)"
+        gather_bound = "l2" if ws_bytes <= (4 << 20) else "infinity_cache"
+    gather_ms = (gathered + index) / (gather_peak * 1e9) * 1e3 if nnz_gather else 0.0
+    tile_flops = 10.0 * d * nnz_tiles
+    dense_ms = dense / (HBM_PEAK_GBS * 1e9) * 1e3
+    mfma_ms = tile_flops / (mfma_peak * 1e12) * 1e3
+    # the gather passes and the tile kernels run one after the other: the floor of the call is the
+    # gather time plus the larger of the dense tensors' HBM time and the tiles' matrix time
+    roof_ms = gather_ms + max(dense_ms, mfma_ms)
+    half_band = a.dtype != "f32" and d in (64, 128) and name in ("local", "local_1d", "local_2d", "bigbird")
+    tile_kernels = ("band_grad_dma_kernel (query pass, key pass%s)" % (" as dK and dV launches" if d == 128 else "")
+                    if half_band else "tile_grad_kernel (query pass, key pass)")
+    if name == "global" or name == "bigbird":
+        tile_kernels += " + tile_grad_kernel / global_grad_merge_kernel for the listed tokens"
+    gather_kernels = "grad_prologue_kernel, grad_rows_kernel (query pass, key pass), grad_items_kernel" + \
+                     (", mask transposition" if not a.planned and name.startswith(("csr", "bigbird")) else "") + \
+                     (", two COO bucketing pre-passes" if name.startswith("coo") else "")
+    if gather_ms >= max(dense_ms, mfma_ms):
+        bound, unit = gather_bound, "GB/s"
+        achieved, peak = total / t_s / 1e9, gather_peak
+    elif dense_ms >= mfma_ms:
+        bound, unit = "hbm", "GB/s"
+        achieved, peak = total / t_s / 1e9, HBM_PEAK_GBS
+    else:
+        bound, unit = "mfma", "TFLOP/s"
+        achieved, peak = flops / t_s / 1e12, mfma_peak
+    roofline = {"bound": bound, "achieved": achieved, "peak": peak, "unit": unit,
+                "frac": roof_ms / ms_per_step, "frac_is": "roofline_time_ms / ms_per_step (the whole call; "
+                "no single kernel dominates a gradient call, so no per-kernel time is taken)",
+                "frac_above_one": bool(roof_ms > ms_per_step), "traffic": None,
+                "kernel": "whole call: " + ", ".join(x for x in (gather_kernels if nnz_gather else None,
+                                                                 tile_kernels if nnz_tiles else None) if x),
+                "roofline_time_ms": roof_ms, "gather_time_ms": gather_ms, "hbm_time_ms": dense_ms,
+                "mfma_time_ms": mfma_ms, "gather_peak_GBs": gather_peak if nnz_gather else None,
+                "gather_peak_source": gather_src if nnz_gather else None,
+                "working_set_bytes": ws_bytes, "algorithmic_bytes": total, "gathered_bytes": gathered,
+                "gathered_positions": nnz_gather, "tile_positions": nnz_tiles,
+                "executed_over_counted_tile_flops": 1.4}
+    if gather is not None:
+        roofline["measured_gather"] = gather["how"]
     out = {
         "metric": "masked-attn backward GFLOP/s (10*d per live position) + algorithmic GB/s",
         "value": flops / (ms_per_step * 1e-3) / 1e9, "unit": "GFLOP/s",
@@ -543,28 +610,22 @@ def measured_gather_ceiling(lib, w, torch, min_entries=8_000_000, reps=5):
         return None
     if idx.numel() < min_entries:
         idx = idx.repeat((min_entries + idx.numel() - 1) // idx.numel())
-    lib.spfa_probe_gather.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64,
-                                      ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64, ctypes.c_int, ctypes.c_int,
-                                      ctypes.c_void_p, ctypes.c_void_p]
+    probe = load_probe_library()
     cursor = torch.zeros(64, dtype=torch.int32, device="cuda")
     stream = torch.cuda.current_stream().cuda_stream
     # timed like the kernel it is compared with: the dispatch's own start and end stamps
     ev = HipEvents()
     best, best_shape = float("inf"), None
     shapes = ((1, 16), (1, 32), (2, 16), (2, 32), (4, 32))
-    try:
-        for wg, fl in shapes:
-            for _ in range(reps):
-                lib.spfa_set_kernel_events(ev.start, ev.stop)
-                rc = lib.spfa_probe_gather(k.data_ptr(), v.data_ptr(), k.shape[0], row_bytes, idx.data_ptr(),
-                                           idx.numel(), 1024, wg, fl, cursor.data_ptr(), stream)
-                assert rc == 0, "spfa_probe_gather rc=%d" % rc
-                torch.cuda.synchronize()
-                ms = ev.elapsed_ms()
-                if ms < best:
-                    best, best_shape = ms, (wg, fl)
-    finally:
-        lib.spfa_set_kernel_events(None, None)
+    for wg, fl in shapes:
+        for _ in range(reps):
+            rc = probe.spfa_probe_gather(k.data_ptr(), v.data_ptr(), k.shape[0], row_bytes, idx.data_ptr(),
+                                         idx.numel(), 1024, wg, fl, cursor.data_ptr(), ev.start, ev.stop, stream)
+            assert rc == 0, "spfa_probe_gather rc=%d" % rc
+            torch.cuda.synchronize()
+            ms = ev.elapsed_ms()
+            if ms < best:
+                best, best_shape = ms, (wg, fl)
     bytes_moved = idx.numel() * (2 * row_bytes + 4)
     return {"GBs": bytes_moved / (best * 1e-3) / 1e9,
             "how": "%d list entries x (2 rows of %d B + 4 B index) in %.3f ms; best of %d launches each of "
@@ -640,7 +701,7 @@ def main():
         return st
 
     if a.backward:
-        return bench_backward(a, w, states[0], dtype, torch, syn)
+        return bench_backward(a, w, states[0], dtype, torch, syn, lib)
 
     n_ev = min(a.steps, 10)
     evs = [HipEvents() for _ in range(n_ev)]
@@ -737,6 +798,10 @@ def main():
                      kernel_rows=w["n"] * w.get("heads", 1))
         achieved_gbs = w["kernel_bytes"] / (k_avg * 1e-3) / 1e9
         kv_bytes = 2 * w["k"].numel() * es
+        traffic, traffic_src = measured_traffic(a.workload, a.dtype)
+        if traffic is not None:
+            traffic_src = "read from %s (two rocprofv3 --pmc runs of this command, FETCH_SIZE and " \
+                          "WRITE_SIZE scaled by a copy kernel); not measured by this process" % traffic_src
         gather = measured_gather_ceiling(lib, w, torch)
         if kv_bytes <= 4 << 20:
             bound = "l2"
@@ -750,7 +815,7 @@ def main():
                     "peak_source": "MI355X HBM3E, published" if peak == HBM_PEAK_GBS else
                                    "measured on this device: the same gather without arithmetic "
                                    "(spfa_probe_gather) over this K and V and this column list",
-                    "traffic": measured_traffic(a.workload, a.dtype), "kernel": kernel_name,
+                    "traffic": traffic, "traffic_source": traffic_src, "kernel": kernel_name,
                     "kv_working_set_bytes": kv_bytes,
                     "hbm_peak_GBs": HBM_PEAK_GBS, "achieved_over_hbm_peak": achieved_gbs / HBM_PEAK_GBS}
         if gather is not None:
@@ -793,7 +858,8 @@ def main():
     roofline["frac_above_one"] = bool(roofline["frac"] > 1.0)
     call_sorted = sorted(call_ms)
     roofline.update({"kernel_ms_avg": k_avg, "kernel_ms_min": min(kernel_ms),
-                     "kernel_ms_from": "event pairs around the kernel in the last %d steps of the timed loop"
+                     "kernel_ms_from": "start / stop events attached to the kernel's own dispatch "
+                                       "(hipExtLaunchKernelGGL) in the last %d steps of the timed loop"
                                        % len(kernel_ms),
                      "algorithmic_bytes": w["kernel_bytes"], "kernel_nnz": w["kernel_nnz"],
                      "kernel_rows": w["kernel_rows"], "call_algorithmic_bytes": w["bytes_total"],

@@ -1,7 +1,8 @@
-"""Build libspfa_hip.so (HIP kernels + C ABI, gfx950) and the six torch host wrappers in-tree.
+"""Build libspfa_hip.so (HIP kernels + C ABI, gfx950), libspfa_probe.so (a measurement aid for
+benchmarks, include/spfa_probe.h) and the torch host wrappers in-tree.
 
     python build.py            # everything
-    python build.py --lib      # only libspfa_hip.so
+    python build.py --lib      # only libspfa_hip.so and libspfa_probe.so
     python build.py --ext      # only the spfa_* Python modules
 
 The wrappers are host-only C++ (g++): they check tensors the way the reference bindings do and
@@ -73,6 +74,15 @@ def build_lib(workers: int) -> str:
         list(ex.map(lambda j: _run(j[1]), jobs))
     out = os.path.join(HERE, "libspfa_hip.so")
     _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", out, *[j[0] for j in jobs]])
+    return out
+
+
+def build_probe() -> str:
+    """libspfa_probe.so: the gather probe that bench.py prices the explicit-mask kernels against
+    (csrc/probe/, apart from the attention library)."""
+    os.makedirs(OBJ, exist_ok=True)
+    out = os.path.join(HERE, "libspfa_probe.so")
+    _run([HIPCC, *HIP_FLAGS, "-shared", "-o", out, os.path.join(CSRC, "probe", "spfa_probe.hip")])
     return out
 
 
@@ -182,8 +192,9 @@ def check_loop_nests(workers: int | None = None) -> None:
 def build_all(workers: int | None = None):
     workers = workers or min(8, os.cpu_count() or 4)
     lib = build_lib(workers)
+    probe = build_probe()
     exts = build_ext(min(workers, 6))
-    return [lib, *exts]
+    return [lib, probe, *exts]
 
 
 if __name__ == "__main__":
@@ -200,6 +211,7 @@ if __name__ == "__main__":
         sys.exit(0)
     if a.lib or not a.ext:
         print(build_lib(w))
+        print(build_probe())
     if a.ext or not a.lib:
         for o in build_ext(min(w, 6)):
             print(o)

@@ -8,6 +8,11 @@
 // HBM figure no longer binds.  This kernel does those loads and nothing else: no dot products, no
 // softmax, no output.  The loaded registers are handed to an empty asm statement so that the
 // loads stay.
+//
+// Built into libspfa_probe.so, apart from the attention library: benchmarks load it, the drop-in
+// boundary does not carry it.
+#include "spfa_probe.h"
+
 #include "spfa_hip.h"
 
 #include "spfa_common.hpp"
@@ -20,9 +25,14 @@ __global__ void probe_reset_kernel(uint32_t* cursor) {
   if (threadIdx.x == 0) *cursor = 0;
 }
 
+// an entry of the list: a row below n_rows, else (top bit set, or out of range) skipped.  The
+// value is consumed one trip after it is loaded, so the comparison costs no wait.
+__device__ __forceinline__ int probe_entry(uint32_t x, uint32_t n_rows) { return x < n_rows ? (int)x : -1; }
+
 template <int LPR, int U>
 __global__ __launch_bounds__(256) void gather_probe_kernel(const char* __restrict__ k,
                                                            const char* __restrict__ v, int64_t row_bytes,
+                                                           uint32_t n_rows,
                                                            const uint32_t* __restrict__ idx, int64_t n_idx,
                                                            int64_t chunk, uint32_t* cursor) {
   constexpr int GS = kWave / LPR;  // rows per wavefront-wide load
@@ -40,10 +50,10 @@ __global__ __launch_bounds__(256) void gather_probe_kernel(const char* __restric
     if ((int64_t)w >= n_chunks) break;
     const int64_t t0 = (int64_t)w * chunk;
     const int64_t t1 = t0 + chunk < n_idx ? t0 + chunk : n_idx;
-    int next = t0 + lane < t1 ? (int)idx[t0 + lane] : -1;
+    int next = t0 + lane < t1 ? probe_entry(idx[t0 + lane], n_rows) : -1;
     for (int64_t tb = t0; tb < t1; tb += kWave) {
       const int cur = next;
-      if (tb + kWave < t1) next = tb + kWave + lane < t1 ? (int)idx[tb + kWave + lane] : -1;
+      if (tb + kWave < t1) next = tb + kWave + lane < t1 ? probe_entry(idx[tb + kWave + lane], n_rows) : -1;
 #pragma unroll 1
       for (int part = 0; part < PARTS; part++) {
         if (tb + part * PER >= t1) break;
@@ -75,6 +85,7 @@ __global__ __launch_bounds__(256) void gather_probe_kernel(const char* __restric
 template <int LPR>
 __global__ __launch_bounds__(256) void gather_probe_deep_kernel(const char* __restrict__ k,
                                                                 const char* __restrict__ v, int64_t row_bytes,
+                                                                uint32_t n_rows,
                                                                 const uint32_t* __restrict__ idx, int64_t n_idx,
                                                                 int64_t chunk, uint32_t* cursor) {
   constexpr int GS = kWave / LPR;
@@ -90,7 +101,7 @@ __global__ __launch_bounds__(256) void gather_probe_deep_kernel(const char* __re
     if ((int64_t)w >= n_chunks) break;
     const int64_t t0 = (int64_t)w * chunk;
     const int64_t t1 = t0 + chunk < n_idx ? t0 + chunk : n_idx;
-    auto fetch = [&](int64_t t) -> int { return t + lane < t1 ? (int)idx[t + lane] : -1; };
+    auto fetch = [&](int64_t t) -> int { return t + lane < t1 ? probe_entry(idx[t + lane], n_rows) : -1; };
     int next0 = fetch(t0), next1 = fetch(t0 + kWave);
     for (int64_t tb = t0; tb < t1; tb += 2 * kWave) {
       const int cur0 = next0, cur1 = next1;
@@ -121,32 +132,32 @@ __global__ __launch_bounds__(256) void gather_probe_deep_kernel(const char* __re
 }
 
 template <int LPR>
-int launch_probe(const void* k, const void* v, int64_t row_bytes, const uint32_t* idx, int64_t n_idx,
-                 int64_t chunk, int wg_per_cu, int in_flight, uint32_t* cursor, hipStream_t stream) {
+int launch_probe(const void* k, const void* v, int64_t row_bytes, uint32_t n_rows, const uint32_t* idx,
+                 int64_t n_idx, int64_t chunk, int wg_per_cu, int in_flight, uint32_t* cursor,
+                 const KernelEvents& ev, hipStream_t stream) {
   int dev = 0, cus = 256;
   if (hipGetDevice(&dev) == hipSuccess)
     (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
   const dim3 grid((unsigned)(cus * wg_per_cu)), block(256);
   hipLaunchKernelGGL(probe_reset_kernel, dim3(1), dim3(64), 0, stream, cursor);
-  // the gather itself takes the caller's event pair, as the kernel it stands in for does
-  const KernelEvents ev = kernel_events();
+  // (the gather itself takes the caller's event pair, as the kernel it stands in for does)
   constexpr int UMAX = LPR;  // a batch of U rows per group covers at most one 64-entry chunk
   if constexpr (LPR <= 16) {
     if (in_flight >= 2 * UMAX) {
       launch_maybe_timed(ev, gather_probe_deep_kernel<LPR>, grid, block, stream, (const char*)k, (const char*)v,
-                         row_bytes, idx, n_idx, chunk, cursor);
+                         row_bytes, n_rows, idx, n_idx, chunk, cursor);
       return hipGetLastError() == hipSuccess ? SPFA_OK : SPFA_ERR_LAUNCH;
     }
   }
   if (in_flight >= 16 && UMAX >= 16)
     launch_maybe_timed(ev, gather_probe_kernel<LPR, (UMAX >= 16 ? 16 : UMAX)>, grid, block, stream,
-                       (const char*)k, (const char*)v, row_bytes, idx, n_idx, chunk, cursor);
+                       (const char*)k, (const char*)v, row_bytes, n_rows, idx, n_idx, chunk, cursor);
   else if (in_flight >= 8 && UMAX >= 8)
     launch_maybe_timed(ev, gather_probe_kernel<LPR, (UMAX >= 8 ? 8 : UMAX)>, grid, block, stream,
-                       (const char*)k, (const char*)v, row_bytes, idx, n_idx, chunk, cursor);
+                       (const char*)k, (const char*)v, row_bytes, n_rows, idx, n_idx, chunk, cursor);
   else
     launch_maybe_timed(ev, gather_probe_kernel<LPR, 4>, grid, block, stream, (const char*)k, (const char*)v,
-                       row_bytes, idx, n_idx, chunk, cursor);
+                       row_bytes, n_rows, idx, n_idx, chunk, cursor);
   return hipGetLastError() == hipSuccess ? SPFA_OK : SPFA_ERR_LAUNCH;
 }
 
@@ -155,17 +166,22 @@ int launch_probe(const void* k, const void* v, int64_t row_bytes, const uint32_t
 
 extern "C" int spfa_probe_gather(const void* k, const void* v, int64_t n_rows, int64_t row_bytes,
                                  const uint32_t* idx, int64_t n_idx, int64_t chunk, int wg_per_cu,
-                                 int in_flight, void* cursor, void* stream) {
+                                 int in_flight, void* cursor, void* ev_start, void* ev_stop, void* stream) {
   using namespace spfa;
-  if (!k || !v || !idx || !cursor || n_rows < 1 || n_idx < 1 || chunk < 64 || wg_per_cu < 1 || wg_per_cu > 8)
+  if (!k || !v || !idx || !cursor || n_rows < 1 || n_rows > (int64_t)0x7fffffff || n_idx < 1 || chunk < 64 ||
+      wg_per_cu < 1 || wg_per_cu > 8)
     return SPFA_ERR_BAD_ARG;
+  KernelEvents ev;
+  ev.start = (hipEvent_t)ev_start;
+  ev.stop = (hipEvent_t)ev_stop;
+  const uint32_t nr = (uint32_t)n_rows;
   if ((((uintptr_t)k | (uintptr_t)v) & 15u) != 0) return SPFA_ERR_BAD_ARG;
   hipStream_t s = (hipStream_t)stream;
   switch (row_bytes) {
-    case 64: return launch_probe<4>(k, v, row_bytes, idx, n_idx, chunk, wg_per_cu, in_flight, (uint32_t*)cursor, s);
-    case 128: return launch_probe<8>(k, v, row_bytes, idx, n_idx, chunk, wg_per_cu, in_flight, (uint32_t*)cursor, s);
-    case 256: return launch_probe<16>(k, v, row_bytes, idx, n_idx, chunk, wg_per_cu, in_flight, (uint32_t*)cursor, s);
-    case 512: return launch_probe<32>(k, v, row_bytes, idx, n_idx, chunk, wg_per_cu, in_flight, (uint32_t*)cursor, s);
+    case 64: return launch_probe<4>(k, v, row_bytes, nr, idx, n_idx, chunk, wg_per_cu, in_flight, (uint32_t*)cursor, ev, s);
+    case 128: return launch_probe<8>(k, v, row_bytes, nr, idx, n_idx, chunk, wg_per_cu, in_flight, (uint32_t*)cursor, ev, s);
+    case 256: return launch_probe<16>(k, v, row_bytes, nr, idx, n_idx, chunk, wg_per_cu, in_flight, (uint32_t*)cursor, ev, s);
+    case 512: return launch_probe<32>(k, v, row_bytes, nr, idx, n_idx, chunk, wg_per_cu, in_flight, (uint32_t*)cursor, ev, s);
   }
   return SPFA_ERR_UNSUPPORTED;
 }

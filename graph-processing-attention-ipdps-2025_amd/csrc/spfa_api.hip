@@ -303,7 +303,7 @@ static __device__ uint32_t spfa_status_word;
 
 namespace spfa {
 KernelEvents& kernel_events() {
-  static KernelEvents ev;
+  static thread_local KernelEvents ev;  // (per host thread: the caller's own calls only)
   return ev;
 }
 

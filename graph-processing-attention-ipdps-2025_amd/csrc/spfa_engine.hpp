@@ -21,6 +21,7 @@
 // form one grid, the work list is shared, partial results are per problem.
 #pragma once
 
+#include <atomic>
 #include <hip/hip_ext.h>
 
 #include "spfa_common.hpp"
@@ -778,6 +779,24 @@ inline WorkspaceLayout engine_workspace(const EngineSizing& s, int64_t n_q, int6
   w.off_pacc = off;     off = align_up(off + nb * (size_t)cap_partials * (size_t)d * sizeof(float), 256);
   w.total = off;
   return w;
+}
+
+// Raises a kernel's dynamic-LDS limit to `bytes`, once per device: `raised` is the caller's table
+// of kLdsLimitDevices flags for that kernel (atomic: callers may be on several host threads; two
+// that meet here both set the attribute, which is idempotent).  A device beyond the table gets
+// the attribute set on every call.  False when the runtime refuses.
+constexpr int kLdsLimitDevices = 64;
+inline bool raise_lds_limit(const void* kernel, int bytes, std::atomic<bool>* raised) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess) return false;
+  const bool tabled = dev >= 0 && dev < kLdsLimitDevices;
+  if (tabled && raised[dev].load(std::memory_order_acquire)) return true;
+  if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes) != hipSuccess) {
+    (void)hipGetLastError();
+    return false;
+  }
+  if (tabled) raised[dev].store(true, std::memory_order_release);
+  return true;
 }
 
 // optional event pair recorded around the dominant kernel (see spfa_set_kernel_events)

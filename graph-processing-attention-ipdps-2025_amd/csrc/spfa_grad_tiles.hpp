@@ -798,17 +798,9 @@ __global__ __launch_bounds__(256, (KEYS && D == 128 && PART == 0) ? 1 : 2) void 
 template <typename T, int D, bool KEYS, int PART = 0>
 bool launch_band_grad_dma(const TileArgs& a, const GradArgs& g, dim3 grid, hipStream_t stream) {
   using C = BandGradDmaCfg<T, D, KEYS, PART>;
-  constexpr int kMaxDevices = 64;
-  static bool raised[kMaxDevices];
-  int dev = 0;
-  (void)hipGetDevice(&dev);
-  if (dev < 0 || dev >= kMaxDevices) return false;
-  if (!raised[dev]) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&band_grad_dma_kernel<T, D, KEYS, PART>),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES) != hipSuccess)
-      return false;
-    raised[dev] = true;
-  }
+  static std::atomic<bool> raised[kLdsLimitDevices];
+  if (!raise_lds_limit(reinterpret_cast<const void*>(&band_grad_dma_kernel<T, D, KEYS, PART>), C::LDS_BYTES, raised))
+    return false;
   hipLaunchKernelGGL((band_grad_dma_kernel<T, D, KEYS, PART>), grid, dim3(256), C::LDS_BYTES, stream, a, g);
   return true;
 }

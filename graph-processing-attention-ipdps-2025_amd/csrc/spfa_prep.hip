@@ -1,6 +1,7 @@
 // Mask pre-passes that run on the device before the attention kernels:
 //   - COO entries -> row buckets (histogram, exclusive scan, scatter), any entry order;
 //   - global-token list -> per-row flag bytes.
+#include <atomic>
 #include "spfa_prep.hpp"
 
 #include <type_traits>
@@ -898,11 +899,13 @@ int coo_to_csr(const void* row_ind, int row_wide, const uint32_t* col_ind, int64
     uint64_t* tmp_pairs = (uint64_t*)(base + w.off_tmp_pairs);
     // 152 KB of LDS per workgroup in both passes: above the 64 KB a kernel gets without asking
     // (set once per device: the attribute belongs to the device's copy of the kernel)
+    // (atomic flags: callers may be on several host threads; two that meet here both set the
+    // attributes, which is idempotent)
     constexpr int kMaxDevices = 64;
-    static bool lds_attr_set[kMaxDevices];
+    static std::atomic<bool> lds_attr_set[kMaxDevices];
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess) return 4;
-    if (dev < 0 || dev >= kMaxDevices || !lds_attr_set[dev]) {
+    if (dev < 0 || dev >= kMaxDevices || !lds_attr_set[dev].load(std::memory_order_acquire)) {
       const int packed_max = (int)part_scatter_packed_lds(kPartMaxBuckets);
       const struct { const void* kernel; int bytes; } big_lds[] = {
           {reinterpret_cast<const void*>(coo_part_scatter_kernel<uint64_t>), (int)kPartScatterLds},
@@ -914,7 +917,7 @@ int coo_to_csr(const void* row_ind, int row_wide, const uint32_t* col_ind, int64
       for (const auto& k : big_lds)
         if (hipFuncSetAttribute(k.kernel, hipFuncAttributeMaxDynamicSharedMemorySize, k.bytes) != hipSuccess)
           return 4;
-      if (dev >= 0 && dev < kMaxDevices) lds_attr_set[dev] = true;
+      if (dev >= 0 && dev < kMaxDevices) lds_attr_set[dev].store(true, std::memory_order_release);
     }
     const int64_t n_hist = w.n_hi * w.n_tiles1;
     const int64_t hist_tiles = (n_hist + kScanTile - 1) / kScanTile;

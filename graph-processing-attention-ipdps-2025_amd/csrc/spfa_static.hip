@@ -46,10 +46,14 @@ int device_scratch(void** out) {
 extern "C" int spfa_csr_forward_static(const spfa_problem_t* p, const void* row_off, int row_off_bytes,
                                        const void* col_ind, int64_t nnz, int use_nan, void* stream) {
   if (p == nullptr || nnz < 0) return SPFA_ERR_BAD_ARG;
-  const int64_t nb = p->n_batch > 1 ? p->n_batch : 1;
-  const size_t one = spfa_csr_workspace_bytes(p->n_q, nnz, p->d, p->dtype);
-  if (one > (size_t)SPFA_STATIC_SCRATCH_BYTES || one * (size_t)nb > (size_t)SPFA_STATIC_SCRATCH_BYTES)
-    return SPFA_ERR_STATIC_LIMIT;
+  // The limit is what the call below asks of its workspace: the work list once, the partial
+  // results once per problem of a batch (a batch too large for one work cursor is walked problem
+  // by problem on one problem's worth).  Sizes that are not a valid problem give 0 here and are
+  // rejected by the call's own checks; fp64 problems use no scratch at all.
+  if (p->dtype != SPFA_DTYPE_F64) {
+    const size_t need = spfa_csr_workspace_bytes_batched(p->n_q, nnz, p->d, p->dtype, p->n_batch > 1 ? p->n_batch : 1);
+    if (need > (size_t)SPFA_STATIC_SCRATCH_BYTES) return SPFA_ERR_STATIC_LIMIT;
+  }
   void* ptr = nullptr;
   const int rc = device_scratch(&ptr);
   if (rc) return rc;

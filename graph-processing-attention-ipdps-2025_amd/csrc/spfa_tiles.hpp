@@ -1806,19 +1806,23 @@ constexpr int64_t kFusedMaxGlobals = 256;
 
 // tile_kernel's launch: shapes whose tile buffers exceed 64 KB get them as dynamic LDS (the limit
 // of the kernel is raised once per device)
+// (tile_kernel_ready: false when the runtime refuses the limit; the callers ask before they
+// launch anything and leave the call to the row-gather engine then)
+template <typename T, int D, int MODE>
+bool tile_kernel_ready() {
+  using C = TileCfg<T, D>;
+  if constexpr (C::kDynLds) {
+    static std::atomic<bool> raised[kLdsLimitDevices];
+    return raise_lds_limit(reinterpret_cast<const void*>(&tile_kernel<T, D, MODE>), C::LDS_BYTES, raised);
+  }
+  return true;
+}
+
 template <typename T, int D, int MODE>
 void launch_tile_kernel(const KernelEvents& ev, dim3 grid, hipStream_t stream, const TileArgs& a) {
   using C = TileCfg<T, D>;
   if constexpr (C::kDynLds) {
-    constexpr int kMaxDevices = 64;
-    static bool raised[kMaxDevices];
-    int dev = 0;
-    (void)hipGetDevice(&dev);
-    if (dev >= 0 && dev < kMaxDevices && !raised[dev]) {
-      (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&tile_kernel<T, D, MODE>),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES);
-      raised[dev] = true;
-    }
+    if (!tile_kernel_ready<T, D, MODE>()) return;  // (asked before; a refusal surfaces as a launch error)
     if (ev.start != nullptr && ev.stop != nullptr)
       hipExtLaunchKernelGGL((tile_kernel<T, D, MODE>), grid, dim3(256), C::LDS_BYTES, stream, ev.start, ev.stop, 0, a);
     else
@@ -1859,7 +1863,10 @@ int launch_band_tiles(const TileArgs& a, int use_nan, hipStream_t stream) {
         const int64_t grid_d = (n_all - at.n_tail + 7) / 8 * 8 + 4 * at.n_tail;
         launch_maybe_timed(ev, band_dma_kernel<T, D, SPFA_BAND_BN(D)>, dim3((unsigned)grid_d), dim3(256), stream, at);
       }
-      if (!dma) launch_tile_kernel<T, D, kTileBand>(ev, dim3((unsigned)grid), stream, a);
+      if (!dma) {
+        if (!tile_kernel_ready<T, D, kTileBand>()) return -1;
+        launch_tile_kernel<T, D, kTileBand>(ev, dim3((unsigned)grid), stream, a);
+      }
     } else {
       // listed global tokens as further keys: only the direct-to-LDS kernel takes them
       if (a.globs != nullptr && !((D == 64 || D == 128) && a.n_globs <= kFusedMaxGlobals)) return -1;
@@ -1896,6 +1903,7 @@ int launch_band_tiles(const TileArgs& a, int use_nan, hipStream_t stream) {
         return -1;
       } else {
         const int64_t grid_t = (n_main + 7) / 8 * 8 + 4 * at.n_tail;
+        if (!tile_kernel_ready<T, D, kTileBand>()) return -1;
         launch_tile_kernel<T, D, kTileBand>(ev, dim3((unsigned)grid_t), stream, at);
       }
     }
@@ -1916,6 +1924,7 @@ int launch_band_tiles(const TileArgs& a, int use_nan, hipStream_t stream) {
 template <typename T, int D>
 int launch_global_tiles(const TileArgs& a, hipStream_t stream, bool rows_only) {
   const KernelEvents ev = kernel_events();
+  if (!tile_kernel_ready<T, D, kTileGlobalCols>() || !tile_kernel_ready<T, D, kTileGlobalRows>()) return -1;
   int64_t grid_cols = (a.n + 127) / 128;
   TileArgs ac = a;
   ac.persist = (a.n_globs <= TileCfg<T, D>::BN) ? 1 : 0;

@@ -105,25 +105,13 @@ enum { SPFA_STATUS_WORK_LIST_OVERFLOW = 1, SPFA_STATUS_ROW_OFFSETS = 2 };
 int spfa_device_status(int reset);
 
 /* Measurement aid; no counterpart in the reference.  While both handles are non-NULL
- * (hipEvent_t passed as void*), every forward call records `start` on its stream immediately
- * before, and `stop` immediately after, the launch of the kernel that does the bulk of the
- * call's attention work (the segment kernel when a mask has long rows, else the row kernel), so a
- * benchmark can time that one kernel with hipEventElapsedTime.  Process-wide and not
- * thread-safe: set it, run, read the events, reset it with NULLs. */
+ * (hipEvent_t passed as void*), every forward call MADE BY THE CALLING HOST THREAD attaches
+ * `start` and `stop` to the dispatch of the kernel that does the bulk of the call's attention
+ * work (the segment kernel when a mask has long rows, else the row kernel; the band kernel; the
+ * global rows' tile kernel), so a benchmark can time that one kernel with hipEventElapsedTime.
+ * The pair is kept per host thread (other threads' calls are not affected and do not race on
+ * it): set it, run, read the events, reset it with NULLs. */
 void spfa_set_kernel_events(void* start, void* stop);
-
-/* Measurement aid; no counterpart in the reference.  The gather of the explicit-mask kernels with
- * the arithmetic taken out: for each of the n_idx entries of `idx` (values < n_rows; entries with
- * the top bit set are skipped) one row of `row_bytes` (64, 128, 256 or 512) bytes is loaded from
- * `k` and one from `v`, 16 bytes per lane, `in_flight` (4, 8, 16 or 32) rows of each per lane group
- * issued back to back, by a persistent grid of wg_per_cu (1..8) four-wavefront workgroups per
- * compute unit whose wavefronts pull runs of `chunk` (>= 64) entries off an atomic cursor
- * (`cursor`: 4 bytes of device memory).  Nothing is computed or written.  Timed by the caller
- * with events on `stream`, it gives the rate the memory system sustains for this access pattern
- * at a given working-set size: the ceiling a gather-bound kernel is priced against. */
-int spfa_probe_gather(const void* k, const void* v, int64_t n_rows, int64_t row_bytes,
-                      const uint32_t* idx, int64_t n_idx, int64_t chunk, int wg_per_cu, int in_flight,
-                      void* cursor, void* stream);
 
 /* Rows of an explicit mask with at most this many entries are finished by the row kernels (a
  * lane group or a wavefront per row); longer rows go through the segment kernel.  Exposed so a
@@ -150,9 +138,12 @@ int spfa_csr_forward(const spfa_problem_t* p, const void* row_off, int row_off_b
  * spfa_csr_forward; the scratch is a device array of SPFA_STATIC_SCRATCH_BYTES bytes inside the
  * library (one per device, held until the process ends), and a call calls neither hipMalloc nor
  * hipFree nor any allocating routine.
- *   - Limit: n_batch * spfa_csr_workspace_bytes(n_q, nnz, d, dtype) <= SPFA_STATIC_SCRATCH_BYTES,
- *     else SPFA_ERR_STATIC_LIMIT and nothing is enqueued (16 MiB holds a mask of 131072 rows and
- *     12.8 M entries at d = 64).
+ *   - Limit: spfa_csr_workspace_bytes_batched(n_q, nnz, d, dtype, n_batch) <=
+ *     SPFA_STATIC_SCRATCH_BYTES, else SPFA_ERR_STATIC_LIMIT and nothing is enqueued (16 MiB holds
+ *     a mask of 131072 rows and 12.8 M entries at d = 64; SPFA_DTYPE_F64 problems use no scratch
+ *     and have no limit).
+ *   - The first call on a device looks the array's address up (hipGetSymbolAddress, under a
+ *     mutex); make one call on each device before capturing the entry point in a HIP graph.
  *   - All calls on one device share that device's array: calls that overlap in time on one
  *     device (two streams, two host threads) race; calls in stream order do not.  Nothing needs
  *     clearing between calls. */

@@ -33,8 +33,8 @@ def lib():
     return L
 
 
-def declared_functions():
-    text = open(HEADER).read()
+def declared_functions(header=HEADER):
+    text = open(header).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     return sorted(set(re.findall(r"\b(spfa_[a-z0-9_]+)\s*\(", text)))
 
@@ -44,6 +44,15 @@ def test_every_declared_symbol_is_exported(lib):
     assert len(names) >= 14
     for n in names:
         assert hasattr(lib, n), n
+
+
+def test_probe_header_symbols_are_exported_by_the_probe_library_only(lib):
+    names = declared_functions(os.path.join(ROOT, "include", "spfa_probe.h"))
+    assert names == ["spfa_probe_gather"]
+    probe = ctypes.CDLL(os.path.join(PKG, "libspfa_probe.so"))
+    for n in names:
+        assert hasattr(probe, n), n
+        assert not hasattr(lib, n), "%s belongs to libspfa_probe.so, not to the drop-in library" % n
 
 
 def test_status_strings_carry_reference_texts(lib):

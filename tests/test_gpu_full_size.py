@@ -113,6 +113,57 @@ def test_csr_zipf_n131072(mods):
     assert torch.allclose(l4, l, rtol=1e-5)
 
 
+# ------------------------------------------------------------------ CSR with more than 2^31 entries
+def test_csr_more_than_2_31_entries(mods):
+    """64-bit row offsets that really need their upper half (the reference indexes its rows with
+    size_t offsets, Sparse_FlashAttention_CSR/sp_flatt_csr_kernel.cu:29-30): 2^20 rows of 2048 to
+    2176 distinct columns each, 2.2e9 entries, against 4096 keys at d = 16 in bf16.  q = 0 gives
+    l == row length exactly and out == the mean of the row's V rows; sampled rows of a call with
+    random q against the oracle, among them the rows whose entries straddle position 2^31."""
+    n_q, n_k, d = 1 << 20, 4096, 16
+    dtype = torch.bfloat16
+    free = torch.cuda.mem_get_info()[0]
+    if free < 40 * (1 << 30):
+        pytest.skip("needs about 40 GiB of free device memory for the mask, has %.1f GiB" % (free / 2**30))
+    rows = torch.arange(n_q, device=DEV, dtype=torch.int64)
+    deg = 2048 + rows % 129
+    ro = torch.zeros(n_q + 1, dtype=torch.int64, device=DEV)
+    ro[1:] = torch.cumsum(deg, 0)
+    nnz = int(ro[-1])
+    assert nnz > (1 << 31)
+    ci = torch.empty(nnz, dtype=torch.int32, device=DEV)
+    step = 1 << 15
+    for a in range(0, n_q, step):  # row i lists (17 i + j) mod n_k, j < deg[i]: distinct, unsorted
+        b = min(n_q, a + step)
+        r = torch.repeat_interleave(rows[a:b], deg[a:b])
+        j = torch.arange(int(ro[a]), int(ro[b]), device=DEV, dtype=torch.int64) - ro[r]
+        ci[int(ro[a]):int(ro[b])] = ((17 * r + j) % n_k).to(torch.int32)
+        del r, j
+    ro_t, ci_t = ro.to(torch.uint64), ci.view(torch.uint32)
+    val = torch.empty(0, device=DEV, dtype=dtype)
+    q, k, v = syn.qkv(n_q, d, dtype=dtype, device=DEV, seed=0, n_k=n_k)
+
+    def live(i):
+        return (17 * i + np.arange(2048 + i % 129)) % n_k
+
+    # q == 0: m == 0, l == row length, out == mean of the listed V rows
+    m, l, o = syn.fresh_state(n_q, d, dtype=dtype, device=DEV, state_dtype=torch.float32)
+    mods["spfa_csr"].forward(torch.zeros_like(q), k, v, ro_t, ci_t, val, m, l, o, False)
+    assert torch.all(m == 0) and torch.equal(l, deg.float())
+    ro_c = ro.cpu().numpy()
+    cross = int(np.searchsorted(ro_c, 1 << 31, side="right")) - 1  # the row that holds entry 2^31
+    sample = np.unique(np.concatenate([[0, 1, cross - 1, cross, cross + 1, n_q - 2, n_q - 1],
+                                       rand_rows(n_q, 24, 5)]))
+    vv = np64(v)
+    for i in sample:
+        want = vv[live(int(i))].mean(axis=0)
+        assert np.abs(np64(o[int(i)]) - want).max() <= 2e-3, int(i)
+    # random q: sampled rows against the oracle
+    m, l, o = syn.fresh_state(n_q, d, dtype=dtype, device=DEV, state_dtype=torch.float32)
+    mods["spfa_csr"].forward(q, k, v, ro_t, ci_t, val, m, l, o, False)
+    sample_check(q, k, v, o, m, l, sample, live, dtype)
+
+
 # ------------------------------------------------------------------ dilated masks N=262144 d=128 bf16
 def test_local_1d_dilated_n262144(mods):
     n, d, w, dil = 262144, 128, 256, 2

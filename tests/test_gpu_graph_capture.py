@@ -1,6 +1,9 @@
 """The calls enqueue kernels only (no allocation inside the library, no memset nodes, no host
 synchronisation), so a caller can capture them in a HIP graph.  Each replay is checked against
 the eager result, with eager work and synchronisations between the replays."""
+import ctypes
+import os
+
 import numpy as np
 import pytest
 import torch
@@ -62,3 +65,70 @@ def test_chained_forward_and_backward_replay_from_a_graph(mods):
         torch.cuda.synchronize()
         for name, got, want in zip(("out", "m", "l", "dq", "dk", "dv"), (o, m, l, dq, dk, dv), eager):
             assert torch.allclose(got, want, atol=1e-5, rtol=1e-5), "replay %d: %s differs from the eager run" % (rep, name)
+
+
+def test_static_csr_entry_replays_from_a_graph():
+    """spfa_csr_forward_static (scratch inside the library, nothing allocated) captured after one
+    eager call on the device: every replay equals spfa_csr_forward bit for bit."""
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    lib = ctypes.CDLL(os.path.join(root, "graph-processing-attention-ipdps-2025_amd", "libspfa_hip.so"))
+
+    class Problem(ctypes.Structure):
+        _fields_ = [("q", ctypes.c_void_p), ("k", ctypes.c_void_p), ("v", ctypes.c_void_p),
+                    ("m", ctypes.c_void_p), ("l", ctypes.c_void_p), ("out", ctypes.c_void_p),
+                    ("n_q", ctypes.c_int64), ("n_k", ctypes.c_int64), ("d", ctypes.c_int64),
+                    ("dtype", ctypes.c_int32), ("state_dtype", ctypes.c_int32), ("n_batch", ctypes.c_int64)]
+    lib.spfa_csr_workspace_bytes.restype = ctypes.c_size_t
+    lib.spfa_csr_workspace_bytes.argtypes = [ctypes.c_int64, ctypes.c_int64, ctypes.c_int64, ctypes.c_int]
+    lib.spfa_csr_forward.argtypes = [ctypes.POINTER(Problem), ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p,
+                                     ctypes.c_int64, ctypes.c_int, ctypes.c_void_p, ctypes.c_size_t,
+                                     ctypes.c_void_p]
+    lib.spfa_csr_forward_static.argtypes = [ctypes.POINTER(Problem), ctypes.c_void_p, ctypes.c_int,
+                                            ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_void_p]
+    n, d = 20000, 64
+    q, k, v = syn.qkv(n, d, device=DEV, seed=5)
+    ro, ci = syn.zipf_csr(n, 1.5, 1, 2048, device=DEV, seed=5)  # long rows: segments and merges
+    ro32, ci32 = ro.to(torch.int32), ci.to(torch.int32)
+    nnz = ci.numel()
+    m = torch.empty(n, device=DEV)
+    l = torch.empty(n, device=DEV)
+    o = torch.empty(n, d, device=DEV)
+    prob = Problem(q.data_ptr(), k.data_ptr(), v.data_ptr(), m.data_ptr(), l.data_ptr(), o.data_ptr(),
+                   n, n, d, 0, 0, 1)
+
+    def reset():
+        m.fill_(-float("inf"))
+        l.zero_()
+        o.zero_()
+
+    need = lib.spfa_csr_workspace_bytes(n, nnz, d, 0)
+    ws = torch.empty(need + 256, dtype=torch.uint8, device=DEV)
+    reset()
+    assert lib.spfa_csr_forward(ctypes.byref(prob), ro32.data_ptr(), 4, ci32.data_ptr(), nnz, 0,
+                                (ws.data_ptr() + 255) // 256 * 256, need,
+                                torch.cuda.current_stream().cuda_stream) == 0
+    torch.cuda.synchronize()
+    want = [x.clone() for x in (m, l, o)]
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):  # the eager call that looks the array's address up
+        reset()
+        assert lib.spfa_csr_forward_static(ctypes.byref(prob), ro32.data_ptr(), 4, ci32.data_ptr(), nnz, 0,
+                                           side.cuda_stream) == 0
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        reset()
+        rc = lib.spfa_csr_forward_static(ctypes.byref(prob), ro32.data_ptr(), 4, ci32.data_ptr(), nnz, 0,
+                                         torch.cuda.current_stream().cuda_stream)
+    assert rc == 0
+    for rep in range(3):
+        for x in (m, l, o):
+            x.fill_(77.0)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for name, got, ref in zip(("m", "l", "out"), (m, l, o), want):
+            assert torch.equal(got, ref), "replay %d: %s differs from spfa_csr_forward" % (rep, name)

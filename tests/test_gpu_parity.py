@@ -606,14 +606,17 @@ def test_bigbird_one_call_equals_dense_union(mods, dtype, d, n, w, n_globs):
 @pytest.mark.parametrize("dtype,d", [(torch.bfloat16, 64), (torch.float16, 128), (torch.bfloat16, 32),
                                      (torch.float16, 256), (torch.float32, 64), (torch.float32, 128)])
 @pytest.mark.parametrize("n,w,kind", [(3000, 16, "one"), (3000, 100, "tile"), (2500, 40, "tile+1"),
-                                      (4100, 64, "many"), (2048, 33, "repeats"), (1000, 999, "tile")])
+                                      (4100, 64, "many"), (2048, 33, "repeats"), (1000, 999, "tile"),
+                                      (3300, 48, "most"), (3300, 48, "most+1")])
 def test_bigbird_window_and_listed_tokens_in_one_kernel(mods, dtype, d, n, w, kind):
     """Half types on the tile kernels: the band kernel takes the listed tokens as further keys.  Against
     the dense union mask where every token is listed once, and against the two chained calls (which
     count a token as often as it is listed and drop entries outside [0, n)) otherwise; three problems
     in one call, on top of a state left by an earlier call."""
     rng = np.random.default_rng(n + w)
-    count = {"one": 1, "tile": 64, "tile+1": 65, "many": 200, "repeats": 40}[kind]
+    # ("most": the largest list the band kernel takes as further keys, "most+1": the first one that
+    # runs as window call + global call)
+    count = {"one": 1, "tile": 64, "tile+1": 65, "many": 200, "repeats": 40, "most": 256, "most+1": 257}[kind]
     globs = rng.choice(n, count, replace=False)
     if kind == "repeats":
         globs = np.concatenate([globs, globs[:7], [-3, n, n + 5]])

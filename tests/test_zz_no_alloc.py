@@ -29,6 +29,9 @@ def lib():
     L = ctypes.CDLL(LIB)
     L.spfa_csr_workspace_bytes.restype = ctypes.c_size_t
     L.spfa_csr_workspace_bytes.argtypes = [ctypes.c_int64, ctypes.c_int64, ctypes.c_int64, ctypes.c_int]
+    L.spfa_csr_workspace_bytes_batched.restype = ctypes.c_size_t
+    L.spfa_csr_workspace_bytes_batched.argtypes = [ctypes.c_int64, ctypes.c_int64, ctypes.c_int64, ctypes.c_int,
+                                                   ctypes.c_int64]
     L.spfa_csr_forward.argtypes = [ctypes.POINTER(Problem), ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p,
                                    ctypes.c_int64, ctypes.c_int, ctypes.c_void_p, ctypes.c_size_t,
                                    ctypes.c_void_p]
@@ -77,15 +80,26 @@ def _run_both(lib, n, d, kmax, seed, use_nan):
                               need, stream)
     assert rc == 0
 
+    # a first call (it looks the array's address up, once per device), then the call that is
+    # watched: the device's free memory as the HIP runtime reports it (hipMemGetInfo - it sees a
+    # hipMalloc inside the library, which torch's own allocator statistics would not) must be the
+    # same before and after
+    warm = syn.fresh_state(n, d, device=dev)
+    p = _problem(q, k, v, warm)
+    rc = lib.spfa_csr_forward_static(ctypes.byref(p), ro32.data_ptr(), 4, ci32.data_ptr(), nnz, use_nan,
+                                     stream)
+    assert rc == 0
     got = syn.fresh_state(n, d, device=dev)
     p = _problem(q, k, v, got)
     torch.cuda.synchronize()
-    before = torch.cuda.memory_allocated()
+    free_before = torch.cuda.mem_get_info()[0]
+    torch_before = torch.cuda.memory_allocated()
     rc = lib.spfa_csr_forward_static(ctypes.byref(p), ro32.data_ptr(), 4, ci32.data_ptr(), nnz, use_nan,
                                      stream)
     assert rc == 0
     torch.cuda.synchronize()
-    assert torch.cuda.memory_allocated() == before
+    assert torch.cuda.mem_get_info()[0] == free_before
+    assert torch.cuda.memory_allocated() == torch_before
 
     # the same kernels on the same inputs: identical results, NaN rows included
     for a, b, name in zip(got, ref, ("m", "l", "out")):
@@ -130,3 +144,45 @@ def test_static_entry_rejects_masks_beyond_its_buffer(lib):
     assert rc == SPFA_ERR_STATIC_LIMIT
     torch.cuda.synchronize()
     assert torch.isinf(st[0]).all() and (st[1] == 0).all()
+
+
+@pytest.mark.gpu
+def test_static_entry_limit_is_the_batched_workspace_size(lib):
+    """A batch whose work list is shared fits the array although n_batch times the single-problem
+    size does not; the call runs and agrees with the workspace entry."""
+    dev = "cuda:0"
+    n, d = 400000, 64
+    # many short rows: the shared work list is most of the scratch
+    deg = 1 + torch.arange(n, device=dev) % 6
+    ro, ci = syn.csr_from_degrees(deg, n, torch.Generator(device=dev).manual_seed(21), dev)
+    nnz = ci.numel()
+    one = lib.spfa_csr_workspace_bytes(n, nnz, d, 0)
+    fits = [b for b in range(2, 9) if one * b > STATIC_BYTES >= lib.spfa_csr_workspace_bytes_batched(n, nnz, d, 0, b)]
+    if not fits:
+        pytest.skip("no batch count separates the two sizes for this mask (single problem: %d bytes)" % one)
+    nb = fits[0]
+    batched = lib.spfa_csr_workspace_bytes_batched(n, nnz, d, 0, nb)
+    q, k, v = [torch.stack([syn.qkv(n, d, device=dev, seed=30 + b)[j] for b in range(nb)]) for j in range(3)]
+    ro32, ci32 = ro.to(torch.int32), ci.to(torch.int32)
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def state():
+        return (torch.full((nb, n), -float("inf"), device=dev), torch.zeros(nb, n, device=dev),
+                torch.zeros(nb, n, d, device=dev))
+
+    def problem(st):
+        return Problem(q.data_ptr(), k.data_ptr(), v.data_ptr(), st[0].data_ptr(), st[1].data_ptr(),
+                       st[2].data_ptr(), n, n, d, 0, 0, nb)
+    ws = torch.empty(batched + 256, dtype=torch.uint8, device=dev)
+    ws_ptr = (ws.data_ptr() + 255) // 256 * 256
+    ref = state()
+    p = problem(ref)
+    assert lib.spfa_csr_forward(ctypes.byref(p), ro32.data_ptr(), 4, ci32.data_ptr(), nnz, 0, ws_ptr, batched,
+                                stream) == 0
+    got = state()
+    p = problem(got)
+    assert lib.spfa_csr_forward_static(ctypes.byref(p), ro32.data_ptr(), 4, ci32.data_ptr(), nnz, 0, stream) == 0
+    torch.cuda.synchronize()
+    for a, b, name in zip(got, ref, ("m", "l", "out")):
+        assert torch.equal(a, b), name
+    assert float(got[1].min()) >= 1.0  # every row has its diagonal
