@@ -456,7 +456,7 @@ def measured_traffic(workload, dtype_name):
              "csr_zipf_hbm": "csr_zipf_hbm_n4194304_d64"}
     stem = names.get(workload)
     if stem is None:
-        return None
+        return None, None
     for path in glob.glob(os.path.join(ROOT, "profiles", "%s_%s_pmc.md" % (stem, {"f32": "f32"}.get(dtype_name, dtype_name)))):
         m = re.search(r"^traffic_bytes_per_launch\s*=\s*(\d+)", open(path).read(), re.M)
         if m:
@@ -503,7 +503,9 @@ def bench_backward(a, w, st, dtype, torch, syn, lib):
     name = w["name"]
     explicit = name.startswith(("csr", "coo"))
     flops = 10.0 * d * nnz
-    dense = heads * n * d * (5 * es + 6 * 4)
+    # (a 2-D dilated mask touches only the rows that have a live column)
+    rows_touched = heads * n if (explicit or name == "bigbird") else w["kernel_rows"]
+    dense = rows_touched * d * (5 * es + 6 * 4)
     nnz_gather = nnz if explicit else (w["params"]["csr_nnz"] if name == "bigbird" else 0)
     nnz_tiles = nnz - nnz_gather
     gathered = nnz_gather * 4 * d * es
@@ -511,19 +513,37 @@ def bench_backward(a, w, st, dtype, torch, syn, lib):
     total = dense + gathered + index
     t_s = ms_per_step * 1e-3
     mfma_peak = FP32_PEAK_TFLOPS if a.dtype == "f32" else HALF_PEAK_TFLOPS
-    # what the gather passes can be served at: the published HBM rate when Q, K, V, dO together do
-    # not fit the 256 MiB memory-side cache, else what the same gather without arithmetic
-    # sustains over this K, V and this column list on this device (as for the forward call)
+    # What the gather passes can be served at: the published HBM rate when Q, K, V, dO together do
+    # not fit the 256 MiB memory-side cache, else what the same gather without arithmetic sustains
+    # on this device - for the query pass over K, V and the mask's entries in row order (as for
+    # the forward call), for the key pass over Q, dO and the entries in column order (a mask with
+    # a few very long rows makes that a gather from a small hot set of Q / dO rows, which the L2
+    # serves: its ceiling is well above the query pass's).
     ws_bytes = 4 * w["k"].numel() * es
-    gather = measured_gather_ceiling(lib, w, torch) if nnz_gather else None
-    if nnz_gather and ws_bytes > (256 << 20) or gather is None:
-        gather_peak, gather_src = HBM_PEAK_GBS, "MI355X HBM3E, published"
+    gq = gk = None
+    if nnz_gather and ws_bytes <= (256 << 20):
+        gq = measured_gather_ceiling(lib, w, torch)
+        if w.get("csr") is not None:
+            ro_m, ci_m = w["csr"]
+            rows_of = torch.repeat_interleave(torch.arange(ro_m.numel() - 1, device=ci_m.device), ro_m[1:] - ro_m[:-1])
+            idx_t = rows_of[torch.argsort(ci_m, stable=True)].to(torch.int32).contiguous()
+        else:
+            r_m, c_m = w["coo"]
+            idx_t = r_m[torch.argsort(c_m, stable=True)].to(torch.int32).contiguous()
+        gk = measured_gather_ceiling(lib, w, torch, tensors=(w["q"], d_out), idx=idx_t)
+        del idx_t
+    if gq is None or gk is None:
+        peak_q = peak_k = HBM_PEAK_GBS
+        gather_src = "MI355X HBM3E, published"
         gather_bound = "hbm"
     else:
-        gather_peak = gather["GBs"]
-        gather_src = "measured on this device: the same gather without arithmetic (spfa_probe_gather)"
+        peak_q, peak_k = gq["GBs"], gk["GBs"]
+        gather_src = "measured on this device: the same gathers without arithmetic (spfa_probe_gather), " \
+                     "query pass over K, V by row-ordered entries, key pass over Q, dO by column-ordered entries"
         gather_bound = "l2" if ws_bytes <= (4 << 20) else "infinity_cache"
-    gather_ms = (gathered + index) / (gather_peak * 1e9) * 1e3 if nnz_gather else 0.0
+    half_bytes = (gathered + index) / 2.0
+    gather_ms = (half_bytes / (peak_q * 1e9) + half_bytes / (peak_k * 1e9)) * 1e3 if nnz_gather else 0.0
+    gather_peak = (gathered + index) / (gather_ms * 1e-3) / 1e9 if nnz_gather else None
     tile_flops = 10.0 * d * nnz_tiles
     dense_ms = dense / (HBM_PEAK_GBS * 1e9) * 1e3
     mfma_ms = tile_flops / (mfma_peak * 1e12) * 1e3
@@ -554,13 +574,16 @@ def bench_backward(a, w, st, dtype, torch, syn, lib):
                 "kernel": "whole call: " + ", ".join(x for x in (gather_kernels if nnz_gather else None,
                                                                  tile_kernels if nnz_tiles else None) if x),
                 "roofline_time_ms": roof_ms, "gather_time_ms": gather_ms, "hbm_time_ms": dense_ms,
-                "mfma_time_ms": mfma_ms, "gather_peak_GBs": gather_peak if nnz_gather else None,
+                "mfma_time_ms": mfma_ms, "gather_peak_GBs": gather_peak,
+                "gather_peak_query_pass_GBs": peak_q if nnz_gather else None,
+                "gather_peak_key_pass_GBs": peak_k if nnz_gather else None,
                 "gather_peak_source": gather_src if nnz_gather else None,
                 "working_set_bytes": ws_bytes, "algorithmic_bytes": total, "gathered_bytes": gathered,
                 "gathered_positions": nnz_gather, "tile_positions": nnz_tiles,
                 "executed_over_counted_tile_flops": 1.4}
-    if gather is not None:
-        roofline["measured_gather"] = gather["how"]
+    if gq is not None and gk is not None:
+        roofline["measured_gather_query_pass"] = gq["how"]
+        roofline["measured_gather_key_pass"] = gk["how"]
     out = {
         "metric": "masked-attn backward GFLOP/s (10*d per live position) + algorithmic GB/s",
         "value": flops / (ms_per_step * 1e-3) / 1e9, "unit": "GFLOP/s",
@@ -596,16 +619,18 @@ def measured_copy_bandwidth(torch, mib=1024, reps=5):
     return 2.0 * src.numel() * 4 / (best * 1e-3) / 1e9
 
 
-def measured_gather_ceiling(lib, w, torch, min_entries=8_000_000, reps=5):
+def measured_gather_ceiling(lib, w, torch, min_entries=8_000_000, reps=5, tensors=None, idx=None):
     """What the memory system delivers to the explicit-mask access pattern at this working set:
     spfa_probe_gather (the gather of segments_kernel without any arithmetic) over the workload's
     own K, V and column list (the list is repeated up to min_entries so that the launch is long
-    enough to time).  Best of a few launch shapes.  None when the row size has no probe."""
-    k, v = w["k"], w["v"]
+    enough to time); `tensors` / `idx`: another pair of row tensors and another list (the key
+    pass of the gradients gathers Q and dO rows by the mask's entries in column order).  Best of
+    a few launch shapes.  None when the row size has no probe."""
+    k, v = tensors if tensors is not None else (w["k"], w["v"])
     if k.dim() != 2:
         k, v = k[-1], v[-1]
     row_bytes = k.shape[1] * k.element_size()
-    idx = w.get("probe_idx")
+    idx = w.get("probe_idx") if idx is None else idx
     if idx is None or row_bytes not in (64, 128, 256, 512) or idx.numel() == 0:
         return None
     if idx.numel() < min_entries:
