@@ -1714,6 +1714,520 @@ __global__ __launch_bounds__(256, 2) void band_dma_f32_kernel(TileArgs a) {
   }
 }
 
+// ---------------------------------------------------------------------------------------
+// Global mask, half types, at most 64 listed tokens: every other token against the listed ones
+// ---------------------------------------------------------------------------------------
+// The column pass of the global mask (queries = the tokens that are not listed, keys = the listed
+// tokens outside the query's window, Sparse_FlashAttention_Global_No_Local/
+// sp_flatt_global_no_local_kernel.cu:38-64,146-162) when all keys fit one 64-key tile: there is no
+// running state across key tiles, so a query tile is one S product, one softmax and one P V
+// product, and everything that does not depend on the query tile is set up once per workgroup:
+//   - the listed tokens' K and V rows are gathered into LDS (band_dma_kernel's layout and loads)
+//     and read from there ONCE, into registers: both matrix operands (K rows; V^T through the
+//     transposing read) stay in registers for every query tile of the workgroup, as do the listed
+//     tokens themselves in the order of the score registers;
+//   - a wavefront's 32 consecutive Q rows are one contiguous piece of memory: the load
+//     instructions write it straight into the wavefront's own LDS buffer (1 KB per instruction,
+//     every cache line whole), two buffers, the next tile's rows asked for before the current
+//     tile is worked on; no barrier in the tile loop;
+//   - almost no wavefront has a listed token within reach of its 32 queries (64 tokens among a
+//     million): one compare per lane (lane = key slot) and a ballot tell, and only then are the
+//     window and "query is listed itself" tests made per score;
+//   - the row sums come out of the matrix pipe (an all-ones operand), which idles here;
+//   - finished rows leave through the wavefront's LDS buffer as whole rows, 1 KB per store
+//     instruction (76 -> 61 us for 1 M tokens at d = 64 without this, 51 us with it: the rate of
+//     a plain device copy of the same bytes); rows with an incoming state, and wavefronts near a
+//     listed token, take the general write-back.
+// A persistent grid; a workgroup walks query tiles blockIdx.x, blockIdx.x + gridDim.x, ...
+template <typename T, int D>
+__global__ __launch_bounds__(256, 2) void global_cols_dma_kernel(TileArgs a) {
+  using C = BandDmaCfg<T, D, 64>;
+  constexpr int BN = 64, EB = C::EB, ROWB = C::ROWB, RPC = C::RPC, CH = C::CH, TILE_B = C::TILE_B;
+  constexpr int QR = C::QREGS, NI = C::NI;
+  constexpr int QB = 32 * ROWB;       // bytes of a wavefront's 32 Q rows
+  constexpr int QNI = QB / 1024;      // load instructions for them
+  constexpr int QROWS = 1024 / ROWB;  // rows per load instruction
+  static_assert(sizeof(T) == 2 && (D == 32 || D == 64), "half types, d = 32 or 64");
+  __shared__ __attribute__((aligned(1024))) char lds[2 * TILE_B + 4 * 2 * QB];
+  __shared__ int gtok_s[BN];  // token of every key slot (-1: no key)
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int r = lane & 31, h = lane >> 5;
+  const int64_t bb = blockIdx.y;             // one grid row per problem
+  const int64_t tok_base = bb * a.n;          // first row of this problem
+  const char* Qp = (const char*)a.t.q + tok_base * ROWB;
+  const char* Kp = (const char*)a.t.k;
+  const char* Vp = (const char*)a.t.v;
+  const float sc = 1.4426950408889634f / sqrtf((float)D);
+  const int n = (int)a.n, ng = (int)a.n_globs;
+  const int wlim = (int)(a.w < (int64_t)0x3fffffff ? a.w : (int64_t)0x3fffffff);
+  const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)lds;
+  constexpr int VPER = CH / 4 > 0 ? CH / 4 : 1;
+
+  // ---- the key tile, once: gathered by token, band_dma_kernel's chunk permutations
+  {
+    constexpr int RPI = 4096 / ROWB;
+    const int j0 = (wave * 1024 + lane * 16) / ROWB, p0 = ((wave * 1024 + lane * 16) % ROWB) / 16;
+#pragma unroll
+    for (int it = 0; it < NI; it++) {
+      const int j = j0 + it * RPI;
+      int g = -1;
+      if (j < ng) g = listed_token(a.globs[j], a.n);
+      if (p0 == 0) gtok_s[j] = g;
+      const uint32_t row_byte = (uint32_t)((tok_base + (g < 0 ? 0 : g)) * (int64_t)ROWB);
+      const uint32_t ko = row_byte + (uint32_t)((p0 ^ C::kperm(j)) * 16);
+      const uint32_t vo = row_byte + (uint32_t)((p0 ^ (4 * ((j / RPC) % VPER))) * 16);
+      const uint32_t lds_k = lds_base + (uint32_t)((4 * it + wave) * 1024);
+      asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                   :: "v"(ko), "s"(Kp), "s"(lds_k) : "memory", "m0");
+      asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                   :: "v"(vo), "s"(Vp), "s"(lds_k + (uint32_t)TILE_B) : "memory", "m0");
+    }
+  }
+
+  // ---- Q rows of a query tile: instruction i of this wavefront fills rows QROWS*i .. of its
+  // buffer; this lane's 16 bytes are row jq, chunk position pq, i.e. source chunk pq ^ kperm(row)
+  // (the layout of a K tile: the B operand reads below are the A operand reads of band_dma_kernel)
+  const int jq = lane * 16 / ROWB, pq = (lane * 16 % ROWB) / 16;
+  char* const qbuf = lds + 2 * TILE_B + wave * 2 * QB;
+  const uint32_t qbuf_lds = lds_base + (uint32_t)(2 * TILE_B + wave * 2 * QB);
+  const int n_tiles = (n + 127) / 128;
+  auto request_q = [&](int qt, int buf) __attribute__((always_inline)) {
+    const int tw0 = qt * 128 + 32 * wave;
+    const char* src = Qp + (int64_t)tw0 * ROWB;  // scalar
+#pragma unroll
+    for (int i = 0; i < QNI; i++) {
+      const int j = QROWS * i + jq;
+      // rows past the last token repeat the last token (their lanes never write)
+      int row = j;
+      if (tw0 + 31 >= n) row = tw0 + j < n ? j : n - 1 - tw0;
+      const uint32_t off = (uint32_t)(row * ROWB + ((pq ^ C::kperm(j)) * 16));
+      const uint32_t dst = qbuf_lds + (uint32_t)(buf * QB + i * 1024);
+      asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                   :: "v"(off), "s"(src), "s"(dst) : "memory", "m0");
+    }
+  };
+  int qt = (int)blockIdx.x;
+  if (qt < n_tiles && qt * 128 + 32 * wave < n) request_q(qt, 0);
+  SPFA_WAIT_VMCNT(0);
+  __syncthreads();  // the key tile and the token table are complete
+
+  // ---- operands that do not depend on the query tile, read once
+  uint4v ka[2][QR], va[2][2 * EB];
+  int tokv[2][16];
+  {
+    typedef short s16x4 __attribute__((ext_vector_type(4)));
+    typedef short s16x8 __attribute__((ext_vector_type(8)));
+    typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+    const int x = (lane & 15) >> 2, y = lane & 3, r_hi = (lane >> 4) & 1;
+    const int key = 4 * h + x;
+    const int gx = (key / RPC) % VPER;
+    const int common = TILE_B + key * ROWB + (2 * r_hi + (y >> 1)) * 16 + (y & 1) * 8;
+#pragma unroll
+    for (int jb = 0; jb < 2; jb++) {
+#pragma unroll
+      for (int ks = 0; ks < QR; ks++)
+        ka[jb][ks] = *reinterpret_cast<const uint4v*>(lds + (32 * jb + r) * ROWB +
+                                                     (((2 * ks + h) ^ C::kperm(32 * jb + r)) * 16));
+#pragma unroll
+      for (int sl = 0; sl < 2; sl++)
+#pragma unroll
+        for (int eb = 0; eb < EB; eb++) {
+          const char* va_p = lds + (32 * jb + 16 * sl) * ROWB + common + 64 * (eb ^ gx);
+          const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)va_p);
+          const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(va_p + 8 * ROWB));
+          const s16x8 both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+          va[jb][sl * EB + eb] = __builtin_bit_cast(uint4v, both);
+        }
+#pragma unroll
+      for (int v = 0; v < 16; v++) tokv[jb][v] = gtok_s[32 * jb + 8 * (v / 4) + 4 * h + (v % 4)];
+    }
+  }
+  const int tok_lane = gtok_s[lane];  // lane = key slot
+  const bool all_keys = __builtin_amdgcn_ballot_w64(tok_lane < 0) == 0;
+  const uint32_t one2 = __is_same(T, bf16) ? 0x3f803f80u : 0x3c003c00u;
+  const uint4v ones = {one2, one2, one2, one2};
+  const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  const bool sf = a.t.state_f32 != 0;
+  const int kq_adr = r * ROWB;  // B operand of step ks: row r, chunk (2*ks + h) ^ kperm(r)
+
+  int buf = 0;
+  for (; qt < n_tiles; qt += (int)gridDim.x, buf ^= 1) {
+    const int tw0 = qt * 128 + 32 * wave;
+    const int qn = qt + (int)gridDim.x;
+    // this tile's rows have landed (asked for a whole tile ago); the next tile's are asked for now
+    SPFA_WAIT_VMCNT(0);
+    asm volatile("" ::: "memory");  // (the reads of the buffer below stay behind the wait)
+    if (qn < n_tiles && qn * 128 + 32 * wave < n) request_q(qn, buf ^ 1);
+    if (tw0 >= n) continue;  // (a wavefront past the end: its workgroup has no barrier to keep)
+    const int tq = tw0 + r;
+    const bool q_ok = tq < n;
+    const int64_t q_row = tok_base + (q_ok ? tq : n - 1);
+    // the row's incoming state, long before the write-back needs it
+    const uint32_t l_raw = load_state_raw<T>(a.t.l, q_row, sf);
+    const uint32_t m_raw = load_state_raw<T>(a.t.m, q_row, sf);
+
+    uint4v qh[QR];
+    char* qb = qbuf + buf * QB;
+#pragma unroll
+    for (int ks = 0; ks < QR; ks++)
+      qh[ks] = *reinterpret_cast<const uint4v*>(qb + kq_adr + (((2 * ks + h) ^ C::kperm(r)) * 16));
+    f32x16 s[2];
+#pragma unroll
+    for (int jb = 0; jb < 2; jb++) {
+      s[jb] = zero16;
+#pragma unroll
+      for (int ks = 0; ks < QR; ks++) s[jb] = mfma16<T>(ka[jb][ks], qh[ks], s[jb]);
+    }
+    // Is any listed token within reach of one of this wavefront's queries (inside a window, or
+    // a query itself)?  Else every pair of the tile is live.
+    const bool near = (uint32_t)(tok_lane - tw0 + wlim) <= (uint32_t)(31 + 2 * wlim) && tok_lane >= 0;
+    bool q_plain = q_ok;
+    if (__builtin_expect(!all_keys || __builtin_amdgcn_ballot_w64(near) != 0, 0)) {
+      q_plain = q_ok && !bit_is_set(a.gbits, tq);
+      const uint32_t d0 = (uint32_t)wlim - (uint32_t)tq, w2 = 2u * (uint32_t)wlim;
+#pragma unroll
+      for (int jb = 0; jb < 2; jb++)
+#pragma unroll
+        for (int v = 0; v < 16; v++) {
+          const int tok = tokv[jb][v];
+          const bool ok = q_plain && tok >= 0 && ((uint32_t)tok + d0 > w2);
+          s[jb][v] = ok ? s[jb][v] : kNegInf;
+        }
+    }
+    float mx = s[0][0];
+#pragma unroll
+    for (int jb = 0; jb < 2; jb++)
+#pragma unroll
+      for (int v = jb == 0 ? 1 : 0; v < 16; v++) mx = fmaxf(mx, s[jb][v]);
+    const float m2 = fmaxf(mx, shfl_xor_f32(mx, 32)) * sc;  // row maximum, log2 units
+    const float neg_m = (m2 > kNegInf) ? -m2 : 0.f;
+    f32x16 o[EB], lsum = zero16;
+#pragma unroll
+    for (int eb = 0; eb < EB; eb++) o[eb] = zero16;
+#pragma unroll
+    for (int jb = 0; jb < 2; jb++) {
+#pragma unroll
+      for (int v = 0; v < 16; v++)
+        s[jb][v] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[jb][v], sc, neg_m));  // exp2(-inf) = 0
+#pragma unroll
+      for (int sl = 0; sl < 2; sl++) {
+        uint4v pb;
+#pragma unroll
+        for (int x = 0; x < 4; x++) pb[x] = pack2<T>(s[jb][8 * sl + 2 * x], s[jb][8 * sl + 2 * x + 1]);
+#pragma unroll
+        for (int eb = 0; eb < EB; eb++) o[eb] = mfma16<T>(va[jb][sl * EB + eb], pb, o[eb]);
+        lsum = mfma16<T>(ones, pb, lsum);
+      }
+    }
+    const float l = lsum[0];  // (summed over both halves of the wavefront by the product)
+    const float l_in = state_from_raw<T>(l_raw, sf);
+    // Every row of the wavefront is written and none has an incoming state (the common case):
+    // the rows go through the wavefront's LDS buffer (its Q rows are in registers by now) and
+    // leave as whole rows, 1 KB per store instruction, instead of 32-byte pieces of 32 rows.
+    const bool plain_rows = q_plain == q_ok && l > 0.f && l_in == 0.f;
+    if (__builtin_amdgcn_ballot_w64(!plain_rows) == 0) {
+      const float inv = 1.f / l;
+      typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+#pragma unroll
+      for (int eb = 0; eb < EB; eb++)
+#pragma unroll
+        for (int g4 = 0; g4 < 4; g4++) {
+          u32x2 y;
+          y[0] = pack2<T>(o[eb][4 * g4] * inv, o[eb][4 * g4 + 1] * inv);
+          y[1] = pack2<T>(o[eb][4 * g4 + 2] * inv, o[eb][4 * g4 + 3] * inv);
+          // element 32*eb + 8*g4 + 4*h: chunk 4*eb + g4 of the row (stored at that ^ row mod 8 ... CH), half h
+          const int pos = (4 * eb + g4) ^ (r & (CH - 1));
+          *reinterpret_cast<u32x2*>(qb + r * ROWB + pos * 16 + 8 * h) = y;
+        }
+      if (h == 0 && q_ok) {
+        store_state<T>(a.t.m, q_row, m2 * 0.6931471805599453f, sf);
+        store_state<T>(a.t.l, q_row, l, sf);
+      }
+      char* orow0 = (char*)a.t.out + (tok_base + tw0) * (int64_t)ROWB;
+#pragma unroll
+      for (int i = 0; i < QNI; i++) {
+        const int row = QROWS * i + jq;
+        const uint4v piece = *reinterpret_cast<const uint4v*>(qb + row * ROWB + ((pq ^ (row & (CH - 1))) * 16));
+        if (tw0 + row < n) *reinterpret_cast<uint4v*>(orow0 + row * ROWB + pq * 16) = piece;
+      }
+      continue;
+    }
+    if (q_plain && l > 0.f)
+      tile_write_row<T, D>(a.t, q_row, h, m2, l, o, 1.f, true, l_in, state_from_raw<T>(m_raw, sf));
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// Global mask, half types, at most 64 listed tokens: the listed tokens' rows against everything
+// ---------------------------------------------------------------------------------------
+// The row pass of the global mask (queries = the distinct listed tokens, keys = every token
+// outside the query's window) is a stream of K and V read once against queries that fit in
+// registers, with next to no arithmetic per byte, so it is written as independent wavefronts
+// instead of workgroups in step: a workgroup owns one split of the key range (as in
+// tile_kernel<.., kTileGlobalRows>), its four wavefronts take 32-key blocks in turn, and each
+// wavefront has its own two LDS buffers that the load instructions fill (a block is 32
+// consecutive rows: one contiguous piece of K and one of V, 1 KB per instruction); no barrier in
+// the loop, the next block is asked for before the current one is worked on.  Both 32-query
+// blocks are computed from one read of a block's operands.  The running maximum is a reference
+// with slack as in band_dma_kernel; row sums come out of the matrix pipe.  At the end the four
+// wavefronts are folded through LDS and the workgroup writes one partial (m, l, acc) per query
+// for global_rows_merge_kernel.
+template <typename T, int D>
+__global__ __launch_bounds__(256, 2) void global_rows_dma_kernel(TileArgs a) {
+  using C = BandDmaCfg<T, D, 64>;
+  constexpr int EB = C::EB, ROWB = C::ROWB, RPC = C::RPC, CH = C::CH, QR = C::QREGS;
+  constexpr int BB = 32 * ROWB;       // bytes of a 32-row block of K (or V)
+  constexpr int BNI = BB / 1024;      // load instructions per block and matrix
+  constexpr int BROWS = 1024 / ROWB;  // rows per load instruction
+  constexpr int VPER = CH / 4 > 0 ? CH / 4 : 1;
+  constexpr int STAGE_B = 2 * BB;     // K block then V block
+  constexpr int XR = EB * 16 + 3;     // floats per lane of a folded state
+  static_assert(sizeof(T) == 2 && (D == 32 || D == 64), "half types, d = 32 or 64");
+  static_assert(2 * XR * kWave * 4 <= 4 * 2 * STAGE_B, "the fold does not fit the block buffers");
+  __shared__ __attribute__((aligned(1024))) char lds[4 * 2 * STAGE_B];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int r = lane & 31, h = lane >> 5;
+  // grid: [problem][key split]
+  const int64_t per_problem = (int64_t)gridDim.x / a.t.n_batch;
+  const int64_t bb = blockIdx.x / per_problem;
+  const int64_t split = blockIdx.x - bb * per_problem;
+  const int nq = (int)*a.n_uq;
+  const int n = (int)a.n;
+  const int u_lo = (int)(split * a.key_run);
+  const int u_hi = u_lo + (int)a.key_run < n ? u_lo + (int)a.key_run : n;
+  if (u_lo >= u_hi || nq <= 0) return;
+  const int64_t tok_base = bb * a.n;
+  const char* Kp = (const char*)a.t.k + tok_base * ROWB;
+  const char* Vp = (const char*)a.t.v + tok_base * ROWB;
+  const float sc = 1.4426950408889634f / sqrtf((float)D);
+  const float inv_sc = sqrtf((float)D) * 0.6931471805599453f;
+  const int wlim = (int)(a.w < (int64_t)0x3fffffff ? a.w : (int64_t)0x3fffffff);
+  const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)lds;
+  char* const wbuf = lds + wave * 2 * STAGE_B;
+  const uint32_t wbuf_lds = lds_base + (uint32_t)(wave * 2 * STAGE_B);
+  const bool two = nq > 32;  // a second block of queries
+
+  // ---- block loads: instruction i fills rows BROWS*i .. of the block; this lane's 16 bytes are
+  // row jl, chunk position pl of it (K and V with band_dma_kernel's chunk permutations)
+  const int jl = lane * 16 / ROWB, pl = (lane * 16 % ROWB) / 16;
+  auto request = [&](int ub, int stage) __attribute__((always_inline)) {
+    const char* ksrc = Kp + (int64_t)ub * ROWB;  // scalar
+    const char* vsrc = Vp + (int64_t)ub * ROWB;
+#pragma unroll
+    for (int i = 0; i < BNI; i++) {
+      const int j = BROWS * i + jl;
+      // rows past the last token repeat the last token (finite values; they are masked out)
+      int row = j;
+      if (ub + 31 >= n) row = ub + j < n ? j : n - 1 - ub;
+      const uint32_t ko = (uint32_t)(row * ROWB + ((pl ^ C::kperm(j)) * 16));
+      const uint32_t vo = (uint32_t)(row * ROWB + ((pl ^ (4 * ((j / RPC) % VPER))) * 16));
+      const uint32_t dst = wbuf_lds + (uint32_t)(stage * STAGE_B + i * 1024);
+      asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                   :: "v"(ko), "s"(ksrc), "s"(dst) : "memory", "m0");
+      asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                   :: "v"(vo), "s"(vsrc), "s"(dst + (uint32_t)BB) : "memory", "m0");
+    }
+  };
+  const int n_blk = (u_hi - u_lo + 31) / 32;
+  if (wave < n_blk) request(u_lo + 32 * wave, 0);
+
+  // ---- the queries: Q^T operands of both 32-query blocks, kept in registers
+  int q_tok[2];
+  bool q_ok[2];
+  uint4v qh[2][QR];
+#pragma unroll
+  for (int qb = 0; qb < 2; qb++) {
+    const int tq = 32 * qb + r;
+    q_ok[qb] = tq < nq;
+    q_tok[qb] = a.uq[q_ok[qb] ? tq : nq - 1];
+    const T* qrow = (const T*)a.t.q + (tok_base + q_tok[qb]) * D;
+#pragma unroll
+    for (int ks = 0; ks < QR; ks++) qh[qb][ks] = *reinterpret_cast<const uint4v*>(qrow + 16 * ks + 8 * h);
+  }
+
+  // ---- operand addresses inside a stage (bytes): K block row r, chunk 2*ks + h; V as in
+  // band_dma_kernel (a group of 16 lanes reads 4 keys x 16 columns transposed)
+  int kadr[QR], vadr[EB];
+#pragma unroll
+  for (int ks = 0; ks < QR; ks++) kadr[ks] = r * ROWB + (((2 * ks + h) ^ C::kperm(r)) * 16);
+  {
+    const int x = (lane & 15) >> 2, y = lane & 3, r_hi = (lane >> 4) & 1;
+    const int key = 4 * h + x;
+    const int gx = (key / RPC) % VPER;
+    const int common = BB + key * ROWB + (2 * r_hi + (y >> 1)) * 16 + (y & 1) * 8;
+#pragma unroll
+    for (int eb = 0; eb < EB; eb++) vadr[eb] = common + 64 * (eb ^ gx);
+  }
+
+  constexpr float kSlack = 8.f;
+  f32x16 o[2][EB], lsum[2];
+  float m[2], neg_m[2], thr_raw[2], mt_raw[2];
+#pragma unroll
+  for (int qb = 0; qb < 2; qb++) {
+#pragma unroll
+    for (int eb = 0; eb < EB; eb++)
+#pragma unroll
+      for (int v = 0; v < 16; v++) o[qb][eb][v] = 0.f;
+#pragma unroll
+    for (int v = 0; v < 16; v++) lsum[qb][v] = 0.f;
+    m[qb] = kNegInf;
+    neg_m[qb] = 0.f;
+    thr_raw[qb] = kNegInf;
+    mt_raw[qb] = kNegInf;
+  }
+  const uint32_t one2 = __is_same(T, bf16) ? 0x3f803f80u : 0x3c003c00u;
+  const uint4v ones = {one2, one2, one2, one2};
+  const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  typedef short s16x4 __attribute__((ext_vector_type(4)));
+  typedef short s16x8 __attribute__((ext_vector_type(8)));
+  typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+
+  int stage = 0;
+  for (int blk = wave; blk < n_blk; blk += 4, stage ^= 1) {
+    const int ub = u_lo + 32 * blk;
+    // this block has landed (asked for a block ago); the next one is asked for now, into the
+    // buffer the previous block has left
+    SPFA_WAIT_VMCNT(0);
+    asm volatile("" ::: "memory");
+    if (blk + 4 < n_blk) request(ub + 128, stage ^ 1);
+    const char* tb = wbuf + stage * STAGE_B;
+    uint4v ka[QR], va[2 * EB];
+#pragma unroll
+    for (int ks = 0; ks < QR; ks++) ka[ks] = *reinterpret_cast<const uint4v*>(tb + kadr[ks]);
+#pragma unroll
+    for (int sl = 0; sl < 2; sl++)
+#pragma unroll
+      for (int eb = 0; eb < EB; eb++) {
+        const char* va_p = tb + 16 * sl * ROWB + vadr[eb];
+        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)va_p);
+        const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(va_p + 8 * ROWB));
+        const s16x8 both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        va[sl * EB + eb] = __builtin_bit_cast(uint4v, both);
+      }
+    const bool partial = ub + 32 > u_hi;
+#pragma unroll
+    for (int qb = 0; qb < 2; qb++) {
+      if (qb == 1 && !two) break;
+      f32x16 s = zero16;
+#pragma unroll
+      for (int ks = 0; ks < QR; ks++) s = mfma16<T>(ka[ks], qh[qb][ks], s);
+      // keys are the tokens ub .. ub+31: live for every query unless the block touches the window
+      // of one of this block's query tokens, runs past the last key, or the query does not exist
+      const bool hit = !q_ok[qb] || ((ub + 31 + wlim >= q_tok[qb]) && (ub <= q_tok[qb] + wlim));
+      if (__builtin_expect(partial || __builtin_amdgcn_ballot_w64(hit) != 0, 0)) {
+        const uint32_t d0 = (uint32_t)(ub - q_tok[qb]) + (uint32_t)wlim, w2 = 2u * (uint32_t)wlim;
+        const int rem = u_hi - ub;
+#pragma unroll
+        for (int v = 0; v < 16; v++) {
+          const int j = 8 * (v / 4) + 4 * h + (v % 4);
+          const bool ok = q_ok[qb] && (d0 + (uint32_t)j > w2) && j < rem;
+          s[v] = ok ? s[v] : kNegInf;
+        }
+      }
+      float mx = mt_raw[qb];
+#pragma unroll
+      for (int v = 0; v < 16; v += 2) mx = fmaxf(fmaxf(mx, s[v]), s[v + 1]);
+      mt_raw[qb] = mx;
+      if (__builtin_expect(__builtin_amdgcn_ballot_w64(mx > thr_raw[qb]) != 0, 0)) {
+        const float mp = fmaxf(mx, shfl_xor_f32(mx, 32)) * sc;
+        const float m_new = (mp > m[qb] + kSlack) ? mp : m[qb];
+        const float alpha = (m[qb] > kNegInf) ? __builtin_amdgcn_exp2f(m[qb] - m_new) : 0.f;
+        m[qb] = m_new;
+        neg_m[qb] = (m_new > kNegInf) ? -m_new : 0.f;
+        thr_raw[qb] = (m_new + kSlack) * inv_sc;
+        lsum[qb][0] *= alpha;
+#pragma unroll
+        for (int eb = 0; eb < EB; eb++)
+#pragma unroll
+          for (int v = 0; v < 16; v++) o[qb][eb][v] *= alpha;
+      }
+#pragma unroll
+      for (int v = 0; v < 16; v++)
+        s[v] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[v], sc, neg_m[qb]));  // exp2(-inf) = 0
+#pragma unroll
+      for (int sl = 0; sl < 2; sl++) {
+        uint4v pb;
+#pragma unroll
+        for (int x = 0; x < 4; x++) pb[x] = pack2<T>(s[8 * sl + 2 * x], s[8 * sl + 2 * x + 1]);
+#pragma unroll
+        for (int eb = 0; eb < EB; eb++) o[qb][eb] = mfma16<T>(va[sl * EB + eb], pb, o[qb][eb]);
+        lsum[qb] = mfma16<T>(ones, pb, lsum[qb]);
+      }
+    }
+  }
+
+  // ---- fold the four wavefronts (same queries, different key blocks) through LDS, 2, 3 into
+  // 0, 1 and then 1 into 0, one block of queries at a time; then the partial result of this split
+  SPFA_WAIT_VMCNT(0);
+#pragma unroll
+  for (int qb = 0; qb < 2; qb++) {
+    if (qb == 1 && !two) break;
+    float l = lsum[qb][0];
+    float mt = fmaxf(mt_raw[qb], shfl_xor_f32(mt_raw[qb], 32)) * sc;  // true maximum, log2 units
+    float mq = m[qb];
+    for (int fs = 2; fs >= 1; fs >>= 1) {
+      const bool gives = wave >= fs && wave < 2 * fs;
+      const bool takes = wave < fs;
+      float* xs = reinterpret_cast<float*>(lds) + (size_t)(gives ? wave - fs : wave) * XR * kWave + lane;
+      __syncthreads();
+      if (gives) {
+#pragma unroll
+        for (int eb = 0; eb < EB; eb++)
+#pragma unroll
+          for (int v = 0; v < 16; v++) xs[(eb * 16 + v) * kWave] = o[qb][eb][v];
+        xs[(EB * 16) * kWave] = mq;
+        xs[(EB * 16 + 1) * kWave] = l;
+        xs[(EB * 16 + 2) * kWave] = mt;
+      }
+      __syncthreads();
+      if (takes) {
+        const float m2 = xs[(EB * 16) * kWave], l2 = xs[(EB * 16 + 1) * kWave];
+        mt = fmaxf(mt, xs[(EB * 16 + 2) * kWave]);
+        const float m_new = fmaxf(mq, m2);
+        if (m_new > kNegInf) {
+          const float fa = __builtin_amdgcn_exp2f(mq - m_new), fb = __builtin_amdgcn_exp2f(m2 - m_new);
+          l = l * fa + l2 * fb;
+#pragma unroll
+          for (int eb = 0; eb < EB; eb++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) o[qb][eb][v] = o[qb][eb][v] * fa + xs[(eb * 16 + v) * kWave] * fb;
+          mq = m_new;
+        }
+      }
+    }
+    if (wave == 0 && q_ok[qb]) {
+      // relative to the true maximum: (m, l, o) -> (mt, l * 2^(m - mt), o * 2^(m - mt)); an empty
+      // split is (-inf, 0, 0)
+      const int64_t slot = (bb * a.n_globs + (32 * qb + r)) * a.n_split + split;
+      const bool any = l > 0.f;
+      const float shrink = any ? __builtin_amdgcn_exp2f(mq - mt) : 0.f;
+      float* prow = a.pacc + slot * D;
+#pragma unroll
+      for (int eb = 0; eb < EB; eb++)
+#pragma unroll
+        for (int g4 = 0; g4 < 4; g4++) {
+          float4v y = {0.f, 0.f, 0.f, 0.f};
+          if (any) {
+#pragma unroll
+            for (int i = 0; i < 4; i++) y[i] = o[qb][eb][4 * g4 + i] * shrink;
+          }
+          *reinterpret_cast<float4v*>(prow + 32 * eb + 8 * g4 + 4 * h) = y;
+        }
+      if (h == 0) {
+        a.pm[slot] = any ? mt * 0.6931471805599453f : kNegInf;
+        a.pl[slot] = any ? l * shrink : 0.f;
+      }
+    }
+    __syncthreads();  // (the exchange area is used again by the second block of queries)
+  }
+}
+
 // rows of a block mask that have no live column: out := NaN (m, l untouched)
 template <typename T>
 __global__ void band_dead_rows_kernel(T* out, int64_t n, int d, int64_t block, int64_t s) {
@@ -1937,11 +2451,32 @@ int launch_global_tiles(const TileArgs& a, hipStream_t stream, bool rows_only) {
     grid_cols = grid_cols / nb;
     if (grid_cols < 1) grid_cols = 1;
   }
-  if (!rows_only) launch_tile_kernel<T, D, kTileGlobalCols>(KernelEvents{}, dim3((unsigned)grid_cols, nb), stream, ac);
+  if (!rows_only) {
+    // all keys in one tile, half types, rows addressed with 32-bit offsets: the single-tile kernel
+    bool single = false;
+    if constexpr (sizeof(T) == 2 && (D == 32 || D == 64))
+      single = ac.persist && a.n * (int64_t)nb * (int64_t)(2 * D) < ((int64_t)1 << 31) &&
+               a.w <= (int64_t)0x3fffffff;
+    if (single) {
+      if constexpr (sizeof(T) == 2 && (D == 32 || D == 64))
+        hipLaunchKernelGGL((global_cols_dma_kernel<T, D>), dim3((unsigned)grid_cols, nb), dim3(256), 0, stream, ac);
+    } else {
+      launch_tile_kernel<T, D, kTileGlobalCols>(KernelEvents{}, dim3((unsigned)grid_cols, nb), stream, ac);
+    }
+  }
   const int64_t q_tiles = (a.n_globs + 127) / 128;
   TileArgs ar = a;
   ar.pair_split = (a.n_globs <= 64 && TileCfg<T, D>::NB == 2) ? 1 : 0;
-  launch_tile_kernel<T, D, kTileGlobalRows>(ev, dim3((unsigned)(q_tiles * a.n_split * nb)), stream, ar);
+  // at most 64 listed tokens, half types: independent wavefronts streaming K and V
+  bool streamed = false;
+  if constexpr (sizeof(T) == 2 && (D == 32 || D == 64))
+    streamed = a.n_globs <= 64 && a.n < ((int64_t)1 << 31) - 64 && a.w <= (int64_t)0x3fffffff;
+  if (streamed) {
+    if constexpr (sizeof(T) == 2 && (D == 32 || D == 64))
+      launch_maybe_timed(ev, global_rows_dma_kernel<T, D>, dim3((unsigned)(a.n_split * nb)), dim3(256), stream, ar);
+  } else {
+    launch_tile_kernel<T, D, kTileGlobalRows>(ev, dim3((unsigned)(q_tiles * a.n_split * nb)), stream, ar);
+  }
   hipLaunchKernelGGL((global_rows_merge_kernel<T, D>), dim3((unsigned)(a.n_globs * nb)), dim3(256), 0,
                      stream, a);
   return hipGetLastError() == hipSuccess ? 0 : 4;
