@@ -905,9 +905,38 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void band_dma_kernel(TileArgs
   // (Through the builtin the compiler forms a 64-bit address per lane and load, and it orders the
   // loads against LDS reads it cannot tell apart from them; the waits for the tiles are explicit
   // below, the compiler does not know of these loads.)
+  // The lane offsets of all NI instructions are kept in registers where there is room (up to
+  // d = 128): a whole tile then costs one 64-bit scalar address per matrix and nothing per
+  // instruction; only the last, partly filled tile of a subsequence computes clamped offsets.
+  constexpr bool kOffRegs = D <= 128;
+  uint32_t koffs[kOffRegs ? NI : 1], voffs[kOffRegs ? NI : 1];
+  if constexpr (kOffRegs) {
+#pragma unroll
+    for (int it = 0; it < NI; it++) {
+      koffs[it] = koff + (uint32_t)(it * RPI) * row_step;
+      voffs[it] = voff + (uint32_t)(it * RPI) * row_step;
+      if constexpr (RPI < 16) koffs[it] ^= (uint32_t)(C::kperm(it * RPI) * 16);
+    }
+  }
+  const int64_t base_byte = base * (int64_t)ROWB;  // scalar
   auto request = [&](int ut, int stage) __attribute__((always_inline)) {
-    const int64_t tile_byte = (base + (int64_t)ut * a.s) * (int64_t)ROWB;  // scalar
+    const int64_t tile_byte = base_byte + (int64_t)ut * (int64_t)row_step;  // scalar
     const bool whole = ut + BN <= u_hi;
+    if constexpr (kOffRegs) {
+      if (whole) {
+        const char* kp = Kp + tile_byte;
+        const char* vp = Vp + tile_byte;
+#pragma unroll
+        for (int it = 0; it < NI; it++) {
+          const uint32_t lds_k = lds_base + (uint32_t)(stage * BUF_B + (4 * it + wave) * 1024);
+          asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                       :: "v"(koffs[it]), "s"(kp), "s"(lds_k) : "memory", "m0");
+          asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                       :: "v"(voffs[it]), "s"(vp), "s"(lds_k + (uint32_t)TILE_B) : "memory", "m0");
+        }
+        return;
+      }
+    }
 #pragma unroll
     for (int it = 0; it < NI; it++) {
       // whole tile: this instruction's rows are added to the scalar base; last tile of a
@@ -1029,19 +1058,23 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void band_dma_kernel(TileArgs
     for (int v = 0; v < 16; v += 2) mx = fmaxf(fmaxf(mx, s[v]), s[v + 1]);
     mt_raw = mx;
     if (__builtin_expect(__builtin_amdgcn_ballot_w64(mx > thr_raw) != 0, 0)) {
-      // (m = -inf: first live block of a row, nothing accumulated yet)
+      // (m = -inf: first live block of a row, nothing accumulated yet - for the whole wavefront
+      // when this is its first live block, and then there is nothing to rescale)
+      const bool fresh = __builtin_amdgcn_ballot_w64(m > kNegInf) == 0;
       const float mp = fmaxf(mx, shfl_xor_f32(mx, 32)) * sc;
       const float m_new = (mp > m + kSlack) ? mp : m;
       const float alpha = (m > kNegInf) ? __builtin_amdgcn_exp2f(m - m_new) : 0.f;
       m = m_new;
       neg_m = (m > kNegInf) ? -m : 0.f;
       thr_raw = (m + kSlack) * inv_sc;
-      lsum[0] *= alpha;
-      l_add *= alpha;
+      if (!fresh) {
+        lsum[0] *= alpha;
+        l_add *= alpha;
 #pragma unroll
-      for (int eb = 0; eb < EB; eb++)
+        for (int eb = 0; eb < EB; eb++)
 #pragma unroll
-        for (int v = 0; v < 16; v++) o[eb][v] *= alpha;
+          for (int v = 0; v < 16; v++) o[eb][v] *= alpha;
+      }
     }
   };
   // ... and its second half: the exponentials, packed as the B operands of the second product
@@ -1087,6 +1120,16 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void band_dma_kernel(TileArgs
     }
   };
 
+  // What a 32-key block that starts at key ub is to this wavefront's 32 queries: dead when
+  // ub < blk_dead_lo or ub > blk_dead_hi (no live pair: before every window, after every window
+  // or past the last key), full when blk_full_lo <= ub <= blk_full_hi (every pair live: inside
+  // every query's window and whole).  Positions and the clamped window are below 2^30.
+  const bool wave_live = tw0 < qlen;
+  const int blk_dead_lo = tw0 - wlim - 31;
+  const int blk_dead_hi = (tw0 + 31 + wlim < u_hi - 1) ? tw0 + 31 + wlim : u_hi - 1;
+  const int blk_full_lo = tw0 + 31 - wlim;
+  const int blk_full_hi = (tw0 - 31 + wlim < u_hi - 32) ? tw0 - 31 + wlim : u_hi - 32;
+
   // one tile: wait for it, publish it, request the tile NBUF - 1 steps ahead into the buffer the
   // previous step has freed, consume it
   auto step = [&](int it, int stage) __attribute__((always_inline)) {
@@ -1111,13 +1154,14 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void band_dma_kernel(TileArgs
     // window starts after the block's first key, or some query's window (or the subsequence)
     // ends before its last key.  A dead block beside a live one is computed and masked out.
     // (positions and the clamped window are below 2^30, so the sums stay inside 32 bits)
+    // (the four bounds of a block's first key are set up once per wavefront, before the loop)
     bool test[NB];
     bool none = true;
 #pragma unroll
     for (int jb = 0; jb < NB; jb++) {
       const int ub = ut + 32 * jb;
-      const bool dead = (tw0 >= qlen) || (ub >= u_hi) || (ub - wlim > tw0 + 31) || (ub + 31 < tw0 - wlim);
-      test[jb] = dead || (ub < tw0 + 31 - wlim) || (ub + 31 - wlim > tw0) || (ub + 32 > u_hi);
+      const bool dead = !wave_live || ub < blk_dead_lo || ub > blk_dead_hi;
+      test[jb] = !(ub >= blk_full_lo && ub <= blk_full_hi);  // (a dead block is never full)
       none = none && dead;
     }
     // (a shared tail tile: the wavefronts take the key tiles in turn)
@@ -1136,20 +1180,23 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void band_dma_kernel(TileArgs
     __builtin_amdgcn_sched_barrier(0);
     if (none) return;
 
-    // key slot j of the tile is live for this lane's query iff jlo <= j <= jhi; the slots this
-    // lane holds are c + 4*h for compile-time c, so the bounds are shifted by 4*h once
-    const int live_slots = (u_hi - ut) < BN ? (u_hi - ut) : BN;
-    const int jlo = (tq - wlim - ut) - 4 * h;
-    const int jhi_band = tq + wlim - ut;
-    const int jhi = (jhi_band < live_slots - 1 ? jhi_band : live_slots - 1) - 4 * h;
-    // both ends at once: (unsigned)(c - jlo) <= jhi - jlo; a query without a live key in the tile
-    // (jhi < jlo) gets bounds that no c meets
-    const int jlo_both = jhi >= jlo ? jlo : 0x40000000;
-    const uint32_t span = jhi >= jlo ? (uint32_t)(jhi - jlo) : 0u;
-
-    // the band test of a block (a compare and a select per element), then the softmax step
+    // the band test of a block (a compare and a select per element); its per-lane bounds are
+    // only worked out for a block that needs them (the opaque copy keeps the compiler from
+    // moving that work in front of the branch, into every step)
     auto band_test = [&](f32x16& s, int jb, bool test) __attribute__((always_inline)) {
       if (test) {
+        int ut_o = ut;
+        asm volatile("" : "+s"(ut_o));
+        // key slot j of the tile is live for this lane's query iff jlo <= j <= jhi; the slots
+        // this lane holds are c + 4*h for compile-time c, so the bounds are shifted by 4*h once
+        const int live_slots = (u_hi - ut_o) < BN ? (u_hi - ut_o) : BN;
+        const int jlo = (tq - wlim - ut_o) - 4 * h;
+        const int jhi_band = tq + wlim - ut_o;
+        const int jhi = (jhi_band < live_slots - 1 ? jhi_band : live_slots - 1) - 4 * h;
+        // both ends at once: (unsigned)(c - jlo) <= jhi - jlo; a query without a live key in the
+        // tile (jhi < jlo) gets bounds that no c meets
+        const int jlo_both = jhi >= jlo ? jlo : 0x40000000;
+        const uint32_t span = jhi >= jlo ? (uint32_t)(jhi - jlo) : 0u;
 #pragma unroll
         for (int v = 0; v < 16; v++) {
           const int c = 32 * jb + 8 * (v / 4) + (v % 4);
