@@ -142,10 +142,13 @@ struct alignas((N & (N - 1)) == 0 ? 4 * N : 4) RowPiece {
 // o holds O^T in the 32x32 result layout: o[eb][v] is element e = 32*eb + i of the row for the
 // half types and e = (D/32)*i + eb for fp32, i = 8*(v/4) + 4*h + v%4; m is the running max in log2 units, l the row sum (already summed over both halves
 // of the wavefront); o * o_scale is the accumulator that goes with (m, l).
+// dr: length of a row of `out` in elements (a multiple of 16 bytes, at most D; the accumulator's
+// elements from dr on belong to zero padding and are not written).
 template <typename T, int D>
 __device__ __forceinline__ void tile_write_row(const Tensors& t, int64_t row, int h, float m, float l,
                                                const f32x16 (&o)[D / 32], float o_scale = 1.f,
-                                               bool have_in = false, float l_pre = 0.f, float m_pre = 0.f) {
+                                               bool have_in = false, float l_pre = 0.f, float m_pre = 0.f,
+                                               int dr = D) {
   constexpr bool kF32 = sizeof(T) == 4;
   const bool sf = t.state_f32 != 0;
   const float m_nat = m * 0.6931471805599453f;
@@ -163,7 +166,7 @@ __device__ __forceinline__ void tile_write_row(const Tensors& t, int64_t row, in
   const float inv = 1.f / l_out;
   wb *= inv * o_scale;  // o_scale: o was accumulated against a reference below the maximum m
   wa *= inv;
-  T* orow = (T*)t.out + row * D;
+  T* orow = (T*)t.out + row * dr;
   if constexpr (kF32) {
     // registers 4*g4 .. 4*g4+3 of all blocks: 4*EB consecutive elements from EB * (8*g4 + 4*h)
     constexpr int EB = D / 32;
@@ -172,6 +175,7 @@ __device__ __forceinline__ void tile_write_row(const Tensors& t, int64_t row, in
 #pragma unroll
       for (int c = 0; c < EB; c++) {
         const int e = EB * (8 * g4 + 4 * h) + 4 * c;
+        if (e >= dr) continue;
         float x[4];
 #pragma unroll
         for (int u = 0; u < 4; u++) x[u] = o[(4 * c + u) % EB][4 * g4 + (4 * c + u) / EB] * wb;
@@ -200,7 +204,7 @@ __device__ __forceinline__ void tile_write_row(const Tensors& t, int64_t row, in
         float x[4];
 #pragma unroll
         for (int i = 0; i < 4; i++) x[i] = o[eb][4 * g4 + i] * wb;
-        if (wa != 0.f) {
+        if (wa != 0.f && e < dr) {
           typedef T t4 __attribute__((ext_vector_type(4)));
           t4 oi = *reinterpret_cast<const t4*>(orow + e);
 #pragma unroll
@@ -218,7 +222,7 @@ __device__ __forceinline__ void tile_write_row(const Tensors& t, int64_t row, in
         got[1] = (uint32_t)__builtin_amdgcn_ds_bpermute(partner, (int)give[1]);
         const uint4v piece = h ? uint4v{got[0], got[1], keep[0], keep[1]}
                                : uint4v{keep[0], keep[1], got[0], got[1]};
-        *reinterpret_cast<uint4v*>(orow + 32 * eb + 8 * (2 * h + k)) = piece;
+        if (32 * eb + 8 * (2 * h + k) < dr) *reinterpret_cast<uint4v*>(orow + 32 * eb + 8 * (2 * h + k)) = piece;
       }
     }
   }
@@ -228,8 +232,9 @@ __device__ __forceinline__ void tile_write_row(const Tensors& t, int64_t row, in
   }
 }
 
-template <typename T, int D, int MODE>
+template <typename T, int D, int MODE, bool PAD = false>
 __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void tile_kernel(TileArgs a) {
+  static_assert(!PAD || MODE == kTileBand, "padded rows: band mode only");
   using C = TileCfg<T, D>;
   constexpr bool kF32 = C::kF32;
   constexpr int BM = C::BM, BN = C::BN, EB = C::EB, NB = C::NB;
@@ -312,7 +317,10 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void tile_kernel(TileArgs a) 
   const T* Qp = (const T*)a.t.q;
   const T* Kp = (const T*)a.t.k;
   const T* Vp = (const T*)a.t.v;
-  const float sc = 1.4426950408889634f / sqrtf((float)D);
+  // PAD: rows of Q, K, V and out are dr < D elements long (a multiple of 16 bytes); the operands
+  // are filled up with zeros, which change neither the scores nor the elements below dr
+  const int dr = PAD ? (int)a.t.d : D;
+  const float sc = 1.4426950408889634f / sqrtf((float)dr);
   const bool persist = (MODE == kTileGlobalCols) && a.persist != 0;
   // global modes: tokens of problem bb are rows bb * n + token of the stacked tensors (masks work
   // on the tokens, only addresses take the offset)
@@ -328,7 +336,8 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void tile_kernel(TileArgs a) 
     if constexpr (kF32) {
 #pragma unroll
       for (int g = 0; g < D / 8; g++) {
-        float4v x = *reinterpret_cast<const float4v*>(qrow + 8 * g + 4 * h);
+        float4v x = {0.f, 0.f, 0.f, 0.f};
+        if (!PAD || 8 * g + 4 * h < dr) x = *reinterpret_cast<const float4v*>(qrow + 8 * g + 4 * h);
         df[4 * g] = x[0];
         df[4 * g + 1] = x[1];
         df[4 * g + 2] = x[2];
@@ -336,8 +345,10 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void tile_kernel(TileArgs a) 
       }
     } else {
 #pragma unroll
-      for (int ks = 0; ks < C::QREGS; ks++)
-        dh[ks] = *reinterpret_cast<const uint4v*>(qrow + 16 * ks + 8 * h);
+      for (int ks = 0; ks < C::QREGS; ks++) {
+        dh[ks] = uint4v{0u, 0u, 0u, 0u};
+        if (!PAD || 16 * ks + 8 * h < dr) dh[ks] = *reinterpret_cast<const uint4v*>(qrow + 16 * ks + 8 * h);
+      }
     }
   };
   bool have_q = false;  // the rows of this trip were asked for during the previous one
@@ -363,7 +374,7 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void tile_kernel(TileArgs a) 
     if (q_ok && bit_is_set(a.gbits, q_tok)) q_ok = false;  // global rows belong to GlobalRows
   }
 
-  if (!have_q) load_q(Qp + (q_tok + tok_off) * D, qh, qf);
+  if (!have_q) load_q(Qp + (q_tok + tok_off) * dr, qh, qf);
   // a persistent workgroup finishes a row every few microseconds: its incoming state is read
   // here, long before the write-back needs it
   float l_pre = 0.f, m_pre = 0.f;
@@ -417,8 +428,8 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void tile_kernel(TileArgs a) 
       const int j = idx / CH, c = idx % CH;
       const int64_t u = ut + j;
       uint4v kx = {0u, 0u, 0u, 0u}, vx = {0u, 0u, 0u, 0u};
-      if (u < u_hi) {
-        const int64_t off = key_tok(u) * D + (16 / (int)sizeof(T)) * c;
+      if (u < u_hi && (!PAD || (16 / (int)sizeof(T)) * c < dr)) {
+        const int64_t off = key_tok(u) * dr + (16 / (int)sizeof(T)) * c;
         kx = *reinterpret_cast<const uint4v*>(Kp + off);
         if constexpr (kF32) vx = *reinterpret_cast<const uint4v*>(Vp + off);
       }
@@ -433,8 +444,9 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void tile_kernel(TileArgs a) 
         const int c = lane / PAIRS + LPP * (wave + 4 * it);
         const int64_t u = ut + 2 * jp;
         uint4v v0 = {0u, 0u, 0u, 0u}, v1 = {0u, 0u, 0u, 0u};
-        if (u < u_hi && c < CH) v0 = *reinterpret_cast<const uint4v*>(Vp + key_tok(u) * D + 8 * c);
-        if (u + 1 < u_hi && c < CH) v1 = *reinterpret_cast<const uint4v*>(Vp + key_tok(u + 1) * D + 8 * c);
+        const bool c_ok = c < CH && (!PAD || 8 * c < dr);
+        if (u < u_hi && c_ok) v0 = *reinterpret_cast<const uint4v*>(Vp + key_tok(u) * dr + 8 * c);
+        if (u + 1 < u_hi && c_ok) v1 = *reinterpret_cast<const uint4v*>(Vp + key_tok(u + 1) * dr + 8 * c);
         vreg[2 * it] = v0;
         vreg[2 * it + 1] = v1;
       }
@@ -741,7 +753,7 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void tile_kernel(TileArgs a) 
     return;
   }
   if (q_ok && l > 0.f && wave_k <= 0)
-    tile_write_row<T, D>(a.t, q_tok + tok_off, h, m, l, o, 1.f, MODE == kTileGlobalCols, l_pre, m_pre);
+    tile_write_row<T, D>(a.t, q_tok + tok_off, h, m, l, o, 1.f, MODE == kTileGlobalCols, l_pre, m_pre, dr);
   if (!persist) break;
   if constexpr (kNextQ) {
     if (have_q) {
@@ -2369,27 +2381,27 @@ constexpr int64_t kFusedMaxGlobals = 256;
 // of the kernel is raised once per device)
 // (tile_kernel_ready: false when the runtime refuses the limit; the callers ask before they
 // launch anything and leave the call to the row-gather engine then)
-template <typename T, int D, int MODE>
+template <typename T, int D, int MODE, bool PAD = false>
 bool tile_kernel_ready() {
   using C = TileCfg<T, D>;
   if constexpr (C::kDynLds) {
     static std::atomic<bool> raised[kLdsLimitDevices];
-    return raise_lds_limit(reinterpret_cast<const void*>(&tile_kernel<T, D, MODE>), C::LDS_BYTES, raised);
+    return raise_lds_limit(reinterpret_cast<const void*>(&tile_kernel<T, D, MODE, PAD>), C::LDS_BYTES, raised);
   }
   return true;
 }
 
-template <typename T, int D, int MODE>
+template <typename T, int D, int MODE, bool PAD = false>
 void launch_tile_kernel(const KernelEvents& ev, dim3 grid, hipStream_t stream, const TileArgs& a) {
   using C = TileCfg<T, D>;
   if constexpr (C::kDynLds) {
-    if (!tile_kernel_ready<T, D, MODE>()) return;  // (asked before; a refusal surfaces as a launch error)
+    if (!tile_kernel_ready<T, D, MODE, PAD>()) return;  // (asked before; a refusal surfaces as a launch error)
     if (ev.start != nullptr && ev.stop != nullptr)
-      hipExtLaunchKernelGGL((tile_kernel<T, D, MODE>), grid, dim3(256), C::LDS_BYTES, stream, ev.start, ev.stop, 0, a);
+      hipExtLaunchKernelGGL((tile_kernel<T, D, MODE, PAD>), grid, dim3(256), C::LDS_BYTES, stream, ev.start, ev.stop, 0, a);
     else
-      hipLaunchKernelGGL((tile_kernel<T, D, MODE>), grid, dim3(256), C::LDS_BYTES, stream, a);
+      hipLaunchKernelGGL((tile_kernel<T, D, MODE, PAD>), grid, dim3(256), C::LDS_BYTES, stream, a);
   } else {
-    launch_maybe_timed(ev, tile_kernel<T, D, MODE>, grid, dim3(256), stream, a);
+    launch_maybe_timed(ev, tile_kernel<T, D, MODE, PAD>, grid, dim3(256), stream, a);
   }
 }
 
@@ -2478,6 +2490,28 @@ int launch_band_tiles(const TileArgs& a, int use_nan, hipStream_t stream) {
   return hipGetLastError() == hipSuccess ? 0 : 4;
 }
 
+// Rows of a.t.d < D elements, D the next multiple of 32 (d = 40, 80, 100 ...): the register-staged
+// kernel with its operands filled up with zeros.  One workgroup per tile; no listed tokens.
+template <typename T, int D>
+int launch_band_tiles_padded(const TileArgs& a, int use_nan, hipStream_t stream) {
+  if (a.globs != nullptr) return -1;
+  const KernelEvents ev = kernel_events();
+  if (a.n_tiles > 0) {
+    const int64_t grid = (a.n_tiles * a.t.n_batch + 7) / 8 * 8;
+    if (!tile_kernel_ready<T, D, kTileBand, true>()) return -1;
+    TileArgs at = a;
+    at.n_tail = 0;
+    launch_tile_kernel<T, D, kTileBand, true>(ev, dim3((unsigned)grid), stream, at);
+  }
+  if (a.block > 0 && use_nan && a.s > 1) {
+    const int64_t rows = a.n * a.t.n_batch;
+    const int64_t total = rows * a.t.d;
+    hipLaunchKernelGGL((band_dead_rows_kernel<T>), dim3((unsigned)((total + 255) / 256)), dim3(256),
+                       0, stream, (T*)a.t.out, rows, (int)a.t.d, a.block, a.s);
+  }
+  return hipGetLastError() == hipSuccess ? 0 : 4;
+}
+
 // Global minus local: non-global rows against the listed globals, then the global rows against
 // everything (key range split over workgroups), then the fold of the splits.
 // rows_only: the listed tokens' own rows only (the other rows have had the listed tokens as keys
@@ -2538,6 +2572,22 @@ inline bool tile_shape_ok(const Tensors& t, size_t elem_bytes) {
 // Returns -1 when the shape is not covered (caller falls back to the row-gather engine).
 template <typename T>
 int run_band_tiles(const TileArgs& a, int use_nan, hipStream_t stream) {
+  if (a.t.d % 32 != 0) {
+    // rows of whole 16-byte pieces: the tiles of the next multiple of 32, filled up with zeros
+    constexpr int64_t kPiece = 16 / (int64_t)sizeof(T);
+    if (!aligned16(a.t.q) || !aligned16(a.t.k) || !aligned16(a.t.v) || !aligned16(a.t.out)) return -1;
+    if (a.t.d % kPiece != 0 || a.t.d < kPiece || a.t.d > 256) return -1;
+    switch ((a.t.d + 31) / 32) {
+      case 1: return launch_band_tiles_padded<T, 32>(a, use_nan, stream);
+      case 2: return launch_band_tiles_padded<T, 64>(a, use_nan, stream);
+      case 3: return launch_band_tiles_padded<T, 96>(a, use_nan, stream);
+      case 4: return launch_band_tiles_padded<T, 128>(a, use_nan, stream);
+      case 5: return launch_band_tiles_padded<T, 160>(a, use_nan, stream);
+      case 6: return launch_band_tiles_padded<T, 192>(a, use_nan, stream);
+      case 7: return launch_band_tiles_padded<T, 224>(a, use_nan, stream);
+      default: return launch_band_tiles_padded<T, 256>(a, use_nan, stream);
+    }
+  }
   if (!tile_shape_ok(a.t, sizeof(T))) return -1;
   if (a.t.d == 64) return launch_band_tiles<T, 64>(a, use_nan, stream);
   if (a.t.d == 128) return launch_band_tiles<T, 128>(a, use_nan, stream);

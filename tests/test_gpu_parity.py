@@ -917,6 +917,49 @@ def test_local_2d_dilated(mods, dtype, d, n, block, dil, use_nan):
     check(o, m, l, *ref, dtype, state_dtype=torch.float32, dead_expect="nan" if use_nan else None)
 
 
+@pytest.mark.parametrize("dtype,d", [(torch.float32, 4), (torch.float32, 40), (torch.float32, 100),
+                                     (torch.float32, 132), (torch.float32, 252), (torch.bfloat16, 8),
+                                     (torch.bfloat16, 40), (torch.float16, 80), (torch.bfloat16, 104),
+                                     (torch.float16, 136), (torch.bfloat16, 200), (torch.float16, 248)])
+def test_band_masks_rows_that_are_no_multiple_of_32(mods, dtype, d):
+    """Rows of whole 16-byte pieces (4 floats, 8 halves) run on the tiles of the next multiple of 32
+    with zero-filled operands: every band mask, ragged last tiles, dead rows, and a chained call
+    whose incoming state is set for some rows and empty for others."""
+    for n, w in [(1000, 128), (777, 776), (130, 0)]:
+        q, k, v = dev_qkv(n, d, dtype, 33)
+        m, l, o = state(n, d, dtype, torch.float32)
+        mods["spfa_local"].forward(q, k, v, m, l, o, w)
+        sync()
+        check(o, m, l, *c_oracle.local(np64(q), np64(k), np64(v), w), dtype, state_dtype=torch.float32)
+    for n, w, dil in [(1001, 100, 1), (5000, 40, 4)]:
+        q, k, v = dev_qkv(n, d, dtype, 34, scale=0.5)
+        m, l, o = state(n, d, dtype, torch.float32)
+        mods["spfa_local_1d_dilated"].forward(q, k, v, m, l, o, w, dil)
+        sync()
+        check(o, m, l, *c_oracle.local_1d_dilated(np64(q), np64(k), np64(v), w, dil), dtype,
+              state_dtype=torch.float32)
+    for n, block, dil, use_nan in [(1200, 300, 1, True), (1024, 64, 1, False), (2048, 2048, 0, True)]:
+        q, k, v = dev_qkv(n, d, dtype, 35, scale=0.5)
+        m, l, o = state(n, d, dtype, torch.float32)
+        mods["spfa_local_2d_dilated"].forward(q, k, v, m, l, o, block, dil, use_nan)
+        sync()
+        ref = c_oracle.local_2d_dilated(np64(q), np64(k), np64(v), block, dil, use_nan=use_nan)
+        check(o, m, l, *ref, dtype, state_dtype=torch.float32, dead_expect="nan" if use_nan else None)
+    # a random mask outside the window first (half of its rows empty), then the window on top
+    n, w = 900, 60
+    rng = np.random.default_rng(36)
+    band = so.mask_local_dense(n, w)
+    rand = (rng.random((n, n)) < 0.03) & ~band
+    rand[rng.random(n) < 0.5] = False
+    q, k, v = dev_qkv(n, d, dtype, 36)
+    ro, ci = so.csr_from_dense(rand)
+    o, m, l = run_csr(mods, q, k, v, ro, ci, False, st=state(n, d, dtype, torch.float32))
+    mods["spfa_local"].forward(q, k, v, m, l, o, w)
+    sync()
+    check(o, m, l, *so.dense_masked_attention(np64(q), np64(k), np64(v), band | rand), dtype,
+          state_dtype=torch.float32)
+
+
 @pytest.mark.parametrize("dtype,d", [(torch.float32, 64), (torch.float32, 128), (torch.bfloat16, 64),
                                      (torch.float16, 128), (torch.float16, 32), (torch.bfloat16, 256),
                                      (torch.float32, 32), (torch.float32, 96), (torch.bfloat16, 192)])
