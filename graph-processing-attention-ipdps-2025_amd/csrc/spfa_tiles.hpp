@@ -234,7 +234,6 @@ __device__ __forceinline__ void tile_write_row(const Tensors& t, int64_t row, in
 
 template <typename T, int D, int MODE, bool PAD = false>
 __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void tile_kernel(TileArgs a) {
-  static_assert(!PAD || MODE == kTileBand, "padded rows: band mode only");
   using C = TileCfg<T, D>;
   constexpr bool kF32 = C::kF32;
   constexpr int BM = C::BM, BN = C::BN, EB = C::EB, NB = C::NB;
@@ -387,7 +386,7 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void tile_kernel(TileArgs a) 
     have_q = persist && t0n < qlen;
     if (have_q) {
       const int64_t tqn = t0n + 32 * wave_q + r;
-      load_q(Qp + ((tqn < qlen ? tqn : qlen - 1) + tok_off) * D, qh_next, qf_next);
+      load_q(Qp + ((tqn < qlen ? tqn : qlen - 1) + tok_off) * dr, qh_next, qf_next);
     }
   }
 
@@ -721,7 +720,7 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void tile_kernel(TileArgs a) 
     if (!q_ok) return;  // (this mode makes a single trip)
     const int64_t slot = (bb * a.n_globs + tq) * a.n_split + split;
     const bool any = l > 0.f;
-    float* prow = a.pacc + slot * D;
+    float* prow = a.pacc + slot * dr;  // (rows of the real length; elements from dr on are padding)
     if constexpr (kF32) {
 #pragma unroll
       for (int g4 = 0; g4 < 4; g4++)
@@ -732,7 +731,8 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void tile_kernel(TileArgs a) 
 #pragma unroll
             for (int u = 0; u < 4; u++) y[u] = o[(4 * c + u) % EB][4 * g4 + (4 * c + u) / EB];
           }
-          *reinterpret_cast<float4v*>(prow + EB * (8 * g4 + 4 * h) + 4 * c) = y;
+          const int e = EB * (8 * g4 + 4 * h) + 4 * c;
+          if (!PAD || e < dr) *reinterpret_cast<float4v*>(prow + e) = y;
         }
     } else {
 #pragma unroll
@@ -743,7 +743,8 @@ __global__ __launch_bounds__(256, D > 128 ? 1 : 2) void tile_kernel(TileArgs a) 
           if (any) {
             y[0] = o[eb][4 * g4]; y[1] = o[eb][4 * g4 + 1]; y[2] = o[eb][4 * g4 + 2]; y[3] = o[eb][4 * g4 + 3];
           }
-          *reinterpret_cast<float4v*>(prow + 32 * eb + 8 * g4 + 4 * h) = y;
+          const int e = 32 * eb + 8 * g4 + 4 * h;
+          if (!PAD || e < dr) *reinterpret_cast<float4v*>(prow + e) = y;
         }
     }
     if (h == 0) {
@@ -2300,9 +2301,11 @@ __global__ void band_dead_rows_kernel(T* out, int64_t n, int d, int64_t block, i
 // One workgroup per distinct global row: fold the key-split partials (two passes: overall max,
 // then weighted sums with the splits spread over the threads), fold the incoming state in,
 // write the row.
-template <typename T, int D>
+template <typename T, int D, bool PAD = false>
 __global__ __launch_bounds__(256) void global_rows_merge_kernel(TileArgs a) {
-  constexpr int NSUB = 256 / D;  // threads per output element
+  // (PAD: rows of a.t.d < D elements, the tile kernels ran with zero-filled operands)
+  const int dd = PAD ? (int)a.t.d : D;
+  const int NSUB = 256 / dd;  // threads per output element
   __shared__ float red[4];
   __shared__ float part[256];
   // grid: [problem][listed global]; the first n_uq of a problem's slots are its distinct rows
@@ -2331,25 +2334,24 @@ __global__ __launch_bounds__(256) void global_rows_merge_kernel(TileArgs a) {
   lsum = (red[0] + red[1]) + (red[2] + red[3]);
 
   // (d that does not divide 256: the threads past NSUB * d have no element)
-  const int e = tid % D, sub = tid / D;
+  const int e = tid % dd, sub = tid / dd;
   float acc = 0.f;
   int64_t k = sub < NSUB ? sub : a.n_split;
   for (; k + 3 * NSUB < a.n_split; k += 4 * NSUB) {
     float x[4], wgt[4];
 #pragma unroll
     for (int u = 0; u < 4; u++) {
-      x[u] = a.pacc[(s0 + k + u * NSUB) * D + e];
+      x[u] = a.pacc[(s0 + k + u * NSUB) * dd + e];
       wgt[u] = a.pm[s0 + k + u * NSUB];
     }
 #pragma unroll
     for (int u = 0; u < 4; u++) acc += __expf(wgt[u] - mx) * x[u];
   }
-  for (; k < a.n_split; k += NSUB) acc += __expf(a.pm[s0 + k] - mx) * a.pacc[(s0 + k) * D + e];
+  for (; k < a.n_split; k += NSUB) acc += __expf(a.pm[s0 + k] - mx) * a.pacc[(s0 + k) * dd + e];
   part[tid] = acc;
   __syncthreads();
   if (sub != 0) return;
-#pragma unroll
-  for (int u = 1; u < NSUB; u++) acc += part[u * D + e];
+  for (int u = 1; u < NSUB; u++) acc += part[u * dd + e];
 
   const int64_t row = a.uq[g] + bb * a.n;
   const bool sf = a.t.state_f32 != 0;
@@ -2363,7 +2365,7 @@ __global__ __launch_bounds__(256) void global_rows_merge_kernel(TileArgs a) {
     l_out = wa + lsum * wb;
   }
   const float inv = 1.f / l_out;
-  T* orow = (T*)a.t.out + row * D;
+  T* orow = (T*)a.t.out + row * dd;
   float x = acc * wb;
   if (wa != 0.f) x += wa * to_f32(orow[e]);
   orow[e] = from_f32<T>(x * inv);
@@ -2563,6 +2565,40 @@ int launch_global_tiles(const TileArgs& a, hipStream_t stream, bool rows_only) {
   return hipGetLastError() == hipSuccess ? 0 : 4;
 }
 
+// The global mask with rows of a.t.d < D elements, D the next multiple of 32: the register-staged
+// kernels with zero-filled operands; the partial results and the merge keep the real row length.
+template <typename T, int D>
+int launch_global_tiles_padded(const TileArgs& a, hipStream_t stream, bool rows_only) {
+  const KernelEvents ev = kernel_events();
+  if (!tile_kernel_ready<T, D, kTileGlobalCols, true>() || !tile_kernel_ready<T, D, kTileGlobalRows, true>()) return -1;
+  int64_t grid_cols = (a.n + 127) / 128;
+  TileArgs ac = a;
+  ac.persist = (a.n_globs <= TileCfg<T, D>::BN) ? 1 : 0;
+  const unsigned nb = (unsigned)a.t.n_batch;
+  if (ac.persist) {
+    const int64_t resident = (int64_t)device_cu_count() * 2;  // two workgroups fit a CU
+    if (grid_cols > resident) grid_cols = resident;
+    if (nb > 1) grid_cols = grid_cols / nb > 0 ? grid_cols / nb : 1;
+  }
+  if (!rows_only)
+    launch_tile_kernel<T, D, kTileGlobalCols, true>(KernelEvents{}, dim3((unsigned)grid_cols, nb), stream, ac);
+  const int64_t q_tiles = (a.n_globs + 127) / 128;
+  TileArgs ar = a;
+  ar.pair_split = (a.n_globs <= 64 && TileCfg<T, D>::NB == 2) ? 1 : 0;
+  launch_tile_kernel<T, D, kTileGlobalRows, true>(ev, dim3((unsigned)(q_tiles * a.n_split * nb)), stream, ar);
+  hipLaunchKernelGGL((global_rows_merge_kernel<T, D, true>), dim3((unsigned)(a.n_globs * nb)), dim3(256), 0,
+                     stream, a);
+  return hipGetLastError() == hipSuccess ? 0 : 4;
+}
+
+// rows of whole 16-byte pieces that are no multiple of 32 elements, up to 256
+template <typename T>
+inline bool tile_shape_padded_ok(const Tensors& t) {
+  constexpr int64_t kPiece = 16 / (int64_t)sizeof(T);
+  if (!aligned16(t.q) || !aligned16(t.k) || !aligned16(t.v) || !aligned16(t.out)) return false;
+  return t.d % 32 != 0 && t.d % kPiece == 0 && t.d >= kPiece && t.d <= 256;
+}
+
 inline bool tile_shape_ok(const Tensors& t, size_t elem_bytes) {
   if (!aligned16(t.q) || !aligned16(t.k) || !aligned16(t.v) || !aligned16(t.out)) return false;
   (void)elem_bytes;
@@ -2574,9 +2610,7 @@ template <typename T>
 int run_band_tiles(const TileArgs& a, int use_nan, hipStream_t stream) {
   if (a.t.d % 32 != 0) {
     // rows of whole 16-byte pieces: the tiles of the next multiple of 32, filled up with zeros
-    constexpr int64_t kPiece = 16 / (int64_t)sizeof(T);
-    if (!aligned16(a.t.q) || !aligned16(a.t.k) || !aligned16(a.t.v) || !aligned16(a.t.out)) return -1;
-    if (a.t.d % kPiece != 0 || a.t.d < kPiece || a.t.d > 256) return -1;
+    if (!tile_shape_padded_ok<T>(a.t)) return -1;
     switch ((a.t.d + 31) / 32) {
       case 1: return launch_band_tiles_padded<T, 32>(a, use_nan, stream);
       case 2: return launch_band_tiles_padded<T, 64>(a, use_nan, stream);
@@ -2602,6 +2636,19 @@ int run_band_tiles(const TileArgs& a, int use_nan, hipStream_t stream) {
 
 template <typename T>
 int run_global_tiles(const TileArgs& a, hipStream_t stream, bool rows_only = false) {
+  if (a.t.d % 32 != 0) {
+    if (!tile_shape_padded_ok<T>(a.t)) return -1;
+    switch ((a.t.d + 31) / 32) {
+      case 1: return launch_global_tiles_padded<T, 32>(a, stream, rows_only);
+      case 2: return launch_global_tiles_padded<T, 64>(a, stream, rows_only);
+      case 3: return launch_global_tiles_padded<T, 96>(a, stream, rows_only);
+      case 4: return launch_global_tiles_padded<T, 128>(a, stream, rows_only);
+      case 5: return launch_global_tiles_padded<T, 160>(a, stream, rows_only);
+      case 6: return launch_global_tiles_padded<T, 192>(a, stream, rows_only);
+      case 7: return launch_global_tiles_padded<T, 224>(a, stream, rows_only);
+      default: return launch_global_tiles_padded<T, 256>(a, stream, rows_only);
+    }
+  }
   if (!tile_shape_ok(a.t, sizeof(T))) return -1;
   if (a.t.d == 64) return launch_global_tiles<T, 64>(a, stream, rows_only);
   if (a.t.d == 128) return launch_global_tiles<T, 128>(a, stream, rows_only);

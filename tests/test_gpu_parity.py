@@ -461,7 +461,7 @@ def test_csr_mostly_empty_rows(mods, shape, use_nan):
 
 @pytest.mark.parametrize("dtype,d", [(torch.float32, 64), (torch.bfloat16, 64), (torch.float32, 40)])
 def test_implicit_masks_batch_of_heads(mods, dtype, d):
-    """d = 64 runs the dense-tile kernels, d = 40 the row-gather engine."""
+    """d = 64 runs the dense-tile kernels as they are, d = 40 those of d = 64 with zero-filled operands."""
     n = 1024
     shape = (2, 2)
     w, dil, blk = 40, 1, 64
@@ -1045,6 +1045,45 @@ def test_global_no_local(mods, dtype, d, n, n_globs, w):
     sync()
     ref = c_oracle.global_no_local(np64(q), np64(k), np64(v), g.numpy(), w)
     check(o, m, l, *ref, dtype, state_dtype=torch.float32)
+
+
+@pytest.mark.parametrize("dtype,d", [(torch.float32, 4), (torch.float32, 40), (torch.float32, 100),
+                                     (torch.float32, 200), (torch.float32, 252), (torch.bfloat16, 8),
+                                     (torch.bfloat16, 40), (torch.float16, 80), (torch.bfloat16, 104),
+                                     (torch.float16, 136), (torch.bfloat16, 200), (torch.float16, 248)])
+def test_global_no_local_rows_that_are_no_multiple_of_32(mods, dtype, d):
+    """Rows of whole 16-byte pieces on the tiles of the next multiple of 32 (zero-filled operands,
+    partial results and merge at the real row length): one tile of listed tokens and several, a
+    chained call on a state that the window call has set, a batch, and the one-call composite."""
+    for n, n_globs, w in [(1024, 4, 10), (1500, 100, 1499), (3000, 200, 7), (8192, 16, 100)]:
+        q, k, v = dev_qkv(n, d, dtype, 37)
+        g = syn.global_indices(n, n_globs, seed=37)
+        m, l, o = state(n, d, dtype, torch.float32)
+        mods["spfa_global_no_local"].forward(q, k, v, m, l, o, g.to(DEV), w)
+        sync()
+        check(o, m, l, *c_oracle.global_no_local(np64(q), np64(k), np64(v), g.numpy(), w), dtype,
+              state_dtype=torch.float32)
+    n, w, globs = 1100, 30, [5, 6, 400, 1099]
+    g = torch.tensor(globs, dtype=torch.int32, device=DEV)
+    union = so.mask_local_dense(n, w) | so.mask_global_no_local_dense(n, globs, w)
+    q, k, v = dev_qkv(n, d, dtype, 38)
+    m, l, o = state(n, d, dtype, torch.float32)
+    mods["spfa_local"].forward(q, k, v, m, l, o, w)
+    mods["spfa_global_no_local"].forward(q, k, v, m, l, o, g, w)
+    sync()
+    ref = so.dense_masked_attention(np64(q), np64(k), np64(v), union)
+    check(o, m, l, *ref, dtype, state_dtype=torch.float32)
+    m2, l2, o2 = state(n, d, dtype, torch.float32)
+    empty = torch.empty(0, device=DEV)
+    mods["spfa_bigbird"].forward(q, k, v, m2, l2, o2, w, g, torch.zeros(0, dtype=torch.uint64, device=DEV),
+                                 torch.zeros(0, dtype=torch.uint32, device=DEV), empty)
+    sync()
+    check(o2, m2, l2, *ref, dtype, state_dtype=torch.float32)
+    q, k, v, m, l, o = _stacked(n, d, dtype, (3,), 39)
+    mods["spfa_global_no_local"].forward(q, k, v, m, l, o, g, w)
+    sync()
+    dense = so.mask_global_no_local_dense(n, globs, w)
+    _check_heads(q, k, v, o, m, l, lambda a, b, c: so.dense_masked_attention(a, b, c, dense), dtype)
 
 
 def test_global_indices_need_not_be_sorted(mods):
