@@ -81,7 +81,9 @@ __global__ __launch_bounds__(256) void grad_prologue_kernel(Tensors t, GradArgs 
   const float l = load_state<T>(t.l, row, sf);
   const bool live = l > 0.f;
   float acc = 0.f;
-  if (live) {
+  // (the rows are read whether the row is live or not, so that their loads do not wait for l; a
+  // dead row's product - its out row may hold NaN - is dropped below)
+  {
     const T* orow = (const T*)t.out + row * t.d;
     const T* drow = (const T*)g.d_out + row * t.d;
     if ((t.d % V) == 0 && (((uintptr_t)t.out | (uintptr_t)g.d_out) & 15) == 0) {
