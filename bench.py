@@ -661,8 +661,10 @@ def measured_gather_ceiling(lib, w, torch, min_entries=8_000_000, reps=5, tensor
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--steps", type=int, default=None,
+                    help="timed steps (default 20; 200 for the workloads whose call takes less than 0.2 ms, "
+                         "which 20 steps would time while the clocks are still ramping up)")
+    ap.add_argument("--warmup", type=int, default=None, help="untimed steps before them (default 3; 20)")
     ap.add_argument("--workload", default="csr_zipf", choices=sorted(WORKLOADS))
     ap.add_argument("--dtype", default="f32", choices=["f32", "f16", "bf16"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
@@ -688,6 +690,11 @@ def main():
                     help="after the timed region, run one plain 256 MiB device copy (a kernel of known "
                          "traffic that counter runs use to scale FETCH_SIZE / WRITE_SIZE)")
     a = ap.parse_args()
+    short = a.workload in ("local", "local_2d", "local_1d", "csr_bernoulli", "global") and not a.backward
+    if a.steps is None:
+        a.steps = 200 if short else 20
+    if a.warmup is None:
+        a.warmup = 20 if short else 3
     if a.gpus != 1:
         sys.exit("bench.py measures one GPU: this path is a single-GPU kernel and every box here has "
                  "one GPU; run with --gpus 1")
@@ -709,7 +716,7 @@ def main():
 
     n_states = a.steps + a.warmup
     state_bytes = max(1, a.heads) * n * d * torch.tensor([], dtype=dtype).element_size()
-    n_alloc = max(1, min(n_states, int(4e9 // max(1, state_bytes))))
+    n_alloc = max(1, min(n_states, int(32e9 // max(1, state_bytes))))
     def new_state():
         if a.heads > 1:
             per = [syn.fresh_state(n, d, dtype=dtype, device="cuda", state_dtype=torch.float32)
