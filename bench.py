@@ -864,7 +864,9 @@ def main():
         if a.workload == "global":
             kernel_flops = 4.0 * d * w["n_global_rows_nnz"]
             kernel_bytes = 2 * n * d * es
-            kernel_name = "tile_kernel (global rows)"
+            # (half types, at most 64 listed tokens, d = 32 / 64: the streaming row kernel)
+            streamed = a.dtype != "f32" and w["params"]["n_globals"] <= 64 and d in (32, 64)
+            kernel_name = "global_rows_dma_kernel" if streamed else "tile_kernel (global rows)"
             w = dict(w, kernel_bytes=kernel_bytes, kernel_nnz=w["n_global_rows_nnz"],
                      kernel_rows=w["params"]["n_globals"])
         else:
