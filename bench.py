@@ -662,9 +662,10 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=None,
-                    help="timed steps (default 20; 200 for the workloads whose call takes less than 0.2 ms, "
-                         "which 20 steps would time while the clocks are still ramping up)")
-    ap.add_argument("--warmup", type=int, default=None, help="untimed steps before them (default 3; 20)")
+                    help="timed steps (default 20; 200 for the workloads whose call takes less than 0.2 ms and 100 "
+                         "for the gradient calls of all but the COO workloads, which 20 steps would time "
+                         "while the clocks are still ramping up)")
+    ap.add_argument("--warmup", type=int, default=None, help="untimed steps before them (default 3; 20; 10)")
     ap.add_argument("--workload", default="csr_zipf", choices=sorted(WORKLOADS))
     ap.add_argument("--dtype", default="f32", choices=["f32", "f16", "bf16"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
@@ -691,10 +692,11 @@ def main():
                          "traffic that counter runs use to scale FETCH_SIZE / WRITE_SIZE)")
     a = ap.parse_args()
     short = a.workload in ("local", "local_2d", "local_1d", "csr_bernoulli", "global") and not a.backward
+    short_bwd = a.backward and not a.workload.startswith("coo")
     if a.steps is None:
-        a.steps = 200 if short else 20
+        a.steps = 200 if short else 100 if short_bwd else 20
     if a.warmup is None:
-        a.warmup = 20 if short else 3
+        a.warmup = 20 if short else 10 if short_bwd else 3
     if a.gpus != 1:
         sys.exit("bench.py measures one GPU: this path is a single-GPU kernel and every box here has "
                  "one GPU; run with --gpus 1")

@@ -565,6 +565,17 @@ __global__ __launch_bounds__(256, (KEYS && D == 128 && PART == 0) ? 1 : 2) void 
   if (t0 >= len) return;
   const int u_lo = t0 > wlim ? t0 - wlim : 0;
   const int u_hi = (len - BM - wlim > t0) ? t0 + BM + wlim : len;
+  // The streamed tiles are visited in a rotated order, as in band_dma_kernel: visit number `it`
+  // is the tile whose number along the subsequence is `it` modulo the tile count, so that the
+  // workgroups of neighbouring owner tiles (resident at the same time, in the same XCD) ask for
+  // the same tile at about the same time.  (The sums do not care about the order.)
+  const int nk = (u_hi - u_lo + BN - 1) / BN;
+  const int rot0 = uni((nk - (int)(((uint32_t)tile * (uint32_t)(BM / BN)) % (uint32_t)nk)) % nk);
+  auto tile_start = [&](int it) __attribute__((always_inline)) {
+    int j = rot0 + it;
+    j = j >= nk ? j - nk : j;
+    return u_lo + j * BN;
+  };
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -619,7 +630,7 @@ __global__ __launch_bounds__(256, (KEYS && D == 128 && PART == 0) ? 1 : 2) void 
   };
 #pragma unroll
   for (int i = 0; i < NBUF - 1; i++)
-    if (u_lo + i * BN < u_hi) request(u_lo + i * BN, i);
+    if (i < nk) request(tile_start(i), i);
 
   const int tw0 = t0 + 32 * wave;  // first owner of this wavefront
   const int tq = tw0 + r;          // this lane's owner position
@@ -681,13 +692,14 @@ __global__ __launch_bounds__(256, (KEYS && D == 128 && PART == 0) ? 1 : 2) void 
   const uint32_t end_hi = (uint32_t)(u_hi - 1 - tq) + w32;
   const uint32_t band_hi = own_ok && end_hi < w2 ? end_hi : w2;
 
-  auto step = [&](int ut, int stage) __attribute__((always_inline)) {
+  auto step = [&](int it, int stage) __attribute__((always_inline)) {
+    const int ut = tile_start(it);
     const char* xs = lds + stage * BUF_B;
     const char* ys = xs + TILE_B;
     const float* lse_s = reinterpret_cast<const float*>(stat + stage * C::STAT_B);
     const float* delta_s = lse_s + BN;
     if constexpr (NBUF > 2) {
-      const int after = (u_hi - ut - 1) / BN;  // tiles behind this one
+      const int after = nk - 1 - it;  // tiles behind this one
       if (after >= 2) SPFA_WAIT_VMCNT(2 * LOADS);
       else if (after == 1) SPFA_WAIT_VMCNT(LOADS);
       else SPFA_WAIT_VMCNT(0);
@@ -695,7 +707,7 @@ __global__ __launch_bounds__(256, (KEYS && D == 128 && PART == 0) ? 1 : 2) void 
       SPFA_WAIT_VMCNT(0);
     }
     __syncthreads();  // the tile has landed for everyone, and everyone is done with the stage before it
-    if (ut + (NBUF - 1) * BN < u_hi) request(ut + (NBUF - 1) * BN, (stage + NBUF - 1) % NBUF);
+    if (it + NBUF - 1 < nk) request(tile_start(it + NBUF - 1), (stage + NBUF - 1) % NBUF);
 
     const uint32_t d0 = (uint32_t)(ut - tq) + w32;
 #pragma unroll
@@ -763,10 +775,10 @@ __global__ __launch_bounds__(256, (KEYS && D == 128 && PART == 0) ? 1 : 2) void 
     }
   };
 
-  for (int ut = u_lo; ut < u_hi; ut += NBUF * BN) {
+  for (int it = 0; it < nk; it += NBUF) {
 #pragma unroll
     for (int sg = 0; sg < NBUF; sg++)
-      if (ut + sg * BN < u_hi) step(ut + sg * BN, sg);
+      if (it + sg < nk) step(it + sg, sg);
   }
 
   // ---- add into the owner's gradient rows (g[eb][v] is element 32*eb + 8*(v/4) + 4*h + v%4)
