@@ -123,9 +123,9 @@ def _source_loop_depth(kname: str) -> int:
     batches (it is unrolled otherwise)."""
     import re
     if "11tile_kernelI" in kname:
-        # key-tile loop; the global-columns mode (third template argument 2) also loops over
-        # query tiles
-        return 2 if re.search(r"Li2EEEv", kname) else 1
+        # key-tile loop; the global-columns mode (third template argument 2, before the flag for
+        # padded rows) also loops over query tiles
+        return 2 if re.search(r"Li2ELb[01]EEEv", kname) else 1
     whole = "17whole_rows_kernelI" in kname  # (a medium-row walk inside its loop over long rows)
     med = "18medium_rows_kernelI" in kname or whole
     if "15segments_kernelI" not in kname and "11rows_kernelI" not in kname and not med:
