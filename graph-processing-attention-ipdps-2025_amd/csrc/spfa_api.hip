@@ -625,7 +625,17 @@ int spfa_local_1d_dilated_forward(const spfa_problem_t* p, int64_t local_size, i
   {
     const int64_t len_max = (n + dil_factor) / (dil_factor + 1);
     const int64_t span = 2 * local_size + 1 < len_max ? 2 * local_size + 1 : len_max;
-    if (span >= kBandTileMinRow && dtype_ok(p->dtype) && local_size <= kTileMaxWindow) {
+    // A tile costs the same whatever part of it is live, a gathered row costs by the candidate.
+    // Measured crossovers of the window kernels (N = 65536 ... 262144, d = 32 ... 256): 5 - 7
+    // candidates per row for the half types, 11 - 27 for fp32 (whose matrix instructions are
+    // sixteen times slower); a call of fewer rows is bound by its launch either way and stays on
+    // the gather engine up to the general limit.
+    int64_t min_row = kBandTileMinRow;
+    if (n * batch_of(p) >= 32768) {
+      if (p->dtype != SPFA_DTYPE_F32) min_row = 7;
+      else min_row = p->d <= 32 ? 13 : p->d <= 64 ? 21 : p->d <= 128 ? 13 : 27;
+    }
+    if (span >= min_row && dtype_ok(p->dtype) && local_size <= kTileMaxWindow) {
       rc = dispatch_band(p, local_size, dil_factor + 1, 0, 0, 0, (hipStream_t)stream);
       if (rc >= 0) return rc;
     }

@@ -7,9 +7,12 @@ from oracle import spfa_oracle as so
 
 # max-abs bars on the output: fp32 1e-4, half types 2e-2
 OUT_TOL = {torch.float32: 1e-4, torch.float16: 2e-2, torch.bfloat16: 2e-2, torch.float64: 1e-11}
-# bar on m + log(l): fp32 statistics 1e-4 / 2e-3 (half inputs, fp32 state); statistics stored in
+# bar on m + log(l): fp32 statistics 1e-4 / 2e-3 (fp16 inputs, fp32 state) / 3e-3 (bf16: where the
+# tile kernels take the row sum off the matrix pipe, l is the sum of the weights as rounded to
+# bf16 for the second product - the ones the numerator is built from - and a row that one weight
+# dominates carries that weight's rounding, up to 2^-9 = 1.95e-3 relative); statistics stored in
 # a half type carry that type's rounding of m (|m| up to ~10): 1e-1
-LSE_TOL_F32_STATE = {torch.float32: 1e-4, torch.float16: 2e-3, torch.bfloat16: 2e-3}
+LSE_TOL_F32_STATE = {torch.float32: 1e-4, torch.float16: 2e-3, torch.bfloat16: 3e-3}
 LSE_TOL_F64 = 1e-11
 LSE_TOL_HALF_STATE = 1e-1
 

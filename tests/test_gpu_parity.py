@@ -917,6 +917,29 @@ def test_local_2d_dilated(mods, dtype, d, n, block, dil, use_nan):
     check(o, m, l, *ref, dtype, state_dtype=torch.float32, dead_expect="nan" if use_nan else None)
 
 
+@pytest.mark.parametrize("dtype,d", [(torch.bfloat16, 64), (torch.float16, 128), (torch.bfloat16, 32),
+                                     (torch.float16, 256), (torch.bfloat16, 96), (torch.float32, 32),
+                                     (torch.float32, 64), (torch.float32, 128), (torch.float32, 256),
+                                     (torch.float32, 40)])
+@pytest.mark.parametrize("w,dil", [(1, 0), (3, 0), (6, 0), (6, 2), (10, 1), (13, 0), (15, 3)])
+def test_narrow_windows_in_calls_of_many_rows(mods, dtype, d, w, dil):
+    """From 32768 rows on, windows of a few candidates per row already run on the tiles (from 7
+    candidates for the half types, 13 - 27 for fp32 depending on d); below, on the row-gather
+    engine.  Both sides of every limit against the oracle."""
+    n = 33001
+    q, k, v = dev_qkv(n, d, dtype, 40, scale=0.7)
+    m, l, o = state(n, d, dtype, torch.float32)
+    mods["spfa_local_1d_dilated"].forward(q, k, v, m, l, o, w, dil)
+    sync()
+    ref = c_oracle.local_1d_dilated(np64(q), np64(k), np64(v), w, dil)
+    check(o, m, l, *ref, dtype, state_dtype=torch.float32)
+    if dil == 0:
+        m, l, o = state(n, d, dtype, torch.float32)
+        mods["spfa_local"].forward(q, k, v, m, l, o, w)
+        sync()
+        check(o, m, l, *ref, dtype, state_dtype=torch.float32)
+
+
 @pytest.mark.parametrize("dtype,d", [(torch.float32, 4), (torch.float32, 40), (torch.float32, 100),
                                      (torch.float32, 132), (torch.float32, 252), (torch.bfloat16, 8),
                                      (torch.bfloat16, 40), (torch.float16, 80), (torch.bfloat16, 104),
