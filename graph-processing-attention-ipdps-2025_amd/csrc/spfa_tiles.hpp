@@ -2434,7 +2434,9 @@ int launch_band_tiles(const TileArgs& a, int use_nan, hipStream_t stream) {
         const int64_t resident = (int64_t)device_cu_count() * (D > 128 ? 1 : 2);
         const int64_t rem = n_all % resident;
         constexpr bool kFoldFits = 2 * (BC::EB * 16 + 3) * kWave * 4 <= BC::NBUF * BC::BUF_B;
-        at.n_tail = (kFoldFits && a.globs == nullptr && n_all > resident && 4 * rem <= resident) ? rem : 0;
+        // (a problem of at most an eighth of a round: every such workgroup has a CU to itself)
+        const bool few = n_all > resident ? 4 * rem <= resident : 8 * rem <= resident;
+        at.n_tail = (kFoldFits && a.globs == nullptr && few) ? rem : 0;
         const int64_t grid_d = (n_all - at.n_tail + 7) / 8 * 8 + 4 * at.n_tail;
         launch_maybe_timed(ev, band_dma_kernel<T, D, SPFA_BAND_BN(D)>, dim3((unsigned)grid_d), dim3(256), stream, at);
       }
