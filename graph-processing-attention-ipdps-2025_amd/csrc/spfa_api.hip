@@ -243,6 +243,24 @@ constexpr int64_t kBandTileMinRow = 32;
 // the tile kernels test windows in 32-bit arithmetic: (unsigned)(delta + w) <= 2w
 constexpr int64_t kTileMaxWindow = (int64_t)1 << 30;
 
+// Shortest row (candidates per query, 2w + 1) of a window mask that goes to the tiles.  A tile
+// costs the same whatever part of it is live, a gathered row costs by the candidate.  Measured
+// crossovers of the window kernels (N = 32768 ... 262144, d = 32 ... 256): forward 5 - 7
+// candidates per row for the half types and 11 - 27 for fp32 (whose matrix instructions are
+// sixteen times slower); the gradient call, whose gather passes cost more per candidate, below
+// 3 for the half types and for fp32 at d = 32, 11 at d = 64, 27 at d = 128.  A call of fewer rows
+// is bound by its launches either way and stays on the gather engine up to the general limit.
+int64_t window_tile_min_row(const spfa_problem_t* p, bool gradient) {
+  if (p->n_q * batch_of(p) < 32768) return kBandTileMinRow;
+  const bool f32 = p->dtype == SPFA_DTYPE_F32;
+  if (gradient) {
+    if (!f32 || p->d <= 32) return 3;
+    return p->d <= 64 ? 13 : p->d <= 128 ? 27 : kBandTileMinRow;
+  }
+  if (!f32) return 7;
+  return p->d <= 32 ? 13 : p->d <= 64 ? 21 : p->d <= 128 ? 13 : 27;
+}
+
 int dispatch_global(const spfa_problem_t* p, const GlobalMask& mask, const EngineSizing& s,
                     void* ws, hipStream_t stream) {
   Tensors t = make_tensors(p);
@@ -630,17 +648,7 @@ int spfa_local_1d_dilated_forward(const spfa_problem_t* p, int64_t local_size, i
   {
     const int64_t len_max = (n + dil_factor) / (dil_factor + 1);
     const int64_t span = 2 * local_size + 1 < len_max ? 2 * local_size + 1 : len_max;
-    // A tile costs the same whatever part of it is live, a gathered row costs by the candidate.
-    // Measured crossovers of the window kernels (N = 65536 ... 262144, d = 32 ... 256): 5 - 7
-    // candidates per row for the half types, 11 - 27 for fp32 (whose matrix instructions are
-    // sixteen times slower); a call of fewer rows is bound by its launch either way and stays on
-    // the gather engine up to the general limit.
-    int64_t min_row = kBandTileMinRow;
-    if (n * batch_of(p) >= 32768) {
-      if (p->dtype != SPFA_DTYPE_F32) min_row = 7;
-      else min_row = p->d <= 32 ? 13 : p->d <= 64 ? 21 : p->d <= 128 ? 13 : 27;
-    }
-    if (span >= min_row && dtype_ok(p->dtype) && local_size <= kTileMaxWindow) {
+    if (span >= window_tile_min_row(p, false) && dtype_ok(p->dtype) && local_size <= kTileMaxWindow) {
       rc = dispatch_band(p, local_size, dil_factor + 1, 0, 0, 0, (hipStream_t)stream);
       if (rc >= 0) return rc;
     }
@@ -1186,7 +1194,7 @@ int spfa_local_1d_dilated_backward(const spfa_problem_t* p, const spfa_grads_t* 
   StrideMask mask{n, local_size, dil_factor + 1, 0, 0};
   const int64_t len_max = (n + dil_factor) / (dil_factor + 1);
   const int64_t span = 2 * local_size + 1 < len_max ? 2 * local_size + 1 : len_max;
-  const bool tiles = span >= kBandTileMinRow && local_size <= kTileMaxWindow;
+  const bool tiles = span >= window_tile_min_row(p, true) && local_size <= kTileMaxWindow;
   return stride_backward(p, g, mask, tiles, lay, workspace, (hipStream_t)stream);
 }
 

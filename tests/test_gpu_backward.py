@@ -138,6 +138,22 @@ def test_band_masks_on_the_tile_path(mods, dtype, d):
             _check_grads([x[b] for x in got], ref, dtype, "%s batch %d" % (parts[0][0], b))
 
 
+@pytest.mark.parametrize("dtype,d", [(torch.bfloat16, 64), (torch.float16, 128), (torch.bfloat16, 32),
+                                     (torch.float32, 32), (torch.float32, 64), (torch.float32, 128)])
+@pytest.mark.parametrize("w,dil", [(1, 0), (2, 1), (5, 0), (6, 0), (12, 2), (13, 0)])
+def test_narrow_windows_in_calls_of_many_rows(mods, dtype, d, w, dil):
+    """From 32768 rows on (16 problems of 2100 tokens here) the gradient of a window mask runs on
+    the tiles from 3 candidates per row for the half types and fp32 at d = 32, from 13 / 27 for
+    fp32 at d = 64 / 128; both sides of the limits against the oracle (first and last problem)."""
+    n, lead = 2100, (16,)
+    q, k, v, d_out = _problem(n, d, dtype, 93, lead=lead)
+    dense = so.mask_local_1d_dilated_dense(n, w, dil)
+    _, got = _grads_of(q, k, v, d_out, [("local_1d_dilated", w, dil)])
+    for b in (0, lead[0] - 1):
+        ref = so.dense_masked_attention_backward(np64(q[b]), np64(k[b]), np64(v[b]), dense, np64(d_out[b]))
+        _check_grads([x[b] for x in got], ref, dtype, "w=%d dil=%d problem %d" % (w, dil, b))
+
+
 @pytest.mark.parametrize("dtype", [torch.float64, torch.float32])
 def test_chained_parts_are_differentiated_as_their_union(mods, dtype):
     """window + global + random, the chain of verification/verify.py:337-352: one backward call
