@@ -40,6 +40,15 @@ constexpr int64_t kExplicitInlineRowLimit = 32;
 // ms); 64 heads of the 2 % Bernoulli mask (rows of ~83) need it above their row length (3.03 ms
 // without, 0.65 with).
 constexpr int64_t kExplicitMediumRowLimit = 256;
+// ... and rows of up to this many when K and V are small enough to stay in the caches: the
+// persistent kernel (one wavefront per SIMD, tuned for the latency of memory-side fills) then
+// leaves most of the cache bandwidth unused on single-segment rows, which an ordinary grid of
+// eight wavefronts per SIMD does not.  Uniform rows of 257 ... 1000 entries, limit 256 -> 1024:
+// 8192 tokens at d = 64 fp32 4.9 ... 12.5 -> 13.2 ... 20.9 TB/s of gathered rows, 20000 tokens bf16
+// 4.8 ... 8.5 -> 12.1 ... 19.0; at K + V = 32 MiB the two are level, beyond that the persistent kernel
+// is ahead (the Zipf headline, 64 MiB: + 2.4 % with 1024 for every size).
+constexpr int64_t kExplicitMediumRowLimitCached = 1024;
+constexpr int64_t kCachedKvBytes = (int64_t)24 << 20;
 
 EngineSizing size_csr(int64_t n_q, int64_t nnz) {
   EngineSizing s{};
@@ -50,6 +59,13 @@ EngineSizing size_csr(int64_t n_q, int64_t nnz) {
   s.seg = pick_segment(nnz);
   s.n_long_bound = n_q;
   return s;
+}
+
+// the medium-row limit of a plain call (a mask plan is built without knowing K and V)
+int64_t explicit_medium_limit(const spfa_problem_t* p) {
+  const int64_t es = p->dtype == SPFA_DTYPE_F32 ? 4 : p->dtype == SPFA_DTYPE_F64 ? 8 : 2;
+  const int64_t kv = 2 * p->n_k * p->d * es * (p->n_batch > 1 ? p->n_batch : 1);
+  return kv <= kCachedKvBytes ? kExplicitMediumRowLimitCached : kExplicitMediumRowLimit;
 }
 
 // Band / block masks are uniform: every row has about the same number of candidates, so rows
@@ -429,6 +445,7 @@ int spfa_csr_forward(const spfa_problem_t* p, const void* row_off, int row_off_b
     return run_f64(make_tensors(p), mask, use_nan ? 1 : 0, (hipStream_t)stream);
   }
   EngineSizing s = size_csr(p->n_q, nnz);
+  s.medium_max = explicit_medium_limit(p);
   if (!batch_fits_engine(s, p)) {
     for (int64_t b = 0; b < batch_of(p); b++) {
       const spfa_problem_t one = batch_slice(p, b);
@@ -521,6 +538,7 @@ int spfa_coo_forward(const spfa_problem_t* p, const void* row_ind, int row_ind_b
   if (p->n_q == 0) return SPFA_OK;
   if (nnz > 0 && (!row_ind || !col_ind)) return SPFA_ERR_BAD_ARG;
   EngineSizing s = size_csr(p->n_q, nnz);
+  s.medium_max = explicit_medium_limit(p);
   const size_t coo_bytes = coo_workspace(p->n_q, nnz).total;
   const bool batched = batch_fits_engine(s, p);
   rc = check_workspace(workspace, workspace_bytes,
