@@ -63,9 +63,10 @@ constexpr int grad_tile_min_blocks() {
   return (D > 64 && (KEYS || sizeof(T) == 4)) ? 1 : 2;
 }
 
-template <typename T, int D, bool KEYS, int MODE>
+template <typename T, int D, bool KEYS, int MODE, bool PAD = false>
 __global__ __launch_bounds__(256, (grad_tile_min_blocks<T, D, KEYS>())) void tile_grad_kernel(TileArgs a,
                                                                                              GradArgs g) {
+  static_assert(!PAD || MODE == kTileBand, "padded rows: band and block masks only");
   using C = GradTileCfg<T, D>;
   constexpr bool kF32 = C::kF32;
   constexpr int BM = C::BM, BN = C::BN, EB = C::EB, NB = C::NB, ST = C::STRIDE;
@@ -137,7 +138,11 @@ __global__ __launch_bounds__(256, (grad_tile_min_blocks<T, D, KEYS>())) void til
   const T* Bp = (const T*)(KEYS ? g.v : g.d_out);
   const T* Xp = (const T*)(KEYS ? g.q : g.k);      // streamed rows
   const T* Yp = (const T*)(KEYS ? g.d_out : g.v);
-  const float scale = 1.0f / sqrtf((float)D);
+  // PAD: rows of dr < D elements (a multiple of 16 bytes); the owner vectors and the streamed
+  // tiles are filled up with zeros, which add nothing to a product, and the gradient elements
+  // from dr on are not written
+  const int dr = PAD ? (int)a.t.d : D;
+  const float scale = 1.0f / sqrtf((float)dr);
   const float sc = 1.4426950408889634f * scale;
 
   // GlobalRows with at most 64 listed tokens: only two wavefronts would have owners.  Wavefronts
@@ -171,16 +176,19 @@ __global__ __launch_bounds__(256, (grad_tile_min_blocks<T, D, KEYS>())) void til
   uint4v ah[kF32 ? 1 : C::AREGS], bh[kF32 ? 1 : C::AREGS];
   float af[kF32 ? C::AREGS : 1], bf[kF32 ? C::AREGS : 1];
   {
-    const T* arow = Ap + own_row * D;
-    const T* brow = Bp + own_row * D;
+    const T* arow = Ap + own_row * dr;
+    const T* brow = Bp + own_row * dr;
     if constexpr (kF32) {
       // the 32x32x2 product takes two k per instruction, one per half of the wavefront: half h
       // takes k = h * D/2 + ks in step ks (any pairing works as long as both operands use it),
       // so that a lane's operands are consecutive in memory and in LDS
 #pragma unroll
       for (int c4 = 0; c4 < D / 8; c4++) {
-        const float4v x = *reinterpret_cast<const float4v*>(arow + h * (D / 2) + 4 * c4);
-        const float4v y = *reinterpret_cast<const float4v*>(brow + h * (D / 2) + 4 * c4);
+        float4v x = {0.f, 0.f, 0.f, 0.f}, y = {0.f, 0.f, 0.f, 0.f};
+        if (!PAD || h * (D / 2) + 4 * c4 < dr) {
+          x = *reinterpret_cast<const float4v*>(arow + h * (D / 2) + 4 * c4);
+          y = *reinterpret_cast<const float4v*>(brow + h * (D / 2) + 4 * c4);
+        }
 #pragma unroll
         for (int i = 0; i < 4; i++) {
           af[4 * c4 + i] = x[i];
@@ -190,8 +198,12 @@ __global__ __launch_bounds__(256, (grad_tile_min_blocks<T, D, KEYS>())) void til
     } else {
 #pragma unroll
       for (int ks = 0; ks < C::AREGS; ks++) {
-        ah[ks] = *reinterpret_cast<const uint4v*>(arow + 16 * ks + 8 * h);
-        bh[ks] = *reinterpret_cast<const uint4v*>(brow + 16 * ks + 8 * h);
+        ah[ks] = uint4v{0u, 0u, 0u, 0u};
+        bh[ks] = uint4v{0u, 0u, 0u, 0u};
+        if (!PAD || 16 * ks + 8 * h < dr) {
+          ah[ks] = *reinterpret_cast<const uint4v*>(arow + 16 * ks + 8 * h);
+          bh[ks] = *reinterpret_cast<const uint4v*>(brow + 16 * ks + 8 * h);
+        }
       }
     }
   }
@@ -235,8 +247,8 @@ __global__ __launch_bounds__(256, (grad_tile_min_blocks<T, D, KEYS>())) void til
       const int j = idx / CH, c = idx % CH;
       const int64_t u = ut + j;
       uint4v xx = {0u, 0u, 0u, 0u}, yy = {0u, 0u, 0u, 0u};
-      if (u < u_hi) {
-        const int64_t off = streamed_row(u) * D + (16 / (int)sizeof(T)) * c;
+      if (u < u_hi && (!PAD || (16 / (int)sizeof(T)) * c < dr)) {
+        const int64_t off = streamed_row(u) * dr + (16 / (int)sizeof(T)) * c;
         xx = *reinterpret_cast<const uint4v*>(Xp + off);
         yy = *reinterpret_cast<const uint4v*>(Yp + off);
       }
@@ -442,8 +454,8 @@ __global__ __launch_bounds__(256, (grad_tile_min_blocks<T, D, KEYS>())) void til
   // types and (D/32)*i + eb for fp32, i = 8*(v/4) + 4*h + v%4: four registers of one block, or of
   // all blocks, are four adjacent elements
   if (!own_ok) return;
-  float* out1 = (KEYS ? g.d_k : g.d_q) + own_row * D;
-  float* out2 = KEYS ? g.d_v + own_row * D : nullptr;
+  float* out1 = (KEYS ? g.d_k : g.d_q) + own_row * dr;
+  float* out2 = KEYS ? g.d_v + own_row * dr : nullptr;
 #pragma unroll
   for (int oc = 0; oc < EB; oc++)
 #pragma unroll
@@ -463,7 +475,7 @@ __global__ __launch_bounds__(256, (grad_tile_min_blocks<T, D, KEYS>())) void til
         float* p1 = a.pacc + (slot0 * a.n_globs + tq) * D + e;
         *reinterpret_cast<float4v*>(p1) = x;
         if constexpr (KEYS) *reinterpret_cast<float4v*>(p1 + a.n_globs * D) = y;
-      } else {
+      } else if (!PAD || e < dr) {
         float4v x0 = *reinterpret_cast<const float4v*>(out1 + e);
 #pragma unroll
         for (int u = 0; u < 4; u++) x0[u] += x[u];
@@ -852,6 +864,22 @@ int launch_band_grad(const TileArgs& a, const GradArgs& g, hipStream_t stream) {
   return hipGetLastError() == hipSuccess ? 0 : 4;
 }
 
+// Rows of a.t.d < D elements, D the next multiple of 32 the tile kernel is built for: the
+// register-staged kernel with zero-filled operands (the forward tiles' rule).
+template <typename T, int D>
+int launch_band_grad_padded(const TileArgs& a, const GradArgs& g, hipStream_t stream) {
+  const int64_t rows = g.n_q * g.n_batch;
+  if (rows == 0 || a.n_tiles == 0) return 0;
+  hipLaunchKernelGGL((grad_prologue_kernel<T>), dim3((unsigned)((rows + 15) / 16)), dim3(256), 0, stream,
+                     a.t, g);
+  const int64_t grid = (a.n_tiles * a.t.n_batch + 7) / 8 * 8;
+  hipLaunchKernelGGL((tile_grad_kernel<T, D, false, kTileBand, true>), dim3((unsigned)grid), dim3(256), 0,
+                     stream, a, g);
+  hipLaunchKernelGGL((tile_grad_kernel<T, D, true, kTileBand, true>), dim3((unsigned)grid), dim3(256), 0,
+                     stream, a, g);
+  return hipGetLastError() == hipSuccess ? 0 : 4;
+}
+
 // Adds the partial sums of the GlobalRows passes into the gradient rows of the listed tokens.
 // Grid: x = (problem, listed token), y = a chunk of the splits; a thread per element of (g1, g2)
 // sums its chunk and adds it to the row with one atomic (gridDim.y adds per address).
@@ -909,8 +937,22 @@ int launch_global_grad(const TileArgs& a, const GradArgs& g, hipStream_t stream)
 // Returns -1 when the shape is not covered (the caller then runs the gather passes).
 template <typename T>
 int run_band_grad_tiles(const TileArgs& a, const GradArgs& g, hipStream_t stream) {
-  if (!tile_shape_ok(a.t, sizeof(T))) return -1;
   if (((uintptr_t)g.d_out | (uintptr_t)g.d_q | (uintptr_t)g.d_k | (uintptr_t)g.d_v) & 15) return -1;
+  if (a.t.d % 32 != 0) {
+    // rows of whole 16-byte pieces: the tiles of the next multiple of 32 that is built
+    if (!tile_shape_padded_ok<T>(a.t)) return -1;
+    const int64_t dp = (a.t.d + 31) / 32 * 32;
+    if (dp == 32) return launch_band_grad_padded<T, 32>(a, g, stream);
+    if (dp == 64) return launch_band_grad_padded<T, 64>(a, g, stream);
+    if (dp == 96) return launch_band_grad_padded<T, 96>(a, g, stream);
+    if (dp == 128) return launch_band_grad_padded<T, 128>(a, g, stream);
+    if constexpr (sizeof(T) == 2) {
+      if (dp == 160) return launch_band_grad_padded<T, 160>(a, g, stream);
+      if (dp == 192) return launch_band_grad_padded<T, 192>(a, g, stream);
+    }
+    return -1;
+  }
+  if (!tile_shape_ok(a.t, sizeof(T))) return -1;
   if (a.t.d == 64) return launch_band_grad<T, 64>(a, g, stream);
   if (a.t.d == 128) return launch_band_grad<T, 128>(a, g, stream);
   if (a.t.d == 32) return launch_band_grad<T, 32>(a, g, stream);

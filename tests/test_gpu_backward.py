@@ -138,6 +138,34 @@ def test_band_masks_on_the_tile_path(mods, dtype, d):
             _check_grads([x[b] for x in got], ref, dtype, "%s batch %d" % (parts[0][0], b))
 
 
+@pytest.mark.parametrize("dtype,d", [(torch.float32, 4), (torch.float32, 40), (torch.float32, 100),
+                                     (torch.float32, 124), (torch.bfloat16, 8), (torch.bfloat16, 40),
+                                     (torch.float16, 80), (torch.bfloat16, 104), (torch.float16, 136),
+                                     (torch.bfloat16, 184), (torch.float16, 200)])
+def test_band_masks_rows_that_are_no_multiple_of_32(mods, dtype, d):
+    """Rows of whole 16-byte pieces on the gradient tiles of the next multiple of 32 that is built
+    (zero-filled operands; d = 200 has none and takes the gather passes): window, dilation, blocks,
+    sequence ends inside a tile, a stacked batch."""
+    cases = [
+        (517, [("local", 16)], lambda n: so.mask_local_dense(n, 16)),
+        (700, [("local", 150)], lambda n: so.mask_local_dense(n, 150)),
+        (1000, [("local_1d_dilated", 40, 2)], lambda n: so.mask_local_1d_dilated_dense(n, 40, 2)),
+        (768, [("local_2d_dilated", 256, 1)], lambda n: so.mask_local_2d_dilated_dense(n, 256, 1)),
+    ]
+    for n, parts, mask_fn in cases:
+        q, k, v, d_out = _problem(n, d, dtype, 94)
+        ref = so.dense_masked_attention_backward(np64(q), np64(k), np64(v), mask_fn(n), np64(d_out))
+        _, got = _grads_of(q, k, v, d_out, parts)
+        _check_grads(got, ref, dtype, "%s n=%d" % (parts[0], n))
+    n, lead = 400, (3,)
+    q, k, v, d_out = _problem(n, d, dtype, 95, lead=lead)
+    dense = so.mask_local_dense(n, 50)
+    _, got = _grads_of(q, k, v, d_out, [("local", 50)])
+    for b in range(lead[0]):
+        ref = so.dense_masked_attention_backward(np64(q[b]), np64(k[b]), np64(v[b]), dense, np64(d_out[b]))
+        _check_grads([x[b] for x in got], ref, dtype, "batch %d" % b)
+
+
 @pytest.mark.parametrize("dtype,d", [(torch.bfloat16, 64), (torch.float16, 128), (torch.bfloat16, 32),
                                      (torch.float32, 32), (torch.float32, 64), (torch.float32, 128)])
 @pytest.mark.parametrize("w,dil", [(1, 0), (2, 1), (5, 0), (6, 0), (12, 2), (13, 0)])
