@@ -66,7 +66,6 @@ constexpr int grad_tile_min_blocks() {
 template <typename T, int D, bool KEYS, int MODE, bool PAD = false>
 __global__ __launch_bounds__(256, (grad_tile_min_blocks<T, D, KEYS>())) void tile_grad_kernel(TileArgs a,
                                                                                              GradArgs g) {
-  static_assert(!PAD || MODE == kTileBand, "padded rows: band and block masks only");
   using C = GradTileCfg<T, D>;
   constexpr bool kF32 = C::kF32;
   constexpr int BM = C::BM, BN = C::BN, EB = C::EB, NB = C::NB, ST = C::STRIDE;
@@ -472,9 +471,12 @@ __global__ __launch_bounds__(256, (grad_tile_min_blocks<T, D, KEYS>())) void til
       if constexpr (MODE == kTileGlobalRows) {
         // partial sums of this split (and half): [problem][split][half][which][listed token][D]
         const int64_t slot0 = ((part_bb * a.n_split + part_split) * 2 + (wave_k > 0 ? 1 : 0)) * (KEYS ? 2 : 1);
-        float* p1 = a.pacc + (slot0 * a.n_globs + tq) * D + e;
-        *reinterpret_cast<float4v*>(p1) = x;
-        if constexpr (KEYS) *reinterpret_cast<float4v*>(p1 + a.n_globs * D) = y;
+        // (rows of the real length: elements from dr on are padding)
+        float* p1 = a.pacc + (slot0 * a.n_globs + tq) * dr + e;
+        if (!PAD || e < dr) {
+          *reinterpret_cast<float4v*>(p1) = x;
+          if constexpr (KEYS) *reinterpret_cast<float4v*>(p1 + a.n_globs * dr) = y;
+        }
       } else if (!PAD || e < dr) {
         float4v x0 = *reinterpret_cast<const float4v*>(out1 + e);
 #pragma unroll
@@ -883,15 +885,16 @@ int launch_band_grad_padded(const TileArgs& a, const GradArgs& g, hipStream_t st
 // Adds the partial sums of the GlobalRows passes into the gradient rows of the listed tokens.
 // Grid: x = (problem, listed token), y = a chunk of the splits; a thread per element of (g1, g2)
 // sums its chunk and adds it to the row with one atomic (gridDim.y adds per address).
-template <typename T, int D>
+template <typename T, int D, bool PAD = false>
 __global__ __launch_bounds__(2 * D) void global_grad_merge_kernel(TileArgs a, GradArgs g, int keys) {
   const int64_t n_uq = (int64_t)*a.n_uq;
   const int64_t bb = blockIdx.x / a.n_globs;
   const int64_t t = blockIdx.x - bb * a.n_globs;
   if (t >= n_uq) return;
+  const int dd = PAD ? (int)a.t.d : D;  // (PAD: rows of a.t.d < D elements)
   const int which = threadIdx.x / D, e = threadIdx.x % D;
   const int n_which = keys ? 2 : 1;
-  if (which >= n_which) return;
+  if (which >= n_which || e >= dd) return;
   const int halves = (GradTileCfg<T, D>::NB == 2 && n_uq <= 64) ? 2 : 1;  // the tile kernel's pair split
   const int64_t per = (a.n_split + gridDim.y - 1) / gridDim.y;
   const int64_t sp0 = (int64_t)blockIdx.y * per;
@@ -900,17 +903,17 @@ __global__ __launch_bounds__(2 * D) void global_grad_merge_kernel(TileArgs a, Gr
   for (int64_t sp = sp0; sp < sp1; sp++)
     for (int hf = 0; hf < halves; hf++) {
       const int64_t slot = (((bb * a.n_split + sp) * 2 + hf) * n_which + which) * a.n_globs + t;
-      acc += a.pacc[slot * D + e];
+      acc += a.pacc[slot * dd + e];
     }
   if (sp0 >= sp1) return;
   const int64_t row = (int64_t)a.uq[t] + bb * a.n;
-  float* out = (keys ? (which ? g.d_v : g.d_k) : g.d_q) + row * D + e;
+  float* out = (keys ? (which ? g.d_v : g.d_k) : g.d_q) + row * dd + e;
   unsafeAtomicAdd(out, acc);
 }
 
 // Both passes of the global-minus-local mask: the ordinary tokens against the listed ones, then
 // the listed ones against everything (a: globs, n_globs, gbits, uq, n_uq, key_run, n_split set).
-template <typename T, int D>
+template <typename T, int D, bool PAD = false>
 int launch_global_grad(const TileArgs& a, const GradArgs& g, hipStream_t stream) {
   const int64_t rows = g.n_q * g.n_batch;
   if (rows == 0) return 0;
@@ -918,8 +921,8 @@ int launch_global_grad(const TileArgs& a, const GradArgs& g, hipStream_t stream)
                      a.t, g);
   const unsigned nb = (unsigned)a.t.n_batch;
   const dim3 grid_cols((unsigned)((a.n + 127) / 128), nb);
-  hipLaunchKernelGGL((tile_grad_kernel<T, D, false, kTileGlobalCols>), grid_cols, dim3(256), 0, stream, a, g);
-  hipLaunchKernelGGL((tile_grad_kernel<T, D, true, kTileGlobalCols>), grid_cols, dim3(256), 0, stream, a, g);
+  hipLaunchKernelGGL((tile_grad_kernel<T, D, false, kTileGlobalCols, PAD>), grid_cols, dim3(256), 0, stream, a, g);
+  hipLaunchKernelGGL((tile_grad_kernel<T, D, true, kTileGlobalCols, PAD>), grid_cols, dim3(256), 0, stream, a, g);
   const int64_t q_tiles = (a.n_globs + 127) / 128;
   const dim3 grid_rows((unsigned)(q_tiles * a.n_split * nb));
   // enough workgroups to fill the device, at least 8 splits each
@@ -927,10 +930,10 @@ int launch_global_grad(const TileArgs& a, const GradArgs& g, hipStream_t stream)
   if (chunks > a.n_split / 8) chunks = a.n_split / 8;
   if (chunks < 1) chunks = 1;
   const dim3 grid_merge((unsigned)(a.n_globs * nb), (unsigned)chunks);
-  hipLaunchKernelGGL((tile_grad_kernel<T, D, false, kTileGlobalRows>), grid_rows, dim3(256), 0, stream, a, g);
-  hipLaunchKernelGGL((global_grad_merge_kernel<T, D>), grid_merge, dim3(2 * D), 0, stream, a, g, 0);
-  hipLaunchKernelGGL((tile_grad_kernel<T, D, true, kTileGlobalRows>), grid_rows, dim3(256), 0, stream, a, g);
-  hipLaunchKernelGGL((global_grad_merge_kernel<T, D>), grid_merge, dim3(2 * D), 0, stream, a, g, 1);
+  hipLaunchKernelGGL((tile_grad_kernel<T, D, false, kTileGlobalRows, PAD>), grid_rows, dim3(256), 0, stream, a, g);
+  hipLaunchKernelGGL((global_grad_merge_kernel<T, D, PAD>), grid_merge, dim3(2 * D), 0, stream, a, g, 0);
+  hipLaunchKernelGGL((tile_grad_kernel<T, D, true, kTileGlobalRows, PAD>), grid_rows, dim3(256), 0, stream, a, g);
+  hipLaunchKernelGGL((global_grad_merge_kernel<T, D, PAD>), grid_merge, dim3(2 * D), 0, stream, a, g, 1);
   return hipGetLastError() == hipSuccess ? 0 : 4;
 }
 
@@ -967,8 +970,17 @@ int run_band_grad_tiles(const TileArgs& a, const GradArgs& g, hipStream_t stream
 
 template <typename T>
 int run_global_grad_tiles(const TileArgs& a, const GradArgs& g, hipStream_t stream) {
-  if (!tile_shape_ok(a.t, sizeof(T))) return -1;
   if (((uintptr_t)g.d_out | (uintptr_t)g.d_q | (uintptr_t)g.d_k | (uintptr_t)g.d_v) & 15) return -1;
+  if (a.t.d % 32 != 0) {
+    if (!tile_shape_padded_ok<T>(a.t)) return -1;
+    const int64_t dp = (a.t.d + 31) / 32 * 32;
+    if (dp == 32) return launch_global_grad<T, 32, true>(a, g, stream);
+    if (dp == 64) return launch_global_grad<T, 64, true>(a, g, stream);
+    if (dp == 96) return launch_global_grad<T, 96, true>(a, g, stream);
+    if (dp == 128) return launch_global_grad<T, 128, true>(a, g, stream);
+    return -1;
+  }
+  if (!tile_shape_ok(a.t, sizeof(T))) return -1;
   if (a.t.d == 64) return launch_global_grad<T, 64>(a, g, stream);
   if (a.t.d == 128) return launch_global_grad<T, 128>(a, g, stream);
   if (a.t.d == 32) return launch_global_grad<T, 32>(a, g, stream);

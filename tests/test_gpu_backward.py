@@ -164,6 +164,27 @@ def test_band_masks_rows_that_are_no_multiple_of_32(mods, dtype, d):
     for b in range(lead[0]):
         ref = so.dense_masked_attention_backward(np64(q[b]), np64(k[b]), np64(v[b]), dense, np64(d_out[b]))
         _check_grads([x[b] for x in got], ref, dtype, "batch %d" % b)
+    # the global mask (its gradient tiles are built up to d = 128): a few listed tokens, more than a
+    # tile of them with repeats, a batch
+    for n, gl, w in [(700, [3, 350, 699], 5), (900, list(range(2, 900, 6)) + [8, 8, 14], 0)]:
+        q, k, v, d_out = _problem(n, d, dtype, 96)
+        dense_w = so.mask_global_no_local_dense(n, gl, w)
+        ref = so.dense_masked_attention_backward(np64(q), np64(k), np64(v), dense_w, np64(d_out)) \
+            if len(set(gl)) == len(gl) else None
+        _, got = _grads_of(q, k, v, d_out, [("global_no_local", torch.tensor(gl, dtype=torch.int32, device=DEV), w)])
+        if ref is not None:
+            _check_grads(got, ref, dtype, "global n=%d" % n)
+        else:
+            # repeats (an ordinary row counts a listed token once per occurrence): against the same
+            # call at the next multiple of 32 with zero columns appended, q and k rescaled so that
+            # q.k / sqrt(d) is unchanged
+            dp = (d + 31) // 32 * 32
+            pad = lambda x: torch.nn.functional.pad(x, (0, dp - d))
+            _, got_p = _grads_of(pad(q) * (dp / d) ** 0.25, pad(k) * (dp / d) ** 0.25, pad(v), pad(d_out),
+                                 [("global_no_local", torch.tensor(gl, dtype=torch.int32, device=DEV), w)])
+            scale_back = (dp / d) ** 0.25
+            ref_p = [np64(got_p[0])[:, :d] * scale_back, np64(got_p[1])[:, :d] * scale_back, np64(got_p[2])[:, :d]]
+            _check_grads(got, ref_p, dtype, "global with repeats n=%d" % n)
 
 
 @pytest.mark.parametrize("dtype,d", [(torch.bfloat16, 64), (torch.float16, 128), (torch.bfloat16, 32),
