@@ -2305,9 +2305,8 @@ template <typename T, int D, bool PAD = false>
 __global__ __launch_bounds__(256) void global_rows_merge_kernel(TileArgs a) {
   // (PAD: rows of a.t.d < D elements, the tile kernels ran with zero-filled operands)
   const int dd = PAD ? (int)a.t.d : D;
-  const int NSUB = 256 / dd;  // threads per output element
   __shared__ float red[4];
-  __shared__ float part[256];
+  __shared__ float4v part[256];
   // grid: [problem][listed global]; the first n_uq of a problem's slots are its distinct rows
   const int64_t bb = blockIdx.x / a.n_globs;
   const int64_t g = blockIdx.x - bb * a.n_globs;
@@ -2333,25 +2332,41 @@ __global__ __launch_bounds__(256) void global_rows_merge_kernel(TileArgs a) {
   __syncthreads();
   lsum = (red[0] + red[1]) + (red[2] + red[3]);
 
-  // (d that does not divide 256: the threads past NSUB * d have no element)
-  const int e = tid % dd, sub = tid / dd;
-  float acc = 0.f;
-  int64_t k = sub < NSUB ? sub : a.n_split;
-  for (; k + 3 * NSUB < a.n_split; k += 4 * NSUB) {
-    float x[4], wgt[4];
+  // A thread sums one 16-byte piece of the row over every nsub-th partial result (rows are whole
+  // 16-byte pieces; where the pieces do not divide 256 the last threads have none).
+  const int c4 = dd / 4, nsub = 256 / c4;
+  const int e4 = tid % c4, sub = tid / c4;
+  float4v acc = {0.f, 0.f, 0.f, 0.f};
+  int64_t k = sub < nsub ? sub : a.n_split;
+  for (; k + 3 * nsub < a.n_split; k += 4 * nsub) {
+    float4v x[4];
+    float wgt[4];
 #pragma unroll
     for (int u = 0; u < 4; u++) {
-      x[u] = a.pacc[(s0 + k + u * NSUB) * dd + e];
-      wgt[u] = a.pm[s0 + k + u * NSUB];
+      x[u] = *reinterpret_cast<const float4v*>(a.pacc + (s0 + k + u * nsub) * dd + 4 * e4);
+      wgt[u] = a.pm[s0 + k + u * nsub];
     }
 #pragma unroll
-    for (int u = 0; u < 4; u++) acc += __expf(wgt[u] - mx) * x[u];
+    for (int u = 0; u < 4; u++) {
+      const float wk = __expf(wgt[u] - mx);
+#pragma unroll
+      for (int i = 0; i < 4; i++) acc[i] += wk * x[u][i];
+    }
   }
-  for (; k < a.n_split; k += NSUB) acc += __expf(a.pm[s0 + k] - mx) * a.pacc[(s0 + k) * dd + e];
+  for (; k < a.n_split; k += nsub) {
+    const float wk = __expf(a.pm[s0 + k] - mx);
+    const float4v x = *reinterpret_cast<const float4v*>(a.pacc + (s0 + k) * dd + 4 * e4);
+#pragma unroll
+    for (int i = 0; i < 4; i++) acc[i] += wk * x[i];
+  }
   part[tid] = acc;
   __syncthreads();
   if (sub != 0) return;
-  for (int u = 1; u < NSUB; u++) acc += part[u * dd + e];
+  for (int u = 1; u < nsub; u++) {
+    const float4v x = part[u * c4 + e4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) acc[i] += x[i];
+  }
 
   const int64_t row = a.uq[g] + bb * a.n;
   const bool sf = a.t.state_f32 != 0;
@@ -2365,11 +2380,21 @@ __global__ __launch_bounds__(256) void global_rows_merge_kernel(TileArgs a) {
     l_out = wa + lsum * wb;
   }
   const float inv = 1.f / l_out;
-  T* orow = (T*)a.t.out + row * dd;
-  float x = acc * wb;
-  if (wa != 0.f) x += wa * to_f32(orow[e]);
-  orow[e] = from_f32<T>(x * inv);
-  if (e == 0) {
+  typedef T t4 __attribute__((ext_vector_type(4)));
+  t4* opiece = reinterpret_cast<t4*>((T*)a.t.out + row * dd + 4 * e4);
+  float x[4];
+#pragma unroll
+  for (int i = 0; i < 4; i++) x[i] = acc[i] * wb;
+  if (wa != 0.f) {
+    const t4 oi = *opiece;
+#pragma unroll
+    for (int i = 0; i < 4; i++) x[i] += wa * (float)oi[i];
+  }
+  t4 y;
+#pragma unroll
+  for (int i = 0; i < 4; i++) y[i] = (T)(x[i] * inv);
+  *opiece = y;
+  if (e4 == 0) {
     store_state<T>(a.t.m, row, m_out, sf);
     store_state<T>(a.t.l, row, l_out, sf);
   }
