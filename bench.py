@@ -641,7 +641,7 @@ def measured_gather_ceiling(lib, w, torch, min_entries=8_000_000, reps=5, tensor
     # timed like the kernel it is compared with: the dispatch's own start and end stamps
     ev = HipEvents()
     best, best_shape = float("inf"), None
-    shapes = ((1, 8), (1, 16), (1, 32), (2, 8), (2, 16), (2, 32), (4, 8), (4, 16), (4, 32), (8, 8), (8, 16))
+    shapes = ((1, 8), (1, 16), (1, 32), (2, 8), (2, 16), (2, 32), (4, 4), (4, 8), (4, 16), (4, 32), (8, 4), (8, 8), (8, 16))
     for wg, fl in shapes:
         for _ in range(reps):
             rc = probe.spfa_probe_gather(k.data_ptr(), v.data_ptr(), k.shape[0], row_bytes, idx.data_ptr(),

@@ -68,6 +68,19 @@ int64_t explicit_medium_limit(const spfa_problem_t* p) {
   return kv <= kCachedKvBytes ? kExplicitMediumRowLimitCached : kExplicitMediumRowLimit;
 }
 
+// ... and its batch size in the medium-row kernel (see there): smaller while K and V are not much
+// larger than the caches and the rows are long enough on average for the wavefronts to fall in
+// step (measured on uniform rows of sorted columns; the Zipf headline - 97 entries per row on
+// average, most of them in few long rows - loses 5 % of that kernel with 4).  CSR calls only:
+// the rows that the COO pre-pass builds keep their entries in the order they came in, and on
+// unsorted columns the smaller batches lose up to 10 %.
+int explicit_medium_batch(const spfa_problem_t* p, int64_t nnz) {
+  if (p->n_q <= 0 || nnz / p->n_q < 128) return 0;
+  const int64_t es = p->dtype == SPFA_DTYPE_F32 ? 4 : p->dtype == SPFA_DTYPE_F64 ? 8 : 2;
+  const int64_t kv = 2 * p->n_k * p->d * es * (p->n_batch > 1 ? p->n_batch : 1);
+  return kv <= kCachedKvBytes ? 2 : kv <= 4 * kCachedKvBytes ? 4 : 0;
+}
+
 // Band / block masks are uniform: every row has about the same number of candidates, so rows
 // are finished in place unless there are too few rows to fill the device and they are long.
 EngineSizing size_stride(int64_t n, int64_t max_deg) {
@@ -446,6 +459,7 @@ int spfa_csr_forward(const spfa_problem_t* p, const void* row_off, int row_off_b
   }
   EngineSizing s = size_csr(p->n_q, nnz);
   s.medium_max = explicit_medium_limit(p);
+  s.medium_batch = explicit_medium_batch(p, nnz);
   if (!batch_fits_engine(s, p)) {
     for (int64_t b = 0; b < batch_of(p); b++) {
       const spfa_problem_t one = batch_slice(p, b);
@@ -495,6 +509,7 @@ int spfa_csr_forward_planned(const spfa_problem_t* p, const void* row_off, int r
     return run_f64(make_tensors(p), mask, use_nan ? 1 : 0, (hipStream_t)stream);
   }
   EngineSizing s = size_csr(p->n_q, nnz);
+  s.medium_batch = explicit_medium_batch(p, nnz);  // (a launch-time choice: the plan does not depend on it)
   rc = check_workspace(plan, plan_bytes, work_list_bytes(p->n_q, nnz));
   if (rc) return rc;
   if (!batch_fits_engine(s, p)) {

@@ -527,7 +527,14 @@ __global__ __launch_bounds__(256) void segments_kernel(Tensors t, Mask mask, Pla
 // the persistent kernel (one wavefront per SIMD) nothing hides them, here the other resident
 // wavefronts do.  (A device-sized grid with a stride loop instead of one wavefront per list
 // slot was measured slower: 1.02 against 0.66 ms on 64 x 4096 rows of ~83 entries.)
-template <class Lay, class Mask>
+// UM: neighbours in flight per lane group.  Rows whose columns are sorted (the usual form of a CSR
+// mask) are walked from low to high columns by every wavefront, so the wavefronts resident at a
+// time touch about the same part of K and V at the same time; smaller batches with more
+// wavefronts resident keep them closer together, and while K and V are not much larger than the
+// caches that is worth more than the loads in flight per wavefront (uniform rows of 192 sorted
+// columns, 65536 tokens, fp32 d = 64: 8.8 TB/s of gathered rows with 8, 11.1 with 4, 9.1 with 2;
+// 20000 tokens: 14.1 / 15.2 / 16.5; from 262144 tokens on it makes no difference).
+template <class Lay, class Mask, int UM = Lay::U_MEDIUM>
 __global__ __launch_bounds__(256) void medium_rows_kernel(Tensors t, Mask mask, Plan plan) {
   using T = typename Lay::elem;
   constexpr int NE = Lay::NE;
@@ -556,9 +563,8 @@ __global__ __launch_bounds__(256) void medium_rows_kernel(Tensors t, Mask mask, 
   float m = kNegInf, l = 0.f, acc[NE];
 #pragma unroll
   for (int e = 0; e < NE; e++) acc[e] = 0.f;
-  attend<Lay, Mask, Lay::U_MEDIUM, kWave>(mask, rc, (const T*)t.k + b * t.kv_stride,
-                                          (const T*)t.v + b * t.kv_stride, t.d, scale, q, 0, rc.deg,
-                                          lane, m, l, acc);
+  attend<Lay, Mask, UM, kWave>(mask, rc, (const T*)t.k + b * t.kv_stride, (const T*)t.v + b * t.kv_stride,
+                               t.d, scale, q, 0, rc.deg, lane, m, l, acc);
 #pragma unroll
   for (int off = LPR; off < kWave; off <<= 1) {
     float m2 = shfl_xor_f32(m, off);
@@ -731,6 +737,7 @@ struct EngineSizing {
   int64_t medium_max;    // rows up to this many get a wavefront of their own (0: same as short_max)
   int64_t seg;           // segment length for longer rows
   int64_t n_long_bound;  // upper bound on the number of rows with deg > short_max
+  int medium_batch;      // neighbours in flight per lane group in medium_rows_kernel (0: the layout's)
 };
 
 struct WorkspaceLayout {
@@ -900,8 +907,21 @@ int launch_engine(const Tensors& t, const Mask& mask, const EngineSizing& s, int
                      stream, t, mask, plan);
   if (has_long && w.cap_medium > 0) {
     const int64_t gridm = ((int64_t)w.cap_medium * t.n_batch + 3) / 4;
-    hipLaunchKernelGGL((medium_rows_kernel<Lay, Mask>), dim3((unsigned)gridm), dim3(256), 0, stream, t,
-                       mask, plan);
+    bool launched = false;
+    if constexpr (Mask::kExplicit && Lay::U_MEDIUM > 2) {
+      if (s.medium_batch == 2) {
+        hipLaunchKernelGGL((medium_rows_kernel<Lay, Mask, 2>), dim3((unsigned)gridm), dim3(256), 0, stream, t,
+                           mask, plan);
+        launched = true;
+      } else if (s.medium_batch == 4 && Lay::U_MEDIUM > 4) {
+        hipLaunchKernelGGL((medium_rows_kernel<Lay, Mask, (Lay::U_MEDIUM > 4 ? 4 : Lay::U_MEDIUM)>),
+                           dim3((unsigned)gridm), dim3(256), 0, stream, t, mask, plan);
+        launched = true;
+      }
+    }
+    if (!launched)
+      hipLaunchKernelGGL((medium_rows_kernel<Lay, Mask>), dim3((unsigned)gridm), dim3(256), 0, stream, t,
+                         mask, plan);
   }
   if (has_long) {
         // One workgroup (one wavefront per SIMD) per CU with 16 neighbours in flight per lane group
