@@ -141,6 +141,11 @@ def _source_loop_depth(kname: str) -> int:
     else:
         m = re.search(r"6GenLayI\w+?Li(\d+)E", kname)
         lpr, unroll = 64, (8 if int(m.group(1)) <= 2 else 2)
+    if med and not whole:
+        # medium_rows_kernel names its batch size as a third template argument
+        m = re.search(r"MaskELi(\d+)EEEv", kname)
+        if m:
+            unroll = min(unroll, int(m.group(1)))
     span = 64 if (seg or med) else lpr
     groups = span // lpr
     unroll = min(unroll, span // groups)

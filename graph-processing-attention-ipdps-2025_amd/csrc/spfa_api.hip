@@ -27,7 +27,7 @@ inline bool dtype_ok(int dtype) {
 // enough that the per-segment overhead (q load, group merge, partial write) stays small
 // Segment length for long rows: long enough to amortise the pipeline fill and the partial
 // result of a segment (1024 candidates: 64 per lane group at d*s = 256 bytes), short enough
-// that the work list holds several items per persistent wavefront (about 1024 of them).
+// that the work list holds several items per persistent wavefront (about 2048 of them).
 inline int64_t pick_segment(int64_t nnz_long) {
   int64_t seg = 128;
   while (seg < 1024 && seg * 2 * 8192 <= nnz_long) seg *= 2;
@@ -41,7 +41,7 @@ constexpr int64_t kExplicitInlineRowLimit = 32;
 // without, 0.65 with).
 constexpr int64_t kExplicitMediumRowLimit = 256;
 // ... and rows of up to this many when K and V are small enough to stay in the caches: the
-// persistent kernel (one wavefront per SIMD, tuned for the latency of memory-side fills) then
+// persistent kernel (two wavefronts per SIMD, tuned for the latency of memory-side fills) then
 // leaves most of the cache bandwidth unused on single-segment rows, which an ordinary grid of
 // eight wavefronts per SIMD does not.  Uniform rows of 257 ... 1000 entries, limit 256 -> 1024:
 // 8192 tokens at d = 64 fp32 4.9 ... 12.5 -> 13.2 ... 20.9 TB/s of gathered rows, 20000 tokens bf16

@@ -7,6 +7,8 @@
 //   plan_kernel        one thread per query row: rows with short_max < deg <= medium_max go on a
 //                      list of their own, longer rows are cut into segments of `seg` candidates
 //                      that are appended to a work list.
+//   order_kernel       copies the work list into the order it is handed out in: segments that
+//                      lie at the same place in their rows together.
 //   rows_kernel        one group of LPR lanes per query row (64/LPR rows per wavefront) finishes
 //                      the rows with deg <= short_max on the spot.
 //   medium_rows_kernel one wavefront per listed medium row, its 64/LPR groups share the row.
@@ -69,8 +71,21 @@ struct Counters {
 struct Item {
   int32_t row;
   int32_t seg;
-  int32_t slot;  // partial slot, or -1 when the row has a single segment
-  int32_t pad;
+  int32_t slot;   // partial slot, or -1 when the row has a single segment
+  int32_t phase;  // which of kPhases parts of the row the middle of the segment lies in
+};
+
+// The work list is handed out ordered by `phase`: segment j of every row that has the same number
+// of segments comes at the same time, and in rows whose columns are sorted (the usual form of a
+// CSR mask) these segments hold about the same columns, so the wavefronts at work at any one time
+// keep to one part of K and V and meet each other's rows in the caches.  Rows of 4096 sorted
+// uniform columns, fp32 d = 64, listed row by row against by phase: K + V of 16 MiB 12.1 -> 15.0
+// TB/s of gathered rows, 64 MiB 8.7 -> 11.9, 256 MiB 8.0 -> 8.6.
+constexpr int kPhases = 64;
+
+struct Phases {
+  uint32_t count[kPhases];  // items per phase (plan_kernel)
+  uint32_t taken[kPhases];  // ... already placed (order_kernel)
 };
 
 struct MultiRow {
@@ -84,7 +99,9 @@ struct Plan {
   Counters* cnt;
   uint32_t* cursor;  // next work item of segments_kernel (separate from cnt so that a plan can
                      // be shared by calls that each bring their own scratch)
-  Item* items;
+  Item* items;       // ordered by phase: what segments_kernel walks
+  Item* listed;      // as plan_kernel appended them
+  Phases* phases;
   MultiRow* multi;
   int32_t* medium;   // rows with short_max < deg <= medium_max: one wavefront each, no queue
   int32_t* shorts;   // rows with 0 < deg <= short_max (null: no list was made)
@@ -95,6 +112,7 @@ struct Plan {
   uint32_t cap_partials;
   uint32_t cap_multi;
   uint32_t cap_medium;
+  uint32_t order_block0;  // workgroups of rows_kernel from this one on order the work list
   uint32_t* status;  // the device's sticky status word (may be null): see device_status_word()
   int32_t use_nan;
   int64_t short_max;
@@ -114,7 +132,10 @@ static __global__ void reset_cursor_kernel(uint32_t* cursor) {
   if (threadIdx.x == 0) *cursor = 0;
 }
 
-static __global__ void reset_counters_kernel(Counters* cnt) {
+static __global__ void reset_counters_kernel(Counters* cnt, Phases* ph) {
+  static_assert(kPhases == kWave, "one lane per phase");
+  ph->count[threadIdx.x] = 0;
+  ph->taken[threadIdx.x] = 0;
   if (threadIdx.x == 0) {
     cnt->n_items = 0;
     cnt->n_partials = 0;
@@ -304,15 +325,22 @@ __device__ __forceinline__ uint32_t wave_inclusive_sum(uint32_t x, int lane) {
 // serialise on them and dominate the kernel).
 constexpr int kPlanThreads = 1024;
 
+// the phase of segment j of nseg: where its middle lies in the row, in kPhases-ths
+__device__ __forceinline__ uint32_t segment_phase(uint32_t j, uint32_t nseg) {
+  return (uint32_t)(((uint64_t)(2 * j + 1) * kPhases) / (2 * (uint64_t)nseg));
+}
+
 template <class Mask>
 __global__ __launch_bounds__(kPlanThreads) void plan_kernel(int64_t n_q, Mask mask, Plan plan) {
   constexpr int NW = kPlanThreads / kWave;
   __shared__ uint32_t wave_tot[NW][5];
   __shared__ uint32_t block_base[5];
   __shared__ uint32_t block_ok;
+  __shared__ uint32_t phase_count[kPhases];
   const int lane = lane_id();
   const int wave = threadIdx.x / kWave;
   const int64_t row = (int64_t)blockIdx.x * kPlanThreads + threadIdx.x;
+  if (threadIdx.x < kPhases) phase_count[threadIdx.x] = 0;
   int64_t deg = 0;
   if (row < n_q) {
     deg = mask.row(row).deg;
@@ -326,6 +354,8 @@ __global__ __launch_bounds__(kPlanThreads) void plan_kernel(int64_t n_q, Mask ma
   const uint32_t nseg = is_long ? (uint32_t)((deg + plan.seg - 1) / plan.seg) : 0u;
   const uint32_t multi = nseg > 1 ? 1u : 0u;
   const uint32_t npart = multi ? nseg : 0u;
+  __syncthreads();  // (phase_count is zero)
+  for (uint32_t j = 0; j < nseg; j++) atomicAdd(&phase_count[segment_phase(j, nseg)], 1u);
   const uint32_t med = is_medium ? 1u : 0u;
   const uint32_t sht = (deg > 0 && deg <= plan.short_max) ? 1u : 0u;
   const uint32_t inc_items = wave_inclusive_sum(nseg, lane);
@@ -375,6 +405,8 @@ __global__ __launch_bounds__(kPlanThreads) void plan_kernel(int64_t n_q, Mask ma
   __syncthreads();
   if (sht) plan.shorts[block_base[4] + wave_tot[wave][4] + inc_sht - 1] = (int32_t)row;
   if (!block_ok) return;
+  if (threadIdx.x < kPhases && phase_count[threadIdx.x] != 0)
+    atomicAdd(&plan.phases->count[threadIdx.x], phase_count[threadIdx.x]);
   if (is_medium) plan.medium[block_base[3] + wave_tot[wave][3] + inc_med - 1] = (int32_t)row;
   if (!is_long) return;
   const uint32_t my_item = block_base[0] + wave_tot[wave][0] + inc_items - nseg;
@@ -392,13 +424,56 @@ __global__ __launch_bounds__(kPlanThreads) void plan_kernel(int64_t n_q, Mask ma
     it.row = (int32_t)row;
     it.seg = (int32_t)j;
     it.slot = multi ? (int32_t)(my_slot + j) : -1;
-    it.pad = 0;
-    plan.items[my_item + j] = it;
+    it.phase = (int32_t)segment_phase(j, nseg);
+    plan.listed[my_item + j] = it;
+  }
+}
+
+// Copies the work list into the order segments_kernel takes it in: by phase, in any order inside
+// a phase (which item a wavefront gets has no influence on any result).  The work of one
+// workgroup of 256 threads; rows_kernel, which does not look at the list, is launched with extra
+// workgroups that do this (a launch of its own would cost a few microseconds more).
+__device__ __forceinline__ void order_block(const Plan& plan, uint32_t block) {
+  __shared__ uint32_t start[kPhases];  // first place of a phase in the ordered list
+  __shared__ uint32_t mine[kPhases];   // items of this workgroup per phase, then their first place
+  if (plan.cnt->overflow) return;
+  uint32_t n_items = plan.cnt->n_items;
+  if (n_items > plan.cap_items) n_items = plan.cap_items;
+  if (block * 256u >= n_items) return;
+  if (threadIdx.x < kWave) {
+    const uint32_t n = plan.phases->count[threadIdx.x];
+    start[threadIdx.x] = wave_inclusive_sum(n, (int)threadIdx.x) - n;
+    mine[threadIdx.x] = 0;
+  }
+  __syncthreads();
+  const uint32_t i = block * 256u + threadIdx.x;
+  Item it{};
+  uint32_t ph = 0, rank = 0;
+  if (i < n_items) {
+    it = plan.listed[i];
+    ph = (uint32_t)it.phase & (kPhases - 1);
+    rank = atomicAdd(&mine[ph], 1u);
+  }
+  __syncthreads();
+  // one reservation per workgroup and phase (an atomic per item on the few phases a mask of
+  // equally long rows has would take longer than the attention)
+  if (threadIdx.x < kWave) {
+    const uint32_t n = mine[threadIdx.x];
+    mine[threadIdx.x] = n ? start[threadIdx.x] + atomicAdd(&plan.phases->taken[threadIdx.x], n) : 0u;
+  }
+  __syncthreads();
+  if (i < n_items) {
+    const uint32_t at = mine[ph] + rank;
+    if (at < n_items) plan.items[at] = it;
   }
 }
 
 template <class Lay, class Mask>
 __global__ __launch_bounds__(256) void rows_kernel(Tensors t, Mask mask, Plan plan) {
+  if (blockIdx.x >= plan.order_block0) {
+    order_block(plan, blockIdx.x - plan.order_block0);
+    return;
+  }
   using T = typename Lay::elem;
   constexpr int NE = Lay::NE;
   constexpr int LPR = Lay::LPR;
@@ -449,6 +524,9 @@ __global__ __launch_bounds__(256) void rows_kernel(Tensors t, Mask mask, Plan pl
   }
   // longer rows were cut into segments by plan_kernel and belong to segments_kernel
 }
+
+// (for a call that only builds the work list)
+static __global__ __launch_bounds__(256) void order_kernel(Plan plan) { order_block(plan, blockIdx.x); }
 
 template <class Lay, class Mask>
 __global__ __launch_bounds__(256) void segments_kernel(Tensors t, Mask mask, Plan plan) {
@@ -524,7 +602,7 @@ __global__ __launch_bounds__(256) void segments_kernel(Tensors t, Mask mask, Pla
 // Rows of medium length (short_max < deg <= medium_max): one wavefront per row and problem, the
 // lane groups share the row's candidates as in segments_kernel, but launched as an ordinary
 // grid.  A row of this size is a handful of dependent memory round trips and little else: in
-// the persistent kernel (one wavefront per SIMD) nothing hides them, here the other resident
+// the persistent kernel (two wavefronts per SIMD) little hides them, here the other resident
 // wavefronts do.  (A device-sized grid with a stride loop instead of one wavefront per list
 // slot was measured slower: 1.02 against 0.66 ms on 64 x 4096 rows of ~83 entries.)
 // UM: neighbours in flight per lane group.  Rows whose columns are sorted (the usual form of a CSR
@@ -741,7 +819,7 @@ struct EngineSizing {
 };
 
 struct WorkspaceLayout {
-  size_t off_cnt, off_items, off_multi, off_medium, off_short, off_pm, off_pl, off_pacc, total;
+  size_t off_cnt, off_phases, off_items, off_listed, off_multi, off_medium, off_short, off_pm, off_pl, off_pacc, total;
   uint32_t cap_items, cap_partials, cap_multi, cap_medium, cap_short;
 };
 
@@ -775,7 +853,9 @@ inline WorkspaceLayout engine_workspace(const EngineSizing& s, int64_t n_q, int6
   w.cap_short = (uint32_t)cap_short;
   size_t off = 0;
   w.off_cnt = off;      off = align_up(off + sizeof(Counters), 256);
+  w.off_phases = off;   off = align_up(off + sizeof(Phases), 256);
   w.off_items = off;    off = align_up(off + (size_t)cap_items * sizeof(Item), 256);
+  w.off_listed = off;   off = align_up(off + (size_t)cap_items * sizeof(Item), 256);
   w.off_multi = off;    off = align_up(off + (size_t)cap_multi * sizeof(MultiRow), 256);
   w.off_medium = off;   off = align_up(off + (size_t)cap_medium * sizeof(int32_t), 256);
   w.off_short = off;    off = align_up(off + (size_t)cap_short * sizeof(int32_t), 256);
@@ -825,7 +905,7 @@ inline void launch_maybe_timed(const KernelEvents& ev, void (*kernel)(KArgs...),
     hipLaunchKernelGGL(kernel, grid, block, 0, stream, static_cast<KArgs>(args)...);
 }
 
-constexpr int kSegmentWorkgroupsPerCu = 1;
+constexpr int kSegmentWorkgroupsPerCu = 2;
 // whole_rows_kernel takes a call of at most this many rows (over all problems), keys and
 // candidates.  What it cannot do is share one very long row over the device, so the limits keep
 // such a row short: K and V of 16384 keys stay in the caches, a row of distinct columns is at
@@ -865,6 +945,8 @@ int launch_engine(const Tensors& t, const Mask& mask, const EngineSizing& s, int
   Plan plan{};
   plan.cnt = (Counters*)(pbase + w.off_cnt);
   plan.items = (Item*)(pbase + w.off_items);
+  plan.listed = (Item*)(pbase + w.off_listed);
+  plan.phases = (Phases*)(pbase + w.off_phases);
   plan.multi = (MultiRow*)(pbase + w.off_multi);
   plan.medium = (int32_t*)(pbase + w.off_medium);
   plan.shorts = w.cap_short > 0 ? (int32_t*)(pbase + w.off_short) : nullptr;
@@ -893,18 +975,24 @@ int launch_engine(const Tensors& t, const Mask& mask, const EngineSizing& s, int
     return hipGetLastError() == hipSuccess ? 0 : 4;
   }
   if (has_long && phase != kEngineRunOnly) {
-    hipLaunchKernelGGL(reset_counters_kernel, dim3(1), dim3(64), 0, stream, plan.cnt);
+    hipLaunchKernelGGL(reset_counters_kernel, dim3(1), dim3(64), 0, stream, plan.cnt, plan.phases);
     hipLaunchKernelGGL((plan_kernel<Mask>), dim3((unsigned)((t.n_q + kPlanThreads - 1) / kPlanThreads)),
                        dim3(kPlanThreads), 0, stream, t.n_q, mask, plan);
   }
-  if (phase == kEnginePlanOnly) return hipGetLastError() == hipSuccess ? 0 : 4;
+  if (phase == kEnginePlanOnly) {
+    if (has_long)
+      hipLaunchKernelGGL(order_kernel, dim3((w.cap_items + 255u) / 256u), dim3(256), 0, stream, plan);
+    return hipGetLastError() == hipSuccess ? 0 : 4;
+  }
   if (has_long && phase == kEngineRunOnly)
     hipLaunchKernelGGL(reset_cursor_kernel, dim3(1), dim3(64), 0, stream, plan.cursor);
 
   const int64_t rows_per_wg = 4 * Lay::GROUPS;
   const int64_t grid1 = (t.n_q * t.n_batch + rows_per_wg - 1) / rows_per_wg;
-  launch_maybe_timed(has_long ? KernelEvents{} : ev, rows_kernel<Lay, Mask>, dim3((unsigned)grid1), dim3(256),
-                     stream, t, mask, plan);
+  const int64_t grid_order = (has_long && phase == kEngineAll) ? ((int64_t)w.cap_items + 255) / 256 : 0;
+  plan.order_block0 = (uint32_t)grid1;
+  launch_maybe_timed(has_long ? KernelEvents{} : ev, rows_kernel<Lay, Mask>, dim3((unsigned)(grid1 + grid_order)),
+                     dim3(256), stream, t, mask, plan);
   if (has_long && w.cap_medium > 0) {
     const int64_t gridm = ((int64_t)w.cap_medium * t.n_batch + 3) / 4;
     bool launched = false;
@@ -924,9 +1012,14 @@ int launch_engine(const Tensors& t, const Mask& mask, const EngineSizing& s, int
                          mask, plan);
   }
   if (has_long) {
-        // One workgroup (one wavefront per SIMD) per CU with 16 neighbours in flight per lane group
-    // is the fastest shape measured: more resident wavefronts only add contention in the
-    // vector L1 (8 workgroups per CU: 0.98 ms at the 12.8 M-position Zipf mask, 1: 0.79 ms).
+    // Two workgroups (two wavefronts per SIMD) per CU with 16 neighbours in flight per lane
+    // group.  With the work list in phase order, on the 12.8 M-position Zipf mask: 1 / 2 / 3 / 4
+    // workgroups per CU 0.730 / 0.716 / 0.728 / 0.740 ms fp32, 0.479 / 0.411 / 0.403 / 0.411 ms
+    // bf16; with K and V far larger than the caches (4 M tokens) the number makes no difference.
+    // Smaller batches with more wavefronts (8 neighbours x 4 workgroups, 4 x 8) lose: 0.752 /
+    // 0.776 ms fp32, 0.410 / 0.470 ms bf16.
+    // (Listed row by row, one workgroup was the fastest, 0.79 ms fp32 against 0.98 with 8: the
+    // wavefronts then spread over all of K and V and only added contention in the vector L1.)
     int64_t grid2 = (int64_t)device_cu_count() * kSegmentWorkgroupsPerCu;
     int64_t need = ((int64_t)w.cap_items * t.n_batch + 3) / 4;
     if (grid2 > need) grid2 = need;
