@@ -167,7 +167,8 @@ def make_workload(name, dtype, torch, syn, inline_limit=32, planned=False, heads
         long_rows = deg > inline_limit
         nnz_long, rows_long = int(deg[long_rows].sum()), int(long_rows.sum())
         if nnz_long > 0:  # the ceiling probe walks what the segment kernel walks: the long rows' columns
-            w["probe_idx"] = w["probe_idx"][torch.repeat_interleave(long_rows, deg)].contiguous()
+            w["probe_idx"] = handed_out_order(w["probe_idx"][torch.repeat_interleave(long_rows, deg)],
+                                              deg[long_rows], torch)
         _, kernel_bytes = syn.explicit_mask_bytes(nnz_long, rows_long, d, es, off_bytes=off_b)
         w.update(n=n, d=d, nnz=nnz * heads, bytes_total=total * heads, bytes_gathered=gathered * heads,
                  bound="hbm", kernel_bytes=kernel_bytes * heads, kernel_nnz=nnz_long * heads,
@@ -619,6 +620,29 @@ def measured_copy_bandwidth(torch, mib=1024, reps=5):
     return 2.0 * src.numel() * 4 / (best * 1e-3) / 1e9
 
 
+def handed_out_order(cols, deg, torch, seg=1024, phases=64):
+    """The columns of the long rows (`cols`, row after row; `deg` entries each) in the order the
+    library's segment kernel takes them: rows cut into segments of `seg`, the segments ordered by the
+    place of their middle in the row (in `phases` steps), every segment filled up to `seg` list
+    slots with entries the probe skips (top bit set), so that one chunk of the probe's list is one
+    segment."""
+    deg = deg.to(torch.int64)
+    nseg = (deg + seg - 1) // seg
+    row_of_seg = torch.repeat_interleave(torch.arange(deg.numel(), device=deg.device), nseg)
+    first_seg = torch.cumsum(nseg, 0) - nseg
+    j = torch.arange(int(nseg.sum()), device=deg.device) - first_seg[row_of_seg]
+    phase = ((2 * j + 1) * phases) // (2 * nseg[row_of_seg])
+    place = torch.empty_like(j)
+    place[torch.argsort(phase, stable=True)] = torch.arange(j.numel(), device=deg.device)
+    # entry t of row r is entry t % seg of the row's segment t // seg
+    row_of_entry = torch.repeat_interleave(torch.arange(deg.numel(), device=deg.device), deg)
+    t = torch.arange(cols.numel(), device=deg.device) - (torch.cumsum(deg, 0) - deg)[row_of_entry]
+    dest = place[first_seg[row_of_entry] + t // seg] * seg + t % seg
+    out = torch.full((j.numel() * seg,), -1, dtype=torch.int32, device=cols.device)
+    out[dest.to(cols.device)] = cols.to(torch.int32)
+    return out.contiguous()
+
+
 def measured_gather_ceiling(lib, w, torch, min_entries=8_000_000, reps=5, tensors=None, idx=None):
     """What the memory system delivers to the explicit-mask access pattern at this working set:
     spfa_probe_gather (the gather of segments_kernel without any arithmetic) over the workload's
@@ -635,6 +659,7 @@ def measured_gather_ceiling(lib, w, torch, min_entries=8_000_000, reps=5, tensor
         return None
     if idx.numel() < min_entries:
         idx = idx.repeat((min_entries + idx.numel() - 1) // idx.numel())
+    n_live = int((idx >= 0).sum())  # (negative: a slot the probe skips)
     probe = load_probe_library()
     cursor = torch.zeros(64, dtype=torch.int32, device="cuda")
     stream = torch.cuda.current_stream().cuda_stream
@@ -651,11 +676,11 @@ def measured_gather_ceiling(lib, w, torch, min_entries=8_000_000, reps=5, tensor
             ms = ev.elapsed_ms()
             if ms < best:
                 best, best_shape = ms, (wg, fl)
-    bytes_moved = idx.numel() * (2 * row_bytes + 4)
+    bytes_moved = n_live * (2 * row_bytes + 4)
     return {"GBs": bytes_moved / (best * 1e-3) / 1e9,
             "how": "%d list entries x (2 rows of %d B + 4 B index) in %.3f ms; best of %d launches each of "
                    "(workgroups per CU, rows in flight) %s: (%d,%d)"
-                   % (idx.numel(), row_bytes, best, reps, " ".join("(%d,%d)" % x for x in shapes), *best_shape)}
+                   % (n_live, row_bytes, best, reps, " ".join("(%d,%d)" % x for x in shapes), *best_shape)}
 
 
 def main():
