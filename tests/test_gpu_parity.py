@@ -267,6 +267,25 @@ def test_csr_small_problem_with_very_long_rows(mods, dtype, d):
     check(o, m, l, *ref, dtype, state_dtype=torch.float32, dead_expect="nan")
 
 
+@pytest.mark.parametrize("dtype,d", [(torch.float32, 64), (torch.bfloat16, 64), (torch.float32, 40)])
+def test_csr_rows_of_more_segments_than_the_work_list_has_phases(mods, dtype, d):
+    """More keys than the single-launch path takes, so the rows go through the work list: rows cut into up to 157
+    segments of 128 (the list is handed out in 64 phases, so several segments of a row share one), rows of one
+    and two segments, medium and short rows, empty rows."""
+    n_q, n_k = 64, 20000
+    rng = np.random.default_rng(91)
+    lengths = [20000, 19999, 9000, 300, 257, 256, 129, 128, 33, 5, 0, 1] + [int(x) for x in rng.integers(0, 400, n_q - 12)]
+    cols, off = [], [0]
+    for ln in lengths:
+        cols.append(np.sort(rng.choice(n_k, ln, replace=False)))
+        off.append(off[-1] + ln)
+    ro, ci = np.array(off, np.int64), np.concatenate(cols).astype(np.int64)
+    q, k, v = dev_qkv(n_q, d, dtype, 92, n_k=n_k)
+    o, m, l = run_csr(mods, q, k, v, ro, ci, True, state_dtype=torch.float32)
+    ref = c_oracle.csr(np64(q), np64(k), np64(v), ro, ci, use_nan=True)
+    check(o, m, l, *ref, dtype, state_dtype=torch.float32, dead_expect="nan")
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_csr_power_law_rows(mods, dtype):
     """Zipf(1.5) degrees clipped to [1, 4096] at N=16384: short rows, single-segment rows and
