@@ -371,36 +371,37 @@ __global__ __launch_bounds__(kPlanThreads) void plan_kernel(int64_t n_q, Mask ma
     wave_tot[wave][4] = inc_sht;
   }
   __syncthreads();
-  if (threadIdx.x == 0) {
-    uint32_t tot[5] = {0u, 0u, 0u, 0u, 0u};
-    for (int w = 0; w < NW; w++)
-      for (int k = 0; k < 5; k++) {
-        const uint32_t x = wave_tot[w][k];
-        wave_tot[w][k] = tot[k];  // exclusive prefix over the wavefronts
-        tot[k] += x;
-      }
-    uint32_t ok = 1;
-    if (tot[0]) {
-      block_base[0] = atomicAdd(&plan.cnt->n_items, tot[0]);
-      block_base[1] = tot[1] ? atomicAdd(&plan.cnt->n_partials, tot[1]) : 0u;
-      block_base[2] = tot[2] ? atomicAdd(&plan.cnt->n_multi, tot[2]) : 0u;
-      if (block_base[0] + tot[0] > plan.cap_items || block_base[1] + tot[1] > plan.cap_partials ||
-          block_base[2] + tot[2] > plan.cap_multi) {
-        ok = 0;
+  if (threadIdx.x < 5) {
+    // one lane per counter (work items, partial results, multi-segment rows, medium rows, short
+    // rows): its exclusive prefix over the wavefronts, then ONE reservation for the workgroup -
+    // the five atomics travel together instead of one after the other
+    const int kk = threadIdx.x;
+    uint32_t tot = 0;
+    for (int w = 0; w < NW; w++) {
+      const uint32_t x = wave_tot[w][kk];
+      wave_tot[w][kk] = tot;
+      tot += x;
+    }
+    uint32_t* const counter = kk == 0 ? &plan.cnt->n_items : kk == 1 ? &plan.cnt->n_partials
+                            : kk == 2 ? &plan.cnt->n_multi : kk == 3 ? &plan.cnt->n_medium : &plan.cnt->n_short;
+    // (as many short-row slots as rows: that list cannot overflow)
+    const uint32_t cap = kk == 0 ? plan.cap_items : kk == 1 ? plan.cap_partials : kk == 2 ? plan.cap_multi
+                       : kk == 3 ? plan.cap_medium : 0xffffffffu;
+    uint32_t base = 0;
+    bool bad = false;
+    if (tot) {
+      base = atomicAdd(counter, tot);
+      bad = base + tot > cap || base + tot < base;
+    }
+    block_base[kk] = base;
+    const bool any_bad = __ballot(bad) != 0;
+    if (kk == 0) {
+      block_ok = any_bad ? 0u : 1u;
+      if (any_bad) {
         atomicOr(&plan.cnt->overflow, 1u);
         if (plan.status != nullptr) atomicOr(plan.status, kStatusWorkListOverflow);
       }
     }
-    if (tot[3]) {
-      block_base[3] = atomicAdd(&plan.cnt->n_medium, tot[3]);
-      if (block_base[3] + tot[3] > plan.cap_medium) {
-        ok = 0;
-        atomicOr(&plan.cnt->overflow, 1u);
-        if (plan.status != nullptr) atomicOr(plan.status, kStatusWorkListOverflow);
-      }
-    }
-    if (tot[4]) block_base[4] = atomicAdd(&plan.cnt->n_short, tot[4]);  // (as many slots as rows)
-    block_ok = ok;
   }
   __syncthreads();
   if (sht) plan.shorts[block_base[4] + wave_tot[wave][4] + inc_sht - 1] = (int32_t)row;
