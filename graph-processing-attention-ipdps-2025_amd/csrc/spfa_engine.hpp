@@ -112,7 +112,6 @@ struct Plan {
   uint32_t cap_partials;
   uint32_t cap_multi;
   uint32_t cap_medium;
-  uint32_t order_block0;  // workgroups of rows_kernel from this one on order the work list
   uint32_t* status;  // the device's sticky status word (may be null): see device_status_word()
   int32_t use_nan;
   int64_t short_max;
@@ -432,49 +431,58 @@ __global__ __launch_bounds__(kPlanThreads) void plan_kernel(int64_t n_q, Mask ma
 
 // Copies the work list into the order segments_kernel takes it in: by phase, in any order inside
 // a phase (which item a wavefront gets has no influence on any result).  The work of one
-// workgroup of 256 threads; rows_kernel, which does not look at the list, is launched with extra
-// workgroups that do this (a launch of its own would cost a few microseconds more).
-__device__ __forceinline__ void order_block(const Plan& plan, uint32_t block) {
-  __shared__ uint32_t start[kPhases];  // first place of a phase in the ordered list
-  __shared__ uint32_t mine[kPhases];   // items of this workgroup per phase, then their first place
+// wavefront on 64 items.  When every item has the same phase (no row has more than one segment:
+// the rows the COO pre-pass builds at the bench size) the list stays where it is and
+// segments_kernel reads it there: one reservation per wavefront on the one phase's counter took
+// 17 us for 66 K items.
+// (Done by extra workgroups of the rows_kernel launch, which does not look at the list, this cost
+// every workgroup of that kernel a scalar load and a wait before its first useful instruction:
+// 224 -> 242 us on the 65 K tiny workgroups of a 1 M-row call, against 5 us for a launch.)
+__device__ __forceinline__ void order_wave(const Plan& plan, uint32_t wave_index, int lane) {
   if (plan.cnt->overflow) return;
   uint32_t n_items = plan.cnt->n_items;
   if (n_items > plan.cap_items) n_items = plan.cap_items;
-  if (block * 256u >= n_items) return;
-  if (threadIdx.x < kWave) {
-    const uint32_t n = plan.phases->count[threadIdx.x];
-    start[threadIdx.x] = wave_inclusive_sum(n, (int)threadIdx.x) - n;
-    mine[threadIdx.x] = 0;
-  }
-  __syncthreads();
-  const uint32_t i = block * 256u + threadIdx.x;
+  if (wave_index * (uint32_t)kWave >= n_items) return;
+  // lane p: first place of phase p in the ordered list
+  const uint32_t n_ph = plan.phases->count[lane];
+  if (__ballot(n_ph == n_items) != 0) return;  // one phase: see work_list()
+  const uint32_t start = wave_inclusive_sum(n_ph, lane) - n_ph;
+  const uint32_t i = wave_index * (uint32_t)kWave + (uint32_t)lane;
+  const bool live = i < n_items;
   Item it{};
-  uint32_t ph = 0, rank = 0;
-  if (i < n_items) {
+  uint32_t ph = 0;
+  if (live) {
     it = plan.listed[i];
     ph = (uint32_t)it.phase & (kPhases - 1);
-    rank = atomicAdd(&mine[ph], 1u);
   }
-  __syncthreads();
-  // one reservation per workgroup and phase (an atomic per item on the few phases a mask of
-  // equally long rows has would take longer than the attention)
-  if (threadIdx.x < kWave) {
-    const uint32_t n = mine[threadIdx.x];
-    mine[threadIdx.x] = n ? start[threadIdx.x] + atomicAdd(&plan.phases->taken[threadIdx.x], n) : 0u;
+  // the lanes that hold the same phase, and the first of them
+  uint64_t same = 0;
+  int leader = lane;
+  uint64_t todo = __ballot(live);
+  while (todo) {
+    const int first = __ffsll((long long)todo) - 1;
+    const uint32_t ph0 = (uint32_t)shfl_i32((int)ph, first);
+    const uint64_t grp = __ballot(live && ph == ph0);
+    if (live && ph == ph0) {
+      same = grp;
+      leader = first;
+    }
+    todo &= ~grp;
   }
-  __syncthreads();
-  if (i < n_items) {
-    const uint32_t at = mine[ph] + rank;
+  // one reservation per wavefront and phase (an atomic per item on the few phases a mask of
+  // equally long rows has would take longer than the attention), all of them in one round trip
+  uint32_t base = 0;
+  if (live && lane == leader) base = atomicAdd(&plan.phases->taken[ph], (uint32_t)__popcll(same));
+  base = (uint32_t)shfl_i32((int)base, leader);
+  const uint32_t first_place = (uint32_t)shfl_i32((int)start, (int)ph);
+  if (live) {
+    const uint32_t at = first_place + base + (uint32_t)__popcll(same & (((uint64_t)1 << lane) - 1));
     if (at < n_items) plan.items[at] = it;
   }
 }
 
 template <class Lay, class Mask>
 __global__ __launch_bounds__(256) void rows_kernel(Tensors t, Mask mask, Plan plan) {
-  if (blockIdx.x >= plan.order_block0) {
-    order_block(plan, blockIdx.x - plan.order_block0);
-    return;
-  }
   using T = typename Lay::elem;
   constexpr int NE = Lay::NE;
   constexpr int LPR = Lay::LPR;
@@ -526,8 +534,16 @@ __global__ __launch_bounds__(256) void rows_kernel(Tensors t, Mask mask, Plan pl
   // longer rows were cut into segments by plan_kernel and belong to segments_kernel
 }
 
-// (for a call that only builds the work list)
-static __global__ __launch_bounds__(256) void order_kernel(Plan plan) { order_block(plan, blockIdx.x); }
+// The list segments_kernel walks: the ordered one, or the list as appended when all its items
+// have one phase (order_wave then leaves it alone).
+__device__ __forceinline__ const Item* work_list(const Plan& plan, uint32_t n_items, int lane) {
+  const uint32_t n_ph = plan.phases->count[lane];
+  return __ballot(n_ph == n_items) != 0 ? plan.listed : plan.items;
+}
+
+static __global__ __launch_bounds__(256) void order_kernel(Plan plan) {
+  order_wave(plan, blockIdx.x * 4u + (threadIdx.x >> 6), (int)(threadIdx.x & (kWave - 1)));
+}
 
 template <class Lay, class Mask>
 __global__ __launch_bounds__(256) void segments_kernel(Tensors t, Mask mask, Plan plan) {
@@ -543,6 +559,7 @@ __global__ __launch_bounds__(256) void segments_kernel(Tensors t, Mask mask, Pla
   // every problem of the batch walks the same work list (the host keeps items * batch < 2^32)
   const uint32_t n_work = n_items * (uint32_t)t.n_batch;
   const float scale = 1.0f / sqrtf((float)t.d);
+  const Item* const items = work_list(plan, n_items, lane);
 
   while (true) {
     uint32_t idx = 0;
@@ -554,7 +571,7 @@ __global__ __launch_bounds__(256) void segments_kernel(Tensors t, Mask mask, Pla
       b = idx / n_items;
       idx -= b * n_items;
     }
-    const Item it = plan.items[idx];
+    const Item it = items[idx];
     const int64_t row = (int64_t)b * t.n_q + it.row;
     const int64_t slot = (int64_t)b * plan.cap_partials + it.slot;
     const typename Mask::Row rc = mask.row(it.row);
@@ -979,21 +996,16 @@ int launch_engine(const Tensors& t, const Mask& mask, const EngineSizing& s, int
     hipLaunchKernelGGL(reset_counters_kernel, dim3(1), dim3(64), 0, stream, plan.cnt, plan.phases);
     hipLaunchKernelGGL((plan_kernel<Mask>), dim3((unsigned)((t.n_q + kPlanThreads - 1) / kPlanThreads)),
                        dim3(kPlanThreads), 0, stream, t.n_q, mask, plan);
+    hipLaunchKernelGGL(order_kernel, dim3((w.cap_items + 255u) / 256u), dim3(256), 0, stream, plan);
   }
-  if (phase == kEnginePlanOnly) {
-    if (has_long)
-      hipLaunchKernelGGL(order_kernel, dim3((w.cap_items + 255u) / 256u), dim3(256), 0, stream, plan);
-    return hipGetLastError() == hipSuccess ? 0 : 4;
-  }
+  if (phase == kEnginePlanOnly) return hipGetLastError() == hipSuccess ? 0 : 4;
   if (has_long && phase == kEngineRunOnly)
     hipLaunchKernelGGL(reset_cursor_kernel, dim3(1), dim3(64), 0, stream, plan.cursor);
 
   const int64_t rows_per_wg = 4 * Lay::GROUPS;
   const int64_t grid1 = (t.n_q * t.n_batch + rows_per_wg - 1) / rows_per_wg;
-  const int64_t grid_order = (has_long && phase == kEngineAll) ? ((int64_t)w.cap_items + 255) / 256 : 0;
-  plan.order_block0 = (uint32_t)grid1;
-  launch_maybe_timed(has_long ? KernelEvents{} : ev, rows_kernel<Lay, Mask>, dim3((unsigned)(grid1 + grid_order)),
-                     dim3(256), stream, t, mask, plan);
+  launch_maybe_timed(has_long ? KernelEvents{} : ev, rows_kernel<Lay, Mask>, dim3((unsigned)grid1), dim3(256),
+                     stream, t, mask, plan);
   if (has_long && w.cap_medium > 0) {
     const int64_t gridm = ((int64_t)w.cap_medium * t.n_batch + 3) / 4;
     bool launched = false;
