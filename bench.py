@@ -632,6 +632,10 @@ def handed_out_order(cols, deg, torch, seg=1024, phases=64):
     first_seg = torch.cumsum(nseg, 0) - nseg
     j = torch.arange(int(nseg.sum()), device=deg.device) - first_seg[row_of_seg]
     phase = ((2 * j + 1) * phases) // (2 * nseg[row_of_seg])
+    # (a row's last segment comes the later the shorter it is)
+    last = j + 1 == nseg[row_of_seg]
+    missing = nseg[row_of_seg] * seg - deg[row_of_seg]
+    phase = torch.where(last, phase + (missing * (phases - phase)) // seg, phase).clamp_(max=phases - 1)
     place = torch.empty_like(j)
     place[torch.argsort(phase, stable=True)] = torch.arange(j.numel(), device=deg.device)
     # entry t of row r is entry t % seg of the row's segment t // seg

@@ -324,9 +324,23 @@ __device__ __forceinline__ uint32_t wave_inclusive_sum(uint32_t x, int lane) {
 // serialise on them and dominate the kernel).
 constexpr int kPlanThreads = 1024;
 
-// the phase of segment j of nseg: where its middle lies in the row, in kPhases-ths
-__device__ __forceinline__ uint32_t segment_phase(uint32_t j, uint32_t nseg) {
-  return (uint32_t)(((uint64_t)(2 * j + 1) * kPhases) / (2 * (uint64_t)nseg));
+// The phase of segment j of the nseg of a row with deg candidates: where its middle lies in the
+// row, in kPhases-ths.  The last segment of a row, the only one that can be short, comes the later
+// the shorter it is (within the half phase step above its middle): the list then ends in short
+// items, and the wavefronts that find it empty wait for short last items, not for full ones.
+// A row of a single segment is all "last segment": such rows spread over the second half of the
+// list, longest first, instead of coming all at once in the middle (their columns span all of K
+// and V, so they are better taken between the others than as a block: the Zipf headline 0.707 ->
+// 0.678 ms fp32, 0.406 -> 0.411 ms bf16, eight heads of it 5.72 -> 5.08 ms; starting them at the
+// front, at a quarter or at three quarters of the list instead of the middle: 0.696, 0.686, 0.700).
+__device__ __forceinline__ uint32_t segment_phase(uint32_t j, uint32_t nseg, int64_t deg, int64_t seg) {
+  uint32_t ph = (uint32_t)(((uint64_t)(2 * j + 1) * kPhases) / (2 * (uint64_t)nseg));
+  if (j + 1 == nseg) {
+    const uint32_t room = kPhases - ph;  // phases from the middle to the end of the row
+    const int64_t missing = (int64_t)nseg * seg - deg;  // 0 ... seg - 1
+    ph += (uint32_t)((missing * room) / seg);
+  }
+  return ph < (uint32_t)kPhases ? ph : (uint32_t)kPhases - 1u;
 }
 
 template <class Mask>
@@ -354,7 +368,7 @@ __global__ __launch_bounds__(kPlanThreads) void plan_kernel(int64_t n_q, Mask ma
   const uint32_t multi = nseg > 1 ? 1u : 0u;
   const uint32_t npart = multi ? nseg : 0u;
   __syncthreads();  // (phase_count is zero)
-  for (uint32_t j = 0; j < nseg; j++) atomicAdd(&phase_count[segment_phase(j, nseg)], 1u);
+  for (uint32_t j = 0; j < nseg; j++) atomicAdd(&phase_count[segment_phase(j, nseg, deg, plan.seg)], 1u);
   const uint32_t med = is_medium ? 1u : 0u;
   const uint32_t sht = (deg > 0 && deg <= plan.short_max) ? 1u : 0u;
   const uint32_t inc_items = wave_inclusive_sum(nseg, lane);
@@ -424,17 +438,16 @@ __global__ __launch_bounds__(kPlanThreads) void plan_kernel(int64_t n_q, Mask ma
     it.row = (int32_t)row;
     it.seg = (int32_t)j;
     it.slot = multi ? (int32_t)(my_slot + j) : -1;
-    it.phase = (int32_t)segment_phase(j, nseg);
+    it.phase = (int32_t)segment_phase(j, nseg, deg, plan.seg);
     plan.listed[my_item + j] = it;
   }
 }
 
 // Copies the work list into the order segments_kernel takes it in: by phase, in any order inside
 // a phase (which item a wavefront gets has no influence on any result).  The work of one
-// wavefront on 64 items.  When every item has the same phase (no row has more than one segment:
-// the rows the COO pre-pass builds at the bench size) the list stays where it is and
-// segments_kernel reads it there: one reservation per wavefront on the one phase's counter took
-// 17 us for 66 K items.
+// wavefront on 64 items.  When every item has the same phase (single-segment rows of one length)
+// the list stays where it is and segments_kernel reads it there: one reservation per wavefront
+// on the one phase's counter took 17 us for 66 K items.
 // (Done by extra workgroups of the rows_kernel launch, which does not look at the list, this cost
 // every workgroup of that kernel a scalar load and a wait before its first useful instruction:
 // 224 -> 242 us on the 65 K tiny workgroups of a 1 M-row call, against 5 us for a launch.)
