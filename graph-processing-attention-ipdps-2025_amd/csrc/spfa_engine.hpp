@@ -72,7 +72,7 @@ struct Item {
   int32_t row;
   int32_t seg;
   int32_t slot;   // partial slot, or -1 when the row has a single segment
-  int32_t phase;  // which of kPhases parts of the row the middle of the segment lies in
+  int32_t phase;  // its place in the order the list is handed out in: segment_phase()
 };
 
 // The work list is handed out ordered by `phase`: segment j of every row that has the same number
