@@ -556,7 +556,7 @@ def bench_backward(a, w, st, dtype, torch, syn, lib):
                     if half_band else "tile_grad_kernel (query pass, key pass)")
     if name == "global" or name == "bigbird":
         tile_kernels += " + tile_grad_kernel / global_grad_merge_kernel for the listed tokens"
-    gather_kernels = "grad_prologue_kernel, grad_rows_kernel (query pass, key pass), grad_items_kernel" + \
+    gather_kernels = "grad_prologue_kernel, grad_rows_kernel (query pass, key pass), order_kernel, grad_segments_kernel" + \
                      (", mask transposition" if not a.planned and name.startswith(("csr", "bigbird")) else "") + \
                      (", two COO bucketing pre-passes" if name.startswith("coo") else "")
     if gather_ms >= max(dense_ms, mfma_ms):

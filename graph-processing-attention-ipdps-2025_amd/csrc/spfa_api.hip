@@ -921,38 +921,63 @@ int check_grads(const spfa_problem_t* p, const spfa_grads_t* g) {
 
 Grads make_grads(const spfa_grads_t* g) { return Grads{g->d_out, g->d_q, g->d_k, g->d_v}; }
 
-// Workspace of a gradient call: lse and delta of every query row (apart and side by side), the two lists of (owner,
-// segment) items of long rows, then whatever the mask needs (`mask_bytes`).
+// Owners (query rows in the query pass, key rows in the key pass) with more candidates than this
+// leave their segments on the work list of the pass instead of walking them with their own
+// wavefront.  Explicit masks, whole gradient call with 128 / 256 / 512 / 1024: the Zipf mask of
+// 131 K rows 1.43 / 1.34 / 1.36 / 1.40 ms fp32 and 1.06 / 1.00 / 1.00 / 1.02 ms bf16, the COO mask
+// of 1 M rows 9.40 / 9.09 / 8.90 / 8.80 ms.  The implicit masks' rows are all about equally long,
+// so a wavefront per row keeps the device busy whatever their length: only what is longer than a
+// segment is shared out.
+constexpr int64_t kGradOwnExplicit = 512;
+constexpr int64_t kGradOwnImplicit = kGradSegment;
+
+// Most work items one pass can leave behind, per problem, and the limit that goes with the count.
+struct ItemsBound {
+  int64_t items;
+  int64_t own_max;
+};
+int64_t grad_items_of(int64_t deg, int64_t own_max) {
+  return deg > own_max ? (deg + kGradSegment - 1) / kGradSegment : 0;
+}
+ItemsBound explicit_items_bound(int64_t nnz) {
+  // every owner of more than own_max candidates: deg / seg + 1 items at most, nnz / (own_max + 1) such owners
+  return ItemsBound{nnz / kGradSegment + nnz / (kGradOwnExplicit + 1), kGradOwnExplicit};
+}
+ItemsBound uniform_items_bound(int64_t n_rows, int64_t max_deg) {
+  return ItemsBound{n_rows * grad_items_of(max_deg, kGradOwnImplicit), kGradOwnImplicit};
+}
+ItemsBound global_items_bound(int64_t n, int64_t n_globals) {
+  return ItemsBound{n_globals * grad_items_of(n, kGradOwnImplicit) + n * grad_items_of(n_globals, kGradOwnImplicit),
+                    kGradOwnImplicit};
+}
+
+// Workspace of a gradient call: lse and delta of every query row (apart and side by side), the counters and the
+// work lists of the two passes (as appended and in hand-out order), then whatever the mask needs (`mask_bytes`).
 struct GradLayout {
-  size_t off_lse, off_delta, off_stat, off_cnt, off_items, off_mask, total;
+  size_t off_lse, off_delta, off_stat, off_cnt, off_phases, off_items, off_mask, total;
   uint32_t cap_items;
+  int32_t own_max;
   bool ok;
 };
 
-// items_bound: most (owner, segment) items one pass can leave behind, per problem
-GradLayout grad_layout(int64_t n_q, int64_t n_batch, int64_t items_bound, size_t mask_bytes) {
+GradLayout grad_layout(int64_t n_q, int64_t n_batch, ItemsBound bound, size_t mask_bytes) {
   GradLayout g{};
   const int64_t b = n_batch > 1 ? n_batch : 1;
-  const int64_t cap = items_bound * b + 1;
+  const int64_t cap = bound.items * b + 1;
   g.ok = cap < ((int64_t)1 << 31);
   g.cap_items = (uint32_t)(g.ok ? cap : 1);
+  g.own_max = (int32_t)bound.own_max;
   size_t off = 0;
-  g.off_lse = off;   off = align_up(off + (size_t)(n_q * b) * 4, 256);
-  g.off_delta = off; off = align_up(off + (size_t)(n_q * b) * 4, 256);
-  g.off_stat = off;  off = align_up(off + (size_t)(n_q * b) * 8, 256);
-  g.off_cnt = off;   off += 256;
-  g.off_items = off; off = align_up(off + (size_t)g.cap_items * 16, 256);  // two lists of pairs
-  g.off_mask = off;  off = align_up(off + mask_bytes, 256);
+  g.off_lse = off;    off = align_up(off + (size_t)(n_q * b) * 4, 256);
+  g.off_delta = off;  off = align_up(off + (size_t)(n_q * b) * 4, 256);
+  g.off_stat = off;   off = align_up(off + (size_t)(n_q * b) * 8, 256);
+  g.off_cnt = off;    off += 2 * 256;                                  // Counters of the two passes
+  g.off_phases = off; off += 2 * align_up(sizeof(Phases), 256);
+  // (a call that leaves no items - cap_items == 1 - never touches the lists)
+  g.off_items = off;  off = align_up(off + 4 * align_up((size_t)g.cap_items * sizeof(Item), 256), 256);
+  g.off_mask = off;   off = align_up(off + mask_bytes, 256);
   g.total = off;
   return g;
-}
-
-int64_t explicit_items_bound(int64_t nnz) { return nnz / kGradSegment + 1; }
-int64_t uniform_items_bound(int64_t n_rows, int64_t max_deg) {
-  return max_deg > kGradSegment ? n_rows * ((max_deg - 1) / kGradSegment) : 0;
-}
-int64_t global_items_bound(int64_t n, int64_t n_globals) {
-  return n_globals * ((n - 1) / kGradSegment) + uniform_items_bound(n, n_globals);
 }
 
 // what the transposed explicit mask needs: the entry list (rows, columns) and the conversion
@@ -988,9 +1013,16 @@ GradArgs make_grad_args(const spfa_problem_t* p, const spfa_grads_t* g, const Gr
   a.n_batch = batch_of(p);
   a.d = (int32_t)p->d;
   a.seg = (int32_t)kGradSegment;
-  a.n_items = (uint32_t*)(base + lay.off_cnt);
-  a.items = (uint32_t*)(base + lay.off_items);
+  a.own_max = lay.own_max;
+  const size_t list_bytes = align_up((size_t)lay.cap_items * sizeof(Item), 256);
+  for (int pass = 0; pass < 2; pass++) {
+    a.cnt[pass] = (Counters*)(base + lay.off_cnt + (size_t)pass * 256);
+    a.phases[pass] = (Phases*)(base + lay.off_phases + (size_t)pass * align_up(sizeof(Phases), 256));
+    a.listed[pass] = (Item*)(base + lay.off_items + (size_t)(2 * pass) * list_bytes);
+    a.ordered[pass] = (Item*)(base + lay.off_items + (size_t)(2 * pass + 1) * list_bytes);
+  }
   a.cap_items = lay.cap_items;
+  a.status = device_status_word();
   return a;
 }
 

@@ -569,6 +569,9 @@ __global__ __launch_bounds__(256) void segments_kernel(Tensors t, Mask mask, Pla
   if (plan.cnt->overflow) return;
   uint32_t n_items = plan.cnt->n_items;
   if (n_items > plan.cap_items) n_items = plan.cap_items;
+  // (an empty list: without this every wavefront would still queue up at the cursor once, 20 us
+  // for the 2048 of them)
+  if (n_items == 0) return;
   // every problem of the batch walks the same work list (the host keeps items * batch < 2^32)
   const uint32_t n_work = n_items * (uint32_t)t.n_batch;
   const float scale = 1.0f / sqrtf((float)t.d);

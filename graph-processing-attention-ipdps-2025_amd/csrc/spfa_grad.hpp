@@ -16,9 +16,10 @@
 // registers, replicated in every lane group; each group of LPR lanes takes one candidate at a
 // time (16 bytes per lane of each of its two rows, U candidates in flight per group), does both
 // dot products with in-group reductions and adds the weighted candidate rows to its
-// accumulators; the groups are summed at the end.  Owners with more than `seg` candidates do
-// their first `seg` here and leave (owner, segment) items behind for grad_items_kernel, whose
-// results are added with floating-point atomics (a few rows only).
+// accumulators; the groups are summed at the end.  Owners with more than `own_max` candidates
+// leave their segments of `seg` candidates on a work list instead, which is handed out in the
+// forward engine's order (segments at the same place in their rows together) to the persistent
+// wavefronts of grad_segments_kernel; their results are added with floating-point atomics.
 #pragma once
 
 #include "spfa_engine.hpp"
@@ -44,9 +45,15 @@ struct GradArgs {
   int64_t n_batch;
   int32_t d;
   int32_t seg;          // candidates one wavefront takes of a row
-  uint32_t* n_items;    // [2] counters of the two item lists (query pass, key pass)
-  uint32_t* items;      // [2][cap_items] pairs (owner among all problems, segment)
+  int32_t own_max;      // owners of more candidates leave all their segments on the work list
+  // the work lists of the two passes (query pass, key pass): the forward engine's items, `row`
+  // being the owner among all problems (32 bits), and its counters (item count, cursor, overflow)
+  Counters* cnt[2];
+  Phases* phases[2];
+  Item* listed[2];      // as appended
+  Item* ordered[2];     // in the order they are handed out in
   uint32_t cap_items;
+  uint32_t* status;     // the device's sticky status word (may be null)
 };
 
 constexpr int kGradWaves = 4;        // owners per workgroup
@@ -61,7 +68,6 @@ template <class Lay>
 constexpr int grad_rows_unroll() {
   return Lay::U_SHORT >= 2 ? Lay::U_SHORT / 2 : 1;
 }
-constexpr int kGradItemBlocks = 2048;
 
 template <class Lay>
 __device__ __forceinline__ int grad_elem_index(int c, int e) {
@@ -107,8 +113,30 @@ __global__ __launch_bounds__(256) void grad_prologue_kernel(Tensors t, GradArgs 
   }
 }
 
-static __global__ void grad_reset_kernel(uint32_t* n_items) {
-  if (threadIdx.x < 2) n_items[threadIdx.x] = 0;
+static __global__ void grad_reset_kernel(GradArgs g) {
+  static_assert(kPhases == kWave, "one lane per phase");
+  for (int p = 0; p < 2; p++) {
+    g.phases[p]->count[threadIdx.x] = 0;
+    g.phases[p]->taken[threadIdx.x] = 0;
+    if (threadIdx.x == 0) {
+      g.cnt[p]->n_items = 0;
+      g.cnt[p]->next_item = 0;
+      g.cnt[p]->overflow = 0;
+    }
+  }
+}
+
+// The work list of a pass as the forward engine's kernels see it (order_kernel, work_list()).
+__host__ __device__ inline Plan grad_plan(const GradArgs& g, int pass) {
+  Plan plan{};
+  plan.cnt = g.cnt[pass];
+  plan.cursor = &g.cnt[pass]->next_item;
+  plan.phases = g.phases[pass];
+  plan.listed = g.listed[pass];
+  plan.items = g.ordered[pass];
+  plan.cap_items = g.cap_items;
+  plan.seg = g.seg;
+  return plan;
 }
 
 // Candidates t_begin .. t_end of one owner, walked by the whole wavefront.
@@ -281,18 +309,31 @@ __global__ __launch_bounds__(kGradWaves* kWave) void grad_rows_kernel(GradArgs g
   const int64_t deg = rc.deg;
   if (deg <= 0) return;
   if (!KEYS && o.lse_o == __builtin_inff()) return;  // the row never saw a live column
-  const int64_t seg = g.seg;
-  if (deg > seg && lane == 0) {  // leave the rest of the row to the item kernel
-    const uint32_t extra = (uint32_t)((deg - 1) / seg);
-    uint32_t* cnt = g.n_items + (KEYS ? 1 : 0);
-    uint32_t* list = g.items + (size_t)(KEYS ? 2 : 0) * g.cap_items;
-    const uint32_t base = atomicAdd(cnt, extra);
-    for (uint32_t s = 0; s < extra; s++) {
-      if (base + s < g.cap_items) {
-        list[2 * (size_t)(base + s)] = (uint32_t)r;
-        list[2 * (size_t)(base + s) + 1] = s + 1;
+  if (deg > g.own_max) {
+    // all of the row goes on the work list, a segment per lane
+    const int pass = KEYS ? 1 : 0;
+    const int64_t seg = g.seg;
+    const uint32_t nseg = (uint32_t)((deg + seg - 1) / seg);
+    uint32_t base = 0;
+    if (lane == 0) base = atomicAdd(&g.cnt[pass]->n_items, nseg);
+    base = (uint32_t)__builtin_amdgcn_readfirstlane((int)base);
+    if (base + nseg > g.cap_items || base + nseg < base) {
+      if (lane == 0) {  // (only a mask whose arrays disagree with the nnz passed can get here)
+        atomicOr(&g.cnt[pass]->overflow, 1u);
+        if (g.status != nullptr) atomicOr(g.status, kStatusWorkListOverflow);
       }
+      return;
     }
+    for (uint32_t j = (uint32_t)lane; j < nseg; j += kWave) {
+      Item it;
+      it.row = (int32_t)(uint32_t)r;
+      it.seg = (int32_t)j;
+      it.slot = -1;
+      it.phase = (int32_t)segment_phase(j, nseg, deg, seg);
+      g.listed[pass][base + j] = it;
+      atomicAdd(&g.phases[pass]->count[it.phase], 1u);
+    }
+    return;
   }
   float acc1[NE], acc2[NE];
 #pragma unroll
@@ -302,7 +343,7 @@ __global__ __launch_bounds__(kGradWaves* kWave) void grad_rows_kernel(GradArgs g
   }
   const float scale = 1.0f / sqrtf((float)g.d);
   grad_walk<Lay, Mask, KEYS, grad_rows_unroll<Lay>()>(mask, rc, o.X, o.Y, o.stat_c, o.lse_o, o.delta_o,
-                                            g.d, scale, o.a, o.b, 0, deg < seg ? deg : seg, lane,
+                                            g.d, scale, o.a, o.b, 0, deg, lane,
                                             acc1, acc2);
   if (lane < Lay::LPR) {  // this wavefront is the only one that touches the row in this launch
     float cur[NE];
@@ -319,24 +360,39 @@ __global__ __launch_bounds__(kGradWaves* kWave) void grad_rows_kernel(GradArgs g
   }
 }
 
-// The segments grad_rows_kernel left behind, a wavefront per item, results added atomically.
+// Candidates in flight per lane group in grad_segments_kernel: the forward segment kernel's, as
+// long as the two owner vectors, the two accumulators and the rows in flight fit 256 registers.
+template <class Lay, bool KEYS>
+constexpr int grad_segments_unroll() {
+  return KEYS ? Lay::U_MEDIUM : Lay::U;
+}
+
+// The segments grad_rows_kernel left on the work list: a persistent grid, two workgroups per CU,
+// each wavefront pulls items off the ordered list (the forward engine's segments_kernel with the
+// gradient's arithmetic), results added atomically.
 template <class Lay, class Mask, bool KEYS>
-__global__ __launch_bounds__(kGradWaves* kWave) void grad_items_kernel(GradArgs g, Mask mask) {
+__global__ __launch_bounds__(256) void grad_segments_kernel(GradArgs g, Mask mask) {
   constexpr int NE = Lay::NE;
   const int lane = threadIdx.x & (kWave - 1);
   const int c = lane % Lay::LPR;
-  uint32_t n = g.n_items[KEYS ? 1 : 0];
-  if (n > g.cap_items) n = g.cap_items;
-  const uint32_t* list = g.items + (size_t)(KEYS ? 2 : 0) * g.cap_items;
-  const uint32_t stride = gridDim.x * kGradWaves;
+  const Plan plan = grad_plan(g, KEYS ? 1 : 0);
+  if (plan.cnt->overflow) return;
+  uint32_t n_items = plan.cnt->n_items;
+  if (n_items > plan.cap_items) n_items = plan.cap_items;
+  if (n_items == 0) return;  // (else every wavefront would still queue up at the cursor once)
+  const Item* const items = work_list(plan, n_items, lane);
   const float scale = 1.0f / sqrtf((float)g.d);
-  for (uint32_t it = blockIdx.x * kGradWaves + (threadIdx.x >> 6); it < n; it += stride) {
-    const int64_t r = (int64_t)list[2 * (size_t)it];
-    const int64_t s = (int64_t)list[2 * (size_t)it + 1];
+  while (true) {
+    uint32_t idx = 0;
+    if (lane == 0) idx = atomicAdd(plan.cursor, 1u);
+    idx = (uint32_t)__builtin_amdgcn_readfirstlane((int)idx);
+    if (idx >= n_items) break;
+    const Item it = items[idx];
+    const int64_t r = (int64_t)(uint32_t)it.row;
     GradOwner<Lay, KEYS> o;
     o.load(g, r, c);
     const typename Mask::Row rc = mask.row(o.ri);
-    const int64_t t0 = s * g.seg;
+    const int64_t t0 = (int64_t)it.seg * g.seg;
     const int64_t t1 = rc.deg < t0 + g.seg ? rc.deg : t0 + g.seg;
     float acc1[NE], acc2[NE];
 #pragma unroll
@@ -344,19 +400,21 @@ __global__ __launch_bounds__(kGradWaves* kWave) void grad_items_kernel(GradArgs 
       acc1[e] = 0.f;
       acc2[e] = 0.f;
     }
-    grad_walk<Lay, Mask, KEYS, Lay::U_MEDIUM>(mask, rc, o.X, o.Y, o.stat_c, o.lse_o,
-                                              o.delta_o, g.d, scale, o.a, o.b, t0, t1, lane, acc1,
-                                              acc2);
+    grad_walk<Lay, Mask, KEYS, grad_segments_unroll<Lay, KEYS>()>(mask, rc, o.X, o.Y, o.stat_c, o.lse_o,
+                                                                 o.delta_o, g.d, scale, o.a, o.b, t0, t1,
+                                                                 lane, acc1, acc2);
     if (lane < Lay::LPR) {
 #pragma unroll
       for (int e = 0; e < NE; e++) {
-        const int idx = grad_elem_index<Lay>(c, e);
-        if (idx < g.d) {
-          unsafeAtomicAdd(o.out1 + idx, acc1[e]);
-          if constexpr (KEYS) unsafeAtomicAdd(o.out2 + idx, acc2[e]);
+        const int idx_e = grad_elem_index<Lay>(c, e);
+        if (idx_e < g.d) {
+          unsafeAtomicAdd(o.out1 + idx_e, acc1[e]);
+          if constexpr (KEYS) unsafeAtomicAdd(o.out2 + idx_e, acc2[e]);
         }
       }
     }
+    // (every lane takes the next trip together: the work index is read across lanes at the top)
+    __builtin_amdgcn_wave_barrier();
   }
 }
 
@@ -368,17 +426,27 @@ int launch_grad(const Tensors& t, const GradArgs& g, const RowMask& rows, const 
   if (nq == 0 || nk == 0) return 0;
   if (nq >= ((int64_t)1 << 32) || nk >= ((int64_t)1 << 32)) return 1;  // items hold 32-bit owners
   const dim3 block(kGradWaves * kWave);
-  hipLaunchKernelGGL(grad_reset_kernel, dim3(1), dim3(64), 0, stream, g.n_items);
+  const bool lists = g.cap_items > 1;  // (no owner of this call can have more than own_max candidates otherwise)
+  const dim3 grid_order((g.cap_items + 255u) / 256u);
+  int64_t grid_seg = (int64_t)device_cu_count() * kSegmentWorkgroupsPerCu;
+  if (grid_seg > ((int64_t)g.cap_items + 3) / 4) grid_seg = ((int64_t)g.cap_items + 3) / 4;
+  hipLaunchKernelGGL(grad_reset_kernel, dim3(1), dim3(64), 0, stream, g);
   hipLaunchKernelGGL((grad_prologue_kernel<T>), dim3((unsigned)((nq + 15) / 16)), dim3(256), 0, stream,
                      t, g);
   hipLaunchKernelGGL((grad_rows_kernel<Lay, RowMask, false>),
                      dim3((unsigned)((nq + kGradWaves - 1) / kGradWaves)), block, 0, stream, g, rows);
-  hipLaunchKernelGGL((grad_items_kernel<Lay, RowMask, false>), dim3(kGradItemBlocks), block, 0, stream,
-                     g, rows);
+  if (lists) {
+    hipLaunchKernelGGL(order_kernel, grid_order, dim3(256), 0, stream, grad_plan(g, 0));
+    hipLaunchKernelGGL((grad_segments_kernel<Lay, RowMask, false>), dim3((unsigned)grid_seg), dim3(256), 0,
+                       stream, g, rows);
+  }
   hipLaunchKernelGGL((grad_rows_kernel<Lay, ColMask, true>),
                      dim3((unsigned)((nk + kGradWaves - 1) / kGradWaves)), block, 0, stream, g, cols);
-  hipLaunchKernelGGL((grad_items_kernel<Lay, ColMask, true>), dim3(kGradItemBlocks), block, 0, stream,
-                     g, cols);
+  if (lists) {
+    hipLaunchKernelGGL(order_kernel, grid_order, dim3(256), 0, stream, grad_plan(g, 1));
+    hipLaunchKernelGGL((grad_segments_kernel<Lay, ColMask, true>), dim3((unsigned)grid_seg), dim3(256), 0,
+                       stream, g, cols);
+  }
   return hipGetLastError() == hipSuccess ? 0 : 4;
 }
 
