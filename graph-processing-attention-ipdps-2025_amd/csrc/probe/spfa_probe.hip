@@ -3,7 +3,7 @@
 // segments_kernel spends its time fetching one K row and one V row per live position.  What the
 // memory system can deliver to exactly that access pattern - rows of `row_bytes` bytes picked by a
 // column list, 16 bytes per lane, a batch of 2 * U row loads issued back to back per lane group,
-// one persistent wavefront per SIMD pulling chunks of the list off an atomic cursor - is the
+// persistent wavefronts pulling chunks of the list off an atomic cursor - is the
 // ceiling that kernel can be priced against when K and V sit in the memory-side cache and the
 // HBM figure no longer binds.  This kernel does those loads and nothing else: no dot products, no
 // softmax, no output.  The loaded registers are handed to an empty asm statement so that the
@@ -43,11 +43,11 @@ __global__ __launch_bounds__(256) void gather_probe_kernel(const char* __restric
   const int gi = lane / LPR;
   const int c = lane % LPR;
   const int64_t n_chunks = (n_idx + chunk - 1) / chunk;
-  while (true) {
-    uint32_t w = 0;
-    if (lane == 0) w = atomicAdd(cursor, 1u);
-    w = (uint32_t)__builtin_amdgcn_readfirstlane((int)w);
-    if ((int64_t)w >= n_chunks) break;
+  // (as in the attention kernel: a wavefront's first chunk is the one with its own number, the
+  // later ones come off the cursor)
+  const uint32_t n_waves = gridDim.x * 4u;
+  uint32_t w = (uint32_t)__builtin_amdgcn_readfirstlane((int)(blockIdx.x * 4u + (threadIdx.x >> 6)));
+  while ((int64_t)w < n_chunks) {
     const int64_t t0 = (int64_t)w * chunk;
     const int64_t t1 = t0 + chunk < n_idx ? t0 + chunk : n_idx;
     int next = t0 + lane < t1 ? probe_entry(idx[t0 + lane], n_rows) : -1;
@@ -75,6 +75,9 @@ __global__ __launch_bounds__(256) void gather_probe_kernel(const char* __restric
         __builtin_amdgcn_sched_barrier(0);  // (one batch in flight at a time, as in the attention kernel)
       }
     }
+    uint32_t nx = 0;
+    if (lane == 0) nx = atomicAdd(cursor, 1u);
+    w = n_waves + (uint32_t)__builtin_amdgcn_readfirstlane((int)nx);
     __builtin_amdgcn_wave_barrier();
   }
 }
@@ -94,11 +97,11 @@ __global__ __launch_bounds__(256) void gather_probe_deep_kernel(const char* __re
   const int gi = lane / LPR;
   const int c = lane % LPR;
   const int64_t n_chunks = (n_idx + chunk - 1) / chunk;
-  while (true) {
-    uint32_t w = 0;
-    if (lane == 0) w = atomicAdd(cursor, 1u);
-    w = (uint32_t)__builtin_amdgcn_readfirstlane((int)w);
-    if ((int64_t)w >= n_chunks) break;
+  // (as in the attention kernel: a wavefront's first chunk is the one with its own number, the
+  // later ones come off the cursor)
+  const uint32_t n_waves = gridDim.x * 4u;
+  uint32_t w = (uint32_t)__builtin_amdgcn_readfirstlane((int)(blockIdx.x * 4u + (threadIdx.x >> 6)));
+  while ((int64_t)w < n_chunks) {
     const int64_t t0 = (int64_t)w * chunk;
     const int64_t t1 = t0 + chunk < n_idx ? t0 + chunk : n_idx;
     auto fetch = [&](int64_t t) -> int { return t + lane < t1 ? probe_entry(idx[t + lane], n_rows) : -1; };
@@ -127,6 +130,9 @@ __global__ __launch_bounds__(256) void gather_probe_deep_kernel(const char* __re
       }
       __builtin_amdgcn_sched_barrier(0);
     }
+    uint32_t nx = 0;
+    if (lane == 0) nx = atomicAdd(cursor, 1u);
+    w = n_waves + (uint32_t)__builtin_amdgcn_readfirstlane((int)nx);
     __builtin_amdgcn_wave_barrier();
   }
 }

@@ -577,11 +577,13 @@ __global__ __launch_bounds__(256) void segments_kernel(Tensors t, Mask mask, Pla
   const float scale = 1.0f / sqrtf((float)t.d);
   const Item* const items = work_list(plan, n_items, lane);
 
-  while (true) {
-    uint32_t idx = 0;
-    if (lane == 0) idx = atomicAdd(plan.cursor, 1u);
-    idx = (uint32_t)__builtin_amdgcn_readfirstlane((int)idx);
-    if (idx >= n_work) break;
+  // The first item of a wavefront is the one with its own number, the later ones come off the
+  // cursor: 2048 wavefronts that all begin with an atomic on the one address wait up to 20 us
+  // for each other before the first K row is asked for.
+  const uint32_t n_waves = gridDim.x * 4u;
+  uint32_t work = (uint32_t)__builtin_amdgcn_readfirstlane((int)(blockIdx.x * 4u + (threadIdx.x >> 6)));
+  while (work < n_work) {
+    uint32_t idx = work;
     uint32_t b = 0;
     if (t.n_batch > 1) {
       b = idx / n_items;
@@ -626,9 +628,12 @@ __global__ __launch_bounds__(256) void segments_kernel(Tensors t, Mask mask, Pla
         }
       }
     }
+    uint32_t next = 0;
+    if (lane == 0) next = atomicAdd(plan.cursor, 1u);
+    work = n_waves + (uint32_t)__builtin_amdgcn_readfirstlane((int)next);
     // Every lane of the wavefront must take the next trip together: the work index is read
-    // across lanes at the top of the loop.  A convergent operation in the only latch keeps the
-    // optimiser from giving the lanes that wrote the statistics a back edge of their own.
+    // across lanes.  A convergent operation in the only latch keeps the optimiser from giving
+    // the lanes that wrote the statistics a back edge of their own.
     __builtin_amdgcn_wave_barrier();
   }
 }

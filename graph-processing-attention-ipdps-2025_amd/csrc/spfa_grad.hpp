@@ -382,11 +382,10 @@ __global__ __launch_bounds__(256) void grad_segments_kernel(GradArgs g, Mask mas
   if (n_items == 0) return;  // (else every wavefront would still queue up at the cursor once)
   const Item* const items = work_list(plan, n_items, lane);
   const float scale = 1.0f / sqrtf((float)g.d);
-  while (true) {
-    uint32_t idx = 0;
-    if (lane == 0) idx = atomicAdd(plan.cursor, 1u);
-    idx = (uint32_t)__builtin_amdgcn_readfirstlane((int)idx);
-    if (idx >= n_items) break;
+  // (a wavefront's first item is the one with its own number, the later ones come off the cursor)
+  const uint32_t n_waves = gridDim.x * 4u;
+  uint32_t idx = (uint32_t)__builtin_amdgcn_readfirstlane((int)(blockIdx.x * 4u + (threadIdx.x >> 6)));
+  while (idx < n_items) {
     const Item it = items[idx];
     const int64_t r = (int64_t)(uint32_t)it.row;
     GradOwner<Lay, KEYS> o;
@@ -413,7 +412,10 @@ __global__ __launch_bounds__(256) void grad_segments_kernel(GradArgs g, Mask mas
         }
       }
     }
-    // (every lane takes the next trip together: the work index is read across lanes at the top)
+    uint32_t next = 0;
+    if (lane == 0) next = atomicAdd(plan.cursor, 1u);
+    idx = n_waves + (uint32_t)__builtin_amdgcn_readfirstlane((int)next);
+    // (every lane takes the next trip together: the work index is read across lanes)
     __builtin_amdgcn_wave_barrier();
   }
 }
