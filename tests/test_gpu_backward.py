@@ -224,14 +224,20 @@ def test_chained_parts_are_differentiated_as_their_union(mods, dtype):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_rows_and_columns_longer_than_one_segment(mods, dtype):
-    """Owners with more than 1024 live positions are split over several wavefronts: a query row
-    and a key column with ~2500 entries (explicit mask), a band of 1401, the rows and columns of
-    listed global tokens."""
+    """Owners with many live positions are split over several wavefronts: a query row and a key
+    column with ~2500 entries, rows and columns of 512 ... 2049 (explicit mask), a band of 1401, the
+    rows and columns of listed global tokens."""
     n, d = 2600, 64
     rng = np.random.default_rng(61)
     dense = rng.random((n, n)) < 0.01
     dense[7, rng.permutation(n)[:2500]] = True
     dense[rng.permutation(n)[:2500], 11] = True
+    # owners around the length from which a row goes on the work list, and around one segment
+    for i, ln in enumerate([512, 513, 1024, 1025, 2049]):
+        dense[20 + i, :] = False
+        dense[20 + i, rng.permutation(n)[:ln]] = True
+        dense[:, 40 + i] = False
+        dense[rng.permutation(n)[:ln], 40 + i] = True
     q, k, v, d_out = _problem(n, d, dtype, 62)
     for parts, mask in [([_csr_part(dense)], dense), ([_coo_part(dense, 63)], dense),
                         ([("local", 700)], so.mask_local_dense(n, 700)),
