@@ -34,7 +34,11 @@ inline int64_t pick_segment(int64_t nnz_long) {
   return seg;
 }
 
-constexpr int64_t kExplicitInlineRowLimit = 32;
+// Rows of up to this many entries are finished by the lane group that looks at them (rows_kernel).
+// 8 / 12 / 16 / 24 / 32 / 64 on the Zipf mask: 0.661 / 0.659 / 0.659 / 0.669 / 0.665 / 0.686 ms
+// fp32, 0.393 / 0.390 / 0.392 / 0.396 / 0.399 / 0.417 ms bf16; the 1 M-row COO mask and the 4 M-row
+// Zipf mask do not care.
+constexpr int64_t kExplicitInlineRowLimit = 16;
 // Rows between the two limits get a wavefront of their own (medium_rows_kernel).  Measured with
 // the limit at 64 / 128 / 256 / 512: the Zipf mask (12.8 M positions) does not care (0.867-0.873
 // ms); 64 heads of the 2 % Bernoulli mask (rows of ~83) need it above their row length (3.03 ms

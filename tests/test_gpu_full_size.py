@@ -86,7 +86,7 @@ def test_csr_zipf_n131072(mods):
     assert deg.min() >= 1 and deg.max() == 4096
     # sample every length class: shortest, longest, around the in-place limit, random
     rows = np.concatenate([np.nonzero(deg == 1)[0][:20], np.nonzero(deg == 4096)[0][:20],
-                           np.nonzero((deg >= 30) & (deg <= 36))[0][:20],
+                           np.nonzero((deg >= 14) & (deg <= 18))[0][:20], np.nonzero((deg >= 30) & (deg <= 36))[0][:20],
                            np.nonzero((deg > 250) & (deg < 520))[0][:20], rand_rows(n, 100, 2)])
     sample_check(q, k, v, o, m, l, rows, lambda i: ci_c[ro_c[i]:ro_c[i + 1]], torch.float32)
     # q == 0 -> l == row length exactly, m == 0

@@ -241,7 +241,7 @@ def test_csr_row_lengths_around_every_threshold(mods, dtype, d):
     segments exactly, and the longest possible row."""
     n = 2048
     rng = np.random.default_rng(3)
-    lengths = [0, 1, 2, 31, 32, 33, 63, 64, 65, 255, 256, 257, 511, 512, 513, 768, 1024, 2048, 0, 7]
+    lengths = [0, 1, 2, 15, 16, 17, 31, 32, 33, 63, 64, 65, 255, 256, 257, 511, 512, 513, 768, 1024, 2048, 0, 7]
     ro, ci = _special_rows_csr(n, rng, lengths)
     q, k, v = dev_qkv(n, d, dtype, 21)
     o, m, l = run_csr(mods, q, k, v, ro, ci, True, state_dtype=torch.float32)
