@@ -73,6 +73,8 @@ def load_library():
     lib.spfa_set_kernel_events.argtypes = [ctypes.c_void_p, ctypes.c_void_p]
     lib.spfa_set_kernel_events.restype = None
     lib.spfa_explicit_inline_row_limit.restype = ctypes.c_int64
+    lib.spfa_explicit_long_rows_on_grid.restype = ctypes.c_int
+    lib.spfa_explicit_long_rows_on_grid.argtypes = [ctypes.c_int64, ctypes.c_int64, ctypes.c_int]
     return lib
 
 
@@ -670,7 +672,9 @@ def measured_gather_ceiling(lib, w, torch, min_entries=8_000_000, reps=5, tensor
     # timed like the kernel it is compared with: the dispatch's own start and end stamps
     ev = HipEvents()
     best, best_shape = float("inf"), None
-    shapes = ((1, 8), (1, 16), (1, 32), (2, 8), (2, 16), (2, 32), (4, 4), (4, 8), (4, 16), (4, 32), (8, 4), (8, 8), (8, 16))
+    # (workgroups per CU of a persistent grid, or 0: an ordinary grid of one wavefront per 1024 list entries)
+    shapes = ((1, 8), (1, 16), (1, 32), (2, 8), (2, 16), (2, 32), (4, 4), (4, 8), (4, 16), (4, 32), (8, 4), (8, 8), (8, 16),
+              (0, 4), (0, 8), (0, 16))
     for wg, fl in shapes:
         for _ in range(reps):
             rc = probe.spfa_probe_gather(k.data_ptr(), v.data_ptr(), k.shape[0], row_bytes, idx.data_ptr(),
@@ -851,7 +855,8 @@ def main():
         # live: every XCD's 4 MiB L2, the 256 MiB memory-side cache, or HBM.  The 8 TB/s HBM figure
         # is only a ceiling when K and V do not fit the memory-side cache; below that the ceiling
         # is what the same gather without arithmetic sustains at this working set (measured here).
-        kernel_name = "segments_kernel"
+        on_grid = lib.spfa_explicit_long_rows_on_grid(int(w["k"].shape[-2]), int(d), {"f32": 0, "f16": 1, "bf16": 2}[a.dtype])
+        kernel_name = "items_grid_kernel" if on_grid else "segments_kernel"
         if w.get("whole_call") or w["kernel_nnz"] == 0:
             # no row is long enough for the segment kernel, or several kernels share the call: the
             # whole call stands in, with the call's algorithmic bytes

@@ -127,7 +127,7 @@ def _source_loop_depth(kname: str) -> int:
         # padded rows) also loops over query tiles
         return 2 if re.search(r"Li2ELb[01]EEEv", kname) else 1
     whole = "17whole_rows_kernelI" in kname  # (a medium-row walk inside its loop over long rows)
-    med = "18medium_rows_kernelI" in kname or whole
+    med = "18medium_rows_kernelI" in kname or "17items_grid_kernelI" in kname or whole
     if "15segments_kernelI" not in kname and "11rows_kernelI" not in kname and not med:
         return 1
     seg = "15segments_kernelI" in kname
@@ -142,7 +142,7 @@ def _source_loop_depth(kname: str) -> int:
         m = re.search(r"6GenLayI\w+?Li(\d+)E", kname)
         lpr, unroll = 64, (8 if int(m.group(1)) <= 2 else 2)
     if med and not whole:
-        # medium_rows_kernel names its batch size as a third template argument
+        # medium_rows_kernel and items_grid_kernel name their batch size as a third template argument
         m = re.search(r"MaskELi(\d+)EEEv", kname)
         if m:
             unroll = min(unroll, int(m.group(1)))

@@ -144,7 +144,9 @@ int launch_probe(const void* k, const void* v, int64_t row_bytes, uint32_t n_row
   int dev = 0, cus = 256;
   if (hipGetDevice(&dev) == hipSuccess)
     (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
-  const dim3 grid((unsigned)(cus * wg_per_cu)), block(256);
+  // wg_per_cu == 0: an ordinary grid, one wavefront per chunk of the list (items_grid_kernel's shape)
+  const int64_t n_chunks = (n_idx + chunk - 1) / chunk;
+  const dim3 grid((unsigned)(wg_per_cu > 0 ? (int64_t)cus * wg_per_cu : (n_chunks + 3) / 4)), block(256);
   hipLaunchKernelGGL(probe_reset_kernel, dim3(1), dim3(64), 0, stream, cursor);
   // (the gather itself takes the caller's event pair, as the kernel it stands in for does)
   constexpr int UMAX = LPR;  // a batch of U rows per group covers at most one 64-entry chunk
@@ -175,7 +177,7 @@ extern "C" int spfa_probe_gather(const void* k, const void* v, int64_t n_rows, i
                                  int in_flight, void* cursor, void* ev_start, void* ev_stop, void* stream) {
   using namespace spfa;
   if (!k || !v || !idx || !cursor || n_rows < 1 || n_rows > (int64_t)0x7fffffff || n_idx < 1 || chunk < 64 ||
-      wg_per_cu < 1 || wg_per_cu > 8)
+      wg_per_cu < 0 || wg_per_cu > 8 || (n_idx + chunk - 1) / chunk > (int64_t)0x7fffffff)
     return SPFA_ERR_BAD_ARG;
   KernelEvents ev;
   ev.start = (hipEvent_t)ev_start;

@@ -54,12 +54,24 @@ constexpr int64_t kExplicitMediumRowLimit = 256;
 constexpr int64_t kExplicitMediumRowLimitCached = 1024;
 constexpr int64_t kCachedKvBytes = (int64_t)24 << 20;
 
+// A mask whose rows hold 128 entries or more on average mostly has rows of about that length (a
+// power-law mask of that density being the exception), and rows of one length with sorted columns
+// are what a wavefront per row does best: launched together they walk K and V from low to high
+// columns in step and find each other's rows in the caches.  Uniform rows of 300 / 600 / 1000
+// sorted columns, fp32 d = 64, segment kernel against a wavefront per row: K + V of 16 MiB 8.9 /
+// 8.9 / 13.6 against 18.1 / 22.5 / 24.9 TB/s of gathered rows, 64 MiB 7.6 / 6.9 / 8.8 against 8.8 /
+// 11.7 / 13.5, 256 MiB 7.3 / 6.4 / 7.5 against 7.2 / 7.6 / 8.2; bf16 at 128 MiB 5.1 / 4.6 / 6.3
+// against 7.5 / 8.4 / 8.3.
+int64_t medium_limit_of_mask(int64_t n_q, int64_t nnz) {
+  return n_q > 0 && nnz / n_q >= 128 ? kExplicitMediumRowLimitCached : kExplicitMediumRowLimit;
+}
+
 EngineSizing size_csr(int64_t n_q, int64_t nnz) {
   EngineSizing s{};
   s.nnz_bound = nnz;
   s.max_deg = nnz;
   s.short_max = kExplicitInlineRowLimit;
-  s.medium_max = kExplicitMediumRowLimit;
+  s.medium_max = medium_limit_of_mask(n_q, nnz);
   s.seg = pick_segment(nnz);
   s.n_long_bound = n_q;
   return s;
@@ -70,6 +82,13 @@ int64_t explicit_medium_limit(const spfa_problem_t* p) {
   const int64_t es = p->dtype == SPFA_DTYPE_F32 ? 4 : p->dtype == SPFA_DTYPE_F64 ? 8 : 2;
   const int64_t kv = 2 * p->n_k * p->d * es * (p->n_batch > 1 ? p->n_batch : 1);
   return kv <= kCachedKvBytes ? kExplicitMediumRowLimitCached : kExplicitMediumRowLimit;
+}
+
+// whether the long rows' work list is walked by an ordinary grid (items_grid_kernel, see there)
+constexpr int64_t kItemsGridKvBytes = (int64_t)48 << 20;
+bool explicit_items_on_grid(int64_t n_k, int64_t d, int dtype) {
+  const int64_t es = dtype == SPFA_DTYPE_F32 ? 4 : dtype == SPFA_DTYPE_F64 ? 8 : 2;
+  return 2 * n_k * d * es <= kItemsGridKvBytes;
 }
 
 // ... and its batch size in the medium-row kernel (see there): smaller while K and V are not much
@@ -387,6 +406,10 @@ int spfa_version(void) { return 1; }
 
 int64_t spfa_explicit_inline_row_limit(void) { return kExplicitMediumRowLimit; }
 
+int spfa_explicit_long_rows_on_grid(int64_t n_k, int64_t d, int dtype) {
+  return explicit_items_on_grid(n_k, d, dtype) ? 1 : 0;
+}
+
 int spfa_device_status(int reset) {
   uint32_t* word = device_status_word();
   if (word == nullptr) return -1;
@@ -462,7 +485,8 @@ int spfa_csr_forward(const spfa_problem_t* p, const void* row_off, int row_off_b
     return run_f64(make_tensors(p), mask, use_nan ? 1 : 0, (hipStream_t)stream);
   }
   EngineSizing s = size_csr(p->n_q, nnz);
-  s.medium_max = explicit_medium_limit(p);
+  s.items_on_grid = explicit_items_on_grid(p->n_k, p->d, p->dtype);
+  if (explicit_medium_limit(p) > s.medium_max) s.medium_max = explicit_medium_limit(p);
   s.medium_batch = explicit_medium_batch(p, nnz);
   if (!batch_fits_engine(s, p)) {
     for (int64_t b = 0; b < batch_of(p); b++) {
@@ -513,6 +537,7 @@ int spfa_csr_forward_planned(const spfa_problem_t* p, const void* row_off, int r
     return run_f64(make_tensors(p), mask, use_nan ? 1 : 0, (hipStream_t)stream);
   }
   EngineSizing s = size_csr(p->n_q, nnz);
+  s.items_on_grid = explicit_items_on_grid(p->n_k, p->d, p->dtype);
   s.medium_batch = explicit_medium_batch(p, nnz);  // (a launch-time choice: the plan does not depend on it)
   rc = check_workspace(plan, plan_bytes, work_list_bytes(p->n_q, nnz));
   if (rc) return rc;
@@ -557,7 +582,8 @@ int spfa_coo_forward(const spfa_problem_t* p, const void* row_ind, int row_ind_b
   if (p->n_q == 0) return SPFA_OK;
   if (nnz > 0 && (!row_ind || !col_ind)) return SPFA_ERR_BAD_ARG;
   EngineSizing s = size_csr(p->n_q, nnz);
-  s.medium_max = explicit_medium_limit(p);
+  s.items_on_grid = explicit_items_on_grid(p->n_k, p->d, p->dtype);
+  if (explicit_medium_limit(p) > s.medium_max) s.medium_max = explicit_medium_limit(p);
   const size_t coo_bytes = coo_workspace(p->n_q, nnz).total;
   const bool batched = batch_fits_engine(s, p);
   rc = check_workspace(workspace, workspace_bytes,
@@ -627,6 +653,7 @@ int spfa_coo_forward_planned(const spfa_problem_t* p, const void* col_ind, int64
   if (p->n_q == 0) return SPFA_OK;
   if (nnz > 0 && !col_ind) return SPFA_ERR_BAD_ARG;
   EngineSizing s = size_csr(p->n_q, nnz);
+  s.items_on_grid = explicit_items_on_grid(p->n_k, p->d, p->dtype);
   const CooWorkspace w = coo_workspace(p->n_q, nnz);
   rc = check_workspace(plan, plan_bytes, w.keep_total + work_list_bytes(p->n_q, nnz));
   if (rc) return rc;

@@ -694,6 +694,72 @@ __global__ __launch_bounds__(256) void medium_rows_kernel(Tensors t, Mask mask, 
   if (g == 0) finish_row<Lay>(t, row, c, m, l, acc);
 }
 
+// The work list walked by an ordinary grid, one wavefront per item in list order, instead of by
+// segments_kernel's persistent wavefronts: the better of the two while K and V are not much
+// larger than the caches.  Eight wavefronts per SIMD with eight neighbours in flight per lane
+// group then draw more from the caches than two with sixteen, and, dispatched in list order,
+// they stay as close together in the list as the persistent ones.  The Zipf mask at N = 16 K /
+// 32 K / 64 K / 128 K / 256 K / 512 K / 1 M tokens, persistent -> grid, whole call: fp32 d = 64
+// - 33 / - 23 / - 13 / - 2 / + 1 / + 2 / + 3 %, bf16 d = 64 - 42 / - 38 / - 29 / - 19 / - 8 / 0 / + 3 %,
+// fp32 d = 128 - 14 / - 6 / + 1 / + 2 %, bf16 d = 128 - 28 / - 17 / - 8 / - 1 / + 2 %; eight heads of
+// the 128 K fp32 mask in one call + 5 %.  Taken when K + V of one problem are at most 48 MiB.
+template <class Lay, class Mask, int UM = Lay::U_MEDIUM>
+__global__ __launch_bounds__(256) void items_grid_kernel(Tensors t, Mask mask, Plan plan) {
+  using T = typename Lay::elem;
+  constexpr int NE = Lay::NE;
+  constexpr int LPR = Lay::LPR;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x >> 6;
+  const int g = lane / LPR;
+  const int c = lane % LPR;
+  if (plan.cnt->overflow) return;
+  uint32_t n_items = plan.cnt->n_items;
+  if (n_items > plan.cap_items) n_items = plan.cap_items;
+  int64_t idx = (int64_t)blockIdx.x * 4 + wave;
+  if (idx >= (int64_t)n_items * t.n_batch) return;
+  int64_t b = 0;
+  if (t.n_batch > 1) {
+    b = idx / n_items;
+    idx -= b * n_items;
+  }
+  const Item* const items = work_list(plan, n_items, lane);
+  const Item it = items[idx];
+  const int64_t row = b * t.n_q + it.row;
+  const int64_t slot = b * plan.cap_partials + it.slot;
+  const typename Mask::Row rc = mask.row(it.row);
+  const int64_t t0 = (int64_t)it.seg * plan.seg;
+  int64_t t1 = t0 + plan.seg;
+  if (t1 > rc.deg) t1 = rc.deg;
+  const float scale = 1.0f / sqrtf((float)t.d);
+  float q[NE];
+  load_q<Lay>(t, row, c, q);
+  float m = kNegInf, l = 0.f, acc[NE];
+#pragma unroll
+  for (int e = 0; e < NE; e++) acc[e] = 0.f;
+  attend<Lay, Mask, UM, kWave>(mask, rc, (const T*)t.k + b * t.kv_stride, (const T*)t.v + b * t.kv_stride,
+                               t.d, scale, q, t0, t1, lane, m, l, acc);
+#pragma unroll
+  for (int off = LPR; off < kWave; off <<= 1) {
+    float m2 = shfl_xor_f32(m, off);
+    float l2 = shfl_xor_f32(l, off);
+    float acc2[NE];
+#pragma unroll
+    for (int e = 0; e < NE; e++) acc2[e] = shfl_xor_f32(acc[e], off);
+    merge_partial<NE>(m, l, acc, m2, l2, acc2);
+  }
+  if (g == 0) {
+    if (it.slot < 0) {
+      finish_row<Lay>(t, row, c, m, l, acc);
+    } else {
+      Lay::store_f32(plan.pacc + slot * t.d, c, t.d, acc);
+      if (c == 0) {
+        plan.pm[slot] = m;
+        plan.pl[slot] = l;
+      }
+    }
+  }
+}
+
 // Small problems in one launch: one wavefront per row and problem (empty rows included), eight
 // rows per workgroup.  The general path is five launches and a work list; below a few tens of
 // thousands of rows those cost more than the attention (4096 rows of ~83 entries: 37 us, against
@@ -855,6 +921,7 @@ struct EngineSizing {
   int64_t seg;           // segment length for longer rows
   int64_t n_long_bound;  // upper bound on the number of rows with deg > short_max
   int medium_batch;      // neighbours in flight per lane group in medium_rows_kernel (0: the layout's)
+  bool items_on_grid;    // the work list is walked by items_grid_kernel (explicit masks)
 };
 
 struct WorkspaceLayout {
@@ -1058,8 +1125,17 @@ int launch_engine(const Tensors& t, const Mask& mask, const EngineSizing& s, int
     int64_t need = ((int64_t)w.cap_items * t.n_batch + 3) / 4;
     if (grid2 > need) grid2 = need;
     if (grid2 < 1) grid2 = 1;
-    launch_maybe_timed(ev, segments_kernel<Lay, Mask>, dim3((unsigned)grid2), dim3(256), stream, t, mask,
-                       plan);
+    bool on_grid = false;
+    if constexpr (Mask::kExplicit) {
+      if (s.items_on_grid) {
+        launch_maybe_timed(ev, items_grid_kernel<Lay, Mask>, dim3((unsigned)need), dim3(256), stream, t, mask,
+                           plan);
+        on_grid = true;
+      }
+    }
+    if (!on_grid)
+      launch_maybe_timed(ev, segments_kernel<Lay, Mask>, dim3((unsigned)grid2), dim3(256), stream, t, mask,
+                         plan);
     const int64_t grid3 = ((int64_t)w.cap_multi * t.n_batch + rows_per_wg - 1) / rows_per_wg;
     hipLaunchKernelGGL((merge_kernel<Lay>), dim3((unsigned)grid3), dim3(256), 0, stream, t, plan);
   }

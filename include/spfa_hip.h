@@ -118,6 +118,12 @@ void spfa_set_kernel_events(void* start, void* stop);
  * benchmark can attribute bytes to kernels. */
 int64_t spfa_explicit_inline_row_limit(void);
 
+/* 1 when a CSR / COO call with n_k keys of d elements of `dtype` walks the segments of its long
+ * rows with an ordinary grid (items_grid_kernel) instead of the persistent segments_kernel: K and V
+ * of one problem small enough to stay in the caches.  Exposed so a benchmark can name the kernel
+ * it times. */
+int spfa_explicit_long_rows_on_grid(int64_t n_k, int64_t d, int dtype);
+
 /* CSR: row i attends col_ind[row_off[i] .. row_off[i+1]).  row_off has n_q+1 entries of
  * row_off_bytes (4 or 8) bytes each, col_ind has nnz 4-byte entries; signed and unsigned
  * index tensors are bit-identical in range.  The reference's value vector is never read

@@ -18,7 +18,8 @@ extern "C" {
  * every entry with the top bit set - is skipped), 16 bytes per lane, `in_flight` (4, 8, 16 or 32)
  * rows of each per lane group issued back to back, by a persistent grid of wg_per_cu (1..8)
  * four-wavefront workgroups per compute unit whose wavefronts pull runs of `chunk` (>= 64) entries
- * off an atomic cursor (`cursor`: 4 bytes of device memory).  Nothing is computed or written.
+ * off an atomic cursor (`cursor`: 4 bytes of device memory), or, with wg_per_cu = 0, by an ordinary
+ * grid of one wavefront per run of `chunk` entries.  Nothing is computed or written.
  * When ev_start and ev_stop (hipEvent_t passed as void*) are both non-NULL they are attached to
  * the gather's own dispatch, so hipEventElapsedTime gives its duration without launch overhead.
  * The rate it reaches is what the memory system sustains for this access pattern at a given
