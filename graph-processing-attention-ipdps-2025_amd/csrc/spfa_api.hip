@@ -1054,6 +1054,9 @@ GradArgs make_grad_args(const spfa_problem_t* p, const spfa_grads_t* g, const Gr
   }
   a.cap_items = lay.cap_items;
   a.status = device_status_word();
+  // (explicit masks whose gathered tensors - K, V in the query pass, Q, dO in the key pass - stay in the caches)
+  a.items_on_grid = lay.own_max == kGradOwnExplicit &&
+                    explicit_items_on_grid(p->n_k > p->n_q ? p->n_k : p->n_q, p->d, p->dtype) ? 1 : 0;
   return a;
 }
 

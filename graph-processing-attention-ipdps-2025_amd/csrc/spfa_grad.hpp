@@ -54,6 +54,7 @@ struct GradArgs {
   Item* ordered[2];     // in the order they are handed out in
   uint32_t cap_items;
   uint32_t* status;     // the device's sticky status word (may be null)
+  int32_t items_on_grid;  // the work lists are walked by an ordinary grid, a wavefront per item
 };
 
 constexpr int kGradWaves = 4;        // owners per workgroup
@@ -370,7 +371,9 @@ constexpr int grad_segments_unroll() {
 // The segments grad_rows_kernel left on the work list: a persistent grid, two workgroups per CU,
 // each wavefront pulls items off the ordered list (the forward engine's segments_kernel with the
 // gradient's arithmetic), results added atomically.
-template <class Lay, class Mask, bool KEYS>
+// GRID: an ordinary grid of one wavefront per item instead (the forward engine's
+// items_grid_kernel: the better shape while the gathered tensors stay in the caches).
+template <class Lay, class Mask, bool KEYS, bool GRID = false>
 __global__ __launch_bounds__(256) void grad_segments_kernel(GradArgs g, Mask mask) {
   constexpr int NE = Lay::NE;
   const int lane = threadIdx.x & (kWave - 1);
@@ -399,7 +402,7 @@ __global__ __launch_bounds__(256) void grad_segments_kernel(GradArgs g, Mask mas
       acc1[e] = 0.f;
       acc2[e] = 0.f;
     }
-    grad_walk<Lay, Mask, KEYS, grad_segments_unroll<Lay, KEYS>()>(mask, rc, o.X, o.Y, o.stat_c, o.lse_o,
+    grad_walk<Lay, Mask, KEYS, (GRID ? Lay::U_MEDIUM : grad_segments_unroll<Lay, KEYS>())>(mask, rc, o.X, o.Y, o.stat_c, o.lse_o,
                                                                  o.delta_o, g.d, scale, o.a, o.b, t0, t1,
                                                                  lane, acc1, acc2);
     if (lane < Lay::LPR) {
@@ -412,6 +415,7 @@ __global__ __launch_bounds__(256) void grad_segments_kernel(GradArgs g, Mask mas
         }
       }
     }
+    if constexpr (GRID) break;
     uint32_t next = 0;
     if (lane == 0) next = atomicAdd(plan.cursor, 1u);
     idx = n_waves + (uint32_t)__builtin_amdgcn_readfirstlane((int)next);
@@ -439,15 +443,23 @@ int launch_grad(const Tensors& t, const GradArgs& g, const RowMask& rows, const 
                      dim3((unsigned)((nq + kGradWaves - 1) / kGradWaves)), block, 0, stream, g, rows);
   if (lists) {
     hipLaunchKernelGGL(order_kernel, grid_order, dim3(256), 0, stream, grad_plan(g, 0));
-    hipLaunchKernelGGL((grad_segments_kernel<Lay, RowMask, false>), dim3((unsigned)grid_seg), dim3(256), 0,
-                       stream, g, rows);
+    if (g.items_on_grid)
+      hipLaunchKernelGGL((grad_segments_kernel<Lay, RowMask, false, true>), dim3((g.cap_items + 3u) / 4u),
+                         dim3(256), 0, stream, g, rows);
+    else
+      hipLaunchKernelGGL((grad_segments_kernel<Lay, RowMask, false>), dim3((unsigned)grid_seg), dim3(256), 0,
+                         stream, g, rows);
   }
   hipLaunchKernelGGL((grad_rows_kernel<Lay, ColMask, true>),
                      dim3((unsigned)((nk + kGradWaves - 1) / kGradWaves)), block, 0, stream, g, cols);
   if (lists) {
     hipLaunchKernelGGL(order_kernel, grid_order, dim3(256), 0, stream, grad_plan(g, 1));
-    hipLaunchKernelGGL((grad_segments_kernel<Lay, ColMask, true>), dim3((unsigned)grid_seg), dim3(256), 0,
-                       stream, g, cols);
+    if (g.items_on_grid)
+      hipLaunchKernelGGL((grad_segments_kernel<Lay, ColMask, true, true>), dim3((g.cap_items + 3u) / 4u),
+                         dim3(256), 0, stream, g, cols);
+    else
+      hipLaunchKernelGGL((grad_segments_kernel<Lay, ColMask, true>), dim3((unsigned)grid_seg), dim3(256), 0,
+                         stream, g, cols);
   }
   return hipGetLastError() == hipSuccess ? 0 : 4;
 }
