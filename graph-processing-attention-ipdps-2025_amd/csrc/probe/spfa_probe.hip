@@ -75,6 +75,7 @@ __global__ __launch_bounds__(256) void gather_probe_kernel(const char* __restric
         __builtin_amdgcn_sched_barrier(0);  // (one batch in flight at a time, as in the attention kernel)
       }
     }
+    if ((int64_t)n_waves >= n_chunks) break;  // (an ordinary grid: a chunk per wavefront, no cursor)
     uint32_t nx = 0;
     if (lane == 0) nx = atomicAdd(cursor, 1u);
     w = n_waves + (uint32_t)__builtin_amdgcn_readfirstlane((int)nx);
@@ -130,6 +131,7 @@ __global__ __launch_bounds__(256) void gather_probe_deep_kernel(const char* __re
       }
       __builtin_amdgcn_sched_barrier(0);
     }
+    if ((int64_t)n_waves >= n_chunks) break;  // (an ordinary grid: a chunk per wavefront, no cursor)
     uint32_t nx = 0;
     if (lane == 0) nx = atomicAdd(cursor, 1u);
     w = n_waves + (uint32_t)__builtin_amdgcn_readfirstlane((int)nx);
