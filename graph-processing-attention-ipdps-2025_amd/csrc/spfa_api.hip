@@ -47,7 +47,7 @@ constexpr int64_t kExplicitMediumRowLimit = 256;
 // ... and rows of up to this many when K and V are small enough to stay in the caches: the
 // persistent kernel (two wavefronts per SIMD, tuned for the latency of memory-side fills) then
 // leaves most of the cache bandwidth unused on single-segment rows, which an ordinary grid of
-// eight wavefronts per SIMD does not.  Uniform rows of 257 ... 1000 entries, limit 256 -> 1024:
+// several wavefronts per SIMD does not.  Uniform rows of 257 ... 1000 entries, limit 256 -> 1024:
 // 8192 tokens at d = 64 fp32 4.9 ... 12.5 -> 13.2 ... 20.9 TB/s of gathered rows, 20000 tokens bf16
 // 4.8 ... 8.5 -> 12.1 ... 19.0; at K + V = 32 MiB the two are level, beyond that the persistent kernel
 // is ahead (the Zipf headline, 64 MiB: + 2.4 % with 1024 for every size).

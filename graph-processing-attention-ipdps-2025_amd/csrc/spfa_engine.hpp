@@ -696,9 +696,10 @@ __global__ __launch_bounds__(256) void medium_rows_kernel(Tensors t, Mask mask, 
 
 // The work list walked by an ordinary grid, one wavefront per item in list order, instead of by
 // segments_kernel's persistent wavefronts: the better of the two while K and V are not much
-// larger than the caches.  Eight wavefronts per SIMD with eight neighbours in flight per lane
-// group then draw more from the caches than two with sixteen, and, dispatched in list order,
-// they stay as close together in the list as the persistent ones.  The Zipf mask at N = 16 K /
+// larger than the caches.  Three or four wavefronts per SIMD (127 / 139 registers at fp32 / bf16
+// d = 64) with eight neighbours in flight per lane group then draw more from the caches than two
+// with sixteen, and, dispatched in list order, they stay as close together in the list as the
+// persistent ones.  The Zipf mask at N = 16 K /
 // 32 K / 64 K / 128 K / 256 K / 512 K / 1 M tokens, persistent -> grid, whole call: fp32 d = 64
 // - 33 / - 23 / - 13 / - 2 / + 1 / + 2 / + 3 %, bf16 d = 64 - 42 / - 38 / - 29 / - 19 / - 8 / 0 / + 3 %,
 // fp32 d = 128 - 14 / - 6 / + 1 / + 2 %, bf16 d = 128 - 28 / - 17 / - 8 / - 1 / + 2 %; eight heads of
