@@ -85,10 +85,12 @@ int64_t explicit_medium_limit(const spfa_problem_t* p) {
 }
 
 // whether the long rows' work list is walked by an ordinary grid (items_grid_kernel, see there)
+// (rows of at most 128 bytes keep the advantage longer: bf16 d = 64 at K + V = 64 MiB - 8 %, even at 128 MiB)
 constexpr int64_t kItemsGridKvBytes = (int64_t)48 << 20;
+constexpr int64_t kItemsGridKvBytesShortRows = (int64_t)96 << 20;
 bool explicit_items_on_grid(int64_t n_k, int64_t d, int dtype) {
   const int64_t es = dtype == SPFA_DTYPE_F32 ? 4 : dtype == SPFA_DTYPE_F64 ? 8 : 2;
-  return 2 * n_k * d * es <= kItemsGridKvBytes;
+  return 2 * n_k * d * es <= (d * es <= 128 ? kItemsGridKvBytesShortRows : kItemsGridKvBytes);
 }
 
 // ... and its batch size in the medium-row kernel (see there): smaller while K and V are not much

@@ -703,7 +703,7 @@ __global__ __launch_bounds__(256) void medium_rows_kernel(Tensors t, Mask mask, 
 // 32 K / 64 K / 128 K / 256 K / 512 K / 1 M tokens, persistent -> grid, whole call: fp32 d = 64
 // - 33 / - 23 / - 13 / - 2 / + 1 / + 2 / + 3 %, bf16 d = 64 - 42 / - 38 / - 29 / - 19 / - 8 / 0 / + 3 %,
 // fp32 d = 128 - 14 / - 6 / + 1 / + 2 %, bf16 d = 128 - 28 / - 17 / - 8 / - 1 / + 2 %; eight heads of
-// the 128 K fp32 mask in one call + 5 %.  Taken when K + V of one problem are at most 48 MiB.
+// the 128 K fp32 mask in one call + 5 %.  Taken when K + V of one problem are at most 48 MiB (96 MiB for rows of at most 128 bytes).
 template <class Lay, class Mask, int UM = Lay::U_MEDIUM>
 __global__ __launch_bounds__(256) void items_grid_kernel(Tensors t, Mask mask, Plan plan) {
   using T = typename Lay::elem;

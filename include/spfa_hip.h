@@ -120,7 +120,7 @@ int64_t spfa_explicit_inline_row_limit(void);
 
 /* 1 when a CSR / COO call with n_k keys of d elements of `dtype` walks the segments of its long
  * rows with an ordinary grid (items_grid_kernel) instead of the persistent segments_kernel: K and V
- * of one problem small enough to stay in the caches.  Exposed so a benchmark can name the kernel
+ * of one problem small enough to stay in the caches (48 MiB; 96 MiB for rows of at most 128 bytes).  Exposed so a benchmark can name the kernel
  * it times. */
 int spfa_explicit_long_rows_on_grid(int64_t n_k, int64_t d, int dtype);
 
