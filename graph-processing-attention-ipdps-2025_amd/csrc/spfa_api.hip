@@ -23,13 +23,14 @@ inline bool dtype_ok(int dtype) {
   return dtype == SPFA_DTYPE_F32 || dtype == SPFA_DTYPE_F16 || dtype == SPFA_DTYPE_BF16;
 }
 
-// segment length: enough segments to keep every wavefront slot busy several times over, long
-// enough that the per-segment overhead (q load, group merge, partial write) stays small
 // Segment length for long rows: long enough to amortise the pipeline fill and the partial
 // result of a segment (1024 candidates: 64 per lane group at d*s = 256 bytes), short enough
-// that the work list holds several items per persistent wavefront (about 2048 of them).
+// that the work list holds several items per persistent wavefront (about 2048 of them) - but
+// never below 512: small masks are walked by an ordinary grid, which does not need the items
+// for its balance and pays for every one of them (the Zipf mask at 8192 / 16384 tokens, 128 ->
+// 512: 0.139 -> 0.121 / 0.172 -> 0.146 ms fp32, 0.108 -> 0.083 / 0.132 -> 0.097 ms bf16).
 inline int64_t pick_segment(int64_t nnz_long) {
-  int64_t seg = 128;
+  int64_t seg = 512;
   while (seg < 1024 && seg * 2 * 8192 <= nnz_long) seg *= 2;
   return seg;
 }

@@ -269,12 +269,13 @@ def test_csr_small_problem_with_very_long_rows(mods, dtype, d):
 
 @pytest.mark.parametrize("dtype,d", [(torch.float32, 64), (torch.bfloat16, 64), (torch.float32, 40)])
 def test_csr_rows_of_more_segments_than_the_work_list_has_phases(mods, dtype, d):
-    """More keys than the single-launch path takes, so the rows go through the work list: rows cut into up to 157
-    segments of 128 (the list is handed out in 64 phases, so several segments of a row share one), rows of one
+    """More keys than the single-launch path takes, so the rows go through the work list: rows cut into up to 79
+    segments of 512 (the list is handed out in 64 phases, so several segments of a row share one), rows of one
     and two segments, medium and short rows, empty rows."""
-    n_q, n_k = 64, 20000
+    n_q, n_k = 64, 40000
     rng = np.random.default_rng(91)
-    lengths = [20000, 19999, 9000, 300, 257, 256, 129, 128, 33, 5, 0, 1] + [int(x) for x in rng.integers(0, 400, n_q - 12)]
+    lengths = [40000, 39999, 9000, 1025, 1024, 513, 512, 300, 257, 256, 129, 128, 33, 17, 16, 5, 0, 1] + \
+        [int(x) for x in rng.integers(0, 400, n_q - 18)]
     cols, off = [], [0]
     for ln in lengths:
         cols.append(np.sort(rng.choice(n_k, ln, replace=False)))
