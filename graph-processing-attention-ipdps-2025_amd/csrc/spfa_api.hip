@@ -45,14 +45,13 @@ constexpr int64_t kExplicitInlineRowLimit = 16;
 // ms); 64 heads of the 2 % Bernoulli mask (rows of ~83) need it above their row length (3.03 ms
 // without, 0.65 with).
 constexpr int64_t kExplicitMediumRowLimit = 256;
-// ... and rows of up to this many when K and V are small enough to stay in the caches: the
-// persistent kernel (two wavefronts per SIMD, tuned for the latency of memory-side fills) then
-// leaves most of the cache bandwidth unused on single-segment rows, which an ordinary grid of
-// several wavefronts per SIMD does not.  Uniform rows of 257 ... 1000 entries, limit 256 -> 1024:
-// 8192 tokens at d = 64 fp32 4.9 ... 12.5 -> 13.2 ... 20.9 TB/s of gathered rows, 20000 tokens bf16
-// 4.8 ... 8.5 -> 12.1 ... 19.0; at K + V = 32 MiB the two are level, beyond that the persistent kernel
-// is ahead (the Zipf headline, 64 MiB: + 2.4 % with 1024 for every size).
-constexpr int64_t kExplicitMediumRowLimitCached = 1024;
+// ... and rows of up to this many in the masks described below.  (A rule that took 1024 for
+// every mask whose K and V stay in the caches, from when the work list was walked row by row by
+// persistent wavefronts only, costs the Zipf mask 19 - 27 % at 8192 ... 32768 tokens now: its
+// rows of 257 ... 1024 entries, each of another length, are better off as items of the ordered
+// work list than as wavefronts of their own.)
+constexpr int64_t kExplicitMediumRowLimitDense = 1024;
+// K + V up to which the medium-row kernel takes smaller batches (explicit_medium_batch)
 constexpr int64_t kCachedKvBytes = (int64_t)24 << 20;
 
 // A mask whose rows hold 128 entries or more on average mostly has rows of about that length (a
@@ -64,7 +63,7 @@ constexpr int64_t kCachedKvBytes = (int64_t)24 << 20;
 // 11.7 / 13.5, 256 MiB 7.3 / 6.4 / 7.5 against 7.2 / 7.6 / 8.2; bf16 at 128 MiB 5.1 / 4.6 / 6.3
 // against 7.5 / 8.4 / 8.3.
 int64_t medium_limit_of_mask(int64_t n_q, int64_t nnz) {
-  return n_q > 0 && nnz / n_q >= 128 ? kExplicitMediumRowLimitCached : kExplicitMediumRowLimit;
+  return n_q > 0 && nnz / n_q >= 128 ? kExplicitMediumRowLimitDense : kExplicitMediumRowLimit;
 }
 
 EngineSizing size_csr(int64_t n_q, int64_t nnz) {
@@ -76,13 +75,6 @@ EngineSizing size_csr(int64_t n_q, int64_t nnz) {
   s.seg = pick_segment(nnz);
   s.n_long_bound = n_q;
   return s;
-}
-
-// the medium-row limit of a plain call (a mask plan is built without knowing K and V)
-int64_t explicit_medium_limit(const spfa_problem_t* p) {
-  const int64_t es = p->dtype == SPFA_DTYPE_F32 ? 4 : p->dtype == SPFA_DTYPE_F64 ? 8 : 2;
-  const int64_t kv = 2 * p->n_k * p->d * es * (p->n_batch > 1 ? p->n_batch : 1);
-  return kv <= kCachedKvBytes ? kExplicitMediumRowLimitCached : kExplicitMediumRowLimit;
 }
 
 // whether the long rows' work list is walked by an ordinary grid (items_grid_kernel, see there)
@@ -489,7 +481,6 @@ int spfa_csr_forward(const spfa_problem_t* p, const void* row_off, int row_off_b
   }
   EngineSizing s = size_csr(p->n_q, nnz);
   s.items_on_grid = explicit_items_on_grid(p->n_k, p->d, p->dtype);
-  if (explicit_medium_limit(p) > s.medium_max) s.medium_max = explicit_medium_limit(p);
   s.medium_batch = explicit_medium_batch(p, nnz);
   if (!batch_fits_engine(s, p)) {
     for (int64_t b = 0; b < batch_of(p); b++) {
@@ -586,7 +577,6 @@ int spfa_coo_forward(const spfa_problem_t* p, const void* row_ind, int row_ind_b
   if (nnz > 0 && (!row_ind || !col_ind)) return SPFA_ERR_BAD_ARG;
   EngineSizing s = size_csr(p->n_q, nnz);
   s.items_on_grid = explicit_items_on_grid(p->n_k, p->d, p->dtype);
-  if (explicit_medium_limit(p) > s.medium_max) s.medium_max = explicit_medium_limit(p);
   const size_t coo_bytes = coo_workspace(p->n_q, nnz).total;
   const bool batched = batch_fits_engine(s, p);
   rc = check_workspace(workspace, workspace_bytes,
