@@ -903,11 +903,25 @@ __global__ __launch_bounds__(256) void merge_kernel(Tensors t, Plan plan) {
   float m = kNegInf, l = 0.f, acc[NE];
 #pragma unroll
   for (int e = 0; e < NE; e++) acc[e] = 0.f;
-  for (int j = 0; j < mr.nseg; j++) {
-    const int64_t slot = b * plan.cap_partials + mr.slot0 + j;
-    float acc2[NE];
-    Lay::load_f32(plan.pacc + slot * t.d, c, t.d, acc2);
-    merge_partial<NE>(m, l, acc, plan.pm[slot], plan.pl[slot], acc2);
+  // four partials per trip, all of them asked for before the first is folded in (a trip per
+  // partial is a memory round trip per partial: 8.1 -> 5 us for rows of up to eight segments)
+  for (int j0 = 0; j0 < mr.nseg; j0 += 4) {
+    float pm4[4], pl4[4], acc4[4][NE];
+#pragma unroll
+    for (int u = 0; u < 4; u++) {
+      pm4[u] = kNegInf;
+      pl4[u] = 0.f;
+#pragma unroll
+      for (int e = 0; e < NE; e++) acc4[u][e] = 0.f;
+      if (j0 + u < mr.nseg) {
+        const int64_t slot = b * plan.cap_partials + mr.slot0 + j0 + u;
+        Lay::load_f32(plan.pacc + slot * t.d, c, t.d, acc4[u]);
+        pm4[u] = plan.pm[slot];
+        pl4[u] = plan.pl[slot];
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < 4; u++) merge_partial<NE>(m, l, acc, pm4[u], pl4[u], acc4[u]);
   }
   finish_row<Lay>(t, b * t.n_q + mr.row, c, m, l, acc);
 }
