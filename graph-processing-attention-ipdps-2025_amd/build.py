@@ -127,6 +127,11 @@ def _source_loop_depth(kname: str) -> int:
         # padded rows) also loops over query tiles
         return 2 if re.search(r"Li2ELb[01]EEEv", kname) else 1
     whole = "17whole_rows_kernelI" in kname  # (a medium-row walk inside its loop over long rows)
+    if "20explicit_rows_kernelI" in kname:
+        # the item, medium-row and short-row kernels in one launch: the deepest nest of the three
+        # (the first two with the layout's own batch size)
+        return max(_source_loop_depth(kname.replace("20explicit_rows_kernelI", "18medium_rows_kernelI")),
+                   _source_loop_depth(kname.replace("20explicit_rows_kernelI", "11rows_kernelI")))
     med = "18medium_rows_kernelI" in kname or "17items_grid_kernelI" in kname or whole
     if "15segments_kernelI" not in kname and "11rows_kernelI" not in kname and not med:
         return 1

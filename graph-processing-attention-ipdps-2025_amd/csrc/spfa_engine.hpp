@@ -495,7 +495,7 @@ __device__ __forceinline__ void order_wave(const Plan& plan, uint32_t wave_index
 }
 
 template <class Lay, class Mask>
-__global__ __launch_bounds__(256) void rows_kernel(Tensors t, Mask mask, Plan plan) {
+__device__ __forceinline__ void rows_body(const Tensors& t, const Mask& mask, const Plan& plan, int64_t block) {
   using T = typename Lay::elem;
   constexpr int NE = Lay::NE;
   constexpr int LPR = Lay::LPR;
@@ -503,7 +503,7 @@ __global__ __launch_bounds__(256) void rows_kernel(Tensors t, Mask mask, Plan pl
   const int wave = threadIdx.x >> 6;
   const int g = lane / LPR;
   const int c = lane % LPR;
-  const int64_t idx = ((int64_t)blockIdx.x * 4 + wave) * Lay::GROUPS + g;
+  const int64_t idx = (block * 4 + wave) * Lay::GROUPS + g;
   // A mask whose rows are mostly empty (and stay untouched) would spend a lane group on every
   // empty row and a wavefront on every four rows that hold one short row among them: the rows are
   // then taken from the list of non-empty short rows that plan_kernel made.
@@ -545,6 +545,11 @@ __global__ __launch_bounds__(256) void rows_kernel(Tensors t, Mask mask, Plan pl
     finish_row<Lay>(t, row, c, m, l, acc);
   }
   // longer rows were cut into segments by plan_kernel and belong to segments_kernel
+}
+
+template <class Lay, class Mask>
+__global__ __launch_bounds__(256) void rows_kernel(Tensors t, Mask mask, Plan plan) {
+  rows_body<Lay, Mask>(t, mask, plan, (int64_t)blockIdx.x);
 }
 
 // The list segments_kernel walks: the ordered one, or the list as appended when all its items
@@ -651,8 +656,8 @@ __global__ __launch_bounds__(256) void segments_kernel(Tensors t, Mask mask, Pla
 // caches that is worth more than the loads in flight per wavefront (uniform rows of 192 sorted
 // columns, 65536 tokens, fp32 d = 64: 8.8 TB/s of gathered rows with 8, 11.1 with 4, 9.1 with 2;
 // 20000 tokens: 14.1 / 15.2 / 16.5; from 262144 tokens on it makes no difference).
-template <class Lay, class Mask, int UM = Lay::U_MEDIUM>
-__global__ __launch_bounds__(256) void medium_rows_kernel(Tensors t, Mask mask, Plan plan) {
+template <class Lay, class Mask, int UM>
+__device__ __forceinline__ void medium_rows_body(const Tensors& t, const Mask& mask, const Plan& plan, int64_t block) {
   using T = typename Lay::elem;
   constexpr int NE = Lay::NE;
   constexpr int LPR = Lay::LPR;
@@ -663,7 +668,7 @@ __global__ __launch_bounds__(256) void medium_rows_kernel(Tensors t, Mask mask, 
   if (plan.cnt->overflow) return;
   uint32_t n_medium = plan.cnt->n_medium;
   if (n_medium > plan.cap_medium) n_medium = plan.cap_medium;
-  int64_t idx = (int64_t)blockIdx.x * 4 + wave;
+  int64_t idx = block * 4 + wave;
   if (idx >= (int64_t)n_medium * t.n_batch) return;
   int64_t b = 0;
   if (t.n_batch > 1) {
@@ -694,6 +699,11 @@ __global__ __launch_bounds__(256) void medium_rows_kernel(Tensors t, Mask mask, 
   if (g == 0) finish_row<Lay>(t, row, c, m, l, acc);
 }
 
+template <class Lay, class Mask, int UM = Lay::U_MEDIUM>
+__global__ __launch_bounds__(256) void medium_rows_kernel(Tensors t, Mask mask, Plan plan) {
+  medium_rows_body<Lay, Mask, UM>(t, mask, plan, (int64_t)blockIdx.x);
+}
+
 // The work list walked by an ordinary grid, one wavefront per item in list order, instead of by
 // segments_kernel's persistent wavefronts: the better of the two while K and V are not much
 // larger than the caches.  Three or four wavefronts per SIMD (127 / 139 registers at fp32 / bf16
@@ -704,8 +714,8 @@ __global__ __launch_bounds__(256) void medium_rows_kernel(Tensors t, Mask mask, 
 // - 33 / - 23 / - 13 / - 2 / + 1 / + 2 / + 3 %, bf16 d = 64 - 42 / - 38 / - 29 / - 19 / - 8 / 0 / + 3 %,
 // fp32 d = 128 - 14 / - 6 / + 1 / + 2 %, bf16 d = 128 - 28 / - 17 / - 8 / - 1 / + 2 %; eight heads of
 // the 128 K fp32 mask in one call + 5 %.  Taken when K + V of one problem are at most 48 MiB (96 MiB for rows of at most 128 bytes).
-template <class Lay, class Mask, int UM = Lay::U_MEDIUM>
-__global__ __launch_bounds__(256) void items_grid_kernel(Tensors t, Mask mask, Plan plan) {
+template <class Lay, class Mask, int UM>
+__device__ __forceinline__ void items_grid_body(const Tensors& t, const Mask& mask, const Plan& plan, int64_t block) {
   using T = typename Lay::elem;
   constexpr int NE = Lay::NE;
   constexpr int LPR = Lay::LPR;
@@ -716,7 +726,7 @@ __global__ __launch_bounds__(256) void items_grid_kernel(Tensors t, Mask mask, P
   if (plan.cnt->overflow) return;
   uint32_t n_items = plan.cnt->n_items;
   if (n_items > plan.cap_items) n_items = plan.cap_items;
-  int64_t idx = (int64_t)blockIdx.x * 4 + wave;
+  int64_t idx = block * 4 + wave;
   if (idx >= (int64_t)n_items * t.n_batch) return;
   int64_t b = 0;
   if (t.n_batch > 1) {
@@ -759,6 +769,33 @@ __global__ __launch_bounds__(256) void items_grid_kernel(Tensors t, Mask mask, P
       }
     }
   }
+}
+
+template <class Lay, class Mask, int UM = Lay::U_MEDIUM>
+__global__ __launch_bounds__(256) void items_grid_kernel(Tensors t, Mask mask, Plan plan) {
+  items_grid_body<Lay, Mask, UM>(t, mask, plan, (int64_t)blockIdx.x);
+}
+
+// The three row kernels of an explicit mask in one launch: the workgroups of the long rows' items
+// first, then those of the medium rows, then those of the short rows.  None of the three fills
+// the device alone at moderate sizes (a chain of dependent round trips per wavefront each), so
+// one after the other they add up to the sum of their latencies, side by side to the longest.
+// The Zipf mask at 8192 / 16384 / 32768 / 65536 tokens, three launches -> one: fp32 0.085 -> 0.060 /
+// 0.104 -> 0.086 / 0.179 -> 0.154 / 0.300 -> 0.291 ms, bf16 0.064 -> 0.044 / 0.074 -> 0.064 / 0.106 ->
+// 0.101 / 0.168 -> 0.172 ms (and 0.316 -> 0.334 at 131072: the short rows then run at the register
+// count of the long rows' kernel, and there are enough of them to notice); planned calls at 2048
+// ... 16384 tokens 0.048 -> 0.029, 0.050 -> 0.031, 0.067 -> 0.043, 0.086 -> 0.068 ms fp32.  Taken for
+// calls of up to kFusedRowsMax rows whose long rows are walked by an ordinary grid anyway.
+constexpr int64_t kFusedRowsMax = 32768;
+template <class Lay, class Mask>
+__global__ __launch_bounds__(256) void explicit_rows_kernel(Tensors t, Mask mask, Plan plan,
+                                                            uint32_t item_blocks, uint32_t medium_blocks) {
+  if (blockIdx.x < item_blocks)
+    items_grid_body<Lay, Mask, Lay::U_MEDIUM>(t, mask, plan, (int64_t)blockIdx.x);
+  else if (blockIdx.x < item_blocks + medium_blocks)
+    medium_rows_body<Lay, Mask, Lay::U_MEDIUM>(t, mask, plan, (int64_t)(blockIdx.x - item_blocks));
+  else
+    rows_body<Lay, Mask>(t, mask, plan, (int64_t)(blockIdx.x - item_blocks - medium_blocks));
 }
 
 // Small problems in one launch: one wavefront per row and problem (empty rows included), eight
@@ -1108,6 +1145,20 @@ int launch_engine(const Tensors& t, const Mask& mask, const EngineSizing& s, int
 
   const int64_t rows_per_wg = 4 * Lay::GROUPS;
   const int64_t grid1 = (t.n_q * t.n_batch + rows_per_wg - 1) / rows_per_wg;
+  if constexpr (Mask::kExplicit) {
+    if (has_long && s.items_on_grid && s.medium_batch == 0 && w.cap_medium > 0 &&
+        t.n_q * t.n_batch <= kFusedRowsMax) {
+      const int64_t gridm = ((int64_t)w.cap_medium * t.n_batch + 3) / 4;
+      const int64_t need = ((int64_t)w.cap_items * t.n_batch + 3) / 4;
+      if (need + gridm + grid1 < ((int64_t)1 << 31)) {
+        launch_maybe_timed(ev, explicit_rows_kernel<Lay, Mask>, dim3((unsigned)(need + gridm + grid1)), dim3(256),
+                           stream, t, mask, plan, (uint32_t)need, (uint32_t)gridm);
+        const int64_t grid3 = ((int64_t)w.cap_multi * t.n_batch + rows_per_wg - 1) / rows_per_wg;
+        hipLaunchKernelGGL((merge_kernel<Lay>), dim3((unsigned)grid3), dim3(256), 0, stream, t, plan);
+        return hipGetLastError() == hipSuccess ? 0 : 4;
+      }
+    }
+  }
   launch_maybe_timed(has_long ? KernelEvents{} : ev, rows_kernel<Lay, Mask>, dim3((unsigned)grid1), dim3(256),
                      stream, t, mask, plan);
   if (has_long && w.cap_medium > 0) {
