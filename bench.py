@@ -74,6 +74,7 @@ def load_library():
     lib.spfa_set_kernel_events.restype = None
     lib.spfa_explicit_inline_row_limit.restype = ctypes.c_int64
     lib.spfa_explicit_long_rows_on_grid.restype = ctypes.c_int
+    lib.spfa_explicit_one_launch_row_limit.restype = ctypes.c_int64
     lib.spfa_explicit_long_rows_on_grid.argtypes = [ctypes.c_int64, ctypes.c_int64, ctypes.c_int]
     return lib
 
@@ -93,7 +94,8 @@ def load_probe_library():
     return probe
 
 
-def make_workload(name, dtype, torch, syn, inline_limit=32, planned=False, heads=1, loop_heads=False, d_local=64):
+def make_workload(name, dtype, torch, syn, inline_limit=32, planned=False, heads=1, loop_heads=False, d_local=64,
+                  tokens=None):
     """Returns dict(call=fn(state) -> None, n, d, nnz, bytes_total, bytes_gathered, sample=fn())."""
     dev = "cuda"
     es = torch.tensor([], dtype=dtype).element_size()
@@ -101,6 +103,9 @@ def make_workload(name, dtype, torch, syn, inline_limit=32, planned=False, heads
     if name in ("csr_zipf", "csr_zipf_hbm", "csr_bernoulli", "coo_zipf", "coo_zipf_sorted"):
         if name in ("csr_zipf", "csr_zipf_hbm"):
             n, d = (131072 if name == "csr_zipf" else 1 << 22), 64
+            if tokens is not None and name == "csr_zipf":  # the headline generator at another size
+                n = tokens
+                w["desc"] = w["desc"].replace("N=131072", "N=%d" % n)
             ro, ci = syn.zipf_csr(n, 1.5, 1, 4096, device=dev, seed=0)
         elif name == "csr_bernoulli":
             n, d = 4096, 64
@@ -705,6 +710,8 @@ def main():
     ap.add_argument("--d", type=int, default=64, choices=[32, 64, 96, 128, 160, 192, 224, 256],
                     help="head dimension of the `local` workload (BASELINE config 2 has 64; the reference's own "
                          "check runs at 32)")
+    ap.add_argument("--tokens", type=int, default=None,
+                    help="csr_zipf only: the headline generator at N tokens instead of 131072 (2048 ... 1048576)")
     ap.add_argument("--heads", type=int, default=1,
                     help="csr_* and local workloads: this many independent problems sharing the mask, stacked "
                          "[heads, n, d] (local: of N=4096 tokens each)")
@@ -743,10 +750,12 @@ def main():
     lib = load_library()
     if a.planned and not (a.workload.startswith(("csr", "coo")) or (a.workload == "bigbird" and a.backward)):
         sys.exit("bench.py: --planned applies to the explicit-mask workloads (csr_*, coo_*; bigbird with --backward)")
+    if a.tokens is not None and (a.workload != "csr_zipf" or not 2048 <= a.tokens <= 1 << 20):
+        sys.exit("bench.py: --tokens applies to the csr_zipf workload, 2048 ... 1048576")
     if a.heads > 1 and not (a.workload.startswith("csr") or a.workload == "local"):
         sys.exit("bench.py: --heads applies to the csr_* and local workloads")
     w = make_workload(a.workload, dtype, torch, syn, int(lib.spfa_explicit_inline_row_limit()), a.planned,
-                      max(1, a.heads), a.loop_heads, a.d)
+                      max(1, a.heads), a.loop_heads, a.d, a.tokens)
     n, d, nnz = w["n"], w["d"], w["nnz"]
 
     n_states = a.steps + a.warmup
@@ -857,6 +866,8 @@ def main():
         # is what the same gather without arithmetic sustains at this working set (measured here).
         on_grid = lib.spfa_explicit_long_rows_on_grid(int(w["k"].shape[-2]), int(d), {"f32": 0, "f16": 1, "bf16": 2}[a.dtype])
         kernel_name = "items_grid_kernel" if on_grid else "segments_kernel"
+        if on_grid and explicit and w["n"] * w.get("heads", 1) <= lib.spfa_explicit_one_launch_row_limit():
+            w = dict(w, whole_call=True)  # (the row kernels of such a call are one launch)
         if w.get("whole_call") or w["kernel_nnz"] == 0:
             # no row is long enough for the segment kernel, or several kernels share the call: the
             # whole call stands in, with the call's algorithmic bytes
@@ -935,7 +946,8 @@ def main():
                      "kernel_rows": w["kernel_rows"], "call_algorithmic_bytes": w["bytes_total"],
                      "call_gathered_bytes": w["bytes_gathered"]})
     out = {
-        "metric": "masked-attn GFLOP/s (nnz-counted) + effective HBM GB/s, CSR N=128K d=64 fp32",
+        "metric": "masked-attn GFLOP/s (nnz-counted) + effective HBM GB/s, CSR N=128K d=64 fp32" if a.tokens is None else
+                  "masked-attn GFLOP/s (nnz-counted) + effective HBM GB/s, CSR N=%d d=64" % a.tokens,
         "value": flops / (ms_per_step * 1e-3) / 1e9,
         "unit": "GFLOP/s",
         "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": ms_per_step,

@@ -405,6 +405,8 @@ int spfa_explicit_long_rows_on_grid(int64_t n_k, int64_t d, int dtype) {
   return explicit_items_on_grid(n_k, d, dtype) ? 1 : 0;
 }
 
+int64_t spfa_explicit_one_launch_row_limit(void) { return kFusedRowsMax; }
+
 int spfa_device_status(int reset) {
   uint32_t* word = device_status_word();
   if (word == nullptr) return -1;

@@ -124,6 +124,10 @@ int64_t spfa_explicit_inline_row_limit(void);
  * it times. */
 int spfa_explicit_long_rows_on_grid(int64_t n_k, int64_t d, int dtype);
 
+/* Such a call of at most this many rows (over all problems) runs its three row kernels - long
+ * rows' items, medium rows, short rows - as one launch, so no single kernel of it can be timed. */
+int64_t spfa_explicit_one_launch_row_limit(void);
+
 /* CSR: row i attends col_ind[row_off[i] .. row_off[i+1]).  row_off has n_q+1 entries of
  * row_off_bytes (4 or 8) bytes each, col_ind has nnz 4-byte entries; signed and unsigned
  * index tensors are bit-identical in range.  The reference's value vector is never read
