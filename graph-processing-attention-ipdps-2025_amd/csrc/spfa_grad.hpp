@@ -297,12 +297,12 @@ struct GradOwner {
 };
 
 template <class Lay, class Mask, bool KEYS>
-__global__ __launch_bounds__(kGradWaves* kWave) void grad_rows_kernel(GradArgs g, Mask mask) {
+__device__ __forceinline__ void grad_rows_body(const GradArgs& g, const Mask& mask, int64_t block) {
   constexpr int NE = Lay::NE;
   const int lane = threadIdx.x & (kWave - 1);
   const int c = lane % Lay::LPR;
   const int64_t n_own = KEYS ? g.n_k : g.n_q;
-  const int64_t r = (int64_t)blockIdx.x * kGradWaves + (threadIdx.x >> 6);
+  const int64_t r = block * kGradWaves + (threadIdx.x >> 6);
   if (r >= n_own * g.n_batch) return;
   GradOwner<Lay, KEYS> o;
   o.load(g, r, c);
@@ -359,6 +359,27 @@ __global__ __launch_bounds__(kGradWaves* kWave) void grad_rows_kernel(GradArgs g
       Lay::store_f32(o.out2, c, g.d, cur);
     }
   }
+}
+
+template <class Lay, class Mask, bool KEYS>
+__global__ __launch_bounds__(kGradWaves* kWave) void grad_rows_kernel(GradArgs g, Mask mask) {
+  grad_rows_body<Lay, Mask, KEYS>(g, mask, (int64_t)blockIdx.x);
+}
+
+// The owners of both passes in one launch, query rows first: the passes do not depend on each
+// other (one adds to dQ, the other to dK and dV), and in a call of a few ten thousand owners
+// neither fills the device - each wavefront is a chain of dependent round trips -, so one after
+// the other they take the sum of their latencies, side by side the longer of the two (the Zipf
+// mask at 16384 tokens: 60 + 53 us).  In larger calls the query rows would pay for running at the
+// key pass's register count.
+constexpr int64_t kGradBothOwnersMax = 65536;
+template <class Lay, class RowMask, class ColMask>
+__global__ __launch_bounds__(kGradWaves* kWave) void grad_rows_both_kernel(GradArgs g, RowMask rows, ColMask cols,
+                                                                           uint32_t query_blocks) {
+  if (blockIdx.x < query_blocks)
+    grad_rows_body<Lay, RowMask, false>(g, rows, (int64_t)blockIdx.x);
+  else
+    grad_rows_body<Lay, ColMask, true>(g, cols, (int64_t)(blockIdx.x - query_blocks));
 }
 
 // Candidates in flight per lane group in grad_segments_kernel: the forward segment kernel's, as
@@ -439,8 +460,13 @@ int launch_grad(const Tensors& t, const GradArgs& g, const RowMask& rows, const 
   hipLaunchKernelGGL(grad_reset_kernel, dim3(1), dim3(64), 0, stream, g);
   hipLaunchKernelGGL((grad_prologue_kernel<T>), dim3((unsigned)((nq + 15) / 16)), dim3(256), 0, stream,
                      t, g);
-  hipLaunchKernelGGL((grad_rows_kernel<Lay, RowMask, false>),
-                     dim3((unsigned)((nq + kGradWaves - 1) / kGradWaves)), block, 0, stream, g, rows);
+  const int64_t q_blocks = (nq + kGradWaves - 1) / kGradWaves, k_blocks = (nk + kGradWaves - 1) / kGradWaves;
+  const bool both = nq + nk <= kGradBothOwnersMax;
+  if (both)
+    hipLaunchKernelGGL((grad_rows_both_kernel<Lay, RowMask, ColMask>), dim3((unsigned)(q_blocks + k_blocks)), block,
+                       0, stream, g, rows, cols, (uint32_t)q_blocks);
+  else
+    hipLaunchKernelGGL((grad_rows_kernel<Lay, RowMask, false>), dim3((unsigned)q_blocks), block, 0, stream, g, rows);
   if (lists) {
     hipLaunchKernelGGL(order_kernel, grid_order, dim3(256), 0, stream, grad_plan(g, 0));
     if (g.items_on_grid)
@@ -450,8 +476,8 @@ int launch_grad(const Tensors& t, const GradArgs& g, const RowMask& rows, const 
       hipLaunchKernelGGL((grad_segments_kernel<Lay, RowMask, false>), dim3((unsigned)grid_seg), dim3(256), 0,
                          stream, g, rows);
   }
-  hipLaunchKernelGGL((grad_rows_kernel<Lay, ColMask, true>),
-                     dim3((unsigned)((nk + kGradWaves - 1) / kGradWaves)), block, 0, stream, g, cols);
+  if (!both)
+    hipLaunchKernelGGL((grad_rows_kernel<Lay, ColMask, true>), dim3((unsigned)k_blocks), block, 0, stream, g, cols);
   if (lists) {
     hipLaunchKernelGGL(order_kernel, grid_order, dim3(256), 0, stream, grad_plan(g, 1));
     if (g.items_on_grid)
