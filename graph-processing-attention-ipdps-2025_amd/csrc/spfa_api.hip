@@ -961,20 +961,29 @@ constexpr int64_t kGradOwnImplicit = kGradSegment;
 struct ItemsBound {
   int64_t items;
   int64_t own_max;
+  int64_t seg;
 };
+// Segments of an explicit mask: half as long below 32 M entries, where a call is short enough for
+// the length of one wavefront's walk to show (whole gradient call of the Zipf mask at 8192 /
+// 16384 / 65536 / 131072 tokens with 1024 -> 512: 0.275 -> 0.237, 0.307 -> 0.262, 0.715 -> 0.672,
+// 1.332 -> 1.324 ms fp32; 256: 0.219, 0.263, 0.656, 1.459; the COO mask of 50 M entries 9.21 -> 9.35
+// -> 9.64 ms).
+constexpr int64_t kGradSegmentShort = 512;
+int64_t explicit_grad_segment(int64_t nnz) { return nnz < ((int64_t)1 << 25) ? kGradSegmentShort : kGradSegment; }
 int64_t grad_items_of(int64_t deg, int64_t own_max) {
   return deg > own_max ? (deg + kGradSegment - 1) / kGradSegment : 0;
 }
 ItemsBound explicit_items_bound(int64_t nnz) {
   // every owner of more than own_max candidates: deg / seg + 1 items at most, nnz / (own_max + 1) such owners
-  return ItemsBound{nnz / kGradSegment + nnz / (kGradOwnExplicit + 1), kGradOwnExplicit};
+  const int64_t seg = explicit_grad_segment(nnz);
+  return ItemsBound{nnz / seg + nnz / (kGradOwnExplicit + 1), kGradOwnExplicit, seg};
 }
 ItemsBound uniform_items_bound(int64_t n_rows, int64_t max_deg) {
-  return ItemsBound{n_rows * grad_items_of(max_deg, kGradOwnImplicit), kGradOwnImplicit};
+  return ItemsBound{n_rows * grad_items_of(max_deg, kGradOwnImplicit), kGradOwnImplicit, kGradSegment};
 }
 ItemsBound global_items_bound(int64_t n, int64_t n_globals) {
   return ItemsBound{n_globals * grad_items_of(n, kGradOwnImplicit) + n * grad_items_of(n_globals, kGradOwnImplicit),
-                    kGradOwnImplicit};
+                    kGradOwnImplicit, kGradSegment};
 }
 
 // Workspace of a gradient call: lse and delta of every query row (apart and side by side), the counters and the
@@ -983,6 +992,7 @@ struct GradLayout {
   size_t off_lse, off_delta, off_stat, off_cnt, off_phases, off_items, off_mask, total;
   uint32_t cap_items;
   int32_t own_max;
+  int32_t seg;
   bool ok;
 };
 
@@ -993,6 +1003,7 @@ GradLayout grad_layout(int64_t n_q, int64_t n_batch, ItemsBound bound, size_t ma
   g.ok = cap < ((int64_t)1 << 31);
   g.cap_items = (uint32_t)(g.ok ? cap : 1);
   g.own_max = (int32_t)bound.own_max;
+  g.seg = (int32_t)bound.seg;
   size_t off = 0;
   g.off_lse = off;    off = align_up(off + (size_t)(n_q * b) * 4, 256);
   g.off_delta = off;  off = align_up(off + (size_t)(n_q * b) * 4, 256);
@@ -1038,7 +1049,7 @@ GradArgs make_grad_args(const spfa_problem_t* p, const spfa_grads_t* g, const Gr
   a.n_k = p->n_k;
   a.n_batch = batch_of(p);
   a.d = (int32_t)p->d;
-  a.seg = (int32_t)kGradSegment;
+  a.seg = lay.seg;
   a.own_max = lay.own_max;
   const size_t list_bytes = align_up((size_t)lay.cap_items * sizeof(Item), 256);
   for (int pass = 0; pass < 2; pass++) {
