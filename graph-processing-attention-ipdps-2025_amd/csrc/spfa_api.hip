@@ -89,13 +89,16 @@ bool explicit_items_on_grid(int64_t n_k, int64_t d, int dtype) {
 // ... and its batch size in the medium-row kernel (see there): smaller while K and V are not much
 // larger than the caches and the rows are long enough on average for the wavefronts to fall in
 // step (measured on uniform rows of sorted columns; the Zipf headline - 97 entries per row on
-// average, most of them in few long rows - loses 5 % of that kernel with 4).  CSR calls only:
+// average, most of them in few long rows - loses 5 % of that kernel with 4, which does not show
+// in the call; 64 heads of the 2 % Bernoulli mask of 4096 tokens, rows of ~83: 0.595 -> 0.510 ms
+// fp32, 0.440 -> 0.396 ms bf16 with 2).  From 64 entries per row on average.  CSR calls only:
 // the rows that the COO pre-pass builds keep their entries in the order they came in, and on
 // unsorted columns the smaller batches lose up to 10 %.
 int explicit_medium_batch(const spfa_problem_t* p, int64_t nnz) {
-  if (p->n_q <= 0 || nnz / p->n_q < 128) return 0;
+  if (p->n_q <= 0 || nnz / p->n_q < 64) return 0;
   const int64_t es = p->dtype == SPFA_DTYPE_F32 ? 4 : p->dtype == SPFA_DTYPE_F64 ? 8 : 2;
-  const int64_t kv = 2 * p->n_k * p->d * es * (p->n_batch > 1 ? p->n_batch : 1);
+  // (K and V of one problem: the problems of a batch are walked one after the other)
+  const int64_t kv = 2 * p->n_k * p->d * es;
   return kv <= kCachedKvBytes ? 2 : kv <= 4 * kCachedKvBytes ? 4 : 0;
 }
 
