@@ -130,7 +130,10 @@ def _source_loop_depth(kname: str) -> int:
     if "20explicit_rows_kernelI" in kname:
         # the item, medium-row and short-row kernels in one launch: the deepest nest of the three
         # (the first two with the layout's own batch size)
+        # (its third template argument is the medium rows' batch size; the items keep the layout's)
+        as_items = re.sub(r"MaskELi\d+EEEv", "MaskEEEv", kname).replace("20explicit_rows_kernelI", "18medium_rows_kernelI")
         return max(_source_loop_depth(kname.replace("20explicit_rows_kernelI", "18medium_rows_kernelI")),
+                   _source_loop_depth(as_items),
                    _source_loop_depth(kname.replace("20explicit_rows_kernelI", "11rows_kernelI")))
     med = "18medium_rows_kernelI" in kname or "17items_grid_kernelI" in kname or whole
     if "15segments_kernelI" not in kname and "11rows_kernelI" not in kname and not med:

@@ -91,7 +91,8 @@ bool explicit_items_on_grid(int64_t n_k, int64_t d, int dtype) {
 // step (measured on uniform rows of sorted columns; the Zipf headline - 97 entries per row on
 // average, most of them in few long rows - loses 5 % of that kernel with 4, which does not show
 // in the call; 64 heads of the 2 % Bernoulli mask of 4096 tokens, rows of ~83: 0.595 -> 0.510 ms
-// fp32, 0.440 -> 0.396 ms bf16 with 2).  From 64 entries per row on average.  CSR calls only:
+// fp32, 0.440 -> 0.396 ms bf16 with 2).  From 128 entries per row on average; from 64 when K and V
+// of a problem fit an L2.  CSR calls only:
 // the rows that the COO pre-pass builds keep their entries in the order they came in, and on
 // unsorted columns the smaller batches lose up to 10 %.
 int explicit_medium_batch(const spfa_problem_t* p, int64_t nnz) {
@@ -99,6 +100,9 @@ int explicit_medium_batch(const spfa_problem_t* p, int64_t nnz) {
   const int64_t es = p->dtype == SPFA_DTYPE_F32 ? 4 : p->dtype == SPFA_DTYPE_F64 ? 8 : 2;
   // (K and V of one problem: the problems of a batch are walked one after the other)
   const int64_t kv = 2 * p->n_k * p->d * es;
+  // 64 ... 127 entries per row: only while K and V fit an L2 (the Zipf mask, ~100 per row, loses
+  // 13 % at 16384 tokens - 8 MiB - with 2 or 4, and nothing at 8192)
+  if (nnz / p->n_q < 128) return kv <= ((int64_t)4 << 20) ? 2 : 0;
   return kv <= kCachedKvBytes ? 2 : kv <= 4 * kCachedKvBytes ? 4 : 0;
 }
 

@@ -787,13 +787,13 @@ __global__ __launch_bounds__(256) void items_grid_kernel(Tensors t, Mask mask, P
 // ... 16384 tokens 0.048 -> 0.029, 0.050 -> 0.031, 0.067 -> 0.043, 0.086 -> 0.068 ms fp32.  Taken for
 // calls of up to kFusedRowsMax rows whose long rows are walked by an ordinary grid anyway.
 constexpr int64_t kFusedRowsMax = 32768;
-template <class Lay, class Mask>
+template <class Lay, class Mask, int UM = Lay::U_MEDIUM>  // (UM: the medium rows' batch size)
 __global__ __launch_bounds__(256) void explicit_rows_kernel(Tensors t, Mask mask, Plan plan,
                                                             uint32_t item_blocks, uint32_t medium_blocks) {
   if (blockIdx.x < item_blocks)
     items_grid_body<Lay, Mask, Lay::U_MEDIUM>(t, mask, plan, (int64_t)blockIdx.x);
   else if (blockIdx.x < item_blocks + medium_blocks)
-    medium_rows_body<Lay, Mask, Lay::U_MEDIUM>(t, mask, plan, (int64_t)(blockIdx.x - item_blocks));
+    medium_rows_body<Lay, Mask, UM>(t, mask, plan, (int64_t)(blockIdx.x - item_blocks));
   else
     rows_body<Lay, Mask>(t, mask, plan, (int64_t)(blockIdx.x - item_blocks - medium_blocks));
 }
@@ -1146,13 +1146,20 @@ int launch_engine(const Tensors& t, const Mask& mask, const EngineSizing& s, int
   const int64_t rows_per_wg = 4 * Lay::GROUPS;
   const int64_t grid1 = (t.n_q * t.n_batch + rows_per_wg - 1) / rows_per_wg;
   if constexpr (Mask::kExplicit) {
-    if (has_long && s.items_on_grid && s.medium_batch == 0 && w.cap_medium > 0 &&
-        t.n_q * t.n_batch <= kFusedRowsMax) {
+    if (has_long && s.items_on_grid && w.cap_medium > 0 && t.n_q * t.n_batch <= kFusedRowsMax) {
       const int64_t gridm = ((int64_t)w.cap_medium * t.n_batch + 3) / 4;
       const int64_t need = ((int64_t)w.cap_items * t.n_batch + 3) / 4;
       if (need + gridm + grid1 < ((int64_t)1 << 31)) {
-        launch_maybe_timed(ev, explicit_rows_kernel<Lay, Mask>, dim3((unsigned)(need + gridm + grid1)), dim3(256),
-                           stream, t, mask, plan, (uint32_t)need, (uint32_t)gridm);
+        const dim3 grid_all((unsigned)(need + gridm + grid1));
+        if (s.medium_batch == 2 && Lay::U_MEDIUM > 2)
+          launch_maybe_timed(ev, explicit_rows_kernel<Lay, Mask, (Lay::U_MEDIUM > 2 ? 2 : Lay::U_MEDIUM)>, grid_all,
+                             dim3(256), stream, t, mask, plan, (uint32_t)need, (uint32_t)gridm);
+        else if (s.medium_batch == 4 && Lay::U_MEDIUM > 4)
+          launch_maybe_timed(ev, explicit_rows_kernel<Lay, Mask, (Lay::U_MEDIUM > 4 ? 4 : Lay::U_MEDIUM)>, grid_all,
+                             dim3(256), stream, t, mask, plan, (uint32_t)need, (uint32_t)gridm);
+        else
+          launch_maybe_timed(ev, explicit_rows_kernel<Lay, Mask>, grid_all, dim3(256), stream, t, mask, plan,
+                             (uint32_t)need, (uint32_t)gridm);
         const int64_t grid3 = ((int64_t)w.cap_multi * t.n_batch + rows_per_wg - 1) / rows_per_wg;
         hipLaunchKernelGGL((merge_kernel<Lay>), dim3((unsigned)grid3), dim3(256), 0, stream, t, plan);
         return hipGetLastError() == hipSuccess ? 0 : 4;
