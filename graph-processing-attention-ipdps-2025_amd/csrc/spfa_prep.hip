@@ -744,69 +744,117 @@ __global__ __launch_bounds__(kPartRowsThreads, 4) void coo_part_rows_kernel(
   else place_all(std::integral_constant<int, 0>{});
 }
 
-// (row, column) of every entry of a CSR mask.  A wavefront takes `rpw` (16 or 64) consecutive
-// rows, one pair of offsets per lane; the rows' entries are one contiguous range, which the
-// wavefront walks 64 entries at a time, every lane finding the row of its entry by a binary search
-// among the wavefront's row ends (six cross-lane reads).  (A wavefront per row spends most of
-// its time on the empty rows of a mask that has many: 360 us for 50 M entries in 1 M rows.)
-// Row ranges are held to [0, nnz) as in CsrMask::row; entries before the first row's range or
-// after the last row's belong to no row and get a column that the bucketing drops.  Offsets that
-// are not in ascending order give entries of the wrong row or none, never a store outside
-// [0, nnz).
+// Row offset `r` of a CSR mask held to [0, nnz] (nnz < 2^32).
+__device__ __forceinline__ uint32_t held_offset(const void* row_off, int64_t r, int off64, int64_t nnz) {
+  int64_t v = load_index(row_off, r, off64);
+  v = v < 0 ? 0 : v;
+  return (uint32_t)(v > nnz ? nnz : v);
+}
+
+// How many of the offsets [lo, hi) are at or below x, plus lo, for offsets in ascending order
+// (all of those before lo are taken to be at or below x).  The wavefront searches together: every
+// lane looks at one of 64 evenly spaced offsets per round, so 2^17 offsets take three dependent
+// loads where a bisection takes seventeen.  Offsets in any other order give some value in
+// [lo, hi].
+__device__ __forceinline__ int64_t wave_offsets_at_or_below(const void* row_off, int off64, int64_t nnz,
+                                                            int64_t lo, int64_t hi, uint32_t x, int lane) {
+  while (lo < hi) {
+    const int64_t step = (hi - lo + kWave - 1) / kWave;
+    const int64_t r = lo + (int64_t)lane * step;
+    const bool below = r < hi && held_offset(row_off, r, off64, nnz) <= x;
+    const uint64_t not_below = ~__ballot(below);
+    const int k = not_below == 0 ? kWave : __builtin_ctzll(not_below);
+    if (k == 0) break;
+    const int64_t next_hi = lo + (int64_t)k * step;
+    lo += (int64_t)(k - 1) * step + 1;
+    hi = next_hi < hi ? next_hi : hi;
+  }
+  return lo;
+}
+
+constexpr int kEntryListInFlight = 8;
+constexpr int kEntryListChunk = 4 * kEntryListInFlight * kWave;
+
+// (row, column) of every entry of a CSR mask.  A wavefront takes 2048 consecutive ENTRIES, finds
+// how many row offsets lie at or below its first entry (the search above) and then holds 64
+// consecutive offsets at a time, one per lane: an entry below the last of them lies in the row
+// given by the number of held offsets at or below it (six cross-lane reads).  When all the held
+// offsets are passed the window moves on by 63, or, over a long run of empty rows, by another
+// search.  (Sharing out rows instead - 16 per wavefront - left the wavefronts that met a few rows
+// of 4096 entries running long after the rest on a power-law mask; a wavefront per row spends most
+// of its time on the empty rows of a mask that has many.)
+// Offsets are held to [0, nnz] as in CsrMask::row; entries before the first offset or at and after
+// the last belong to no row and get a column that the bucketing drops.  Offsets that are not in
+// ascending order give entries of the wrong row or none; every entry of [0, nnz) is written once
+// and nothing outside.
 __global__ __launch_bounds__(256) void csr_entry_list_kernel(const void* row_off, int off64,
                                                              const uint32_t* __restrict__ cols,
                                                              const uint32_t* __restrict__ alt_cols,
                                                              const uint32_t* use_alt, int64_t n_rows,
-                                                             int64_t nnz, int rpw,
-                                                             uint32_t* __restrict__ rows_out,
+                                                             int64_t nnz, uint32_t* __restrict__ rows_out,
                                                              uint32_t* __restrict__ cols_out) {
   const int lane = threadIdx.x & (kWave - 1);
   const uint32_t* __restrict__ cp = (use_alt != nullptr && *use_alt != 0u) ? alt_cols : cols;
-  const int64_t r0 = ((int64_t)blockIdx.x * 4 + (threadIdx.x >> 6)) * rpw;
-  if (r0 >= n_rows) return;
-  const int n_here = n_rows - r0 < rpw ? (int)(n_rows - r0) : rpw;
-  // lane l < n_here: the range of row r0 + l; the other lanes: an empty range at the end
-  const int64_t r = r0 + (lane < n_here ? lane : n_here - 1);
-  int64_t a = load_index(row_off, r, off64);
-  int64_t b = load_index(row_off, r + 1, off64);
-  if (b > nnz) b = nnz;
-  if (a < 0) a = 0;
-  if (a > b) a = b;
-  if (lane >= n_here) a = b;
+  const int64_t begin = ((int64_t)blockIdx.x * 4 + (threadIdx.x >> 6)) * kEntryListChunk;
+  if (begin >= nnz) return;
   // (nnz < 2^32: the offsets of the bucketed mask are 32 bits wide)
-  const uint32_t end32 = (uint32_t)b;
-  const uint32_t first = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)a, 0);
-  const uint32_t last = (uint32_t)__builtin_amdgcn_readlane((int)end32, kWave - 1);
-  // (eight loads in flight per lane: one load per trip makes a row of 4096 entries a chain of 64
-  // memory round trips, which was the whole of the kernel's time on a power-law mask)
-  constexpr int kInFlight = 8;
-  for (uint32_t e0 = first; e0 < last; e0 += kInFlight * kWave) {
-    uint32_t col[kInFlight];
-#pragma unroll
-    for (int u = 0; u < kInFlight; u++) {
-      const uint32_t e = e0 + u * kWave + lane;
-      col[u] = e < last ? cp[e] : 0u;
-    }
-#pragma unroll
-    for (int u = 0; u < kInFlight; u++) {
-      const uint32_t e = e0 + u * kWave + lane;
-      // number of rows of this wavefront that end at or before e
-      int lo = 0;
-#pragma unroll
-      for (int step = kWave / 2; step >= 1; step >>= 1) {
-        const uint32_t end_v = (uint32_t)__builtin_amdgcn_ds_bpermute((lo + step - 1) << 2, (int)end32);
-        if (end_v <= e) lo += step;
-      }
-      if (e < last) {
-        rows_out[e] = (uint32_t)(r0 + lo);
-        cols_out[e] = col[u];
+  const uint32_t end = (uint32_t)(nnz - begin < kEntryListChunk ? nnz : begin + kEntryListChunk);
+  const int64_t n_off = n_rows + 1;
+  uint32_t pos = (uint32_t)begin;
+  // offsets [0, c) are at or below pos
+  int64_t c = wave_offsets_at_or_below(row_off, off64, nnz, 0, n_off, pos, lane);
+  // lane l: offset c + l; past the last offset: one that no entry reaches
+  auto hold = [&](int64_t first) -> uint32_t {
+    return first + lane < n_off ? held_offset(row_off, first + lane, off64, nnz) : 0xffffffffu;
+  };
+  uint32_t held = hold(c);
+  while (pos < end) {
+    uint32_t held_last = (uint32_t)__builtin_amdgcn_readlane((int)held, kWave - 1);
+    if (held_last <= pos) {
+      const int64_t from = c + kWave < n_off ? c + kWave : n_off;
+      c = wave_offsets_at_or_below(row_off, off64, nnz, from, n_off, pos, lane);
+      held = hold(c);
+      held_last = (uint32_t)__builtin_amdgcn_readlane((int)held, kWave - 1);
+      if (held_last <= pos) {  // offsets out of order: go on window by window
+        c = c + kWave < n_off ? c + kWave : n_off;
+        held = hold(c);
+        continue;
       }
     }
+    // (the next window's offsets are on their way while this one's entries are written)
+    const uint32_t held_next = hold(c + kWave - 1);
+    const uint32_t stop = held_last < end ? held_last : end;
+    // (eight loads in flight per lane: one load per trip makes a row of 4096 entries a chain of 64
+    // memory round trips)
+    for (uint32_t e0 = pos; e0 < stop; e0 += kEntryListInFlight * kWave) {
+      uint32_t col[kEntryListInFlight];
+#pragma unroll
+      for (int u = 0; u < kEntryListInFlight; u++) {
+        const uint32_t e = e0 + u * kWave + lane;
+        col[u] = e < stop ? cp[e] : 0u;
+      }
+#pragma unroll
+      for (int u = 0; u < kEntryListInFlight; u++) {
+        const uint32_t e = e0 + u * kWave + lane;
+        // number of held offsets at or below e (fewer than 64 for e < stop)
+        int lo = 0;
+#pragma unroll
+        for (int step = kWave / 2; step >= 1; step >>= 1) {
+          const uint32_t v = (uint32_t)__builtin_amdgcn_ds_bpermute((lo + step - 1) << 2, (int)held);
+          if (v <= e) lo += step;
+        }
+        if (e < stop) {
+          const int64_t row = c + lo - 1;
+          const bool in_a_row = row >= 0 && row < n_rows;
+          rows_out[e] = in_a_row ? (uint32_t)row : 0u;
+          cols_out[e] = in_a_row ? col[u] : 0xffffffffu;
+        }
+      }
+    }
+    pos = stop;
+    c += kWave - 1;
+    held = held_next;
   }
-  if (r0 == 0)
-    for (uint32_t e = lane; e < first; e += kWave) cols_out[e] = 0xffffffffu;
-  if (r0 + rpw >= n_rows)
-    for (int64_t e = (int64_t)last + lane; e < nnz; e += kWave) cols_out[e] = 0xffffffffu;
 }
 
 __global__ void coo_csr_export_kernel(const uint32_t* row_off, const uint32_t* bucketed,
@@ -982,11 +1030,10 @@ int coo_to_csr(const void* row_ind, int row_wide, const uint32_t* col_ind, int64
 int csr_entry_list(const void* row_off, int off64, const uint32_t* cols, const uint32_t* alt_cols,
                    const uint32_t* use_alt, int64_t n_rows, int64_t nnz, uint32_t* rows_out,
                    uint32_t* cols_out, hipStream_t stream) {
-  if (n_rows <= 0) return 0;
-  // (64 rows per wavefront when that still leaves a few wavefronts for every SIMD)
-  const int rpw = n_rows >= ((int64_t)1 << 19) ? kWave : 16;
-  hipLaunchKernelGGL(csr_entry_list_kernel, dim3((unsigned)((n_rows + 4 * rpw - 1) / (4 * rpw))), dim3(256), 0,
-                     stream, row_off, off64, cols, alt_cols, use_alt, n_rows, nnz, rpw, rows_out, cols_out);
+  if (n_rows <= 0 || nnz <= 0) return 0;
+  const int64_t per_block = 4 * (int64_t)kEntryListChunk;
+  hipLaunchKernelGGL(csr_entry_list_kernel, dim3((unsigned)((nnz + per_block - 1) / per_block)), dim3(256), 0,
+                     stream, row_off, off64, cols, alt_cols, use_alt, n_rows, nnz, rows_out, cols_out);
   return hipGetLastError() == hipSuccess ? 0 : 4;
 }
 

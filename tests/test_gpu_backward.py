@@ -309,6 +309,35 @@ def test_transposed_mask_is_exact_and_reusable(mods):
     assert z_ro.cpu().tolist() == [0] * 7 and z_ci.numel() == 0
 
 
+def test_transposition_of_masks_with_runs_of_empty_and_of_one_entry_rows(mods):
+    """The transposition walks the entries in fixed chunks and finds their rows from windows of 64
+    row offsets: rows longer than a chunk, runs of more than 64 and more than 128 empty rows (also
+    first and last), runs of rows of one entry, and a number of entries that is no multiple of the
+    chunk, against a CPU transposition."""
+    n_k = 5000
+    rng = np.random.default_rng(83)
+    deg = np.concatenate([
+        np.zeros(70, np.int64), [3], np.ones(150, np.int64), [4100], np.zeros(200, np.int64),
+        rng.integers(0, 3, 300), [2048, 2049, 1], np.zeros(64, np.int64), [5], np.zeros(63, np.int64),
+        rng.integers(0, 40, 200), np.ones(1000, np.int64), [0, 0, 2500], np.zeros(130, np.int64)])
+    n = len(deg)
+    ro = np.concatenate([[0], np.cumsum(deg)])
+    ci = np.concatenate([np.sort(rng.choice(n_k, int(g), replace=False)) for g in deg]).astype(np.int64)
+    rows = np.repeat(np.arange(n), deg)
+    order = np.lexsort((rows, ci))
+    t_ro_ref = np.concatenate([[0], np.cumsum(np.bincount(ci, minlength=n_k))])
+    t_ci_ref = rows[order]
+    for off_dtype in (torch.int64, torch.int32):
+        t_ro, t_ci = mods["spfa_csr"].transpose(torch.as_tensor(ro).to(off_dtype).to(DEV),
+                                                torch.as_tensor(ci).to(torch.int32).to(DEV), n_k)
+        torch.cuda.synchronize()
+        t_ro, t_ci = t_ro.cpu().numpy().astype(np.int64), t_ci.cpu().numpy().astype(np.int64)
+        assert np.array_equal(t_ro, t_ro_ref)
+        # (the rows of a column come in no particular order)
+        key = np.repeat(np.arange(n_k), np.diff(t_ro))
+        assert np.array_equal(t_ci[np.lexsort((t_ci, key))], t_ci_ref)
+
+
 def test_batch_of_heads_shares_the_mask(mods):
     n, d, lead = 200, 64, (2, 3)
     q, k, v, d_out = _problem(n, d, torch.float32, 31, lead=lead)
