@@ -86,6 +86,18 @@ bool explicit_items_on_grid(int64_t n_k, int64_t d, int dtype) {
   return 2 * n_k * d * es <= (d * es <= 128 ? kItemsGridKvBytesShortRows : kItemsGridKvBytes);
 }
 
+// ... and whether the list is walked as plan_kernel appended it.  The order it is handed out in
+// otherwise keeps the wavefronts at work to one part of K and V at a time, which is worth nothing
+// while K and V of a problem fit the L2s anyway; order_kernel's launch then only adds its 4 - 5 us
+// to a short call (Zipf mask, d = 64, fp32 / bf16: 8192 tokens 0.063 -> 0.058 / 0.050 -> 0.043 ms,
+// 16384 tokens 0.088 -> 0.084 / 0.072 -> 0.065, 32768 tokens 0.154 -> 0.170 / 0.105 -> 0.103: K + V
+// of 4, 8 and 16 MiB in fp32).
+constexpr int64_t kItemsAsListedKvBytes = (int64_t)8 << 20;
+bool explicit_items_as_listed(int64_t n_k, int64_t d, int dtype) {
+  const int64_t es = dtype == SPFA_DTYPE_F32 ? 4 : dtype == SPFA_DTYPE_F64 ? 8 : 2;
+  return 2 * n_k * d * es <= kItemsAsListedKvBytes;
+}
+
 // ... and its batch size in the medium-row kernel (see there): smaller while K and V are not much
 // larger than the caches and the rows are long enough on average for the wavefronts to fall in
 // step (measured on uniform rows of sorted columns; the Zipf headline - 97 entries per row on
@@ -490,6 +502,7 @@ int spfa_csr_forward(const spfa_problem_t* p, const void* row_off, int row_off_b
   }
   EngineSizing s = size_csr(p->n_q, nnz);
   s.items_on_grid = explicit_items_on_grid(p->n_k, p->d, p->dtype);
+  s.items_as_listed = explicit_items_as_listed(p->n_k, p->d, p->dtype);
   s.medium_batch = explicit_medium_batch(p, nnz);
   if (!batch_fits_engine(s, p)) {
     for (int64_t b = 0; b < batch_of(p); b++) {
@@ -541,6 +554,7 @@ int spfa_csr_forward_planned(const spfa_problem_t* p, const void* row_off, int r
   }
   EngineSizing s = size_csr(p->n_q, nnz);
   s.items_on_grid = explicit_items_on_grid(p->n_k, p->d, p->dtype);
+  s.items_as_listed = explicit_items_as_listed(p->n_k, p->d, p->dtype);
   s.medium_batch = explicit_medium_batch(p, nnz);  // (a launch-time choice: the plan does not depend on it)
   rc = check_workspace(plan, plan_bytes, work_list_bytes(p->n_q, nnz));
   if (rc) return rc;
@@ -586,6 +600,7 @@ int spfa_coo_forward(const spfa_problem_t* p, const void* row_ind, int row_ind_b
   if (nnz > 0 && (!row_ind || !col_ind)) return SPFA_ERR_BAD_ARG;
   EngineSizing s = size_csr(p->n_q, nnz);
   s.items_on_grid = explicit_items_on_grid(p->n_k, p->d, p->dtype);
+  s.items_as_listed = explicit_items_as_listed(p->n_k, p->d, p->dtype);
   const size_t coo_bytes = coo_workspace(p->n_q, nnz).total;
   const bool batched = batch_fits_engine(s, p);
   rc = check_workspace(workspace, workspace_bytes,
@@ -656,6 +671,7 @@ int spfa_coo_forward_planned(const spfa_problem_t* p, const void* col_ind, int64
   if (nnz > 0 && !col_ind) return SPFA_ERR_BAD_ARG;
   EngineSizing s = size_csr(p->n_q, nnz);
   s.items_on_grid = explicit_items_on_grid(p->n_k, p->d, p->dtype);
+  s.items_as_listed = explicit_items_as_listed(p->n_k, p->d, p->dtype);
   const CooWorkspace w = coo_workspace(p->n_q, nnz);
   rc = check_workspace(plan, plan_bytes, w.keep_total + work_list_bytes(p->n_q, nnz));
   if (rc) return rc;
@@ -1070,6 +1086,11 @@ GradArgs make_grad_args(const spfa_problem_t* p, const spfa_grads_t* g, const Gr
   // (explicit masks whose gathered tensors - K, V in the query pass, Q, dO in the key pass - stay in the caches)
   a.items_on_grid = lay.own_max == kGradOwnExplicit &&
                     explicit_items_on_grid(p->n_k > p->n_q ? p->n_k : p->n_q, p->d, p->dtype) ? 1 : 0;
+  // (Zipf mask, d = 64, gradient call with and without the two order_kernel launches, fp32 / bf16:
+  // 8192 tokens 0.197 -> 0.191 / 0.148 -> 0.140 ms, 16384 tokens 0.226 -> 0.220 / 0.188 -> 0.182,
+  // 32768 tokens 0.347 -> 0.352 / 0.273 -> 0.278)
+  a.items_as_listed = lay.own_max == kGradOwnExplicit &&
+                      explicit_items_as_listed(p->n_k > p->n_q ? p->n_k : p->n_q, p->d, p->dtype) ? 1 : 0;
   return a;
 }
 

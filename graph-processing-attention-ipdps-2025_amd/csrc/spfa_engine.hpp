@@ -975,6 +975,7 @@ struct EngineSizing {
   int64_t n_long_bound;  // upper bound on the number of rows with deg > short_max
   int medium_batch;      // neighbours in flight per lane group in medium_rows_kernel (0: the layout's)
   bool items_on_grid;    // the work list is walked by items_grid_kernel (explicit masks)
+  bool items_as_listed;  // ... in the order plan_kernel appended it in: no order_kernel (plain calls only)
 };
 
 struct WorkspaceLayout {
@@ -1137,7 +1138,11 @@ int launch_engine(const Tensors& t, const Mask& mask, const EngineSizing& s, int
     hipLaunchKernelGGL(reset_counters_kernel, dim3(1), dim3(64), 0, stream, plan.cnt, plan.phases);
     hipLaunchKernelGGL((plan_kernel<Mask>), dim3((unsigned)((t.n_q + kPlanThreads - 1) / kPlanThreads)),
                        dim3(kPlanThreads), 0, stream, t.n_q, mask, plan);
-    hipLaunchKernelGGL(order_kernel, dim3((w.cap_items + 255u) / 256u), dim3(256), 0, stream, plan);
+    // (a plan that is kept is always ordered: it is made without knowing K and V)
+    if (phase == kEngineAll && s.items_as_listed)
+      plan.items = plan.listed;
+    else
+      hipLaunchKernelGGL(order_kernel, dim3((w.cap_items + 255u) / 256u), dim3(256), 0, stream, plan);
   }
   if (phase == kEnginePlanOnly) return hipGetLastError() == hipSuccess ? 0 : 4;
   if (has_long && phase == kEngineRunOnly)

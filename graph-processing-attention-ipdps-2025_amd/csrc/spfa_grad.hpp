@@ -55,6 +55,8 @@ struct GradArgs {
   uint32_t cap_items;
   uint32_t* status;     // the device's sticky status word (may be null)
   int32_t items_on_grid;  // the work lists are walked by an ordinary grid, a wavefront per item
+  int32_t items_as_listed;  // ... and in the order they were appended in (no order_kernel): the
+                            // gathered tensors fit the L2s, the hand-out order is worth nothing
 };
 
 constexpr int kGradWaves = 4;        // owners per workgroup
@@ -454,6 +456,13 @@ int launch_grad(const Tensors& t, const GradArgs& g, const RowMask& rows, const 
   if (nq >= ((int64_t)1 << 32) || nk >= ((int64_t)1 << 32)) return 1;  // items hold 32-bit owners
   const dim3 block(kGradWaves * kWave);
   const bool lists = g.cap_items > 1;  // (no owner of this call can have more than own_max candidates otherwise)
+  // (the lists walked as they were appended, see GradArgs::items_as_listed)
+  const bool as_listed = g.items_as_listed != 0;
+  GradArgs gl = g;
+  if (as_listed) {
+    gl.ordered[0] = gl.listed[0];
+    gl.ordered[1] = gl.listed[1];
+  }
   const dim3 grid_order((g.cap_items + 255u) / 256u);
   int64_t grid_seg = (int64_t)device_cu_count() * kSegmentWorkgroupsPerCu;
   if (grid_seg > ((int64_t)g.cap_items + 3) / 4) grid_seg = ((int64_t)g.cap_items + 3) / 4;
@@ -468,24 +477,24 @@ int launch_grad(const Tensors& t, const GradArgs& g, const RowMask& rows, const 
   else
     hipLaunchKernelGGL((grad_rows_kernel<Lay, RowMask, false>), dim3((unsigned)q_blocks), block, 0, stream, g, rows);
   if (lists) {
-    hipLaunchKernelGGL(order_kernel, grid_order, dim3(256), 0, stream, grad_plan(g, 0));
+    if (!as_listed) hipLaunchKernelGGL(order_kernel, grid_order, dim3(256), 0, stream, grad_plan(g, 0));
     if (g.items_on_grid)
       hipLaunchKernelGGL((grad_segments_kernel<Lay, RowMask, false, true>), dim3((g.cap_items + 3u) / 4u),
-                         dim3(256), 0, stream, g, rows);
+                         dim3(256), 0, stream, gl, rows);
     else
       hipLaunchKernelGGL((grad_segments_kernel<Lay, RowMask, false>), dim3((unsigned)grid_seg), dim3(256), 0,
-                         stream, g, rows);
+                         stream, gl, rows);
   }
   if (!both)
     hipLaunchKernelGGL((grad_rows_kernel<Lay, ColMask, true>), dim3((unsigned)k_blocks), block, 0, stream, g, cols);
   if (lists) {
-    hipLaunchKernelGGL(order_kernel, grid_order, dim3(256), 0, stream, grad_plan(g, 1));
+    if (!as_listed) hipLaunchKernelGGL(order_kernel, grid_order, dim3(256), 0, stream, grad_plan(g, 1));
     if (g.items_on_grid)
       hipLaunchKernelGGL((grad_segments_kernel<Lay, ColMask, true, true>), dim3((g.cap_items + 3u) / 4u),
-                         dim3(256), 0, stream, g, cols);
+                         dim3(256), 0, stream, gl, cols);
     else
       hipLaunchKernelGGL((grad_segments_kernel<Lay, ColMask, true>), dim3((unsigned)grid_seg), dim3(256), 0,
-                         stream, g, cols);
+                         stream, gl, cols);
   }
   return hipGetLastError() == hipSuccess ? 0 : 4;
 }
