@@ -16,6 +16,8 @@ using bf16 = __bf16;
 typedef float float4v __attribute__((ext_vector_type(4)));
 typedef _Float16 half8v __attribute__((ext_vector_type(8)));
 typedef __bf16 bhalf8v __attribute__((ext_vector_type(8)));
+typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+typedef __bf16 bhalf2v __attribute__((ext_vector_type(2)));
 typedef uint32_t uint4v __attribute__((ext_vector_type(4)));
 
 template <typename T>
@@ -140,6 +142,41 @@ struct VecLay {
       }
     }
   }
+  // The dot product of a gathered piece with the owner's piece.  For the two-byte types the
+  // owner's floats came out of that type, so they pack again exactly and two products at a time
+  // go through the dot instructions (fp32 sums of exact products): 4 instructions a piece where
+  // unpacking and multiplying takes 16.
+  static constexpr bool kPackedDot = sizeof(T) == 2;
+  __device__ static __forceinline__ raw pack_exact(const float (&f)[NE]) {
+    raw r{0u, 0u, 0u, 0u};
+    if constexpr (__is_same(T, f16)) {
+      half8v x;
+#pragma unroll
+      for (int e = 0; e < 8; e++) x[e] = (f16)f[e];
+      r = __builtin_bit_cast(raw, x);
+    } else if constexpr (sizeof(T) == 2) {
+#pragma unroll
+      for (int e = 0; e < 4; e++)
+        r[e] = (__builtin_bit_cast(uint32_t, f[2 * e]) >> 16) |
+               (__builtin_bit_cast(uint32_t, f[2 * e + 1]) & 0xffff0000u);
+    }
+    return r;
+  }
+  __device__ static __forceinline__ float packed_dot(const raw& x, const raw& y) {
+    float acc = 0.f;
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+      // (copies first: a bit cast applied to an element of a vector reads the vector's first
+      // element whichever one is named)
+      const uint32_t xe = x[e], ye = y[e];
+      if constexpr (__is_same(T, f16))
+        acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2v, xe), __builtin_bit_cast(half2v, ye), acc, false);
+      else if constexpr (sizeof(T) == 2)
+        acc = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bhalf2v, xe), __builtin_bit_cast(bhalf2v, ye), acc,
+                                              false);
+    }
+    return acc;
+  }
   __device__ static __forceinline__ void store(T* row_ptr, int c, int d, const float (&f)[NE]) {
     if constexpr (PAD) {
       if (c * NE >= d) return;
@@ -205,6 +242,7 @@ struct WideLay {
   static constexpr int U = 16 / NCH;  // (the bytes in flight per lane of VecLay)
   static constexpr int U_SHORT = U >= 4 ? U / 4 : 1;
   static constexpr int U_MEDIUM = U >= 2 ? U / 2 : 1;
+  static constexpr bool kPackedDot = false;
   static_assert(NCH == 2 || NCH == 4 || NCH == 8, "two to eight chunks per lane");
   struct raw { uint4v x[NCH]; };
   __device__ static __forceinline__ int elem_index(int c, int e) { return (c + 32 * (e / NC)) * NC + e % NC; }
@@ -273,6 +311,7 @@ struct GenLay {
   static constexpr int U = (EPL <= 2) ? 8 : 2;
   static constexpr int U_SHORT = U;
   static constexpr int U_MEDIUM = U;
+  static constexpr bool kPackedDot = false;
   struct raw { T x[EPL]; };
   __device__ static __forceinline__ int elem_index(int c, int e) { return c + e * kWave; }
 

@@ -199,6 +199,8 @@ __device__ __forceinline__ void attend(const Mask& mask, const typename Mask::Ro
     return valid ? (int)col : -1;
   };
 
+  typename Lay::raw qp{};
+  if constexpr (Lay::kPackedDot) qp = Lay::pack_exact(q);
   int next = fetch(t_begin);
   for (int64_t tb = t_begin; tb < t_end; tb += SPAN) {
     int cur = next;
@@ -224,10 +226,14 @@ __device__ __forceinline__ void attend(const Mask& mask, const typename Mask::Ro
       for (int u = 0; u < U; u++) {
         float part_dot = 0.f;
         if (cols[u] >= 0) {
-          float kf[NE];
-          Lay::unpack(kr[u], kf);
+          if constexpr (Lay::kPackedDot) {
+            part_dot = Lay::packed_dot(kr[u], qp);
+          } else {
+            float kf[NE];
+            Lay::unpack(kr[u], kf);
 #pragma unroll
-          for (int e = 0; e < NE; e++) part_dot += q[e] * kf[e];
+            for (int e = 0; e < NE; e++) part_dot += q[e] * kf[e];
+          }
         }
         float tot = group_sum<LPR>(part_dot) * scale;
         s[u] = cols[u] >= 0 ? tot : kNegInf;

@@ -178,6 +178,12 @@ __device__ __forceinline__ void grad_walk(const Mask& mask, const typename Mask:
     return valid ? (int)col : -1;
   };
 
+  // (the owner's two vectors came out of the element type: see Lay::packed_dot)
+  typename Lay::raw ap{}, bp{};
+  if constexpr (Lay::kPackedDot) {
+    ap = Lay::pack_exact(a);
+    bp = Lay::pack_exact(b);
+  }
   int next = fetch(t_begin);
   for (int64_t tb = t_begin; tb < t_end; tb += kWave) {
     int cur = next;
@@ -215,11 +221,17 @@ __device__ __forceinline__ void grad_walk(const Mask& mask, const typename Mask:
         float s = 0.f, t = 0.f;
         if (cols[u] >= 0) {
           Lay::unpack(xr[u], xf);
-          Lay::unpack(yr[u], yf);
+          if constexpr (Lay::kPackedDot) {
+            s = Lay::packed_dot(xr[u], ap);
+            t = Lay::packed_dot(yr[u], bp);
+            if constexpr (KEYS) Lay::unpack(yr[u], yf);
+          } else {
+            Lay::unpack(yr[u], yf);
 #pragma unroll
-          for (int e = 0; e < NE; e++) {
-            s += a[e] * xf[e];
-            t += b[e] * yf[e];
+            for (int e = 0; e < NE; e++) {
+              s += a[e] * xf[e];
+              t += b[e] * yf[e];
+            }
           }
         }
         s = group_sum<LPR>(s);
