@@ -919,11 +919,13 @@ int coo_to_csr(const void* row_ind, int row_wide, const uint32_t* col_ind, int64
   uint32_t* flag = (uint32_t*)(kbase + w.off_flag);
   const int64_t n_tiles = (n_rows + kScanTile - 1) / kScanTile;
 
-  hipLaunchKernelGGL(fill_u32_kernel, dim3(grid_for(n_rows + 1, 256, 4096)), dim3(256), 0, stream,
-                     counts, n_rows + 1, 0u);
   hipLaunchKernelGGL(fill_u32_kernel, dim3(1), dim3(64), 0, stream, flag, (int64_t)1, 0u);
   // sorted or not: decided on the device (by the first pass of the partition where there is one)
   const bool part = nnz > 0 && w.partition;
+  // (the per-row counts belong to the histogram path below; the partition keeps its own)
+  if (!part && nnz > 0)
+    hipLaunchKernelGGL(fill_u32_kernel, dim3(grid_for(n_rows + 1, 256, 4096)), dim3(256), 0, stream,
+                       counts, n_rows + 1, 0u);
   if (part) {
     const dim3 grid_c(part_grid(w.n_tiles1));
     if (row_wide)
