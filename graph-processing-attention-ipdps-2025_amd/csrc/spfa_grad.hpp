@@ -78,12 +78,31 @@ __device__ __forceinline__ int grad_elem_index(int c, int e) {
 }
 
 // lse and delta of every query row: 16 lanes per row, 16 bytes per lane and step
-template <typename T>
+// Clears the counters and phase counts of both work lists (64 lanes).
+__device__ __forceinline__ void grad_reset(const GradArgs& g, int lane) {
+  static_assert(kPhases == kWave, "one lane per phase");
+  for (int p = 0; p < 2; p++) {
+    g.phases[p]->count[lane] = 0;
+    g.phases[p]->taken[lane] = 0;
+    if (lane == 0) {
+      g.cnt[p]->n_items = 0;
+      g.cnt[p]->next_item = 0;
+      g.cnt[p]->overflow = 0;
+    }
+  }
+}
+
+// (RESET: the first wavefront also clears the gather passes' work lists - a launch of its own for
+// that costs a short call 4 - 5 us)
+template <typename T, bool RESET = false>
 __global__ __launch_bounds__(256) void grad_prologue_kernel(Tensors t, GradArgs g) {
   constexpr int V = 16 / (int)sizeof(T);
   typedef T vec __attribute__((ext_vector_type(V)));
   const int c = threadIdx.x & 15;
   const int64_t row = (int64_t)blockIdx.x * 16 + (threadIdx.x >> 4);
+  if constexpr (RESET) {
+    if (blockIdx.x == 0 && threadIdx.x < kWave) grad_reset(g, (int)threadIdx.x);
+  }
   if (row >= t.n_q * t.n_batch) return;
   const bool sf = t.state_f32 != 0;
   const float m = load_state<T>(t.m, row, sf);
@@ -113,19 +132,6 @@ __global__ __launch_bounds__(256) void grad_prologue_kernel(Tensors t, GradArgs 
     g.lse[row] = lse;
     g.delta[row] = delta;
     g.stat[row] = make_float2(lse, delta);
-  }
-}
-
-static __global__ void grad_reset_kernel(GradArgs g) {
-  static_assert(kPhases == kWave, "one lane per phase");
-  for (int p = 0; p < 2; p++) {
-    g.phases[p]->count[threadIdx.x] = 0;
-    g.phases[p]->taken[threadIdx.x] = 0;
-    if (threadIdx.x == 0) {
-      g.cnt[p]->n_items = 0;
-      g.cnt[p]->next_item = 0;
-      g.cnt[p]->overflow = 0;
-    }
   }
 }
 
@@ -478,8 +484,7 @@ int launch_grad(const Tensors& t, const GradArgs& g, const RowMask& rows, const 
   const dim3 grid_order((g.cap_items + 255u) / 256u);
   int64_t grid_seg = (int64_t)device_cu_count() * kSegmentWorkgroupsPerCu;
   if (grid_seg > ((int64_t)g.cap_items + 3) / 4) grid_seg = ((int64_t)g.cap_items + 3) / 4;
-  hipLaunchKernelGGL(grad_reset_kernel, dim3(1), dim3(64), 0, stream, g);
-  hipLaunchKernelGGL((grad_prologue_kernel<T>), dim3((unsigned)((nq + 15) / 16)), dim3(256), 0, stream,
+  hipLaunchKernelGGL((grad_prologue_kernel<T, true>), dim3((unsigned)((nq + 15) / 16)), dim3(256), 0, stream,
                      t, g);
   const int64_t q_blocks = (nq + kGradWaves - 1) / kGradWaves, k_blocks = (nk + kGradWaves - 1) / kGradWaves;
   const bool both = nq + nk <= kGradBothOwnersMax;
